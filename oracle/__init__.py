@@ -1,0 +1,340 @@
+"""ctypes front-end of the CPU oracle — TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+
+Loads ``oracle/librp_oracle.so`` (this repository's restatement of the RecPulse
+reference's CPU arithmetic, ``rp_oracle.c``) and, when it has been built,
+``oracle/_ref/libref_host.so`` (the reference's own host kernels compiled
+unchanged).  Only ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` may import this package; the shipped
+library never does.
+
+16-bit tensors travel as ``numpy.uint16`` bit patterns: numpy has no bfloat16,
+and the reference's narrowing (round half away from zero, reference
+core/half_precision.h:50-97) differs from numpy's float16 casts on ties.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+F32, F64, F16, BF16 = 0, 1, 2, 3          # reference core/tensor.h:7-13
+DTYPE_NAMES = {F32: "float32", F64: "float64", F16: "float16", BF16: "bfloat16"}
+NP_STORAGE = {F32: np.float32, F64: np.float64, F16: np.uint16, BF16: np.uint16}
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "librp_oracle.so")
+_REF_PATH = os.path.join(_HERE, "_ref", "libref_host.so")
+
+
+def build():
+    """Compile the oracle (and oracle/_ref when the reference tree is mounted)."""
+    subprocess.check_call(["make", "-s", "-C", _HERE, "all"])
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        build()
+    return ctypes.CDLL(_LIB_PATH)
+
+
+_lib = _load()
+_vp, _i, _ll, _sz, _d = ctypes.c_void_p, ctypes.c_int, ctypes.c_longlong, ctypes.c_size_t, ctypes.c_double
+_ip = ctypes.POINTER(ctypes.c_int)
+_llp = ctypes.POINTER(ctypes.c_longlong)
+
+
+def _sig(name, res, *args):
+    fn = getattr(_lib, name)
+    fn.restype = res
+    fn.argtypes = list(args)
+    return fn
+
+
+_matmul = _sig("orc_matmul", _i, _vp, _vp, _vp, _i, _i, _i, _i)
+_gemm = _sig("orc_gemm_strided_batched", _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
+             _ll, _ll, _ll, _ll, _ll, _ll, _ll, _ll, _ll, _i, _i)
+_add = _sig("orc_add", _i, _vp, _vp, _vp, _sz, _i)
+_add_strided = _sig("orc_add_strided", _i, _vp, _vp, _vp, _i, _ip, _ip, _ip, _sz, _i)
+_mul_scalar = _sig("orc_mul_scalar", _i, _vp, _vp, _d, _sz, _i)
+_relu = _sig("orc_relu", _i, _vp, _vp, _sz, _i)
+_bw_relu = _sig("orc_backwards_relu", _i, _vp, _vp, _vp, _sz, _i)
+_softmax = _sig("orc_softmax", _i, _vp, _vp, _sz, _sz, _sz, _i)
+_log_softmax = _sig("orc_log_softmax", _i, _vp, _vp, _sz, _sz, _sz, _i)
+_bw_softmax = _sig("orc_backwards_softmax", _i, _vp, _vp, _vp, _sz, _sz, _sz, _i)
+_sum_all = _sig("orc_sum_all", _i, _vp, _vp, _sz, _i)
+_reduce_rows = _sig("orc_reduce_rows", _i, _vp, _vp, _i, _i, _i)
+_contig = _sig("orc_contiguous_copy", _i, _vp, _vp, _i, _ip, _llp, _i)
+_ce = _sig("orc_cross_entropy_mean", _i, _vp, _vp, _vp, _ip, _i, _i, _d, _i)
+_widen = _sig("orc_widen", None, _vp, _vp, _sz, _i)
+_narrow = _sig("orc_narrow", None, _vp, _vp, _sz, _i)
+
+
+def _ptr(a):
+    return a.ctypes.data_as(_vp)
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise RuntimeError(f"oracle {what} failed")
+
+
+# ---------------------------------------------------------------------------
+# dtype helpers
+# ---------------------------------------------------------------------------
+def widen(bits, dtype):
+    """uint16 bit patterns (fp16 or bf16) -> float32, exact."""
+    bits = np.ascontiguousarray(bits, dtype=np.uint16)
+    out = np.empty(bits.shape, dtype=np.float32)
+    _widen(_ptr(bits), _ptr(out), bits.size, dtype)
+    return out
+
+
+def narrow(x, dtype):
+    """float32 -> uint16 bit patterns with the reference's rounding."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint16)
+    _narrow(_ptr(x), _ptr(out), x.size, dtype)
+    return out
+
+
+def to_storage(x64, dtype):
+    """float64 array -> the storage array of `dtype` (cast once, reference rounding for 16-bit)."""
+    if dtype == F64:
+        return np.ascontiguousarray(x64, dtype=np.float64)
+    x32 = np.ascontiguousarray(x64, dtype=np.float32)
+    if dtype == F32:
+        return x32
+    return narrow(x32, dtype)
+
+
+def to_f64(x, dtype):
+    """storage array of `dtype` -> float64 values, exact."""
+    if dtype in (F16, BF16):
+        return widen(x, dtype).astype(np.float64)
+    return np.asarray(x, dtype=np.float64)
+
+
+# ---------------------------------------------------------------------------
+# the restated ops (all take and return storage arrays of `dtype`)
+# ---------------------------------------------------------------------------
+def matmul(a, b, dtype):
+    a = np.ascontiguousarray(a); b = np.ascontiguousarray(b)
+    m, k = a.shape; k2, n = b.shape
+    assert k == k2
+    c = np.empty((m, n), dtype=NP_STORAGE[dtype])
+    _check(_matmul(_ptr(c), _ptr(a), _ptr(b), m, k, n, dtype), "matmul")
+    return c
+
+
+def gemm_strided_batched(c_buf, a_buf, b_buf, bias, batch, m, k, n, a_st, b_st, c_st, accumulate, dtype):
+    """In-place on the flat storage buffer `c_buf`; *_st = (batch, row, col) strides in elements."""
+    _check(_gemm(_ptr(c_buf), _ptr(a_buf), _ptr(b_buf), _ptr(bias) if bias is not None else None,
+                 batch, m, k, n, *a_st, *b_st, *c_st, int(bool(accumulate)), dtype), "gemm_strided_batched")
+    return c_buf
+
+
+def add(x1, x2, dtype):
+    x1 = np.ascontiguousarray(x1); x2 = np.ascontiguousarray(x2)
+    out = np.empty_like(x1)
+    _check(_add(_ptr(out), _ptr(x1), _ptr(x2), x1.size, dtype), "add")
+    return out
+
+
+def add_strided(x1, x2, out_shape, s1, s2, dtype):
+    out = np.empty(out_shape, dtype=NP_STORAGE[dtype])
+    nd = len(out_shape)
+    arr = lambda v: (ctypes.c_int * nd)(*[int(t) for t in v])
+    _check(_add_strided(_ptr(out), _ptr(x1), _ptr(x2), nd, arr(out_shape), arr(s1), arr(s2), out.size, dtype),
+           "add_strided")
+    return out
+
+
+def bias_add(y, bias, dtype):
+    """[m, n] + [n] the way Linear does it (reference recpulse/module.py:110-114)."""
+    m, n = y.shape
+    return add_strided(np.ascontiguousarray(y), np.ascontiguousarray(bias), (m, n), (n, 1), (0, 1), dtype)
+
+
+def mul_scalar(x, scalar, dtype):
+    x = np.ascontiguousarray(x)
+    out = np.empty_like(x)
+    _check(_mul_scalar(_ptr(out), _ptr(x), float(scalar), x.size, dtype), "mul_scalar")
+    return out
+
+
+def relu(x, dtype):
+    x = np.ascontiguousarray(x)
+    out = np.empty_like(x)
+    _check(_relu(_ptr(out), _ptr(x), x.size, dtype), "relu")
+    return out
+
+
+def backwards_relu(grad_c, x, dtype):
+    grad_c = np.ascontiguousarray(grad_c); x = np.ascontiguousarray(x)
+    out = np.empty_like(x)
+    _check(_bw_relu(_ptr(grad_c), _ptr(x), _ptr(out), x.size, dtype), "backwards_relu")
+    return out
+
+
+def _split(shape, dim):
+    dim = dim % len(shape)
+    outer = int(np.prod(shape[:dim], dtype=np.int64)) if dim > 0 else 1
+    inner = int(np.prod(shape[dim + 1:], dtype=np.int64)) if dim + 1 < len(shape) else 1
+    return outer, int(shape[dim]), inner
+
+
+def softmax(x, dtype, dim=-1, log=False):
+    x = np.ascontiguousarray(x)
+    out = np.empty_like(x)
+    o, d, i = _split(x.shape, dim)
+    _check((_log_softmax if log else _softmax)(_ptr(out), _ptr(x), o, d, i, dtype), "softmax")
+    return out
+
+
+def backwards_softmax(grad_c, y, dtype, dim=-1):
+    grad_c = np.ascontiguousarray(grad_c); y = np.ascontiguousarray(y)
+    out = np.empty_like(y)
+    o, d, i = _split(y.shape, dim)
+    _check(_bw_softmax(_ptr(grad_c), _ptr(y), _ptr(out), o, d, i, dtype), "backwards_softmax")
+    return out
+
+
+def sum_all(x, dtype):
+    x = np.ascontiguousarray(x)
+    out = np.empty((1,), dtype=NP_STORAGE[dtype])
+    _check(_sum_all(_ptr(out), _ptr(x), x.size, dtype), "sum_all")
+    return out
+
+
+def reduce_rows(grad, dtype):
+    """Bias gradient of Linear: [rows, cols] -> [cols] (reference ops/ops.c:6970-7101)."""
+    grad = np.ascontiguousarray(grad)
+    rows, cols = grad.shape
+    out = np.empty((cols,), dtype=NP_STORAGE[dtype])
+    _check(_reduce_rows(_ptr(out), _ptr(grad), rows, cols, dtype), "reduce_rows")
+    return out
+
+
+def contiguous_copy(buf, shape, strides, dtype, offset=0):
+    """Gather the view (shape, strides in elements, offset in elements) of flat `buf`."""
+    nd = len(shape)
+    out = np.empty(shape, dtype=NP_STORAGE[dtype])
+    base = buf.reshape(-1)[offset:]
+    _check(_contig(_ptr(out), _ptr(base), nd, (ctypes.c_int * nd)(*[int(s) for s in shape]),
+                   (ctypes.c_longlong * nd)(*[int(s) for s in strides]), dtype), "contiguous_copy")
+    return out
+
+
+def cross_entropy_mean(logits, targets, dtype, upstream=1.0):
+    """Returns (loss scalar, dlogits) for mean cross-entropy on logits; f32/f64 only."""
+    logits = np.ascontiguousarray(logits)
+    b, c = logits.shape
+    t = np.ascontiguousarray(targets, dtype=np.int32)
+    loss = np.empty((1,), dtype=NP_STORAGE[dtype])
+    grad = np.empty_like(logits)
+    _check(_ce(_ptr(loss), _ptr(grad), _ptr(logits), t.ctypes.data_as(_ip), b, c, float(upstream), dtype),
+           "cross_entropy_mean")
+    return loss, grad
+
+
+# ---------------------------------------------------------------------------
+# compositions used by the parity tests (pure chaining of the ops above, in the
+# order the reference's autograd runs them)
+# ---------------------------------------------------------------------------
+def linear_forward(x, w, bias, dtype):
+    """reference recpulse/module.py:110-114."""
+    y = matmul(x, w, dtype)
+    return bias_add(y, bias, dtype) if bias is not None else y
+
+
+def matmul_backward(a, b, dc, dtype):
+    """reference ops/ops.c:6759-6814: dA = dC @ B^T, dB = A^T @ dC on densified transposes."""
+    da = matmul(dc, np.ascontiguousarray(b.T), dtype)
+    db = matmul(np.ascontiguousarray(a.T), dc, dtype)
+    return da, db
+
+
+def mlp_step(x, weights, biases, targets, dtype=F32):
+    """Config-2 style MLP (Linear+ReLU ... Linear, mean cross-entropy) forward and backward.
+
+    Returns dict(loss, logits, dW=[...], db=[...], dX).  Order of operations follows
+    the reference autograd: Linear = matmul then broadcasting add; backward of add
+    hands dY to the matmul and reduces it over rows for the bias.
+    """
+    acts, pre = [x], []
+    h = x
+    nl = len(weights)
+    for li in range(nl):
+        z = linear_forward(h, weights[li], biases[li], dtype)
+        pre.append(z)
+        h = relu(z, dtype) if li + 1 < nl else z
+        acts.append(h)
+    loss, g = cross_entropy_mean(h, targets, dtype)
+    dws, dbs = [None] * nl, [None] * nl
+    for li in reversed(range(nl)):
+        if li + 1 < nl:
+            g = backwards_relu(g, pre[li], dtype)
+        dbs[li] = reduce_rows(g, dtype) if biases[li] is not None else None
+        da, dw = matmul_backward(acts[li], weights[li], g, dtype)
+        dws[li] = dw
+        g = da
+    return {"loss": loss, "logits": h, "dW": dws, "db": dbs, "dX": g}
+
+
+def attention(q, k, v, dtype, scale=0.125, d_out=None):
+    """Config-4 attention for ONE (batch, head) slice: S=q@k^T, P=softmax(S*scale), O=P@v.
+
+    With d_out (dO) also returns dQ, dK, dV following the reference autograd chain
+    matmul -> mul_scalar -> softmax -> matmul.
+    """
+    kt = np.ascontiguousarray(k.T)
+    s = matmul(q, kt, dtype)
+    ss = mul_scalar(s, scale, dtype)
+    p = softmax(ss, dtype)
+    o = matmul(p, v, dtype)
+    if d_out is None:
+        return {"S": s, "P": p, "O": o}
+    dp, dv = matmul_backward(p, v, d_out, dtype)
+    dss = backwards_softmax(dp, p, dtype)
+    ds = mul_scalar(dss, scale, dtype)
+    dq, dkt = matmul_backward(q, kt, ds, dtype)
+    dk = np.ascontiguousarray(dkt.T)       # permute backward = inverse permutation (reference ops/ops.c:7977-8014)
+    return {"S": s, "P": p, "O": o, "dQ": dq, "dK": dk, "dV": dv}
+
+
+def matmul_f64(a, b, dtype):
+    """The float64 oracle: exact inputs of `dtype`, float64 numpy product."""
+    return to_f64(a, dtype) @ to_f64(b, dtype)
+
+
+def rel_err(x, ref):
+    """Normwise relative error ||x - ref||_F / ||ref||_F in float64."""
+    x = np.asarray(x, dtype=np.float64); ref = np.asarray(ref, dtype=np.float64)
+    den = np.linalg.norm(ref.ravel())
+    num = np.linalg.norm((x - ref).ravel())
+    return num / den if den > 0 else num
+
+
+# ---------------------------------------------------------------------------
+# the reference's own host kernels (oracle/_ref), when built
+# ---------------------------------------------------------------------------
+def load_reference():
+    """ctypes handle of oracle/_ref/libref_host.so, or None when it was not built."""
+    if not os.path.exists(_REF_PATH):
+        return None
+    ref = ctypes.CDLL(_REF_PATH)
+    for name, ct in (("matmul_kernel_host_f32", ctypes.c_float), ("matmul_kernel_host_f64", ctypes.c_double)):
+        fn = getattr(ref, name)
+        fn.restype = _i
+        fn.argtypes = [_vp, _vp, _vp, _i, _i, _i]
+    return ref
+
+
+def reference_matmul(ref, a, b, dtype):
+    """C = A @ B through the reference's matmul_kernel_host_f32/f64 (f32/f64 only)."""
+    a = np.ascontiguousarray(a); b = np.ascontiguousarray(b)
+    m, k = a.shape; n = b.shape[1]
+    c = np.empty((m, n), dtype=NP_STORAGE[dtype])
+    fn = ref.matmul_kernel_host_f32 if dtype == F32 else ref.matmul_kernel_host_f64
+    _check(fn(_ptr(c), _ptr(a), _ptr(b), m, k, n), "reference matmul")
+    return c
