@@ -1,0 +1,170 @@
+/*
+ * rp_hip.h — C ABI of librp_hip.so, the MI355X (gfx950) device layer for the
+ * RecPulse matmul path.
+ *
+ * Plain C: pointers, sizes, ints.  Every function returns 0 on success and -1
+ * on failure (the reference's convention for its *_kernel_device functions);
+ * rp_hip_last_error() gives the text.  Device pointers are raw HIP device
+ * addresses.  All work is enqueued on the calling thread's current stream
+ * (the null stream unless rp_hip_set_stream() changed it) and is NOT waited
+ * for: completion is stream-ordered, as with the reference's CUDA entry points.
+ *
+ * Entry points that keep the reference's own symbol name replace the function
+ * of that name in the reference's CUDA files one for one, so the reference's
+ * host C links against this library unchanged.  Entry points named rp_hip_*
+ * are new; each comment names the reference code it stands in for.
+ */
+#ifndef RP_HIP_H
+#define RP_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* dtype codes: identical to the reference's DType (core/tensor.h:7-13). */
+enum {
+    RP_DTYPE_FLOAT32 = 0,
+    RP_DTYPE_FLOAT64 = 1,
+    RP_DTYPE_FLOAT16 = 2,
+    RP_DTYPE_BFLOAT16 = 3
+};
+
+/* ------------------------------------------------------------------------
+ * Device runtime shim.  Replaces the direct CUDA runtime calls the
+ * reference's host C makes (cudaGetDeviceCount core/tensor.c:14; cudaSetDevice
+ * e.g. functional/functional.c:1004; cudaMalloc + cudaMemset
+ * core/tensor_device.cu:44-46; cudaFree core/tensor_device.cu:273-281;
+ * cudaMemcpy H2D/D2H/D2D core/tensor_device.cu:295-531; the error text and
+ * device synchronisation of core/cuda_helpers.cu:6-26).
+ * ---------------------------------------------------------------------- */
+int rp_hip_device_count(int* count);
+int rp_hip_set_device(int device_id);
+int rp_hip_get_device(int* device_id);
+/* Allocations come from a per-device caching pool (freed blocks are kept and
+ * handed out again, so a steady-state training step performs no hipMalloc).
+ * Blocks are reused in stream order on one stream; a caller that uses several
+ * streams must synchronise before freeing.  RP_HIP_NO_CACHE=1 in the
+ * environment turns the pool off. */
+int rp_hip_malloc(void** ptr, size_t bytes);
+int rp_hip_free(void* ptr);
+int rp_hip_empty_cache(void);
+int rp_hip_memset(void* ptr, int value, size_t bytes);
+int rp_hip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes);
+int rp_hip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes);
+int rp_hip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes);
+int rp_hip_synchronize(void);
+const char* rp_hip_last_error(void);
+/* Stream the calling thread's launches go to; stream is a hipStream_t (NULL = null stream). */
+int rp_hip_set_stream(void* stream);
+void* rp_hip_get_stream(void);
+/* HIP events on the current stream, for timing from hosts that have no HIP binding. */
+int rp_hip_event_create(void** event);
+int rp_hip_event_record(void* event);
+int rp_hip_event_synchronize(void* event);
+int rp_hip_event_elapsed_ms(float* ms, void* start, void* stop);
+int rp_hip_event_destroy(void* event);
+
+/* ------------------------------------------------------------------------
+ * GEMM.
+ * ---------------------------------------------------------------------- */
+
+/* Dense row-major C[m,n] = A[m,k] · B[k,n], C fully overwritten.
+ * Same name, arguments and meaning as the reference's cuBLAS-backed seam
+ * (functional/functional.h:426, functional/functional_device.cu:991-1071),
+ * which rp_matmul calls after selecting the device
+ * (functional/functional.c:1004-1005). */
+int matmul_kernel_device(void* C, const void* A, const void* B, int m, int k, int n, int dtype);
+
+/* Strided, batched generalisation of the seam with the Linear epilogue:
+ *
+ *   for z in [0,batch):  C_z = A_z · B_z  (+ bias[j] on every row)  (+ previous C_z)
+ *
+ * X_z[i,j] lives at X + z*x_bs + i*x_rs + j*x_cs (strides in ELEMENTS, any
+ * sign-free combination: transposed and permuted views are passed as they
+ * are and are never copied).  bias is NULL or a dense vector of n elements.
+ * accumulate != 0 adds the product into the existing C (beta = 1).
+ * fp16/bf16 accumulate in fp32 and narrow once per reference op in the chain
+ * (matmul, then bias add, then accumulation), with the reference's rounding.
+ *
+ * Stands in for: ensure_contiguous + rp_matmul in op_matmul
+ * (ops/ops.c:6830-6838); rp_transpose + rp_contiguous + rp_matmul + rp_add in
+ * backward_matmul_fn (ops/ops.c:6770-6811); the broadcasting op_add that
+ * Linear.forward issues after the matmul (recpulse/module.py:110-114,
+ * ops/ops.c:129-210).  The reference has no batched matmul (op_matmul is 2-D
+ * only, ops/ops.c:6818); batch > 1 equals a loop of 2-D calls. */
+int rp_hip_gemm_strided_batched(void* C, const void* A, const void* B, const void* bias,
+                                int batch, int m, int k, int n,
+                                long long a_bs, long long a_rs, long long a_cs,
+                                long long b_bs, long long b_rs, long long b_cs,
+                                long long c_bs, long long c_rs, long long c_cs,
+                                int accumulate, int dtype);
+
+/* Name of the kernel family the dispatcher picks for a problem, for logs and
+ * tests ("mfma16_256x256", "skinny", "generic", ...).  No device work. */
+const char* rp_hip_gemm_kernel_name(int batch, int m, int k, int n,
+                                    long long a_rs, long long a_cs,
+                                    long long b_rs, long long b_cs,
+                                    long long c_rs, long long c_cs, int dtype);
+
+/* ------------------------------------------------------------------------
+ * The other device entry points BASELINE's configs touch.  Names and
+ * arguments are the reference's (functional/functional.h:363-428,
+ * ops/ops.h backwards_*_device declarations).
+ * ---------------------------------------------------------------------- */
+/* functional/functional_device.cu:94-246 */
+int add_kernel_device(void* out, const void* x1, const void* x2, size_t size, int dtype);
+/* functional/functional_device.cu:248-330: out is dense row-major of out_shape;
+ * operands are indexed with per-dimension element strides (0 = broadcast). */
+int add_strided_kernel_device(void* out, const void* x1, const void* x2, int ndim, const int* out_shape,
+                              const int* x1_strides, const int* x2_strides, size_t out_size, int dtype);
+/* functional/functional_device.cu:333-389: scalar points to HOST memory holding
+ * a double for float64 and a float for every other dtype. */
+int mul_scalar_kernel_device(void* out, const void* x, const void* scalar, size_t size, int dtype);
+/* functional/functional_device.cu:495-523 */
+int relu_kernel_device(void* out, const void* x, size_t size, int dtype);
+/* ops/grad_device.cu:523-555 */
+int backwards_relu_device(const void* grad_c, const void* x, void* grad_x, size_t size, int dtype);
+/* functional/functional_device.cu:1486-1565: tensor viewed as [outer, dim, inner] */
+int softmax_kernel_device(void* out, const void* x, size_t outer_size, size_t dim_size, size_t inner_size, int dtype);
+int log_softmax_kernel_device(void* out, const void* x, size_t outer_size, size_t dim_size, size_t inner_size, int dtype);
+/* ops/grad_device.cu:1236-1291 */
+int backwards_softmax_device(const void* grad_c, const void* softmax_out, void* grad_x,
+                             size_t outer_size, size_t dim_size, size_t inner_size, int dtype);
+/* functional/functional_device.cu:1197-1266: gather a strided view (element strides) into dense memory */
+int contiguous_copy_kernel_device(void* out, const void* in, int ndim, int* shape, int* strides, size_t size, int dtype);
+/* functional/functional_device.cu:756-989: out is a one-element device buffer */
+int sum_all_kernel_device(void* out, const void* x, size_t size, int dtype);
+int mean_all_kernel_device(void* out, const void* x, size_t size, int dtype);
+/* functional/functional_device.cu:1348-1484: reduce the middle axis of [outer, dim, inner] */
+int sum_dim_kernel_device(void* out, const void* x, size_t outer_size, size_t dim_size, size_t inner_size, int dtype);
+
+/* core/tensor_device.cu:66-114 (fill_value_kernel, copy_value_kernel<Src,Dst>) */
+int rp_hip_fill(void* ptr, double value, size_t size, int dtype);
+int rp_hip_convert(void* dst, int dst_dtype, const void* src, int src_dtype, size_t size);
+
+/* Bias gradient of Linear on the device: grad [rows, cols] dense -> out [cols],
+ * each column summed top to bottom in fp32 (fp64 for float64).  Stands in for
+ * the device->host->device round trip of reduce_grad_to_shape
+ * (ops/ops.c:6970-7101) in the [rows, cols] -> [cols] case. */
+int rp_hip_reduce_rows(void* out, const void* grad, int rows, int cols, int accumulate, int dtype);
+
+/* Mean cross-entropy on logits [batch, classes] (float32 / float64) on the
+ * device.  targets: device int32[batch], range-checked by the caller (the
+ * reference checks them on the host, ops/ops.c:5547-5549; an out-of-range
+ * index here yields a NaN loss, never an out-of-bounds read).  loss_out: one
+ * element of dtype.
+ * grad_logits (may be NULL): (softmax - onehot) * (1/batch) * upstream.
+ * Stands in for op_cross_entropy_loss / backward_cross_entropy_loss_fn, which
+ * run the NLL sum and the whole backward on the host (ops/ops.c:5318-5352,
+ * 5412-5543, 5545-5643). */
+int rp_hip_cross_entropy_mean(void* loss_out, void* grad_logits, const void* logits, const int* targets,
+                              int batch, int classes, double upstream, int dtype);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* RP_HIP_H */

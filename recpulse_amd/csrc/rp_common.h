@@ -1,0 +1,102 @@
+// Shared helpers of the gfx950 device layer: error reporting, the per-thread
+// stream, dtype traits and the reference's 16-bit rounding on the device.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "../../include/rp_hip.h"
+
+namespace rp {
+
+// ---- host side ------------------------------------------------------------
+void set_error(const char* fmt, ...);
+hipStream_t current_stream();
+bool check_hip(hipError_t e, const char* what);          // false (and error text) on failure
+bool check_launch(const char* what);                     // hipGetLastError after a launch
+
+inline size_t dtype_size(int dtype) {                    // reference core/half_precision.h:10-18
+    switch (dtype) {
+        case RP_DTYPE_FLOAT32: return 4;
+        case RP_DTYPE_FLOAT64: return 8;
+        case RP_DTYPE_FLOAT16: return 2;
+        case RP_DTYPE_BFLOAT16: return 2;
+        default: return 0;
+    }
+}
+
+// ---- device side ----------------------------------------------------------
+// Storage types.  16-bit values are carried as raw bit patterns so that the
+// reference's own rounding (not the hardware's round-to-nearest-even) decides
+// every narrowing.
+struct f16_t { uint16_t bits; };
+struct bf16_t { uint16_t bits; };
+
+template <typename T> struct traits;
+template <> struct traits<float>  { using acc = float;  static constexpr int code = RP_DTYPE_FLOAT32; };
+template <> struct traits<double> { using acc = double; static constexpr int code = RP_DTYPE_FLOAT64; };
+template <> struct traits<f16_t>  { using acc = float;  static constexpr int code = RP_DTYPE_FLOAT16; };
+template <> struct traits<bf16_t> { using acc = float;  static constexpr int code = RP_DTYPE_BFLOAT16; };
+
+__device__ __forceinline__ float widen(float x) { return x; }
+__device__ __forceinline__ double widen(double x) { return x; }
+__device__ __forceinline__ float widen(bf16_t x) { return __uint_as_float((uint32_t)x.bits << 16); }
+__device__ __forceinline__ float widen(f16_t x) {
+    // every fp16 value (subnormals included) is exact in fp32; the hardware
+    // conversion is exact too and keeps NaN payload bits in place
+    _Float16 h = __builtin_bit_cast(_Float16, x.bits);
+    return (float)h;
+}
+
+// fp32 -> bf16: truncate and add the first dropped bit (reference
+// core/half_precision.h:92-97; no NaN special case there either).
+__device__ __forceinline__ uint16_t narrow_bf16_bits(float f) {
+    uint32_t w = __float_as_uint(f);
+    return (uint16_t)((w >> 16) + ((w >> 15) & 1u));
+}
+
+// fp32 -> fp16 with the same "add the first dropped bit" rule, including the
+// subnormal and overflow branches (reference core/half_precision.h:50-83).
+__device__ __forceinline__ uint16_t narrow_f16_bits(float x) {
+    uint32_t w = __float_as_uint(x);
+    uint32_t s = (w >> 16) & 0x8000u;
+    uint32_t e32 = (w >> 23) & 0xFFu;
+    uint32_t f = w & 0x7FFFFFu;
+    int e = (int)e32 - 112;
+    if (e32 == 0xFFu) return (uint16_t)(f ? (s | 0x7C00u | (f >> 13) | 1u) : (s | 0x7C00u));
+    if (e <= 0) {
+        if (e < -10) return (uint16_t)s;
+        f |= 0x800000u;
+        int sh = 14 - e;
+        return (uint16_t)((s | (f >> sh)) + ((f >> (sh - 1)) & 1u));
+    }
+    if (e >= 0x1F) return (uint16_t)(s | 0x7C00u);
+    return (uint16_t)((s | ((uint32_t)e << 10) | (f >> 13)) + ((f >> 12) & 1u));
+}
+
+template <typename T> __device__ __forceinline__ T narrow(typename traits<T>::acc v);
+template <> __device__ __forceinline__ float narrow<float>(float v) { return v; }
+template <> __device__ __forceinline__ double narrow<double>(double v) { return v; }
+template <> __device__ __forceinline__ bf16_t narrow<bf16_t>(float v) { bf16_t r; r.bits = narrow_bf16_bits(v); return r; }
+template <> __device__ __forceinline__ f16_t narrow<f16_t>(float v) { f16_t r; r.bits = narrow_f16_bits(v); return r; }
+
+// The GEMM epilogue: one narrowing per reference op in the chain
+//   matmul (ops/ops.c:6838) -> bias add (ops/ops.c:162) -> grad accumulation (ops/ops.c:6785).
+template <typename T>
+__device__ __forceinline__ T finish(typename traits<T>::acc acc, bool has_bias, T bias, bool accumulate, T old) {
+    T y = narrow<T>(acc);
+    if (has_bias) y = narrow<T>(widen(y) + widen(bias));
+    if (accumulate) y = narrow<T>(widen(old) + widen(y));
+    return y;
+}
+
+}  // namespace rp
+
+#define RP_DISPATCH_DTYPE(dtype, ...)                                              \
+    switch (dtype) {                                                               \
+        case RP_DTYPE_FLOAT32:  { using T = float;       __VA_ARGS__; break; }     \
+        case RP_DTYPE_FLOAT64:  { using T = double;      __VA_ARGS__; break; }     \
+        case RP_DTYPE_FLOAT16:  { using T = rp::f16_t;   __VA_ARGS__; break; }     \
+        case RP_DTYPE_BFLOAT16: { using T = rp::bf16_t;  __VA_ARGS__; break; }     \
+        default: rp::set_error("unsupported dtype %d", (int)(dtype)); return -1;   \
+    }

@@ -1,0 +1,545 @@
+// Element-wise, row-wise and reduction entry points that BASELINE's configs run
+// around the GEMMs: add / broadcasting add, scalar multiply, relu and softmax
+// with their VJPs, strided gather, reductions, fill / convert, and the
+// on-device bias gradient and cross-entropy.  16-bit dtypes compute in fp32
+// and narrow once with the reference's rounding, like the reference's host
+// path (functional/functional.c:10-56).
+#include "rp_common.h"
+
+#include <cfloat>
+
+namespace rp {
+
+static constexpr int kThreads = 256;
+static constexpr int kMaxDims = 8;
+
+static inline unsigned grid_for(size_t n, int threads = kThreads, size_t cap = 1u << 20) {
+    size_t b = (n + threads - 1) / threads;
+    if (b < 1) b = 1;
+    if (b > cap) b = cap;
+    return (unsigned)b;
+}
+
+// ---- flat maps ----------------------------------------------------------------
+template <typename T>
+__global__ void add_kernel(T* out, const T* x1, const T* x2, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        out[i] = narrow<T>(widen(x1[i]) + widen(x2[i]));
+}
+
+template <typename T>
+__global__ void mul_scalar_kernel(T* out, const T* x, typename traits<T>::acc s, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        out[i] = narrow<T>(widen(x[i]) * s);
+}
+
+template <typename T>
+__global__ void relu_kernel(T* out, const T* x, size_t n) {
+    using A = typename traits<T>::acc;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        A v = widen(x[i]);
+        out[i] = narrow<T>(v > (A)0 ? v : (A)0);
+    }
+}
+
+template <typename T>
+__global__ void backwards_relu_kernel(const T* gc, const T* x, T* gx, size_t n) {
+    using A = typename traits<T>::acc;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        gx[i] = narrow<T>(widen(x[i]) > (A)0 ? widen(gc[i]) : (A)0);
+}
+
+template <typename T>
+__global__ void fill_kernel(T* p, T v, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
+// dtype conversion pivots through fp32 like the reference (core/tensor_host.c:130-207),
+// except float64 <-> float64 / float32 which are direct.
+template <typename D, typename S>
+__global__ void convert_kernel(D* dst, const S* src, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        auto w = widen(src[i]);
+        dst[i] = narrow<D>((typename traits<D>::acc)w);
+    }
+}
+
+// ---- broadcasting add ------------------------------------------------------------
+struct StridedArgs {
+    int ndim;
+    int shape[kMaxDims];
+    long long s1[kMaxDims];
+    long long s2[kMaxDims];
+};
+
+template <typename T>
+__global__ void add_strided_kernel(T* out, const T* x1, const T* x2, StridedArgs a, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        size_t rem = i;
+        long long i1 = 0, i2 = 0;
+        for (int d = a.ndim - 1; d >= 0; d--) {
+            size_t c = rem % (size_t)a.shape[d];
+            rem /= (size_t)a.shape[d];
+            i1 += (long long)c * a.s1[d];
+            i2 += (long long)c * a.s2[d];
+        }
+        out[i] = narrow<T>(widen(x1[i1]) + widen(x2[i2]));
+    }
+}
+
+// the Linear case: [rows, cols] dense + [cols]
+template <typename T>
+__global__ void add_row_vector_kernel(T* out, const T* x, const T* v, size_t n, int cols) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        out[i] = narrow<T>(widen(x[i]) + widen(v[i % (size_t)cols]));
+}
+
+struct GatherArgs {
+    int ndim;
+    int shape[kMaxDims];
+    long long strides[kMaxDims];
+};
+
+template <typename T>
+__global__ void gather_kernel(T* out, const T* in, GatherArgs a, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        size_t rem = i;
+        long long off = 0;
+        for (int d = a.ndim - 1; d >= 0; d--) {
+            off += (long long)(rem % (size_t)a.shape[d]) * a.strides[d];
+            rem /= (size_t)a.shape[d];
+        }
+        out[i] = in[off];
+    }
+}
+
+// ---- softmax family ----------------------------------------------------------------
+// inner == 1: one 64-lane wave per row, lanes stride the row, wave reductions
+// by DPP-free shuffles.  Otherwise one thread per (outer, inner) pair walks
+// its row serially (the reference device kernel's shape,
+// functional/functional_device.cu:1486-1508).
+template <typename A>
+__device__ __forceinline__ A wave_max(A v) {
+    for (int o = 32; o > 0; o >>= 1) { A t = __shfl_xor(v, o, 64); v = t > v ? t : v; }
+    return v;
+}
+template <typename A>
+__device__ __forceinline__ A wave_sum(A v) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float rp_exp(float x) { return expf(x); }
+__device__ __forceinline__ double rp_exp(double x) { return exp(x); }
+__device__ __forceinline__ float rp_log(float x) { return logf(x); }
+__device__ __forceinline__ double rp_log(double x) { return log(x); }
+template <typename A> __device__ __forceinline__ A lowest();
+template <> __device__ __forceinline__ float lowest<float>() { return -FLT_MAX; }
+template <> __device__ __forceinline__ double lowest<double>() { return -DBL_MAX; }
+
+template <typename T, bool LOG>
+__global__ void softmax_rows_kernel(T* out, const T* x, size_t rows, size_t dim) {
+    using A = typename traits<T>::acc;
+    int lane = threadIdx.x & 63;
+    size_t wave = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    size_t nwaves = ((size_t)gridDim.x * blockDim.x) >> 6;
+    for (size_t r = wave; r < rows; r += nwaves) {
+        const T* xr = x + r * dim;
+        T* orow = out + r * dim;
+        A mx = lowest<A>();
+        for (size_t d = lane; d < dim; d += 64) { A v = widen(xr[d]); mx = v > mx ? v : mx; }
+        mx = wave_max(mx);
+        A sum = 0;
+        for (size_t d = lane; d < dim; d += 64) sum += rp_exp(widen(xr[d]) - mx);
+        sum = wave_sum(sum);
+        if (LOG) {
+            A lse = rp_log(sum);
+            for (size_t d = lane; d < dim; d += 64) orow[d] = narrow<T>(widen(xr[d]) - mx - lse);
+        } else {
+            for (size_t d = lane; d < dim; d += 64) orow[d] = narrow<T>(rp_exp(widen(xr[d]) - mx) / sum);
+        }
+    }
+}
+
+template <typename T, bool LOG>
+__global__ void softmax_strided_kernel(T* out, const T* x, size_t outer, size_t dim, size_t inner) {
+    using A = typename traits<T>::acc;
+    size_t n = outer * inner;
+    for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (size_t)gridDim.x * blockDim.x) {
+        size_t base = (t / inner) * dim * inner + (t % inner);
+        A mx = lowest<A>();
+        for (size_t d = 0; d < dim; d++) { A v = widen(x[base + d * inner]); mx = v > mx ? v : mx; }
+        A sum = 0;
+        for (size_t d = 0; d < dim; d++) sum += rp_exp(widen(x[base + d * inner]) - mx);
+        if (LOG) {
+            A lse = rp_log(sum);
+            for (size_t d = 0; d < dim; d++) out[base + d * inner] = narrow<T>(widen(x[base + d * inner]) - mx - lse);
+        } else {
+            for (size_t d = 0; d < dim; d++) out[base + d * inner] = narrow<T>(rp_exp(widen(x[base + d * inner]) - mx) / sum);
+        }
+    }
+}
+
+template <typename T>
+__global__ void backwards_softmax_rows_kernel(const T* gc, const T* y, T* gx, size_t rows, size_t dim) {
+    using A = typename traits<T>::acc;
+    int lane = threadIdx.x & 63;
+    size_t wave = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    size_t nwaves = ((size_t)gridDim.x * blockDim.x) >> 6;
+    for (size_t r = wave; r < rows; r += nwaves) {
+        const T* g = gc + r * dim;
+        const T* s = y + r * dim;
+        A dot = 0;
+        for (size_t d = lane; d < dim; d += 64) dot += widen(g[d]) * widen(s[d]);
+        dot = wave_sum(dot);
+        for (size_t d = lane; d < dim; d += 64) gx[r * dim + d] = narrow<T>(widen(s[d]) * (widen(g[d]) - dot));
+    }
+}
+
+template <typename T>
+__global__ void backwards_softmax_strided_kernel(const T* gc, const T* y, T* gx, size_t outer, size_t dim, size_t inner) {
+    using A = typename traits<T>::acc;
+    size_t n = outer * inner;
+    for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (size_t)gridDim.x * blockDim.x) {
+        size_t base = (t / inner) * dim * inner + (t % inner);
+        A dot = 0;
+        for (size_t d = 0; d < dim; d++) dot += widen(gc[base + d * inner]) * widen(y[base + d * inner]);
+        for (size_t d = 0; d < dim; d++)
+            gx[base + d * inner] = narrow<T>(widen(y[base + d * inner]) * (widen(gc[base + d * inner]) - dot));
+    }
+}
+
+// ---- reductions ----------------------------------------------------------------------
+// Deterministic two-level sum: each block sums a contiguous slab (threads
+// stride it, then a fixed-order LDS tree); block partials land in a
+// file-scope array and the block that finishes last adds them in index order.
+// Calls that overlap on one device would share the array: the library's
+// single-stream ordering keeps them apart.
+static constexpr int kMaxPartials = 1024;
+__device__ double g_partials[kMaxPartials];
+__device__ unsigned int g_partial_count;
+
+template <typename T>
+__global__ void sum_all_kernel(T* out, const T* x, size_t n, double scale) {
+    using A = typename traits<T>::acc;
+    __shared__ A red[kThreads];
+    __shared__ bool last;
+    size_t per_block = (n + gridDim.x - 1) / gridDim.x;
+    size_t lo = (size_t)blockIdx.x * per_block;
+    size_t hi = lo + per_block < n ? lo + per_block : n;
+    A s = 0;
+    for (size_t i = lo + threadIdx.x; i < hi; i += blockDim.x) s += widen(x[i]);
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int o = kThreads / 2; o > 0; o >>= 1) {
+        if ((int)threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        g_partials[blockIdx.x] = (double)red[0];
+        __threadfence();
+        unsigned int done = atomicAdd(&g_partial_count, 1u);
+        last = (done == gridDim.x - 1);
+    }
+    __syncthreads();
+    if (last && threadIdx.x == 0) {
+        __threadfence();
+        A total = 0;
+        for (unsigned b = 0; b < gridDim.x; b++) total += (A)((volatile double*)g_partials)[b];
+        if (scale != 1.0) total = (A)(total / (A)scale);
+        out[0] = narrow<T>(total);
+        g_partial_count = 0;
+    }
+}
+
+// reduce the middle axis of [outer, dim, inner]; one thread per output, serial in dim
+template <typename T>
+__global__ void sum_dim_kernel(T* out, const T* x, size_t outer, size_t dim, size_t inner) {
+    using A = typename traits<T>::acc;
+    size_t n = outer * inner;
+    for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (size_t)gridDim.x * blockDim.x) {
+        size_t base = (t / inner) * dim * inner + (t % inner);
+        A s = 0;
+        for (size_t d = 0; d < dim; d++) s += widen(x[base + d * inner]);
+        out[t] = narrow<T>(s);
+    }
+}
+
+// Linear's bias gradient: out[j] = sum_i grad[i, j], rows added top to bottom
+// in the accumulate type — the order the reference's host loop produces
+// (ops/ops.c:7048-7061).  Threads of a block own adjacent columns, so every
+// row read is one coalesced segment.
+template <typename T>
+__global__ void reduce_rows_kernel(T* out, const T* g, int rows, int cols, int accumulate) {
+    using A = typename traits<T>::acc;
+    int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= cols) return;
+    A s = 0;
+    const T* p = g + j;
+    int i = 0;
+    for (; i + 4 <= rows; i += 4) {
+        A v0 = widen(p[(size_t)(i + 0) * cols]);
+        A v1 = widen(p[(size_t)(i + 1) * cols]);
+        A v2 = widen(p[(size_t)(i + 2) * cols]);
+        A v3 = widen(p[(size_t)(i + 3) * cols]);
+        s += v0; s += v1; s += v2; s += v3;
+    }
+    for (; i < rows; i++) s += widen(p[(size_t)i * cols]);
+    T r = narrow<T>(s);
+    if (accumulate) r = narrow<T>(widen(out[j]) + widen(r));
+    out[j] = r;
+}
+
+// ---- cross-entropy ----------------------------------------------------------------------
+// One block.  Threads stride the batch; each computes its row's log-softmax
+// and softmax serially (class counts are small), writes the scaled gradient
+// and leaves -logp[target] in global scratch; thread 0 then adds those in
+// batch order in fp64, as the reference's host loop does (ops/ops.c:5342-5352).
+template <typename T>
+__global__ void cross_entropy_kernel(T* loss, T* grad, const T* logits, const int* targets,
+                                     int batch, int classes, T upstream, double* nll_scratch) {
+    for (int b = threadIdx.x; b < batch; b += blockDim.x) {
+        const T* row = logits + (size_t)b * classes;
+        T mx = lowest<T>();
+        for (int c = 0; c < classes; c++) mx = row[c] > mx ? row[c] : mx;
+        T sum = 0;
+        for (int c = 0; c < classes; c++) sum += rp_exp(row[c] - mx);
+        T lse = rp_log(sum);
+        int t = targets[b];
+        bool valid = (t >= 0 && t < classes);      // callers validate; a bad index poisons the loss instead of reading out of bounds
+        nll_scratch[b] = valid ? -(double)(row[t] - mx - lse) : (double)NAN;
+        if (grad) {
+            T sc = (T)1 / (T)batch;
+            for (int c = 0; c < classes; c++) {
+                T p = rp_exp(row[c] - mx) / sum;
+                if (c == t) p -= (T)1;
+                p *= sc;
+                grad[(size_t)b * classes + c] = p * upstream;
+            }
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0 && loss) {
+        double s = 0.0;
+        for (int b = 0; b < batch; b++) s += nll_scratch[b];
+        if (sizeof(T) == 8) loss[0] = (T)(s / (double)batch);
+        else { float f = (float)s; f /= (float)batch; loss[0] = (T)f; }
+    }
+}
+
+}  // namespace rp
+
+using namespace rp;
+
+#define RP_REQUIRE(cond, name)                                              \
+    do { if (!(cond)) { set_error("%s: invalid argument", name); return -1; } } while (0)
+
+// Host-side narrowing of a fill value with the same bit rules as the device.
+template <typename T> static T host_narrow(double value);
+template <> double host_narrow<double>(double value) { return value; }
+template <> float host_narrow<float>(double value) { return (float)value; }
+template <> bf16_t host_narrow<bf16_t>(double value) {
+    float f = (float)value;
+    uint32_t w;
+    __builtin_memcpy(&w, &f, 4);
+    bf16_t r;
+    r.bits = (uint16_t)((w >> 16) + ((w >> 15) & 1u));
+    return r;
+}
+template <> f16_t host_narrow<f16_t>(double value) {
+    float f = (float)value;
+    uint32_t w;
+    __builtin_memcpy(&w, &f, 4);
+    uint32_t s = (w >> 16) & 0x8000u, e32 = (w >> 23) & 0xFFu, f23 = w & 0x7FFFFFu;
+    int e = (int)e32 - 112;
+    f16_t r;
+    if (e32 == 0xFFu) r.bits = (uint16_t)(f23 ? (s | 0x7C00u | (f23 >> 13) | 1u) : (s | 0x7C00u));
+    else if (e <= 0) {
+        if (e < -10) r.bits = (uint16_t)s;
+        else { f23 |= 0x800000u; int sh = 14 - e; r.bits = (uint16_t)((s | (f23 >> sh)) + ((f23 >> (sh - 1)) & 1u)); }
+    } else if (e >= 0x1F) r.bits = (uint16_t)(s | 0x7C00u);
+    else r.bits = (uint16_t)((s | ((uint32_t)e << 10) | (f23 >> 13)) + ((f23 >> 12) & 1u));
+    return r;
+}
+
+template <typename D>
+static int convert_from(void* dst, const void* src, int src_dtype, size_t size) {
+    unsigned blocks = grid_for(size);
+    switch (src_dtype) {
+        case RP_DTYPE_FLOAT32:  hipLaunchKernelGGL((convert_kernel<D, float>), dim3(blocks), dim3(kThreads), 0, current_stream(), (D*)dst, (const float*)src, size); break;
+        case RP_DTYPE_FLOAT64:  hipLaunchKernelGGL((convert_kernel<D, double>), dim3(blocks), dim3(kThreads), 0, current_stream(), (D*)dst, (const double*)src, size); break;
+        case RP_DTYPE_FLOAT16:  hipLaunchKernelGGL((convert_kernel<D, f16_t>), dim3(blocks), dim3(kThreads), 0, current_stream(), (D*)dst, (const f16_t*)src, size); break;
+        case RP_DTYPE_BFLOAT16: hipLaunchKernelGGL((convert_kernel<D, bf16_t>), dim3(blocks), dim3(kThreads), 0, current_stream(), (D*)dst, (const bf16_t*)src, size); break;
+        default: set_error("rp_hip_convert: unsupported source dtype %d", src_dtype); return -1;
+    }
+    return check_launch("convert_kernel") ? 0 : -1;
+}
+
+extern "C" {
+
+int add_kernel_device(void* out, const void* x1, const void* x2, size_t size, int dtype) {
+    RP_REQUIRE(out && x1 && x2 && size, "add_kernel_device");
+    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(add_kernel<T>, dim3(grid_for(size)), dim3(kThreads), 0, current_stream(),
+                                               (T*)out, (const T*)x1, (const T*)x2, size));
+    return check_launch("add_kernel") ? 0 : -1;
+}
+
+int add_strided_kernel_device(void* out, const void* x1, const void* x2, int ndim, const int* out_shape,
+                              const int* x1_strides, const int* x2_strides, size_t out_size, int dtype) {
+    RP_REQUIRE(out && x1 && x2 && out_shape && x1_strides && x2_strides && out_size && ndim > 0, "add_strided_kernel_device");
+    if (ndim > kMaxDims) { set_error("add_strided_kernel_device: more than %d dimensions", kMaxDims); return -1; }
+    // [rows, cols] dense + row vector: the Linear bias add
+    if (ndim == 2 && x1_strides[0] == out_shape[1] && x1_strides[1] == 1 && x2_strides[0] == 0 && x2_strides[1] == 1) {
+        RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(add_row_vector_kernel<T>, dim3(grid_for(out_size)), dim3(kThreads), 0,
+                                                   current_stream(), (T*)out, (const T*)x1, (const T*)x2, out_size, out_shape[1]));
+        return check_launch("add_row_vector_kernel") ? 0 : -1;
+    }
+    StridedArgs a;
+    a.ndim = ndim;
+    for (int d = 0; d < ndim; d++) { a.shape[d] = out_shape[d]; a.s1[d] = x1_strides[d]; a.s2[d] = x2_strides[d]; }
+    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(add_strided_kernel<T>, dim3(grid_for(out_size)), dim3(kThreads), 0, current_stream(),
+                                               (T*)out, (const T*)x1, (const T*)x2, a, out_size));
+    return check_launch("add_strided_kernel") ? 0 : -1;
+}
+
+int mul_scalar_kernel_device(void* out, const void* x, const void* scalar, size_t size, int dtype) {
+    RP_REQUIRE(out && x && scalar && size, "mul_scalar_kernel_device");
+    RP_DISPATCH_DTYPE(dtype, {
+        using A = typename traits<T>::acc;
+        A s = *(const A*)scalar;
+        hipLaunchKernelGGL(mul_scalar_kernel<T>, dim3(grid_for(size)), dim3(kThreads), 0, current_stream(), (T*)out, (const T*)x, s, size);
+    });
+    return check_launch("mul_scalar_kernel") ? 0 : -1;
+}
+
+int relu_kernel_device(void* out, const void* x, size_t size, int dtype) {
+    RP_REQUIRE(out && x && size, "relu_kernel_device");
+    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(relu_kernel<T>, dim3(grid_for(size)), dim3(kThreads), 0, current_stream(),
+                                               (T*)out, (const T*)x, size));
+    return check_launch("relu_kernel") ? 0 : -1;
+}
+
+int backwards_relu_device(const void* grad_c, const void* x, void* grad_x, size_t size, int dtype) {
+    RP_REQUIRE(grad_c && x && grad_x && size, "backwards_relu_device");
+    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(backwards_relu_kernel<T>, dim3(grid_for(size)), dim3(kThreads), 0, current_stream(),
+                                               (const T*)grad_c, (const T*)x, (T*)grad_x, size));
+    return check_launch("backwards_relu_kernel") ? 0 : -1;
+}
+
+static int softmax_any(void* out, const void* x, size_t outer, size_t dim, size_t inner, int dtype, bool take_log) {
+    RP_REQUIRE(out && x && outer && dim && inner, "softmax_kernel_device");
+    if (inner == 1) {
+        unsigned blocks = grid_for(outer * 64, kThreads, 1u << 16);
+        RP_DISPATCH_DTYPE(dtype, {
+            if (take_log) hipLaunchKernelGGL((softmax_rows_kernel<T, true>), dim3(blocks), dim3(kThreads), 0, current_stream(), (T*)out, (const T*)x, outer, dim);
+            else          hipLaunchKernelGGL((softmax_rows_kernel<T, false>), dim3(blocks), dim3(kThreads), 0, current_stream(), (T*)out, (const T*)x, outer, dim);
+        });
+    } else {
+        unsigned blocks = grid_for(outer * inner);
+        RP_DISPATCH_DTYPE(dtype, {
+            if (take_log) hipLaunchKernelGGL((softmax_strided_kernel<T, true>), dim3(blocks), dim3(kThreads), 0, current_stream(), (T*)out, (const T*)x, outer, dim, inner);
+            else          hipLaunchKernelGGL((softmax_strided_kernel<T, false>), dim3(blocks), dim3(kThreads), 0, current_stream(), (T*)out, (const T*)x, outer, dim, inner);
+        });
+    }
+    return check_launch("softmax kernel") ? 0 : -1;
+}
+
+int softmax_kernel_device(void* out, const void* x, size_t outer_size, size_t dim_size, size_t inner_size, int dtype) {
+    return softmax_any(out, x, outer_size, dim_size, inner_size, dtype, false);
+}
+
+int log_softmax_kernel_device(void* out, const void* x, size_t outer_size, size_t dim_size, size_t inner_size, int dtype) {
+    return softmax_any(out, x, outer_size, dim_size, inner_size, dtype, true);
+}
+
+int backwards_softmax_device(const void* grad_c, const void* softmax_out, void* grad_x,
+                             size_t outer_size, size_t dim_size, size_t inner_size, int dtype) {
+    RP_REQUIRE(grad_c && softmax_out && grad_x && outer_size && dim_size && inner_size, "backwards_softmax_device");
+    if (inner_size == 1) {
+        unsigned blocks = grid_for(outer_size * 64, kThreads, 1u << 16);
+        RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(backwards_softmax_rows_kernel<T>, dim3(blocks), dim3(kThreads), 0, current_stream(),
+                                                   (const T*)grad_c, (const T*)softmax_out, (T*)grad_x, outer_size, dim_size));
+    } else {
+        RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(backwards_softmax_strided_kernel<T>, dim3(grid_for(outer_size * inner_size)), dim3(kThreads), 0,
+                                                   current_stream(), (const T*)grad_c, (const T*)softmax_out, (T*)grad_x,
+                                                   outer_size, dim_size, inner_size));
+    }
+    return check_launch("backwards_softmax kernel") ? 0 : -1;
+}
+
+int contiguous_copy_kernel_device(void* out, const void* in, int ndim, int* shape, int* strides, size_t size, int dtype) {
+    RP_REQUIRE(out && in && shape && strides && size && ndim > 0, "contiguous_copy_kernel_device");
+    if (ndim > kMaxDims) { set_error("contiguous_copy_kernel_device: more than %d dimensions", kMaxDims); return -1; }
+    GatherArgs a;
+    a.ndim = ndim;
+    for (int d = 0; d < ndim; d++) { a.shape[d] = shape[d]; a.strides[d] = strides[d]; }
+    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(gather_kernel<T>, dim3(grid_for(size)), dim3(kThreads), 0, current_stream(),
+                                               (T*)out, (const T*)in, a, size));
+    return check_launch("gather_kernel") ? 0 : -1;
+}
+
+static int sum_all_any(void* out, const void* x, size_t size, int dtype, double scale) {
+    RP_REQUIRE(out && x && size, "sum_all_kernel_device");
+    unsigned blocks = grid_for(size, kThreads * 16, kMaxPartials);
+    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(sum_all_kernel<T>, dim3(blocks), dim3(kThreads), 0, current_stream(),
+                                               (T*)out, (const T*)x, size, scale));
+    return check_launch("sum_all_kernel") ? 0 : -1;
+}
+
+int sum_all_kernel_device(void* out, const void* x, size_t size, int dtype) { return sum_all_any(out, x, size, dtype, 1.0); }
+
+int mean_all_kernel_device(void* out, const void* x, size_t size, int dtype) { return sum_all_any(out, x, size, dtype, (double)size); }
+
+int sum_dim_kernel_device(void* out, const void* x, size_t outer_size, size_t dim_size, size_t inner_size, int dtype) {
+    RP_REQUIRE(out && x && outer_size && dim_size && inner_size, "sum_dim_kernel_device");
+    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(sum_dim_kernel<T>, dim3(grid_for(outer_size * inner_size)), dim3(kThreads), 0, current_stream(),
+                                               (T*)out, (const T*)x, outer_size, dim_size, inner_size));
+    return check_launch("sum_dim_kernel") ? 0 : -1;
+}
+
+int rp_hip_fill(void* ptr, double value, size_t size, int dtype) {
+    RP_REQUIRE(ptr && size, "rp_hip_fill");
+    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(fill_kernel<T>, dim3(grid_for(size)), dim3(kThreads), 0, current_stream(),
+                                               (T*)ptr, host_narrow<T>(value), size));
+    return check_launch("fill_kernel") ? 0 : -1;
+}
+
+int rp_hip_convert(void* dst, int dst_dtype, const void* src, int src_dtype, size_t size) {
+    RP_REQUIRE(dst && src && size, "rp_hip_convert");
+    RP_DISPATCH_DTYPE(dst_dtype, return convert_from<T>(dst, src, src_dtype, size));
+    return -1;
+}
+
+int rp_hip_reduce_rows(void* out, const void* grad, int rows, int cols, int accumulate, int dtype) {
+    RP_REQUIRE(out && grad && rows > 0 && cols > 0, "rp_hip_reduce_rows");
+    unsigned blocks = (unsigned)((cols + 63) / 64);
+    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(reduce_rows_kernel<T>, dim3(blocks), dim3(64), 0, current_stream(),
+                                               (T*)out, (const T*)grad, rows, cols, accumulate));
+    return check_launch("reduce_rows_kernel") ? 0 : -1;
+}
+
+int rp_hip_cross_entropy_mean(void* loss_out, void* grad_logits, const void* logits, const int* targets,
+                              int batch, int classes, double upstream, int dtype) {
+    RP_REQUIRE(logits && targets && batch > 0 && classes > 0 && (loss_out || grad_logits), "rp_hip_cross_entropy_mean");
+    if (dtype != RP_DTYPE_FLOAT32 && dtype != RP_DTYPE_FLOAT64) {
+        set_error("rp_hip_cross_entropy_mean: float32 and float64 only");
+        return -1;
+    }
+    // scratch: batch doubles for the per-row losses, from the caching pool
+    void* scratch = nullptr;
+    if (rp_hip_malloc(&scratch, (size_t)batch * 8) != 0) return -1;
+    double* nll = (double*)scratch;
+    bool ok = true;
+    {
+        if (dtype == RP_DTYPE_FLOAT32)
+            hipLaunchKernelGGL(cross_entropy_kernel<float>, dim3(1), dim3(kThreads), 0, current_stream(), (float*)loss_out, (float*)grad_logits,
+                               (const float*)logits, targets, batch, classes, (float)upstream, nll);
+        else
+            hipLaunchKernelGGL(cross_entropy_kernel<double>, dim3(1), dim3(kThreads), 0, current_stream(), (double*)loss_out, (double*)grad_logits,
+                               (const double*)logits, targets, batch, classes, upstream, nll);
+        ok = check_launch("cross_entropy_kernel");
+    }
+    rp_hip_free(scratch);
+    return ok ? 0 : -1;
+}
+
+}  // extern "C"

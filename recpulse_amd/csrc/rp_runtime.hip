@@ -1,0 +1,228 @@
+// Device runtime shim of the C ABI: device selection, a caching allocator,
+// copies, streams, events and the error text.
+#include "rp_common.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+namespace rp {
+
+static thread_local char g_error[512] = "";
+static thread_local hipStream_t g_stream = nullptr;
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    if (getenv("RP_HIP_VERBOSE")) fprintf(stderr, "rp_hip: %s\n", g_error);
+}
+
+hipStream_t current_stream() { return g_stream; }
+
+bool check_hip(hipError_t e, const char* what) {
+    if (e == hipSuccess) return true;
+    set_error("%s: %s", what, hipGetErrorString(e));
+    return false;
+}
+
+bool check_launch(const char* what) { return check_hip(hipGetLastError(), what); }
+
+// ---- caching allocator ------------------------------------------------------
+// The reference allocates and zero-fills device memory for every op output
+// (core/tensor_device.cu:44-46) and frees it when the tensor dies; hipMalloc /
+// hipFree cost tens of microseconds and hipFree synchronises the device, which
+// would dominate the small-GEMM configs.  Freed blocks are therefore kept per
+// device in size-keyed lists and reused.
+struct Pool {
+    std::mutex mu;
+    std::unordered_map<void*, std::pair<int, size_t>> live;       // ptr -> (device, rounded size)
+    std::map<std::pair<int, size_t>, std::vector<void*>> free_lists;
+    bool enabled = true;
+    Pool() { const char* e = getenv("RP_HIP_NO_CACHE"); enabled = !(e && e[0] == '1'); }
+};
+
+static Pool& pool() { static Pool* p = new Pool(); return *p; }   // leaked on purpose: outlives HIP teardown
+
+static size_t round_size(size_t bytes) {
+    if (bytes == 0) bytes = 1;
+    if (bytes <= (1u << 20)) return (bytes + 511) & ~(size_t)511;          // 512 B steps up to 1 MiB
+    return (bytes + ((1u << 21) - 1)) & ~(size_t)((1u << 21) - 1);         // 2 MiB steps above
+}
+
+// Byte fill: a 16-byte aligned body written as uint4 plus scalar head and tail.
+__global__ void fill_bytes_kernel(unsigned char* p, unsigned char v, size_t bytes) {
+    size_t head = (16 - ((uintptr_t)p & 15)) & 15;
+    if (head > bytes) head = bytes;
+    size_t body = (bytes - head) / 16;
+    size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t nth = (size_t)gridDim.x * blockDim.x;
+    uint32_t w = 0x01010101u * v;
+    uint4 w4 = make_uint4(w, w, w, w);
+    uint4* q = (uint4*)(p + head);
+    for (size_t i = tid; i < body; i += nth) q[i] = w4;
+    size_t tail0 = head + body * 16;
+    for (size_t i = tid; i < head; i += nth) p[i] = v;
+    for (size_t i = tail0 + tid; i < bytes; i += nth) p[i] = v;
+}
+
+}  // namespace rp
+
+using namespace rp;
+
+extern "C" {
+
+int rp_hip_device_count(int* count) {
+    if (!count) { set_error("rp_hip_device_count: null argument"); return -1; }
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) { (void)hipGetLastError(); n = 0; }       // no device is an answer, not a failure
+    *count = n;
+    return 0;
+}
+
+int rp_hip_set_device(int device_id) {
+    return check_hip(hipSetDevice(device_id), "hipSetDevice") ? 0 : -1;
+}
+
+int rp_hip_get_device(int* device_id) {
+    if (!device_id) { set_error("rp_hip_get_device: null argument"); return -1; }
+    return check_hip(hipGetDevice(device_id), "hipGetDevice") ? 0 : -1;
+}
+
+int rp_hip_malloc(void** ptr, size_t bytes) {
+    if (!ptr) { set_error("rp_hip_malloc: null argument"); return -1; }
+    *ptr = nullptr;
+    int dev = 0;
+    if (!check_hip(hipGetDevice(&dev), "hipGetDevice")) return -1;
+    Pool& p = pool();
+    size_t sz = round_size(bytes);
+    if (p.enabled) {
+        std::lock_guard<std::mutex> lk(p.mu);
+        auto it = p.free_lists.find({dev, sz});
+        if (it != p.free_lists.end() && !it->second.empty()) {
+            *ptr = it->second.back();
+            it->second.pop_back();
+            p.live[*ptr] = {dev, sz};
+            return 0;
+        }
+    }
+    void* d = nullptr;
+    hipError_t e = hipMalloc(&d, sz);
+    if (e != hipSuccess && p.enabled) {            // out of memory: give cached blocks back and retry once
+        (void)hipGetLastError();
+        rp_hip_empty_cache();
+        e = hipMalloc(&d, sz);
+    }
+    if (!check_hip(e, "hipMalloc")) return -1;
+    {
+        std::lock_guard<std::mutex> lk(p.mu);
+        p.live[d] = {dev, sz};
+    }
+    *ptr = d;
+    return 0;
+}
+
+int rp_hip_free(void* ptr) {
+    if (!ptr) return 0;
+    Pool& p = pool();
+    {
+        std::lock_guard<std::mutex> lk(p.mu);
+        auto it = p.live.find(ptr);
+        if (it == p.live.end()) { set_error("rp_hip_free: pointer %p was not allocated by rp_hip_malloc", ptr); return -1; }
+        auto key = it->second;
+        p.live.erase(it);
+        if (p.enabled) { p.free_lists[key].push_back(ptr); return 0; }
+    }
+    return check_hip(hipFree(ptr), "hipFree") ? 0 : -1;
+}
+
+int rp_hip_empty_cache(void) {
+    Pool& p = pool();
+    std::vector<void*> blocks;
+    {
+        std::lock_guard<std::mutex> lk(p.mu);
+        for (auto& kv : p.free_lists) for (void* b : kv.second) blocks.push_back(b);
+        p.free_lists.clear();
+    }
+    bool ok = true;
+    for (void* b : blocks) ok = check_hip(hipFree(b), "hipFree") && ok;
+    return ok ? 0 : -1;
+}
+
+// A fill kernel rather than hipMemsetAsync, so the call can be captured into a
+// HIP graph by callers that record their step.
+int rp_hip_memset(void* ptr, int value, size_t bytes) {
+    if (!ptr && bytes) { set_error("rp_hip_memset: null pointer"); return -1; }
+    if (!bytes) return 0;
+    size_t per_block = (size_t)256 * 16;
+    size_t blocks = (bytes + per_block - 1) / per_block;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(rp::fill_bytes_kernel, dim3((unsigned)blocks), dim3(256), 0, current_stream(),
+                       (unsigned char*)ptr, (unsigned char)value, bytes);
+    return check_launch("fill_bytes_kernel") ? 0 : -1;
+}
+
+// Host copies block until the data has landed, like the reference's cudaMemcpy
+// calls (core/tensor_device.cu:295-531); device-to-device copies are stream-ordered.
+int rp_hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+    if (!bytes) return 0;
+    if (!dst || !src) { set_error("rp_hip_memcpy_h2d: null pointer"); return -1; }
+    if (!check_hip(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, current_stream()), "hipMemcpy H2D")) return -1;
+    return check_hip(hipStreamSynchronize(current_stream()), "hipStreamSynchronize") ? 0 : -1;
+}
+
+int rp_hip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+    if (!bytes) return 0;
+    if (!dst || !src) { set_error("rp_hip_memcpy_d2h: null pointer"); return -1; }
+    if (!check_hip(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, current_stream()), "hipMemcpy D2H")) return -1;
+    return check_hip(hipStreamSynchronize(current_stream()), "hipStreamSynchronize") ? 0 : -1;
+}
+
+int rp_hip_memcpy_d2d(void* dst, const void* src, size_t bytes) {
+    if (!bytes) return 0;
+    if (!dst || !src) { set_error("rp_hip_memcpy_d2d: null pointer"); return -1; }
+    return check_hip(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, current_stream()), "hipMemcpy D2D") ? 0 : -1;
+}
+
+int rp_hip_synchronize(void) {
+    return check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize") ? 0 : -1;
+}
+
+const char* rp_hip_last_error(void) { return g_error; }
+
+int rp_hip_set_stream(void* stream) { g_stream = (hipStream_t)stream; return 0; }
+void* rp_hip_get_stream(void) { return (void*)g_stream; }
+
+int rp_hip_event_create(void** event) {
+    if (!event) { set_error("rp_hip_event_create: null argument"); return -1; }
+    hipEvent_t ev;
+    if (!check_hip(hipEventCreate(&ev), "hipEventCreate")) return -1;
+    *event = (void*)ev;
+    return 0;
+}
+
+int rp_hip_event_record(void* event) {
+    return check_hip(hipEventRecord((hipEvent_t)event, current_stream()), "hipEventRecord") ? 0 : -1;
+}
+
+int rp_hip_event_synchronize(void* event) {
+    return check_hip(hipEventSynchronize((hipEvent_t)event), "hipEventSynchronize") ? 0 : -1;
+}
+
+int rp_hip_event_elapsed_ms(float* ms, void* start, void* stop) {
+    if (!ms) { set_error("rp_hip_event_elapsed_ms: null argument"); return -1; }
+    return check_hip(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop), "hipEventElapsedTime") ? 0 : -1;
+}
+
+int rp_hip_event_destroy(void* event) {
+    return check_hip(hipEventDestroy((hipEvent_t)event), "hipEventDestroy") ? 0 : -1;
+}
+
+}  // extern "C"

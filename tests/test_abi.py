@@ -1,0 +1,51 @@
+"""The C-ABI library loads and exports every symbol include/rp_hip.h declares (no GPU needed)."""
+import os
+import re
+
+from recpulse_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "rp_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"\b([A-Za-z_][A-Za-z0-9_]*)\s*\([^;{}]*\)\s*;", text)
+
+
+def test_header_declares_the_expected_entry_points():
+    names = _declared()
+    assert len(names) == len(set(names))
+    for must in ("matmul_kernel_device", "rp_hip_gemm_strided_batched", "rp_hip_malloc", "add_strided_kernel_device",
+                 "softmax_kernel_device", "backwards_softmax_device", "rp_hip_reduce_rows"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = capi.lib()
+    for name in _declared():
+        assert hasattr(lib, name), f"{name} declared in rp_hip.h but not exported by librp_hip.so"
+
+
+def test_python_binding_covers_every_declared_symbol():
+    assert set(_declared()) == set(capi.SIGNATURES)
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    lib = capi.lib()
+    assert lib.rp_hip_gemm_strided_batched(None, None, None, None, 1, 1, 1, 1, 0, 1, 1, 0, 1, 1, 0, 1, 1, 0, 0) == -1
+    assert b"null operand" in lib.rp_hip_last_error()
+    assert lib.matmul_kernel_device(None, None, None, 2, 2, 2, 0) == -1
+    assert lib.add_kernel_device(None, None, None, 4, 0) == -1
+    assert lib.rp_hip_free(None) == 0
+
+
+def test_kernel_selection_names():
+    name = capi.gemm_kernel_name
+    assert name(1, 8192, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "mfma16_256x256"
+    assert name(1, 8192, 8192, 8192, (1, 8192), (8192, 1), (8192, 1), capi.F16) == "mfma16_256x256"       # A^T view
+    assert name(1, 8, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "skinny"
+    assert name(1, 128, 784, 256, (784, 1), (256, 1), (256, 1), capi.F32) == "mfma32_128x128"
+    assert name(1, 2048, 2048, 2048, (2048, 1), (2048, 1), (2048, 1), capi.F64) == "mfma64_128x128"
+    assert name(1, 5, 7, 3, (7, 1), (3, 1), (3, 1), capi.F32) == "generic"                                 # odd extents
+    assert name(1, 64, 64, 64, (128, 2), (64, 1), (64, 1), capi.F32) == "generic"                          # no unit stride

@@ -1,0 +1,175 @@
+"""GPU parity of the non-GEMM entry points against the CPU oracle."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import oracle
+from recpulse_amd import capi
+from devhelp import ALL, BF16, F16, F32, F64, NAMES, Dev, rand_storage, scalar_arg
+
+pytestmark = pytest.mark.gpu
+L = capi.lib
+
+
+def _tol(dt):
+    # element-wise ops differ from the oracle only through expf/logf and summation order
+    return {F32: 2e-6, F64: 1e-14, F16: 2e-3, BF16: 1.6e-2}[dt]
+
+
+def _arr(*v):
+    return (ctypes.c_int * len(v))(*[int(x) for x in v])
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_flat_maps_bit_exact(dt):
+    rng = np.random.default_rng(40)
+    for n in (1, 7, 256, 1000, 65537):
+        x = rand_storage(rng, (n,), dt); y = rand_storage(rng, (n,), dt)
+        dx, dy, do = Dev(x, dt), Dev(y, dt), Dev.empty((n,), dt)
+        capi.check(L().add_kernel_device(do.ptr, dx.ptr, dy.ptr, n, dt), "add")
+        assert np.array_equal(do.numpy(), oracle.add(x, y, dt))
+        capi.check(L().mul_scalar_kernel_device(do.ptr, dx.ptr, scalar_arg(0.125, dt), n, dt), "mul_scalar")
+        assert np.array_equal(do.numpy(), oracle.mul_scalar(x, 0.125, dt))
+        capi.check(L().mul_scalar_kernel_device(do.ptr, dx.ptr, scalar_arg(1.0 / 3.0, dt), n, dt), "mul_scalar")
+        assert np.array_equal(do.numpy(), oracle.mul_scalar(x, 1.0 / 3.0, dt))
+        capi.check(L().relu_kernel_device(do.ptr, dx.ptr, n, dt), "relu")
+        assert np.array_equal(do.numpy(), oracle.relu(x, dt))
+        capi.check(L().backwards_relu_device(dy.ptr, dx.ptr, do.ptr, n, dt), "backwards_relu")
+        assert np.array_equal(do.numpy(), oracle.backwards_relu(y, x, dt))
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_broadcasting_add_bit_exact(dt):
+    rng = np.random.default_rng(41)
+    y = rand_storage(rng, (37, 53), dt); b = rand_storage(rng, (53,), dt)
+    dy, db, do = Dev(y, dt), Dev(b, dt), Dev.empty((37, 53), dt)
+    capi.check(L().add_strided_kernel_device(do.ptr, dy.ptr, db.ptr, 2, _arr(37, 53), _arr(53, 1), _arr(0, 1), y.size, dt), "add_strided")
+    assert np.array_equal(do.numpy(), oracle.bias_add(y, b, dt))
+    # general case: [4,1,6] + [5,1] -> [4,5,6]
+    x1 = rand_storage(rng, (4, 1, 6), dt); x2 = rand_storage(rng, (5, 1), dt)
+    d1, d2, d3 = Dev(x1, dt), Dev(x2, dt), Dev.empty((4, 5, 6), dt)
+    capi.check(L().add_strided_kernel_device(d3.ptr, d1.ptr, d2.ptr, 3, _arr(4, 5, 6), _arr(6, 0, 1), _arr(0, 1, 0), 120, dt), "add_strided")
+    assert np.array_equal(d3.numpy(), oracle.add_strided(x1, x2, (4, 5, 6), (6, 0, 1), (0, 1, 0), dt))
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_softmax_family(dt):
+    rng = np.random.default_rng(42)
+    for shape, dim in (((9, 10), -1), ((33, 512), -1), ((3, 17, 5), 1), ((2, 3, 64), -1)):
+        x = oracle.to_storage(rng.normal(0, 2, shape), dt); g = rand_storage(rng, shape, dt)
+        o, d, i = oracle._split(shape, dim)
+        dx, dg, do = Dev(x, dt), Dev(g, dt), Dev.empty(shape, dt)
+        capi.check(L().softmax_kernel_device(do.ptr, dx.ptr, o, d, i, dt), "softmax")
+        y = do.numpy()
+        want = oracle.softmax(x, dt, dim=dim)
+        assert oracle.rel_err(oracle.to_f64(y, dt), oracle.to_f64(want, dt)) <= _tol(dt)
+        capi.check(L().log_softmax_kernel_device(do.ptr, dx.ptr, o, d, i, dt), "log_softmax")
+        assert oracle.rel_err(oracle.to_f64(do.numpy(), dt), oracle.to_f64(oracle.softmax(x, dt, dim=dim, log=True), dt)) <= _tol(dt)
+        dy = Dev(want, dt)
+        capi.check(L().backwards_softmax_device(dg.ptr, dy.ptr, do.ptr, o, d, i, dt), "backwards_softmax")
+        wantg = oracle.backwards_softmax(g, want, dt, dim=dim)
+        assert oracle.rel_err(oracle.to_f64(do.numpy(), dt), oracle.to_f64(wantg, dt)) <= 4 * _tol(dt)
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_contiguous_copy_of_views(dt):
+    rng = np.random.default_rng(43)
+    base = rand_storage(rng, (4, 6, 10), dt)
+    view = base.transpose(2, 0, 1)[2:, :, ::2]
+    strides = [s // base.itemsize for s in view.strides]
+    off = (view.__array_interface__["data"][0] - base.__array_interface__["data"][0])
+    db, do = Dev(base, dt), Dev.empty(view.shape, dt)
+    capi.check(L().contiguous_copy_kernel_device(do.ptr, db.ptr + off, view.ndim, _arr(*view.shape), _arr(*strides), view.size, dt), "contiguous_copy")
+    assert np.array_equal(do.numpy(), view)
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_reductions(dt):
+    rng = np.random.default_rng(44)
+    for n in (1, 100, 4097, 300000):
+        x = rand_storage(rng, (n,), dt)
+        dx, do = Dev(x, dt), Dev.empty((1,), dt)
+        x64 = oracle.to_f64(x, dt)
+        scale = np.abs(x64).sum()
+        capi.check(L().sum_all_kernel_device(do.ptr, dx.ptr, n, dt), "sum_all")
+        got = oracle.to_f64(do.numpy(), dt)[0]
+        unit = {F32: 1e-6, F64: 1e-15, F16: 1e-3, BF16: 8e-3}[dt]
+        assert abs(got - x64.sum()) <= unit * scale + unit * abs(x64.sum()) * 4
+        capi.check(L().mean_all_kernel_device(do.ptr, dx.ptr, n, dt), "mean_all")
+        got = oracle.to_f64(do.numpy(), dt)[0]
+        assert abs(got - x64.mean()) <= (unit * scale + unit * abs(x64.sum()) * 4) / n
+        again = Dev.empty((1,), dt)
+        capi.check(L().mean_all_kernel_device(again.ptr, dx.ptr, n, dt), "mean_all")
+        assert np.array_equal(again.numpy(), do.numpy())        # deterministic
+    x = rand_storage(rng, (3, 50, 7), dt)
+    dx, do = Dev(x, dt), Dev.empty((3, 7), dt)
+    capi.check(L().sum_dim_kernel_device(do.ptr, dx.ptr, 3, 50, 7, dt), "sum_dim")
+    assert oracle.rel_err(oracle.to_f64(do.numpy(), dt), oracle.to_f64(x, dt).sum(1)) <= 8 * _tol(dt)
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_reduce_rows_matches_reference_order_bit_exact(dt):
+    rng = np.random.default_rng(45)
+    for rows, cols in ((1, 1), (256, 10), (256, 256), (37, 131)):
+        g = rand_storage(rng, (rows, cols), dt)
+        dg, do = Dev(g, dt), Dev.empty((cols,), dt)
+        capi.check(L().rp_hip_reduce_rows(do.ptr, dg.ptr, rows, cols, 0, dt), "reduce_rows")
+        want = oracle.reduce_rows(g, dt)
+        assert np.array_equal(do.numpy(), want)
+        capi.check(L().rp_hip_reduce_rows(do.ptr, dg.ptr, rows, cols, 1, dt), "reduce_rows")
+        assert np.array_equal(do.numpy(), oracle.add(want, want, dt))
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_fill_and_convert(dt):
+    rng = np.random.default_rng(46)
+    d = Dev.empty((1000,), dt)
+    capi.check(L().rp_hip_fill(d.ptr, 1.0 / 3.0, 1000, dt), "fill")
+    assert np.array_equal(d.numpy(), oracle.to_storage(np.full(1000, np.float32(1.0 / 3.0) if dt != F64 else 1.0 / 3.0), dt))
+    x = rand_storage(rng, (777,), dt)
+    dx = Dev(x, dt)
+    for dst in ALL:
+        do = Dev.empty((777,), dst)
+        capi.check(L().rp_hip_convert(do.ptr, dst, dx.ptr, dt, 777), "convert")
+        want = oracle.to_storage(oracle.to_f64(x, dt), dst)
+        assert np.array_equal(do.numpy(), want), (dt, dst)
+    buf = Dev.empty((1001,), F32)
+    capi.check(L().rp_hip_fill(buf.ptr, 5.0, 1001, F32), "fill")
+    capi.check(L().rp_hip_memset(buf.ptr + 4, 0, 4 * 999), "memset")
+    got = buf.numpy()
+    assert got[0] == 5.0 and got[-1] == 5.0 and not got[1:-1].any()
+
+
+@pytest.mark.parametrize("dt", [F32, F64], ids=lambda d: NAMES[d])
+def test_cross_entropy(dt):
+    rng = np.random.default_rng(47)
+    for batch, classes in ((256, 10), (7, 3), (1000, 33)):
+        logits = oracle.to_storage(rng.normal(0, 3, (batch, classes)), dt)
+        t = rng.integers(0, classes, batch).astype(np.int32)
+        dl, dt_ = Dev(logits, dt), capi.DeviceBuffer.from_numpy(t)
+        dloss, dgrad = Dev.empty((1,), dt), Dev.empty((batch, classes), dt)
+        capi.check(L().rp_hip_cross_entropy_mean(dloss.ptr, dgrad.ptr, dl.ptr, dt_.ptr, batch, classes, 1.0, dt), "ce")
+        loss, grad = oracle.cross_entropy_mean(logits, t, dt)
+        tolv = 4e-6 if dt == F32 else 1e-13
+        assert abs(float(dloss.numpy()[0]) - float(loss[0])) <= tolv * max(1.0, abs(float(loss[0])))
+        assert oracle.rel_err(dgrad.numpy(), grad) <= tolv
+    bad = capi.DeviceBuffer.from_numpy(np.array([0, 3, 1], dtype=np.int32))
+    lg = Dev(oracle.to_storage(rng.normal(0, 1, (3, 3)), dt), dt)
+    ls = Dev.empty((1,), dt)
+    capi.check(L().rp_hip_cross_entropy_mean(ls.ptr, None, lg.ptr, bad.ptr, 3, 3, 1.0, dt), "ce")
+    assert np.isnan(ls.numpy()[0])
+    assert L().rp_hip_cross_entropy_mean(ls.ptr, None, lg.ptr, bad.ptr, 3, 3, 1.0, BF16) == -1
+
+
+def test_allocator_reuses_blocks_and_reports_errors():
+    a = capi.DeviceBuffer(1000); p = a.ptr
+    a.free()
+    b = capi.DeviceBuffer(900)
+    assert b.ptr == p                       # same 512-byte size class, handed out again
+    assert L().rp_hip_free(ctypes.c_void_p(12345)) == -1
+    assert b"not allocated" in L().rp_hip_last_error()
+    assert capi.device_count() >= 1
+    e0, e1 = capi.Event(), capi.Event()
+    e0.record(); e1.record(); e1.synchronize()
+    assert e0.elapsed_ms(e1) >= 0.0

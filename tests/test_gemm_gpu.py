@@ -1,0 +1,214 @@
+"""GPU parity of the GEMM entry points against the CPU oracle and a float64 oracle.
+
+Every case goes through the C ABI (rp_hip_gemm_strided_batched or
+matmul_kernel_device).  Small cases are compared with the oracle's full
+result; integer-valued cases must match bit for bit.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from recpulse_amd import capi
+from devhelp import ALL, BF16, F16, F32, F64, NAMES, device_gemm, f64_gemm, oracle_gemm, rand_storage, tol
+
+pytestmark = pytest.mark.gpu
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")))
+
+
+def _check(got, a, b, dtype, k, **kw):
+    want = oracle_gemm(a, b, dtype, **kw)
+    want64 = f64_gemm(a, b, dtype, **kw)
+    e_orc = oracle.rel_err(oracle.to_f64(got, dtype), oracle.to_f64(want, dtype))
+    e_64 = oracle.rel_err(oracle.to_f64(got, dtype), want64)
+    assert e_orc <= tol(dtype, k), f"vs oracle {e_orc:.3e} > {tol(dtype, k):.3e}"
+    assert e_64 <= tol(dtype, k), f"vs f64 {e_64:.3e} > {tol(dtype, k):.3e}"
+    return e_orc, e_64
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_reference_known_answers_bit_exact(dt):
+    for key in ("matmul_2x3_3x2", "matmul_identity"):
+        g = GOLD[key]
+        a = oracle.to_storage(np.array(g["a"], dtype=np.float64), dt)
+        b = oracle.to_storage(np.array(g["b"], dtype=np.float64), dt)
+        got = device_gemm(a, b, dt)
+        assert np.array_equal(oracle.to_f64(got, dt), np.array(g["c"], dtype=np.float64)), key
+    for key in ("backward_a", "backward_both_2x2", "backward_nonsquare_2x4_4x3"):
+        g = GOLD[key]
+        a = oracle.to_storage(np.array(g["a"], dtype=np.float64), dt)
+        b = oracle.to_storage(np.array(g["b"], dtype=np.float64), dt)
+        dc = oracle.to_storage(np.ones((a.shape[0], b.shape[1])), dt)
+        da = device_gemm(dc, b.T, dt)            # dA = dC · Bᵀ, Bᵀ passed as a stride view
+        db = device_gemm(a.T, dc, dt)            # dB = Aᵀ · dC
+        assert np.array_equal(oracle.to_f64(da, dt), np.array(g["da"], dtype=np.float64)), key
+        assert np.array_equal(oracle.to_f64(db, dt), np.array(g["db"], dtype=np.float64)), key
+
+
+def test_matmul_kernel_device_seam_f64_parity_shapes():
+    rng = np.random.default_rng(30)
+    g = GOLD["parity_shapes"]
+    for m, k, n in g["mkn"]:
+        a = rng.uniform(-1, 1, (m, k)); b = rng.uniform(-1, 1, (k, n))
+        da, db = capi.DeviceBuffer.from_numpy(a), capi.DeviceBuffer.from_numpy(b)
+        dc = capi.DeviceBuffer(m * n * 8)
+        capi.check(capi.lib().matmul_kernel_device(dc.ptr, da.ptr, db.ptr, m, k, n, F64), "matmul_kernel_device")
+        capi.synchronize()
+        np.testing.assert_allclose(dc.to_numpy(np.float64, (m, n)), a @ b, rtol=g["rtol"], atol=g["atol"])
+
+
+LAYOUTS = ["nn", "nt", "tn", "tt"]
+
+
+def _operands(rng, m, k, n, dt, layout, dist="normal"):
+    a = rand_storage(rng, (m, k), dt, dist) if layout[0] == "n" else rand_storage(rng, (k, m), dt, dist).T
+    b = rand_storage(rng, (k, n), dt, dist) if layout[1] == "n" else rand_storage(rng, (n, k), dt, dist).T
+    return a, b
+
+
+SHAPES = [
+    (3, 4, 5), (1, 7, 1), (16, 32, 8), (33, 65, 17),          # generic (odd extents)
+    (64, 64, 64), (64, 128, 64), (48, 80, 56),                # 64x64 tiles, full and edge
+    (128, 192, 128), (256, 64, 384), (200, 136, 264),         # 128x128 tiles, full and edge
+    (128, 784, 256),                                          # config 1 shape
+]
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_small_shapes_all_layouts(dt, layout):
+    rng = np.random.default_rng(31)
+    for m, k, n in SHAPES:
+        a, b = _operands(rng, m, k, n, dt, layout)
+        got = device_gemm(a, b, dt)
+        _check(got, a, b, dt, k)
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_integer_valued_inputs_are_exact(dt):
+    """Small integers: every partial sum is exact in every dtype's accumulator, so any order must agree bit for bit."""
+    rng = np.random.default_rng(32)
+    for (m, k, n), layout in [((64, 64, 64), "nn"), ((128, 128, 128), "tn"), ((40, 24, 72), "nt"), ((130, 96, 66), "tt")]:
+        a = oracle.to_storage(rng.integers(-3, 4, (m, k) if layout[0] == "n" else (k, m)).astype(np.float64), dt)
+        b = oracle.to_storage(rng.integers(-3, 4, (k, n) if layout[1] == "n" else (n, k)).astype(np.float64), dt)
+        a = a if layout[0] == "n" else a.T
+        b = b if layout[1] == "n" else b.T
+        got = device_gemm(a, b, dt)
+        want = oracle_gemm(a, b, dt)
+        assert np.array_equal(got, want), (m, k, n, layout)
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_bias_and_accumulate_epilogue(dt):
+    rng = np.random.default_rng(33)
+    for m, k, n in [(5, 9, 7), (64, 64, 64), (128, 784, 256), (72, 40, 136)]:
+        a, b = _operands(rng, m, k, n, dt, "nn")
+        bias = rand_storage(rng, (n,), dt)
+        c0 = rand_storage(rng, (m, n), dt)
+        for kw in ({"bias": bias}, {"c_init": c0, "accumulate": True}, {"bias": bias, "c_init": c0, "accumulate": True}):
+            got = device_gemm(a, b, dt, **kw)
+            _check(got, a, b, dt, k, **kw)
+    # exact epilogue: integer data makes the whole chain exact, so the three roundings of the 16-bit chain must agree
+    a = oracle.to_storage(rng.integers(-2, 3, (64, 64)).astype(np.float64), dt)
+    b = oracle.to_storage(rng.integers(-2, 3, (64, 64)).astype(np.float64), dt)
+    bias = oracle.to_storage(rng.integers(-4, 5, (64,)).astype(np.float64), dt)
+    c0 = oracle.to_storage(rng.integers(-4, 5, (64, 64)).astype(np.float64), dt)
+    got = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)
+    assert np.array_equal(got, oracle_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True))
+
+
+@pytest.mark.parametrize("dt", [F16, BF16], ids=lambda d: NAMES[d])
+def test_16bit_rounding_is_the_references_half_away_from_zero(dt):
+    """Products chosen so the fp32 sum sits exactly on a 16-bit tie: round-to-nearest-even would differ."""
+    if dt == BF16:
+        vals = [257.0, 259.0, -257.0]                        # 257 = 0x1.01p8: tie between 256 and 258 in bf16
+    else:
+        vals = [2049.0, 2051.0, -2049.0]                     # 2049: tie between 2048 and 2050 in fp16
+    m = len(vals)
+    a64 = np.zeros((m, 8)); b64 = np.zeros((8, 8))
+    for i, v in enumerate(vals):
+        a64[i, 0] = 1.0 if v > 0 else -1.0
+        a64[i, 1] = 1.0 if v > 0 else -1.0
+    b64[0, :] = 1.0
+    got_all = []
+    for i, v in enumerate(vals):
+        b = b64.copy(); b[1, :] = abs(v) - 1.0              # |v|-1 is representable in both 16-bit formats for these values
+        a_s = oracle.to_storage(a64[i:i + 1], dt); b_s = oracle.to_storage(b, dt)
+        assert oracle.to_f64(b_s, dt)[1, 0] == abs(v) - 1.0
+        got = device_gemm(a_s, b_s, dt)
+        want = oracle_gemm(a_s, b_s, dt)
+        assert np.array_equal(got, want), v
+        got_all.append(oracle.to_f64(got, dt)[0, 0])
+    assert got_all[0] == (258.0 if dt == BF16 else 2050.0)
+    assert got_all[2] == (-258.0 if dt == BF16 else -2050.0)
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_batched_strided_views(dt):
+    rng = np.random.default_rng(34)
+    B, H, S, D = 2, 3, 64, 32
+    q = rand_storage(rng, (B * H, S, D), dt); kmat = rand_storage(rng, (B * H, S, D), dt)
+    kt = kmat.transpose(0, 2, 1)                       # permuted view, no copy
+    s = device_gemm(q, kt, dt)
+    _check(s, q, kt, dt, D)
+    p = rand_storage(rng, (B * H, S, S), dt); v = rand_storage(rng, (B * H, S, D), dt)
+    o = device_gemm(p, v, dt)
+    _check(o, p, v, dt, S)
+    # dV = Pᵀ · dO with Pᵀ a view, odd sizes (generic path with batch)
+    p2 = rand_storage(rng, (4, 9, 13), dt); do = rand_storage(rng, (4, 9, 5), dt)
+    dv = device_gemm(p2.transpose(0, 2, 1), do, dt)
+    _check(dv, p2.transpose(0, 2, 1), do, dt, 9)
+
+
+def test_sliced_operand_with_offset_and_padding():
+    rng = np.random.default_rng(35)
+    big_a = rand_storage(rng, (96, 200), F32); big_b = rand_storage(rng, (200, 160), F32)
+    a = big_a[16:80, 8:136]          # 64 x 128 window, row stride 200, base offset
+    b = big_b[8:136, 32:96]
+    got = device_gemm(a, b, F32)
+    _check(got, a, b, F32, 128)
+    a2 = big_a[::2, ::2]             # no unit stride at all -> generic
+    b2 = big_b[:100:1, ::2]
+    got = device_gemm(a2, b2, F32)
+    _check(got, a2, b2, F32, 100)
+
+
+@pytest.mark.parametrize("dt", [BF16, F16, F32], ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("m", [1, 2, 5, 8])
+def test_skinny_rows(dt, m):
+    rng = np.random.default_rng(36)
+    k, n = 2048, 1024
+    assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == "skinny"
+    a, b = _operands(rng, m, k, n, dt, "nn")
+    bias = rand_storage(rng, (n,), dt)
+    got = device_gemm(a, b, dt, bias=bias)
+    _check(got, a, b, dt, k, bias=bias)
+    got2 = device_gemm(a, b, dt, bias=bias)
+    assert np.array_equal(got, got2)                   # split-k partials are combined in a fixed order
+
+
+def test_large_tile_kernel_multi_slab():
+    """4096 x 4096 outputs select the 256x256 tile; checked against float64 everywhere and the oracle on a row slab."""
+    rng = np.random.default_rng(37)
+    m = n = 4096; k = 320
+    for dt, layout in [(BF16, "nn"), (F16, "tn"), (BF16, "nt"), (F16, "tt")]:
+        assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == "mfma16_256x256"
+        a, b = _operands(rng, m, k, n, dt, layout)
+        got = device_gemm(a, b, dt)
+        e64 = oracle.rel_err(oracle.to_f64(got, dt), f64_gemm(a, b, dt))
+        assert e64 <= tol(dt, k), e64
+        rows = np.array([0, 1, 255, 256, 1023, 2048, 4095])
+        want = oracle.matmul(np.ascontiguousarray(a[rows]), np.ascontiguousarray(b), dt)
+        assert oracle.rel_err(oracle.to_f64(got[rows], dt), oracle.to_f64(want, dt)) <= tol(dt, k)
+
+
+def test_rejects_bad_arguments():
+    lib = capi.lib()
+    d = capi.DeviceBuffer(64)
+    assert lib.rp_hip_gemm_strided_batched(d.ptr, d.ptr, None, None, 1, 2, 2, 2, 0, 2, 1, 0, 2, 1, 0, 2, 1, 0, F32) == -1
+    assert lib.rp_hip_gemm_strided_batched(d.ptr, d.ptr, d.ptr, None, 1, 0, 2, 2, 0, 2, 1, 0, 2, 1, 0, 2, 1, 0, F32) == -1
+    assert lib.rp_hip_gemm_strided_batched(d.ptr, d.ptr, d.ptr, None, 1, 2, 2, 2, 0, 2, 1, 0, 2, 1, 0, 2, 1, 0, 7) == -1
+    assert lib.matmul_kernel_device(d.ptr, d.ptr, d.ptr, 2, -1, 2, F32) == -1
+    assert b"extent" in lib.rp_hip_last_error()
