@@ -1,0 +1,248 @@
+#!/usr/bin/env python3
+"""Benchmark of the matmul hot path on one MI355X.
+
+A "step" is one pass of the path over one synthetic batch: the forward GEMM
+C = A·B and both backward GEMMs dA = dC·Bᵀ and dB = Aᵀ·dC at M = N = K = 8192 in
+bf16 (fp32 accumulate, bf16 output), operands resident in HBM, transposes passed
+as stride views.  Prints ONE JSON line: whole-step TFLOP/s as `value`, the
+forward kernel's roofline fraction, a one-core CPU baseline on a bounded slab of
+the same workload, and secondary figures (skinny GEMM GB/s, fp32 / fp64 GEMMs,
+the config-2 MLP step) under `secondary`.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3, "f64": 78.6}     # MI355X dense MFMA
+PEAK_HBM_GBS = 8000.0
+
+
+def _bf16_bits(x32):
+    """fp32 -> bf16 bit patterns, the reference's rounding (truncate + first dropped bit)."""
+    w = np.ascontiguousarray(x32, dtype=np.float32).view(np.uint32)
+    return ((w >> 16) + ((w >> 15) & 1)).astype(np.uint16)
+
+
+def _normal_bf16(rng, shape):
+    out = np.empty(shape, dtype=np.uint16)
+    rows = shape[0]
+    step = max(1, (1 << 22) // max(1, int(np.prod(shape[1:]))))
+    for r0 in range(0, rows, step):
+        out[r0:r0 + step] = _bf16_bits(rng.standard_normal((min(step, rows - r0),) + tuple(shape[1:]), dtype=np.float32))
+    return out
+
+
+def _time_launches(capi, fn, reps, warmup):
+    """Average milliseconds per call of fn(), HIP events on the launch stream."""
+    for _ in range(warmup):
+        fn()
+    e0, e1 = capi.Event(), capi.Event()
+    capi.synchronize()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_ms(e1) / reps
+
+
+def headline(capi, steps, warmup, n=8192):
+    rng = np.random.default_rng(2)
+    dt = capi.BF16
+    a, b, dc = (_normal_bf16(rng, (n, n)) for _ in range(3))
+    d_a, d_b, d_dc = (capi.DeviceBuffer.from_numpy(t) for t in (a, b, dc))
+    d_c, d_da, d_db = (capi.DeviceBuffer(n * n * 2) for _ in range(3))
+    rm, tr = (0, n, 1), (0, 1, n)            # row-major and transposed-view strides (batch, row, col)
+
+    def fwd():
+        capi.gemm(d_c.ptr, d_a.ptr, d_b.ptr, None, 1, n, n, n, rm, rm, rm, False, dt)
+
+    def bwd_a():                              # dA = dC · Bᵀ
+        capi.gemm(d_da.ptr, d_dc.ptr, d_b.ptr, None, 1, n, n, n, rm, tr, rm, False, dt)
+
+    def bwd_b():                              # dB = Aᵀ · dC
+        capi.gemm(d_db.ptr, d_a.ptr, d_dc.ptr, None, 1, n, n, n, tr, rm, rm, False, dt)
+
+    kernels = (("fwd_nn", fwd), ("dA_nt", bwd_a), ("dB_tn", bwd_b))
+    for _ in range(warmup):
+        for _, fn in kernels:
+            fn()
+    capi.synchronize()
+    # timed region: exactly `steps` steps; an event after every launch gives per-kernel durations
+    marks = [capi.Event() for _ in range(steps * 3 + 1)]
+    capi.synchronize()
+    t0 = time.perf_counter()
+    marks[0].record()
+    for s in range(steps):
+        for j, (_, fn) in enumerate(kernels):
+            fn()
+            marks[s * 3 + j + 1].record()
+    marks[-1].synchronize()
+    capi.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    total_ms = marks[0].elapsed_ms(marks[-1])
+    per = {name: 0.0 for name, _ in kernels}
+    for s in range(steps):
+        for j, (name, _) in enumerate(kernels):
+            per[name] += marks[s * 3 + j].elapsed_ms(marks[s * 3 + j + 1])
+    per = {k: v / steps for k, v in per.items()}
+    flops = 2.0 * n * n * n
+
+    # spot parity inside the bench: sampled entries against float64 dot products
+    c = d_c.to_numpy(np.uint16, (n, n))
+    rows = np.array([0, 257, 4095, 8191]); cols = np.array([1, 300, 5000, 8190])
+    a64 = (a[rows].astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    b64 = (b[:, cols].astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    ref = a64 @ b64
+    got = (c[np.ix_(rows, cols)].astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    err = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
+    if not err <= 2e-2:
+        raise RuntimeError(f"bf16 8192^3 forward GEMM fails parity: sampled normwise error {err}")
+    return {
+        "ms_per_step": total_ms / steps, "wall_ms_per_step": wall_ms / steps,
+        "tflops": 3 * flops / (total_ms / steps * 1e-3) / 1e12,
+        "kernel_ms": per, "fwd_tflops": flops / (per["fwd_nn"] * 1e-3) / 1e12,
+        "sampled_rel_err": err, "operands": (a, b),
+        "kernel": capi.gemm_kernel_name(1, n, n, n, (n, 1), (n, 1), (n, 1), dt),
+    }
+
+
+def cpu_baseline(a, b, rows=8):
+    """The oracle's restatement of the reference CPU matmul on a `rows`-row slab of the 8192^3 bf16 GEMM, one core."""
+    import oracle
+    n = b.shape[0]
+    slab = np.ascontiguousarray(a[:rows])
+    t0 = time.perf_counter()
+    oracle.matmul(slab, b, oracle.BF16)
+    dt = time.perf_counter() - t0
+    flops = 2.0 * rows * n * n
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"{rows} of {n} rows of the bf16 {n}^3 forward GEMM (fp32 pivot, i-j-l loop), {dt:.1f} s; "
+                      f"host has {os.cpu_count()} logical cores"}
+
+
+def secondary(capi, quick_reps=20):
+    out = {}
+    rng = np.random.default_rng(4)
+    # config 5a: skinny bf16 GEMMs, K = N = 8192
+    k = n = 8192
+    w = _normal_bf16(rng, (k, n))
+    d_w = capi.DeviceBuffer.from_numpy(w)
+    for m in (1, 8, 32):
+        a = _normal_bf16(rng, (m, k))
+        d_a = capi.DeviceBuffer.from_numpy(a); d_y = capi.DeviceBuffer(m * n * 2)
+        fn = lambda: capi.gemm(d_y.ptr, d_a.ptr, d_w.ptr, None, 1, m, k, n, (0, k, 1), (0, n, 1), (0, n, 1), False, capi.BF16)
+        ms = _time_launches(capi, fn, quick_reps, 5)
+        nbytes = (m * k + k * n + m * n) * 2
+        out[f"skinny_bf16_m{m}"] = {"us": ms * 1e3, "GB/s": nbytes / (ms * 1e-3) / 1e9, "frac_hbm": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                    "kernel": capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), capi.BF16)}
+    # config 3: fp32 at 4096, fp16 at 8192; config 5b: fp64 at 2048
+    for name, dt, npdt, size, peak in (("gemm_f32_4096", capi.F32, np.float32, 4096, PEAK_TFLOPS["f32"]),
+                                       ("gemm_f64_2048", capi.F64, np.float64, 2048, PEAK_TFLOPS["f64"])):
+        a = rng.standard_normal((size, size)).astype(npdt); b = rng.standard_normal((size, size)).astype(npdt)
+        d_a, d_b = capi.DeviceBuffer.from_numpy(a), capi.DeviceBuffer.from_numpy(b)
+        d_c = capi.DeviceBuffer(a.nbytes)
+        s = (0, size, 1)
+        fn = lambda: capi.gemm(d_c.ptr, d_a.ptr, d_b.ptr, None, 1, size, size, size, s, s, s, False, dt)
+        ms = _time_launches(capi, fn, 10, 3)
+        tf = 2.0 * size ** 3 / (ms * 1e-3) / 1e12
+        out[name] = {"ms": ms, "TFLOP/s": tf, "frac_mfma": tf / peak}
+    # config 2: fp32 MLP 784-256-128-10, batch 256, forward + backward through the C ABI (9 GEMMs + neighbours)
+    out["mlp_f32_step"] = mlp_step_time(capi)
+    return out
+
+
+def mlp_step_time(capi, reps=50):
+    import ctypes
+    rng = np.random.default_rng(1)
+    dims = [784, 256, 128, 10]; batch = 256
+    F = capi.F32
+    L = capi.lib()
+    x = rng.uniform(0, 1, (batch, dims[0])).astype(np.float32)
+    ws = [rng.normal(0, np.sqrt(2.0 / dims[i]), (dims[i], dims[i + 1])).astype(np.float32) for i in range(3)]
+    bs = [np.zeros(dims[i + 1], np.float32) for i in range(3)]
+    y = rng.integers(0, 10, batch).astype(np.int32)
+    D = capi.DeviceBuffer
+    d_x = D.from_numpy(x); d_w = [D.from_numpy(w) for w in ws]; d_b = [D.from_numpy(b) for b in bs]; d_y = D.from_numpy(y)
+    d_z = [D(batch * dims[i + 1] * 4) for i in range(3)]; d_h = [D(batch * dims[i + 1] * 4) for i in range(2)]
+    d_g = [D(batch * dims[i + 1] * 4) for i in range(3)]; d_gh = [D(batch * dims[i + 1] * 4) for i in range(2)]
+    d_dw = [D(ws[i].nbytes) for i in range(3)]; d_db = [D(bs[i].nbytes) for i in range(3)]
+    d_dx = D(x.nbytes); d_loss = D(4)
+
+    def step():
+        h = d_x
+        for i in range(3):
+            m, k, n = batch, dims[i], dims[i + 1]
+            capi.gemm(d_z[i].ptr, h.ptr, d_w[i].ptr, d_b[i].ptr, 1, m, k, n, (0, k, 1), (0, n, 1), (0, n, 1), False, F)
+            if i < 2:
+                L.relu_kernel_device(d_h[i].ptr, d_z[i].ptr, m * n, F)
+                h = d_h[i]
+        L.rp_hip_cross_entropy_mean(d_loss.ptr, d_g[2].ptr, d_z[2].ptr, d_y.ptr, batch, 10, 1.0, F)
+        for i in (2, 1, 0):
+            m, k, n = batch, dims[i], dims[i + 1]
+            inp = d_x if i == 0 else d_h[i - 1]
+            L.rp_hip_reduce_rows(d_db[i].ptr, d_g[i].ptr, m, n, 0, F)
+            # dW[k,n] = inpᵀ[k,m] · g[m,n]
+            capi.gemm(d_dw[i].ptr, inp.ptr, d_g[i].ptr, None, 1, k, m, n, (0, 1, k), (0, n, 1), (0, n, 1), False, F)
+            # dIn[m,k] = g[m,n] · Wᵀ[n,k]
+            dst = d_dx if i == 0 else d_gh[i - 1]
+            capi.gemm(dst.ptr, d_g[i].ptr, d_w[i].ptr, None, 1, m, n, k, (0, n, 1), (0, 1, n), (0, k, 1), False, F)
+            if i > 0:
+                L.backwards_relu_device(d_gh[i - 1].ptr, d_z[i - 1].ptr, d_g[i - 1].ptr, m * k, F)
+
+    ms = _time_launches(capi, step, reps, 5)
+    return {"ms": ms, "launches": 18, "note": "9 GEMMs (bias fused into the 3 forward ones), 2 relu, 2 relu-backward, "
+            "cross-entropy fwd+bwd, 3 bias-gradient reductions; C ABI called from Python"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-secondary", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    from recpulse_amd import capi
+    if capi.device_count() < 1:
+        print("bench.py needs a GPU and the built librp_hip.so; there is no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+    capi.check(capi.lib().rp_hip_set_device(0), "rp_hip_set_device")
+
+    h = headline(capi, args.steps, args.warmup)
+    a, b = h.pop("operands")
+    line = {
+        "metric": "GEMM TFLOP/s (bf16 8192^3, forward + both backward GEMMs per step)",
+        "value": h["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": h["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "config 3 at N=8192: bf16 square GEMM, fp32 accumulate, bf16 output; "
+                               "C=A·B, dA=dC·Bᵀ, dB=Aᵀ·dC with transposes as stride views; A,B,dC ~ N(0,1) seed 2",
+                   "m": 8192, "n": 8192, "k": 8192, "gemms_per_step": 3},
+        "roofline": {"bound": "mfma", "achieved": h["fwd_tflops"], "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
+                     "frac": h["fwd_tflops"] / PEAK_TFLOPS["bf16"], "traffic": None,
+                     "kernel": h["kernel"] + " (forward, A row-major x B row-major)",
+                     "avg_launch_ms": h["kernel_ms"]["fwd_nn"]},
+        "kernel_ms": h["kernel_ms"], "sampled_rel_err": h["sampled_rel_err"],
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(a, b)
+    del a, b
+    if not args.no_secondary:
+        line["secondary"] = secondary(capi)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

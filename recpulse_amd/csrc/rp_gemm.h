@@ -1,0 +1,90 @@
+// Shared declarations of the GEMM translation units: the problem descriptor,
+// the dispatcher's plan, the XCD-aware tile schedule and the per-family launchers.
+#pragma once
+#include "rp_common.h"
+
+#include <cstdlib>
+#include <cstring>
+
+namespace rp {
+
+struct GemmArgs {
+    void* C;
+    const void* A;
+    const void* B;
+    const void* bias;
+    int batch, m, k, n;
+    long long a_bs, a_rs, a_cs;
+    long long b_bs, b_rs, b_cs;
+    long long c_bs, c_rs, c_cs;
+    int accumulate;
+};
+
+enum Family { FAM_GENERIC = 0, FAM_SKINNY, FAM_MFMA16, FAM_MFMAW };
+
+struct Plan {
+    Family fam;
+    int bm, bn;
+    bool a_mc, b_mc, edge;
+    const char* name;
+};
+
+constexpr int SK_MAX_M = 8;           // rows the skinny kernel takes
+constexpr int SK_MAX_GROUPS = 4096;   // column groups it can track
+constexpr int M16_BK = 64;            // k slab of the 16-bit MFMA kernels
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(8))) short s16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) double f64x4_t;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+
+// Tile scheduling shared by the MFMA kernels.
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2), so a
+// linear block id is first split into (xcd, slot); every XCD then walks its
+// own sequence of 4x8-tile super-tiles, which keeps the 32 tiles resident on an
+// XCD at one time inside a compact window of the output (4 A row panels and
+// 8 B column panels shared through that XCD's L2).
+// ----------------------------------------------------------------------------
+struct TileCoord { int tm, tn; bool valid; };
+
+constexpr int SCHED_MIN_TILES = 64;      // below this a launch does not fill the chip and plain row-major order is used
+
+__device__ __forceinline__ TileCoord schedule_tile(int bid, int tiles_m, int tiles_n) {
+    constexpr int XCDS = 8, GM = 4, GN = 8, PER = GM * GN;
+    if (tiles_m * tiles_n < SCHED_MIN_TILES) {
+        TileCoord lin;
+        lin.tm = bid / tiles_n; lin.tn = bid % tiles_n; lin.valid = bid < tiles_m * tiles_n;
+        return lin;
+    }
+    int sup_m = (tiles_m + GM - 1) / GM, sup_n = (tiles_n + GN - 1) / GN;
+    int xcd = bid % XCDS, slot = bid / XCDS;
+    int sup = (slot / PER) * XCDS + xcd;
+    int within = slot % PER;
+    TileCoord tc;
+    int sm = sup / sup_n, sn = sup % sup_n;
+    tc.tm = sm * GM + within / GN;
+    tc.tn = sn * GN + within % GN;
+    tc.valid = (sm < sup_m) && (tc.tm < tiles_m) && (tc.tn < tiles_n);
+    return tc;
+}
+
+static inline int scheduled_grid(int tiles_m, int tiles_n) {
+    constexpr int XCDS = 8, GM = 4, GN = 8, PER = GM * GN;
+    if (tiles_m * tiles_n < SCHED_MIN_TILES) return tiles_m * tiles_n;
+    int sup = ((tiles_m + GM - 1) / GM) * ((tiles_n + GN - 1) / GN);
+    int rounds = (sup + XCDS - 1) / XCDS;
+    return rounds * XCDS * PER;
+}
+
+
+// per-family launchers (dtype is one of the RP_DTYPE_* codes the family supports)
+int launch_generic(const GemmArgs& g, int dtype);
+int launch_skinny(const GemmArgs& g, int dtype);
+int launch_mfma16(const GemmArgs& g, const Plan& p, int dtype);
+int launch_mfmaw(const GemmArgs& g, const Plan& p, int dtype);
+
+}  // namespace rp

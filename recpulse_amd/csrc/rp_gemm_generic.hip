@@ -1,0 +1,314 @@
+// The two non-MFMA GEMM kernels: the generic strided kernel that takes any
+// shape and stride, and the skinny split-k kernel for a few rows of A against a
+// row-major B (bound by streaming B from HBM).
+#include "rp_gemm.h"
+
+namespace rp {
+
+// ============================================================================
+// generic: 64x64 output tile, 16-deep k slabs, 256 threads each owning 4x4.
+// ============================================================================
+template <typename T>
+__global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g) {
+    using Acc = typename traits<T>::acc;
+    constexpr int TM = 64, TN = 64, TK = 16;
+    __shared__ Acc As[TK][TM + 1];
+    __shared__ Acc Bs[TK][TN + 1];
+
+    const int z = blockIdx.z;
+    const T* A = (const T*)g.A + (long long)z * g.a_bs;
+    const T* B = (const T*)g.B + (long long)z * g.b_bs;
+    T* C = (T*)g.C + (long long)z * g.c_bs;
+    const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
+    const int t = threadIdx.x;
+    const int ty = t / 16, tx = t % 16;
+    const bool a_kfast = (g.a_cs == 1), b_nfast = (g.b_cs == 1);
+
+    Acc acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = (Acc)0;
+
+    for (int k0 = 0; k0 < g.k; k0 += TK) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int id = t + 256 * i;
+            int kk = a_kfast ? id % TK : id / TM;
+            int r = a_kfast ? id / TK : id % TM;
+            int gm = m0 + r, gk = k0 + kk;
+            Acc v = (Acc)0;
+            if (gm < g.m && gk < g.k) v = widen(A[(long long)gm * g.a_rs + (long long)gk * g.a_cs]);
+            As[kk][r] = v;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int id = t + 256 * i;
+            int kk = b_nfast ? id / TN : id % TK;
+            int c = b_nfast ? id % TN : id / TK;
+            int gn = n0 + c, gk = k0 + kk;
+            Acc v = (Acc)0;
+            if (gn < g.n && gk < g.k) v = widen(B[(long long)gk * g.b_rs + (long long)gn * g.b_cs]);
+            Bs[kk][c] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < TK; kk++) {
+            Acc a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; j++) b[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] += a[i] * b[j];
+        }
+        __syncthreads();
+    }
+
+    const T* bias = (const T*)g.bias;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        int gm = m0 + ty * 4 + i;
+        if (gm >= g.m) continue;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            int gn = n0 + tx * 4 + j;
+            if (gn >= g.n) continue;
+            T* p = C + (long long)gm * g.c_rs + (long long)gn * g.c_cs;
+            T old = g.accumulate ? *p : T{};
+            T bv = bias ? bias[gn] : T{};
+            *p = finish<T>(acc[i][j], bias != nullptr, bv, g.accumulate != 0, old);
+        }
+    }
+}
+
+// ============================================================================
+// skinny: m <= 8 rows of A against a row-major B (unit column stride).
+// The cost is streaming B once from HBM.  Each lane owns VEC adjacent columns
+// (one 16-byte load per k row) and a wave covers 64*VEC columns.  The 8 waves
+// of a block share a column group and take interleaved k rows of the block's
+// k range; they combine through LDS in a fixed tree.  The grid's second axis
+// splits k further: split partials go to a workspace, and the block that
+// arrives last for a column group adds them in split order (so the result
+// does not depend on scheduling) and runs the epilogue.
+// ============================================================================
+constexpr int SK_THREADS = 512, SK_WAVES = SK_THREADS / 64;
+__device__ unsigned int g_skinny_arrivals[SK_MAX_GROUPS];     // zero at load; the last block of a group re-zeroes its slot
+
+template <typename T, int MROWS>
+__global__ void __launch_bounds__(SK_THREADS) gemm_skinny_kernel(GemmArgs g, float* partials, int k_per_block) {
+    constexpr int VEC = 16 / sizeof(T);
+    extern __shared__ __attribute__((aligned(16))) float sk_lds[];   // first A's slice [k_per_block][MROWS], later the wave-combine buffer
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col0 = (blockIdx.x * 64 + lane) * VEC;
+    const int split = blockIdx.y, nsplit = gridDim.y;
+    const bool col_ok = col0 < g.n;          // n is a multiple of VEC, so a vector is wholly in or out
+    const T* A = (const T*)g.A;
+    const T* B = (const T*)g.B;
+
+    float acc[MROWS][VEC];
+#pragma unroll
+    for (int r = 0; r < MROWS; r++)
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[r][e] = 0.f;
+
+    const int kb = split * k_per_block;
+    const int ke = kb + k_per_block < g.k ? kb + k_per_block : g.k;
+    const int klen = ke - kb;
+    // this block's slice of A, widened once, rows beyond m as zeros
+    for (int i = threadIdx.x; i < MROWS * klen; i += SK_THREADS) {
+        int r = i / klen, kl = i - r * klen;
+        sk_lds[kl * MROWS + r] = (r < g.m) ? widen(A[(long long)r * g.a_rs + (long long)(kb + kl) * g.a_cs]) : 0.f;
+    }
+    __syncthreads();
+
+    if (col_ok) {
+        const T* bp = B + col0 + (long long)kb * g.b_rs;
+        constexpr int U = 8;
+        int kl = wave;
+        for (; kl + SK_WAVES * (U - 1) < klen; kl += SK_WAVES * U) {
+            u32x4_t raw[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) raw[u] = __builtin_nontemporal_load((const u32x4_t*)(bp + (long long)(kl + SK_WAVES * u) * g.b_rs));
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                T bv[VEC];
+                memcpy(bv, &raw[u], 16);
+                float bw[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; e++) bw[e] = widen(bv[e]);
+#pragma unroll
+                for (int r = 0; r < MROWS; r++) {
+                    float a = sk_lds[(kl + SK_WAVES * u) * MROWS + r];
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) acc[r][e] += a * bw[e];
+                }
+            }
+        }
+        for (; kl < klen; kl += SK_WAVES) {
+            u32x4_t raw = *(const u32x4_t*)(bp + (long long)kl * g.b_rs);
+            T bv[VEC];
+            memcpy(bv, &raw, 16);
+#pragma unroll
+            for (int r = 0; r < MROWS; r++) {
+                float a = sk_lds[kl * MROWS + r];
+#pragma unroll
+                for (int e = 0; e < VEC; e++) acc[r][e] += a * widen(bv[e]);
+            }
+        }
+    }
+    __syncthreads();            // everyone is done with A's slice; the buffer now carries wave partials
+
+    // fixed tree over the 8 waves: (4..7 -> 0..3), (2..3 -> 0..1), (1 -> 0)
+    constexpr int WSZ = MROWS * VEC * 64;
+#pragma unroll
+    for (int half = SK_WAVES / 2; half >= 1; half >>= 1) {
+        if (wave >= half && wave < 2 * half) {
+            float* dst = sk_lds + (wave - half) * WSZ;
+#pragma unroll
+            for (int r = 0; r < MROWS; r++)
+#pragma unroll
+                for (int e = 0; e < VEC; e++) dst[(r * VEC + e) * 64 + lane] = acc[r][e];
+        }
+        __syncthreads();
+        if (wave < half) {
+            const float* src = sk_lds + wave * WSZ;
+#pragma unroll
+            for (int r = 0; r < MROWS; r++)
+#pragma unroll
+                for (int e = 0; e < VEC; e++) acc[r][e] += src[(r * VEC + e) * 64 + lane];
+        }
+        __syncthreads();
+    }
+
+    T* C = (T*)g.C;
+    const T* bias = (const T*)g.bias;
+    const bool has_bias = bias != nullptr, accum = g.accumulate != 0;
+    if (nsplit == 1) {
+        if (wave == 0 && col_ok) {
+#pragma unroll
+            for (int r = 0; r < MROWS; r++) {
+                if (r >= g.m) break;
+#pragma unroll
+                for (int e = 0; e < VEC; e++) {
+                    T* p = C + (long long)r * g.c_rs + (long long)(col0 + e) * g.c_cs;
+                    T old = accum ? *p : T{};
+                    *p = finish<T>(acc[r][e], has_bias, has_bias ? bias[col0 + e] : T{}, accum, old);
+                }
+            }
+        }
+        return;
+    }
+
+    // partial layout: [split][row][n] fp32
+    if (wave == 0 && col_ok) {
+#pragma unroll
+        for (int r = 0; r < MROWS; r++) {
+            if (r >= g.m) break;
+            float* q = partials + ((long long)split * g.m + r) * g.n + col0;
+#pragma unroll
+            for (int e = 0; e < VEC; e += 4) *(f32x4_t*)(q + e) = f32x4_t{acc[r][e], acc[r][e + 1], acc[r][e + 2], acc[r][e + 3]};
+        }
+    }
+    __shared__ bool last;
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned int done = atomicAdd(&g_skinny_arrivals[blockIdx.x], 1u);
+        last = (done == (unsigned)nsplit - 1);
+    }
+    __syncthreads();
+    if (!last) return;
+    __threadfence();
+    // the last block: one (row, 64-lane column vector) item per thread, splits added in order
+    {
+        const int r = threadIdx.x >> 6;
+        if (r < g.m && col_ok) {
+            float sum[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; e++) sum[e] = 0.f;
+            for (int s = 0; s < nsplit; s++) {
+                const float* q = partials + ((long long)s * g.m + r) * g.n + col0;
+#pragma unroll
+                for (int e = 0; e < VEC; e += 4) {
+                    f32x4_t v = *(const f32x4_t*)(q + e);
+                    sum[e] += v[0]; sum[e + 1] += v[1]; sum[e + 2] += v[2]; sum[e + 3] += v[3];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                T* p = C + (long long)r * g.c_rs + (long long)(col0 + e) * g.c_cs;
+                T old = accum ? *p : T{};
+                *p = finish<T>(sum[e], has_bias, has_bias ? bias[col0 + e] : T{}, accum, old);
+            }
+        }
+    }
+    if (threadIdx.x == 0) g_skinny_arrivals[blockIdx.x] = 0;
+}
+
+template <typename T>
+static int launch_generic_t(const GemmArgs& g) {
+    dim3 grid((g.n + 63) / 64, (g.m + 63) / 64, g.batch);
+    hipLaunchKernelGGL(gemm_generic_kernel<T>, grid, dim3(256), 0, current_stream(), g);
+    return check_launch("gemm_generic_kernel") ? 0 : -1;
+}
+
+static int skinny_k_per_block() {
+    static int v = -1;
+    if (v < 0) { const char* e = getenv("RP_HIP_SKINNY_KPB"); v = e ? atoi(e) : 0; if (v < 0) v = 0; }
+    return v;
+}
+
+template <typename T>
+static int launch_skinny_t(const GemmArgs& g) {
+    constexpr int VEC = 16 / sizeof(T);
+    int groups = (g.n + 64 * VEC - 1) / (64 * VEC);
+    // enough blocks to put two on every CU, each wave keeping at least 32 k rows
+    int k_per_block = skinny_k_per_block();
+    if (k_per_block == 0) {
+        int want = (512 + groups - 1) / groups;
+        k_per_block = (g.k + want - 1) / want;
+        if (k_per_block < 256) k_per_block = 256;
+    }
+    if (k_per_block > 2048) k_per_block = 2048;            // bounds the LDS copy of A (2048 x 8 floats = 64 KB)
+    k_per_block = (k_per_block + SK_WAVES - 1) / SK_WAVES * SK_WAVES;
+    int nsplit = (g.k + k_per_block - 1) / k_per_block;
+    if (nsplit > 65535) { set_error("gemm skinny: k too large"); return -1; }
+    void* ws = nullptr;
+    if (nsplit > 1 && rp_hip_malloc(&ws, (size_t)nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
+    dim3 grid(groups, nsplit);
+    auto smem = [&](int mrows) {
+        size_t a_slice = (size_t)k_per_block * mrows * 4, combine = (size_t)(SK_WAVES / 2) * mrows * VEC * 64 * 4;
+        return a_slice > combine ? a_slice : combine;
+    };
+    hipError_t attr = hipSuccess;
+    if (g.m <= 1)      hipLaunchKernelGGL((gemm_skinny_kernel<T, 1>), grid, dim3(SK_THREADS), smem(1), current_stream(), g, (float*)ws, k_per_block);
+    else if (g.m <= 2) hipLaunchKernelGGL((gemm_skinny_kernel<T, 2>), grid, dim3(SK_THREADS), smem(2), current_stream(), g, (float*)ws, k_per_block);
+    else if (g.m <= 4) hipLaunchKernelGGL((gemm_skinny_kernel<T, 4>), grid, dim3(SK_THREADS), smem(4), current_stream(), g, (float*)ws, k_per_block);
+    else {
+        auto kern = gemm_skinny_kernel<T, 8>;
+        if (smem(8) > 64 * 1024) attr = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem(8));
+        if (attr == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(SK_THREADS), smem(8), current_stream(), g, (float*)ws, k_per_block);
+    }
+    bool ok = check_hip(attr, "hipFuncSetAttribute") && check_launch("gemm_skinny_kernel");
+    if (ws) rp_hip_free(ws);      // stream-ordered reuse: the pool hands it out again only to later work on this stream
+    return ok ? 0 : -1;
+}
+
+int launch_generic(const GemmArgs& g, int dtype) {
+    RP_DISPATCH_DTYPE(dtype, return launch_generic_t<T>(g));
+    return -1;
+}
+
+int launch_skinny(const GemmArgs& g, int dtype) {
+    switch (dtype) {
+        case RP_DTYPE_FLOAT32:  return launch_skinny_t<float>(g);
+        case RP_DTYPE_FLOAT16:  return launch_skinny_t<f16_t>(g);
+        case RP_DTYPE_BFLOAT16: return launch_skinny_t<bf16_t>(g);
+        default: set_error("skinny GEMM: unsupported dtype %d", dtype); return -1;
+    }
+}
+
+}  // namespace rp
