@@ -60,6 +60,20 @@ const char* rp_hip_last_error(void);
 /* Stream the calling thread's launches go to; stream is a hipStream_t (NULL = null stream). */
 int rp_hip_set_stream(void* stream);
 void* rp_hip_get_stream(void);
+/* Streams (default priority, non-blocking) and the current stream's completion. */
+int rp_hip_stream_create(void** stream);
+int rp_hip_stream_destroy(void* stream);
+int rp_hip_stream_synchronize(void);
+/* HIP graphs: record what the calling thread enqueues on its current (created) stream between
+ * begin and end, then replay it with one launch.  The library's entry points only launch kernels
+ * (clears are fill kernels, never memset nodes), so recorded sequences replay exactly; run the
+ * sequence once before capturing so that the allocation pool already holds every block it needs,
+ * and keep host-blocking copies outside.  No counterpart in the reference, whose ops synchronise
+ * the device after every launch (core/cuda_helpers.cu:14-26). */
+int rp_hip_graph_capture_begin(void);
+int rp_hip_graph_capture_end(void** graph_exec);
+int rp_hip_graph_launch(void* graph_exec);
+int rp_hip_graph_destroy(void* graph_exec);
 /* HIP events on the current stream, for timing from hosts that have no HIP binding. */
 int rp_hip_event_create(void** event);
 int rp_hip_event_record(void* event);

@@ -13,7 +13,8 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 BUILD_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(LIB_DIR, "librp_hip.so")
-SOURCES = ["rp_runtime.hip", "rp_elementwise.hip", "rp_gemm.hip", "rp_gemm_generic.hip", "rp_gemm_mfma16.hip", "rp_gemm_mfmaw.hip"]
+SOURCES = ["rp_runtime.hip", "rp_elementwise.hip", "rp_gemm.hip", "rp_gemm_generic.hip", "rp_gemm_mfma16.hip", "rp_gemm_mfma16_256.hip",
+           "rp_gemm_mfma16_128.hip", "rp_gemm_mfma16_64.hip", "rp_gemm_mfma16_skinny.hip", "rp_gemm_mfmaw.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed-fp32 code generation is switched off for all device code
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
@@ -37,7 +38,7 @@ def build(extra_flags=(), verbose=True):
     os.makedirs(LIB_DIR, exist_ok=True)
     os.makedirs(BUILD_DIR, exist_ok=True)
     extra = list(extra_flags)
-    with ThreadPoolExecutor(max_workers=len(SOURCES)) as ex:
+    with ThreadPoolExecutor(max_workers=8) as ex:
         objs = list(ex.map(lambda s: _compile(s, extra), SOURCES))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
     res = subprocess.run(cmd, capture_output=True, text=True)

@@ -36,6 +36,13 @@ SIGNATURES = {
     "rp_hip_last_error": (ctypes.c_char_p, []),
     "rp_hip_set_stream": (_i, [_vp]),
     "rp_hip_get_stream": (_vp, []),
+    "rp_hip_stream_create": (_i, [ctypes.POINTER(_vp)]),
+    "rp_hip_stream_destroy": (_i, [_vp]),
+    "rp_hip_stream_synchronize": (_i, []),
+    "rp_hip_graph_capture_begin": (_i, []),
+    "rp_hip_graph_capture_end": (_i, [ctypes.POINTER(_vp)]),
+    "rp_hip_graph_launch": (_i, [_vp]),
+    "rp_hip_graph_destroy": (_i, [_vp]),
     "rp_hip_event_create": (_i, [ctypes.POINTER(_vp)]),
     "rp_hip_event_record": (_i, [_vp]),
     "rp_hip_event_synchronize": (_i, [_vp]),
@@ -148,6 +155,72 @@ def gemm(c_ptr, a_ptr, b_ptr, bias_ptr, batch, m, k, n, a_st, b_st, c_st, accumu
 def gemm_kernel_name(batch, m, k, n, a_rc, b_rc, c_rc, dtype):
     return lib().rp_hip_gemm_kernel_name(batch, m, k, n, *[int(s) for s in a_rc], *[int(s) for s in b_rc],
                                          *[int(s) for s in c_rc], dtype).decode()
+
+
+class Stream:
+    """A created stream; `with stream:` makes it the calling thread's current stream."""
+
+    def __init__(self):
+        p = _vp()
+        check(lib().rp_hip_stream_create(ctypes.byref(p)), "rp_hip_stream_create")
+        self.ptr = p.value
+        self._prev = None
+
+    def __enter__(self):
+        self._prev = lib().rp_hip_get_stream()
+        lib().rp_hip_set_stream(self.ptr)
+        return self
+
+    def __exit__(self, *exc):
+        lib().rp_hip_set_stream(self._prev)
+        return False
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                lib().rp_hip_stream_destroy(self.ptr)
+                self.ptr = None
+        except Exception:
+            pass
+
+
+class Graph:
+    """Capture of the calls made inside `with Graph.capture() as g:` on the current (created) stream."""
+
+    def __init__(self):
+        self.ptr = None
+
+    @classmethod
+    def capture(cls):
+        return _GraphCapture(cls())
+
+    def launch(self):
+        check(lib().rp_hip_graph_launch(self.ptr), "rp_hip_graph_launch")
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                lib().rp_hip_graph_destroy(self.ptr)
+                self.ptr = None
+        except Exception:
+            pass
+
+
+class _GraphCapture:
+    def __init__(self, graph):
+        self.graph = graph
+
+    def __enter__(self):
+        check(lib().rp_hip_graph_capture_begin(), "rp_hip_graph_capture_begin")
+        return self.graph
+
+    def __exit__(self, exc_type, exc, tb):
+        p = _vp()
+        rc = lib().rp_hip_graph_capture_end(ctypes.byref(p))
+        if exc_type is None:
+            check(rc, "rp_hip_graph_capture_end")
+            self.graph.ptr = p.value
+        return False
 
 
 class Event:

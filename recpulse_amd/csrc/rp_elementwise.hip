@@ -209,20 +209,18 @@ __global__ void backwards_softmax_strided_kernel(const T* gc, const T* y, T* gx,
 }
 
 // ---- reductions ----------------------------------------------------------------------
-// Deterministic two-level sum: each block sums a contiguous slab (threads
-// stride it, then a fixed-order LDS tree); block partials land in a
-// file-scope array and the block that finishes last adds them in index order.
-// Calls that overlap on one device would share the array: the library's
-// single-stream ordering keeps them apart.
+// Deterministic two-level sum in two launches: each block sums a contiguous slab
+// (threads stride it, then a fixed-order LDS tree) into a file-scope partials
+// array; a one-thread second kernel adds the partials in index order.  Calls that
+// overlap on one device would share the array: the library's single-stream
+// ordering keeps them apart.
 static constexpr int kMaxPartials = 1024;
 __device__ double g_partials[kMaxPartials];
-__device__ unsigned int g_partial_count;
 
 template <typename T>
-__global__ void sum_all_kernel(T* out, const T* x, size_t n, double scale) {
+__global__ void sum_partials_kernel(const T* x, size_t n) {
     using A = typename traits<T>::acc;
     __shared__ A red[kThreads];
-    __shared__ bool last;
     size_t per_block = (n + gridDim.x - 1) / gridDim.x;
     size_t lo = (size_t)blockIdx.x * per_block;
     size_t hi = lo + per_block < n ? lo + per_block : n;
@@ -234,21 +232,16 @@ __global__ void sum_all_kernel(T* out, const T* x, size_t n, double scale) {
         if ((int)threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
         __syncthreads();
     }
-    if (threadIdx.x == 0) {
-        g_partials[blockIdx.x] = (double)red[0];
-        __threadfence();
-        unsigned int done = atomicAdd(&g_partial_count, 1u);
-        last = (done == gridDim.x - 1);
-    }
-    __syncthreads();
-    if (last && threadIdx.x == 0) {
-        __threadfence();
-        A total = 0;
-        for (unsigned b = 0; b < gridDim.x; b++) total += (A)((volatile double*)g_partials)[b];
-        if (scale != 1.0) total = (A)(total / (A)scale);
-        out[0] = narrow<T>(total);
-        g_partial_count = 0;
-    }
+    if (threadIdx.x == 0) g_partials[blockIdx.x] = (double)red[0];
+}
+
+template <typename T>
+__global__ void sum_finish_kernel(T* out, int nparts, double scale) {
+    using A = typename traits<T>::acc;
+    A total = 0;
+    for (int b = 0; b < nparts; b++) total += (A)g_partials[b];
+    if (scale != 1.0) total = (A)(total / (A)scale);
+    out[0] = narrow<T>(total);
 }
 
 // reduce the middle axis of [outer, dim, inner]; one thread per output, serial in dim
@@ -480,9 +473,11 @@ int contiguous_copy_kernel_device(void* out, const void* in, int ndim, int* shap
 static int sum_all_any(void* out, const void* x, size_t size, int dtype, double scale) {
     RP_REQUIRE(out && x && size, "sum_all_kernel_device");
     unsigned blocks = grid_for(size, kThreads * 16, kMaxPartials);
-    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(sum_all_kernel<T>, dim3(blocks), dim3(kThreads), 0, current_stream(),
-                                               (T*)out, (const T*)x, size, scale));
-    return check_launch("sum_all_kernel") ? 0 : -1;
+    RP_DISPATCH_DTYPE(dtype, {
+        hipLaunchKernelGGL(sum_partials_kernel<T>, dim3(blocks), dim3(kThreads), 0, current_stream(), (const T*)x, size);
+        hipLaunchKernelGGL(sum_finish_kernel<T>, dim3(1), dim3(1), 0, current_stream(), (T*)out, (int)blocks, scale);
+    });
+    return check_launch("sum_all kernels") ? 0 : -1;
 }
 
 int sum_all_kernel_device(void* out, const void* x, size_t size, int dtype) { return sum_all_any(out, x, size, dtype, 1.0); }

@@ -49,7 +49,8 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     (void)c_rs; (void)c_cs;
 
     // skinny: few rows, row-major B, enough columns and depth to be worth streaming
-    if (batch == 1 && dtype != RP_DTYPE_FLOAT64 && m <= SK_MAX_M && b_mc && n >= 64 * vec && (long long)k * n >= (1ll << 20) &&
+    const int valu_rows = (dtype == RP_DTYPE_FLOAT32) ? SK_MAX_M : 4;        // 16-bit inputs with more rows go to the MFMA skinny kernel
+    if (batch == 1 && dtype != RP_DTYPE_FLOAT64 && m <= valu_rows && b_mc && n >= 64 * vec && (long long)k * n >= (1ll << 20) &&
         (n + 64 * vec - 1) / (64 * vec) <= SK_MAX_GROUPS) {
         p.fam = FAM_SKINNY; p.name = "skinny"; p.b_mc = true;
         return p;
@@ -62,6 +63,11 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     p.b_mc = b_mc;
 
     if (dtype == RP_DTYPE_FLOAT16 || dtype == RP_DTYPE_BFLOAT16) {
+        // few rows, deep k: split k over many blocks so that B streams at HBM speed (output columns in whole 8s)
+        if (batch == 1 && m <= 32 && n % 8 == 0 && n >= 256 && k >= 1024 && (long long)k * n >= (1ll << 22)) {
+            p.fam = FAM_MFMA16_SKINNY; p.bm = 32; p.bn = 128; p.edge = true; p.name = "mfma16_skinny_32x128";
+            return p;
+        }
         p.fam = FAM_MFMA16;
         long long tiles256 = (long long)((m + 255) / 256) * ((n + 255) / 256) * batch;
         if (m >= 256 && n >= 256 && tiles256 >= 128) { p.bm = 256; p.bn = 256; p.name = "mfma16_256x256"; }
@@ -81,7 +87,8 @@ static int run_gemm(const GemmArgs& g, int dtype) {
     Plan p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype);
     if (p.fam != FAM_GENERIC && !(aligned16(g.A) && aligned16(g.B))) p.fam = FAM_GENERIC;
     switch (p.fam) {
-        case FAM_MFMA16: return launch_mfma16(g, p, dtype);
+        case FAM_MFMA16:
+        case FAM_MFMA16_SKINNY: return launch_mfma16(g, p, dtype);
         case FAM_MFMAW:  return launch_mfmaw(g, p, dtype);
         case FAM_SKINNY: return launch_skinny(g, dtype);
         default:         return launch_generic(g, dtype);

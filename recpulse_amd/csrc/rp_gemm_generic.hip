@@ -90,12 +90,13 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g) {
 // (one 16-byte load per k row) and a wave covers 64*VEC columns.  The 8 waves
 // of a block share a column group and take interleaved k rows of the block's
 // k range; they combine through LDS in a fixed tree.  The grid's second axis
-// splits k further: split partials go to a workspace, and the block that
-// arrives last for a column group adds them in split order (so the result
-// does not depend on scheduling) and runs the epilogue.
+// splits k further: split partials go to a workspace and a small second kernel
+// adds them in split order (so the result does not depend on scheduling) and
+// runs the epilogue.  (A single-kernel "last block reduces" scheme needs
+// device-scope fences, which write back and invalidate the whole per-XCD L2
+// and cost far more than the second launch.)
 // ============================================================================
 constexpr int SK_THREADS = 512, SK_WAVES = SK_THREADS / 64;
-__device__ unsigned int g_skinny_arrivals[SK_MAX_GROUPS];     // zero at load; the last block of a group re-zeroes its slot
 
 template <typename T, int MROWS>
 __global__ void __launch_bounds__(SK_THREADS) gemm_skinny_kernel(GemmArgs g, float* partials, int k_per_block) {
@@ -202,7 +203,7 @@ __global__ void __launch_bounds__(SK_THREADS) gemm_skinny_kernel(GemmArgs g, flo
         return;
     }
 
-    // partial layout: [split][row][n] fp32
+    // partial layout: [split][row][n] fp32; a second kernel adds the splits in order and runs the epilogue
     if (wave == 0 && col_ok) {
 #pragma unroll
         for (int r = 0; r < MROWS; r++) {
@@ -212,40 +213,50 @@ __global__ void __launch_bounds__(SK_THREADS) gemm_skinny_kernel(GemmArgs g, flo
             for (int e = 0; e < VEC; e += 4) *(f32x4_t*)(q + e) = f32x4_t{acc[r][e], acc[r][e + 1], acc[r][e + 2], acc[r][e + 3]};
         }
     }
-    __shared__ bool last;
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned int done = atomicAdd(&g_skinny_arrivals[blockIdx.x], 1u);
-        last = (done == (unsigned)nsplit - 1);
+}
+
+// Sum the k-split partials [nsplit][m][n] in split order (fixed, so results do not depend on scheduling),
+// then bias / accumulate / narrow.  One thread per 4 adjacent columns of one row (n is a multiple of 4);
+// loads are issued eight splits at a time so the sum is not a chain of dependent memory latencies.
+template <typename T>
+__global__ void __launch_bounds__(256) gemm_splitk_combine_kernel(GemmArgs g, const float* partials, int nsplit, int part_rows) {
+    const int quads = g.n / 4;
+    const int item = blockIdx.x * 256 + threadIdx.x;
+    if (item >= g.m * quads) return;
+    const int r = item / quads, c0 = (item - r * quads) * 4;
+    f32x4_t sum = {0.f, 0.f, 0.f, 0.f};
+    const float* q = partials + (long long)r * g.n + c0;
+    const long long split_stride = (long long)part_rows * g.n;
+    int s = 0;
+    for (; s + 8 <= nsplit; s += 8) {
+        f32x4_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = *(const f32x4_t*)(q + (s + u) * split_stride);
+#pragma unroll
+        for (int u = 0; u < 8; u++) sum += v[u];
     }
-    __syncthreads();
-    if (!last) return;
-    __threadfence();
-    // the last block: one (row, 64-lane column vector) item per thread, splits added in order
-    {
-        const int r = threadIdx.x >> 6;
-        if (r < g.m && col_ok) {
-            float sum[VEC];
+    for (; s < nsplit; s++) sum += *(const f32x4_t*)(q + s * split_stride);
+    T* C = (T*)g.C;
+    const T* bias = (const T*)g.bias;
+    const bool has_bias = bias != nullptr, accum = g.accumulate != 0;
 #pragma unroll
-            for (int e = 0; e < VEC; e++) sum[e] = 0.f;
-            for (int s = 0; s < nsplit; s++) {
-                const float* q = partials + ((long long)s * g.m + r) * g.n + col0;
-#pragma unroll
-                for (int e = 0; e < VEC; e += 4) {
-                    f32x4_t v = *(const f32x4_t*)(q + e);
-                    sum[e] += v[0]; sum[e + 1] += v[1]; sum[e + 2] += v[2]; sum[e + 3] += v[3];
-                }
-            }
-#pragma unroll
-            for (int e = 0; e < VEC; e++) {
-                T* p = C + (long long)r * g.c_rs + (long long)(col0 + e) * g.c_cs;
-                T old = accum ? *p : T{};
-                *p = finish<T>(sum[e], has_bias, has_bias ? bias[col0 + e] : T{}, accum, old);
-            }
-        }
+    for (int e = 0; e < 4; e++) {
+        T* p = C + (long long)r * g.c_rs + (long long)(c0 + e) * g.c_cs;
+        T old = accum ? *p : T{};
+        *p = finish<T>(sum[e], has_bias, has_bias ? bias[c0 + e] : T{}, accum, old);
     }
-    if (threadIdx.x == 0) g_skinny_arrivals[blockIdx.x] = 0;
+}
+
+int launch_splitk_combine(const GemmArgs& g, const float* partials, int nsplit, int part_rows, int dtype) {
+    int items = g.m * (g.n / 4);
+    dim3 grid((items + 255) / 256);
+    switch (dtype) {
+        case RP_DTYPE_FLOAT32:  hipLaunchKernelGGL(gemm_splitk_combine_kernel<float>, grid, dim3(256), 0, current_stream(), g, partials, nsplit, part_rows); break;
+        case RP_DTYPE_FLOAT16:  hipLaunchKernelGGL(gemm_splitk_combine_kernel<f16_t>, grid, dim3(256), 0, current_stream(), g, partials, nsplit, part_rows); break;
+        case RP_DTYPE_BFLOAT16: hipLaunchKernelGGL(gemm_splitk_combine_kernel<bf16_t>, grid, dim3(256), 0, current_stream(), g, partials, nsplit, part_rows); break;
+        default: set_error("split-k combine: unsupported dtype %d", dtype); return -1;
+    }
+    return check_launch("gemm_splitk_combine_kernel") ? 0 : -1;
 }
 
 template <typename T>
@@ -293,6 +304,7 @@ static int launch_skinny_t(const GemmArgs& g) {
         if (attr == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(SK_THREADS), smem(8), current_stream(), g, (float*)ws, k_per_block);
     }
     bool ok = check_hip(attr, "hipFuncSetAttribute") && check_launch("gemm_skinny_kernel");
+    if (ok && nsplit > 1) ok = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, traits<T>::code) == 0;
     if (ws) rp_hip_free(ws);      // stream-ordered reuse: the pool hands it out again only to later work on this stream
     return ok ? 0 : -1;
 }

@@ -1,404 +1,18 @@
-// bf16 / fp16 MFMA GEMM kernels (fp32 accumulate) and their launcher.
+// bf16 / fp16 MFMA GEMM: tile selection across the per-tile translation units.
 #include "rp_gemm.h"
-
-#include <type_traits>
 
 namespace rp {
 
-// ============================================================================
-// mfma16: bf16 / fp16 inputs, fp32 accumulate.
-//
-// Block tile BM x BN, k slab 64, 256 threads = 4 waves in a 2x2 grid (one wave
-// per SIMD), each wave owning a (BM/2) x (BN/2) patch of 32x32x16 MFMA tiles.
-//
-// Software pipeline, per slab s (4 k-steps of 16):
-//   k-step 0   MFMAs on fragments(0) | read fragments(1) | A regs of slab s+1 -> other LDS buffer | issue global loads of A, slab s+2
-//   k-step 1   MFMAs on fragments(1) | read fragments(2) | B regs of slab s+1 -> other LDS buffer | issue global loads of B, slab s+2
-//   k-step 2   MFMAs on fragments(2) | read fragments(3)
-//   barrier    (slab s+1 is now complete in LDS, and nobody reads this slab's buffer any more)
-//   k-step 3   MFMAs on fragments(3) | read fragments(0) of slab s+1
-// so LDS reads run one k-step ahead of the MFMAs that use them, global loads
-// have more than a full slab of MFMA time to land, and the single barrier per
-// slab sits where only one MFMA group is left to issue.  sched_group_barrier
-// sequences pin the interleaving (one MFMA, then its share of DS / VMEM work).
-//
-// LDS layouts (16-bit elements):
-//   KC operand: [rows][64 + 8]   row pitch 144 B -> the 16 rows a quarter-wave
-//               reads with ds_read_b128 land in 16 different 16-byte bank groups
-//   MC operand: [64][cols + 32]  row pitch 2*cols + 64 B -> the 4 k-rows a
-//               16-lane group reads with ds_read_b64_tr_b16 start 16 banks apart
-// The epilogue stages fp32 accumulators through the (now idle) LDS so that each
-// lane narrows and stores 8 adjacent columns with one 16-byte store.
-// ============================================================================
-template <typename T> struct mfma16_ops;
-template <> struct mfma16_ops<bf16_t> {
-    static __device__ __forceinline__ f32x16_t mma(s16x8_t a, s16x8_t b, f32x16_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-    }
-};
-template <> struct mfma16_ops<f16_t> {
-    static __device__ __forceinline__ f32x16_t mma(s16x8_t a, s16x8_t b, f32x16_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
-    }
-};
-
-constexpr int M16_KC_PITCH = M16_BK + 8;                       // elements
-__host__ __device__ constexpr int m16_mc_pitch(int cols) { return cols + 32; }
-__host__ __device__ constexpr int m16_tile_elems(int rows, bool mc) {
-    return mc ? M16_BK * m16_mc_pitch(rows) : rows * M16_KC_PITCH;
-}
-__host__ __device__ constexpr int m16_epi_cols(int wn) { return wn >= 64 ? 64 : wn; }      // columns staged per epilogue pass
-__host__ __device__ constexpr size_t m16_smem_bytes(int bm, int bn, bool a_mc, bool b_mc) {
-    size_t loop = 2 * (size_t)(m16_tile_elems(bm, a_mc) + m16_tile_elems(bn, b_mc)) * 2;
-    size_t epi = 4 * (size_t)(bm / 2) * (m16_epi_cols(bn / 2) + 4) * 4;
-    return loop > epi ? loop : epi;
-}
-
-typedef uint16_t __attribute__((address_space(3))) lds_u16;
-
-
-template <int I, int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
-
-// Raw buffer descriptor over [base, base + bytes): loads past the end return zero.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t m16_rsrc(const void* base, long long bytes) {
-    int n = bytes <= 0 ? 0 : (bytes > 0x7fffffffll ? 0x7fffffff : (int)bytes);
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, n, 0x00020000);
-}
-constexpr uint32_t M16_OOB = 0x80000000u;        // an offset no descriptor covers
-
-// Per-thread constants of one operand's slab traffic: NL 16-byte pieces per slab; piece i sits a fixed
-// number of rows (KC) or k-rows (MC) after piece 0, so LDS offsets are piece 0's plus a compile-time step.
-template <int ROWS, bool MC>
-struct SlabMap {
-    static constexpr int NL = ROWS * 8 / 256;
-    static constexpr int PIECE_ROWS = MC ? 256 / (ROWS / 8) : 32;        // k-rows (MC) or free rows (KC) between consecutive pieces
-    static constexpr int LDS_STEP = MC ? PIECE_ROWS * m16_mc_pitch(ROWS) : PIECE_ROWS * M16_KC_PITCH;   // elements
-    // piece 0 of thread t: free index r (first of 8 for MC) and slab-local k (first of 8 for KC)
-    static __device__ __forceinline__ void coords0(int t, int& r, int& kk) {
-        if (MC) { kk = t / (ROWS / 8); r = (t % (ROWS / 8)) * 8; }
-        else    { r = t / 8; kk = (t % 8) * 8; }
-    }
-    static __device__ __forceinline__ int lds_off(int r, int kk) {          // element offset inside the operand's LDS tile
-        return MC ? kk * m16_mc_pitch(ROWS) + r : r * M16_KC_PITCH + kk;
-    }
-};
-
-// Lane's base element offset for MFMA fragments of an operand tile whose wave patch starts at free index w0.
-// Fragment (tile i, k-step ks, read h) then sits at base + step(i, ks, h), a compile-time constant.
-template <int ROWS, bool MC>
-struct FragMap {
-    static __device__ __forceinline__ int base(int w0, int lane) {
-        if (!MC) return (w0 + (lane & 31)) * M16_KC_PITCH + (lane >> 5) * 8;
-        // ds_read_b64_tr_b16: inside each 16-lane group, source lane s points at 4 consecutive free
-        // indices of k-row s/4; destination lane j receives free index j of k-rows 0..3.
-        int grp = lane >> 4, s = lane & 15;
-        return (8 * (grp >> 1) + (s >> 2)) * m16_mc_pitch(ROWS) + w0 + 16 * (grp & 1) + 4 * (s & 3);
-    }
-    static constexpr int READS = MC ? 2 : 1;                 // DS instructions per fragment
-    static constexpr int step(int i, int ks, int h) {
-        return MC ? ks * 16 * m16_mc_pitch(ROWS) + i * 32 + h * 4 * m16_mc_pitch(ROWS)
-                  : i * 32 * M16_KC_PITCH + ks * 16;
-    }
-    // DS read H of the fragment into v (KC: the whole fragment; MC: k values 4H .. 4H+3)
-    template <int H>
-    static __device__ __forceinline__ void read(s16x8_t& v, const uint16_t* p) {
-        if constexpr (!MC) {
-            v = *(const s16x8_t*)p;
-        } else {
-            s16x4_t q = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3)))*)(lds_u16*)p);
-            v[4 * H + 0] = q[0]; v[4 * H + 1] = q[1]; v[4 * H + 2] = q[2]; v[4 * H + 3] = q[3];
-        }
-    }
-};
-
-template <typename T, int BM, int BN, bool A_MC, bool B_MC, bool EDGE>
-__global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_m, int tiles_n) {
-    constexpr int WM = BM / 2, WN = BN / 2;           // wave patch
-    constexpr int TMI = WM / 32, TNI = WN / 32;       // MFMA tiles per wave
-    constexpr int A_ELEMS = m16_tile_elems(BM, A_MC), B_ELEMS = m16_tile_elems(BN, B_MC);
-    constexpr int STAGE = A_ELEMS + B_ELEMS;          // stage s: A at smem + s*STAGE, B right after it
-    using MapA = SlabMap<BM, A_MC>;
-    using MapB = SlabMap<BN, B_MC>;
-    using FragA = FragMap<BM, A_MC>;
-    using FragB = FragMap<BN, B_MC>;
-    constexpr int NA = MapA::NL, NB = MapB::NL;
-    constexpr int RD_A = TMI * FragA::READS, RD_B = TNI * FragB::READS;      // DS read instructions per k-step
-    constexpr int NMFMA = TMI * TNI;
-    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-
-    TileCoord tc = schedule_tile(blockIdx.x, tiles_m, tiles_n);
-    if (!tc.valid) return;
-    const int z = blockIdx.y;
-    const int m0 = tc.tm * BM, n0 = tc.tn * BN;
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
-
-    // A: free axis = m (stride a_rs), k stride a_cs.  B: free axis = n (stride b_cs), k stride b_rs.
-    const long long a_fs = g.a_rs, a_ks = g.a_cs, b_fs = g.b_cs, b_ks = g.b_rs;
-    const uint16_t* a_mat = (const uint16_t*)g.A + (long long)z * g.a_bs;
-    const uint16_t* b_mat = (const uint16_t*)g.B + (long long)z * g.b_bs;
-    // uniform pointers to the tile's current slab and one past the operand's last valid element
-    const char* a_slab = (const char*)(a_mat + (long long)m0 * a_fs);
-    const char* b_slab = (const char*)(b_mat + (long long)n0 * b_fs);
-    const char* a_end = (const char*)(a_mat + ((long long)(g.m - 1) * a_fs + (long long)(g.k - 1) * a_ks + 1));
-    const char* b_end = (const char*)(b_mat + ((long long)(g.n - 1) * b_fs + (long long)(g.k - 1) * b_ks + 1));
-    const long long a_step = (long long)M16_BK * a_ks * 2, b_step = (long long)M16_BK * b_ks * 2;
-
-    // Per-thread piece offsets (bytes from the slab pointer).  The buffer descriptor ends at the operand's last
-    // element, which zero-fills rows past the free extent (KC) or k past the end (MC); the other axis of each
-    // layout is masked explicitly by swapping in an offset no descriptor covers.
-    uint32_t a_goff[NA], b_goff[NB];
-    int a_r0, a_kk0, b_r0, b_kk0;
-    MapA::coords0(t, a_r0, a_kk0);
-    MapB::coords0(t, b_r0, b_kk0);
-#pragma unroll
-    for (int i = 0; i < NA; i++) {
-        int r = a_r0 + (A_MC ? 0 : i * MapA::PIECE_ROWS), kk = a_kk0 + (A_MC ? i * MapA::PIECE_ROWS : 0);
-        a_goff[i] = (uint32_t)(((long long)r * a_fs + (long long)kk * a_ks) * 2);
-        if (EDGE && A_MC && m0 + r >= g.m) a_goff[i] = M16_OOB;
-    }
-#pragma unroll
-    for (int i = 0; i < NB; i++) {
-        int r = b_r0 + (B_MC ? 0 : i * MapB::PIECE_ROWS), kk = b_kk0 + (B_MC ? i * MapB::PIECE_ROWS : 0);
-        b_goff[i] = (uint32_t)(((long long)r * b_fs + (long long)kk * b_ks) * 2);
-        if (EDGE && B_MC && n0 + r >= g.n) b_goff[i] = M16_OOB;
-    }
-    const int a_wr0 = MapA::lds_off(a_r0, a_kk0), b_wr0 = A_ELEMS + MapB::lds_off(b_r0, b_kk0);     // LDS element offsets of piece 0
-    const int a_fr0 = FragA::base(wm0, lane), b_fr0 = A_ELEMS + FragB::base(wn0, lane);
-
-    f32x16_t acc[TMI][TNI];
-#pragma unroll
-    for (int i = 0; i < TMI; i++)
-#pragma unroll
-        for (int j = 0; j < TNI; j++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
-
-    u32x4_t ra[NA], rb[NB];
-    const int nslabs = (g.k + M16_BK - 1) / M16_BK;
-    __amdgpu_buffer_rsrc_t a_rsrc, b_rsrc;
-    int kleft = 0;        // k still in range counted from the slab the descriptors point at (EDGE, KC operands)
-
-    auto point_at_slab = [&](int k0) {
-        a_rsrc = m16_rsrc(a_slab, EDGE ? (long long)(a_end - a_slab) : 0x7fffffffll);
-        b_rsrc = m16_rsrc(b_slab, EDGE ? (long long)(b_end - b_slab) : 0x7fffffffll);
-        kleft = g.k - k0;
-    };
-    auto load_piece_a = [&](auto ic) {
-        constexpr int i = decltype(ic)::value;
-        uint32_t off = a_goff[i];
-        if (EDGE && !A_MC && a_kk0 >= kleft) off = M16_OOB;
-        ra[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)off, 0, 0);
-    };
-    auto load_piece_b = [&](auto ic) {
-        constexpr int i = decltype(ic)::value;
-        uint32_t off = b_goff[i];
-        if (EDGE && !B_MC && b_kk0 >= kleft) off = M16_OOB;
-        rb[i] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, (int)off, 0, 0);
-    };
-    auto store_piece_a = [&](uint16_t* stage, auto ic) {
-        constexpr int i = decltype(ic)::value;
-        *(u32x4_t*)(stage + a_wr0 + i * MapA::LDS_STEP) = ra[i];
-    };
-    auto store_piece_b = [&](uint16_t* stage, auto ic) {
-        constexpr int i = decltype(ic)::value;
-        *(u32x4_t*)(stage + b_wr0 + i * MapB::LDS_STEP) = rb[i];
-    };
-
-    s16x8_t af[2][TMI], bf[2][TNI];
-    // DS read number r (0 .. RD_A+RD_B-1) of the fragments for k-step KS into fragment slot SLOT
-    auto read_item = [&](const uint16_t* stage, auto ksc, auto slotc, auto rc) {
-        constexpr int KS = decltype(ksc)::value, SLOT = decltype(slotc)::value, r = decltype(rc)::value;
-        if constexpr (r < RD_A) {
-            constexpr int i = r / FragA::READS, h = r % FragA::READS;
-            FragA::template read<h>(af[SLOT][i], stage + a_fr0 + FragA::step(i, KS, h));
-        } else {
-            constexpr int q = r - RD_A, j = q / FragB::READS, h = q % FragB::READS;
-            FragB::template read<h>(bf[SLOT][j], stage + b_fr0 + FragB::step(j, KS, h));
-        }
-    };
-
-    using I0 = std::integral_constant<int, 0>;
-    using I1 = std::integral_constant<int, 1>;
-    using I2 = std::integral_constant<int, 2>;
-    using I3 = std::integral_constant<int, 3>;
-
-    // ---- prologue: slab 0 into LDS buffer 0, slab 1 into registers, fragments(0) of slab 0 ----
-    point_at_slab(0);
-    static_for<0, NA>([&](auto ic) { load_piece_a(ic); });
-    static_for<0, NB>([&](auto ic) { load_piece_b(ic); });
-    static_for<0, NA>([&](auto ic) { store_piece_a(smem, ic); });
-    static_for<0, NB>([&](auto ic) { store_piece_b(smem, ic); });
-    a_slab += a_step;
-    b_slab += b_step;
-    if (nslabs > 1) {
-        point_at_slab(M16_BK);
-        static_for<0, NA>([&](auto ic) { load_piece_a(ic); });
-        static_for<0, NB>([&](auto ic) { load_piece_b(ic); });
-    }
-    a_slab += a_step;
-    b_slab += b_step;
-    __syncthreads();
-    static_for<0, RD_A + RD_B>([&](auto rc) { read_item(smem, I0{}, I0{}, rc); });
-
-    // One k-step: NMFMA micro-steps, each one MFMA on fragment slot MSLOT followed by its share of the side
-    // work (fragment reads for k-step RKS into the other slot; LDS stores and global loads of operand OP:
-    // 0 none, 1 A, 2 B).  A scheduling barrier closes every micro-step so the interleaving is the one written.
-    auto kstep = [&](auto mslotc, auto rksc, auto readc, auto wrc, auto ldc, const uint16_t* rd_stage, uint16_t* wr_stage) {
-        constexpr int MSLOT = decltype(mslotc)::value;
-        constexpr bool DO_READ = decltype(readc)::value;
-        constexpr int WR = decltype(wrc)::value, LD = decltype(ldc)::value;
-        constexpr int NR = DO_READ ? RD_A + RD_B : 0;
-        constexpr int NW = WR == 1 ? NA : (WR == 2 ? NB : 0);
-        constexpr int NG = LD == 1 ? NA : (LD == 2 ? NB : 0);
-        static_for<0, NMFMA>([&](auto qc) {
-            constexpr int q = decltype(qc)::value, i = q / TNI, j = q % TNI;
-            acc[i][j] = mfma16_ops<T>::mma(af[MSLOT][i], bf[MSLOT][j], acc[i][j]);
-            static_for<(NR * q) / NMFMA, (NR * (q + 1)) / NMFMA>([&](auto rc) {
-                read_item(rd_stage, rksc, std::integral_constant<int, MSLOT ^ 1>{}, rc);
-            });
-            static_for<(NW * q) / NMFMA, (NW * (q + 1)) / NMFMA>([&](auto ic) {
-                if constexpr (WR == 1) store_piece_a(wr_stage, ic);
-                else store_piece_b(wr_stage, ic);
-            });
-            static_for<(NG * q) / NMFMA, (NG * (q + 1)) / NMFMA>([&](auto ic) {
-                if constexpr (LD == 1) load_piece_a(ic);
-                else load_piece_b(ic);
-            });
-            __builtin_amdgcn_sched_barrier(0);
-        });
-    };
-
-    int cur = 0;
-    // One slab of the pipeline.  NEXT: slab s+1 exists (its registers are written to LDS here and the barrier runs);
-    // NEXT2: slab s+2 exists (its global loads are issued here).
-    auto slab_step = [&](int s, auto next_tag, auto next2_tag) {
-        constexpr bool NEXT = decltype(next_tag)::value, NEXT2 = decltype(next2_tag)::value;
-        using WrA = std::integral_constant<int, NEXT ? 1 : 0>;
-        using WrB = std::integral_constant<int, NEXT ? 2 : 0>;
-        using LdA = std::integral_constant<int, NEXT2 ? 1 : 0>;
-        using LdB = std::integral_constant<int, NEXT2 ? 2 : 0>;
-        const uint16_t* stage = smem + cur * STAGE;
-        uint16_t* other = smem + (cur ^ 1) * STAGE;
-        if constexpr (NEXT2) point_at_slab((s + 2) * M16_BK);
-        kstep(I0{}, I1{}, std::true_type{}, WrA{}, LdA{}, stage, other);
-        kstep(I1{}, I2{}, std::true_type{}, WrB{}, LdB{}, stage, other);
-        kstep(I0{}, I3{}, std::true_type{}, I0{}, I0{}, stage, other);
-        if constexpr (NEXT) __syncthreads();
-        kstep(I1{}, I0{}, std::integral_constant<bool, NEXT>{}, I0{}, I0{}, other, other);
-        a_slab += a_step;
-        b_slab += b_step;
-        cur ^= 1;
-    };
-
-    using yes = std::true_type;
-    using no = std::false_type;
-    int s = 0;
-    for (; s + 2 < nslabs; s++) slab_step(s, yes{}, yes{});
-    if (s + 1 < nslabs) { slab_step(s, yes{}, no{}); s++; }
-    slab_step(s, no{}, no{});
-
-    // ---- epilogue ----
-    // Pass p covers CN columns of every wave's patch: accumulators go to the wave's private fp32 LDS region
-    // [WM][CN + 4]; then each lane takes 8 adjacent columns of one row per step: narrow, bias, accumulate, one store.
-    constexpr int CN = m16_epi_cols(WN), EP = CN + 4, TJ = CN / 32, PASSES = WN / CN;
-    constexpr int LPR = CN / 8;                 // lanes per row
-    constexpr int RPS = 64 / LPR;               // rows per step
-    float* region = (float*)smem + wave * (WM * EP);
-    T* C = (T*)g.C + (long long)z * g.c_bs;
-    const T* bias = (const T*)g.bias;
-    const bool has_bias = bias != nullptr, accum = g.accumulate != 0;
-    const bool c_vec = (g.c_cs == 1) && (g.c_rs % 8 == 0) && (((uintptr_t)C & 15) == 0);
-    const int ecol = (lane % LPR) * 8, erow = lane / LPR;
-#pragma unroll
-    for (int p = 0; p < PASSES; p++) {
-        __syncthreads();                        // main loop (or the previous pass) is done with LDS
-#pragma unroll
-        for (int i = 0; i < TMI; i++)
-#pragma unroll
-            for (int jj = 0; jj < TJ; jj++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    int row = i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-                    region[row * EP + jj * 32 + (lane & 31)] = acc[i][p * TJ + jj][v];
-                }
-        __syncthreads();
-        const int gn = n0 + wn0 + p * CN + ecol;
-        T bv[8];
-#pragma unroll
-        for (int e = 0; e < 8; e++) bv[e] = (has_bias && (!EDGE || gn + e < g.n)) ? bias[gn + e] : T{};
-#pragma unroll 2
-        for (int r = erow; r < WM; r += RPS) {
-            const int gm = m0 + wm0 + r;
-            if (EDGE && gm >= g.m) break;
-            f32x4_t lo = *(const f32x4_t*)(region + r * EP + ecol);
-            f32x4_t hi = *(const f32x4_t*)(region + r * EP + ecol + 4);
-            float vals[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            T* crow = C + (long long)gm * g.c_rs;
-            if (c_vec && (!EDGE || gn + 8 <= g.n)) {
-                T out[8], old[8];
-                if (accum) { uint4 o = *(const uint4*)(crow + gn); memcpy(old, &o, 16); }
-#pragma unroll
-                for (int e = 0; e < 8; e++) out[e] = finish<T>(vals[e], has_bias, bv[e], accum, accum ? old[e] : T{});
-                uint4 o;
-                memcpy(&o, out, 16);
-                *(uint4*)(crow + gn) = o;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    if (EDGE && gn + e >= g.n) break;
-                    T* pc = crow + (long long)(gn + e) * g.c_cs;
-                    T old = accum ? *pc : T{};
-                    *pc = finish<T>(vals[e], has_bias, bv[e], accum, old);
-                }
-            }
-        }
-    }
-}
-
-template <typename T, int BM, int BN, bool A_MC, bool B_MC>
-static int launch_mfma16_edge(const GemmArgs& g, bool edge) {
-    int tiles_m = (g.m + BM - 1) / BM, tiles_n = (g.n + BN - 1) / BN;
-    dim3 grid(scheduled_grid(tiles_m, tiles_n), g.batch);
-    size_t smem = m16_smem_bytes(BM, BN, A_MC, B_MC);
-    if (edge) {
-        auto kern = gemm_mfma16_kernel<T, BM, BN, A_MC, B_MC, true>;
-        if (smem > 64 * 1024 && !check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem), "hipFuncSetAttribute")) return -1;
-        hipLaunchKernelGGL(kern, grid, dim3(256), smem, current_stream(), g, tiles_m, tiles_n);
-    } else {
-        auto kern = gemm_mfma16_kernel<T, BM, BN, A_MC, B_MC, false>;
-        if (smem > 64 * 1024 && !check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem), "hipFuncSetAttribute")) return -1;
-        hipLaunchKernelGGL(kern, grid, dim3(256), smem, current_stream(), g, tiles_m, tiles_n);
-    }
-    return check_launch("gemm_mfma16_kernel") ? 0 : -1;
-}
-
-template <typename T, int BM, int BN>
-static int launch_mfma16_layout(const GemmArgs& g, const Plan& p) {
-    if (!p.a_mc && p.b_mc) return launch_mfma16_edge<T, BM, BN, false, true>(g, p.edge);
-    if (!p.a_mc && !p.b_mc) return launch_mfma16_edge<T, BM, BN, false, false>(g, p.edge);
-    if (p.a_mc && p.b_mc) return launch_mfma16_edge<T, BM, BN, true, true>(g, p.edge);
-    return launch_mfma16_edge<T, BM, BN, true, false>(g, p.edge);
-}
-
-template <typename T>
-static int launch_mfma16_t(const GemmArgs& g, const Plan& p) {
-    if (p.bm == 256) return launch_mfma16_layout<T, 256, 256>(g, p);
-    if (p.bm == 128) return launch_mfma16_layout<T, 128, 128>(g, p);
-    return launch_mfma16_layout<T, 64, 64>(g, p);
-}
+int launch_mfma16_256(const GemmArgs& g, const Plan& p, int dtype);
+int launch_mfma16_128(const GemmArgs& g, const Plan& p, int dtype);
+int launch_mfma16_64(const GemmArgs& g, const Plan& p, int dtype);
+int launch_mfma16_skinny(const GemmArgs& g, const Plan& p, int dtype);
 
 int launch_mfma16(const GemmArgs& g, const Plan& p, int dtype) {
-    if (dtype == RP_DTYPE_BFLOAT16) return launch_mfma16_t<bf16_t>(g, p);
-    if (dtype == RP_DTYPE_FLOAT16) return launch_mfma16_t<f16_t>(g, p);
-    set_error("mfma16 GEMM: unsupported dtype %d", dtype);
-    return -1;
+    if (p.fam == FAM_MFMA16_SKINNY) return launch_mfma16_skinny(g, p, dtype);
+    if (p.bm == 256) return launch_mfma16_256(g, p, dtype);
+    if (p.bm == 128) return launch_mfma16_128(g, p, dtype);
+    return launch_mfma16_64(g, p, dtype);
 }
 
 }  // namespace rp

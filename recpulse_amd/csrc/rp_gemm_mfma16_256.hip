@@ -1,0 +1,8 @@
+// bf16 / fp16 MFMA GEMM, 256 x 256 block tile (2 x 2 waves).
+#include "rp_gemm_mfma16_kernel.h"
+
+namespace rp {
+
+int launch_mfma16_256(const GemmArgs& g, const Plan& p, int dtype) { return m16_launch_tile_dtype<256, 256, 2>(g, p, dtype); }
+
+}  // namespace rp

@@ -200,6 +200,51 @@ const char* rp_hip_last_error(void) { return g_error; }
 int rp_hip_set_stream(void* stream) { g_stream = (hipStream_t)stream; return 0; }
 void* rp_hip_get_stream(void) { return (void*)g_stream; }
 
+int rp_hip_stream_create(void** stream) {
+    if (!stream) { set_error("rp_hip_stream_create: null argument"); return -1; }
+    hipStream_t st;
+    if (!check_hip(hipStreamCreateWithFlags(&st, hipStreamNonBlocking), "hipStreamCreate")) return -1;   // default priority
+    *stream = (void*)st;
+    return 0;
+}
+
+int rp_hip_stream_destroy(void* stream) {
+    if (g_stream == (hipStream_t)stream) g_stream = nullptr;
+    return check_hip(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy") ? 0 : -1;
+}
+
+int rp_hip_stream_synchronize(void) {
+    return check_hip(hipStreamSynchronize(current_stream()), "hipStreamSynchronize") ? 0 : -1;
+}
+
+// Record everything the calling thread enqueues on its current stream (which must be a created stream, not
+// the null stream) into a graph.  Entry points of this library launch kernels only (clears are fill kernels,
+// not memset nodes), so a recorded sequence replays exactly; host-blocking copies must stay outside.
+int rp_hip_graph_capture_begin(void) {
+    if (!g_stream) { set_error("rp_hip_graph_capture_begin: set a created stream first (the null stream cannot be captured)"); return -1; }
+    return check_hip(hipStreamBeginCapture(g_stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture") ? 0 : -1;
+}
+
+int rp_hip_graph_capture_end(void** graph_exec) {
+    if (!graph_exec) { set_error("rp_hip_graph_capture_end: null argument"); return -1; }
+    hipGraph_t graph = nullptr;
+    if (!check_hip(hipStreamEndCapture(g_stream, &graph), "hipStreamEndCapture")) return -1;
+    hipGraphExec_t exec = nullptr;
+    bool ok = check_hip(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate");
+    (void)hipGraphDestroy(graph);
+    if (!ok) return -1;
+    *graph_exec = (void*)exec;
+    return 0;
+}
+
+int rp_hip_graph_launch(void* graph_exec) {
+    return check_hip(hipGraphLaunch((hipGraphExec_t)graph_exec, current_stream()), "hipGraphLaunch") ? 0 : -1;
+}
+
+int rp_hip_graph_destroy(void* graph_exec) {
+    return check_hip(hipGraphExecDestroy((hipGraphExec_t)graph_exec), "hipGraphExecDestroy") ? 0 : -1;
+}
+
 int rp_hip_event_create(void** event) {
     if (!event) { set_error("rp_hip_event_create: null argument"); return -1; }
     hipEvent_t ev;
