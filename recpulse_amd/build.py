@@ -49,5 +49,32 @@ def build(extra_flags=(), verbose=True):
     return LIB_PATH
 
 
+HOST_DIR = os.path.join(HERE, "host")
+DROPIN_DIR = os.path.join(HERE, "dropin")
+
+
+def build_host(verbose=True):
+    """Build the CPython extension `recpulse_cuda` (host tensor / autograd layer + pybind11 binding) into
+    recpulse_amd/dropin/, linked against lib/librp_hip.so.  Plain g++: the host layer includes no HIP header."""
+    import sysconfig
+    import pybind11
+    os.makedirs(DROPIN_DIR, exist_ok=True)
+    ext = sysconfig.get_config_var("EXT_SUFFIX")
+    out = os.path.join(DROPIN_DIR, "recpulse_cuda" + ext)
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall",
+           "-I" + pybind11.get_include(), "-I" + sysconfig.get_paths()["include"],
+           os.path.join(HOST_DIR, "rp_host.cpp"), os.path.join(HOST_DIR, "py_module.cpp"),
+           "-o", out, "-L" + LIB_DIR, "-lrp_hip", "-Wl,-rpath,$ORIGIN/../lib"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("host extension build failed:\n" + res.stderr)
+    if res.stderr.strip():
+        sys.stderr.write(res.stderr)
+    if verbose:
+        print(f"built {out}")
+    return out
+
+
 if __name__ == "__main__":
     build(sys.argv[1:])
+    build_host()

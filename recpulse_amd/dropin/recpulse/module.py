@@ -1,0 +1,121 @@
+"""Parameter bookkeeping (`Module`) and the affine layer (`Linear`).
+
+Behaviour kept from the reference's recpulse/module.py:
+  * a module records its parameters in `tracked` under their attribute names; assigning a
+    child module copies the child's entries under dotted names ("fc1.weight") and lists the
+    child (and its own children) in `_modules` (reference :14-26);
+  * `parameters()` is the tracked tensors that require grad (:37-44);
+  * `to()` moves every tracked tensor in place and re-arms requires_grad (:46-60);
+  * `load_state()` copies by name and ignores unknown names (:62-71);
+  * `Linear` stores its weight as [in_features, out_features] (not transposed), initialised
+    N(0, 1/in_features), bias zeros (:91-108), and computes x·W then + bias (:110-114).
+The forward pass issues ONE launch (GEMM with the bias add in its epilogue) through
+`Tensor.op_linear`; the two-op form the reference uses gives the same values and is kept as
+`forward_two_ops` for comparison.
+"""
+import math
+
+import recpulse_cuda as rp
+
+
+def _is_private(name):
+    return name == "tracked" or name.startswith("_")
+
+
+class Module:
+    def __init__(self):
+        self.tracked = {}
+        self._modules = {}
+        self._training = True
+
+    # -- registration ---------------------------------------------------------------
+    def track(self, name, tensor):
+        """Record `tensor` as a parameter (or buffer) called `name`; returns the tensor."""
+        self.tracked[name] = tensor
+        return tensor
+
+    def __setattr__(self, name, value):
+        if not _is_private(name) and isinstance(value, Module):
+            self._adopt(name, value)
+        object.__setattr__(self, name, value)
+
+    def _adopt(self, name, child):
+        self._modules[name] = child
+        self.tracked.update({f"{name}.{key}": tensor for key, tensor in child.tracked.items()})
+        self._modules.update({f"{name}.{key}": sub for key, sub in child._modules.items()})
+
+    # -- calling ----------------------------------------------------------------------
+    def forward(self, *args, **kwargs):
+        raise NotImplementedError(f"{type(self).__name__} does not define forward()")
+
+    def __call__(self, *args, **kwargs):
+        return self.forward(*args, **kwargs)
+
+    def keep(self, tensor):
+        return tensor
+
+    # -- views of the parameters -------------------------------------------------------
+    def learnable(self):
+        return {name: t for name, t in self.tracked.items() if t.requires_grad}
+
+    def frozen(self):
+        return {name: t for name, t in self.tracked.items() if not t.requires_grad}
+
+    def parameters(self):
+        return list(self.learnable().values())
+
+    def zero_grad(self):
+        for tensor in self.parameters():
+            tensor.zero_grad()
+
+    # -- placement and state -----------------------------------------------------------
+    def to(self, device=None, dtype=None):
+        where = {key: val for key, val in (("device", device), ("dtype", dtype)) if val is not None}
+        if where:
+            for tensor in self.tracked.values():
+                wanted_grad = tensor.requires_grad
+                tensor.to(inplace=True, **where)
+                if wanted_grad:
+                    tensor.requires_grad_(True)
+        return self
+
+    def load_state(self, state_dict):
+        for name in state_dict.keys() & self.tracked.keys():
+            target = self.tracked[name]
+            wanted_grad = target.requires_grad
+            target.copy_(state_dict[name])
+            if wanted_grad:
+                target.requires_grad_(True)
+
+    def state(self):
+        return dict(self.tracked)
+
+    def train(self):
+        return self._set_mode(True)
+
+    def eval(self):
+        return self._set_mode(False)
+
+    def _set_mode(self, training):
+        self._training = training
+        for child in self._modules.values():
+            child._set_mode(training)
+        return self
+
+
+class Linear(Module):
+    """y = x · W + b with W of shape [in_features, out_features]."""
+
+    def __init__(self, in_features, out_features, bias=True):
+        super().__init__()
+        self.in_features, self.out_features = in_features, out_features
+        init = rp.randn([in_features, out_features]).mul_scalar(1.0 / math.sqrt(in_features))
+        self.weight = self.track("weight", init.requires_grad_(True))
+        self.bias = self.track("bias", rp.zeros([out_features]).requires_grad_(True)) if bias else None
+
+    def forward(self, x):
+        return self.keep(x.op_linear(self.weight, self.bias))
+
+    def forward_two_ops(self, x):
+        out = self.keep(x.op_matmul(self.weight))
+        return out if self.bias is None else self.keep(out.op_add(self.bias))

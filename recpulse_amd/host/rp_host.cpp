@@ -1,0 +1,1056 @@
+// Host-side tensor, functional and autograd layer for the matmul path, written
+// against the C ABI in include/rp_hip.h.  Structure follows the reference's
+// three C layers (core / functional / ops) so that its Python-facing behaviour
+// can be reproduced; every citation below names the reference code whose
+// behaviour the function keeps.
+#include "rp_host.h"
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <unordered_map>
+#include <unordered_set>
+#include <vector>
+
+#include "../../include/rp_hip.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+void fail(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+// a device call failed: keep the device layer's own text
+int dev_fail(const char* what) {
+    fail("%s: %s", what, rp_hip_last_error());
+    return -1;
+}
+
+bool on_device(int device_id) {
+    return device_id >= 0 && rp_hip_set_device(device_id) == 0;
+}
+
+// ---- 16-bit conversions on the host, same bit rules as the device layer ----
+// (reference core/half_precision.h:20-97: exact widening, narrowing adds the first dropped bit)
+float f16_to_f32(uint16_t h) {
+    uint32_t s = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 0x1Fu, f = h & 0x3FFu, w;
+    float out;
+    if (e == 0) {
+        if (f == 0) { w = s; memcpy(&out, &w, 4); return out; }
+        out = ((float)f / 1024.0f) * (1.0f / 16384.0f);
+        return s ? -out : out;
+    }
+    w = (e == 0x1Fu) ? (s | 0x7F800000u | (f << 13)) : (s | ((e + 112u) << 23) | (f << 13));
+    memcpy(&out, &w, 4);
+    return out;
+}
+
+uint16_t f32_to_f16(float x) {
+    uint32_t w;
+    memcpy(&w, &x, 4);
+    uint32_t s = (w >> 16) & 0x8000u, e32 = (w >> 23) & 0xFFu, f = w & 0x7FFFFFu;
+    int e = (int)e32 - 112;
+    if (e32 == 0xFFu) return (uint16_t)(f ? (s | 0x7C00u | (f >> 13) | 1u) : (s | 0x7C00u));
+    if (e <= 0) {
+        if (e < -10) return (uint16_t)s;
+        f |= 0x800000u;
+        int sh = 14 - e;
+        return (uint16_t)((s | (f >> sh)) + ((f >> (sh - 1)) & 1u));
+    }
+    if (e >= 0x1F) return (uint16_t)(s | 0x7C00u);
+    return (uint16_t)((s | ((uint32_t)e << 10) | (f >> 13)) + ((f >> 12) & 1u));
+}
+
+float bf16_to_f32(uint16_t h) {
+    uint32_t w = (uint32_t)h << 16;
+    float out;
+    memcpy(&out, &w, 4);
+    return out;
+}
+
+uint16_t f32_to_bf16(float x) {
+    uint32_t w;
+    memcpy(&w, &x, 4);
+    return (uint16_t)((w >> 16) + ((w >> 15) & 1u));
+}
+
+double load_as_double(const void* p, size_t i, DType dt) {
+    switch (dt) {
+        case DTYPE_FLOAT32: return ((const float*)p)[i];
+        case DTYPE_FLOAT64: return ((const double*)p)[i];
+        case DTYPE_FLOAT16: return f16_to_f32(((const uint16_t*)p)[i]);
+        default: return bf16_to_f32(((const uint16_t*)p)[i]);
+    }
+}
+
+// the reference converts between dtypes through an fp32 pivot (core/tensor_host.c:130-207)
+void store_from_double(void* p, size_t i, DType dt, double v) {
+    switch (dt) {
+        case DTYPE_FLOAT32: ((float*)p)[i] = (float)v; break;
+        case DTYPE_FLOAT64: ((double*)p)[i] = v; break;
+        case DTYPE_FLOAT16: ((uint16_t*)p)[i] = f32_to_f16((float)v); break;
+        default: ((uint16_t*)p)[i] = f32_to_bf16((float)v); break;
+    }
+}
+
+void host_convert(void* dst, DType ddt, const void* src, DType sdt, size_t n) {
+    if (ddt == sdt) { memcpy(dst, src, n * dtype_size(ddt)); return; }
+    for (size_t i = 0; i < n; i++) {
+        double v = load_as_double(src, i, sdt);
+        if (ddt != DTYPE_FLOAT64 && sdt == DTYPE_FLOAT64) v = (double)(float)v;
+        store_from_double(dst, i, ddt, v);
+    }
+}
+
+size_t shape_size(int ndim, const int* shape) {
+    size_t n = 1;
+    for (int i = 0; i < ndim; i++) n *= (size_t)shape[i];
+    return n;
+}
+
+Tensor* alloc_header(DType dtype, int device_id, int ndim, const int* shape) {
+    if (ndim <= 0 || !shape || !dtype_size(dtype)) { fail("invalid shape or dtype"); return nullptr; }
+    for (int i = 0; i < ndim; i++) if (shape[i] <= 0) { fail("shape entries must be positive"); return nullptr; }
+    Tensor* t = (Tensor*)calloc(1, sizeof(Tensor));
+    if (!t) return nullptr;
+    t->dtype = dtype;
+    t->ndim = ndim;
+    t->size = shape_size(ndim, shape);
+    t->shape = (int*)malloc(sizeof(int) * ndim);
+    t->strides = (int*)malloc(sizeof(int) * ndim);
+    memcpy(t->shape, shape, sizeof(int) * ndim);
+    int s = 1;                                              // row-major strides in elements (reference core/tensor_host.c:31-35)
+    for (int d = ndim - 1; d >= 0; d--) { t->strides[d] = s; s *= shape[d]; }
+    t->device_id = device_id;
+    t->owns_data = true;
+    t->refcount = 1;
+    return t;
+}
+
+void release_storage(Tensor* t) {
+    if (!t->owns_data || !t->data) return;
+    if (t->device_id == -1) free(t->data);
+    else if (on_device(t->device_id)) rp_hip_free(t->data);
+    t->data = nullptr;
+}
+
+void free_grad_fn(GradFn* gf) {
+    if (!gf) return;
+    for (int i = 0; i < gf->num_inputs; i++)
+        if (gf->inputs[i] && gf->inputs[i] != gf->owner) free_tensor(gf->inputs[i]);        // releases what attach() retained
+    free(gf->inputs);
+    if (gf->saved_data) { if (gf->free_saved) gf->free_saved(gf->saved_data); else free(gf->saved_data); }
+    free(gf);
+}
+
+bool needs_grad(const Tensor* t) { return t && t->metadata && t->metadata->requires_grad; }
+
+Meta* ensure_meta(Tensor* t) {
+    if (!t->metadata) t->metadata = (Meta*)calloc(1, sizeof(Meta));
+    return t->metadata;
+}
+
+// Attach a GradFn to an op output; the node retains its inputs (reference ops/ops.c:11-19).
+GradFn* attach(Tensor* out, void (*backward)(GradFn*, Tensor*), std::initializer_list<Tensor*> inputs) {
+    Meta* m = ensure_meta(out);
+    m->requires_grad = true;
+    m->is_leaf = false;
+    GradFn* gf = (GradFn*)calloc(1, sizeof(GradFn));
+    gf->backward = backward;
+    gf->num_inputs = (int)inputs.size();
+    gf->inputs = (Tensor**)malloc(sizeof(Tensor*) * (gf->num_inputs ? gf->num_inputs : 1));
+    int i = 0;
+    for (Tensor* t : inputs) { gf->inputs[i++] = t; if (t && t != out) tensor_retain(t); }
+    gf->owner = out;
+    m->grad_fn = gf;
+    return gf;
+}
+
+bool same_shape(const Tensor* a, const Tensor* b) {
+    if (a->ndim != b->ndim) return false;
+    for (int i = 0; i < a->ndim; i++) if (a->shape[i] != b->shape[i]) return false;
+    return true;
+}
+
+Tensor* make_view(Tensor* x, int ndim, const int* shape, const int* strides, size_t elem_offset) {
+    Tensor* v = (Tensor*)calloc(1, sizeof(Tensor));
+    v->dtype = x->dtype;
+    v->ndim = ndim;
+    v->size = shape_size(ndim, shape);
+    v->shape = (int*)malloc(sizeof(int) * ndim);
+    v->strides = (int*)malloc(sizeof(int) * ndim);
+    memcpy(v->shape, shape, sizeof(int) * ndim);
+    memcpy(v->strides, strides, sizeof(int) * ndim);
+    v->device_id = x->device_id;
+    v->owns_data = false;
+    v->refcount = 1;
+    v->data = (char*)x->data + elem_offset * dtype_size(x->dtype);            // views point at their first element (reference functional/functional.c:1103)
+    v->base_tensor = x->base_tensor ? x->base_tensor : x;                    // ... and keep the root owner alive (:1110)
+    tensor_retain(v->base_tensor);
+    return v;
+}
+
+// dense tensor of the same values (new reference either way), like ensure_contiguous (reference ops/ops.c:21-25)
+Tensor* dense(Tensor* x) { return rp_is_contiguous(x) ? tensor_retain(x) : rp_contiguous(x); }
+
+// Accumulate rule of every backward function (reference ops/ops.c:6781-6788): the first gradient is stored,
+// later ones are added in place.  `g` is consumed.
+void accumulate_grad(Tensor* x, Tensor* g) {
+    if (!g) return;
+    Meta* m = ensure_meta(x);
+    if (!m->grad) { m->grad = g; return; }
+    if (m->grad->device_id >= 0) {
+        if (on_device(x->device_id)) add_kernel_device(m->grad->data, m->grad->data, g->data, x->size, x->dtype);
+    }
+    free_tensor(g);
+}
+
+std::mt19937_64 g_rng(0x2545F4914F6CDD1Dull);
+
+}  // namespace
+
+extern "C" {
+
+size_t dtype_size(DType dtype) {
+    switch (dtype) {
+        case DTYPE_FLOAT32: return 4;
+        case DTYPE_FLOAT64: return 8;
+        case DTYPE_FLOAT16: return 2;
+        case DTYPE_BFLOAT16: return 2;
+        default: return 0;
+    }
+}
+
+const char* rp_last_error(void) { return g_err; }
+
+// ======================================================================== core
+bool validate_device_id(int device_id) {              // reference core/tensor.c:10-16
+    if (device_id == -1) return true;
+    if (device_id < 0) return false;
+    int n = 0;
+    if (rp_hip_device_count(&n) != 0) return false;
+    return device_id < n;
+}
+
+Tensor* empty_tensor(DType dtype, int device_id, int ndim, const int* shape) {
+    if (!validate_device_id(device_id)) { fail("invalid device id %d", device_id); return nullptr; }
+    Tensor* t = alloc_header(dtype, device_id, ndim, shape);
+    if (!t) return nullptr;
+    size_t bytes = t->size * dtype_size(dtype);
+    if (device_id == -1) t->data = malloc(bytes);
+    else if (!on_device(device_id) || rp_hip_malloc(&t->data, bytes) != 0) { dev_fail("device allocation"); t->data = nullptr; }
+    if (!t->data) { free(t->shape); free(t->strides); free(t); return nullptr; }
+    return t;
+}
+
+Tensor* fill_value_tensor(double value, Tensor* t) {
+    if (!t) return nullptr;
+    if (t->device_id == -1) for (size_t i = 0; i < t->size; i++) store_from_double(t->data, i, t->dtype, t->dtype == DTYPE_FLOAT64 ? value : (double)(float)value);
+    else if (!on_device(t->device_id) || rp_hip_fill(t->data, value, t->size, t->dtype) != 0) { dev_fail("fill"); return nullptr; }
+    return t;
+}
+
+Tensor* zeros_tensor(DType dtype, int device_id, int ndim, int* shape, Meta* metadata) {      // reference core/tensor.h:60
+    Tensor* t = empty_tensor(dtype, device_id, ndim, shape);
+    if (!t) return nullptr;
+    if (device_id == -1) memset(t->data, 0, t->size * dtype_size(dtype));
+    else if (rp_hip_memset(t->data, 0, t->size * dtype_size(dtype)) != 0) { dev_fail("memset"); free_tensor(t); return nullptr; }
+    t->metadata = metadata;
+    return t;
+}
+
+Tensor* ones_tensor(DType dtype, int device_id, int ndim, int* shape, Meta* metadata) {
+    Tensor* t = empty_tensor(dtype, device_id, ndim, shape);
+    if (!t) return nullptr;
+    if (!fill_value_tensor(1.0, t)) { free_tensor(t); return nullptr; }
+    t->metadata = metadata;
+    return t;
+}
+
+// vals: host array of vals_dtype with shape_size(shape) elements (source_device_id must be -1 here).
+Tensor* values_tensor(void* vals, DType vals_dtype, DType target_dtype, int source_device_id, int device_id, int ndim, int* shape, Meta* metadata) {
+    if (!vals || source_device_id != -1) { fail("values_tensor: host source required"); return nullptr; }
+    if (target_dtype == DTYPE_PRESERVE) target_dtype = vals_dtype;
+    Tensor* host = empty_tensor(target_dtype, -1, ndim, shape);
+    if (!host) return nullptr;
+    host_convert(host->data, target_dtype, vals, vals_dtype, host->size);
+    host->metadata = metadata;
+    if (device_id == -1) return host;
+    Tensor* dev = tensor_to(host, device_id, target_dtype, false);
+    host->metadata = nullptr;
+    free_tensor(host);
+    if (dev) dev->metadata = metadata;
+    return dev;
+}
+
+Tensor* tensor_retain(Tensor* t) {                     // reference core/tensor.c:355-360
+    if (t) t->refcount++;
+    return t;
+}
+
+void free_tensor(Tensor* t) {                          // reference core/tensor.c:362-379
+    if (!t) return;
+    if (t->refcount > 1) { t->refcount--; return; }
+    if (t->metadata) {
+        if (t->metadata->grad_fn) free_grad_fn(t->metadata->grad_fn);
+        if (t->metadata->grad) free_tensor(t->metadata->grad);
+        free(t->metadata);
+    }
+    release_storage(t);
+    Tensor* base = t->base_tensor;
+    free(t->shape);
+    free(t->strides);
+    free(t);
+    if (base) free_tensor(base);
+}
+
+Tensor* tensor_copy(Tensor* t) { return t ? tensor_to(t, t->device_id, t->dtype, false) : nullptr; }
+
+// Move / convert (reference core/tensor.c:82-144): a non-contiguous source is densified first, the gradient
+// travels along, and inplace rebinds `src` itself to the new storage.
+Tensor* tensor_to(Tensor* src, int target_device_id, DType target_dtype, bool inplace) {
+    if (!src) return nullptr;
+    if (target_dtype == DTYPE_PRESERVE) target_dtype = src->dtype;
+    if (!validate_device_id(target_device_id)) { fail("invalid device id %d", target_device_id); return nullptr; }
+    if (inplace && target_device_id == src->device_id && target_dtype == src->dtype && rp_is_contiguous(src) && src->owns_data) return src;
+    Tensor* s = dense(src);
+    if (!s) return nullptr;
+    Tensor* out = empty_tensor(target_dtype, target_device_id, s->ndim, s->shape);
+    if (!out) { free_tensor(s); return nullptr; }
+    size_t n = s->size;
+    int rc = 0;
+    if (s->device_id == -1 && target_device_id == -1) {
+        host_convert(out->data, target_dtype, s->data, s->dtype, n);
+    } else if (s->device_id == -1) {                       // host -> device: convert on the host, then copy up
+        void* staged = (target_dtype == s->dtype) ? s->data : malloc(n * dtype_size(target_dtype));
+        if (staged != s->data) host_convert(staged, target_dtype, s->data, s->dtype, n);
+        rc = on_device(target_device_id) ? rp_hip_memcpy_h2d(out->data, staged, n * dtype_size(target_dtype)) : -1;
+        if (staged != s->data) free(staged);
+    } else if (target_device_id == -1) {                   // device -> host: copy down, convert on the host
+        void* staged = (target_dtype == s->dtype) ? out->data : malloc(n * dtype_size(s->dtype));
+        rc = on_device(s->device_id) ? rp_hip_memcpy_d2h(staged, s->data, n * dtype_size(s->dtype)) : -1;
+        if (rc == 0 && staged != out->data) host_convert(out->data, target_dtype, staged, s->dtype, n);
+        if (staged != out->data) free(staged);
+    } else if (s->device_id == target_device_id) {
+        rc = on_device(target_device_id) ? (target_dtype == s->dtype ? rp_hip_memcpy_d2d(out->data, s->data, n * dtype_size(s->dtype))
+                                                                     : rp_hip_convert(out->data, target_dtype, s->data, s->dtype, n)) : -1;
+    } else {
+        fail("tensor_to: copies between two GPUs are outside this build");
+        rc = -2;
+    }
+    free_tensor(s);
+    if (rc != 0) { if (rc == -1) dev_fail("tensor_to"); free_tensor(out); return nullptr; }
+    Tensor* grad = (src->metadata && src->metadata->grad) ? tensor_to(src->metadata->grad, target_device_id, target_dtype, false) : nullptr;
+    if (!inplace) {
+        if (src->metadata) {
+            Meta* m = ensure_meta(out);
+            m->requires_grad = src->metadata->requires_grad;
+            m->is_leaf = true;
+            m->grad = grad;
+        }
+        return out;
+    }
+    // inplace: src keeps its identity (and metadata) and takes over the new storage
+    release_storage(src);
+    if (src->base_tensor) { free_tensor(src->base_tensor); src->base_tensor = nullptr; }
+    free(src->shape);
+    free(src->strides);
+    src->shape = out->shape; src->strides = out->strides; src->data = out->data;
+    src->dtype = target_dtype; src->device_id = target_device_id; src->owns_data = true;
+    if (src->metadata) { if (src->metadata->grad) free_tensor(src->metadata->grad); src->metadata->grad = grad; }
+    else if (grad) free_tensor(grad);
+    free(out);
+    return src;
+}
+
+// Tensor.copy_: overwrite dst's values with src's (same element count), converting dtype / device as needed.
+int tensor_copy_into(Tensor* dst, Tensor* src) {
+    if (!dst || !src || dst->size != src->size) { fail("copy_: size mismatch"); return -1; }
+    if (!rp_is_contiguous(dst)) { fail("copy_: destination must be contiguous"); return -1; }
+    Tensor* tmp = tensor_to(src, dst->device_id, dst->dtype, false);
+    if (!tmp) return -1;
+    size_t bytes = dst->size * dtype_size(dst->dtype);
+    int rc = 0;
+    if (dst->device_id == -1) memcpy(dst->data, tmp->data, bytes);
+    else rc = on_device(dst->device_id) ? rp_hip_memcpy_d2d(dst->data, tmp->data, bytes) : -1;
+    free_tensor(tmp);
+    return rc == 0 ? 0 : dev_fail("copy_");
+}
+
+int tensor_read_scalar(Tensor* t, double* out) {
+    if (!t || !out) return -1;
+    unsigned char buf[8];
+    if (t->device_id == -1) memcpy(buf, t->data, dtype_size(t->dtype));
+    else if (!on_device(t->device_id) || rp_hip_memcpy_d2h(buf, t->data, dtype_size(t->dtype)) != 0) return dev_fail("read scalar");
+    *out = load_as_double(buf, 0, t->dtype);
+    return 0;
+}
+
+void tensor_zero_grad(Tensor* t) {                     // frees the gradient rather than zero-filling it (reference core/tensor.c:349-353)
+    if (t && t->metadata && t->metadata->grad) { free_tensor(t->metadata->grad); t->metadata->grad = nullptr; }
+}
+
+// Reverse-mode driver (reference core/tensor.c:219-347): seed with ones of the root's own shape, run every
+// GradFn once all of its consumers have contributed, then free the graph (it is single-use).
+int tensor_backward(Tensor* root) {
+    if (!root || !needs_grad(root)) { fail("backward: tensor does not require grad"); return -1; }
+    if (!root->metadata->grad_fn) return 0;
+    if (!root->metadata->grad) {
+        root->metadata->grad = ones_tensor(root->dtype, root->device_id, root->ndim, root->shape, nullptr);
+        if (!root->metadata->grad) return -1;
+    }
+    // post-order DFS over grad_fn inputs gives a topological order of the non-leaf tensors
+    std::vector<Tensor*> order;
+    std::unordered_set<Tensor*> seen;
+    std::vector<std::pair<Tensor*, int>> stack{{root, 0}};
+    seen.insert(root);
+    while (!stack.empty()) {
+        auto& [t, next] = stack.back();
+        GradFn* gf = t->metadata ? t->metadata->grad_fn : nullptr;
+        if (gf && next < gf->num_inputs) {
+            Tensor* in = gf->inputs[next++];
+            if (in && in->metadata && in->metadata->grad_fn && !seen.count(in)) { seen.insert(in); stack.push_back({in, 0}); }
+        } else {
+            order.push_back(t);
+            stack.pop_back();
+        }
+    }
+    for (auto it = order.rbegin(); it != order.rend(); ++it) {
+        Tensor* t = *it;
+        GradFn* gf = t->metadata->grad_fn;
+        if (gf && t->metadata->grad) gf->backward(gf, t->metadata->grad);
+    }
+    for (Tensor* t : order) {
+        GradFn* gf = t->metadata->grad_fn;
+        t->metadata->grad_fn = nullptr;
+        free_grad_fn(gf);                                   // may drop the last reference to intermediates; `order` is not touched again
+    }
+    return 0;
+}
+
+// ================================================================== functional
+int rp_matmul(void* C, const void* A, const void* B, int m, int k, int n, DType dtype, int device_id) {    // reference functional/functional.c:978-1006
+    if (!C || !A || !B || m <= 0 || k <= 0 || n <= 0) return -1;
+    if (device_id == -1) { fail("matmul on host tensors is not provided by this build; move the operands to a GPU"); return -1; }
+    if (!on_device(device_id)) return dev_fail("set device");
+    return matmul_kernel_device(C, A, B, m, k, n, dtype) == 0 ? 0 : dev_fail("matmul");
+}
+
+int rp_add(void* out, const void* x1, const void* x2, size_t size, DType dtype, int device_id) {           // reference functional/functional.c:58-74
+    if (!out || !x1 || !x2 || size == 0) return -1;
+    if (device_id == -1) { fail("add on host tensors is not provided by this build"); return -1; }
+    if (!on_device(device_id)) return dev_fail("set device");
+    return add_kernel_device(out, x1, x2, size, dtype) == 0 ? 0 : dev_fail("add");
+}
+
+// scalar: float* for every dtype but float64 (double*), as in the reference (functional/functional.c:241-258).
+// The host branch exists because parameter initialisation scales a host randn tensor (recpulse/module.py:97-99).
+int rp_mul_scalar(void* out, const void* x, const void* scalar, size_t size, DType dtype, int device_id) {
+    if (!out || !x || !scalar || size == 0) return -1;
+    if (device_id == -1) {
+        if (dtype == DTYPE_FLOAT64) { double s = *(const double*)scalar; for (size_t i = 0; i < size; i++) ((double*)out)[i] = ((const double*)x)[i] * s; return 0; }
+        float s = *(const float*)scalar;
+        for (size_t i = 0; i < size; i++) {
+            float v = (float)load_as_double(x, i, dtype) * s;
+            store_from_double(out, i, dtype, v);
+        }
+        return 0;
+    }
+    if (!on_device(device_id)) return dev_fail("set device");
+    return mul_scalar_kernel_device(out, x, scalar, size, dtype) == 0 ? 0 : dev_fail("mul_scalar");
+}
+
+bool rp_is_contiguous(Tensor* x) {                     // reference functional/functional.c:1117-1128
+    if (!x) return false;
+    int expect = 1;
+    for (int d = x->ndim - 1; d >= 0; d--) {
+        if (x->shape[d] != 1 && x->strides[d] != expect) return false;
+        expect *= x->shape[d];
+    }
+    return true;
+}
+
+Tensor* rp_contiguous(Tensor* x) {                     // reference functional/functional.c:1130-1220
+    if (!x) return nullptr;
+    Tensor* out = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
+    if (!out) return nullptr;
+    if (x->device_id >= 0) {
+        if (!on_device(x->device_id) || contiguous_copy_kernel_device(out->data, x->data, x->ndim, x->shape, x->strides, x->size, x->dtype) != 0) {
+            dev_fail("contiguous"); free_tensor(out); return nullptr;
+        }
+        return out;
+    }
+    size_t es = dtype_size(x->dtype);
+    for (size_t i = 0; i < x->size; i++) {
+        size_t rem = i; long long off = 0;
+        for (int d = x->ndim - 1; d >= 0; d--) { off += (long long)(rem % x->shape[d]) * x->strides[d]; rem /= x->shape[d]; }
+        memcpy((char*)out->data + i * es, (const char*)x->data + off * (long long)es, es);
+    }
+    return out;
+}
+
+Tensor* rp_transpose(Tensor* x, int dim0, int dim1) {  // reference functional/functional.c:1340-1435
+    if (!x) return nullptr;
+    if (dim0 < 0) dim0 += x->ndim;
+    if (dim1 < 0) dim1 += x->ndim;
+    if (dim0 < 0 || dim1 < 0 || dim0 >= x->ndim || dim1 >= x->ndim) { fail("transpose: dimension out of range"); return nullptr; }
+    std::vector<int> shape(x->shape, x->shape + x->ndim), strides(x->strides, x->strides + x->ndim);
+    std::swap(shape[dim0], shape[dim1]);
+    std::swap(strides[dim0], strides[dim1]);
+    return make_view(x, x->ndim, shape.data(), strides.data(), 0);
+}
+
+Tensor* rp_permute(Tensor* x, int* dims, int ndim) {   // reference functional/functional.c:1812-1875
+    if (!x || !dims || ndim != x->ndim) { fail("permute: need one entry per dimension"); return nullptr; }
+    std::vector<int> shape(ndim), strides(ndim), used(ndim, 0);
+    for (int i = 0; i < ndim; i++) {
+        int d = dims[i] < 0 ? dims[i] + ndim : dims[i];
+        if (d < 0 || d >= ndim || used[d]) { fail("permute: not a permutation"); return nullptr; }
+        used[d] = 1;
+        shape[i] = x->shape[d];
+        strides[i] = x->strides[d];
+    }
+    return make_view(x, ndim, shape.data(), strides.data(), 0);
+}
+
+Tensor* rp_reshape(Tensor* x, int ndim, int* shape) {  // one -1 entry is inferred; a non-contiguous source is copied first
+    if (!x || ndim <= 0 || !shape) return nullptr;
+    std::vector<int> shp(shape, shape + ndim);
+    long long known = 1; int infer = -1;
+    for (int i = 0; i < ndim; i++) {
+        if (shp[i] == -1) { if (infer >= 0) { fail("reshape: only one -1"); return nullptr; } infer = i; }
+        else if (shp[i] <= 0) { fail("reshape: bad extent"); return nullptr; }
+        else known *= shp[i];
+    }
+    if (infer >= 0) { if (known == 0 || x->size % known) { fail("reshape: cannot infer extent"); return nullptr; } shp[infer] = (int)(x->size / known); known *= shp[infer]; }
+    if ((size_t)known != x->size) { fail("reshape: element count changes"); return nullptr; }
+    Tensor* src = dense(x);
+    if (!src) return nullptr;
+    std::vector<int> strides(ndim);
+    int s = 1;
+    for (int d = ndim - 1; d >= 0; d--) { strides[d] = s; s *= shp[d]; }
+    Tensor* v = make_view(src, ndim, shp.data(), strides.data(), 0);
+    free_tensor(src);
+    return v;
+}
+
+Tensor* rp_slice(Tensor* x, int* start, int* stop, int* step) {
+    if (!x) return nullptr;
+    std::vector<int> shape(x->ndim), strides(x->ndim);
+    size_t off = 0;
+    for (int d = 0; d < x->ndim; d++) {
+        int b = start ? start[d] : 0, e = stop ? stop[d] : x->shape[d], st = step ? step[d] : 1;
+        if (b < 0) b += x->shape[d];
+        if (e < 0) e += x->shape[d];
+        if (e > x->shape[d]) e = x->shape[d];
+        if (st <= 0 || b < 0 || b >= e) { fail("slice: empty or invalid range in dimension %d", d); return nullptr; }
+        shape[d] = (e - b + st - 1) / st;
+        strides[d] = x->strides[d] * st;
+        off += (size_t)b * x->strides[d];
+    }
+    return make_view(x, x->ndim, shape.data(), strides.data(), off);
+}
+
+Tensor* rp_expand(Tensor* x, int ndim, int* shape) {   // broadcast view: stride 0 along stretched dims (reference functional/functional.c:1931-2003)
+    if (!x || ndim < x->ndim) { fail("expand: rank must not shrink"); return nullptr; }
+    std::vector<int> strides(ndim);
+    int lead = ndim - x->ndim;
+    for (int d = 0; d < ndim; d++) {
+        if (d < lead) { strides[d] = 0; continue; }
+        int xs = x->shape[d - lead];
+        if (xs == shape[d]) strides[d] = x->strides[d - lead];
+        else if (xs == 1) strides[d] = 0;
+        else { fail("expand: extent %d cannot stretch to %d", xs, shape[d]); return nullptr; }
+    }
+    return make_view(x, ndim, shape, strides.data(), 0);
+}
+
+// ========================================================================= ops
+namespace {
+
+bool same_place(const Tensor* a, const Tensor* b) { return a->dtype == b->dtype && a->device_id == b->device_id; }
+
+// Describe x's last two dims as a GEMM operand and its leading dims as one batch stride.
+// Returns false when the leading dims do not collapse into a single stride.
+bool batch_layout(const Tensor* x, int* batch, long long* bs) {
+    *batch = 1; *bs = 0;
+    int lead = x->ndim - 2;
+    if (lead <= 0) return true;
+    long long expect = -1;
+    for (int d = lead - 1; d >= 0; d--) {
+        if (x->shape[d] == 1) continue;
+        if (expect >= 0 && x->strides[d] != expect) return false;
+        if (*batch == 1) *bs = x->strides[d];
+        expect = (long long)x->strides[d] * x->shape[d];
+        *batch *= x->shape[d];
+    }
+    return true;
+}
+
+int device_gemm(Tensor* c, Tensor* a, bool a_t, Tensor* b, bool b_t, Tensor* bias, int accumulate) {
+    // a, b: tensors whose last two dims are the matrices; *_t reads them transposed (a stride swap, never a copy)
+    int an = a->ndim, bn = b->ndim, cn = c->ndim;
+    int m = a_t ? a->shape[an - 1] : a->shape[an - 2], k = a_t ? a->shape[an - 2] : a->shape[an - 1];
+    int n = b_t ? b->shape[bn - 2] : b->shape[bn - 1];
+    long long a_rs = a->strides[an - 2], a_cs = a->strides[an - 1], b_rs = b->strides[bn - 2], b_cs = b->strides[bn - 1];
+    if (a_t) std::swap(a_rs, a_cs);
+    if (b_t) std::swap(b_rs, b_cs);
+    int ba, bb, bc; long long a_bs, b_bs, c_bs;
+    if (!batch_layout(a, &ba, &a_bs) || !batch_layout(b, &bb, &b_bs) || !batch_layout(c, &bc, &c_bs)) { fail("matmul: batch dimensions must share one stride"); return -1; }
+    int batch = bc;
+    if ((ba != batch && ba != 1) || (bb != batch && bb != 1)) { fail("matmul: batch sizes differ"); return -1; }
+    if (ba == 1) a_bs = 0;
+    if (bb == 1) b_bs = 0;
+    if (!on_device(c->device_id)) return dev_fail("set device");
+    int rc = rp_hip_gemm_strided_batched(c->data, a->data, b->data, bias ? bias->data : nullptr, batch, m, k, n,
+                                         a_bs, a_rs, a_cs, b_bs, b_rs, b_cs, c_bs, c->strides[cn - 2], c->strides[cn - 1], accumulate, c->dtype);
+    return rc == 0 ? 0 : dev_fail("matmul");
+}
+
+// gradient of a GEMM operand: writes into a fresh tensor, or straight into the existing gradient (beta = 1)
+void gemm_grad(Tensor* target, Tensor* a, bool a_t, Tensor* b, bool b_t) {
+    Meta* m = ensure_meta(target);
+    if (m->grad && rp_is_contiguous(m->grad)) { device_gemm(m->grad, a, a_t, b, b_t, nullptr, 1); return; }
+    Tensor* g = empty_tensor(target->dtype, target->device_id, target->ndim, target->shape);
+    if (!g) return;
+    if (device_gemm(g, a, a_t, b, b_t, nullptr, 0) != 0) { free_tensor(g); return; }
+    accumulate_grad(target, g);
+}
+
+// dA = dC · Bᵀ and dB = Aᵀ · dC (reference ops/ops.c:6759-6814), with the transposes passed as stride views
+// and accumulation done by the GEMM itself instead of rp_transpose + rp_contiguous + rp_matmul + rp_add.
+void backward_matmul_fn(GradFn* self, Tensor* grad_output) {
+    Tensor* a = self->inputs[0];
+    Tensor* b = self->inputs[1];
+    if (needs_grad(a)) {
+        if (a->ndim == b->ndim || b->ndim == 2) gemm_grad(a, grad_output, false, b, true);
+    }
+    if (needs_grad(b)) {
+        if (b->ndim == a->ndim) gemm_grad(b, a, true, grad_output, false);
+        else {
+            // shared 2-D weight under a batched activation: fold the batch into the rows, dB = A2dᵀ · dC2d
+            Tensor* a2 = dense(a); Tensor* g2 = dense(grad_output);
+            int sa[2] = {(int)(a2->size / a2->shape[a2->ndim - 1]), a2->shape[a2->ndim - 1]};
+            int sg[2] = {(int)(g2->size / g2->shape[g2->ndim - 1]), g2->shape[g2->ndim - 1]};
+            Tensor* av = rp_reshape(a2, 2, sa); Tensor* gv = rp_reshape(g2, 2, sg);
+            if (av && gv) gemm_grad(b, av, true, gv, false);
+            free_tensor(av); free_tensor(gv); free_tensor(a2); free_tensor(g2);
+        }
+    }
+}
+
+// sum a gradient down to a broadcast operand's shape (reference ops/ops.c:6970-7101), on the device
+Tensor* reduce_grad_to_shape(Tensor* grad, int target_ndim, const int* target_shape) {
+    Tensor* g = dense(grad);
+    if (!g) return nullptr;
+    size_t target_size = shape_size(target_ndim, target_shape);
+    // trailing-dims case (bias of Linear): grad viewed as [outer, inner], columns summed top to bottom
+    bool trailing = target_ndim <= g->ndim;
+    for (int d = 0; trailing && d < target_ndim; d++) trailing = target_shape[target_ndim - 1 - d] == g->shape[g->ndim - 1 - d];
+    if (trailing) {
+        Tensor* out = empty_tensor(g->dtype, g->device_id, target_ndim, target_shape);
+        size_t rows = g->size / target_size;
+        int rc = out ? (rows == 1 ? rp_hip_memcpy_d2d(out->data, g->data, g->size * dtype_size(g->dtype))
+                                  : rp_hip_reduce_rows(out->data, g->data, (int)rows, (int)target_size, 0, g->dtype)) : -1;
+        free_tensor(g);
+        if (rc != 0) { dev_fail("bias gradient"); free_tensor(out); return nullptr; }
+        return out;
+    }
+    // general case: sum one stretched dimension at a time
+    int lead = g->ndim - target_ndim;
+    Tensor* cur = g;
+    for (int d = 0; d < g->ndim; d++) {
+        int tgt = d < lead ? 1 : target_shape[d - lead];
+        if (cur->shape[d] == tgt) continue;
+        if (tgt != 1) { fail("reduce_grad_to_shape: shapes do not broadcast"); free_tensor(cur); return nullptr; }
+        std::vector<int> shp(cur->shape, cur->shape + cur->ndim);
+        size_t outer = 1, inner = 1;
+        for (int i = 0; i < d; i++) outer *= shp[i];
+        for (int i = d + 1; i < cur->ndim; i++) inner *= shp[i];
+        size_t dim = shp[d];
+        shp[d] = 1;
+        Tensor* nxt = empty_tensor(cur->dtype, cur->device_id, cur->ndim, shp.data());
+        if (!nxt || sum_dim_kernel_device(nxt->data, cur->data, outer, dim, inner, cur->dtype) != 0) { dev_fail("sum_dim"); free_tensor(nxt); free_tensor(cur); return nullptr; }
+        free_tensor(cur);
+        cur = nxt;
+    }
+    std::vector<int> tshape(target_shape, target_shape + target_ndim);
+    Tensor* out = rp_reshape(cur, target_ndim, tshape.data());
+    free_tensor(cur);
+    return out;
+}
+
+void backward_add_fn(GradFn* self, Tensor* grad_output) {            // reference ops/ops.c:77-127
+    for (int i = 0; i < 2; i++) {
+        Tensor* x = self->inputs[i];
+        if (!needs_grad(x)) continue;
+        Tensor* g = same_shape(x, grad_output) ? tensor_copy(grad_output) : reduce_grad_to_shape(grad_output, x->ndim, x->shape);
+        accumulate_grad(x, g);
+    }
+}
+
+void backward_linear_fn(GradFn* self, Tensor* grad_output) {
+    Tensor* bias = self->num_inputs > 2 ? self->inputs[2] : nullptr;
+    if (bias && needs_grad(bias)) accumulate_grad(bias, reduce_grad_to_shape(grad_output, bias->ndim, bias->shape));
+    backward_matmul_fn(self, grad_output);
+}
+
+void backward_relu_fn(GradFn* self, Tensor* grad_output) {           // reference ops/ops.c:1590-1617
+    Tensor* x = self->inputs[0];
+    if (!needs_grad(x)) return;
+    Tensor* xd = dense(x); Tensor* gd = dense(grad_output);
+    Tensor* g = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
+    if (g && on_device(x->device_id) && backwards_relu_device(gd->data, xd->data, g->data, x->size, x->dtype) == 0) accumulate_grad(x, g);
+    else free_tensor(g);
+    free_tensor(xd); free_tensor(gd);
+}
+
+struct DimSaved { int dim; };
+
+void split_dims(const Tensor* x, int dim, size_t* outer, size_t* d, size_t* inner) {
+    *outer = 1; *inner = 1;
+    for (int i = 0; i < dim; i++) *outer *= x->shape[i];
+    for (int i = dim + 1; i < x->ndim; i++) *inner *= x->shape[i];
+    *d = x->shape[dim];
+}
+
+void backward_softmax_fn(GradFn* self, Tensor* grad_output) {        // reference ops/ops.c:5665-5719; y is the op's own output
+    Tensor* x = self->inputs[0];
+    if (!needs_grad(x)) return;
+    Tensor* y = self->owner;
+    int dim = ((DimSaved*)self->saved_data)->dim;
+    size_t outer, d, inner;
+    split_dims(y, dim, &outer, &d, &inner);
+    Tensor* gd = dense(grad_output);
+    Tensor* g = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
+    if (g && on_device(x->device_id) && backwards_softmax_device(gd->data, y->data, g->data, outer, d, inner, x->dtype) == 0) accumulate_grad(x, g);
+    else free_tensor(g);
+    free_tensor(gd);
+}
+
+struct ScalarSaved { double s; };
+
+void backward_mul_scalar_fn(GradFn* self, Tensor* grad_output) {     // reference ops/ops.c:5966-6020
+    Tensor* x = self->inputs[0];
+    if (!needs_grad(x)) return;
+    double s = ((ScalarSaved*)self->saved_data)->s;
+    float sf = (float)s;
+    Tensor* gd = dense(grad_output);
+    Tensor* g = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
+    if (g && rp_mul_scalar(g->data, gd->data, x->dtype == DTYPE_FLOAT64 ? (const void*)&s : (const void*)&sf, x->size, x->dtype, x->device_id) == 0) accumulate_grad(x, g);
+    else free_tensor(g);
+    free_tensor(gd);
+}
+
+void backward_reduce_all_fn(GradFn* self, Tensor* grad_output) {     // sum_all / mean_all: every element receives g (or g / size)
+    Tensor* x = self->inputs[0];
+    if (!needs_grad(x)) return;
+    double g0 = 0, scale = ((ScalarSaved*)self->saved_data)->s;
+    if (tensor_read_scalar(grad_output, &g0) != 0) return;
+    Tensor* g = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
+    if (g && fill_value_tensor(g0 * scale, g)) accumulate_grad(x, g);
+    else free_tensor(g);
+}
+
+struct CESaved { int batch, classes; void* targets_dev; int device_id; };
+
+void free_ce_saved(void* p) {
+    CESaved* s = (CESaved*)p;
+    if (s->targets_dev && on_device(s->device_id)) rp_hip_free(s->targets_dev);
+    free(s);
+}
+
+// (softmax - onehot) / batch * upstream on the device (reference ops/ops.c:5412-5543 builds it on the host)
+void backward_cross_entropy_fn(GradFn* self, Tensor* grad_output) {
+    Tensor* x = self->inputs[0];
+    if (!needs_grad(x)) return;
+    CESaved* s = (CESaved*)self->saved_data;
+    double up = 1.0;
+    if (tensor_read_scalar(grad_output, &up) != 0) return;
+    Tensor* xd = dense(x);
+    Tensor* g = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
+    if (g && on_device(x->device_id) &&
+        rp_hip_cross_entropy_mean(nullptr, g->data, xd->data, (const int*)s->targets_dev, s->batch, s->classes, up, x->dtype) == 0) accumulate_grad(x, g);
+    else free_tensor(g);
+    free_tensor(xd);
+}
+
+struct PermSaved { int ndim; int dims[8]; };
+
+void backward_permute_fn(GradFn* self, Tensor* grad_output) {        // inverse permutation of the gradient (reference ops/ops.c:7977-8014)
+    Tensor* x = self->inputs[0];
+    if (!needs_grad(x)) return;
+    PermSaved* p = (PermSaved*)self->saved_data;
+    int inv[8];
+    for (int i = 0; i < p->ndim; i++) inv[p->dims[i]] = i;
+    Tensor* v = rp_permute(grad_output, inv, p->ndim);
+    Tensor* g = v ? rp_contiguous(v) : nullptr;
+    free_tensor(v);
+    accumulate_grad(x, g);
+}
+
+void backward_reshape_fn(GradFn* self, Tensor* grad_output) {
+    Tensor* x = self->inputs[0];
+    if (!needs_grad(x)) return;
+    Tensor* gd = rp_contiguous(grad_output);
+    Tensor* v = gd ? rp_reshape(gd, x->ndim, x->shape) : nullptr;
+    Tensor* g = v ? rp_contiguous(v) : nullptr;
+    free_tensor(v); free_tensor(gd);
+    accumulate_grad(x, g);
+}
+
+Tensor* unary_device_op(Tensor* x, int (*kernel)(void*, const void*, size_t, int)) {
+    if (!x) return nullptr;
+    if (x->device_id == -1) { fail("this op runs on the device only; move the tensor to a GPU"); return nullptr; }
+    Tensor* xd = dense(x);
+    Tensor* out = xd ? empty_tensor(x->dtype, x->device_id, x->ndim, x->shape) : nullptr;
+    if (!out || !on_device(x->device_id) || kernel(out->data, xd->data, x->size, x->dtype) != 0) { dev_fail("device op"); free_tensor(out); out = nullptr; }
+    free_tensor(xd);
+    return out;
+}
+
+}  // namespace
+
+Tensor* op_matmul(Tensor* a, Tensor* b) {              // reference ops/ops.c:6816-6884; ndim > 2 is the batched extension
+    if (!a || !b) return nullptr;
+    if (a->ndim < 2 || b->ndim < 2) { fail("op_matmul: operands need at least two dimensions"); return nullptr; }
+    if (!same_place(a, b)) { fail("op_matmul: dtype or device mismatch"); return nullptr; }
+    if (a->shape[a->ndim - 1] != b->shape[b->ndim - 2]) { fail("op_matmul: inner dimensions differ"); return nullptr; }
+    if (b->ndim > 2 && b->ndim != a->ndim) { fail("op_matmul: batched operands need equal rank"); return nullptr; }
+    for (int d = 0; b->ndim > 2 && d < a->ndim - 2; d++)
+        if (a->shape[d] != b->shape[d]) { fail("op_matmul: batch dimensions differ"); return nullptr; }
+    if (a->device_id == -1) { fail("op_matmul on host tensors is not provided by this build; move the operands to a GPU"); return nullptr; }
+    std::vector<int> shape(a->shape, a->shape + a->ndim);
+    shape[a->ndim - 1] = b->shape[b->ndim - 1];
+    Tensor* out = empty_tensor(a->dtype, a->device_id, a->ndim, shape.data());
+    if (!out) return nullptr;
+    // strided operands go to the GEMM as they are; only batch dims that do not share one stride are densified
+    int bt; long long bs;
+    Tensor* aa = batch_layout(a, &bt, &bs) ? tensor_retain(a) : rp_contiguous(a);
+    Tensor* bb = batch_layout(b, &bt, &bs) ? tensor_retain(b) : rp_contiguous(b);
+    int rc = (aa && bb) ? device_gemm(out, aa, false, bb, false, nullptr, 0) : -1;
+    free_tensor(aa); free_tensor(bb);
+    if (rc != 0) { free_tensor(out); return nullptr; }
+    if (needs_grad(a) || needs_grad(b)) attach(out, backward_matmul_fn, {a, b});
+    return out;
+}
+
+Tensor* op_linear(Tensor* x, Tensor* w, Tensor* bias) {
+    if (!x || !w) return nullptr;
+    if (x->ndim < 2 || w->ndim != 2 || !same_place(x, w) || x->shape[x->ndim - 1] != w->shape[0]) { fail("op_linear: shape, dtype or device mismatch"); return nullptr; }
+    if (bias && (bias->ndim != 1 || bias->shape[0] != w->shape[1] || !same_place(x, bias) || !rp_is_contiguous(bias))) { fail("op_linear: bias must be a dense vector of out_features"); return nullptr; }
+    if (x->device_id == -1) { fail("op_linear on host tensors is not provided by this build; move the operands to a GPU"); return nullptr; }
+    std::vector<int> shape(x->shape, x->shape + x->ndim);
+    shape[x->ndim - 1] = w->shape[1];
+    Tensor* out = empty_tensor(x->dtype, x->device_id, x->ndim, shape.data());
+    if (!out) return nullptr;
+    int bt; long long bs;
+    Tensor* xx = batch_layout(x, &bt, &bs) ? tensor_retain(x) : rp_contiguous(x);
+    int rc = xx ? device_gemm(out, xx, false, w, false, bias, 0) : -1;
+    free_tensor(xx);
+    if (rc != 0) { free_tensor(out); return nullptr; }
+    if (needs_grad(x) || needs_grad(w) || needs_grad(bias)) {
+        if (bias) attach(out, backward_linear_fn, {x, w, bias});
+        else attach(out, backward_linear_fn, {x, w});
+    }
+    return out;
+}
+
+Tensor* op_add(Tensor* x1, Tensor* x2) {               // reference ops/ops.c:129-210
+    if (!x1 || !x2) return nullptr;
+    if (!same_place(x1, x2)) { fail("op_add: dtype or device mismatch"); return nullptr; }
+    if (x1->device_id == -1) { fail("op_add on host tensors is not provided by this build"); return nullptr; }
+    int nd = x1->ndim > x2->ndim ? x1->ndim : x2->ndim;
+    if (nd > 8) { fail("op_add: more than 8 dimensions"); return nullptr; }
+    std::vector<int> shape(nd);
+    for (int i = 0; i < nd; i++) {                      // broadcast_shapes (reference ops/ops.c:6941-6968)
+        int d1 = x1->ndim - nd + i, d2 = x2->ndim - nd + i;
+        int s1 = d1 >= 0 ? x1->shape[d1] : 1, s2 = d2 >= 0 ? x2->shape[d2] : 1;
+        if (s1 == s2) shape[i] = s1;
+        else if (s1 == 1) shape[i] = s2;
+        else if (s2 == 1) shape[i] = s1;
+        else { fail("op_add: shapes do not broadcast"); return nullptr; }
+    }
+    Tensor* out = empty_tensor(x1->dtype, x1->device_id, nd, shape.data());
+    if (!out) return nullptr;
+    int rc;
+    if (!on_device(x1->device_id)) rc = -1;
+    else if (same_shape(x1, x2) && rp_is_contiguous(x1) && rp_is_contiguous(x2)) rc = add_kernel_device(out->data, x1->data, x2->data, x1->size, x1->dtype);
+    else {
+        Tensor* e1 = rp_expand(x1, nd, shape.data());
+        Tensor* e2 = rp_expand(x2, nd, shape.data());
+        rc = (e1 && e2) ? add_strided_kernel_device(out->data, e1->data, e2->data, nd, shape.data(), e1->strides, e2->strides, out->size, x1->dtype) : -1;
+        free_tensor(e1); free_tensor(e2);
+    }
+    if (rc != 0) { dev_fail("op_add"); free_tensor(out); return nullptr; }
+    if (needs_grad(x1) || needs_grad(x2)) attach(out, backward_add_fn, {x1, x2});
+    return out;
+}
+
+Tensor* op_relu(Tensor* x) {                           // reference ops/ops.c:2382-2431
+    Tensor* out = unary_device_op(x, relu_kernel_device);
+    if (out && needs_grad(x)) attach(out, backward_relu_fn, {x});
+    return out;
+}
+
+static Tensor* softmax_any(Tensor* x, int dim, bool take_log) {
+    if (!x) return nullptr;
+    if (dim < 0) dim += x->ndim;
+    if (dim < 0 || dim >= x->ndim) { fail("softmax: dimension out of range"); return nullptr; }
+    if (x->device_id == -1) { fail("softmax on host tensors is not provided by this build"); return nullptr; }
+    Tensor* xd = dense(x);
+    Tensor* out = xd ? empty_tensor(x->dtype, x->device_id, x->ndim, x->shape) : nullptr;
+    size_t outer, d, inner;
+    split_dims(x, dim, &outer, &d, &inner);
+    int rc = (out && on_device(x->device_id)) ? (take_log ? log_softmax_kernel_device(out->data, xd->data, outer, d, inner, x->dtype)
+                                                          : softmax_kernel_device(out->data, xd->data, outer, d, inner, x->dtype)) : -1;
+    free_tensor(xd);
+    if (rc != 0) { dev_fail("softmax"); free_tensor(out); return nullptr; }
+    if (!take_log && needs_grad(x)) {
+        GradFn* gf = attach(out, backward_softmax_fn, {x});
+        DimSaved* s = (DimSaved*)malloc(sizeof(DimSaved));
+        s->dim = dim;
+        gf->saved_data = s;
+    }
+    return out;
+}
+
+Tensor* op_softmax(Tensor* x, int dim) { return softmax_any(x, dim, false); }            // reference ops/ops.c:5721-5788
+Tensor* op_log_softmax(Tensor* x, int dim) { return softmax_any(x, dim, true); }
+
+Tensor* op_mul_scalar(Tensor* x, double scalar) {      // reference ops/ops.c:6022-6086
+    if (!x) return nullptr;
+    Tensor* xd = dense(x);
+    Tensor* out = xd ? empty_tensor(x->dtype, x->device_id, x->ndim, x->shape) : nullptr;
+    float sf = (float)scalar;                           // scalars are narrowed to float for every dtype but float64 (reference python/tensor_python.c:475-485)
+    int rc = out ? rp_mul_scalar(out->data, xd->data, x->dtype == DTYPE_FLOAT64 ? (const void*)&scalar : (const void*)&sf, x->size, x->dtype, x->device_id) : -1;
+    free_tensor(xd);
+    if (rc != 0) { free_tensor(out); return nullptr; }
+    if (needs_grad(x)) {
+        GradFn* gf = attach(out, backward_mul_scalar_fn, {x});
+        ScalarSaved* s = (ScalarSaved*)malloc(sizeof(ScalarSaved));
+        s->s = scalar;
+        gf->saved_data = s;
+    }
+    return out;
+}
+
+static Tensor* reduce_all(Tensor* x, bool mean) {      // result has shape [1] (reference ops/ops.c:3221-3222)
+    if (!x) return nullptr;
+    if (x->device_id == -1) { fail("reductions on host tensors are not provided by this build"); return nullptr; }
+    Tensor* xd = dense(x);
+    int one = 1;
+    Tensor* out = xd ? empty_tensor(x->dtype, x->device_id, 1, &one) : nullptr;
+    int rc = (out && on_device(x->device_id)) ? (mean ? mean_all_kernel_device(out->data, xd->data, x->size, x->dtype)
+                                                      : sum_all_kernel_device(out->data, xd->data, x->size, x->dtype)) : -1;
+    free_tensor(xd);
+    if (rc != 0) { dev_fail("reduction"); free_tensor(out); return nullptr; }
+    if (needs_grad(x)) {
+        GradFn* gf = attach(out, backward_reduce_all_fn, {x});
+        ScalarSaved* s = (ScalarSaved*)malloc(sizeof(ScalarSaved));
+        s->s = mean ? 1.0 / (double)x->size : 1.0;
+        gf->saved_data = s;
+    }
+    return out;
+}
+
+Tensor* op_sum_all(Tensor* x) { return reduce_all(x, false); }
+Tensor* op_mean_all(Tensor* x) { return reduce_all(x, true); }
+
+// reduction: 0 none, 1 mean, 2 sum as in the reference; this build provides mean on raw logits
+// (reference ops/ops.c:5545-5643 with from_logits detection; out-of-range targets fail, :5547-5549).
+Tensor* op_cross_entropy_loss(Tensor* input, const int* targets, int batch_size, int num_classes, int reduction, int from_logits) {
+    if (!input || !targets) return nullptr;
+    for (int b = 0; b < batch_size; b++) if (targets[b] < 0 || targets[b] >= num_classes) { fail("op_cross_entropy_loss: target out of range"); return nullptr; }
+    if (input->ndim != 2 || input->shape[0] != batch_size || input->shape[1] != num_classes) { fail("op_cross_entropy_loss: input must be [batch, classes]"); return nullptr; }
+    if (reduction != 1 || from_logits == 0) { fail("op_cross_entropy_loss: this build provides reduction='mean' on logits"); return nullptr; }
+    if (input->dtype != DTYPE_FLOAT32 && input->dtype != DTYPE_FLOAT64) { fail("op_cross_entropy_loss: float32 / float64 only"); return nullptr; }
+    if (input->device_id == -1) { fail("op_cross_entropy_loss on host tensors is not provided by this build"); return nullptr; }
+    if (!on_device(input->device_id)) { dev_fail("set device"); return nullptr; }
+    void* tdev = nullptr;
+    if (rp_hip_malloc(&tdev, sizeof(int) * batch_size) != 0 || rp_hip_memcpy_h2d(tdev, targets, sizeof(int) * batch_size) != 0) { dev_fail("targets upload"); if (tdev) rp_hip_free(tdev); return nullptr; }
+    Tensor* xd = dense(input);
+    int one = 1;
+    Tensor* out = xd ? empty_tensor(input->dtype, input->device_id, 1, &one) : nullptr;
+    int rc = out ? rp_hip_cross_entropy_mean(out->data, nullptr, xd->data, (const int*)tdev, batch_size, num_classes, 1.0, input->dtype) : -1;
+    free_tensor(xd);
+    if (rc != 0) { dev_fail("cross entropy"); rp_hip_free(tdev); free_tensor(out); return nullptr; }
+    if (needs_grad(input)) {
+        GradFn* gf = attach(out, backward_cross_entropy_fn, {input});
+        CESaved* s = (CESaved*)calloc(1, sizeof(CESaved));
+        s->batch = batch_size; s->classes = num_classes; s->targets_dev = tdev; s->device_id = input->device_id;
+        gf->saved_data = s;
+        gf->free_saved = free_ce_saved;
+    } else {
+        rp_hip_free(tdev);
+    }
+    return out;
+}
+
+Tensor* op_transpose(Tensor* x, int dim0, int dim1) {  // reference ops/ops.c:8397-8451
+    if (!x) return nullptr;
+    if (dim0 < 0) dim0 += x->ndim;
+    if (dim1 < 0) dim1 += x->ndim;
+    Tensor* out = rp_transpose(x, dim0, dim1);
+    if (out && needs_grad(x)) {
+        GradFn* gf = attach(out, backward_permute_fn, {x});
+        PermSaved* p = (PermSaved*)calloc(1, sizeof(PermSaved));
+        p->ndim = x->ndim;
+        for (int i = 0; i < x->ndim; i++) p->dims[i] = i;
+        std::swap(p->dims[dim0], p->dims[dim1]);
+        gf->saved_data = p;
+    }
+    return out;
+}
+
+Tensor* op_permute(Tensor* x, int* dims, int ndim) {   // reference ops/ops.c:8639-8697
+    if (!x || ndim > 8) return nullptr;
+    Tensor* out = rp_permute(x, dims, ndim);
+    if (out && needs_grad(x)) {
+        GradFn* gf = attach(out, backward_permute_fn, {x});
+        PermSaved* p = (PermSaved*)calloc(1, sizeof(PermSaved));
+        p->ndim = ndim;
+        for (int i = 0; i < ndim; i++) p->dims[i] = dims[i] < 0 ? dims[i] + ndim : dims[i];
+        gf->saved_data = p;
+    }
+    return out;
+}
+
+Tensor* op_reshape(Tensor* x, int ndim, int* shape) {
+    if (!x) return nullptr;
+    Tensor* out = rp_reshape(x, ndim, shape);
+    if (out && needs_grad(x)) attach(out, backward_reshape_fn, {x});
+    return out;
+}
+
+// ====================================================================== random
+void rp_manual_seed(unsigned long long seed) { g_rng.seed(seed); }
+
+static Tensor* random_tensor(DType dtype, int device_id, int ndim, int* shape, bool normal) {
+    Tensor* host = empty_tensor(dtype, -1, ndim, shape);
+    if (!host) return nullptr;
+    std::normal_distribution<double> nd(0.0, 1.0);
+    std::uniform_real_distribution<double> ud(0.0, 1.0);
+    for (size_t i = 0; i < host->size; i++) {
+        double v = normal ? nd(g_rng) : ud(g_rng);
+        store_from_double(host->data, i, dtype, dtype == DTYPE_FLOAT64 ? v : (double)(float)v);
+    }
+    if (device_id == -1) return host;
+    Tensor* dev = tensor_to(host, device_id, dtype, false);
+    free_tensor(host);
+    return dev;
+}
+
+Tensor* rp_randn(DType dtype, int device_id, int ndim, int* shape) { return random_tensor(dtype, device_id, ndim, shape, true); }
+Tensor* rp_rand(DType dtype, int device_id, int ndim, int* shape) { return random_tensor(dtype, device_id, ndim, shape, false); }
+
+}  // extern "C"
