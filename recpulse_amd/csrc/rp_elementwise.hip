@@ -269,12 +269,13 @@ __global__ void reduce_rows_kernel(T* out, const T* g, int rows, int cols, int a
     A s = 0;
     const T* p = g + j;
     int i = 0;
-    for (; i + 4 <= rows; i += 4) {
-        A v0 = widen(p[(size_t)(i + 0) * cols]);
-        A v1 = widen(p[(size_t)(i + 1) * cols]);
-        A v2 = widen(p[(size_t)(i + 2) * cols]);
-        A v3 = widen(p[(size_t)(i + 3) * cols]);
-        s += v0; s += v1; s += v2; s += v3;
+    constexpr int U = 16;                       // independent loads in flight; the adds stay in row order
+    for (; i + U <= rows; i += U) {
+        A v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) v[u] = widen(p[(size_t)(i + u) * cols]);
+#pragma unroll
+        for (int u = 0; u < U; u++) s += v[u];
     }
     for (; i < rows; i++) s += widen(p[(size_t)i * cols]);
     T r = narrow<T>(s);
@@ -283,39 +284,47 @@ __global__ void reduce_rows_kernel(T* out, const T* g, int rows, int cols, int a
 }
 
 // ---- cross-entropy ----------------------------------------------------------------------
-// One block.  Threads stride the batch; each computes its row's log-softmax
-// and softmax serially (class counts are small), writes the scaled gradient
-// and leaves -logp[target] in global scratch; thread 0 then adds those in
-// batch order in fp64, as the reference's host loop does (ops/ops.c:5342-5352).
+// One block.  Threads stride the batch in chunks of blockDim rows; each computes its row's
+// log-softmax and softmax serially (class counts are small), writes the scaled gradient and
+// leaves -logp[target] in LDS; thread 0 adds every chunk's losses in batch order in fp64, as
+// the reference's host loop does (ops/ops.c:5342-5352).
 template <typename T>
 __global__ void cross_entropy_kernel(T* loss, T* grad, const T* logits, const int* targets,
-                                     int batch, int classes, T upstream, double* nll_scratch) {
-    for (int b = threadIdx.x; b < batch; b += blockDim.x) {
-        const T* row = logits + (size_t)b * classes;
-        T mx = lowest<T>();
-        for (int c = 0; c < classes; c++) mx = row[c] > mx ? row[c] : mx;
-        T sum = 0;
-        for (int c = 0; c < classes; c++) sum += rp_exp(row[c] - mx);
-        T lse = rp_log(sum);
-        int t = targets[b];
-        bool valid = (t >= 0 && t < classes);      // callers validate; a bad index poisons the loss instead of reading out of bounds
-        nll_scratch[b] = valid ? -(double)(row[t] - mx - lse) : (double)NAN;
-        if (grad) {
-            T sc = (T)1 / (T)batch;
-            for (int c = 0; c < classes; c++) {
-                T p = rp_exp(row[c] - mx) / sum;
-                if (c == t) p -= (T)1;
-                p *= sc;
-                grad[(size_t)b * classes + c] = p * upstream;
+                                     int batch, int classes, T upstream) {
+    __shared__ double nll[kThreads];
+    double total = 0.0;
+    for (int b0 = 0; b0 < batch; b0 += blockDim.x) {
+        int b = b0 + threadIdx.x;
+        if (b < batch) {
+            const T* row = logits + (size_t)b * classes;
+            T mx = lowest<T>();
+            for (int c = 0; c < classes; c++) mx = row[c] > mx ? row[c] : mx;
+            T sum = 0;
+            for (int c = 0; c < classes; c++) sum += rp_exp(row[c] - mx);
+            T lse = rp_log(sum);
+            int t = targets[b];
+            bool valid = (t >= 0 && t < classes);      // callers validate; a bad index poisons the loss instead of reading out of bounds
+            nll[threadIdx.x] = valid ? -(double)(row[t] - mx - lse) : (double)NAN;
+            if (grad) {
+                T sc = (T)1 / (T)batch;
+                for (int c = 0; c < classes; c++) {
+                    T p = rp_exp(row[c] - mx) / sum;
+                    if (c == t) p -= (T)1;
+                    p *= sc;
+                    grad[(size_t)b * classes + c] = p * upstream;
+                }
             }
         }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int lim = batch - b0 < (int)blockDim.x ? batch - b0 : (int)blockDim.x;
+            for (int i = 0; i < lim; i++) total += nll[i];
+        }
+        __syncthreads();
     }
-    __syncthreads();
     if (threadIdx.x == 0 && loss) {
-        double s = 0.0;
-        for (int b = 0; b < batch; b++) s += nll_scratch[b];
-        if (sizeof(T) == 8) loss[0] = (T)(s / (double)batch);
-        else { float f = (float)s; f /= (float)batch; loss[0] = (T)f; }
+        if (sizeof(T) == 8) loss[0] = (T)(total / (double)batch);
+        else { float f = (float)total; f /= (float)batch; loss[0] = (T)f; }
     }
 }
 
@@ -519,22 +528,13 @@ int rp_hip_cross_entropy_mean(void* loss_out, void* grad_logits, const void* log
         set_error("rp_hip_cross_entropy_mean: float32 and float64 only");
         return -1;
     }
-    // scratch: batch doubles for the per-row losses, from the caching pool
-    void* scratch = nullptr;
-    if (rp_hip_malloc(&scratch, (size_t)batch * 8) != 0) return -1;
-    double* nll = (double*)scratch;
-    bool ok = true;
-    {
-        if (dtype == RP_DTYPE_FLOAT32)
-            hipLaunchKernelGGL(cross_entropy_kernel<float>, dim3(1), dim3(kThreads), 0, current_stream(), (float*)loss_out, (float*)grad_logits,
-                               (const float*)logits, targets, batch, classes, (float)upstream, nll);
-        else
-            hipLaunchKernelGGL(cross_entropy_kernel<double>, dim3(1), dim3(kThreads), 0, current_stream(), (double*)loss_out, (double*)grad_logits,
-                               (const double*)logits, targets, batch, classes, upstream, nll);
-        ok = check_launch("cross_entropy_kernel");
-    }
-    rp_hip_free(scratch);
-    return ok ? 0 : -1;
+    if (dtype == RP_DTYPE_FLOAT32)
+        hipLaunchKernelGGL(cross_entropy_kernel<float>, dim3(1), dim3(kThreads), 0, current_stream(), (float*)loss_out, (float*)grad_logits,
+                           (const float*)logits, targets, batch, classes, (float)upstream);
+    else
+        hipLaunchKernelGGL(cross_entropy_kernel<double>, dim3(1), dim3(kThreads), 0, current_stream(), (double*)loss_out, (double*)grad_logits,
+                           (const double*)logits, targets, batch, classes, upstream);
+    return check_launch("cross_entropy_kernel") ? 0 : -1;
 }
 
 }  // extern "C"

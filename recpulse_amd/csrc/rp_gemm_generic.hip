@@ -30,16 +30,17 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[i][j] = (Acc)0;
 
-    for (int k0 = 0; k0 < g.k; k0 += TK) {
+    // slab k0 sits in registers while slab k0 - TK is being multiplied out of LDS, so the latency of
+    // the strided element loads overlaps the FMAs instead of adding to every slab
+    Acc ra[4], rb[4];
+    auto fetch = [&](int k0) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             int id = t + 256 * i;
             int kk = a_kfast ? id % TK : id / TM;
             int r = a_kfast ? id / TK : id % TM;
             int gm = m0 + r, gk = k0 + kk;
-            Acc v = (Acc)0;
-            if (gm < g.m && gk < g.k) v = widen(A[(long long)gm * g.a_rs + (long long)gk * g.a_cs]);
-            As[kk][r] = v;
+            ra[i] = (gm < g.m && gk < g.k) ? widen(A[(long long)gm * g.a_rs + (long long)gk * g.a_cs]) : (Acc)0;
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -47,11 +48,19 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g) {
             int kk = b_nfast ? id / TN : id % TK;
             int c = b_nfast ? id % TN : id / TK;
             int gn = n0 + c, gk = k0 + kk;
-            Acc v = (Acc)0;
-            if (gn < g.n && gk < g.k) v = widen(B[(long long)gk * g.b_rs + (long long)gn * g.b_cs]);
-            Bs[kk][c] = v;
+            rb[i] = (gn < g.n && gk < g.k) ? widen(B[(long long)gk * g.b_rs + (long long)gn * g.b_cs]) : (Acc)0;
+        }
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < g.k; k0 += TK) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int id = t + 256 * i;
+            As[a_kfast ? id % TK : id / TM][a_kfast ? id / TK : id % TM] = ra[i];
+            Bs[b_nfast ? id / TN : id % TK][b_nfast ? id % TN : id / TK] = rb[i];
         }
         __syncthreads();
+        if (k0 + TK < g.k) fetch(k0 + TK);
 #pragma unroll
         for (int kk = 0; kk < TK; kk++) {
             Acc a[4], b[4];

@@ -70,8 +70,10 @@ __device__ __forceinline__ void mw_store_slab(const T (&regs)[ROWS * mfmaw_cfg<T
     }
 }
 
-template <typename T, int BM, int BN, bool A_MC, bool B_MC, bool EDGE>
-__global__ void __launch_bounds__(256) gemm_mfmaw_kernel(GemmArgs g, int tiles_m, int tiles_n) {
+// With SPLITK the grid's z axis splits k (k_per_split is a multiple of BK): every block writes its fp32 partial
+// tile [split][m][n] to a workspace and the shared combine kernel finishes (fp32 only).
+template <typename T, int BM, int BN, bool A_MC, bool B_MC, bool EDGE, bool SPLITK>
+__global__ void __launch_bounds__(256) gemm_mfmaw_kernel(GemmArgs g, int tiles_m, int tiles_n, float* partials, int k_per_split) {
     using cfg = mfmaw_cfg<T>;
     constexpr int MT = cfg::MT, BK = cfg::BK;
     constexpr int WM = BM / 2, WN = BN / 2, TMI = WM / MT, TNI = WN / MT;
@@ -86,9 +88,12 @@ __global__ void __launch_bounds__(256) gemm_mfmaw_kernel(GemmArgs g, int tiles_m
     const int m0 = tc.tm * BM, n0 = tc.tn * BN;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
-    const T* A = (const T*)g.A + (long long)z * g.a_bs;
-    const T* B = (const T*)g.B + (long long)z * g.b_bs;
     const long long a_fs = g.a_rs, a_ks = g.a_cs, b_fs = g.b_cs, b_ks = g.b_rs;
+    const int kbeg = SPLITK ? blockIdx.z * k_per_split : 0;
+    const int kend = SPLITK ? (kbeg + k_per_split < g.k ? kbeg + k_per_split : g.k) : g.k;
+    const int klen = kend - kbeg;              // loaders see a k axis that starts at kbeg and is klen long
+    const T* A = (const T*)g.A + (long long)z * g.a_bs + (long long)kbeg * a_ks;
+    const T* B = (const T*)g.B + (long long)z * g.b_bs + (long long)kbeg * b_ks;
 
     typename cfg::acc_t acc[TMI][TNI];
 #pragma unroll
@@ -99,9 +104,9 @@ __global__ void __launch_bounds__(256) gemm_mfmaw_kernel(GemmArgs g, int tiles_m
             for (int v = 0; v < cfg::NV; v++) acc[i][j][v] = (T)0;
 
     T ra[BM * BK / 256], rb[BN * BK / 256];
-    const int nslabs = (g.k + BK - 1) / BK;
-    mw_load_slab<T, BM, A_MC, EDGE>(ra, A, a_fs, a_ks, m0, 0, g.m, g.k, t);
-    mw_load_slab<T, BN, B_MC, EDGE>(rb, B, b_fs, b_ks, n0, 0, g.n, g.k, t);
+    const int nslabs = (klen + BK - 1) / BK;
+    mw_load_slab<T, BM, A_MC, EDGE>(ra, A, a_fs, a_ks, m0, 0, g.m, klen, t);
+    mw_load_slab<T, BN, B_MC, EDGE>(rb, B, b_fs, b_ks, n0, 0, g.n, klen, t);
     mw_store_slab<T, BM, A_MC>(ra, smem, t);
     mw_store_slab<T, BN, B_MC>(rb, smem + A_ELEMS, t);
     __syncthreads();
@@ -111,8 +116,8 @@ __global__ void __launch_bounds__(256) gemm_mfmaw_kernel(GemmArgs g, int tiles_m
         const int cur = s & 1;
         const bool more = (s + 1 < nslabs);
         if (more) {
-            mw_load_slab<T, BM, A_MC, EDGE>(ra, A, a_fs, a_ks, m0, (s + 1) * BK, g.m, g.k, t);
-            mw_load_slab<T, BN, B_MC, EDGE>(rb, B, b_fs, b_ks, n0, (s + 1) * BK, g.n, g.k, t);
+            mw_load_slab<T, BM, A_MC, EDGE>(ra, A, a_fs, a_ks, m0, (s + 1) * BK, g.m, klen, t);
+            mw_load_slab<T, BN, B_MC, EDGE>(rb, B, b_fs, b_ks, n0, (s + 1) * BK, g.n, klen, t);
         }
         const T* a_lds = smem + cur * STAGE;
         const T* b_lds = a_lds + A_ELEMS;
@@ -150,9 +155,13 @@ __global__ void __launch_bounds__(256) gemm_mfmaw_kernel(GemmArgs g, int tiles_m
             for (int v = 0; v < cfg::NV; v++) {
                 int gm = m0 + wm0 + i * MT + cfg::acc_row(v, lane);
                 if (n_ok && (!EDGE || gm < g.m)) {
-                    T* p = C + (long long)gm * g.c_rs + (long long)gn * g.c_cs;
-                    T old = accum ? *p : (T)0;
-                    *p = finish<T>(acc[i][j][v], has_bias, bv, accum, old);
+                    if constexpr (SPLITK) {
+                        partials[((long long)blockIdx.z * g.m + gm) * g.n + gn] = (float)acc[i][j][v];
+                    } else {
+                        T* p = C + (long long)gm * g.c_rs + (long long)gn * g.c_cs;
+                        T old = accum ? *p : (T)0;
+                        *p = finish<T>(acc[i][j][v], has_bias, bv, accum, old);
+                    }
                 }
             }
         }
@@ -160,28 +169,55 @@ __global__ void __launch_bounds__(256) gemm_mfmaw_kernel(GemmArgs g, int tiles_m
 }
 
 template <typename T, int BM, int BN, bool A_MC, bool B_MC>
-static int launch_mfmaw_edge(const GemmArgs& g, bool edge) {
+static int launch_mfmaw_edge(const GemmArgs& g, bool edge, float* partials, int nsplit, int k_per_split) {
     int tiles_m = (g.m + BM - 1) / BM, tiles_n = (g.n + BN - 1) / BN;
+    if (nsplit > 1) {
+        if constexpr (sizeof(T) == 4) {           // split-k partials are fp32; always the predicated variant
+            dim3 grid(scheduled_grid(tiles_m, tiles_n), g.batch, nsplit);
+            hipLaunchKernelGGL((gemm_mfmaw_kernel<T, BM, BN, A_MC, B_MC, true, true>), grid, dim3(256), 0, current_stream(), g, tiles_m, tiles_n, partials, k_per_split);
+            return check_launch("gemm_mfmaw_kernel") ? 0 : -1;
+        }
+        set_error("mfmaw GEMM: split-k is fp32 only");
+        return -1;
+    }
     dim3 grid(scheduled_grid(tiles_m, tiles_n), g.batch);
-    if (edge) hipLaunchKernelGGL((gemm_mfmaw_kernel<T, BM, BN, A_MC, B_MC, true>), grid, dim3(256), 0, current_stream(), g, tiles_m, tiles_n);
-    else      hipLaunchKernelGGL((gemm_mfmaw_kernel<T, BM, BN, A_MC, B_MC, false>), grid, dim3(256), 0, current_stream(), g, tiles_m, tiles_n);
+    if (edge) hipLaunchKernelGGL((gemm_mfmaw_kernel<T, BM, BN, A_MC, B_MC, true, false>), grid, dim3(256), 0, current_stream(), g, tiles_m, tiles_n, nullptr, 0);
+    else      hipLaunchKernelGGL((gemm_mfmaw_kernel<T, BM, BN, A_MC, B_MC, false, false>), grid, dim3(256), 0, current_stream(), g, tiles_m, tiles_n, nullptr, 0);
     return check_launch("gemm_mfmaw_kernel") ? 0 : -1;
 }
 
 template <typename T, int BM, int BN>
-static int launch_mfmaw_layout(const GemmArgs& g, const Plan& p) {
-    if (!p.a_mc && p.b_mc) return launch_mfmaw_edge<T, BM, BN, false, true>(g, p.edge);
-    if (!p.a_mc && !p.b_mc) return launch_mfmaw_edge<T, BM, BN, false, false>(g, p.edge);
-    if (p.a_mc && p.b_mc) return launch_mfmaw_edge<T, BM, BN, true, true>(g, p.edge);
-    return launch_mfmaw_edge<T, BM, BN, true, false>(g, p.edge);
+static int launch_mfmaw_layout(const GemmArgs& g, const Plan& p, float* partials, int nsplit, int k_per_split) {
+    if (!p.a_mc && p.b_mc) return launch_mfmaw_edge<T, BM, BN, false, true>(g, p.edge, partials, nsplit, k_per_split);
+    if (!p.a_mc && !p.b_mc) return launch_mfmaw_edge<T, BM, BN, false, false>(g, p.edge, partials, nsplit, k_per_split);
+    if (p.a_mc && p.b_mc) return launch_mfmaw_edge<T, BM, BN, true, true>(g, p.edge, partials, nsplit, k_per_split);
+    return launch_mfmaw_edge<T, BM, BN, true, false>(g, p.edge, partials, nsplit, k_per_split);
 }
 
 template <typename T>
 static int launch_mfmaw_t(const GemmArgs& g, const Plan& p) {
-    if (p.bm == 128) return launch_mfmaw_layout<T, 128, 128>(g, p);
-    return launch_mfmaw_layout<T, 64, 64>(g, p);
+    // Small outputs with a deep k leave most CUs idle: split k so that about 256 blocks run (each split at
+    // least four slabs deep), and add the partials in split order afterwards.  fp32 only, one matrix at a time.
+    int nsplit = 1, k_per_split = 0;
+    constexpr int BK = mfmaw_cfg<T>::BK;
+    if (sizeof(T) == 4 && g.batch == 1 && p.bm == 64 && g.n % 4 == 0) {
+        int tiles = ((g.m + 63) / 64) * ((g.n + 63) / 64);
+        int want = (256 + tiles - 1) / tiles, deep = g.k / (4 * BK);
+        nsplit = want < deep ? want : deep;
+        if (nsplit > 1) {
+            k_per_split = ((g.k + nsplit - 1) / nsplit + BK - 1) / BK * BK;
+            nsplit = (g.k + k_per_split - 1) / k_per_split;
+        }
+        if (nsplit < 2) nsplit = 1;
+    }
+    void* ws = nullptr;
+    if (nsplit > 1 && rp_hip_malloc(&ws, (size_t)nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
+    int rc = (p.bm == 128) ? launch_mfmaw_layout<T, 128, 128>(g, p, (float*)ws, nsplit, k_per_split)
+                           : launch_mfmaw_layout<T, 64, 64>(g, p, (float*)ws, nsplit, k_per_split);
+    if (rc == 0 && nsplit > 1) rc = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, traits<T>::code);
+    if (ws) rp_hip_free(ws);          // stream-ordered reuse: the pool hands it out again only to later work on this stream
+    return rc;
 }
-
 
 int launch_mfmaw(const GemmArgs& g, const Plan& p, int dtype) {
     if (dtype == RP_DTYPE_FLOAT32) return launch_mfmaw_t<float>(g, p);
