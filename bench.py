@@ -22,6 +22,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3, "f64": 78.6}     # MI355X dense MFMA
 PEAK_HBM_GBS = 8000.0
+FWD_TRAFFIC_BYTES = 1.745e9      # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the forward GEMM, see profiles/pmc_traffic_gemm_bf16_8192.md
 
 
 def _bf16_bits(x32):
@@ -75,10 +76,15 @@ def _time_graph(capi, fn, reps, warmup, replays=5):
     return ms
 
 
-def headline(capi, steps, warmup, n=8192):
+def headline(capi, steps, warmup, n=8192, data="normal"):
     rng = np.random.default_rng(2)
     dt = capi.BF16
-    a, b, dc = (_normal_bf16(rng, (n, n)) for _ in range(3))
+    if data == "normal":
+        a, b, dc = (_normal_bf16(rng, (n, n)) for _ in range(3))
+    elif data == "ints":
+        a, b, dc = (_bf16_bits(rng.integers(-3, 4, (n, n)).astype(np.float32)) for _ in range(3))
+    else:
+        a, b, dc = (np.full((n, n), 0x3f80 if data == "ones" else 0, dtype=np.uint16) for _ in range(3))
     d_a, d_b, d_dc = (capi.DeviceBuffer.from_numpy(t) for t in (a, b, dc))
     d_c, d_da, d_db = (capi.DeviceBuffer(n * n * 2) for _ in range(3))
     rm, tr = (0, n, 1), (0, 1, n)            # row-major and transposed-view strides (batch, row, col)
@@ -124,7 +130,7 @@ def headline(capi, steps, warmup, n=8192):
     b64 = (b[:, cols].astype(np.uint32) << 16).view(np.float32).astype(np.float64)
     ref = a64 @ b64
     got = (c[np.ix_(rows, cols)].astype(np.uint32) << 16).view(np.float32).astype(np.float64)
-    err = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
+    err = float(np.linalg.norm(got - ref) / max(np.linalg.norm(ref), 1e-30))
     if not err <= 2e-2:
         raise RuntimeError(f"bf16 8192^3 forward GEMM fails parity: sampled normwise error {err}")
     return {
@@ -233,6 +239,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--data", choices=["normal", "ints", "ones", "zeros"], default="normal",
+                    help="operand values of the headline GEMMs: N(0,1) (the configuration) or low-toggle data, to show how far the "
+                         "power-managed shader clock, and with it the throughput, depends on the values multiplied")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run a plain copy kernel of known size (256 MiB in, 256 MiB out), the yardstick for FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -244,18 +255,28 @@ def main():
         sys.exit(1)
     capi.check(capi.lib().rp_hip_set_device(0), "rp_hip_set_device")
 
-    h = headline(capi, args.steps, args.warmup)
+    if args.calibrate:
+        n = 64 << 20
+        src, dst = capi.DeviceBuffer(4 * n), capi.DeviceBuffer(4 * n)
+        capi.check(capi.lib().rp_hip_fill(src.ptr, 1.0, n, capi.F32), "fill")
+        for _ in range(3):
+            capi.check(capi.lib().rp_hip_convert(dst.ptr, capi.F32, src.ptr, capi.F32, n), "copy")
+        capi.synchronize()
+        src.free(); dst.free()
+    h = headline(capi, args.steps, args.warmup, data=args.data)
     a, b = h.pop("operands")
     line = {
         "metric": "GEMM TFLOP/s (bf16 8192^3, forward + both backward GEMMs per step)",
         "value": h["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": h["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": "bf16", "data": "synthetic" if args.data == "normal" else f"synthetic ({args.data}: diagnostic, not the configuration)",
         "config": {"workload": "config 3 at N=8192: bf16 square GEMM, fp32 accumulate, bf16 output; "
                                "C=A·B, dA=dC·Bᵀ, dB=Aᵀ·dC with transposes as stride views; A,B,dC ~ N(0,1) seed 2",
                    "m": 8192, "n": 8192, "k": 8192, "gemms_per_step": 3},
         "roofline": {"bound": "mfma", "achieved": h["fwd_tflops"], "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
-                     "frac": h["fwd_tflops"] / PEAK_TFLOPS["bf16"], "traffic": None,
+                     "frac": h["fwd_tflops"] / PEAK_TFLOPS["bf16"], "traffic": FWD_TRAFFIC_BYTES,
+                     "traffic_note": "bytes per launch below the L2s (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, scaled by a copy kernel), "
+                                     "from profiles/pmc_traffic_gemm_bf16_8192.md; algorithmic bytes are 4.027e8",
                      "kernel": h["kernel"] + " (forward, A row-major x B row-major)",
                      "avg_launch_ms": h["kernel_ms"]["fwd_nn"]},
         "kernel_ms": h["kernel_ms"], "sampled_rel_err": h["sampled_rel_err"],
