@@ -48,26 +48,30 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     bool batch_ok = (batch == 1) || ((a_bs % vec == 0) && (b_bs % vec == 0));
     (void)c_rs; (void)c_cs;
 
-    // skinny: few rows, row-major B, enough columns and depth to be worth streaming
-    const int valu_rows = (dtype == RP_DTYPE_FLOAT32) ? SK_MAX_M : 4;        // 16-bit inputs with more rows go to the MFMA skinny kernel
+    // the MFMA kernels address a tile with 32-bit byte offsets from a 64-bit tile pointer
+    const long long max_stride = 1ll << 22;
+    const bool strides_ok = a_rs < max_stride && a_cs < max_stride && b_rs < max_stride && b_cs < max_stride;
+    const bool mfma_ok = (a_kc || a_mc) && (b_kc || b_mc) && batch_ok && strides_ok;
+    const bool is16 = dtype == RP_DTYPE_FLOAT16 || dtype == RP_DTYPE_BFLOAT16;
+
+    // 16-bit, few rows, deep k: split k over many blocks so that B streams at HBM speed (output columns in whole 8s)
+    if (is16 && mfma_ok && batch == 1 && m <= 32 && n % 8 == 0 && n >= 256 && k >= 1024 && (long long)k * n >= (1ll << 22)) {
+        p.fam = FAM_MFMA16_SKINNY; p.bm = 32; p.bn = 128; p.edge = true; p.a_mc = !a_kc; p.b_mc = b_mc;
+        p.name = (!p.a_mc && p.b_mc && m <= 16) ? "mfma16_stream_32x256" : "mfma16_skinny_32x128";
+        return p;
+    }
+    // VALU skinny: few rows, row-major B, enough columns and depth to be worth streaming
+    const int valu_rows = (dtype == RP_DTYPE_FLOAT32) ? SK_MAX_M : 4;
     if (batch == 1 && dtype != RP_DTYPE_FLOAT64 && m <= valu_rows && b_mc && n >= 64 * vec && (long long)k * n >= (1ll << 20) &&
         (n + 64 * vec - 1) / (64 * vec) <= SK_MAX_GROUPS) {
         p.fam = FAM_SKINNY; p.name = "skinny"; p.b_mc = true;
         return p;
     }
-    // the MFMA kernels address a tile with 32-bit byte offsets from a 64-bit tile pointer
-    const long long max_stride = 1ll << 22;
-    bool strides_ok = a_rs < max_stride && a_cs < max_stride && b_rs < max_stride && b_cs < max_stride;
-    if (!(a_kc || a_mc) || !(b_kc || b_mc) || !batch_ok || !strides_ok) return p;
+    if (!mfma_ok) return p;
     p.a_mc = !a_kc;             // when both qualify (extent-1 corner cases) keep the row-major reading
     p.b_mc = b_mc;
 
-    if (dtype == RP_DTYPE_FLOAT16 || dtype == RP_DTYPE_BFLOAT16) {
-        // few rows, deep k: split k over many blocks so that B streams at HBM speed (output columns in whole 8s)
-        if (batch == 1 && m <= 32 && n % 8 == 0 && n >= 256 && k >= 1024 && (long long)k * n >= (1ll << 22)) {
-            p.fam = FAM_MFMA16_SKINNY; p.bm = 32; p.bn = 128; p.edge = true; p.name = "mfma16_skinny_32x128";
-            return p;
-        }
+    if (is16) {
         p.fam = FAM_MFMA16;
         long long tiles256 = (long long)((m + 255) / 256) * ((n + 255) / 256) * batch;
         if (m >= 256 && n >= 256 && tiles256 >= 128) { p.bm = 256; p.bn = 256; p.name = "mfma16_256x256"; }

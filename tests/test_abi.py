@@ -44,9 +44,11 @@ def test_kernel_selection_names():
     name = capi.gemm_kernel_name
     assert name(1, 8192, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "mfma16_256x256"
     assert name(1, 8192, 8192, 8192, (1, 8192), (8192, 1), (8192, 1), capi.F16) == "mfma16_256x256"       # A^T view
-    assert name(1, 1, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "skinny"
-    assert name(1, 8, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "mfma16_skinny_32x128"
+    assert name(1, 1, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "mfma16_stream_32x256"
+    assert name(1, 8, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "mfma16_stream_32x256"
+    assert name(1, 16, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F16) == "mfma16_stream_32x256"
     assert name(1, 32, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F16) == "mfma16_skinny_32x128"
+    assert name(1, 8, 8192, 8192, (8192, 1), (1, 8192), (8192, 1), capi.BF16) == "mfma16_skinny_32x128"
     assert name(1, 8, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F32) == "skinny"
     assert name(1, 128, 784, 256, (784, 1), (256, 1), (256, 1), capi.F32) == "mfma32_64x64"          # few tiles: small tile + split-k
     assert name(1, 4096, 4096, 4096, (4096, 1), (4096, 1), (4096, 1), capi.F32) == "mfma32_128x128"

@@ -199,7 +199,8 @@ def test_skinny_rows_mfma_split_k(dt, layout):
             continue                                   # a transposed A needs whole 16-byte vectors along m
         a, b = _operands(rng, m, k, n, dt, layout)
         a_st = (a.strides[0] // 2, a.strides[1] // 2); b_st = (b.strides[0] // 2, b.strides[1] // 2)
-        assert capi.gemm_kernel_name(1, m, k, n, a_st, b_st, (n, 1), dt) == "mfma16_skinny_32x128"
+        want_kernel = "mfma16_stream_32x256" if layout == "nn" and m <= 16 else "mfma16_skinny_32x128"
+        assert capi.gemm_kernel_name(1, m, k, n, a_st, b_st, (n, 1), dt) == want_kernel
         bias = rand_storage(rng, (n,), dt); c0 = rand_storage(rng, (m, n), dt)
         got = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)
         _check(got, a, b, dt, k, bias=bias, c_init=c0, accumulate=True)
@@ -208,6 +209,26 @@ def test_skinny_rows_mfma_split_k(dt, layout):
     a = oracle.to_storage(rng.integers(-2, 3, (8, 4096)).astype(np.float64), dt)
     b = oracle.to_storage(rng.integers(-2, 3, (4096, 1024)).astype(np.float64), dt)
     assert np.array_equal(device_gemm(a, b, dt), oracle_gemm(a, b, dt))
+
+
+@pytest.mark.parametrize("m", [1, 3, 8, 11, 16])
+def test_streaming_rows_single_launch_finish(m):
+    """Row-major A times row-major B with few rows: one launch, the last block of a column group to arrive adds the
+    k splits.  Repeated launches must reproduce the first result bit for bit (fixed summation order, counters left
+    clean), with ragged k and n, a bias and an accumulating epilogue."""
+    rng = np.random.default_rng(39)
+    for dt, k, n in [(BF16, 8192, 2048), (F16, 4104, 1288), (BF16, 1024, 4096)]:
+        a, b = _operands(rng, m, k, n, dt, "nn")
+        assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == "mfma16_stream_32x256"
+        bias = rand_storage(rng, (n,), dt); c0 = rand_storage(rng, (m, n), dt)
+        first = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)
+        _check(first, a, b, dt, k, bias=bias, c_init=c0, accumulate=True)
+        for _ in range(20):
+            assert np.array_equal(first, device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True))
+    # integer data is exact in fp32 whatever the split: bit-equal to the oracle, NaN and Inf carried through
+    a = oracle.to_storage(rng.integers(-2, 3, (m, 4096)).astype(np.float64), BF16)
+    b = oracle.to_storage(rng.integers(-2, 3, (4096, 1024)).astype(np.float64), BF16)
+    assert np.array_equal(device_gemm(a, b, BF16), oracle_gemm(a, b, BF16))
 
 
 def test_large_tile_kernel_multi_slab():
