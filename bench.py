@@ -182,8 +182,50 @@ def secondary(capi, quick_reps=20):
         ms = _time_launches(capi, fn, 10, 3)
         tf = 2.0 * size ** 3 / (ms * 1e-3) / 1e12
         out[name] = {"ms": ms, "TFLOP/s": tf, "frac_mfma": tf / peak}
+    # config 4: attention-shaped batched GEMMs on stride views, bf16
+    out["attention_bf16"] = attention_times(capi, "bf16")
     # config 2: fp32 MLP 784-256-128-10, batch 256, forward + backward through the C ABI (9 GEMMs + neighbours)
     out["mlp_f32_step"] = mlp_step_time(capi)
+    return out
+
+
+def attention_times(capi, dt_name="bf16"):
+    """Config 4: Q, K, V [16*12, 512, 64]; S = Q·Kᵀ (Kᵀ a stride view), P = softmax(S/8), O = P·V, and the four
+    backward GEMMs, each timed on its own from a HIP graph.  GEMM bytes are A, B and C once."""
+    rng = np.random.default_rng(3)
+    Z, S, D = 16 * 12, 512, 64
+    dt = {"bf16": capi.BF16, "f32": capi.F32}[dt_name]
+    esz = 2 if dt == capi.BF16 else 4
+    mk = (lambda shape: _normal_bf16(rng, shape)) if dt == capi.BF16 else (lambda shape: rng.standard_normal(shape).astype(np.float32))
+    D_ = capi.DeviceBuffer
+    d_q, d_k, d_v, d_do = (D_.from_numpy(mk((Z, S, D))) for _ in range(4))
+    d_s, d_ss, d_p, d_dp, d_dss = (D_(Z * S * S * esz) for _ in range(5))
+    d_o, d_dq, d_dk, d_dv = (D_(Z * S * D * esz) for _ in range(4))
+    sd, ss = S * D, S * S
+    L = capi.lib()
+    import ctypes
+    scale = (ctypes.c_float * 1)(0.125)              # scalars travel as float for every dtype but float64
+    ops = {
+        "S=Q.Kt": (lambda: capi.gemm(d_s.ptr, d_q.ptr, d_k.ptr, None, Z, S, D, S, (sd, D, 1), (sd, 1, D), (ss, S, 1), False, dt), 2.0 * Z * S * S * D, (2 * sd + ss) * Z * esz),
+        "scale": (lambda: capi.check(L.mul_scalar_kernel_device(d_ss.ptr, d_s.ptr, scale, Z * ss, dt), "mul_scalar"), 0.0, 2 * ss * Z * esz),
+        "softmax": (lambda: capi.check(L.softmax_kernel_device(d_p.ptr, d_ss.ptr, Z * S, S, 1, dt), "softmax"), 0.0, 2 * ss * Z * esz),
+        "O=P.V": (lambda: capi.gemm(d_o.ptr, d_p.ptr, d_v.ptr, None, Z, S, S, D, (ss, S, 1), (sd, D, 1), (sd, D, 1), False, dt), 2.0 * Z * S * S * D, (2 * sd + ss) * Z * esz),
+        "dP=dO.Vt": (lambda: capi.gemm(d_dp.ptr, d_do.ptr, d_v.ptr, None, Z, S, D, S, (sd, D, 1), (sd, 1, D), (ss, S, 1), False, dt), 2.0 * Z * S * S * D, (2 * sd + ss) * Z * esz),
+        "dV=Pt.dO": (lambda: capi.gemm(d_dv.ptr, d_p.ptr, d_do.ptr, None, Z, S, S, D, (ss, 1, S), (sd, D, 1), (sd, D, 1), False, dt), 2.0 * Z * S * S * D, (2 * sd + ss) * Z * esz),
+        "softmax_bwd": (lambda: capi.check(L.backwards_softmax_device(d_dp.ptr, d_p.ptr, d_dss.ptr, Z * S, S, 1, dt), "backwards_softmax"), 0.0, 3 * ss * Z * esz),
+        "dQ=dS.K": (lambda: capi.gemm(d_dq.ptr, d_dss.ptr, d_k.ptr, None, Z, S, S, D, (ss, S, 1), (sd, D, 1), (sd, D, 1), False, dt), 2.0 * Z * S * S * D, (2 * sd + ss) * Z * esz),
+        "dK=dSt.Q": (lambda: capi.gemm(d_dk.ptr, d_dss.ptr, d_q.ptr, None, Z, S, S, D, (ss, 1, S), (sd, D, 1), (sd, D, 1), False, dt), 2.0 * Z * S * S * D, (2 * sd + ss) * Z * esz),
+    }
+    for fn, _, _ in ops.values():        # eager once, in dependency order, so every buffer holds finite values
+        fn()
+    out, total = {}, 0.0
+    for name, (fn, flops, nbytes) in ops.items():
+        ms = _time_graph(capi, fn, 10, 2)
+        total += ms
+        out[name] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1), "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 3)}
+        if flops:
+            out[name]["TFLOP/s"] = round(flops / ms / 1e9, 1)
+    out["fwd_bwd_ms"] = round(total + out["scale"]["us"] * 1e-3, 4)     # the scale runs twice (S/8 and dS/8)
     return out
 
 

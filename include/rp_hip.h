@@ -124,7 +124,7 @@ const char* rp_hip_gemm_kernel_name(int batch, int m, int k, int n,
                                     long long c_rs, long long c_cs, int dtype);
 
 /* ------------------------------------------------------------------------
- * The other device entry points BASELINE's configs touch.  Names and
+ * The other device entry points the benchmark configurations touch.  Names and
  * arguments are the reference's (functional/functional.h:363-428,
  * ops/ops.h backwards_*_device declarations).
  * ---------------------------------------------------------------------- */

@@ -1,5 +1,5 @@
-// Element-wise, row-wise and reduction entry points that BASELINE's configs run
-// around the GEMMs: add / broadcasting add, scalar multiply, relu and softmax
+// Element-wise, row-wise and reduction entry points that the benchmark
+// configurations run around the GEMMs: add / broadcasting add, scalar multiply, relu and softmax
 // with their VJPs, strided gather, reductions, fill / convert, and the
 // on-device bias gradient and cross-entropy.  16-bit dtypes compute in fp32
 // and narrow once with the reference's rounding, like the reference's host
@@ -9,6 +9,8 @@
 #include <cfloat>
 
 namespace rp {
+
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;      // one 16-byte memory access
 
 static constexpr int kThreads = 256;
 static constexpr int kMaxDims = 8;
@@ -21,32 +23,67 @@ static inline unsigned grid_for(size_t n, int threads = kThreads, size_t cap = 1
 }
 
 // ---- flat maps ----------------------------------------------------------------
-template <typename T>
-__global__ void add_kernel(T* out, const T* x1, const T* x2, size_t n) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
-        out[i] = narrow<T>(widen(x1[i]) + widen(x2[i]));
-}
+// out[i] = op(x1[i], x2[i]) in the accumulate type, narrowed once.  When every pointer is 16-byte aligned each
+// thread moves whole 16-byte vectors, four per pass with all four loads in flight; a scalar loop takes the rest.
+template <typename A> struct AddOp { __device__ __forceinline__ A operator()(A a, A b) const { return a + b; } };
+template <typename A> struct MulScalarOp { A s; __device__ __forceinline__ A operator()(A a, A) const { return a * s; } };
+template <typename A> struct ReluOp { __device__ __forceinline__ A operator()(A a, A) const { return a > (A)0 ? a : (A)0; } };
+template <typename A> struct BackReluOp { __device__ __forceinline__ A operator()(A g, A x) const { return x > (A)0 ? g : (A)0; } };   // (grad, input)
 
-template <typename T>
-__global__ void mul_scalar_kernel(T* out, const T* x, typename traits<T>::acc s, size_t n) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
-        out[i] = narrow<T>(widen(x[i]) * s);
-}
-
-template <typename T>
-__global__ void relu_kernel(T* out, const T* x, size_t n) {
+template <typename T, bool TWO, typename Op>
+__global__ void map_scalar_kernel(T* out, const T* x1, const T* x2, Op op, size_t begin, size_t n) {
     using A = typename traits<T>::acc;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
-        A v = widen(x[i]);
-        out[i] = narrow<T>(v > (A)0 ? v : (A)0);
+    for (size_t i = begin + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        out[i] = narrow<T>(op(widen(x1[i]), TWO ? widen(x2[i]) : (A)0));
+}
+
+template <typename T, bool TWO, typename Op>
+__global__ void __launch_bounds__(kThreads) map_vec_kernel(T* out, const T* x1, const T* x2, Op op, size_t nvec) {
+    using A = typename traits<T>::acc;
+    constexpr int VEC = 16 / sizeof(T), U = 4;
+    const u32x4_t* p1 = (const u32x4_t*)x1;
+    const u32x4_t* p2 = (const u32x4_t*)x2;
+    u32x4_t* po = (u32x4_t*)out;
+    for (size_t base = (size_t)blockIdx.x * (kThreads * U); base < nvec; base += (size_t)gridDim.x * (kThreads * U)) {
+        u32x4_t r1[U], r2[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            size_t i = base + u * kThreads + threadIdx.x;
+            if (i < nvec) {
+                r1[u] = __builtin_nontemporal_load(p1 + i);
+                if (TWO) r2[u] = __builtin_nontemporal_load(p2 + i);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            size_t i = base + u * kThreads + threadIdx.x;
+            if (i >= nvec) continue;
+            T a[VEC], b[VEC], o[VEC];
+            memcpy(a, &r1[u], 16);
+            if (TWO) memcpy(b, &r2[u], 16);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) o[e] = narrow<T>(op(widen(a[e]), TWO ? widen(b[e]) : (A)0));
+            u32x4_t w;
+            memcpy(&w, o, 16);
+            __builtin_nontemporal_store(w, po + i);
+        }
     }
 }
 
-template <typename T>
-__global__ void backwards_relu_kernel(const T* gc, const T* x, T* gx, size_t n) {
-    using A = typename traits<T>::acc;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
-        gx[i] = narrow<T>(widen(x[i]) > (A)0 ? widen(gc[i]) : (A)0);
+static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+template <typename T, bool TWO, typename Op>
+static void launch_map(T* out, const T* x1, const T* x2, Op op, size_t n) {
+    constexpr int VEC = 16 / sizeof(T);
+    size_t nvec = (aligned16(out) && aligned16(x1) && (!TWO || aligned16(x2))) ? n / VEC : 0;
+    if (nvec) {
+        size_t blocks = (nvec + kThreads * 4 - 1) / (kThreads * 4);
+        if (blocks > (1u << 20)) blocks = 1u << 20;
+        hipLaunchKernelGGL((map_vec_kernel<T, TWO, Op>), dim3((unsigned)blocks), dim3(kThreads), 0, current_stream(), out, x1, x2, op, nvec);
+    }
+    size_t done = nvec * VEC;
+    if (done < n)
+        hipLaunchKernelGGL((map_scalar_kernel<T, TWO, Op>), dim3(grid_for(n - done)), dim3(kThreads), 0, current_stream(), out, x1, x2, op, done, n);
 }
 
 template <typename T>
@@ -158,6 +195,156 @@ __global__ void softmax_rows_kernel(T* out, const T* x, size_t rows, size_t dim)
             for (size_t d = lane; d < dim; d += 64) orow[d] = narrow<T>(rp_exp(widen(xr[d]) - mx) / sum);
         }
     }
+}
+
+// Rows that fit a wave's registers (dim <= 64 lanes * CH chunks * 16 bytes, dim a whole number of 16-byte
+// vectors, aligned rows): each lane loads CH 16-byte pieces of the row once, everything else happens in
+// registers, and the result leaves as 16-byte stores.  One wave per row, four rows per block.
+template <typename T, bool LOG, int CH>
+__global__ void __launch_bounds__(kThreads) softmax_rows_reg_kernel(T* out, const T* x, size_t rows, int dim) {
+    using A = typename traits<T>::acc;
+    constexpr int VEC = 16 / sizeof(T);
+    const int lane = threadIdx.x & 63;
+    const size_t wave = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const size_t nwaves = ((size_t)gridDim.x * blockDim.x) >> 6;
+    for (size_t r = wave; r < rows; r += nwaves) {
+        const T* xr = x + r * (size_t)dim;
+        T* orow = out + r * (size_t)dim;
+        u32x4_t raw[CH];
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int e0 = (c * 64 + lane) * VEC;
+            if (e0 < dim) raw[c] = __builtin_nontemporal_load((const u32x4_t*)(xr + e0));
+        }
+        A v[CH][VEC];
+        A mx = lowest<A>();
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const bool in = (c * 64 + lane) * VEC < dim;
+            T t[VEC];
+            memcpy(t, &raw[c], 16);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                v[c][e] = in ? widen(t[e]) : lowest<A>();
+                mx = v[c][e] > mx ? v[c][e] : mx;
+            }
+        }
+        mx = wave_max(mx);
+        A sum = 0;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const bool in = (c * 64 + lane) * VEC < dim;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                // 16-bit outputs keep 8 or 11 significant bits: the hardware exp2 (1 ulp of fp32) is ample there
+                A ex;
+                if constexpr (sizeof(T) == 2) ex = __builtin_amdgcn_exp2f((v[c][e] - mx) * 1.44269504088896341f);
+                else ex = rp_exp(v[c][e] - mx);
+                sum += in ? ex : (A)0;
+                if (!LOG) v[c][e] = ex;
+            }
+        }
+        sum = wave_sum(sum);
+        const A lse = LOG ? rp_log(sum) : (A)0;
+        const A inv = (A)1 / sum;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int e0 = (c * 64 + lane) * VEC;
+            if (e0 >= dim) continue;
+            T o[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; e++) o[e] = narrow<T>(LOG ? v[c][e] - mx - lse : (sizeof(T) == 2 ? v[c][e] * inv : v[c][e] / sum));
+            u32x4_t w;
+            memcpy(&w, o, 16);
+            __builtin_nontemporal_store(w, (u32x4_t*)(orow + e0));
+        }
+    }
+}
+
+template <typename T, int CH>
+__global__ void __launch_bounds__(kThreads) backwards_softmax_rows_reg_kernel(const T* gc, const T* y, T* gx, size_t rows, int dim) {
+    using A = typename traits<T>::acc;
+    constexpr int VEC = 16 / sizeof(T);
+    const int lane = threadIdx.x & 63;
+    const size_t wave = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const size_t nwaves = ((size_t)gridDim.x * blockDim.x) >> 6;
+    for (size_t r = wave; r < rows; r += nwaves) {
+        const size_t row0 = r * (size_t)dim;
+        u32x4_t rg[CH], ry[CH];
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int e0 = (c * 64 + lane) * VEC;
+            if (e0 < dim) {
+                rg[c] = __builtin_nontemporal_load((const u32x4_t*)(gc + row0 + e0));
+                ry[c] = __builtin_nontemporal_load((const u32x4_t*)(y + row0 + e0));
+            }
+        }
+        A g[CH][VEC], s[CH][VEC];
+        A dot = 0;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const bool in = (c * 64 + lane) * VEC < dim;
+            T tg[VEC], ty[VEC];
+            memcpy(tg, &rg[c], 16);
+            memcpy(ty, &ry[c], 16);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                g[c][e] = in ? widen(tg[e]) : (A)0;
+                s[c][e] = in ? widen(ty[e]) : (A)0;
+                dot += g[c][e] * s[c][e];
+            }
+        }
+        dot = wave_sum(dot);
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int e0 = (c * 64 + lane) * VEC;
+            if (e0 >= dim) continue;
+            T o[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; e++) o[e] = narrow<T>(s[c][e] * (g[c][e] - dot));
+            u32x4_t w;
+            memcpy(&w, o, 16);
+            __builtin_nontemporal_store(w, (u32x4_t*)(gx + row0 + e0));
+        }
+    }
+}
+
+// chunks per lane the register kernels need for this row length, or 0 when the row does not qualify
+template <typename T>
+static int reg_row_chunks(size_t dim, const void* p0, const void* p1, const void* p2) {
+    constexpr size_t VEC = 16 / sizeof(T);
+    if (dim % VEC || dim > 64 * VEC * 8 || !aligned16(p0) || !aligned16(p1) || (p2 && !aligned16(p2))) return 0;
+    size_t ch = (dim + 64 * VEC - 1) / (64 * VEC);
+    return ch <= 1 ? 1 : ch <= 2 ? 2 : ch <= 4 ? 4 : 8;
+}
+
+template <typename T, int CH>
+static void launch_softmax_reg_ch(T* out, const T* x, size_t rows, size_t dim, unsigned blocks, bool take_log) {
+    if (take_log) hipLaunchKernelGGL((softmax_rows_reg_kernel<T, true, CH>), dim3(blocks), dim3(kThreads), 0, current_stream(), out, x, rows, (int)dim);
+    else          hipLaunchKernelGGL((softmax_rows_reg_kernel<T, false, CH>), dim3(blocks), dim3(kThreads), 0, current_stream(), out, x, rows, (int)dim);
+}
+// launch the register kernel when the rows qualify; false means the caller takes the general one
+template <typename T>
+static bool launch_softmax_reg(T* out, const T* x, size_t rows, size_t dim, unsigned blocks, bool take_log) {
+    switch (reg_row_chunks<T>(dim, out, x, nullptr)) {
+        case 1: launch_softmax_reg_ch<T, 1>(out, x, rows, dim, blocks, take_log); return true;
+        case 2: launch_softmax_reg_ch<T, 2>(out, x, rows, dim, blocks, take_log); return true;
+        case 4: launch_softmax_reg_ch<T, 4>(out, x, rows, dim, blocks, take_log); return true;
+        case 8: launch_softmax_reg_ch<T, 8>(out, x, rows, dim, blocks, take_log); return true;
+        default: return false;
+    }
+}
+template <typename T>
+static bool launch_bsoftmax_reg(const T* gc, const T* y, T* gx, size_t rows, size_t dim, unsigned blocks) {
+#define RP_BSOFTMAX_REG(CH) hipLaunchKernelGGL((backwards_softmax_rows_reg_kernel<T, CH>), dim3(blocks), dim3(kThreads), 0, current_stream(), gc, y, gx, rows, (int)dim)
+    switch (reg_row_chunks<T>(dim, gc, y, gx)) {
+        case 1: RP_BSOFTMAX_REG(1); return true;
+        case 2: RP_BSOFTMAX_REG(2); return true;
+        case 4: RP_BSOFTMAX_REG(4); return true;
+        case 8: RP_BSOFTMAX_REG(8); return true;
+        default: return false;
+    }
+#undef RP_BSOFTMAX_REG
 }
 
 template <typename T, bool LOG>
@@ -380,8 +567,7 @@ extern "C" {
 
 int add_kernel_device(void* out, const void* x1, const void* x2, size_t size, int dtype) {
     RP_REQUIRE(out && x1 && x2 && size, "add_kernel_device");
-    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(add_kernel<T>, dim3(grid_for(size)), dim3(kThreads), 0, current_stream(),
-                                               (T*)out, (const T*)x1, (const T*)x2, size));
+    RP_DISPATCH_DTYPE(dtype, launch_map<T, true>((T*)out, (const T*)x1, (const T*)x2, AddOp<typename traits<T>::acc>{}, size));
     return check_launch("add_kernel") ? 0 : -1;
 }
 
@@ -408,22 +594,20 @@ int mul_scalar_kernel_device(void* out, const void* x, const void* scalar, size_
     RP_DISPATCH_DTYPE(dtype, {
         using A = typename traits<T>::acc;
         A s = *(const A*)scalar;
-        hipLaunchKernelGGL(mul_scalar_kernel<T>, dim3(grid_for(size)), dim3(kThreads), 0, current_stream(), (T*)out, (const T*)x, s, size);
+        launch_map<T, false>((T*)out, (const T*)x, (const T*)nullptr, MulScalarOp<A>{s}, size);
     });
     return check_launch("mul_scalar_kernel") ? 0 : -1;
 }
 
 int relu_kernel_device(void* out, const void* x, size_t size, int dtype) {
     RP_REQUIRE(out && x && size, "relu_kernel_device");
-    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(relu_kernel<T>, dim3(grid_for(size)), dim3(kThreads), 0, current_stream(),
-                                               (T*)out, (const T*)x, size));
+    RP_DISPATCH_DTYPE(dtype, launch_map<T, false>((T*)out, (const T*)x, (const T*)nullptr, ReluOp<typename traits<T>::acc>{}, size));
     return check_launch("relu_kernel") ? 0 : -1;
 }
 
 int backwards_relu_device(const void* grad_c, const void* x, void* grad_x, size_t size, int dtype) {
     RP_REQUIRE(grad_c && x && grad_x && size, "backwards_relu_device");
-    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(backwards_relu_kernel<T>, dim3(grid_for(size)), dim3(kThreads), 0, current_stream(),
-                                               (const T*)grad_c, (const T*)x, (T*)grad_x, size));
+    RP_DISPATCH_DTYPE(dtype, launch_map<T, true>((T*)grad_x, (const T*)grad_c, (const T*)x, BackReluOp<typename traits<T>::acc>{}, size));
     return check_launch("backwards_relu_kernel") ? 0 : -1;
 }
 
@@ -432,7 +616,8 @@ static int softmax_any(void* out, const void* x, size_t outer, size_t dim, size_
     if (inner == 1) {
         unsigned blocks = grid_for(outer * 64, kThreads, 1u << 16);
         RP_DISPATCH_DTYPE(dtype, {
-            if (take_log) hipLaunchKernelGGL((softmax_rows_kernel<T, true>), dim3(blocks), dim3(kThreads), 0, current_stream(), (T*)out, (const T*)x, outer, dim);
+            if (launch_softmax_reg<T>((T*)out, (const T*)x, outer, dim, blocks, take_log)) {}
+            else if (take_log) hipLaunchKernelGGL((softmax_rows_kernel<T, true>), dim3(blocks), dim3(kThreads), 0, current_stream(), (T*)out, (const T*)x, outer, dim);
             else          hipLaunchKernelGGL((softmax_rows_kernel<T, false>), dim3(blocks), dim3(kThreads), 0, current_stream(), (T*)out, (const T*)x, outer, dim);
         });
     } else {
@@ -458,8 +643,11 @@ int backwards_softmax_device(const void* grad_c, const void* softmax_out, void* 
     RP_REQUIRE(grad_c && softmax_out && grad_x && outer_size && dim_size && inner_size, "backwards_softmax_device");
     if (inner_size == 1) {
         unsigned blocks = grid_for(outer_size * 64, kThreads, 1u << 16);
-        RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(backwards_softmax_rows_kernel<T>, dim3(blocks), dim3(kThreads), 0, current_stream(),
-                                                   (const T*)grad_c, (const T*)softmax_out, (T*)grad_x, outer_size, dim_size));
+        RP_DISPATCH_DTYPE(dtype, {
+            if (launch_bsoftmax_reg<T>((const T*)grad_c, (const T*)softmax_out, (T*)grad_x, outer_size, dim_size, blocks)) {}
+            else hipLaunchKernelGGL(backwards_softmax_rows_kernel<T>, dim3(blocks), dim3(kThreads), 0, current_stream(),
+                                    (const T*)grad_c, (const T*)softmax_out, (T*)grad_x, outer_size, dim_size);
+        });
     } else {
         RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(backwards_softmax_strided_kernel<T>, dim3(grid_for(outer_size * inner_size)), dim3(kThreads), 0,
                                                    current_stream(), (const T*)grad_c, (const T*)softmax_out, (T*)grad_x,

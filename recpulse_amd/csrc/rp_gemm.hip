@@ -74,7 +74,9 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     if (is16) {
         p.fam = FAM_MFMA16;
         long long tiles256 = (long long)((m + 255) / 256) * ((n + 255) / 256) * batch;
-        if (m >= 256 && n >= 256 && tiles256 >= 128) { p.bm = 256; p.bn = 256; p.name = "mfma16_256x256"; }
+        // the 256 x 256 tile runs one block per CU, so it needs a k loop long enough to hide its prologue and
+        // epilogue; with fewer than four slabs the smaller tile (two blocks per CU) overlaps them instead
+        if (m >= 256 && n >= 256 && tiles256 >= 128 && k >= 4 * M16_BK) { p.bm = 256; p.bn = 256; p.name = "mfma16_256x256"; }
         else if (m > 64 || n > 64) { p.bm = 128; p.bn = 128; p.name = "mfma16_128x128"; }
         else { p.bm = 64; p.bn = 64; p.name = "mfma16_64x64"; }
         p.edge = (m % p.bm) || (n % p.bn) || (k % M16_BK);

@@ -1,4 +1,4 @@
-"""The five BASELINE configurations at their real sizes, through the C ABI.
+"""The five benchmark configurations at their real sizes, through the C ABI.
 
 Full results are compared with a float64 oracle; the CPU oracle (the
 restatement of the reference's own loops) is run in full where it finishes in

@@ -188,7 +188,7 @@ class MLP(Module):
         return x
 
 
-# ---- BASELINE config 2 through the Python API: every dW, db and dX against the CPU oracle (reference autograd order)
+# ---- benchmark configuration 2 through the Python API: every dW, db and dX against the CPU oracle (reference autograd order)
 def test_config2_mlp_through_modules_matches_oracle():
     rng = np.random.default_rng(1)
     dims = [784, 256, 128, 10]; batch = 256
@@ -215,7 +215,7 @@ def test_config2_mlp_through_modules_matches_oracle():
         net(xt).op_cross_entropy_loss([10] * batch)        # out-of-range target (reference ops/ops.c:5547-5549)
 
 
-# ---- BASELINE config 4 shape (scaled down) through the Python API: batched matmul on a permuted view, forward + backward
+# ---- benchmark configuration 4 shape (scaled down) through the Python API: batched matmul on a permuted view, forward + backward
 @pytest.mark.parametrize("dtype,tol", [("float64", 1e-11), ("float32", 2e-5), ("bfloat16", 4e-2)])
 def test_attention_batched_matmul_on_permuted_view(dtype, tol):
     import torch

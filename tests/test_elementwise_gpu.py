@@ -56,7 +56,8 @@ def test_broadcasting_add_bit_exact(dt):
 @pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
 def test_softmax_family(dt):
     rng = np.random.default_rng(42)
-    for shape, dim in (((9, 10), -1), ((33, 512), -1), ((3, 17, 5), 1), ((2, 3, 64), -1)):
+    # rows of 64 .. 4096 elements take the kernels that hold a row in registers (1, 2, 4 or 8 pieces per lane, partly filled)
+    for shape, dim in (((9, 10), -1), ((33, 512), -1), ((3, 17, 5), 1), ((2, 3, 64), -1), ((5, 1024), -1), ((3, 2040), -1), ((2, 4096), -1), ((2, 4104), -1)):
         x = oracle.to_storage(rng.normal(0, 2, shape), dt); g = rand_storage(rng, shape, dt)
         o, d, i = oracle._split(shape, dim)
         dx, dg, do = Dev(x, dt), Dev(g, dt), Dev.empty(shape, dt)
