@@ -83,9 +83,10 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     } else {
         p.fam = FAM_MFMAW;
         long long tiles128 = (long long)((m + 127) / 128) * ((n + 127) / 128) * batch;
-        if ((m > 64 || n > 64) && tiles128 >= 128) { p.bm = 128; p.bn = 128; p.name = (dtype == RP_DTYPE_FLOAT32) ? "mfma32_128x128" : "mfma64_128x128"; }
+        // a 128 x 128 tile over a 64-wide output would compute and fetch half of it for nothing
+        if (m > 64 && n > 64 && tiles128 >= 128) { p.bm = 128; p.bn = 128; p.name = (dtype == RP_DTYPE_FLOAT32) ? "mfma32_128x128" : "mfma64_128x128"; }
         else { p.bm = 64; p.bn = 64; p.name = (dtype == RP_DTYPE_FLOAT32) ? "mfma32_64x64" : "mfma64_64x64"; }
-        p.edge = (m % p.bm) || (n % p.bn) || (k % (dtype == RP_DTYPE_FLOAT32 ? 16 : 8));
+        p.edge = (m % p.bm) || (n % p.bn) || (k % (dtype == RP_DTYPE_FLOAT32 ? 32 : 16));
     }
     return p;
 }

@@ -1,6 +1,8 @@
 // fp32 / fp64 MFMA GEMM kernels and their launcher.
 #include "rp_gemm.h"
 
+#include <type_traits>
+
 namespace rp {
 
 // ============================================================================
@@ -13,74 +15,94 @@ namespace rp {
 // ============================================================================
 template <typename T> struct mfmaw_cfg;
 template <> struct mfmaw_cfg<float> {
-    static constexpr int MT = 32, KS = 2, NV = 16, VEC = 4, BK = 16, PAD = 4;
+    static constexpr int MT = 32, KS = 2, NV = 16, VEC = 4, BK = 32, PAD = 4;
     using acc_t = f32x16_t;
     static __device__ __forceinline__ acc_t mma(float a, float b, acc_t c) { return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0); }
     // row of accumulator register v inside the MFMA tile
     static __device__ __forceinline__ int acc_row(int v, int lane) { return 8 * (v / 4) + 4 * (lane >> 5) + (v % 4); }
 };
 template <> struct mfmaw_cfg<double> {
-    static constexpr int MT = 16, KS = 4, NV = 4, VEC = 2, BK = 8, PAD = 2;
+    static constexpr int MT = 16, KS = 4, NV = 4, VEC = 2, BK = 16, PAD = 2;
     using acc_t = f64x4_t;
     static __device__ __forceinline__ acc_t mma(double a, double b, acc_t c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
     static __device__ __forceinline__ int acc_row(int v, int lane) { return 4 * v + (lane >> 4); }
 };
 
+template <int I, int N, typename F>
+__device__ __forceinline__ void mw_static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        mw_static_for<I + 1, N>(f);
+    }
+}
+
+// One operand's slab traffic, a 16-byte piece per thread at a time: piece i of thread t covers V consecutive
+// elements along the operand's unit-stride axis.  LDS is k-major, [BK][ROWS + PAD]; a KC piece (V consecutive k
+// of one row) is transposed on the way in with V scalar writes.
 template <typename T, int ROWS, bool MC, bool EDGE>
-__device__ __forceinline__ void mw_load_slab(T (&regs)[ROWS * mfmaw_cfg<T>::BK / 256], const T* base, long long free_stride, long long k_stride,
-                                             int row0, int k0, int free_extent, int k_extent, int t) {
+struct MwSlab {
     using cfg = mfmaw_cfg<T>;
-    constexpr int V = cfg::VEC, NVEC = ROWS * cfg::BK / V / 256;
-#pragma unroll
-    for (int i = 0; i < NVEC; i++) {
+    static constexpr int V = cfg::VEC, NP = ROWS * cfg::BK / V / 256, PITCH = ROWS + cfg::PAD;
+    static __device__ __forceinline__ void coords(int t, int i, int& r, int& kk) {
         int id = t + 256 * i;
-        int r, kk;
         if (MC) { kk = id / (ROWS / V); r = (id % (ROWS / V)) * V; }
         else    { r = id / (cfg::BK / V); kk = (id % (cfg::BK / V)) * V; }
-        const T* p = base + (long long)(row0 + r) * free_stride + (long long)(k0 + kk) * k_stride;
-        bool ok = true;
-        if (EDGE) ok = (row0 + r < free_extent) && (k0 + kk < k_extent);
-        if (ok) {
-            uint4 raw = *(const uint4*)p;
-            memcpy(&regs[i * V], &raw, 16);
-        } else {
-#pragma unroll
-            for (int e = 0; e < V; e++) regs[i * V + e] = (T)0;
-        }
     }
-}
-
-template <typename T, int ROWS, bool MC>
-__device__ __forceinline__ void mw_store_slab(const T (&regs)[ROWS * mfmaw_cfg<T>::BK / 256], T* lds, int t) {
-    using cfg = mfmaw_cfg<T>;
-    constexpr int V = cfg::VEC, NVEC = ROWS * cfg::BK / V / 256, PITCH = ROWS + cfg::PAD;
-#pragma unroll
-    for (int i = 0; i < NVEC; i++) {
-        int id = t + 256 * i;
+    // piece i of the slab that starts at k0 (relative to the block's k range of length k_extent)
+    static __device__ __forceinline__ uint4 load(const T* base, long long free_stride, long long k_stride, int row0, int k0,
+                                                 int free_extent, int k_extent, int t, int i) {
+        int r, kk;
+        coords(t, i, r, kk);
+        if (EDGE && !((row0 + r < free_extent) && (k0 + kk < k_extent))) return uint4{0u, 0u, 0u, 0u};
+        return *(const uint4*)(base + (long long)(row0 + r) * free_stride + (long long)(k0 + kk) * k_stride);
+    }
+    static __device__ __forceinline__ void store(T* lds, uint4 raw, int t, int i) {
+        int r, kk;
+        coords(t, i, r, kk);
         if (MC) {
-            int kk = id / (ROWS / V), r = (id % (ROWS / V)) * V;
-            uint4 raw;
-            memcpy(&raw, &regs[i * V], 16);
             *(uint4*)(lds + kk * PITCH + r) = raw;
         } else {
-            int r = id / (cfg::BK / V), kk = (id % (cfg::BK / V)) * V;
+            T e[V];
+            memcpy(e, &raw, 16);
 #pragma unroll
-            for (int e = 0; e < V; e++) lds[(kk + e) * PITCH + r] = regs[i * V + e];
+            for (int q = 0; q < V; q++) lds[(kk + q) * PITCH + r] = e[q];
         }
     }
+};
+
+// ============================================================================
+// Block tile BM x BN, 4 waves in a 2 x 2 grid, k slab BK, two LDS stages.
+// Software pipeline per slab s (NKS k-steps of one MFMA depth each):
+//   k-steps 0 .. NKS-2   MFMAs(ks) | fragments(ks+1) from LDS | a share of: registers holding slab s+1 -> the
+//                        other LDS stage, then the global load of slab s+2 into the register just freed
+//   barrier              slab s+1 is complete in LDS and nobody reads this slab's stage any more
+//   k-step NKS-1         MFMAs | fragments(0) of slab s+1
+// so LDS reads run a k-step ahead of the MFMAs, global loads get a whole slab to land, and one barrier per
+// slab sits where a single MFMA group is left to issue.  The epilogue stages accumulators through LDS, 32
+// columns per pass, so that every lane stores 16 bytes of one output row.
+// With SPLITK the grid's z axis splits k (k_per_split a multiple of BK): blocks write fp32 partial tiles
+// [split][m][n] and the shared combine kernel finishes (fp32 only).
+// ============================================================================
+template <typename T> __host__ __device__ constexpr int mw_epi_pitch() { return 32 + 16 / (int)sizeof(T); }
+template <typename T>
+__host__ __device__ constexpr size_t mw_smem_bytes(int bm, int bn) {
+    size_t loop = 2 * (size_t)mfmaw_cfg<T>::BK * (bm + bn + 2 * mfmaw_cfg<T>::PAD) * sizeof(T);
+    size_t epi = 4 * (size_t)(bm / 2) * mw_epi_pitch<T>() * sizeof(T);
+    return loop > epi ? loop : epi;
 }
 
-// With SPLITK the grid's z axis splits k (k_per_split is a multiple of BK): every block writes its fp32 partial
-// tile [split][m][n] to a workspace and the shared combine kernel finishes (fp32 only).
 template <typename T, int BM, int BN, bool A_MC, bool B_MC, bool EDGE, bool SPLITK>
-__global__ void __launch_bounds__(256) gemm_mfmaw_kernel(GemmArgs g, int tiles_m, int tiles_n, float* partials, int k_per_split) {
+__global__ void __launch_bounds__(256, 2) gemm_mfmaw_kernel(GemmArgs g, int tiles_m, int tiles_n, float* partials, int k_per_split) {
     using cfg = mfmaw_cfg<T>;
-    constexpr int MT = cfg::MT, BK = cfg::BK;
+    constexpr int MT = cfg::MT, BK = cfg::BK, NKS = BK / cfg::KS;
     constexpr int WM = BM / 2, WN = BN / 2, TMI = WM / MT, TNI = WN / MT;
     constexpr int PA = BM + cfg::PAD, PB = BN + cfg::PAD;
-    constexpr int A_ELEMS = BK * PA, B_ELEMS = BK * PB;
-    __shared__ __attribute__((aligned(16))) T smem[2 * (A_ELEMS + B_ELEMS)];
-    constexpr int STAGE = A_ELEMS + B_ELEMS;
+    constexpr int A_ELEMS = BK * PA, B_ELEMS = BK * PB, STAGE = A_ELEMS + B_ELEMS;
+    using SlabA = MwSlab<T, BM, A_MC, EDGE>;
+    using SlabB = MwSlab<T, BN, B_MC, EDGE>;
+    constexpr int NA = SlabA::NP, NB = SlabB::NP, NP_ALL = NA + NB;
+    extern __shared__ __attribute__((aligned(16))) unsigned char mw_smem_raw[];
+    T* smem = (T*)mw_smem_raw;
 
     TileCoord tc = schedule_tile(blockIdx.x, tiles_m, tiles_n);
     if (!tc.valid) return;
@@ -103,69 +125,137 @@ __global__ void __launch_bounds__(256) gemm_mfmaw_kernel(GemmArgs g, int tiles_m
 #pragma unroll
             for (int v = 0; v < cfg::NV; v++) acc[i][j][v] = (T)0;
 
-    T ra[BM * BK / 256], rb[BN * BK / 256];
+    uint4 regs[NP_ALL];                        // pieces 0 .. NA-1 are A's, the rest B's
     const int nslabs = (klen + BK - 1) / BK;
-    mw_load_slab<T, BM, A_MC, EDGE>(ra, A, a_fs, a_ks, m0, 0, g.m, klen, t);
-    mw_load_slab<T, BN, B_MC, EDGE>(rb, B, b_fs, b_ks, n0, 0, g.n, klen, t);
-    mw_store_slab<T, BM, A_MC>(ra, smem, t);
-    mw_store_slab<T, BN, B_MC>(rb, smem + A_ELEMS, t);
-    __syncthreads();
+    auto load_piece = [&](auto pc, int k0) {
+        constexpr int p = decltype(pc)::value;
+        if constexpr (p < NA) regs[p] = SlabA::load(A, a_fs, a_ks, m0, k0, g.m, klen, t, p);
+        else regs[p] = SlabB::load(B, b_fs, b_ks, n0, k0, g.n, klen, t, p - NA);
+    };
+    auto store_piece = [&](auto pc, T* stage) {
+        constexpr int p = decltype(pc)::value;
+        if constexpr (p < NA) SlabA::store(stage, regs[p], t, p);
+        else SlabB::store(stage + A_ELEMS, regs[p], t, p - NA);
+    };
 
     const int lf = lane % MT, lk = lane / MT;         // lane's free index and k index inside one MFMA
-    for (int s = 0; s < nslabs; s++) {
-        const int cur = s & 1;
-        const bool more = (s + 1 < nslabs);
-        if (more) {
-            mw_load_slab<T, BM, A_MC, EDGE>(ra, A, a_fs, a_ks, m0, (s + 1) * BK, g.m, klen, t);
-            mw_load_slab<T, BN, B_MC, EDGE>(rb, B, b_fs, b_ks, n0, (s + 1) * BK, g.n, klen, t);
-        }
-        const T* a_lds = smem + cur * STAGE;
-        const T* b_lds = a_lds + A_ELEMS;
+    T af[2][TMI], bf[2][TNI];
+    auto read_frags = [&](const T* stage, int ks, int slot) {
+        const int kk = ks * cfg::KS + lk;
 #pragma unroll
-        for (int ks = 0; ks < BK / cfg::KS; ks++) {
-            T af[TMI], bf[TNI];
-            int kk = ks * cfg::KS + lk;
+        for (int i = 0; i < TMI; i++) af[slot][i] = stage[kk * PA + wm0 + i * MT + lf];
 #pragma unroll
-            for (int i = 0; i < TMI; i++) af[i] = a_lds[kk * PA + wm0 + i * MT + lf];
-#pragma unroll
-            for (int j = 0; j < TNI; j++) bf[j] = b_lds[kk * PB + wn0 + j * MT + lf];
+        for (int j = 0; j < TNI; j++) bf[slot][j] = stage[A_ELEMS + kk * PB + wn0 + j * MT + lf];
+    };
+
+    // prologue: slab 0 into stage 0, slab 1 into registers, fragments(0) of slab 0
+    mw_static_for<0, NP_ALL>([&](auto pc) { load_piece(pc, 0); });
+    mw_static_for<0, NP_ALL>([&](auto pc) { store_piece(pc, smem); });
+    if (nslabs > 1) mw_static_for<0, NP_ALL>([&](auto pc) { load_piece(pc, BK); });
+    __syncthreads();
+    read_frags(smem, 0, 0);
+
+    // One slab.  NEXT: slab s+1 exists (its registers go to LDS here and the barrier runs); NEXT2: slab s+2 exists
+    // (its global loads are issued here).  Both are compile-time so that the steady-state loop issues its loads
+    // unconditionally and the waits the compiler places before each LDS store count them exactly.
+    auto slab_step = [&](int s, auto next_tag, auto next2_tag) {
+        constexpr bool NEXT = decltype(next_tag)::value, NEXT2 = decltype(next2_tag)::value;
+        const T* stage = smem + (s & 1) * STAGE;
+        T* other = smem + ((s & 1) ^ 1) * STAGE;
+        mw_static_for<0, NKS>([&](auto ksc) {
+            constexpr int ks = decltype(ksc)::value, slot = ks & 1;
+            if constexpr (ks + 1 < NKS) {
+                read_frags(stage, ks + 1, slot ^ 1);
+                // this k-step's share of the slab traffic
+                constexpr int P0 = (NP_ALL * ks) / (NKS - 1), P1 = (NP_ALL * (ks + 1)) / (NKS - 1);
+                if constexpr (NEXT) {
+                    mw_static_for<P0, P1>([&](auto pc) {
+                        store_piece(pc, other);
+                        if constexpr (NEXT2) load_piece(pc, (s + 2) * BK);
+                    });
+                }
+            } else if constexpr (NEXT) {
+                __syncthreads();
+                read_frags(other, 0, slot ^ 1);
+            }
 #pragma unroll
             for (int i = 0; i < TMI; i++)
 #pragma unroll
-                for (int j = 0; j < TNI; j++) acc[i][j] = cfg::mma(af[i], bf[j], acc[i][j]);
-        }
-        if (more) {
-            mw_store_slab<T, BM, A_MC>(ra, smem + (cur ^ 1) * STAGE, t);
-            mw_store_slab<T, BN, B_MC>(rb, smem + (cur ^ 1) * STAGE + A_ELEMS, t);
-        }
-        __syncthreads();
-    }
+                for (int j = 0; j < TNI; j++) acc[i][j] = cfg::mma(af[slot][i], bf[slot][j], acc[i][j]);
+        });
+    };
+    using yes = std::true_type;
+    using no = std::false_type;
+    int s = 0;
+    for (; s + 2 < nslabs; s++) slab_step(s, yes{}, yes{});
+    if (s + 1 < nslabs) { slab_step(s, yes{}, no{}); s++; }
+    slab_step(s, no{}, no{});
 
+    // ---- epilogue: 32 columns of every wave's patch per pass through the wave's private LDS region ----
+    constexpr int V = cfg::VEC, CN = 32, EP = mw_epi_pitch<T>(), TJ = CN / MT, PASSES = WN / CN;
+    constexpr int LPR = CN / V, RPS = 64 / LPR;          // lanes per row, rows per step
+    T* region = smem + wave * (WM * EP);
     T* C = (T*)g.C + (long long)z * g.c_bs;
     const T* bias = (const T*)g.bias;
     const bool has_bias = bias != nullptr, accum = g.accumulate != 0;
+    const bool c_vec = (g.c_cs == 1) && (g.c_rs % V == 0) && (((uintptr_t)C & 15) == 0);
+    const int ecol = (lane % LPR) * V, erow = lane / LPR;
 #pragma unroll
-    for (int j = 0; j < TNI; j++) {
-        int gn = n0 + wn0 + j * MT + lf;
-        bool n_ok = !EDGE || gn < g.n;
-        T bv = (has_bias && n_ok) ? bias[gn] : (T)0;
+    for (int p = 0; p < PASSES; p++) {
+        __syncthreads();                        // the main loop (or the previous pass) is done with LDS
 #pragma unroll
-        for (int i = 0; i < TMI; i++) {
+        for (int i = 0; i < TMI; i++)
 #pragma unroll
-            for (int v = 0; v < cfg::NV; v++) {
-                int gm = m0 + wm0 + i * MT + cfg::acc_row(v, lane);
-                if (n_ok && (!EDGE || gm < g.m)) {
-                    if constexpr (SPLITK) {
-                        partials[((long long)blockIdx.z * g.m + gm) * g.n + gn] = (float)acc[i][j][v];
-                    } else {
-                        T* p = C + (long long)gm * g.c_rs + (long long)gn * g.c_cs;
-                        T old = accum ? *p : (T)0;
-                        *p = finish<T>(acc[i][j][v], has_bias, bv, accum, old);
-                    }
+            for (int jj = 0; jj < TJ; jj++)
+#pragma unroll
+                for (int v = 0; v < cfg::NV; v++)
+                    region[(i * MT + cfg::acc_row(v, lane)) * EP + jj * MT + lf] = acc[i][p * TJ + jj][v];
+        __syncthreads();
+        const int gn = n0 + wn0 + p * CN + ecol;
+        T bv[V];
+#pragma unroll
+        for (int e = 0; e < V; e++) bv[e] = (has_bias && (!EDGE || gn + e < g.n)) ? bias[gn + e] : (T)0;
+#pragma unroll 2
+        for (int r = erow; r < WM; r += RPS) {
+            const int gm = m0 + wm0 + r;
+            if (EDGE && gm >= g.m) break;
+            uint4 raw = *(const uint4*)(region + r * EP + ecol);
+            T vals[V];
+            memcpy(vals, &raw, 16);
+            if constexpr (SPLITK) {
+                // fp32 partial tile [split][m][n]; n is a multiple of 4 on this path, so the vector is wholly in or out
+                if (!EDGE || gn + V <= g.n) *(uint4*)(partials + ((long long)blockIdx.z * g.m + gm) * g.n + gn) = raw;
+                continue;
+            }
+            T* crow = C + (long long)gm * g.c_rs;
+            if (c_vec && (!EDGE || gn + V <= g.n)) {
+                T old[V], out[V];
+                if (accum) { uint4 o = *(const uint4*)(crow + gn); memcpy(old, &o, 16); }
+#pragma unroll
+                for (int e = 0; e < V; e++) out[e] = finish<T>(vals[e], has_bias, bv[e], accum, accum ? old[e] : (T)0);
+                uint4 o;
+                memcpy(&o, out, 16);
+                *(uint4*)(crow + gn) = o;
+            } else {
+#pragma unroll
+                for (int e = 0; e < V; e++) {
+                    if (EDGE && gn + e >= g.n) break;
+                    T* pc = crow + (long long)(gn + e) * g.c_cs;
+                    T old = accum ? *pc : (T)0;
+                    *pc = finish<T>(vals[e], has_bias, bv[e], accum, old);
                 }
             }
         }
     }
+}
+
+template <typename T, int BM, int BN, bool A_MC, bool B_MC, bool EDGE, bool SPLITK>
+static int mw_launch(const GemmArgs& g, dim3 grid, int tiles_m, int tiles_n, float* partials, int k_per_split) {
+    constexpr size_t smem = mw_smem_bytes<T>(BM, BN);
+    auto kern = gemm_mfmaw_kernel<T, BM, BN, A_MC, B_MC, EDGE, SPLITK>;
+    if (smem > 64 * 1024 && !check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem), "hipFuncSetAttribute")) return -1;
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, current_stream(), g, tiles_m, tiles_n, partials, k_per_split);
+    return check_launch("gemm_mfmaw_kernel") ? 0 : -1;
 }
 
 template <typename T, int BM, int BN, bool A_MC, bool B_MC>
@@ -174,16 +264,14 @@ static int launch_mfmaw_edge(const GemmArgs& g, bool edge, float* partials, int 
     if (nsplit > 1) {
         if constexpr (sizeof(T) == 4) {           // split-k partials are fp32; always the predicated variant
             dim3 grid(scheduled_grid(tiles_m, tiles_n), g.batch, nsplit);
-            hipLaunchKernelGGL((gemm_mfmaw_kernel<T, BM, BN, A_MC, B_MC, true, true>), grid, dim3(256), 0, current_stream(), g, tiles_m, tiles_n, partials, k_per_split);
-            return check_launch("gemm_mfmaw_kernel") ? 0 : -1;
+            return mw_launch<T, BM, BN, A_MC, B_MC, true, true>(g, grid, tiles_m, tiles_n, partials, k_per_split);
         }
         set_error("mfmaw GEMM: split-k is fp32 only");
         return -1;
     }
     dim3 grid(scheduled_grid(tiles_m, tiles_n), g.batch);
-    if (edge) hipLaunchKernelGGL((gemm_mfmaw_kernel<T, BM, BN, A_MC, B_MC, true, false>), grid, dim3(256), 0, current_stream(), g, tiles_m, tiles_n, nullptr, 0);
-    else      hipLaunchKernelGGL((gemm_mfmaw_kernel<T, BM, BN, A_MC, B_MC, false, false>), grid, dim3(256), 0, current_stream(), g, tiles_m, tiles_n, nullptr, 0);
-    return check_launch("gemm_mfmaw_kernel") ? 0 : -1;
+    if (edge) return mw_launch<T, BM, BN, A_MC, B_MC, true, false>(g, grid, tiles_m, tiles_n, nullptr, 0);
+    return mw_launch<T, BM, BN, A_MC, B_MC, false, false>(g, grid, tiles_m, tiles_n, nullptr, 0);
 }
 
 template <typename T, int BM, int BN>
@@ -197,12 +285,12 @@ static int launch_mfmaw_layout(const GemmArgs& g, const Plan& p, float* partials
 template <typename T>
 static int launch_mfmaw_t(const GemmArgs& g, const Plan& p) {
     // Small outputs with a deep k leave most CUs idle: split k so that about 256 blocks run (each split at
-    // least four slabs deep), and add the partials in split order afterwards.  fp32 only, one matrix at a time.
+    // least two slabs deep), and add the partials in split order afterwards.  fp32 only, one matrix at a time.
     int nsplit = 1, k_per_split = 0;
     constexpr int BK = mfmaw_cfg<T>::BK;
     if (sizeof(T) == 4 && g.batch == 1 && p.bm == 64 && g.n % 4 == 0) {
         int tiles = ((g.m + 63) / 64) * ((g.n + 63) / 64);
-        int want = (256 + tiles - 1) / tiles, deep = g.k / (4 * BK);
+        int want = (256 + tiles - 1) / tiles, deep = g.k / (2 * BK);
         nsplit = want < deep ? want : deep;
         if (nsplit > 1) {
             k_per_split = ((g.k + nsplit - 1) / nsplit + BK - 1) / BK * BK;
