@@ -156,14 +156,14 @@ def cpu_baseline(a, b, rows=8):
                       f"host has {os.cpu_count()} logical cores"}
 
 
-def secondary(capi, quick_reps=20):
+def skinny_times(capi, quick_reps=20, rows=(1, 8, 32)):
+    """Config 5a: bf16 A[m, 8192] x W[8192, 8192], replayed from a HIP graph; bytes are A, W and the output once."""
     out = {}
     rng = np.random.default_rng(4)
-    # config 5a: skinny bf16 GEMMs, K = N = 8192
     k = n = 8192
     w = _normal_bf16(rng, (k, n))
     d_w = capi.DeviceBuffer.from_numpy(w)
-    for m in (1, 8, 32):
+    for m in rows:
         a = _normal_bf16(rng, (m, k))
         d_a = capi.DeviceBuffer.from_numpy(a); d_y = capi.DeviceBuffer(m * n * 2)
         fn = lambda: capi.gemm(d_y.ptr, d_a.ptr, d_w.ptr, None, 1, m, k, n, (0, k, 1), (0, n, 1), (0, n, 1), False, capi.BF16)
@@ -171,7 +171,13 @@ def secondary(capi, quick_reps=20):
         nbytes = (m * k + k * n + m * n) * 2
         out[f"skinny_bf16_m{m}"] = {"us": ms * 1e3, "GB/s": nbytes / (ms * 1e-3) / 1e9, "frac_hbm": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
                                     "kernel": capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), capi.BF16)}
-    # config 3: fp32 at 4096, fp16 at 8192; config 5b: fp64 at 2048
+    return out
+
+
+def secondary(capi, quick_reps=20):
+    out = skinny_times(capi, quick_reps)
+    rng = np.random.default_rng(5)
+    # config 3: fp32 at 4096; config 5b: fp64 at 2048
     for name, dt, npdt, size, peak in (("gemm_f32_4096", capi.F32, np.float32, 4096, PEAK_TFLOPS["f32"]),
                                        ("gemm_f64_2048", capi.F64, np.float64, 2048, PEAK_TFLOPS["f64"])):
         a = rng.standard_normal((size, size)).astype(npdt); b = rng.standard_normal((size, size)).astype(npdt)
@@ -182,8 +188,9 @@ def secondary(capi, quick_reps=20):
         ms = _time_launches(capi, fn, 10, 3)
         tf = 2.0 * size ** 3 / (ms * 1e-3) / 1e12
         out[name] = {"ms": ms, "TFLOP/s": tf, "frac_mfma": tf / peak}
-    # config 4: attention-shaped batched GEMMs on stride views, bf16
+    # config 4: attention-shaped batched GEMMs on stride views
     out["attention_bf16"] = attention_times(capi, "bf16")
+    out["attention_f32"] = attention_times(capi, "f32")
     # config 2: fp32 MLP 784-256-128-10, batch 256, forward + backward through the C ABI (9 GEMMs + neighbours)
     out["mlp_f32_step"] = mlp_step_time(capi)
     return out
@@ -284,6 +291,8 @@ def main():
     ap.add_argument("--data", choices=["normal", "ints", "ones", "zeros"], default="normal",
                     help="operand values of the headline GEMMs: N(0,1) (the configuration) or low-toggle data, to show how far the "
                          "power-managed shader clock, and with it the throughput, depends on the values multiplied")
+    ap.add_argument("--skinny-only", action="store_true",
+                    help="run only the few-row bf16 GEMMs of configuration 5a and print their figures (for profiling that kernel alone)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain copy kernel of known size (256 MiB in, 256 MiB out), the yardstick for FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
@@ -305,6 +314,9 @@ def main():
             capi.check(capi.lib().rp_hip_convert(dst.ptr, capi.F32, src.ptr, capi.F32, n), "copy")
         capi.synchronize()
         src.free(); dst.free()
+    if args.skinny_only:
+        print(json.dumps({"skinny": skinny_times(capi, rows=(1, 8))}))
+        return
     h = headline(capi, args.steps, args.warmup, data=args.data)
     a, b = h.pop("operands")
     line = {

@@ -81,6 +81,34 @@ static inline int scheduled_grid(int tiles_m, int tiles_n) {
 }
 
 
+// ----------------------------------------------------------------------------
+// Single-launch finish of a k split.
+// The blocks that share an output tile write fp32 partial tiles [split][m][n] with device-scope stores (cache
+// policy sc1: written through the per-XCD L2s, which are not coherent with each other), wait until their own
+// stores are acknowledged, and count themselves in with a device-scope atomic.  The block that arrives last
+// re-reads every split's tile with device-scope loads, adds them in split order (so the result does not depend
+// on which block that is), runs the epilogue and leaves the counter at zero for the next launch.  No cache-wide
+// write-back or invalidate is involved.  The finish is a chain of three device-scope round trips (store
+// acknowledge, atomic, partial loads), about 3 us: it beats a second launch for the long streaming kernel, whose
+// blocks all end together, and loses to it for the few-microsecond split-k GEMMs of small layers, which
+// therefore keep the separate combine kernel.
+// ----------------------------------------------------------------------------
+constexpr int SPLITK_DEVICE_SCOPE = 16;      // buffer cache-policy bit sc1
+constexpr int SPLITK_MAX_TILES = 1024;       // arrival counters per device
+constexpr uint32_t SPLITK_OOB = 0x80000000u; // an offset no partial buffer covers (they are kept below 2 GiB)
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t splitk_rsrc(const float* partials, long long bytes) {
+    int n = bytes <= 0 ? 0 : (bytes > 0x7fffffffll ? 0x7fffffff : (int)bytes);
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(partials), 0, n, 0x00020000);
+}
+
+// The device's block of SPLITK_MAX_TILES zeroed arrival counters (created on first use, kept for the life of the
+// process), or nullptr when the single-launch finish cannot be used: more tiles than counters, partials of 2 GiB
+// or more, RP_HIP_SPLITK_TWO_LAUNCH=1, or an allocation failure (then last_error is set and *failed is true).
+// Like the workspace pool the block is not stream-aware: launches that may run at the same time on different
+// streams of one device must be serialised by the caller.
+int* splitk_arrival_counters(long long tiles, size_t partial_bytes, bool* failed);
+
 // per-family launchers (dtype is one of the RP_DTYPE_* codes the family supports)
 int launch_generic(const GemmArgs& g, int dtype);
 int launch_skinny(const GemmArgs& g, int dtype);

@@ -3,19 +3,25 @@
 // row-major B (bound by streaming B from HBM).
 #include "rp_gemm.h"
 
+#include <mutex>
+
 namespace rp {
 
 // ============================================================================
 // generic: 64x64 output tile, 16-deep k slabs, 256 threads each owning 4x4.
 // ============================================================================
-template <typename T>
-__global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g) {
+// With SPLITK (one matrix, fp32 accumulation) the grid's z axis splits k instead of walking the batch: every
+// block writes its fp32 partial tile [split][m][n] to a workspace and the combine kernel finishes.
+template <typename T, bool SPLITK>
+__global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g, float* partials, int k_per_split) {
     using Acc = typename traits<T>::acc;
     constexpr int TM = 64, TN = 64, TK = 16;
     __shared__ Acc As[TK][TM + 1];
     __shared__ Acc Bs[TK][TN + 1];
 
-    const int z = blockIdx.z;
+    const int z = SPLITK ? 0 : blockIdx.z;
+    const int kbeg = SPLITK ? blockIdx.z * k_per_split : 0;
+    const int kend = SPLITK ? (kbeg + k_per_split < g.k ? kbeg + k_per_split : g.k) : g.k;
     const T* A = (const T*)g.A + (long long)z * g.a_bs;
     const T* B = (const T*)g.B + (long long)z * g.b_bs;
     T* C = (T*)g.C + (long long)z * g.c_bs;
@@ -40,7 +46,7 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g) {
             int kk = a_kfast ? id % TK : id / TM;
             int r = a_kfast ? id / TK : id % TM;
             int gm = m0 + r, gk = k0 + kk;
-            ra[i] = (gm < g.m && gk < g.k) ? widen(A[(long long)gm * g.a_rs + (long long)gk * g.a_cs]) : (Acc)0;
+            ra[i] = (gm < g.m && gk < kend) ? widen(A[(long long)gm * g.a_rs + (long long)gk * g.a_cs]) : (Acc)0;
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -48,11 +54,11 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g) {
             int kk = b_nfast ? id / TN : id % TK;
             int c = b_nfast ? id % TN : id / TK;
             int gn = n0 + c, gk = k0 + kk;
-            rb[i] = (gn < g.n && gk < g.k) ? widen(B[(long long)gk * g.b_rs + (long long)gn * g.b_cs]) : (Acc)0;
+            rb[i] = (gn < g.n && gk < kend) ? widen(B[(long long)gk * g.b_rs + (long long)gn * g.b_cs]) : (Acc)0;
         }
     };
-    fetch(0);
-    for (int k0 = 0; k0 < g.k; k0 += TK) {
+    fetch(kbeg);
+    for (int k0 = kbeg; k0 < kend; k0 += TK) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             int id = t + 256 * i;
@@ -60,7 +66,7 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g) {
             Bs[b_nfast ? id / TN : id % TK][b_nfast ? id % TN : id / TK] = rb[i];
         }
         __syncthreads();
-        if (k0 + TK < g.k) fetch(k0 + TK);
+        if (k0 + TK < kend) fetch(k0 + TK);
 #pragma unroll
         for (int kk = 0; kk < TK; kk++) {
             Acc a[4], b[4];
@@ -85,6 +91,10 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g) {
         for (int j = 0; j < 4; j++) {
             int gn = n0 + tx * 4 + j;
             if (gn >= g.n) continue;
+            if constexpr (SPLITK) {
+                partials[((long long)blockIdx.z * g.m + gm) * g.n + gn] = (float)acc[i][j];
+                continue;
+            }
             T* p = C + (long long)gm * g.c_rs + (long long)gn * g.c_cs;
             T old = g.accumulate ? *p : T{};
             T bv = bias ? bias[gn] : T{};
@@ -256,7 +266,63 @@ __global__ void __launch_bounds__(256) gemm_splitk_combine_kernel(GemmArgs g, co
     }
 }
 
+int* splitk_arrival_counters(long long tiles, size_t partial_bytes, bool* failed) {
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex mu;
+    static int* blocks[MAX_DEVICES] = {};
+    static int two_launch = -1;
+    *failed = false;
+    if (two_launch < 0) { const char* e = getenv("RP_HIP_SPLITK_TWO_LAUNCH"); two_launch = (e && e[0] == '1') ? 1 : 0; }
+    if (two_launch == 1 || tiles > SPLITK_MAX_TILES || partial_bytes >= (1ull << 31)) return nullptr;
+    int dev = 0;
+    if (rp_hip_get_device(&dev) != 0) { *failed = true; return nullptr; }
+    if (dev < 0 || dev >= MAX_DEVICES) return nullptr;
+    std::lock_guard<std::mutex> lock(mu);
+    if (blocks[dev]) return blocks[dev];
+    void* p = nullptr;
+    if (rp_hip_malloc(&p, SPLITK_MAX_TILES * sizeof(int)) != 0) { *failed = true; return nullptr; }
+    if (rp_hip_memset(p, 0, SPLITK_MAX_TILES * sizeof(int)) != 0) { rp_hip_free(p); *failed = true; return nullptr; }      // a fill kernel on the current stream
+    blocks[dev] = (int*)p;
+    return blocks[dev];
+}
+
+// the same for any n: one thread per output element
+template <typename T>
+__global__ void __launch_bounds__(256) gemm_splitk_combine_scalar_kernel(GemmArgs g, const float* partials, int nsplit, int part_rows) {
+    const int item = blockIdx.x * 256 + threadIdx.x;
+    if (item >= g.m * g.n) return;
+    const int r = item / g.n, c = item - r * g.n;
+    const float* q = partials + (long long)r * g.n + c;
+    const long long split_stride = (long long)part_rows * g.n;
+    float sum = 0.f;
+    int s = 0;
+    for (; s + 8 <= nsplit; s += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = q[(s + u) * split_stride];
+#pragma unroll
+        for (int u = 0; u < 8; u++) sum += v[u];
+    }
+    for (; s < nsplit; s++) sum += q[s * split_stride];
+    T* C = (T*)g.C;
+    const T* bias = (const T*)g.bias;
+    const bool has_bias = bias != nullptr, accum = g.accumulate != 0;
+    T* p = C + (long long)r * g.c_rs + (long long)c * g.c_cs;
+    T old = accum ? *p : T{};
+    *p = finish<T>(sum, has_bias, has_bias ? bias[c] : T{}, accum, old);
+}
+
 int launch_splitk_combine(const GemmArgs& g, const float* partials, int nsplit, int part_rows, int dtype) {
+    if (g.n % 4) {
+        dim3 sgrid((g.m * g.n + 255) / 256);
+        switch (dtype) {
+            case RP_DTYPE_FLOAT32:  hipLaunchKernelGGL(gemm_splitk_combine_scalar_kernel<float>, sgrid, dim3(256), 0, current_stream(), g, partials, nsplit, part_rows); break;
+            case RP_DTYPE_FLOAT16:  hipLaunchKernelGGL(gemm_splitk_combine_scalar_kernel<f16_t>, sgrid, dim3(256), 0, current_stream(), g, partials, nsplit, part_rows); break;
+            case RP_DTYPE_BFLOAT16: hipLaunchKernelGGL(gemm_splitk_combine_scalar_kernel<bf16_t>, sgrid, dim3(256), 0, current_stream(), g, partials, nsplit, part_rows); break;
+            default: set_error("split-k combine: unsupported dtype %d", dtype); return -1;
+        }
+        return check_launch("gemm_splitk_combine_scalar_kernel") ? 0 : -1;
+    }
     int items = g.m * (g.n / 4);
     dim3 grid((items + 255) / 256);
     switch (dtype) {
@@ -270,8 +336,27 @@ int launch_splitk_combine(const GemmArgs& g, const float* partials, int nsplit, 
 
 template <typename T>
 static int launch_generic_t(const GemmArgs& g) {
+    const int tiles = ((g.n + 63) / 64) * ((g.m + 63) / 64);
+    // A single small output with a deep k would run on a handful of CUs: split k across about 128 blocks, each
+    // at least two 16-deep slabs, and add the partials in split order afterwards (fp32 accumulation only).
+    if (sizeof(typename traits<T>::acc) == 4 && g.batch == 1 && tiles < 64 && g.k >= 64) {
+        int nsplit = (128 + tiles - 1) / tiles;
+        if (nsplit > g.k / 32) nsplit = g.k / 32;
+        int k_per_split = ((g.k + nsplit - 1) / nsplit + 15) / 16 * 16;
+        nsplit = (g.k + k_per_split - 1) / k_per_split;
+        if (nsplit > 1) {
+            void* ws = nullptr;
+            if (rp_hip_malloc(&ws, (size_t)nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
+            dim3 grid((g.n + 63) / 64, (g.m + 63) / 64, nsplit);
+            hipLaunchKernelGGL((gemm_generic_kernel<T, true>), grid, dim3(256), 0, current_stream(), g, (float*)ws, k_per_split);
+            int rc = check_launch("gemm_generic_kernel") ? 0 : -1;
+            if (rc == 0) rc = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, traits<T>::code);
+            rp_hip_free(ws);      // stream-ordered reuse: the pool hands it out again only to later work on this stream
+            return rc;
+        }
+    }
     dim3 grid((g.n + 63) / 64, (g.m + 63) / 64, g.batch);
-    hipLaunchKernelGGL(gemm_generic_kernel<T>, grid, dim3(256), 0, current_stream(), g);
+    hipLaunchKernelGGL((gemm_generic_kernel<T, false>), grid, dim3(256), 0, current_stream(), g, nullptr, 0);
     return check_launch("gemm_generic_kernel") ? 0 : -1;
 }
 

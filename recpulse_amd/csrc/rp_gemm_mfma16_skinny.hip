@@ -6,7 +6,6 @@
 // across the grid so that enough waves stream B to saturate HBM, and both add the splits in split order.
 #include "rp_gemm_mfma16_kernel.h"
 
-#include <mutex>
 
 namespace rp {
 
@@ -31,8 +30,6 @@ namespace rp {
 // the group's partials and writes the output (otherwise a second kernel does).
 // ============================================================================
 constexpr int SS_WAVES = 4, SS_COLS = 256, SS_ROUND = 16, SS_RED_PITCH = SS_COLS + 8;
-constexpr int SS_DEVICE_SCOPE = 16;    // buffer cache-policy bit sc1: the access is coherent across the device's XCDs
-constexpr int SS_MAX_FUSED_GROUPS = 1024;
 constexpr int SS_MAX_M = 16;
 constexpr int SS_DEPTH = 4;            // rounds a wave keeps in flight (register slots)
 
@@ -142,7 +139,7 @@ __global__ void __launch_bounds__(256) gemm_stream16_kernel(GemmArgs g, float* p
             for (int w = 1; w < SS_WAVES; w++) sum += *(const f32x4_t*)(red + (w * 8 + r) * SS_RED_PITCH + c4);
             if (nsplit > 1) {
                 const long long at = ((long long)split * g.m + gm) * g.n + gn;
-                if (arrivals) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sum), part_rsrc, (int)(at * 4), 0, SS_DEVICE_SCOPE);
+                if (arrivals) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sum), part_rsrc, (int)(at * 4), 0, SPLITK_DEVICE_SCOPE);
                 else *(f32x4_t*)(partials + at) = sum;
             } else {
 #pragma unroll
@@ -190,7 +187,7 @@ __global__ void __launch_bounds__(256) gemm_stream16_kernel(GemmArgs g, float* p
 #pragma unroll
                 for (int q = 0; q < 2; q++) {
                     const bool in = live[q] && sp + u < nsplit;
-                    v[q][u] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, in ? (int)(at[q] + (sp + u) * split_stride * 4) : (int)M16_OOB, 0, SS_DEVICE_SCOPE);
+                    v[q][u] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, in ? (int)(at[q] + (sp + u) * split_stride * 4) : (int)M16_OOB, 0, SPLITK_DEVICE_SCOPE);
                 }
 #pragma unroll
             for (int u = 0; u < 8; u++)
@@ -219,32 +216,6 @@ static int launch_stream16_t(const GemmArgs& g, float* partials, int nsplit, int
     return check_launch("gemm_stream16_kernel") ? 0 : -1;
 }
 
-// Arrival counters of the single-launch finish: one zeroed block of SS_MAX_FUSED_GROUPS ints per device, created
-// on first use and kept for the life of the process.  A launch leaves its counters at zero again, so launches
-// that follow each other in stream order share them.  Like the workspace pool, the block is not stream-aware:
-// launches that may run at the same time on different streams of one device must be serialised by the caller.
-static int* arrival_counters() {
-    constexpr int MAX_DEVICES = 64;
-    static std::mutex mu;
-    static int* blocks[MAX_DEVICES] = {};
-    int dev = 0;
-    if (rp_hip_get_device(&dev) != 0) return nullptr;
-    if (dev < 0 || dev >= MAX_DEVICES) { set_error("streaming GEMM: device ordinal %d out of range", dev); return nullptr; }
-    std::lock_guard<std::mutex> lock(mu);
-    if (blocks[dev]) return blocks[dev];
-    void* p = nullptr;
-    if (rp_hip_malloc(&p, SS_MAX_FUSED_GROUPS * sizeof(int)) != 0) return nullptr;
-    if (rp_hip_memset(p, 0, SS_MAX_FUSED_GROUPS * sizeof(int)) != 0) { rp_hip_free(p); return nullptr; }      // a fill kernel on the current stream
-    blocks[dev] = (int*)p;
-    return blocks[dev];
-}
-
-static bool two_launch_forced() {            // RP_HIP_SKINNY_TWO_LAUNCH=1: finish with the separate combine kernel
-    static int v = -1;
-    if (v < 0) { const char* e = getenv("RP_HIP_SKINNY_TWO_LAUNCH"); v = (e && e[0] == '1') ? 1 : 0; }
-    return v == 1;
-}
-
 static int launch_stream16(const GemmArgs& g, int dtype) {
     const int groups = (g.n + SS_COLS - 1) / SS_COLS;
     constexpr int QUANTUM = SS_WAVES * SS_ROUND;             // k rows one pass of a block's waves covers
@@ -258,9 +229,10 @@ static int launch_stream16(const GemmArgs& g, int dtype) {
     void* ws = nullptr;
     if (nsplit > 1 && rp_hip_malloc(&ws, part_bytes) != 0) return -1;
     int* arrivals = nullptr;
-    if (nsplit > 1 && groups <= SS_MAX_FUSED_GROUPS && part_bytes < (1ull << 31) && !two_launch_forced()) {
-        arrivals = arrival_counters();
-        if (!arrivals) { rp_hip_free(ws); return -1; }
+    if (nsplit > 1) {
+        bool failed = false;
+        arrivals = splitk_arrival_counters(groups, part_bytes, &failed);
+        if (failed) { rp_hip_free(ws); return -1; }
     }
     int rc;
     if (dtype == RP_DTYPE_BFLOAT16) rc = launch_stream16_t<bf16_t>(g, (float*)ws, nsplit, k_per_split, arrivals);
