@@ -174,13 +174,14 @@ def skinny_times(capi, quick_reps=20, rows=(1, 8, 32)):
     return out
 
 
-def secondary(capi, quick_reps=20):
-    out = skinny_times(capi, quick_reps)
+def wide_times(capi, cases=(("gemm_f32_4096", "f32", 4096), ("gemm_f64_2048", "f64", 2048))):
+    """Config 3's fp32 GEMM at 4096 and config 5b's fp64 GEMM at 2048 (square, row-major, N(0,1))."""
+    out = {}
     rng = np.random.default_rng(5)
-    # config 3: fp32 at 4096; config 5b: fp64 at 2048
-    for name, dt, npdt, size, peak in (("gemm_f32_4096", capi.F32, np.float32, 4096, PEAK_TFLOPS["f32"]),
-                                       ("gemm_f64_2048", capi.F64, np.float64, 2048, PEAK_TFLOPS["f64"])):
-        a = rng.standard_normal((size, size)).astype(npdt); b = rng.standard_normal((size, size)).astype(npdt)
+    for name, which, size in cases:
+        dt, npdt, peak = (capi.F32, np.float32, PEAK_TFLOPS["f32"]) if which == "f32" else (capi.F64, np.float64, PEAK_TFLOPS["f64"])
+        draw = (lambda: rng.standard_normal((size, size))) if which == "f32" else (lambda: rng.uniform(-1.0, 1.0, (size, size)))     # as the configurations say
+        a = draw().astype(npdt); b = draw().astype(npdt)
         d_a, d_b = capi.DeviceBuffer.from_numpy(a), capi.DeviceBuffer.from_numpy(b)
         d_c = capi.DeviceBuffer(a.nbytes)
         s = (0, size, 1)
@@ -188,6 +189,12 @@ def secondary(capi, quick_reps=20):
         ms = _time_launches(capi, fn, 10, 3)
         tf = 2.0 * size ** 3 / (ms * 1e-3) / 1e12
         out[name] = {"ms": ms, "TFLOP/s": tf, "frac_mfma": tf / peak}
+    return out
+
+
+def secondary(capi, quick_reps=20):
+    out = skinny_times(capi, quick_reps)
+    out.update(wide_times(capi))
     # config 4: attention-shaped batched GEMMs on stride views
     out["attention_bf16"] = attention_times(capi, "bf16")
     out["attention_f32"] = attention_times(capi, "f32")
@@ -293,6 +300,8 @@ def main():
                          "power-managed shader clock, and with it the throughput, depends on the values multiplied")
     ap.add_argument("--skinny-only", action="store_true",
                     help="run only the few-row bf16 GEMMs of configuration 5a and print their figures (for profiling that kernel alone)")
+    ap.add_argument("--wide-only", action="store_true",
+                    help="run only the fp32 (4096) and fp64 (2048, 4096) square GEMMs and print their figures (for profiling those kernels alone)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain copy kernel of known size (256 MiB in, 256 MiB out), the yardstick for FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
@@ -316,6 +325,9 @@ def main():
         src.free(); dst.free()
     if args.skinny_only:
         print(json.dumps({"skinny": skinny_times(capi, rows=(1, 8))}))
+        return
+    if args.wide_only:
+        print(json.dumps({"wide": wide_times(capi, (("gemm_f32_4096", "f32", 4096), ("gemm_f64_2048", "f64", 2048), ("gemm_f64_4096", "f64", 4096)))}))
         return
     h = headline(capi, args.steps, args.warmup, data=args.data)
     a, b = h.pop("operands")

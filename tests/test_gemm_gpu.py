@@ -231,6 +231,22 @@ def test_streaming_rows_single_launch_finish(m):
     assert np.array_equal(device_gemm(a, b, BF16), oracle_gemm(a, b, BF16))
 
 
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_ragged_small_outputs_deep_k(dt):
+    """Outputs that no vector kernel takes (n = 10, odd strides) with a deep k: the generic kernel splits k across
+    blocks and a scalar kernel adds the partials in split order, so results repeat bit for bit.  fp64 does not split."""
+    rng = np.random.default_rng(40)
+    for m, k, n, layout in [(128, 256, 10, "tn"), (256, 128, 10, "nn"), (17, 1000, 3, "nn"), (70, 333, 65, "nt"), (10, 96, 130, "tt")]:
+        a, b = _operands(rng, m, k, n, dt, layout)
+        es = a.itemsize
+        if dt != F64:              # 2-element vectors fit some of these shapes, which then take the fp64 MFMA kernel
+            assert capi.gemm_kernel_name(1, m, k, n, (a.strides[0] // es, a.strides[1] // es), (b.strides[0] // es, b.strides[1] // es), (n, 1), dt) == "generic"
+        bias = rand_storage(rng, (n,), dt); c0 = rand_storage(rng, (m, n), dt)
+        got = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)
+        _check(got, a, b, dt, k, bias=bias, c_init=c0, accumulate=True)
+        assert np.array_equal(got, device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True))
+
+
 def test_large_tile_kernel_multi_slab():
     """4096 x 4096 outputs select the 256x256 tile; checked against float64 everywhere and the oracle on a row slab."""
     rng = np.random.default_rng(37)
