@@ -55,23 +55,24 @@ __device__ __forceinline__ uint16_t narrow_bf16_bits(float f) {
     return (uint16_t)((w >> 16) + ((w >> 15) & 1u));
 }
 
-// fp32 -> fp16 with the same "add the first dropped bit" rule, including the
-// subnormal and overflow branches (reference core/half_precision.h:50-83).
+// fp32 -> fp16 with the same "add the first dropped bit" rule, including the subnormal and overflow branches
+// (reference core/half_precision.h:50-83).  Adding the first dropped bit and truncating is truncating
+// |x| + half an fp16 ulp: the half ulp is 2^(E-11) for an fp16-normal result and 2^-25 below that, the sum is
+// exact in fp32 up to a carry that cannot reach the truncation point, and the hardware's round-toward-zero
+// conversion does the truncation, subnormal results included.  Sums of 65536 or more are the reference's
+// infinity; inputs below 2^-25 are its signed zero; Inf and NaN inputs take its bit formula.
 __device__ __forceinline__ uint16_t narrow_f16_bits(float x) {
-    uint32_t w = __float_as_uint(x);
-    uint32_t s = (w >> 16) & 0x8000u;
-    uint32_t e32 = (w >> 23) & 0xFFu;
-    uint32_t f = w & 0x7FFFFFu;
-    int e = (int)e32 - 112;
-    if (e32 == 0xFFu) return (uint16_t)(f ? (s | 0x7C00u | (f >> 13) | 1u) : (s | 0x7C00u));
-    if (e <= 0) {
-        if (e < -10) return (uint16_t)s;
-        f |= 0x800000u;
-        int sh = 14 - e;
-        return (uint16_t)((s | (f >> sh)) + ((f >> (sh - 1)) & 1u));
-    }
-    if (e >= 0x1F) return (uint16_t)(s | 0x7C00u);
-    return (uint16_t)((s | ((uint32_t)e << 10) | (f >> 13)) + ((f >> 12) & 1u));
+    const uint32_t w = __float_as_uint(x);
+    const uint32_t s = (w >> 16) & 0x8000u;
+    const int e32 = (int)((w >> 23) & 0xFFu);
+    const int eh = e32 - 11 > 102 ? e32 - 11 : 102;                               // biased exponent of the half ulp
+    const float sum = x + __uint_as_float((w & 0x80000000u) | ((uint32_t)eh << 23));
+    uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(sum, 0.f)) & 0xFFFFu;
+    // branch-free selects for the three rare cases
+    bits = e32 < 102 ? s : bits;                                                  // below 2^-25: the sum above may round up to 2^-24
+    bits = __builtin_fabsf(sum) >= 65536.f ? (s | 0x7C00u) : bits;                // overflow and infinities
+    bits = x != x ? (s | 0x7C01u | ((w >> 13) & 0x3FFu)) : bits;                  // NaN keeps its top payload bits, never becomes Inf
+    return (uint16_t)bits;
 }
 
 template <typename T> __device__ __forceinline__ T narrow(typename traits<T>::acc v);

@@ -374,7 +374,7 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
                 for (int e = 0; e < 8; e++) out[e] = finish<T>(vals[e], has_bias, bv[e], accum, accum ? old[e] : T{});
                 uint4 o;
                 memcpy(&o, out, 16);
-                *(uint4*)(crow + gn) = o;
+                __builtin_nontemporal_store(__builtin_bit_cast(u32x4_t, o), (u32x4_t*)(crow + gn));      // written once, never re-read: keep it out of the way of the operand panels in L2
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; e++) {

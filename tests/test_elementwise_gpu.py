@@ -207,3 +207,26 @@ def test_graph_replay_matches_eager():
             got = (dr.numpy(), dg.numpy(), dy.numpy(), dz.numpy())
             for g_, w_ in zip(got, want):
                 assert np.array_equal(g_, w_)
+
+
+def test_narrowing_to_fp16_every_exponent_and_rounding_case():
+    """fp32 -> fp16 on the device against the oracle, bit for bit: every sign and exponent with mantissas that sit
+    on, just below and just above every rounding boundary (ties, carries into the next binade, the subnormal range,
+    the overflow threshold), random mantissas, infinities and NaNs with payloads."""
+    rng = np.random.default_rng(48)
+    exps = np.arange(256, dtype=np.uint32)
+    edge = []
+    for sh in range(0, 24):                       # a dropped-bit position for every subnormal shift and the normal one
+        bit = np.uint32(1) << np.uint32(sh)
+        for m in (bit - 1, bit, bit + 1, (bit << 1) - 1 if sh < 23 else bit, 0x7FFFFF & ~(bit - 1), 0x7FFFFF, 0x7FFFFF - bit + 1):
+            edge.append(np.uint32(m) & np.uint32(0x7FFFFF))
+    mant = np.unique(np.concatenate([np.array(edge, dtype=np.uint32), np.array([0, 1, 0x1000, 0x0FFF, 0x1001, 0x1FFF, 0x2000, 0x3000, 0x7FE000, 0x7FF000, 0x7FEFFF], dtype=np.uint32),
+                                     rng.integers(0, 1 << 23, 3000, dtype=np.uint32)]))
+    w = (exps[:, None] << np.uint32(23)) | mant[None, :]
+    w = np.concatenate([w.ravel(), w.ravel() | np.uint32(0x80000000)])
+    x = w.view(np.float32)
+    dx, do = Dev(x, F32), Dev.empty(x.shape, F16)
+    capi.check(L().rp_hip_convert(do.ptr, F16, dx.ptr, F32, x.size), "convert")
+    got, want = do.numpy(), oracle.narrow(x, F16)
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, [(hex(int(w[i])), hex(int(got[i])), hex(int(want[i]))) for i in bad[:8]]
