@@ -282,10 +282,26 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
             static_for<(NR * q) / NMFMA, (NR * (q + 1)) / NMFMA>([&](auto rc) {
                 read_item(rd_stage, rksc, std::integral_constant<int, MSLOT ^ 1>{}, rc);
             });
-            static_for<P0 + (NP * q) / NMFMA, P0 + (NP * (q + 1)) / NMFMA>([&](auto pc) {
-                if constexpr (WR) store_piece(wr_stage, pc);
-                if constexpr (LD) load_piece(pc);
-            });
+            if constexpr (NMFMA >= 4) {
+                // a piece's LDS store and the global load that refills its register go to neighbouring micro-steps,
+                // so no MFMA has both (and a fragment read) to wait behind
+                constexpr int D = NMFMA - 1;
+                if constexpr (q < D) {
+                    static_for<P0 + (NP * q) / D, P0 + (NP * (q + 1)) / D>([&](auto pc) {
+                        if constexpr (WR) store_piece(wr_stage, pc);
+                    });
+                }
+                if constexpr (q > 0) {
+                    static_for<P0 + (NP * (q - 1)) / D, P0 + (NP * q) / D>([&](auto pc) {
+                        if constexpr (LD) load_piece(pc);
+                    });
+                }
+            } else {
+                static_for<P0 + (NP * q) / NMFMA, P0 + (NP * (q + 1)) / NMFMA>([&](auto pc) {
+                    if constexpr (WR) store_piece(wr_stage, pc);
+                    if constexpr (LD) load_piece(pc);
+                });
+            }
             __builtin_amdgcn_sched_barrier(0);
         });
     };
