@@ -200,6 +200,7 @@ def secondary(capi, quick_reps=20):
     out["attention_f32"] = attention_times(capi, "f32")
     # config 2: fp32 MLP 784-256-128-10, batch 256, forward + backward through the C ABI (9 GEMMs + neighbours)
     out["mlp_f32_step"] = mlp_step_time(capi)
+    out["mlp_f32_step"]["ms_through_python_api"] = mlp_step_time_dropin()
     return out
 
 
@@ -285,7 +286,49 @@ def mlp_step_time(capi, reps=50):
     ms_graph = _time_graph(capi, step, 10, 2)
     return {"ms": ms_graph, "ms_eager_from_python": ms, "launches": 18, "note": "9 GEMMs (bias fused into the 3 forward ones), 2 relu, 2 relu-backward, "
             "cross-entropy fwd+bwd, 3 bias-gradient reductions; `ms` replays the step from a HIP graph, "
-            "`ms_eager_from_python` launches it call by call through ctypes"}
+            "`ms_eager_from_python` launches it call by call through ctypes, `ms_through_python_api` is the same step through "
+            "the drop-in recpulse_cuda tensors, recpulse.module.Linear and autograd (wall clock, allocation and graph bookkeeping included)"}
+
+
+def mlp_step_time_dropin(reps=200, warmup=20):
+    """Config 2 end to end through the drop-in Python API (recpulse_cuda tensors, recpulse.module.Linear, autograd):
+    forward, mean cross-entropy, backward, zero_grad.  Wall-clock per step with one synchronising read at the end."""
+    sys.path.insert(0, os.path.join(ROOT, "recpulse_amd", "dropin"))
+    import recpulse_cuda as rp
+    from recpulse.module import Linear, Module
+
+    class MLP(Module):
+        def __init__(self):
+            super().__init__()
+            self.fc1, self.fc2, self.fc3 = Linear(784, 256), Linear(256, 128), Linear(128, 10)
+
+        def forward(self, x):
+            return self.fc3(self.fc2(self.fc1(x).op_relu()).op_relu())
+
+    rng = np.random.default_rng(1)
+    rp.manual_seed(1)
+    net = MLP().to(device="cuda")
+    x = rp.from_numpy(rng.uniform(0, 1, (256, 784)).astype(np.float32)).to(device="cuda").requires_grad_(True)
+    y = rng.integers(0, 10, 256).tolist()
+    params = list(net.learnable().values())
+
+    def step():
+        loss = net(x).op_cross_entropy_loss(y)
+        loss.backward()
+        return loss
+
+    for _ in range(warmup):
+        loss = step()
+        for p in params + [x]:
+            p.zero_grad()
+    loss.sum_all()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        loss = step()
+        for p in params + [x]:
+            p.zero_grad()
+    loss.sum_all()                      # device -> host read: everything before it has finished
+    return (time.perf_counter() - t0) / reps * 1e3
 
 
 def main():

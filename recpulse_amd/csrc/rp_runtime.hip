@@ -56,6 +56,12 @@ static size_t round_size(size_t bytes) {
     return (bytes + ((1u << 21) - 1)) & ~(size_t)((1u << 21) - 1);         // 2 MiB steps above
 }
 
+struct SmallPayload { uint32_t w[512]; };            // 2 KiB, passed by value in the kernel arguments
+__global__ void upload_small_kernel(uint32_t* dst, SmallPayload payload, int nwords) {
+    int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < nwords) dst[i] = payload.w[i];
+}
+
 // Byte fill: a 16-byte aligned body written as uint4 plus scalar head and tail.
 __global__ void fill_bytes_kernel(unsigned char* p, unsigned char v, size_t bytes) {
     size_t head = (16 - ((uintptr_t)p & 15)) & 15;
@@ -171,9 +177,21 @@ int rp_hip_memset(void* ptr, int value, size_t bytes) {
 
 // Host copies block until the data has landed, like the reference's cudaMemcpy
 // calls (core/tensor_device.cu:295-531); device-to-device copies are stream-ordered.
+// Exception: a host-to-device copy of at most 2 KiB of whole words travels inside a
+// kernel's arguments.  The source is read before the call returns and the data is
+// in place for everything that follows on the stream, which is all a caller of
+// cudaMemcpy can observe, but the host does not wait for the stream to drain (class
+// targets uploaded between a forward and a backward pass would otherwise stall both).
 int rp_hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
     if (!bytes) return 0;
     if (!dst || !src) { set_error("rp_hip_memcpy_h2d: null pointer"); return -1; }
+    if (bytes <= sizeof(rp::SmallPayload) && bytes % 4 == 0 && ((uintptr_t)dst & 3) == 0) {
+        rp::SmallPayload payload;
+        memcpy(payload.w, src, bytes);
+        const int nwords = (int)(bytes / 4);
+        hipLaunchKernelGGL(rp::upload_small_kernel, dim3((nwords + 255) / 256), dim3(256), 0, current_stream(), (uint32_t*)dst, payload, nwords);
+        return check_launch("upload_small_kernel") ? 0 : -1;
+    }
     if (!check_hip(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, current_stream()), "hipMemcpy H2D")) return -1;
     return check_hip(hipStreamSynchronize(current_stream()), "hipStreamSynchronize") ? 0 : -1;
 }
