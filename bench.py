@@ -192,8 +192,23 @@ def wide_times(capi, cases=(("gemm_f32_4096", "f32", 4096), ("gemm_f64_2048", "f
     return out
 
 
+def f16_time(capi, n=8192):
+    """Config 3 in fp16 at N = 8192: the forward GEMM (fp32 accumulate, fp16 output), N(0,1) operands."""
+    rng = np.random.default_rng(2)
+    a = rng.standard_normal((n, n)).astype(np.float16).view(np.uint16); b = rng.standard_normal((n, n)).astype(np.float16).view(np.uint16)
+    d_a, d_b = capi.DeviceBuffer.from_numpy(a), capi.DeviceBuffer.from_numpy(b)
+    d_c = capi.DeviceBuffer(a.nbytes)
+    s = (0, n, 1)
+    ms = _time_launches(capi, lambda: capi.gemm(d_c.ptr, d_a.ptr, d_b.ptr, None, 1, n, n, n, s, s, s, False, capi.F16), 10, 5)
+    tf = 2.0 * n ** 3 / (ms * 1e-3) / 1e12
+    for d in (d_a, d_b, d_c):
+        d.free()
+    return {"ms": ms, "TFLOP/s": tf, "frac_mfma": tf / PEAK_TFLOPS["f16"]}
+
+
 def secondary(capi, quick_reps=20):
     out = skinny_times(capi, quick_reps)
+    out["gemm_f16_8192"] = f16_time(capi)
     out.update(wide_times(capi))
     # config 4: attention-shaped batched GEMMs on stride views
     out["attention_bf16"] = attention_times(capi, "bf16")

@@ -59,20 +59,20 @@ __device__ __forceinline__ uint16_t narrow_bf16_bits(float f) {
 // (reference core/half_precision.h:50-83).  Adding the first dropped bit and truncating is truncating
 // |x| + half an fp16 ulp: the half ulp is 2^(E-11) for an fp16-normal result and 2^-25 below that, the sum is
 // exact in fp32 up to a carry that cannot reach the truncation point, and the hardware's round-toward-zero
-// conversion does the truncation, subnormal results included.  Sums of 65536 or more are the reference's
-// infinity; inputs below 2^-25 are its signed zero; Inf and NaN inputs take its bit formula.
+// conversion does the truncation, subnormal results included.  Magnitudes below 2^-25 are the reference's zero
+// (their sum could round up to 2^-24, so they are cleared first); sums of 65536 or more, infinities included,
+// are its infinity; a NaN stays a NaN (the hardware's quiet NaN; the reference keeps the top payload bits).
+// Straight-line code on the magnitude, the sign is put back at the end.
 __device__ __forceinline__ uint16_t narrow_f16_bits(float x) {
     const uint32_t w = __float_as_uint(x);
-    const uint32_t s = (w >> 16) & 0x8000u;
-    const int e32 = (int)((w >> 23) & 0xFFu);
-    const int eh = e32 - 11 > 102 ? e32 - 11 : 102;                               // biased exponent of the half ulp
-    const float sum = x + __uint_as_float((w & 0x80000000u) | ((uint32_t)eh << 23));
-    uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(sum, 0.f)) & 0xFFFFu;
-    // branch-free selects for the three rare cases
-    bits = e32 < 102 ? s : bits;                                                  // below 2^-25: the sum above may round up to 2^-24
-    bits = __builtin_fabsf(sum) >= 65536.f ? (s | 0x7C00u) : bits;                // overflow and infinities
-    bits = x != x ? (s | 0x7C01u | ((w >> 13) & 0x3FFu)) : bits;                  // NaN keeps its top payload bits, never becomes Inf
-    return (uint16_t)bits;
+    uint32_t a = w & 0x7FFFFFFFu;
+    a = a < 0x33000000u ? 0u : a;                                                  // below 2^-25
+    const uint32_t he = (a & 0x7F800000u) - (11u << 23);                           // exponent field of 2^(E-11); wraps for tiny a,
+    const uint32_t hb = (int32_t)he > (int32_t)(102u << 23) ? he : (102u << 23);   // which the signed maximum with 2^-25 absorbs
+    const float sum = __uint_as_float(a) + __uint_as_float(hb);
+    uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(sum, 0.f));     // upper half: +0
+    bits = sum >= 65536.f ? 0x7C00u : bits;
+    return (uint16_t)(bits | ((w >> 16) & 0x8000u));
 }
 
 template <typename T> __device__ __forceinline__ T narrow(typename traits<T>::acc v);

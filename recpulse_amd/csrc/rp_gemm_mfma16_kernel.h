@@ -30,8 +30,8 @@ namespace rp {
 //               reads with ds_read_b128 land in 16 different 16-byte bank groups
 //   MC operand: [64][cols + 32]  row pitch 2*cols + 64 B -> the 4 k-rows a
 //               16-lane group reads with ds_read_b64_tr_b16 start 16 banks apart
-// The epilogue stages fp32 accumulators through the (now idle) LDS so that each
-// lane narrows and stores 8 adjacent columns with one 16-byte store.
+// The epilogue narrows the accumulators, stages them through the (now idle) LDS
+// and stores 8 adjacent columns per lane with one 16-byte store.
 // ============================================================================
 template <typename T> struct mfma16_ops;
 template <> struct mfma16_ops<bf16_t> {
@@ -53,7 +53,9 @@ __host__ __device__ constexpr int m16_tile_elems(int rows, bool mc) {
 __host__ __device__ constexpr int m16_epi_cols(int wn) { return wn >= 64 ? 64 : wn; }      // columns staged per epilogue pass
 __host__ __device__ constexpr size_t m16_smem_bytes(int bm, int bn, int wgm, bool a_mc, bool b_mc) {
     size_t loop = 2 * (size_t)(m16_tile_elems(bm, a_mc) + m16_tile_elems(bn, b_mc)) * 2;
-    size_t epi = 4 * (size_t)(bm / wgm) * (m16_epi_cols(bn / (4 / wgm)) + 4) * 4;
+    size_t epi = 4 * (size_t)(bm / wgm) * (m16_epi_cols(bn / (4 / wgm)) + 4) * 4;      // split-k: fp32, 64 columns per pass
+    size_t epi16 = 4 * (size_t)(bm / wgm) * (bn / (4 / wgm) + 8) * 2;                  // otherwise: the whole patch as 16-bit values
+    if (epi16 > epi) epi = epi16;
     return loop > epi ? loop : epi;
 }
 
@@ -338,66 +340,99 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     slab_step(s, no{}, no{});
 
     // ---- epilogue ----
-    // Pass p covers CN columns of every wave's patch: accumulators go to the wave's private fp32 LDS region
-    // [WM][CN + 4]; then each lane takes 8 adjacent columns of one row per step: narrow, bias, accumulate, one store.
-    constexpr int CN = m16_epi_cols(WN), EP = CN + 4, TJ = CN / 32, PASSES = WN / CN;
-    constexpr int LPR = CN / 8;                 // lanes per row
-    constexpr int RPS = 64 / LPR;               // rows per step
-    float* region = (float*)smem + wave * (WM * EP);
     T* C = (T*)g.C + (long long)z * g.c_bs;
     const T* bias = (const T*)g.bias;
     const bool has_bias = bias != nullptr, accum = g.accumulate != 0;
-    const bool c_vec = (g.c_cs == 1) && (g.c_rs % 8 == 0) && (((uintptr_t)C & 15) == 0);
-    const int ecol = (lane % LPR) * 8, erow = lane / LPR;
+    if constexpr (!SPLITK) {
+        // Each lane narrows its accumulators (and adds the bias of its column) first, then the wave's whole patch
+        // goes through its private LDS region as 16-bit values, so that every lane stores 8 adjacent columns of one
+        // output row with one 16-byte store and the read side has no arithmetic left unless C is accumulated into.
+        constexpr int EP = WN + 8;                       // 16-bit elements per staged row (16-byte aligned pitch)
+        constexpr int LPR = WN / 8, RPS = 64 / LPR;      // lanes per row, rows per step
+        uint16_t* region = smem + wave * (WM * EP);
+        const bool c_vec = (g.c_cs == 1) && (g.c_rs % 8 == 0) && (((uintptr_t)C & 15) == 0);
+        __syncthreads();                                 // every wave is done with the main loop's LDS
 #pragma unroll
-    for (int p = 0; p < PASSES; p++) {
-        __syncthreads();                        // main loop (or the previous pass) is done with LDS
+        for (int j = 0; j < TNI; j++) {
+            const int col = j * 32 + (lane & 31), gnl = n0 + wn0 + col;
+            const float bcol = (has_bias && (!EDGE || gnl < g.n)) ? widen(bias[gnl]) : 0.f;
+            auto stage = [&](auto with_bias) {
 #pragma unroll
-        for (int i = 0; i < TMI; i++)
+                for (int i = 0; i < TMI; i++)
 #pragma unroll
-            for (int jj = 0; jj < TJ; jj++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    int row = i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-                    region[row * EP + jj * 32 + (lane & 31)] = acc[i][p * TJ + jj][v];
-                }
+                    for (int v = 0; v < 16; v++) {
+                        const int row = i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                        T y = narrow<T>(acc[i][j][v]);
+                        if constexpr (decltype(with_bias)::value) y = narrow<T>(widen(y) + bcol);
+                        region[row * EP + col] = y.bits;
+                    }
+            };
+            if (has_bias) stage(std::true_type{});
+            else stage(std::false_type{});
+        }
         __syncthreads();
-        const int gn = n0 + wn0 + p * CN + ecol;
-        T bv[8];
-#pragma unroll
-        for (int e = 0; e < 8; e++) bv[e] = (has_bias && (!EDGE || gn + e < g.n)) ? bias[gn + e] : T{};
-#pragma unroll 2
+        const int ecol = (lane % LPR) * 8, erow = lane / LPR;
+        const int gn = n0 + wn0 + ecol;
+#pragma unroll 4
         for (int r = erow; r < WM; r += RPS) {
             const int gm = m0 + wm0 + r;
             if (EDGE && gm >= g.m) break;
-            f32x4_t lo = *(const f32x4_t*)(region + r * EP + ecol);
-            f32x4_t hi = *(const f32x4_t*)(region + r * EP + ecol + 4);
-            float vals[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            if constexpr (SPLITK) {
-                // fp32 partial tile [split][m][n]; n is a multiple of 8 on this path, so the 8 columns are all in or all out
-                if (!EDGE || gn + 8 <= g.n) {
-                    float* prow = partials + ((long long)blockIdx.z * g.m + gm) * g.n + gn;
-                    *(f32x4_t*)prow = lo;
-                    *(f32x4_t*)(prow + 4) = hi;
-                }
-                continue;
-            }
+            const u32x4_t staged = *(const u32x4_t*)(region + r * EP + ecol);
             T* crow = C + (long long)gm * g.c_rs;
             if (c_vec && (!EDGE || gn + 8 <= g.n)) {
-                T out[8], old[8];
-                if (accum) { uint4 o = *(const uint4*)(crow + gn); memcpy(old, &o, 16); }
+                u32x4_t o = staged;
+                if (accum) {
+                    T y[8], old[8], out[8];
+                    const u32x4_t was = *(const u32x4_t*)(crow + gn);
+                    memcpy(y, &staged, 16);
+                    memcpy(old, &was, 16);
 #pragma unroll
-                for (int e = 0; e < 8; e++) out[e] = finish<T>(vals[e], has_bias, bv[e], accum, accum ? old[e] : T{});
-                uint4 o;
-                memcpy(&o, out, 16);
-                __builtin_nontemporal_store(__builtin_bit_cast(u32x4_t, o), (u32x4_t*)(crow + gn));      // written once, never re-read: keep it out of the way of the operand panels in L2
+                    for (int e = 0; e < 8; e++) out[e] = narrow<T>(widen(old[e]) + widen(y[e]));
+                    memcpy(&o, out, 16);
+                }
+                __builtin_nontemporal_store(o, (u32x4_t*)(crow + gn));      // written once, never re-read: keep it out of the way of the operand panels in L2
             } else {
+                T y[8];
+                memcpy(y, &staged, 16);
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     if (EDGE && gn + e >= g.n) break;
                     T* pc = crow + (long long)(gn + e) * g.c_cs;
-                    T old = accum ? *pc : T{};
-                    *pc = finish<T>(vals[e], has_bias, bv[e], accum, old);
+                    *pc = accum ? narrow<T>(widen(*pc) + widen(y[e])) : y[e];
+                }
+            }
+        }
+    } else {
+        // Split-k: fp32 partial tiles [split][m][n].  Pass p covers CN columns of every wave's patch: accumulators go
+        // to the wave's private fp32 LDS region [WM][CN + 4]; then each lane stores 8 adjacent columns of one row.
+        constexpr int CN = m16_epi_cols(WN), EP = CN + 4, TJ = CN / 32, PASSES = WN / CN;
+        constexpr int LPR = CN / 8;                 // lanes per row
+        constexpr int RPS = 64 / LPR;               // rows per step
+        float* region = (float*)smem + wave * (WM * EP);
+        const int ecol = (lane % LPR) * 8, erow = lane / LPR;
+#pragma unroll
+        for (int p = 0; p < PASSES; p++) {
+            __syncthreads();                        // main loop (or the previous pass) is done with LDS
+#pragma unroll
+            for (int i = 0; i < TMI; i++)
+#pragma unroll
+                for (int jj = 0; jj < TJ; jj++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        int row = i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                        region[row * EP + jj * 32 + (lane & 31)] = acc[i][p * TJ + jj][v];
+                    }
+            __syncthreads();
+            const int gn = n0 + wn0 + p * CN + ecol;
+#pragma unroll 2
+            for (int r = erow; r < WM; r += RPS) {
+                const int gm = m0 + wm0 + r;
+                if (EDGE && gm >= g.m) break;
+                // n is a multiple of 8 on this path, so the 8 columns are all in or all out
+                if (!EDGE || gn + 8 <= g.n) {
+                    float* prow = partials + ((long long)blockIdx.z * g.m + gm) * g.n + gn;
+                    *(f32x4_t*)prow = *(const f32x4_t*)(region + r * EP + ecol);
+                    *(f32x4_t*)(prow + 4) = *(const f32x4_t*)(region + r * EP + ecol + 4);
                 }
             }
         }
