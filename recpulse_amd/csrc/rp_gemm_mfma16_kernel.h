@@ -51,8 +51,10 @@ __host__ __device__ constexpr int m16_tile_elems(int rows, bool mc) {
     return mc ? M16_BK * m16_mc_pitch(rows) : rows * M16_KC_PITCH;
 }
 __host__ __device__ constexpr int m16_epi_cols(int wn) { return wn >= 64 ? 64 : wn; }      // columns staged per epilogue pass
-__host__ __device__ constexpr size_t m16_smem_bytes(int bm, int bn, int wgm, bool a_mc, bool b_mc) {
-    size_t loop = 2 * (size_t)(m16_tile_elems(bm, a_mc) + m16_tile_elems(bn, b_mc)) * 2;
+// `stages` is 2, or 1 when k fits a single slab (the loop then never touches the second stage), which lets twice
+// as many blocks of a short-k batched GEMM share a CU and overlap their load, multiply and store phases.
+__host__ __device__ constexpr size_t m16_smem_bytes(int bm, int bn, int wgm, bool a_mc, bool b_mc, int stages = 2) {
+    size_t loop = stages * (size_t)(m16_tile_elems(bm, a_mc) + m16_tile_elems(bn, b_mc)) * 2;
     size_t epi = 4 * (size_t)(bm / wgm) * (m16_epi_cols(bn / (4 / wgm)) + 4) * 4;      // split-k: fp32, 64 columns per pass
     size_t epi16 = 4 * (size_t)(bm / wgm) * (bn / (4 / wgm) + 8) * 2;                  // otherwise: the whole patch as 16-bit values
     if (epi16 > epi) epi = epi16;
@@ -444,7 +446,7 @@ template <typename T, int BM, int BN, int WGM, bool A_MC, bool B_MC, bool EDGE, 
 static int m16_launch(const GemmArgs& g, float* partials, int nsplit, int k_per_split) {
     int tiles_m = (g.m + BM - 1) / BM, tiles_n = (g.n + BN - 1) / BN;
     dim3 grid(scheduled_grid(tiles_m, tiles_n), g.batch, SPLITK ? nsplit : 1);
-    size_t smem = m16_smem_bytes(BM, BN, WGM, A_MC, B_MC);
+    size_t smem = m16_smem_bytes(BM, BN, WGM, A_MC, B_MC, (!SPLITK && g.k <= M16_BK) ? 1 : 2);
     auto kern = gemm_mfma16_kernel<T, BM, BN, WGM, A_MC, B_MC, EDGE, SPLITK>;
     if (smem > 64 * 1024 && !check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem), "hipFuncSetAttribute")) return -1;
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, current_stream(), g, tiles_m, tiles_n, partials, k_per_split);
