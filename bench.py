@@ -206,8 +206,34 @@ def f16_time(capi, n=8192):
     return {"ms": ms, "TFLOP/s": tf, "frac_mfma": tf / PEAK_TFLOPS["f16"]}
 
 
+def square_sweep(capi, sizes=(1024, 4096)):
+    """Config 3 below the headline size: C = A.B, dA = dC.Bt, dB = At.dC (transposes as stride views) in bf16 and
+    fp16 at N = 1024 and 4096, each replayed from a HIP graph; microseconds and TFLOP/s."""
+    out = {}
+    rng = np.random.default_rng(2)
+    for n in sizes:
+        for name, dt in (("bf16", capi.BF16), ("f16", capi.F16)):
+            mk = (lambda: _normal_bf16(rng, (n, n))) if dt == capi.BF16 else (lambda: rng.standard_normal((n, n)).astype(np.float16).view(np.uint16))
+            d_a, d_b, d_dc = (capi.DeviceBuffer.from_numpy(mk()) for _ in range(3))
+            d_c = capi.DeviceBuffer(n * n * 2)
+            s, st = (0, n, 1), (0, 1, n)
+            ops = {"fwd": lambda: capi.gemm(d_c.ptr, d_a.ptr, d_b.ptr, None, 1, n, n, n, s, s, s, False, dt),
+                   "dA": lambda: capi.gemm(d_c.ptr, d_dc.ptr, d_b.ptr, None, 1, n, n, n, s, st, s, False, dt),
+                   "dB": lambda: capi.gemm(d_c.ptr, d_a.ptr, d_dc.ptr, None, 1, n, n, n, st, s, s, False, dt)}
+            _time_graph(capi, ops["fwd"], 10, 2)            # clocks up before the first figure
+            row = {}
+            for op, fn in ops.items():
+                ms = _time_graph(capi, fn, 10, 2)
+                row[op] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(2.0 * n ** 3 / ms / 1e9, 1)}
+            out[f"{name}_{n}"] = row
+            for d in (d_a, d_b, d_dc, d_c):
+                d.free()
+    return out
+
+
 def secondary(capi, quick_reps=20):
     out = skinny_times(capi, quick_reps)
+    out["square_sweep"] = square_sweep(capi)
     out["gemm_f16_8192"] = f16_time(capi)
     out.update(wide_times(capi))
     # config 4: attention-shaped batched GEMMs on stride views

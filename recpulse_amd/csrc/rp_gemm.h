@@ -51,11 +51,18 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
 // ----------------------------------------------------------------------------
 struct TileCoord { int tm, tn; bool valid; };
 
-constexpr int SCHED_MIN_TILES = 64;      // below this a launch does not fill the chip and plain row-major order is used
+// The XCD-aware order launches whole rounds of 8 super-tiles (one per XCD): a super-tile count that is neither a
+// multiple of 8 nor large leaves XCDs idle in the last round (with 2 super-tiles only 2 of the 8 XCDs would work,
+// for every matrix of a batch), so those cases use plain row-major order, which deals tiles evenly.
+__host__ __device__ __forceinline__ bool schedule_by_xcd(int tiles_m, int tiles_n) {
+    constexpr int XCDS = 8, GM = 4, GN = 8;
+    int sup = ((tiles_m + GM - 1) / GM) * ((tiles_n + GN - 1) / GN);
+    return sup % XCDS == 0 || sup >= 4 * XCDS;
+}
 
 __device__ __forceinline__ TileCoord schedule_tile(int bid, int tiles_m, int tiles_n) {
     constexpr int XCDS = 8, GM = 4, GN = 8, PER = GM * GN;
-    if (tiles_m * tiles_n < SCHED_MIN_TILES) {
+    if (!schedule_by_xcd(tiles_m, tiles_n)) {
         TileCoord lin;
         lin.tm = bid / tiles_n; lin.tn = bid % tiles_n; lin.valid = bid < tiles_m * tiles_n;
         return lin;
@@ -74,7 +81,7 @@ __device__ __forceinline__ TileCoord schedule_tile(int bid, int tiles_m, int til
 
 static inline int scheduled_grid(int tiles_m, int tiles_n) {
     constexpr int XCDS = 8, GM = 4, GN = 8, PER = GM * GN;
-    if (tiles_m * tiles_n < SCHED_MIN_TILES) return tiles_m * tiles_n;
+    if (!schedule_by_xcd(tiles_m, tiles_n)) return tiles_m * tiles_n;
     int sup = ((tiles_m + GM - 1) / GM) * ((tiles_n + GN - 1) / GN);
     int rounds = (sup + XCDS - 1) / XCDS;
     return rounds * XCDS * PER;
