@@ -142,10 +142,15 @@ def headline(capi, steps, warmup, n=8192, data="normal"):
     }
 
 
-def cpu_baseline(a, b, rows=8):
-    """The oracle's restatement of the reference CPU matmul on a `rows`-row slab of the 8192^3 bf16 GEMM, one core."""
+def cpu_baseline(a, b, target_s=15.0):
+    """The oracle's restatement of the reference CPU matmul on a row slab of the 8192^3 bf16 GEMM, one core.  Two rows
+    are timed first and the slab is sized from them for about `target_s` seconds of CPU work (4 to 256 rows)."""
     import oracle
     n = b.shape[0]
+    t0 = time.perf_counter()
+    oracle.matmul(np.ascontiguousarray(a[:2]), b, oracle.BF16)       # includes widening B to fp32 once, as every call does
+    probe = time.perf_counter() - t0
+    rows = int(min(256, max(4, round(target_s / (probe / 2)))))
     slab = np.ascontiguousarray(a[:rows])
     t0 = time.perf_counter()
     oracle.matmul(slab, b, oracle.BF16)
