@@ -124,9 +124,16 @@ int rp_hip_gemm_strided_batched(void* C, const void* A, const void* B, const voi
         set_error("rp_hip_gemm_strided_batched: negative stride");
         return -1;
     }
-    if (batch > 65535) { set_error("rp_hip_gemm_strided_batched: batch %d exceeds 65535", batch); return -1; }
-    GemmArgs g{C, A, B, bias, batch, m, k, n, a_bs, a_rs, a_cs, b_bs, b_rs, b_cs, c_bs, c_rs, c_cs, accumulate};
-    return run_gemm(g, dtype);
+    // the batch rides on a grid axis that holds at most 65535 blocks: longer batches go in chunks
+    constexpr int MAX_BATCH = 65535;
+    const long long esz = (long long)dtype_size(dtype);
+    for (int b0 = 0; b0 < batch; b0 += MAX_BATCH) {
+        const int nb = batch - b0 < MAX_BATCH ? batch - b0 : MAX_BATCH;
+        GemmArgs g{(char*)C + b0 * c_bs * esz, (const char*)A + b0 * a_bs * esz, (const char*)B + b0 * b_bs * esz, bias,
+                   nb, m, k, n, a_bs, a_rs, a_cs, b_bs, b_rs, b_cs, c_bs, c_rs, c_cs, accumulate};
+        if (run_gemm(g, dtype) != 0) return -1;
+    }
+    return 0;
 }
 
 int matmul_kernel_device(void* C, const void* A, const void* B, int m, int k, int n, int dtype) {

@@ -262,6 +262,20 @@ def test_large_tile_kernel_multi_slab():
         assert oracle.rel_err(oracle.to_f64(got[rows], dt), oracle.to_f64(want, dt)) <= tol(dt, k)
 
 
+def test_batch_longer_than_a_grid_axis():
+    """70 000 tiny matrices in one call (the batch index rides on a grid axis of at most 65 535 blocks), A shared by
+    all of them through a zero batch stride."""
+    rng = np.random.default_rng(41)
+    Z, m, k, n = 70000, 4, 8, 4
+    a = rand_storage(rng, (m, k), F32); b = rand_storage(rng, (Z, k, n), F32)
+    da, db, dc = capi.DeviceBuffer.from_numpy(a), capi.DeviceBuffer.from_numpy(b), capi.DeviceBuffer(Z * m * n * 4)
+    capi.gemm(dc.ptr, da.ptr, db.ptr, None, Z, m, k, n, (0, k, 1), (k * n, n, 1), (m * n, n, 1), False, F32)
+    got = dc.to_numpy(np.float32, (Z, m, n))
+    want = np.einsum("ik,zkj->zij", a.astype(np.float64), b.astype(np.float64))
+    assert oracle.rel_err(got.astype(np.float64), want) <= 1e-6
+    assert oracle.rel_err(got[69999].astype(np.float64), oracle.matmul(a, np.ascontiguousarray(b[69999]), F32).astype(np.float64)) <= tol(F32, k)
+
+
 def test_rejects_bad_arguments():
     lib = capi.lib()
     d = capi.DeviceBuffer(64)
