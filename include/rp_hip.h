@@ -177,6 +177,19 @@ int rp_hip_reduce_rows(void* out, const void* grad, int rows, int cols, int accu
 int rp_hip_cross_entropy_mean(void* loss_out, void* grad_logits, const void* logits, const int* targets,
                               int batch, int classes, double upstream, int dtype);
 
+/* Fused attention forward for bfloat16 / float16: O[b] = softmax(scale * Q[b] * K[b]^T) * V[b], the score matrix never
+ * leaves the chip.  Q, O: [batch, sq, d]; K, V: [batch, sk, d]; d in {32, 64, 128} and contiguous (unit stride);
+ * *_bs / *_rs are the batch and row strides in elements (multiples of 8; operands 16-byte aligned).
+ * lse (may be NULL): float32 [batch, sq], log of the row sums of exp(scale * scores), for a backward pass.
+ * No counterpart in the reference, which composes the same value from op_matmul, op_mul_scalar, op_softmax and
+ * op_matmul (ops/ops.c:6816-6884, 6022-6086, 5721-5788) and rounds the scores to the tensor dtype on the way;
+ * here only the probabilities are rounded (as the reference's P is), accumulation is float32. */
+int rp_hip_attention_forward(void* O, const void* Q, const void* K, const void* V, float* lse,
+                             int batch, int sq, int sk, int d,
+                             long long q_bs, long long q_rs, long long k_bs, long long k_rs,
+                             long long v_bs, long long v_rs, long long o_bs, long long o_rs,
+                             double scale, int dtype);
+
 #ifdef __cplusplus
 }
 #endif

@@ -67,6 +67,7 @@ SIGNATURES = {
     "rp_hip_convert": (_i, [_vp, _i, _vp, _i, _sz]),
     "rp_hip_reduce_rows": (_i, [_vp, _vp, _i, _i, _i, _i]),
     "rp_hip_cross_entropy_mean": (_i, [_vp, _vp, _vp, _vp, _i, _i, _d, _i]),
+    "rp_hip_attention_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i] + [_ll] * 8 + [_d, _i]),
 }
 
 _lib = None

@@ -1,0 +1,76 @@
+"""Fused attention forward (rp_hip_attention_forward) against a float64 oracle and the reference's op chain."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import oracle
+from recpulse_amd import capi
+from devhelp import BF16, F16, NAMES, Dev, rand_storage
+
+pytestmark = pytest.mark.gpu
+
+
+def _fused(q, k, v, dt, scale, q_view=None, want_lse=False):
+    """q, k, v: storage arrays [Z, S, D] (dense).  Returns O (and the log-sum-exp rows)."""
+    Z, sq, d = q.shape
+    sk = k.shape[1]
+    dq, dk, dv = Dev(q, dt), Dev(k, dt), Dev(v, dt)
+    do = Dev.empty((Z, sq, d), dt)
+    lse = capi.DeviceBuffer(Z * sq * 4) if want_lse else None
+    rc = capi.lib().rp_hip_attention_forward(do.ptr, dq.ptr, dk.ptr, dv.ptr, lse.ptr if lse else None, Z, sq, sk, d,
+                                             sq * d, d, sk * d, d, sk * d, d, sq * d, d, float(scale), dt)
+    capi.check(rc, "rp_hip_attention_forward")
+    out = do.numpy()
+    return (out, lse.to_numpy(np.float32, (Z, sq))) if want_lse else out
+
+
+def _f64(q, k, v, dt, scale):
+    q64, k64, v64 = (oracle.to_f64(x, dt) for x in (q, k, v))
+    s = np.einsum("zqd,zkd->zqk", q64, k64) * scale
+    m = s.max(-1, keepdims=True)
+    e = np.exp(s - m)
+    l = e.sum(-1, keepdims=True)
+    return np.einsum("zqk,zkd->zqd", e / l, v64), (m + np.log(l))[..., 0]
+
+
+@pytest.mark.parametrize("dt", [BF16, F16], ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("shape", [(6, 512, 512, 64), (3, 200, 333, 64), (2, 130, 65, 32), (2, 96, 160, 128), (1, 1, 1, 64), (5, 33, 31, 64)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_fused_attention_forward(dt, shape):
+    Z, sq, sk, d = shape
+    rng = np.random.default_rng(60)
+    q, k, v = rand_storage(rng, (Z, sq, d), dt), rand_storage(rng, (Z, sk, d), dt), rand_storage(rng, (Z, sk, d), dt)
+    scale = 1.0 / np.sqrt(d)
+    got, lse = _fused(q, k, v, dt, scale, want_lse=True)
+    want, want_lse = _f64(q, k, v, dt, scale)
+    # probabilities are rounded to the tensor dtype before the second product, as the reference's P is
+    assert oracle.rel_err(oracle.to_f64(got, dt), want) <= (1e-2 if dt == BF16 else 2e-3)
+    assert np.max(np.abs(lse - want_lse)) <= 1e-3 * max(1.0, np.max(np.abs(want_lse)))
+    # the reference's chain (matmul, mul_scalar, softmax, matmul with a rounding after each) on one slice
+    ref = oracle.attention(q[Z - 1], k[Z - 1], v[Z - 1], dt, scale=scale)["O"]
+    assert oracle.rel_err(oracle.to_f64(got[Z - 1], dt), oracle.to_f64(ref, dt)) <= 2e-2
+    # running it again gives the same bits
+    assert np.array_equal(got, _fused(q, k, v, dt, scale))
+
+
+def test_fused_attention_large_scores_and_config4_size():
+    """Scores far from zero (the online softmax must not overflow) at the configuration's full size."""
+    rng = np.random.default_rng(61)
+    Z, S, D = 16 * 12, 512, 64
+    q = oracle.to_storage(rng.normal(0, 4, (Z, S, D)), BF16); k = oracle.to_storage(rng.normal(0, 4, (Z, S, D)), BF16)
+    v = rand_storage(rng, (Z, S, D), BF16)
+    got = _fused(q, k, v, BF16, 0.125)
+    assert np.all(np.isfinite(oracle.to_f64(got, BF16)))
+    sel = [0, 77, Z - 1]
+    want, _ = _f64(q[sel], k[sel], v[sel], BF16, 0.125)
+    assert oracle.rel_err(oracle.to_f64(got[sel], BF16), want) <= 1e-2
+
+
+def test_fused_attention_rejects_bad_arguments():
+    d = capi.DeviceBuffer(4096)
+    L = capi.lib()
+    assert L.rp_hip_attention_forward(d.ptr, d.ptr, d.ptr, d.ptr, None, 1, 4, 4, 48, 192, 48, 192, 48, 192, 48, 192, 48, 1.0, BF16) == -1
+    assert b"head dimension" in L.rp_hip_last_error()
+    assert L.rp_hip_attention_forward(d.ptr, d.ptr, d.ptr, d.ptr, None, 1, 4, 4, 64, 256, 64, 256, 64, 256, 64, 256, 64, 1.0, capi.F32) == -1
+    assert L.rp_hip_attention_forward(d.ptr, d.ptr, d.ptr, d.ptr, None, 1, 4, 4, 64, 256, 60, 256, 64, 256, 64, 256, 64, 1.0, BF16) == -1
