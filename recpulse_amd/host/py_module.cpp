@@ -180,6 +180,8 @@ PYBIND11_MODULE(recpulse_cuda, m) {
         .def("op_linear", [](PyTensor& x, PyTensor& w, py::object bias) {
             return wrap(op_linear(x.t, w.t, bias.is_none() ? nullptr : bias.cast<PyTensor&>().t), "op_linear");
         }, py::arg("weight"), py::arg("bias") = py::none())
+        .def("op_attention", [](PyTensor& q, PyTensor& k, PyTensor& v, double scale) { return wrap(op_attention(q.t, k.t, v.t, scale), "op_attention"); },
+             py::arg("k"), py::arg("v"), py::arg("scale"))
         .def("op_add", [](PyTensor& a, PyTensor& b) { return wrap(op_add(a.t, b.t), "op_add"); })
         .def("op_relu", [](PyTensor& a) { return wrap(op_relu(a.t), "op_relu"); })
         .def("op_softmax", [](PyTensor& a, int dim) { return wrap(op_softmax(a.t, dim), "op_softmax"); }, py::arg("dim") = -1)

@@ -751,6 +751,37 @@ void backward_mul_scalar_fn(GradFn* self, Tensor* grad_output) {     // referenc
     free_tensor(gd);
 }
 
+// Backward of the fused attention: the probabilities are recomputed with the unfused kernels (S = Q·Kᵀ, scale,
+// softmax), then dV = Pᵀ·dO, dP = dO·Vᵀ, dS = softmax'(dP)·scale, dQ = dS·K, dK = dSᵀ·Q — the chain the reference's
+// autograd runs for matmul -> mul_scalar -> softmax -> matmul (ops/ops.c:6759-6814, 5966-6020, 5665-5719), with the
+// transposes as stride views and the gradient accumulation inside the GEMMs.
+void backward_attention_fn(GradFn* self, Tensor* grad_output) {
+    Tensor* q = self->inputs[0]; Tensor* k = self->inputs[1]; Tensor* v = self->inputs[2];
+    if (!needs_grad(q) && !needs_grad(k) && !needs_grad(v)) return;
+    const double scale = ((ScalarSaved*)self->saved_data)->s;
+    const float sf = (float)scale;
+    const int nd = q->ndim, sq = q->shape[nd - 2], sk = k->shape[nd - 2];
+    std::vector<int> sshape(q->shape, q->shape + nd);
+    sshape[nd - 1] = sk;
+    Tensor* g = dense(grad_output);
+    Tensor* qd = dense(q); Tensor* kd = dense(k); Tensor* vd = dense(v);        // the operands as the forward read them
+    Tensor* s = empty_tensor(q->dtype, q->device_id, nd, sshape.data());
+    Tensor* p = empty_tensor(q->dtype, q->device_id, nd, sshape.data());
+    bool ok = g && qd && kd && vd && s && p && device_gemm(s, qd, false, kd, true, nullptr, 0) == 0 &&
+              rp_mul_scalar(s->data, s->data, &sf, s->size, s->dtype, s->device_id) == 0 &&
+              softmax_kernel_device(p->data, s->data, s->size / sk, sk, 1, s->dtype) == 0;
+    if (ok && needs_grad(v)) gemm_grad(v, p, true, g, false);
+    if (ok && (needs_grad(q) || needs_grad(k))) {
+        ok = device_gemm(s, g, false, vd, true, nullptr, 0) == 0 &&                                          // dP, in S's buffer
+             backwards_softmax_device(s->data, p->data, p->data, p->size / sk, sk, 1, p->dtype) == 0 &&     // softmax'(dP), over P
+             rp_mul_scalar(p->data, p->data, &sf, p->size, p->dtype, p->device_id) == 0;                    // dS
+        if (ok && needs_grad(q)) gemm_grad(q, p, false, kd, false);
+        if (ok && needs_grad(k)) gemm_grad(k, p, true, qd, false);
+    }
+    (void)sq;
+    free_tensor(g); free_tensor(qd); free_tensor(kd); free_tensor(vd); free_tensor(s); free_tensor(p);
+}
+
 void backward_reduce_all_fn(GradFn* self, Tensor* grad_output) {     // sum_all / mean_all: every element receives g (or g / size)
     Tensor* x = self->inputs[0];
     if (!needs_grad(x)) return;
@@ -862,6 +893,37 @@ Tensor* op_linear(Tensor* x, Tensor* w, Tensor* bias) {
         if (bias) attach(out, backward_linear_fn, {x, w, bias});
         else attach(out, backward_linear_fn, {x, w});
     }
+    return out;
+}
+
+// O = softmax(scale · Q · Kᵀ) · V in one launch (extension; bfloat16 / float16, head dimension 32, 64 or 128).
+// q: [..., sq, d], k and v: [..., sk, d] with equal leading dims.  Equals q.op_matmul(kᵀ).op_mul_scalar(scale)
+// .op_softmax(-1).op_matmul(v) up to the roundings of the score matrix that the fused kernel does not make.
+Tensor* op_attention(Tensor* q, Tensor* k, Tensor* v, double scale) {
+    if (!q || !k || !v) return nullptr;
+    const int nd = q->ndim;
+    if (nd < 2 || k->ndim != nd || v->ndim != nd || !same_place(q, k) || !same_place(q, v)) { fail("op_attention: rank, dtype or device mismatch"); return nullptr; }
+    if (q->dtype != DTYPE_BFLOAT16 && q->dtype != DTYPE_FLOAT16) { fail("op_attention: bfloat16 or float16 tensors only"); return nullptr; }
+    if (q->device_id == -1) { fail("op_attention on host tensors is not provided by this build; move the operands to a GPU"); return nullptr; }
+    const int sq = q->shape[nd - 2], d = q->shape[nd - 1], sk = k->shape[nd - 2];
+    bool shapes = k->shape[nd - 1] == d && v->shape[nd - 1] == d && v->shape[nd - 2] == sk;
+    long long batch = 1;
+    for (int i = 0; i < nd - 2; i++) { shapes = shapes && k->shape[i] == q->shape[i] && v->shape[i] == q->shape[i]; batch *= q->shape[i]; }
+    if (!shapes || batch > 0x7fffffffll) { fail("op_attention: q [..., sq, d], k and v [..., sk, d] with equal leading dimensions"); return nullptr; }
+    Tensor* qd = dense(q); Tensor* kd = dense(k); Tensor* vd = dense(v);
+    Tensor* out = (qd && kd && vd) ? empty_tensor(q->dtype, q->device_id, nd, q->shape) : nullptr;
+    int rc = -1;
+    if (out && on_device(q->device_id))
+        rc = rp_hip_attention_forward(out->data, qd->data, kd->data, vd->data, nullptr, (int)batch, sq, sk, d,
+                                      (long long)sq * d, d, (long long)sk * d, d, (long long)sk * d, d, (long long)sq * d, d, scale, q->dtype);
+    if (rc != 0) { dev_fail("op_attention"); free_tensor(out); out = nullptr; }
+    if (out && (needs_grad(q) || needs_grad(k) || needs_grad(v))) {
+        GradFn* gf = attach(out, backward_attention_fn, {q, k, v});
+        ScalarSaved* sv = (ScalarSaved*)malloc(sizeof(ScalarSaved));
+        sv->s = scale;
+        gf->saved_data = sv;
+    }
+    free_tensor(qd); free_tensor(kd); free_tensor(vd);
     return out;
 }
 

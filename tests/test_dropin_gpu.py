@@ -244,6 +244,37 @@ def test_attention_batched_matmul_on_permuted_view(dtype, tol):
         assert oracle.rel_err(host(got.grad), want.grad.numpy()) <= tol
 
 
+# ---- the fused extension: one call for softmax(scale·q·kᵀ)·v, gradients through the recomputing backward
+@pytest.mark.parametrize("dtype,tol", [("bfloat16", 4e-2), ("float16", 6e-3)])
+def test_fused_attention_op_matches_the_unfused_chain_and_torch(dtype, tol):
+    import torch
+    rng = np.random.default_rng(54)
+    B, H, S, D = 2, 3, 96, 64
+    q, k, v, do = (rng.normal(0, 1, (B, H, S, D)) for _ in range(4))
+    qt, kt, vt = (dev(a, dtype, grad=True) for a in (q, k, v))
+    scale = 1.0 / np.sqrt(D)
+    o = qt.op_attention(kt, vt, scale)
+    assert o.shape == (B, H, S, D) and o.dtype == dtype and o.requires_grad
+    w = dev(do, dtype)
+    o.reshape([B * H * S, D]).op_matmul(w.reshape([B * H * S, D]).transpose(0, 1)).op_sum_all().backward()
+    # the same through the four separate ops
+    q2, k2, v2 = (dev(host(t), dtype, grad=True) for t in (qt, kt, vt))
+    o2 = q2.op_matmul(k2.permute([0, 1, 3, 2])).op_mul_scalar(scale).op_softmax(dim=-1).op_matmul(v2)
+    o2.reshape([B * H * S, D]).op_matmul(w.reshape([B * H * S, D]).transpose(0, 1)).op_sum_all().backward()
+    assert oracle.rel_err(host(o), host(o2)) <= tol
+    # and against float64 autograd
+    tq, tk, tv = (torch.tensor(host(t), requires_grad=True) for t in (qt, kt, vt))
+    to = torch.softmax(tq @ tk.transpose(2, 3) * scale, -1) @ tv
+    (to.reshape(-1, D) @ torch.tensor(host(w)).reshape(-1, D).T).sum().backward()
+    assert oracle.rel_err(host(o), to.detach().numpy()) <= tol
+    for got, chain, want in ((qt, q2, tq), (kt, k2, tk), (vt, v2, tv)):
+        assert got.grad.shape == (B, H, S, D)
+        assert oracle.rel_err(host(got.grad), want.grad.numpy()) <= tol
+        assert oracle.rel_err(host(got.grad), host(chain.grad)) <= tol
+    with pytest.raises(RuntimeError, match="op_attention operation failed"):
+        dev(q, "float32").op_attention(dev(k, "float32"), dev(v, "float32"), scale)      # 16-bit dtypes only
+
+
 # ---- reference tests/stress/stress_edge_cases.py:41-42, 193-198
 def test_error_conventions():
     a = rp.zeros([2, 3], device="cuda"); b = rp.zeros([2, 3], device="cuda")
