@@ -68,6 +68,7 @@ SIGNATURES = {
     "rp_hip_reduce_rows": (_i, [_vp, _vp, _i, _i, _i, _i]),
     "rp_hip_cross_entropy_mean": (_i, [_vp, _vp, _vp, _vp, _i, _i, _d, _i]),
     "rp_hip_attention_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i] + [_ll] * 8 + [_d, _i]),
+    "rp_hip_attention_backward": (_i, [_vp] * 9 + [_i] * 4 + [_ll] * 10 + [_d, _i]),
 }
 
 _lib = None

@@ -204,6 +204,348 @@ __global__ void __launch_bounds__(256) attention_fwd16_kernel(AttnArgs g) {
     }
 }
 
+// ============================================================================
+// Backward, two kernels plus a row-dot.  With P = softmax(scale * Q K^T), O = P V and upstream dO:
+//   Dq[q] = sum_d dO[q,d] O[q,d]
+//   dV = P^T dO          dP = dO V^T          dS = P o (dP - Dq) * scale          dQ = dS K          dK = dS^T Q
+// P is recomputed from the saved row-wise log-sum-exp: P = exp(scale * s - L[q]); nothing of size S x S is stored.
+// Every product is arranged so that the fp32 accumulator of one MFMA, narrowed to 16 bits, is the B operand of the
+// next without leaving the lane (see the forward kernel): the dQ kernel works on S^T tiles (lane = query), the
+// dK/dV kernel on S tiles (lane = key).  Operands whose rows are d-contiguous in memory load straight into MFMA
+// registers; the ones that must be read transposed (K^T for dQ; dO^T and Q^T for dV and dK) go through LDS and
+// ds_read_tr16_b64.
+// ============================================================================
+struct AttnBwdArgs {
+    void* dQ; void* dK; void* dV;           // dense [batch, s, d]
+    const void* Q; const void* K; const void* V; const void* dO;
+    const float* L;                         // [batch, sq] log-sum-exp rows from the forward
+    const float* Dq;                        // [batch, sq] row dots of dO and O
+    int batch, sq, sk;
+    long long q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, do_bs, do_rs;
+    float scale;
+};
+
+// A [32 rows][D] block of a d-contiguous matrix, staged in LDS for transposed MFMA operand reads.
+template <int D>
+struct AttnBlock {
+    static constexpr int VP = m16_mc_pitch(D);
+    static constexpr int ELEMS = AT_KEYS * VP;
+    static constexpr int PIECES = AT_KEYS * D / 8 / 256 > 0 ? AT_KEYS * D / 8 / 256 : 1;
+    static __device__ __forceinline__ void load(u32x4_t (&r)[PIECES], const uint16_t* M, long long rs, int row0, int rows, const char* end) {
+        const char* p = (const char*)(M + (long long)row0 * rs);
+        const __amdgpu_buffer_rsrc_t rsrc = m16_rsrc(p, row0 < rows ? (long long)(end - p) : 0);
+#pragma unroll
+        for (int i = 0; i < PIECES; i++) {
+            const int id = threadIdx.x + 256 * i, row = id / (D / 8), d8 = (id % (D / 8)) * 8;
+            const bool live = AT_KEYS * D / 8 >= 256 || id < AT_KEYS * D / 8;
+            r[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, live ? (int)(((long long)row * rs + d8) * 2) : (int)M16_OOB, 0, 0);
+        }
+    }
+    static __device__ __forceinline__ void store(const u32x4_t (&r)[PIECES], uint16_t* stage) {
+#pragma unroll
+        for (int i = 0; i < PIECES; i++) {
+            const int id = threadIdx.x + 256 * i, row = id / (D / 8), d8 = (id % (D / 8)) * 8;
+            if (AT_KEYS * D / 8 >= 256 || id < AT_KEYS * D / 8) *(u32x4_t*)(stage + row * VP + d8) = r[i];
+        }
+    }
+    // lane's base offset for transposed reads: k slot e of MFMA t <-> block row 16t + 8*(e/4) + 4*(lane/32) + e%4
+    static __device__ __forceinline__ int tr_base(int lane) {
+        const int grp = lane >> 4, s16 = lane & 15;
+        return (4 * (grp >> 1) + (s16 >> 2)) * VP + 16 * (grp & 1) + 4 * (s16 & 3);
+    }
+    static __device__ __forceinline__ s16x8_t read_tr(const uint16_t* stage, int base, int dt, int t) {
+        s16x8_t f;
+#pragma unroll
+        for (int H = 0; H < 2; H++) {
+            s16x4_t q4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3)))*)(lds_u16*)(stage + base + (16 * t + 8 * H) * VP + 32 * dt));
+            f[4 * H + 0] = q4[0]; f[4 * H + 1] = q4[1]; f[4 * H + 2] = q4[2]; f[4 * H + 3] = q4[3];
+        }
+        return f;
+    }
+};
+
+// rows row0 + c of a d-contiguous matrix as MFMA operand fragments (A: row = lane % 32; B: column = lane % 32), zero past `rows`
+template <int KS>
+__device__ __forceinline__ void attn_load_rows(s16x8_t (&f)[KS], const uint16_t* M, long long rs, int row0, int rows, const char* end, int c, int h) {
+    const char* p = (const char*)(M + (long long)row0 * rs);
+    const __amdgpu_buffer_rsrc_t rsrc = m16_rsrc(p, row0 < rows ? (long long)(end - p) : 0);
+    const int voff = (int)(((long long)c * rs + 8 * h) * 2);
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) f[ks] = __builtin_bit_cast(s16x8_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, 32 * ks, 0));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) attention_rowdot_kernel(float* out, const T* a, const T* b, int rows, int d, long long a_bs, long long a_rs,
+                                                               long long b_bs, long long b_rs, int sq) {
+    // one row per 8 lanes: out[r] = sum_d a[r, d] * b[r, d], r = z * sq + q
+    const long long r = ((long long)blockIdx.x * 256 + threadIdx.x) >> 3;
+    const int part = threadIdx.x & 7;
+    float acc = 0.f;
+    if (r < rows) {
+        const long long z = r / sq, q = r % sq;
+        const T* pa = a + z * a_bs + q * a_rs;
+        const T* pb = b + z * b_bs + q * b_rs;
+        for (int i = part * 8; i < d; i += 64) {
+            u32x4_t ra = *(const u32x4_t*)(pa + i), rb = *(const u32x4_t*)(pb + i);
+            T va[8], vb[8];
+            memcpy(va, &ra, 16); memcpy(vb, &rb, 16);
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc += widen(va[e]) * widen(vb[e]);
+        }
+    }
+    acc += __shfl_xor(acc, 1, 64); acc += __shfl_xor(acc, 2, 64); acc += __shfl_xor(acc, 4, 64);
+    if (r < rows && part == 0) out[r] = acc;
+}
+
+// dQ: a wave owns 32 queries and walks the keys.
+template <typename T, int D>
+__global__ void __launch_bounds__(256) attention_bwd_dq16_kernel(AttnBwdArgs g) {
+    constexpr int KS = D / 16, DT = D / 32;
+    using Blk = AttnBlock<D>;
+    __shared__ __attribute__((aligned(16))) uint16_t klds[2][Blk::ELEMS];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int h = lane >> 5, c = lane & 31;
+    const int z = blockIdx.y;
+    const int q0 = blockIdx.x * AT_QROWS + wave * 32;
+    const uint16_t* Q = (const uint16_t*)g.Q + (long long)z * g.q_bs;
+    const uint16_t* K = (const uint16_t*)g.K + (long long)z * g.k_bs;
+    const uint16_t* V = (const uint16_t*)g.V + (long long)z * g.v_bs;
+    const uint16_t* dO = (const uint16_t*)g.dO + (long long)z * g.do_bs;
+    const char* q_end = (const char*)(Q + ((long long)(g.sq - 1) * g.q_rs + D));
+    const char* k_end = (const char*)(K + ((long long)(g.sk - 1) * g.k_rs + D));
+    const char* v_end = (const char*)(V + ((long long)(g.sk - 1) * g.v_rs + D));
+    const char* do_end = (const char*)(dO + ((long long)(g.sq - 1) * g.do_rs + D));
+    const float sc = g.scale * 1.44269504088896341f;
+
+    s16x8_t qf[KS], dof[KS];                 // B operands: column = query q0 + c
+    attn_load_rows<KS>(qf, Q, g.q_rs, q0, g.sq, q_end, c, h);
+    attn_load_rows<KS>(dof, dO, g.do_rs, q0, g.sq, do_end, c, h);
+    const int q = q0 + c;
+    const float lq = q < g.sq ? g.L[(long long)z * g.sq + q] * 1.44269504088896341f : 0.f;
+    const float dq_dot = q < g.sq ? g.Dq[(long long)z * g.sq + q] : 0.f;
+
+    f32x16_t acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[dt][v] = 0.f;
+
+    const int tr0 = Blk::tr_base(lane);
+    const int nblocks = (g.sk + AT_KEYS - 1) / AT_KEYS;
+    s16x8_t kf[2][KS], vf[2][KS];
+    u32x4_t kr[Blk::PIECES];
+    attn_load_rows<KS>(kf[0], K, g.k_rs, 0, g.sk, k_end, c, h);
+    attn_load_rows<KS>(vf[0], V, g.v_rs, 0, g.sk, v_end, c, h);
+    Blk::load(kr, K, g.k_rs, 0, g.sk, k_end);
+    Blk::store(kr, klds[0]);
+    attn_load_rows<KS>(kf[1], K, g.k_rs, AT_KEYS, g.sk, k_end, c, h);
+    attn_load_rows<KS>(vf[1], V, g.v_rs, AT_KEYS, g.sk, v_end, c, h);
+    Blk::load(kr, K, g.k_rs, AT_KEYS, g.sk, k_end);
+    __syncthreads();
+
+    auto step = [&](int blk, auto slotc) {
+        constexpr int SLOT = decltype(slotc)::value;
+        const int kb = blk * AT_KEYS;
+        const uint16_t* stage = klds[blk & 1];
+        f32x16_t st, dp;
+#pragma unroll
+        for (int v = 0; v < 16; v++) { st[v] = 0.f; dp[v] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) st = mfma16_ops<T>::mma(kf[SLOT][ks], qf[ks], st);        // S^T: keys x queries
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) dp = mfma16_ops<T>::mma(vf[SLOT][ks], dof[ks], dp);       // dP^T
+        attn_load_rows<KS>(kf[SLOT], K, g.k_rs, kb + 2 * AT_KEYS, g.sk, k_end, c, h);
+        attn_load_rows<KS>(vf[SLOT], V, g.v_rs, kb + 2 * AT_KEYS, g.sk, v_end, c, h);
+        Blk::store(kr, klds[(blk & 1) ^ 1]);
+        Blk::load(kr, K, g.k_rs, kb + 2 * AT_KEYS, g.sk, k_end);
+        T ds[16];
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int key = kb + 8 * (v / 4) + 4 * h + (v % 4);
+            const float p = key < g.sk ? widen(narrow<T>(__builtin_amdgcn_exp2f(st[v] * sc - lq))) : 0.f;     // the P the forward multiplied with
+            ds[v] = narrow<T>(p * (dp[v] - dq_dot) * g.scale);
+        }
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            s16x8_t dsb;
+#pragma unroll
+            for (int e = 0; e < 8; e++) dsb[e] = (short)ds[8 * t + e].bits;
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) acc[dt] = mfma16_ops<T>::mma(Blk::read_tr(stage, tr0, dt, t), dsb, acc[dt]);      // dQ^T += K^T dS^T
+        }
+        __syncthreads();
+    };
+    for (int blk = 0; blk < nblocks; blk += 2) {
+        step(blk, std::integral_constant<int, 0>{});
+        if (blk + 1 < nblocks) step(blk + 1, std::integral_constant<int, 1>{});
+    }
+    if (q < g.sq) {
+        T* row = (T*)g.dQ + ((long long)z * g.sq + q) * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int v4 = 0; v4 < 4; v4++) {
+                T out[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) out[e] = narrow<T>(acc[dt][4 * v4 + e]);
+                uint2 w;
+                memcpy(&w, out, 8);
+                *(uint2*)(row + 32 * dt + 8 * v4 + 4 * h) = w;
+            }
+    }
+}
+
+// dK and dV: a wave owns 32 keys and walks the queries.
+template <typename T, int D>
+__global__ void __launch_bounds__(256) attention_bwd_dkv16_kernel(AttnBwdArgs g) {
+    constexpr int KS = D / 16, DT = D / 32;
+    using Blk = AttnBlock<D>;
+    __shared__ __attribute__((aligned(16))) uint16_t qlds[2][Blk::ELEMS];
+    __shared__ __attribute__((aligned(16))) uint16_t dolds[2][Blk::ELEMS];
+    __shared__ __attribute__((aligned(16))) float rowlds[2][2][AT_KEYS];        // [stage][L, Dq][query of the block]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int h = lane >> 5, c = lane & 31;
+    const int z = blockIdx.y;
+    const int k0 = blockIdx.x * AT_QROWS + wave * 32;               // this wave's first key
+    const uint16_t* Q = (const uint16_t*)g.Q + (long long)z * g.q_bs;
+    const uint16_t* K = (const uint16_t*)g.K + (long long)z * g.k_bs;
+    const uint16_t* V = (const uint16_t*)g.V + (long long)z * g.v_bs;
+    const uint16_t* dO = (const uint16_t*)g.dO + (long long)z * g.do_bs;
+    const char* q_end = (const char*)(Q + ((long long)(g.sq - 1) * g.q_rs + D));
+    const char* k_end = (const char*)(K + ((long long)(g.sk - 1) * g.k_rs + D));
+    const char* v_end = (const char*)(V + ((long long)(g.sk - 1) * g.v_rs + D));
+    const char* do_end = (const char*)(dO + ((long long)(g.sq - 1) * g.do_rs + D));
+    const float sc = g.scale * 1.44269504088896341f;
+    const float* Lz = g.L + (long long)z * g.sq;
+    const float* Dz = g.Dq + (long long)z * g.sq;
+
+    s16x8_t kf[KS], vf[KS];                  // B operands: column = key k0 + c
+    attn_load_rows<KS>(kf, K, g.k_rs, k0, g.sk, k_end, c, h);
+    attn_load_rows<KS>(vf, V, g.v_rs, k0, g.sk, v_end, c, h);
+
+    f32x16_t dkt[DT], dvt[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) { dkt[dt][v] = 0.f; dvt[dt][v] = 0.f; }
+
+    const int tr0 = Blk::tr_base(lane);
+    const int nblocks = (g.sq + AT_KEYS - 1) / AT_KEYS;
+    s16x8_t qf[2][KS], dof[2][KS];           // A operands: row = query qb + c
+    u32x4_t qr[Blk::PIECES], dor[Blk::PIECES];
+    float rowv = 0.f;                        // threads 0..31: L of query qb + t; 32..63: Dq of query qb + t - 32
+    auto load_rowv = [&](int qb) {
+        const int t = threadIdx.x, qq = qb + (t & 31);
+        rowv = (t < 64 && qq < g.sq) ? (t < 32 ? Lz[qq] * 1.44269504088896341f : Dz[qq]) : 0.f;
+    };
+    auto store_rowv = [&](int stage) { if (threadIdx.x < 64) rowlds[stage][threadIdx.x >> 5][threadIdx.x & 31] = rowv; };
+    attn_load_rows<KS>(qf[0], Q, g.q_rs, 0, g.sq, q_end, c, h);
+    attn_load_rows<KS>(dof[0], dO, g.do_rs, 0, g.sq, do_end, c, h);
+    Blk::load(qr, Q, g.q_rs, 0, g.sq, q_end);
+    Blk::load(dor, dO, g.do_rs, 0, g.sq, do_end);
+    load_rowv(0);
+    Blk::store(qr, qlds[0]);
+    Blk::store(dor, dolds[0]);
+    store_rowv(0);
+    attn_load_rows<KS>(qf[1], Q, g.q_rs, AT_KEYS, g.sq, q_end, c, h);
+    attn_load_rows<KS>(dof[1], dO, g.do_rs, AT_KEYS, g.sq, do_end, c, h);
+    Blk::load(qr, Q, g.q_rs, AT_KEYS, g.sq, q_end);
+    Blk::load(dor, dO, g.do_rs, AT_KEYS, g.sq, do_end);
+    load_rowv(AT_KEYS);
+    __syncthreads();
+
+    auto step = [&](int blk, auto slotc) {
+        constexpr int SLOT = decltype(slotc)::value;
+        const int qb = blk * AT_KEYS;
+        const int cur = blk & 1;
+        f32x16_t st, dp;
+#pragma unroll
+        for (int v = 0; v < 16; v++) { st[v] = 0.f; dp[v] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) st = mfma16_ops<T>::mma(qf[SLOT][ks], kf[ks], st);        // S: queries x keys
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) dp = mfma16_ops<T>::mma(dof[SLOT][ks], vf[ks], dp);       // dP
+        attn_load_rows<KS>(qf[SLOT], Q, g.q_rs, qb + 2 * AT_KEYS, g.sq, q_end, c, h);
+        attn_load_rows<KS>(dof[SLOT], dO, g.do_rs, qb + 2 * AT_KEYS, g.sq, do_end, c, h);
+        Blk::store(qr, qlds[cur ^ 1]);
+        Blk::store(dor, dolds[cur ^ 1]);
+        store_rowv(cur ^ 1);
+        Blk::load(qr, Q, g.q_rs, qb + 2 * AT_KEYS, g.sq, q_end);
+        Blk::load(dor, dO, g.do_rs, qb + 2 * AT_KEYS, g.sq, do_end);
+        load_rowv(qb + 2 * AT_KEYS);
+        T p[16], ds[16];
+#pragma unroll
+        for (int v4 = 0; v4 < 4; v4++) {
+            // registers 4*v4 .. 4*v4+3 are queries qb + 8*v4 + 4h + (0..3): their L and Dq are 16 contiguous bytes each
+            const f32x4_t l4 = *(const f32x4_t*)&rowlds[cur][0][8 * v4 + 4 * h];
+            const f32x4_t d4 = *(const f32x4_t*)&rowlds[cur][1][8 * v4 + 4 * h];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int v = 4 * v4 + e, qrow = qb + 8 * v4 + 4 * h + e;
+                const float pe = qrow < g.sq ? __builtin_amdgcn_exp2f(st[v] * sc - l4[e]) : 0.f;
+                p[v] = narrow<T>(pe);
+                ds[v] = narrow<T>(widen(p[v]) * (dp[v] - d4[e]) * g.scale);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            s16x8_t pb, dsb;
+#pragma unroll
+            for (int e = 0; e < 8; e++) { pb[e] = (short)p[8 * t + e].bits; dsb[e] = (short)ds[8 * t + e].bits; }
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+                dvt[dt] = mfma16_ops<T>::mma(Blk::read_tr(dolds[cur], tr0, dt, t), pb, dvt[dt]);      // dV^T += dO^T P
+                dkt[dt] = mfma16_ops<T>::mma(Blk::read_tr(qlds[cur], tr0, dt, t), dsb, dkt[dt]);      // dK^T += Q^T dS
+            }
+        }
+        __syncthreads();
+    };
+    for (int blk = 0; blk < nblocks; blk += 2) {
+        step(blk, std::integral_constant<int, 0>{});
+        if (blk + 1 < nblocks) step(blk + 1, std::integral_constant<int, 1>{});
+    }
+    const int key = k0 + c;
+    if (key < g.sk) {
+        T* krow = (T*)g.dK + ((long long)z * g.sk + key) * D;
+        T* vrow = (T*)g.dV + ((long long)z * g.sk + key) * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int v4 = 0; v4 < 4; v4++) {
+                T ok[4], ov[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) { ok[e] = narrow<T>(dkt[dt][4 * v4 + e]); ov[e] = narrow<T>(dvt[dt][4 * v4 + e]); }
+                uint2 wk, wv;
+                memcpy(&wk, ok, 8); memcpy(&wv, ov, 8);
+                *(uint2*)(krow + 32 * dt + 8 * v4 + 4 * h) = wk;
+                *(uint2*)(vrow + 32 * dt + 8 * v4 + 4 * h) = wv;
+            }
+    }
+}
+
+template <typename T>
+static int launch_attention_bwd_t(const AttnBwdArgs& g, int d) {
+    dim3 gq((g.sq + AT_QROWS - 1) / AT_QROWS, g.batch), gk((g.sk + AT_QROWS - 1) / AT_QROWS, g.batch);
+    switch (d) {
+        case 32:
+            hipLaunchKernelGGL((attention_bwd_dq16_kernel<T, 32>), gq, dim3(256), 0, current_stream(), g);
+            hipLaunchKernelGGL((attention_bwd_dkv16_kernel<T, 32>), gk, dim3(256), 0, current_stream(), g);
+            break;
+        case 64:
+            hipLaunchKernelGGL((attention_bwd_dq16_kernel<T, 64>), gq, dim3(256), 0, current_stream(), g);
+            hipLaunchKernelGGL((attention_bwd_dkv16_kernel<T, 64>), gk, dim3(256), 0, current_stream(), g);
+            break;
+        case 128:
+            hipLaunchKernelGGL((attention_bwd_dq16_kernel<T, 128>), gq, dim3(256), 0, current_stream(), g);
+            hipLaunchKernelGGL((attention_bwd_dkv16_kernel<T, 128>), gk, dim3(256), 0, current_stream(), g);
+            break;
+        default: set_error("rp_hip_attention_backward: head dimension %d (supported: 32, 64, 128)", d); return -1;
+    }
+    return check_launch("attention backward kernels") ? 0 : -1;
+}
+
 template <typename T>
 static int launch_attention_t(const AttnArgs& g, int d) {
     dim3 grid((g.sq + AT_QROWS - 1) / AT_QROWS, g.batch);
@@ -245,3 +587,42 @@ extern "C" int rp_hip_attention_forward(void* O, const void* Q, const void* K, c
     }
     return 0;
 }
+
+extern "C" int rp_hip_attention_backward(void* dQ, void* dK, void* dV, const void* Q, const void* K, const void* V,
+                                         const void* O, const void* dO, const float* lse,
+                                         int batch, int sq, int sk, int d,
+                                         long long q_bs, long long q_rs, long long k_bs, long long k_rs,
+                                         long long v_bs, long long v_rs, long long o_bs, long long o_rs,
+                                         long long do_bs, long long do_rs, double scale, int dtype) {
+    if (!dQ || !dK || !dV || !Q || !K || !V || !O || !dO || !lse || batch <= 0 || sq <= 0 || sk <= 0 || d <= 0) {
+        set_error("rp_hip_attention_backward: null operand or non-positive extent (batch=%d sq=%d sk=%d d=%d)", batch, sq, sk, d);
+        return -1;
+    }
+    if (dtype != RP_DTYPE_BFLOAT16 && dtype != RP_DTYPE_FLOAT16) { set_error("rp_hip_attention_backward: bfloat16 / float16 only (dtype %d)", dtype); return -1; }
+    if (d != 32 && d != 64 && d != 128) { set_error("rp_hip_attention_backward: head dimension %d (supported: 32, 64, 128)", d); return -1; }
+    if (batch > 65535) { set_error("rp_hip_attention_backward: batch %d exceeds 65535", batch); return -1; }
+    const long long strides[] = {q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs, do_bs, do_rs};
+    for (long long s : strides)
+        if (s < 0 || s % 8) { set_error("rp_hip_attention_backward: strides must be non-negative multiples of 8 elements"); return -1; }
+    if (q_rs >= (1ll << 22) || k_rs >= (1ll << 22) || v_rs >= (1ll << 22) || do_rs >= (1ll << 22)) { set_error("rp_hip_attention_backward: row stride too large"); return -1; }
+    if (((uintptr_t)dQ | (uintptr_t)dK | (uintptr_t)dV | (uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)O | (uintptr_t)dO) & 15) {
+        set_error("rp_hip_attention_backward: operands must be 16-byte aligned");
+        return -1;
+    }
+    void* dots = nullptr;
+    if (rp_hip_malloc(&dots, (size_t)batch * sq * sizeof(float)) != 0) return -1;
+    const int rows = batch * sq;
+    const unsigned blocks = (unsigned)(((long long)rows * 8 + 255) / 256);
+    if (dtype == RP_DTYPE_BFLOAT16)
+        hipLaunchKernelGGL(attention_rowdot_kernel<bf16_t>, dim3(blocks), dim3(256), 0, current_stream(), (float*)dots, (const bf16_t*)dO, (const bf16_t*)O, rows, d, do_bs, do_rs, o_bs, o_rs, sq);
+    else
+        hipLaunchKernelGGL(attention_rowdot_kernel<f16_t>, dim3(blocks), dim3(256), 0, current_stream(), (float*)dots, (const f16_t*)dO, (const f16_t*)O, rows, d, do_bs, do_rs, o_bs, o_rs, sq);
+    int rc = check_launch("attention_rowdot_kernel") ? 0 : -1;
+    if (rc == 0) {
+        AttnBwdArgs g{dQ, dK, dV, Q, K, V, dO, lse, (const float*)dots, batch, sq, sk, q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, do_bs, do_rs, (float)scale};
+        rc = dtype == RP_DTYPE_BFLOAT16 ? launch_attention_bwd_t<bf16_t>(g, d) : launch_attention_bwd_t<f16_t>(g, d);
+    }
+    rp_hip_free(dots);        // stream-ordered reuse: the pool hands it out again only to later work on this stream
+    return rc;
+}
+

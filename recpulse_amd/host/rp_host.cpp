@@ -751,35 +751,40 @@ void backward_mul_scalar_fn(GradFn* self, Tensor* grad_output) {     // referenc
     free_tensor(gd);
 }
 
-// Backward of the fused attention: the probabilities are recomputed with the unfused kernels (S = Q·Kᵀ, scale,
-// softmax), then dV = Pᵀ·dO, dP = dO·Vᵀ, dS = softmax'(dP)·scale, dQ = dS·K, dK = dSᵀ·Q — the chain the reference's
-// autograd runs for matmul -> mul_scalar -> softmax -> matmul (ops/ops.c:6759-6814, 5966-6020, 5665-5719), with the
-// transposes as stride views and the gradient accumulation inside the GEMMs.
+// Backward of op_attention in three launches (rp_hip_attention_backward): the probabilities are recomputed tile by
+// tile from the row-wise log-sum-exp the forward saved, so nothing of size sq x sk is allocated.  The values are those
+// of the chain the reference's autograd runs for matmul -> mul_scalar -> softmax -> matmul (ops/ops.c:6759-6814,
+// 5966-6020, 5665-5719): dV = P^T dO, dP = dO V^T, dS = softmax'(dP) * scale, dQ = dS K, dK = dS^T Q.
+struct AttnSaved { double scale; void* lse; int device_id; };
+
+void free_attn_saved(void* p) {
+    AttnSaved* s = (AttnSaved*)p;
+    if (s->lse && on_device(s->device_id)) rp_hip_free(s->lse);
+    free(s);
+}
+
 void backward_attention_fn(GradFn* self, Tensor* grad_output) {
     Tensor* q = self->inputs[0]; Tensor* k = self->inputs[1]; Tensor* v = self->inputs[2];
     if (!needs_grad(q) && !needs_grad(k) && !needs_grad(v)) return;
-    const double scale = ((ScalarSaved*)self->saved_data)->s;
-    const float sf = (float)scale;
-    const int nd = q->ndim, sq = q->shape[nd - 2], sk = k->shape[nd - 2];
-    std::vector<int> sshape(q->shape, q->shape + nd);
-    sshape[nd - 1] = sk;
+    AttnSaved* sv = (AttnSaved*)self->saved_data;
+    Tensor* o = self->owner;
+    const int nd = q->ndim, sq = q->shape[nd - 2], sk = k->shape[nd - 2], d = q->shape[nd - 1];
+    const int batch = (int)(q->size / ((size_t)sq * d));
     Tensor* g = dense(grad_output);
+    Tensor* od = o ? dense(o) : nullptr;
     Tensor* qd = dense(q); Tensor* kd = dense(k); Tensor* vd = dense(v);        // the operands as the forward read them
-    Tensor* s = empty_tensor(q->dtype, q->device_id, nd, sshape.data());
-    Tensor* p = empty_tensor(q->dtype, q->device_id, nd, sshape.data());
-    bool ok = g && qd && kd && vd && s && p && device_gemm(s, qd, false, kd, true, nullptr, 0) == 0 &&
-              rp_mul_scalar(s->data, s->data, &sf, s->size, s->dtype, s->device_id) == 0 &&
-              softmax_kernel_device(p->data, s->data, s->size / sk, sk, 1, s->dtype) == 0;
-    if (ok && needs_grad(v)) gemm_grad(v, p, true, g, false);
-    if (ok && (needs_grad(q) || needs_grad(k))) {
-        ok = device_gemm(s, g, false, vd, true, nullptr, 0) == 0 &&                                          // dP, in S's buffer
-             backwards_softmax_device(s->data, p->data, p->data, p->size / sk, sk, 1, p->dtype) == 0 &&     // softmax'(dP), over P
-             rp_mul_scalar(p->data, p->data, &sf, p->size, p->dtype, p->device_id) == 0;                    // dS
-        if (ok && needs_grad(q)) gemm_grad(q, p, false, kd, false);
-        if (ok && needs_grad(k)) gemm_grad(k, p, true, qd, false);
-    }
-    (void)sq;
-    free_tensor(g); free_tensor(qd); free_tensor(kd); free_tensor(vd); free_tensor(s); free_tensor(p);
+    Tensor* dq = empty_tensor(q->dtype, q->device_id, nd, q->shape);
+    Tensor* dk = empty_tensor(k->dtype, k->device_id, nd, k->shape);
+    Tensor* dv = empty_tensor(v->dtype, v->device_id, nd, v->shape);
+    const long long qs = (long long)sq * d, ks = (long long)sk * d;
+    bool ok = g && od && qd && kd && vd && dq && dk && dv && on_device(q->device_id) &&
+              rp_hip_attention_backward(dq->data, dk->data, dv->data, qd->data, kd->data, vd->data, od->data, g->data, (const float*)sv->lse,
+                                        batch, sq, sk, d, qs, d, ks, d, ks, d, qs, d, qs, d, sv->scale, q->dtype) == 0;
+    if (!ok) dev_fail("op_attention backward");
+    if (ok && needs_grad(q)) accumulate_grad(q, dq); else free_tensor(dq);
+    if (ok && needs_grad(k)) accumulate_grad(k, dk); else free_tensor(dk);
+    if (ok && needs_grad(v)) accumulate_grad(v, dv); else free_tensor(dv);
+    free_tensor(g); free_tensor(od); free_tensor(qd); free_tensor(kd); free_tensor(vd);
 }
 
 void backward_reduce_all_fn(GradFn* self, Tensor* grad_output) {     // sum_all / mean_all: every element receives g (or g / size)
@@ -912,16 +917,19 @@ Tensor* op_attention(Tensor* q, Tensor* k, Tensor* v, double scale) {
     if (!shapes || batch > 0x7fffffffll) { fail("op_attention: q [..., sq, d], k and v [..., sk, d] with equal leading dimensions"); return nullptr; }
     Tensor* qd = dense(q); Tensor* kd = dense(k); Tensor* vd = dense(v);
     Tensor* out = (qd && kd && vd) ? empty_tensor(q->dtype, q->device_id, nd, q->shape) : nullptr;
+    const bool track = needs_grad(q) || needs_grad(k) || needs_grad(v);
+    void* lse = nullptr;                                 // row-wise log-sum-exp, kept for the backward
     int rc = -1;
-    if (out && on_device(q->device_id))
-        rc = rp_hip_attention_forward(out->data, qd->data, kd->data, vd->data, nullptr, (int)batch, sq, sk, d,
+    if (out && on_device(q->device_id) && (!track || rp_hip_malloc(&lse, sizeof(float) * (size_t)batch * sq) == 0))
+        rc = rp_hip_attention_forward(out->data, qd->data, kd->data, vd->data, (float*)lse, (int)batch, sq, sk, d,
                                       (long long)sq * d, d, (long long)sk * d, d, (long long)sk * d, d, (long long)sq * d, d, scale, q->dtype);
-    if (rc != 0) { dev_fail("op_attention"); free_tensor(out); out = nullptr; }
-    if (out && (needs_grad(q) || needs_grad(k) || needs_grad(v))) {
+    if (rc != 0) { dev_fail("op_attention"); free_tensor(out); out = nullptr; if (lse) rp_hip_free(lse); lse = nullptr; }
+    if (out && track) {
         GradFn* gf = attach(out, backward_attention_fn, {q, k, v});
-        ScalarSaved* sv = (ScalarSaved*)malloc(sizeof(ScalarSaved));
-        sv->s = scale;
+        AttnSaved* sv = (AttnSaved*)malloc(sizeof(AttnSaved));
+        sv->scale = scale; sv->lse = lse; sv->device_id = q->device_id;
         gf->saved_data = sv;
+        gf->free_saved = free_attn_saved;
     }
     free_tensor(qd); free_tensor(kd); free_tensor(vd);
     return out;

@@ -74,3 +74,72 @@ def test_fused_attention_rejects_bad_arguments():
     assert b"head dimension" in L.rp_hip_last_error()
     assert L.rp_hip_attention_forward(d.ptr, d.ptr, d.ptr, d.ptr, None, 1, 4, 4, 64, 256, 64, 256, 64, 256, 64, 256, 64, 1.0, capi.F32) == -1
     assert L.rp_hip_attention_forward(d.ptr, d.ptr, d.ptr, d.ptr, None, 1, 4, 4, 64, 256, 60, 256, 64, 256, 64, 256, 64, 1.0, BF16) == -1
+
+
+def _f64_backward(q, k, v, g, dt, scale):
+    """Closed-form gradients of O = softmax(scale q k^T) v in float64 (the chain rule the reference's autograd applies)."""
+    q64, k64, v64, g64 = (oracle.to_f64(x, dt) for x in (q, k, v, g))
+    s = np.einsum("zqd,zkd->zqk", q64, k64) * scale
+    e = np.exp(s - s.max(-1, keepdims=True))
+    p = e / e.sum(-1, keepdims=True)
+    dv = np.einsum("zqk,zqd->zkd", p, g64)
+    dp = np.einsum("zqd,zkd->zqk", g64, v64)
+    ds = p * (dp - (dp * p).sum(-1, keepdims=True)) * scale
+    return np.einsum("zqk,zkd->zqd", ds, k64), np.einsum("zqk,zqd->zkd", ds, q64), dv
+
+
+def _fused_backward(q, k, v, g, dt, scale):
+    Z, sq, d = q.shape
+    sk = k.shape[1]
+    dq, dk, dv, dg = Dev(q, dt), Dev(k, dt), Dev(v, dt), Dev(g, dt)
+    do = Dev.empty((Z, sq, d), dt)
+    lse = capi.DeviceBuffer(Z * sq * 4)
+    L = capi.lib()
+    capi.check(L.rp_hip_attention_forward(do.ptr, dq.ptr, dk.ptr, dv.ptr, lse.ptr, Z, sq, sk, d,
+                                          sq * d, d, sk * d, d, sk * d, d, sq * d, d, float(scale), dt), "rp_hip_attention_forward")
+    gq, gk, gv = Dev.empty((Z, sq, d), dt), Dev.empty((Z, sk, d), dt), Dev.empty((Z, sk, d), dt)
+    capi.check(L.rp_hip_attention_backward(gq.ptr, gk.ptr, gv.ptr, dq.ptr, dk.ptr, dv.ptr, do.ptr, dg.ptr, lse.ptr, Z, sq, sk, d,
+                                           sq * d, d, sk * d, d, sk * d, d, sq * d, d, sq * d, d, float(scale), dt), "rp_hip_attention_backward")
+    return gq.numpy(), gk.numpy(), gv.numpy()
+
+
+@pytest.mark.parametrize("dt", [BF16, F16], ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("shape", [(6, 512, 512, 64), (3, 200, 333, 64), (2, 130, 65, 32), (2, 96, 160, 128), (1, 1, 1, 64), (5, 33, 31, 64)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_fused_attention_backward(dt, shape):
+    Z, sq, sk, d = shape
+    rng = np.random.default_rng(62)
+    q, k, v = rand_storage(rng, (Z, sq, d), dt), rand_storage(rng, (Z, sk, d), dt), rand_storage(rng, (Z, sk, d), dt)
+    g = rand_storage(rng, (Z, sq, d), dt)
+    scale = 1.0 / np.sqrt(d)
+    got = _fused_backward(q, k, v, g, dt, scale)
+    want = _f64_backward(q, k, v, g, dt, scale)
+    # P and dS are rounded to the tensor dtype before they enter a product (as the reference's chain rounds them)
+    tol = 2e-2 if dt == BF16 else 4e-3
+    for name, a, b in zip(("dQ", "dK", "dV"), got, want):
+        assert oracle.rel_err(oracle.to_f64(a, dt), b) <= tol, name
+    again = _fused_backward(q, k, v, g, dt, scale)
+    assert all(np.array_equal(a, b) for a, b in zip(got, again))
+
+
+def test_fused_attention_backward_large_scores():
+    """Rows whose softmax is nearly one-hot: exp(scale s - lse) must reproduce the forward's probabilities."""
+    rng = np.random.default_rng(63)
+    Z, S, D = 4, 256, 64
+    q = oracle.to_storage(rng.normal(0, 3, (Z, S, D)), BF16); k = oracle.to_storage(rng.normal(0, 3, (Z, S, D)), BF16)
+    v, g = rand_storage(rng, (Z, S, D), BF16), rand_storage(rng, (Z, S, D), BF16)
+    got = _fused_backward(q, k, v, g, BF16, 0.125)
+    want = _f64_backward(q, k, v, g, BF16, 0.125)
+    for a, b in zip(got, want):
+        assert np.all(np.isfinite(oracle.to_f64(a, BF16)))
+        assert oracle.rel_err(oracle.to_f64(a, BF16), b) <= 3e-2
+
+
+def test_fused_attention_backward_rejects_bad_arguments():
+    d = capi.DeviceBuffer(4096)
+    L = capi.lib()
+    p = d.ptr
+    assert L.rp_hip_attention_backward(p, p, p, p, p, p, p, p, p, 1, 4, 4, 48, 192, 48, 192, 48, 192, 48, 192, 48, 192, 48, 1.0, BF16) == -1
+    assert b"head dimension" in L.rp_hip_last_error()
+    assert L.rp_hip_attention_backward(p, p, p, p, p, p, p, p, None, 1, 4, 4, 64, 256, 64, 256, 64, 256, 64, 256, 64, 256, 64, 1.0, BF16) == -1
+    assert L.rp_hip_attention_backward(p, p, p, p, p, p, p, p, p, 1, 4, 4, 64, 256, 64, 256, 64, 256, 64, 256, 64, 256, 64, 1.0, capi.F32) == -1
