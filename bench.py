@@ -296,7 +296,7 @@ def attention_times(capi, dt_name="bf16"):
         nbytes = 4 * sd * Z * esz
         out["fused_forward"] = {"us": round(ms * 1e3, 1), "unfused_chain_us": round(chain, 1), "TFLOP/s": round(4.0 * Z * S * S * D / ms / 1e9, 1),
                                 "GB/s": round(nbytes / ms / 1e6, 1)}
-        # and the backward (dQ, dK, dV from Q, K, V, O, dO and the saved row statistics) as three launches
+        # and the backward (dQ, dK, dV from Q, K, V, O, dO and the saved row statistics) as two launches
         d_lse = D_(Z * S * 4)
         capi.check(L.rp_hip_attention_forward(d_o.ptr, d_q.ptr, d_k.ptr, d_v.ptr, d_lse.ptr, Z, S, S, D, sd, D, sd, D, sd, D, sd, D, 0.125, dt), "rp_hip_attention_forward")
         fused_b = lambda: capi.check(L.rp_hip_attention_backward(d_dq.ptr, d_dk.ptr, d_dv.ptr, d_q.ptr, d_k.ptr, d_v.ptr, d_o.ptr, d_do.ptr, d_lse.ptr,

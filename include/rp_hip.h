@@ -192,7 +192,7 @@ int rp_hip_attention_forward(void* O, const void* Q, const void* K, const void* 
 
 /* Backward of rp_hip_attention_forward: dQ [batch, sq, d], dK and dV [batch, sk, d] (dense, overwritten) from the
  * forward's operands, its output O, its lse and the upstream gradient dO [batch, sq, d].  The probabilities are
- * recomputed on chip as exp(scale * q.k - lse); device memory beyond the operands is one float per query row, taken
+ * recomputed on chip as exp(scale * q.k - lse) in two launches (dQ, then dK and dV); device memory beyond the operands is one float per query row, taken
  * from and returned to the stream-ordered pool.  Same dtype, head-dimension, stride and alignment rules as the forward.
  * No counterpart in the reference, whose autograd runs backward_matmul_fn, backward_softmax_fn, backward_mul_scalar_fn
  * and backward_matmul_fn for the same values (ops/ops.c:6759-6814, 5665-5719, 5966-6020). */

@@ -37,7 +37,7 @@ constexpr int AT_KEYS = 32;                 // keys per step
 constexpr int AT_QROWS = 128;               // query rows per workgroup (32 per wave)
 
 template <typename T, int D>
-__global__ void __launch_bounds__(256) attention_fwd16_kernel(AttnArgs g) {
+__global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_fwd16_kernel(AttnArgs g) {
     static_assert(D % 32 == 0 && D <= 128, "head dimension: a multiple of 32 up to 128");
     constexpr int KS = D / 16;              // k-steps of the first product
     constexpr int DT = D / 32;              // 32-row tiles of O^T
@@ -140,15 +140,25 @@ __global__ void __launch_bounds__(256) attention_fwd16_kernel(AttnArgs g) {
         store_v(vr, vlds[(blk & 1) ^ 1]);
         load_v(vr, kb + 2 * AT_KEYS);
 
+        // this step's V^T fragments, requested before the softmax arithmetic that hides their latency
+        s16x8_t vfr[2][DT];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) vfr[t][dt] = read_v(stage, dt, t);
+
+#pragma unroll
+        for (int v = 0; v < 16; v++) st[v] *= sc;
+        if (kb + AT_KEYS > g.sk) {                          // the last block of a ragged sk
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+                if (kb + 8 * (v / 4) + 4 * h + (v % 4) >= g.sk) st[v] = -INFINITY;
+        }
         float mx = m_run;
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int key = kb + 8 * (v / 4) + 4 * h + (v % 4);
-            st[v] = key < g.sk ? st[v] * sc : -INFINITY;
-            mx = st[v] > mx ? st[v] : mx;
-        }
+        for (int v = 0; v < 16; v++) mx = fmaxf(st[v], mx);
         const float other = __shfl_xor(mx, 32, 64);         // the lane that holds this query's other 16 keys
-        mx = other > mx ? other : mx;
+        mx = fmaxf(other, mx);
         // a query row beyond sq (or a block of masked keys met first) keeps mx = -inf: exp2(-inf - -inf) must not produce NaN
         const float m_use = mx == -INFINITY ? 0.f : mx;
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
@@ -162,10 +172,12 @@ __global__ void __launch_bounds__(256) attention_fwd16_kernel(AttnArgs g) {
         }
         l_run = l_run * alpha + psum;
         m_run = mx;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {   // once the running maxima have settled there is nothing to rescale
 #pragma unroll
-        for (int dt = 0; dt < DT; dt++)
+            for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) ot[dt][v] *= alpha;
+                for (int v = 0; v < 16; v++) ot[dt][v] *= alpha;
+        }
         // O^T += V^T * P^T, 16 keys per MFMA
 #pragma unroll
         for (int t = 0; t < 2; t++) {
@@ -173,7 +185,7 @@ __global__ void __launch_bounds__(256) attention_fwd16_kernel(AttnArgs g) {
 #pragma unroll
             for (int e = 0; e < 8; e++) pb[e] = (short)p[8 * t + e].bits;
 #pragma unroll
-            for (int dt = 0; dt < DT; dt++) ot[dt] = mfma16_ops<T>::mma(read_v(stage, dt, t), pb, ot[dt]);
+            for (int dt = 0; dt < DT; dt++) ot[dt] = mfma16_ops<T>::mma(vfr[t][dt], pb, ot[dt]);
         }
         __syncthreads();                                    // next stage is written, this one is free
     };
@@ -205,7 +217,7 @@ __global__ void __launch_bounds__(256) attention_fwd16_kernel(AttnArgs g) {
 }
 
 // ============================================================================
-// Backward, two kernels plus a row-dot.  With P = softmax(scale * Q K^T), O = P V and upstream dO:
+// Backward, two kernels.  With P = softmax(scale * Q K^T), O = P V and upstream dO:
 //   Dq[q] = sum_d dO[q,d] O[q,d]
 //   dV = P^T dO          dP = dO V^T          dS = P o (dP - Dq) * scale          dQ = dS K          dK = dS^T Q
 // P is recomputed from the saved row-wise log-sum-exp: P = exp(scale * s - L[q]); nothing of size S x S is stored.
@@ -217,11 +229,11 @@ __global__ void __launch_bounds__(256) attention_fwd16_kernel(AttnArgs g) {
 // ============================================================================
 struct AttnBwdArgs {
     void* dQ; void* dK; void* dV;           // dense [batch, s, d]
-    const void* Q; const void* K; const void* V; const void* dO;
+    const void* Q; const void* K; const void* V; const void* O; const void* dO;
     const float* L;                         // [batch, sq] log-sum-exp rows from the forward
-    const float* Dq;                        // [batch, sq] row dots of dO and O
+    float* Dq;                              // [batch, sq] row dots of dO and O: written by the dQ kernel, read by the dK/dV kernel
     int batch, sq, sk;
-    long long q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, do_bs, do_rs;
+    long long q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs, do_bs, do_rs;
     float scale;
 };
 
@@ -274,32 +286,9 @@ __device__ __forceinline__ void attn_load_rows(s16x8_t (&f)[KS], const uint16_t*
     for (int ks = 0; ks < KS; ks++) f[ks] = __builtin_bit_cast(s16x8_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, 32 * ks, 0));
 }
 
-template <typename T>
-__global__ void __launch_bounds__(256) attention_rowdot_kernel(float* out, const T* a, const T* b, int rows, int d, long long a_bs, long long a_rs,
-                                                               long long b_bs, long long b_rs, int sq) {
-    // one row per 8 lanes: out[r] = sum_d a[r, d] * b[r, d], r = z * sq + q
-    const long long r = ((long long)blockIdx.x * 256 + threadIdx.x) >> 3;
-    const int part = threadIdx.x & 7;
-    float acc = 0.f;
-    if (r < rows) {
-        const long long z = r / sq, q = r % sq;
-        const T* pa = a + z * a_bs + q * a_rs;
-        const T* pb = b + z * b_bs + q * b_rs;
-        for (int i = part * 8; i < d; i += 64) {
-            u32x4_t ra = *(const u32x4_t*)(pa + i), rb = *(const u32x4_t*)(pb + i);
-            T va[8], vb[8];
-            memcpy(va, &ra, 16); memcpy(vb, &rb, 16);
-#pragma unroll
-            for (int e = 0; e < 8; e++) acc += widen(va[e]) * widen(vb[e]);
-        }
-    }
-    acc += __shfl_xor(acc, 1, 64); acc += __shfl_xor(acc, 2, 64); acc += __shfl_xor(acc, 4, 64);
-    if (r < rows && part == 0) out[r] = acc;
-}
-
 // dQ: a wave owns 32 queries and walks the keys.
 template <typename T, int D>
-__global__ void __launch_bounds__(256) attention_bwd_dq16_kernel(AttnBwdArgs g) {
+__global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_bwd_dq16_kernel(AttnBwdArgs g) {
     constexpr int KS = D / 16, DT = D / 32;
     using Blk = AttnBlock<D>;
     __shared__ __attribute__((aligned(16))) uint16_t klds[2][Blk::ELEMS];
@@ -323,7 +312,23 @@ __global__ void __launch_bounds__(256) attention_bwd_dq16_kernel(AttnBwdArgs g) 
     attn_load_rows<KS>(dof, dO, g.do_rs, q0, g.sq, do_end, c, h);
     const int q = q0 + c;
     const float lq = q < g.sq ? g.L[(long long)z * g.sq + q] * 1.44269504088896341f : 0.f;
-    const float dq_dot = q < g.sq ? g.Dq[(long long)z * g.sq + q] : 0.f;
+    // Dq[q] = sum_d dO[q, d] * O[q, d]: the lane holds 8 of every 16 d of its query, the lane 32 away the rest
+    float dq_dot = 0.f;
+    {
+        const uint16_t* O = (const uint16_t*)g.O + (long long)z * g.o_bs;
+        s16x8_t of[KS];
+        attn_load_rows<KS>(of, O, g.o_rs, q0, g.sq, (const char*)(O + ((long long)(g.sq - 1) * g.o_rs + D)), c, h);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                T a, b;
+                a.bits = (uint16_t)dof[ks][e]; b.bits = (uint16_t)of[ks][e];
+                dq_dot += widen(a) * widen(b);
+            }
+        dq_dot += __shfl_xor(dq_dot, 32, 64);
+        if (q < g.sq && h == 0) g.Dq[(long long)z * g.sq + q] = dq_dot;
+    }
 
     f32x16_t acc[DT];
 #pragma unroll
@@ -333,38 +338,45 @@ __global__ void __launch_bounds__(256) attention_bwd_dq16_kernel(AttnBwdArgs g) 
 
     const int tr0 = Blk::tr_base(lane);
     const int nblocks = (g.sk + AT_KEYS - 1) / AT_KEYS;
-    s16x8_t kf[2][KS], vf[2][KS];
+    s16x8_t kf[KS], vf[KS];                  // A operands: row = key kb + c; reloaded for the next block right after their last use
     u32x4_t kr[Blk::PIECES];
-    attn_load_rows<KS>(kf[0], K, g.k_rs, 0, g.sk, k_end, c, h);
-    attn_load_rows<KS>(vf[0], V, g.v_rs, 0, g.sk, v_end, c, h);
+    attn_load_rows<KS>(kf, K, g.k_rs, 0, g.sk, k_end, c, h);
+    attn_load_rows<KS>(vf, V, g.v_rs, 0, g.sk, v_end, c, h);
     Blk::load(kr, K, g.k_rs, 0, g.sk, k_end);
     Blk::store(kr, klds[0]);
-    attn_load_rows<KS>(kf[1], K, g.k_rs, AT_KEYS, g.sk, k_end, c, h);
-    attn_load_rows<KS>(vf[1], V, g.v_rs, AT_KEYS, g.sk, v_end, c, h);
     Blk::load(kr, K, g.k_rs, AT_KEYS, g.sk, k_end);
     __syncthreads();
 
-    auto step = [&](int blk, auto slotc) {
-        constexpr int SLOT = decltype(slotc)::value;
+    auto step = [&](int blk) {
         const int kb = blk * AT_KEYS;
         const uint16_t* stage = klds[blk & 1];
         f32x16_t st, dp;
 #pragma unroll
         for (int v = 0; v < 16; v++) { st[v] = 0.f; dp[v] = 0.f; }
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) st = mfma16_ops<T>::mma(kf[SLOT][ks], qf[ks], st);        // S^T: keys x queries
+        for (int ks = 0; ks < KS; ks++) st = mfma16_ops<T>::mma(kf[ks], qf[ks], st);        // S^T: keys x queries
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) dp = mfma16_ops<T>::mma(vf[SLOT][ks], dof[ks], dp);       // dP^T
-        attn_load_rows<KS>(kf[SLOT], K, g.k_rs, kb + 2 * AT_KEYS, g.sk, k_end, c, h);
-        attn_load_rows<KS>(vf[SLOT], V, g.v_rs, kb + 2 * AT_KEYS, g.sk, v_end, c, h);
+        for (int ks = 0; ks < KS; ks++) dp = mfma16_ops<T>::mma(vf[ks], dof[ks], dp);       // dP^T
+        attn_load_rows<KS>(kf, K, g.k_rs, kb + AT_KEYS, g.sk, k_end, c, h);
+        attn_load_rows<KS>(vf, V, g.v_rs, kb + AT_KEYS, g.sk, v_end, c, h);
+        // this step's K^T fragments, requested before the arithmetic that hides their latency
+        s16x8_t ktf[2][DT];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) ktf[t][dt] = Blk::read_tr(stage, tr0, dt, t);
         Blk::store(kr, klds[(blk & 1) ^ 1]);
         Blk::load(kr, K, g.k_rs, kb + 2 * AT_KEYS, g.sk, k_end);
         T ds[16];
 #pragma unroll
         for (int v = 0; v < 16; v++) {
-            const int key = kb + 8 * (v / 4) + 4 * h + (v % 4);
-            const float p = key < g.sk ? widen(narrow<T>(__builtin_amdgcn_exp2f(st[v] * sc - lq))) : 0.f;     // the P the forward multiplied with
+            const float p = widen(narrow<T>(__builtin_amdgcn_exp2f(st[v] * sc - lq)));     // the P the forward multiplied with
             ds[v] = narrow<T>(p * (dp[v] - dq_dot) * g.scale);
+        }
+        if (kb + AT_KEYS > g.sk) {                          // the last block of a ragged sk: keys past the end count for nothing
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+                if (kb + 8 * (v / 4) + 4 * h + (v % 4) >= g.sk) ds[v].bits = 0;
         }
 #pragma unroll
         for (int t = 0; t < 2; t++) {
@@ -372,14 +384,11 @@ __global__ void __launch_bounds__(256) attention_bwd_dq16_kernel(AttnBwdArgs g) 
 #pragma unroll
             for (int e = 0; e < 8; e++) dsb[e] = (short)ds[8 * t + e].bits;
 #pragma unroll
-            for (int dt = 0; dt < DT; dt++) acc[dt] = mfma16_ops<T>::mma(Blk::read_tr(stage, tr0, dt, t), dsb, acc[dt]);      // dQ^T += K^T dS^T
+            for (int dt = 0; dt < DT; dt++) acc[dt] = mfma16_ops<T>::mma(ktf[t][dt], dsb, acc[dt]);      // dQ^T += K^T dS^T
         }
         __syncthreads();
     };
-    for (int blk = 0; blk < nblocks; blk += 2) {
-        step(blk, std::integral_constant<int, 0>{});
-        if (blk + 1 < nblocks) step(blk + 1, std::integral_constant<int, 1>{});
-    }
+    for (int blk = 0; blk < nblocks; blk++) step(blk);
     if (q < g.sq) {
         T* row = (T*)g.dQ + ((long long)z * g.sq + q) * D;
 #pragma unroll
@@ -433,45 +442,48 @@ __global__ void __launch_bounds__(256) attention_bwd_dkv16_kernel(AttnBwdArgs g)
 
     const int tr0 = Blk::tr_base(lane);
     const int nblocks = (g.sq + AT_KEYS - 1) / AT_KEYS;
-    s16x8_t qf[2][KS], dof[2][KS];           // A operands: row = query qb + c
+    s16x8_t qf[KS], dof[KS];                 // A operands: row = query qb + c; reloaded for the next block right after their last use
     u32x4_t qr[Blk::PIECES], dor[Blk::PIECES];
-    float rowv = 0.f;                        // threads 0..31: L of query qb + t; 32..63: Dq of query qb + t - 32
+    // L and Dq of the block's 32 queries: every lane requests query qb + lane % 32 (buffer loads, zero past sq, so
+    // that no branch surrounds them and the wait for them can be counted); wave 0 puts them in LDS: its lower half
+    // the L (in log2 units, +inf past sq, which makes those rows' probabilities exactly 0), its upper half the Dq
+    const __amdgpu_buffer_rsrc_t l_rsrc = m16_rsrc(Lz, (long long)g.sq * 4), d_rsrc = m16_rsrc(Dz, (long long)g.sq * 4);
+    float row_l = 0.f, row_d = 0.f;
     auto load_rowv = [&](int qb) {
-        const int t = threadIdx.x, qq = qb + (t & 31);
-        rowv = (t < 64 && qq < g.sq) ? (t < 32 ? Lz[qq] * 1.44269504088896341f : Dz[qq]) : 0.f;
+        row_l = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(l_rsrc, (qb + c) * 4, 0, 0));
+        row_d = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(d_rsrc, (qb + c) * 4, 0, 0));
     };
-    auto store_rowv = [&](int stage) { if (threadIdx.x < 64) rowlds[stage][threadIdx.x >> 5][threadIdx.x & 31] = rowv; };
-    attn_load_rows<KS>(qf[0], Q, g.q_rs, 0, g.sq, q_end, c, h);
-    attn_load_rows<KS>(dof[0], dO, g.do_rs, 0, g.sq, do_end, c, h);
+    auto store_rowv = [&](int stage, int qb) {
+        if (wave == 0) rowlds[stage][h][c] = h ? row_d : (qb + c < g.sq ? row_l * 1.44269504088896341f : INFINITY);
+    };
+    attn_load_rows<KS>(qf, Q, g.q_rs, 0, g.sq, q_end, c, h);
+    attn_load_rows<KS>(dof, dO, g.do_rs, 0, g.sq, do_end, c, h);
     Blk::load(qr, Q, g.q_rs, 0, g.sq, q_end);
     Blk::load(dor, dO, g.do_rs, 0, g.sq, do_end);
     load_rowv(0);
     Blk::store(qr, qlds[0]);
     Blk::store(dor, dolds[0]);
-    store_rowv(0);
-    attn_load_rows<KS>(qf[1], Q, g.q_rs, AT_KEYS, g.sq, q_end, c, h);
-    attn_load_rows<KS>(dof[1], dO, g.do_rs, AT_KEYS, g.sq, do_end, c, h);
+    store_rowv(0, 0);
     Blk::load(qr, Q, g.q_rs, AT_KEYS, g.sq, q_end);
     Blk::load(dor, dO, g.do_rs, AT_KEYS, g.sq, do_end);
     load_rowv(AT_KEYS);
     __syncthreads();
 
-    auto step = [&](int blk, auto slotc) {
-        constexpr int SLOT = decltype(slotc)::value;
+    auto step = [&](int blk) {
         const int qb = blk * AT_KEYS;
         const int cur = blk & 1;
         f32x16_t st, dp;
 #pragma unroll
         for (int v = 0; v < 16; v++) { st[v] = 0.f; dp[v] = 0.f; }
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) st = mfma16_ops<T>::mma(qf[SLOT][ks], kf[ks], st);        // S: queries x keys
+        for (int ks = 0; ks < KS; ks++) st = mfma16_ops<T>::mma(qf[ks], kf[ks], st);        // S: queries x keys
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) dp = mfma16_ops<T>::mma(dof[SLOT][ks], vf[ks], dp);       // dP
-        attn_load_rows<KS>(qf[SLOT], Q, g.q_rs, qb + 2 * AT_KEYS, g.sq, q_end, c, h);
-        attn_load_rows<KS>(dof[SLOT], dO, g.do_rs, qb + 2 * AT_KEYS, g.sq, do_end, c, h);
+        for (int ks = 0; ks < KS; ks++) dp = mfma16_ops<T>::mma(dof[ks], vf[ks], dp);       // dP
+        attn_load_rows<KS>(qf, Q, g.q_rs, qb + AT_KEYS, g.sq, q_end, c, h);
+        attn_load_rows<KS>(dof, dO, g.do_rs, qb + AT_KEYS, g.sq, do_end, c, h);
         Blk::store(qr, qlds[cur ^ 1]);
         Blk::store(dor, dolds[cur ^ 1]);
-        store_rowv(cur ^ 1);
+        store_rowv(cur ^ 1, qb + AT_KEYS);
         Blk::load(qr, Q, g.q_rs, qb + 2 * AT_KEYS, g.sq, q_end);
         Blk::load(dor, dO, g.do_rs, qb + 2 * AT_KEYS, g.sq, do_end);
         load_rowv(qb + 2 * AT_KEYS);
@@ -483,9 +495,8 @@ __global__ void __launch_bounds__(256) attention_bwd_dkv16_kernel(AttnBwdArgs g)
             const f32x4_t d4 = *(const f32x4_t*)&rowlds[cur][1][8 * v4 + 4 * h];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const int v = 4 * v4 + e, qrow = qb + 8 * v4 + 4 * h + e;
-                const float pe = qrow < g.sq ? __builtin_amdgcn_exp2f(st[v] * sc - l4[e]) : 0.f;
-                p[v] = narrow<T>(pe);
+                const int v = 4 * v4 + e;
+                p[v] = narrow<T>(__builtin_amdgcn_exp2f(st[v] * sc - l4[e]));          // 0 for a query past sq: its L is +inf
                 ds[v] = narrow<T>(widen(p[v]) * (dp[v] - d4[e]) * g.scale);
             }
         }
@@ -502,10 +513,7 @@ __global__ void __launch_bounds__(256) attention_bwd_dkv16_kernel(AttnBwdArgs g)
         }
         __syncthreads();
     };
-    for (int blk = 0; blk < nblocks; blk += 2) {
-        step(blk, std::integral_constant<int, 0>{});
-        if (blk + 1 < nblocks) step(blk + 1, std::integral_constant<int, 1>{});
-    }
+    for (int blk = 0; blk < nblocks; blk++) step(blk);
     const int key = k0 + c;
     if (key < g.sk) {
         T* krow = (T*)g.dK + ((long long)z * g.sk + key) * D;
@@ -604,24 +612,15 @@ extern "C" int rp_hip_attention_backward(void* dQ, void* dK, void* dV, const voi
     const long long strides[] = {q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs, do_bs, do_rs};
     for (long long s : strides)
         if (s < 0 || s % 8) { set_error("rp_hip_attention_backward: strides must be non-negative multiples of 8 elements"); return -1; }
-    if (q_rs >= (1ll << 22) || k_rs >= (1ll << 22) || v_rs >= (1ll << 22) || do_rs >= (1ll << 22)) { set_error("rp_hip_attention_backward: row stride too large"); return -1; }
+    if (q_rs >= (1ll << 22) || k_rs >= (1ll << 22) || v_rs >= (1ll << 22) || o_rs >= (1ll << 22) || do_rs >= (1ll << 22)) { set_error("rp_hip_attention_backward: row stride too large"); return -1; }
     if (((uintptr_t)dQ | (uintptr_t)dK | (uintptr_t)dV | (uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)O | (uintptr_t)dO) & 15) {
         set_error("rp_hip_attention_backward: operands must be 16-byte aligned");
         return -1;
     }
     void* dots = nullptr;
     if (rp_hip_malloc(&dots, (size_t)batch * sq * sizeof(float)) != 0) return -1;
-    const int rows = batch * sq;
-    const unsigned blocks = (unsigned)(((long long)rows * 8 + 255) / 256);
-    if (dtype == RP_DTYPE_BFLOAT16)
-        hipLaunchKernelGGL(attention_rowdot_kernel<bf16_t>, dim3(blocks), dim3(256), 0, current_stream(), (float*)dots, (const bf16_t*)dO, (const bf16_t*)O, rows, d, do_bs, do_rs, o_bs, o_rs, sq);
-    else
-        hipLaunchKernelGGL(attention_rowdot_kernel<f16_t>, dim3(blocks), dim3(256), 0, current_stream(), (float*)dots, (const f16_t*)dO, (const f16_t*)O, rows, d, do_bs, do_rs, o_bs, o_rs, sq);
-    int rc = check_launch("attention_rowdot_kernel") ? 0 : -1;
-    if (rc == 0) {
-        AttnBwdArgs g{dQ, dK, dV, Q, K, V, dO, lse, (const float*)dots, batch, sq, sk, q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, do_bs, do_rs, (float)scale};
-        rc = dtype == RP_DTYPE_BFLOAT16 ? launch_attention_bwd_t<bf16_t>(g, d) : launch_attention_bwd_t<f16_t>(g, d);
-    }
+    AttnBwdArgs g{dQ, dK, dV, Q, K, V, O, dO, lse, (float*)dots, batch, sq, sk, q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs, do_bs, do_rs, (float)scale};
+    const int rc = dtype == RP_DTYPE_BFLOAT16 ? launch_attention_bwd_t<bf16_t>(g, d) : launch_attention_bwd_t<f16_t>(g, d);
     rp_hip_free(dots);        // stream-ordered reuse: the pool hands it out again only to later work on this stream
     return rc;
 }

@@ -751,7 +751,7 @@ void backward_mul_scalar_fn(GradFn* self, Tensor* grad_output) {     // referenc
     free_tensor(gd);
 }
 
-// Backward of op_attention in three launches (rp_hip_attention_backward): the probabilities are recomputed tile by
+// Backward of op_attention in two launches (rp_hip_attention_backward): the probabilities are recomputed tile by
 // tile from the row-wise log-sum-exp the forward saved, so nothing of size sq x sk is allocated.  The values are those
 // of the chain the reference's autograd runs for matmul -> mul_scalar -> softmax -> matmul (ops/ops.c:6759-6814,
 // 5966-6020, 5665-5719): dV = P^T dO, dP = dO V^T, dS = softmax'(dP) * scale, dQ = dS K, dK = dS^T Q.
