@@ -177,6 +177,36 @@ int rp_hip_reduce_rows(void* out, const void* grad, int rows, int cols, int accu
 int rp_hip_cross_entropy_mean(void* loss_out, void* grad_logits, const void* logits, const int* targets,
                               int batch, int classes, double upstream, int dtype);
 
+/* ---- conv2d lowering (the callers of the GEMM in op_conv2d, ops/ops.c:4723-4870 and 4473-4720) ---- */
+
+/* Same contract as the reference's single-sample entry points (functional/functional.h:183-190,
+ * functional/functional_device.cu:1723-1761): col [C_in*kH*kW, out_H*out_W] row-major from im [C_in, H, W], and
+ * the adjoint, which ADDS col's entries into im (the reference zeroes im first, ops/ops.c:4541).  col2im here is a
+ * gather in (kh, kw) order with one rounding, i.e. the value of the reference's host path
+ * (functional/functional.c:885-912), where the reference's device kernel scatters with atomicAdd. */
+int im2col_kernel_device(void* col, const void* im, int C_in, int H, int W, int kH, int kW, int stride_h, int stride_w,
+                         int pad_h, int pad_w, int dilation_h, int dilation_w, int out_H, int out_W, int dtype);
+int col2im_kernel_device(void* im, const void* col, int C_in, int H, int W, int kH, int kW, int stride_h, int stride_w,
+                         int pad_h, int pad_w, int dilation_h, int dilation_w, int out_H, int out_W, int dtype);
+
+/* The same for a whole batch in one launch: im [batch, C_in, H, W], col [batch, C_in*kH*kW, out_H*out_W].  This is what
+ * lets op_conv2d replace the reference's per-sample loop of im2col + rp_matmul (ops/ops.c:4759-4770) with one
+ * lowering and one rp_hip_gemm_strided_batched call.  accumulate = 0 overwrites im, 1 adds to it. */
+int rp_hip_im2col_batched(void* col, const void* im, int batch, int C_in, int H, int W, int kH, int kW,
+                          int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h, int dilation_w,
+                          int out_H, int out_W, int dtype);
+int rp_hip_col2im_batched(void* im, const void* col, int batch, int C_in, int H, int W, int kH, int kW,
+                          int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h, int dilation_w,
+                          int out_H, int out_W, int accumulate, int dtype);
+
+/* y[n, c, :] += bias[c] for y [batch, channels, hw]: the reference pulls y to the host for this loop
+ * (ops/ops.c:4772-4836). */
+int rp_hip_channel_bias_add(void* y, const void* bias, int batch, int channels, int hw, int dtype);
+
+/* out[c] (+)= sum over n and hw of grad[n, c, hw], accumulated in float32 (float64 for float64): the bias gradient
+ * that the reference sums on the host (ops/ops.c:4620-4716). */
+int rp_hip_channel_sums(void* out, const void* grad, int batch, int channels, int hw, int accumulate, int dtype);
+
 /* Fused attention forward for bfloat16 / float16: O[b] = softmax(scale * Q[b] * K[b]^T) * V[b], the score matrix never
  * leaves the chip.  Q, O: [batch, sq, d]; K, V: [batch, sk, d]; d in {32, 64, 128} and contiguous (unit stride);
  * *_bs / *_rs are the batch and row strides in elements (multiples of 8; operands 16-byte aligned).

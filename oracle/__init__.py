@@ -65,6 +65,8 @@ _sum_all = _sig("orc_sum_all", _i, _vp, _vp, _sz, _i)
 _reduce_rows = _sig("orc_reduce_rows", _i, _vp, _vp, _i, _i, _i)
 _contig = _sig("orc_contiguous_copy", _i, _vp, _vp, _i, _ip, _llp, _i)
 _ce = _sig("orc_cross_entropy_mean", _i, _vp, _vp, _vp, _ip, _i, _i, _d, _i)
+_im2col = _sig("orc_im2col", _i, _vp, _vp, *([_i] * 14))
+_col2im = _sig("orc_col2im", _i, _vp, _vp, *([_i] * 14))
 _widen = _sig("orc_widen", None, _vp, _vp, _sz, _i)
 _narrow = _sig("orc_narrow", None, _vp, _vp, _sz, _i)
 
@@ -302,6 +304,83 @@ def attention(q, k, v, dtype, scale=0.125, d_out=None):
     return {"S": s, "P": p, "O": o, "dQ": dq, "dK": dk, "dV": dv}
 
 
+def conv_out_size(size, k, stride, pad, dilation):
+    """reference ops/ops.c:4740-4741."""
+    return (size + 2 * pad - dilation * (k - 1) - 1) // stride + 1
+
+
+def im2col(im, kernel, stride, pad, dilation, dtype):
+    """im [C, H, W] -> col [C*kH*kW, oH*oW] (reference functional/functional.c:855-883)."""
+    im = np.ascontiguousarray(im)
+    C, H, W = im.shape
+    (kH, kW), (sh, sw), (ph, pw), (dh, dw) = kernel, stride, pad, dilation
+    oH, oW = conv_out_size(H, kH, sh, ph, dh), conv_out_size(W, kW, sw, pw, dw)
+    col = np.empty((C * kH * kW, oH * oW), dtype=NP_STORAGE[dtype])
+    _check(_im2col(_ptr(col), _ptr(im), C, H, W, kH, kW, sh, sw, ph, pw, dh, dw, oH, oW, dtype), "im2col")
+    return col
+
+
+def col2im(im, col, kernel, stride, pad, dilation, dtype):
+    """Adds col [C*kH*kW, oH*oW] into a copy of im [C, H, W] (reference functional/functional.c:885-913)."""
+    im = np.array(im, copy=True, order="C")
+    col = np.ascontiguousarray(col)
+    C, H, W = im.shape
+    (kH, kW), (sh, sw), (ph, pw), (dh, dw) = kernel, stride, pad, dilation
+    oH, oW = conv_out_size(H, kH, sh, ph, dh), conv_out_size(W, kW, sw, pw, dw)
+    assert col.shape == (C * kH * kW, oH * oW)
+    _check(_col2im(_ptr(im), _ptr(col), C, H, W, kH, kW, sh, sw, ph, pw, dh, dw, oH, oW, dtype), "col2im")
+    return im
+
+
+def conv2d_forward(x, w, bias, stride, pad, dilation, dtype):
+    """reference ops/ops.c:4723-4836: per sample im2col + matmul, then y[n, c] += bias[c] with one rounding."""
+    N, C, H, W = x.shape
+    Co, _, kH, kW = w.shape
+    oH, oW = conv_out_size(H, kH, stride[0], pad[0], dilation[0]), conv_out_size(W, kW, stride[1], pad[1], dilation[1])
+    w2 = np.ascontiguousarray(w).reshape(Co, C * kH * kW)
+    y = np.empty((N, Co, oH * oW), dtype=NP_STORAGE[dtype])
+    for n in range(N):
+        y[n] = matmul(w2, im2col(x[n], (kH, kW), stride, pad, dilation, dtype), dtype)
+    if bias is not None:
+        b = np.ascontiguousarray(np.broadcast_to(np.asarray(bias)[None, :, None], y.shape))
+        y = add(y, b, dtype)
+    return y.reshape(N, Co, oH, oW)
+
+
+def conv2d_backward(x, w, dy, stride, pad, dilation, dtype, with_bias=True):
+    """reference ops/ops.c:4473-4720.  Returns (dx, dw, db), each the first gradient written into a zeroed buffer:
+    dx[n] = 0 + col2im(W^T dy[n]); dw = ((0 + dy[0] col[0]^T) + dy[1] col[1]^T) + ... with a rounding per add;
+    db = the float32 (float64 for float64) sum over n, c-major, hw, added to zero."""
+    N, C, H, W = x.shape
+    Co, _, kH, kW = w.shape
+    oH, oW = dy.shape[2], dy.shape[3]
+    w2 = np.ascontiguousarray(w).reshape(Co, C * kH * kW)
+    wt = np.ascontiguousarray(w2.T)
+    dy2 = np.ascontiguousarray(dy).reshape(N, Co, oH * oW)
+    zero_im = np.zeros((C, H, W), dtype=NP_STORAGE[dtype])
+    dx = np.zeros(x.shape, dtype=NP_STORAGE[dtype])
+    dw = np.zeros(w2.shape, dtype=NP_STORAGE[dtype])
+    for n in range(N):
+        dcol = matmul(wt, dy2[n], dtype)
+        dx[n] = add(dx[n], col2im(zero_im, dcol, (kH, kW), stride, pad, dilation, dtype), dtype)
+        col_t = np.ascontiguousarray(im2col(x[n], (kH, kW), stride, pad, dilation, dtype).T)
+        dw = add(dw, matmul(dy2[n], col_t, dtype), dtype)
+    db = None
+    if with_bias:
+        if dtype == F64:
+            acc = np.zeros(Co, dtype=np.float64)
+            g = dy2
+        else:
+            acc = np.zeros(Co, dtype=np.float32)
+            g = dy2 if dtype == F32 else widen(dy2, dtype)
+        for n in range(N):
+            for c in range(Co):
+                for v in g[n, c]:
+                    acc[c] += v
+        db = acc if dtype in (F32, F64) else narrow(acc, dtype)       # zeros + sum, one rounding for 16-bit
+    return dx, dw.reshape(w.shape), db
+
+
 def matmul_f64(a, b, dtype):
     """The float64 oracle: exact inputs of `dtype`, float64 numpy product."""
     return to_f64(a, dtype) @ to_f64(b, dtype)
@@ -327,6 +406,11 @@ def load_reference():
         fn = getattr(ref, name)
         fn.restype = _i
         fn.argtypes = [_vp, _vp, _vp, _i, _i, _i]
+    for name in ("im2col_kernel_host_f32", "im2col_kernel_host_f64", "col2im_kernel_host_f32", "col2im_kernel_host_f64"):
+        if hasattr(ref, name):
+            fn = getattr(ref, name)
+            fn.restype = _i
+            fn.argtypes = [_vp, _vp] + [_i] * 13
     return ref
 
 

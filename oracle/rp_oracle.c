@@ -580,3 +580,86 @@ done:
     free(lp); free(sm);
     return rc;
 }
+
+/* ---------------------------------------------------------------------------
+ * conv2d lowering.  reference functional/functional_host.c:1237-1262 (im2col)
+ * and 1291-1313 (col2im, which ADDS into im); 16-bit through the fp32 pivot with
+ * one narrowing at the end (functional/functional.c:866-879, 896-911).
+ * Written as a gather per destination element rather than the reference's
+ * five nested loops; for col2im the contributions to one pixel still arrive in
+ * ascending (kh, kw) order, which is the order the reference's loops visit them.
+ * ------------------------------------------------------------------------- */
+#define ORC_IM2COL(NAME, TYPE)                                                                          \
+    static void NAME(TYPE* col, const TYPE* im, int C, int H, int W, int kH, int kW, int sh, int sw,   \
+                     int ph, int pw, int dh, int dw, int oH, int oW) {                                  \
+        size_t cols = (size_t)oH * oW;                                                                  \
+        for (int r = 0; r < C * kH * kW; r++) {                                                         \
+            int kw = r % kW, kh = (r / kW) % kH, c = r / (kW * kH);                                     \
+            for (int oh = 0; oh < oH; oh++)                                                             \
+                for (int ow = 0; ow < oW; ow++) {                                                       \
+                    int h = oh * sh + kh * dh - ph, w = ow * sw + kw * dw - pw;                         \
+                    int inside = h >= 0 && h < H && w >= 0 && w < W;                                    \
+                    col[r * cols + (size_t)oh * oW + ow] = inside ? im[((size_t)c * H + h) * W + w] : (TYPE)0; \
+                }                                                                                       \
+        }                                                                                               \
+    }
+ORC_IM2COL(orc_im2col_f32, float)
+ORC_IM2COL(orc_im2col_f64, double)
+
+#define ORC_COL2IM(NAME, TYPE)                                                                          \
+    static void NAME(TYPE* im, const TYPE* col, int C, int H, int W, int kH, int kW, int sh, int sw,   \
+                     int ph, int pw, int dh, int dw, int oH, int oW) {                                  \
+        size_t cols = (size_t)oH * oW;                                                                  \
+        for (int c = 0; c < C; c++)                                                                     \
+            for (int h = 0; h < H; h++)                                                                 \
+                for (int w = 0; w < W; w++) {                                                           \
+                    TYPE acc = im[((size_t)c * H + h) * W + w];                                         \
+                    for (int kh = 0; kh < kH; kh++)                                                     \
+                        for (int kw = 0; kw < kW; kw++) {                                               \
+                            int hh = h + ph - kh * dh, ww = w + pw - kw * dw;                           \
+                            if (hh < 0 || ww < 0 || hh % sh || ww % sw) continue;                       \
+                            int oh = hh / sh, ow = ww / sw;                                             \
+                            if (oh >= oH || ow >= oW) continue;                                         \
+                            acc += col[((size_t)(c * kH + kh) * kW + kw) * cols + (size_t)oh * oW + ow]; \
+                        }                                                                               \
+                    im[((size_t)c * H + h) * W + w] = acc;                                              \
+                }                                                                                       \
+    }
+ORC_COL2IM(orc_col2im_f32, float)
+ORC_COL2IM(orc_col2im_f64, double)
+
+int orc_im2col(void* col, const void* im, int C, int H, int W, int kH, int kW, int sh, int sw,
+               int ph, int pw, int dh, int dw, int oH, int oW, int dtype) {
+    if (!col || !im) return -1;
+    size_t nim = (size_t)C * H * W, ncol = (size_t)C * kH * kW * oH * oW;
+    if (dtype == ORC_F32) { orc_im2col_f32((float*)col, (const float*)im, C, H, W, kH, kW, sh, sw, ph, pw, dh, dw, oH, oW); return 0; }
+    if (dtype == ORC_F64) { orc_im2col_f64((double*)col, (const double*)im, C, H, W, kH, kW, sh, sw, ph, pw, dh, dw, oH, oW); return 0; }
+    if (dtype != ORC_F16 && dtype != ORC_BF16) return -1;
+    float* a = (float*)malloc(nim * 4);
+    float* b = (float*)malloc(ncol * 4);
+    if (!a || !b) { free(a); free(b); return -1; }
+    orc_widen(im, a, nim, dtype);
+    orc_im2col_f32(b, a, C, H, W, kH, kW, sh, sw, ph, pw, dh, dw, oH, oW);
+    orc_narrow(b, col, ncol, dtype);
+    free(a); free(b);
+    return 0;
+}
+
+int orc_col2im(void* im, const void* col, int C, int H, int W, int kH, int kW, int sh, int sw,
+               int ph, int pw, int dh, int dw, int oH, int oW, int dtype) {
+    if (!col || !im) return -1;
+    size_t nim = (size_t)C * H * W, ncol = (size_t)C * kH * kW * oH * oW;
+    if (dtype == ORC_F32) { orc_col2im_f32((float*)im, (const float*)col, C, H, W, kH, kW, sh, sw, ph, pw, dh, dw, oH, oW); return 0; }
+    if (dtype == ORC_F64) { orc_col2im_f64((double*)im, (const double*)col, C, H, W, kH, kW, sh, sw, ph, pw, dh, dw, oH, oW); return 0; }
+    if (dtype != ORC_F16 && dtype != ORC_BF16) return -1;
+    float* a = (float*)malloc(nim * 4);
+    float* b = (float*)malloc(ncol * 4);
+    if (!a || !b) { free(a); free(b); return -1; }
+    orc_widen(im, a, nim, dtype);
+    orc_widen(col, b, ncol, dtype);
+    orc_col2im_f32(a, b, C, H, W, kH, kW, sh, sw, ph, pw, dh, dw, oH, oW);
+    orc_narrow(a, im, nim, dtype);
+    free(a); free(b);
+    return 0;
+}
+

@@ -67,6 +67,12 @@ SIGNATURES = {
     "rp_hip_convert": (_i, [_vp, _i, _vp, _i, _sz]),
     "rp_hip_reduce_rows": (_i, [_vp, _vp, _i, _i, _i, _i]),
     "rp_hip_cross_entropy_mean": (_i, [_vp, _vp, _vp, _vp, _i, _i, _d, _i]),
+    "im2col_kernel_device": (_i, [_vp, _vp] + [_i] * 14),
+    "col2im_kernel_device": (_i, [_vp, _vp] + [_i] * 14),
+    "rp_hip_im2col_batched": (_i, [_vp, _vp] + [_i] * 15),
+    "rp_hip_col2im_batched": (_i, [_vp, _vp] + [_i] * 16),
+    "rp_hip_channel_bias_add": (_i, [_vp, _vp, _i, _i, _i, _i]),
+    "rp_hip_channel_sums": (_i, [_vp, _vp, _i, _i, _i, _i, _i]),
     "rp_hip_attention_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i] + [_ll] * 8 + [_d, _i]),
     "rp_hip_attention_backward": (_i, [_vp] * 9 + [_i] * 4 + [_ll] * 10 + [_d, _i]),
 }

@@ -1,10 +1,10 @@
-"""`recpulse` — the Python layer of the drop-in: Module and Linear over `recpulse_cuda`.
+"""`recpulse` — the Python layer of the drop-in: Module, Linear and Conv2d over `recpulse_cuda`.
 
 Only the layers whose cost is the matmul path are provided here; the behaviour
 each one keeps is cited in `recpulse.module`.
 """
 __version__ = "0.2.0b1+mi355x"
 
-from recpulse.module import Linear, Module
+from recpulse.module import Conv2d, Linear, Module
 
-__all__ = ["Module", "Linear"]
+__all__ = ["Module", "Linear", "Conv2d"]

@@ -1,4 +1,4 @@
-"""Parameter bookkeeping (`Module`) and the affine layer (`Linear`).
+"""Parameter bookkeeping (`Module`), the affine layer (`Linear`) and the convolution layer (`Conv2d`).
 
 Behaviour kept from the reference's recpulse/module.py:
   * a module records its parameters in `tracked` under their attribute names; assigning a
@@ -9,7 +9,10 @@ Behaviour kept from the reference's recpulse/module.py:
   * `load_state()` copies by name and ignores unknown names (:62-71);
   * `Linear` stores its weight as [in_features, out_features] (not transposed), initialised
     N(0, 1/in_features), bias zeros (:91-108), and computes x·W then + bias (:110-114).
-The forward pass issues ONE launch (GEMM with the bias add in its epilogue) through
+  * `Conv2d` stores its weight as [out_channels, in_channels, kH, kW], initialised
+    N(0, 1/(in_channels*kH*kW)), bias zeros, and accepts ints or pairs for kernel size, stride,
+    padding and dilation (:117-155).
+The Linear forward pass issues ONE launch (GEMM with the bias add in its epilogue) through
 `Tensor.op_linear`; the two-op form the reference uses gives the same values and is kept as
 `forward_two_ops` for comparison.
 """
@@ -119,3 +122,27 @@ class Linear(Module):
     def forward_two_ops(self, x):
         out = self.keep(x.op_matmul(self.weight))
         return out if self.bias is None else self.keep(out.op_add(self.bias))
+
+
+def _pair(value):
+    return (value, value) if isinstance(value, int) else tuple(value)
+
+
+class Conv2d(Module):
+    """y = conv2d(x, W) + b over x [N, in_channels, H, W] with W [out_channels, in_channels, kH, kW]."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1, bias=True):
+        super().__init__()
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.kernel_size, self.stride, self.padding, self.dilation = _pair(kernel_size), _pair(stride), _pair(padding), _pair(dilation)
+        kh, kw = self.kernel_size
+        fan_in = in_channels * kh * kw
+        init = rp.randn([out_channels, in_channels, kh, kw]).mul_scalar(1.0 / math.sqrt(fan_in))
+        self.weight = self.track("weight", init.requires_grad_(True))
+        self.bias = self.track("bias", rp.zeros([out_channels]).requires_grad_(True)) if bias else None
+
+    def forward(self, x):
+        return self.keep(x.op_conv2d(self.weight, bias=self.bias, stride_h=self.stride[0], stride_w=self.stride[1],
+                                     pad_h=self.padding[0], pad_w=self.padding[1],
+                                     dilation_h=self.dilation[0], dilation_w=self.dilation[1]))
+

@@ -180,6 +180,10 @@ PYBIND11_MODULE(recpulse_cuda, m) {
         .def("op_linear", [](PyTensor& x, PyTensor& w, py::object bias) {
             return wrap(op_linear(x.t, w.t, bias.is_none() ? nullptr : bias.cast<PyTensor&>().t), "op_linear");
         }, py::arg("weight"), py::arg("bias") = py::none())
+        .def("op_conv2d", [](PyTensor& x, PyTensor& w, py::object bias, int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h, int dilation_w) {
+            return wrap(op_conv2d(x.t, w.t, bias.is_none() ? nullptr : bias.cast<PyTensor&>().t, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w), "op_conv2d");
+        }, py::arg("weight"), py::arg("bias") = py::none(), py::arg("stride_h") = 1, py::arg("stride_w") = 1, py::arg("pad_h") = 0, py::arg("pad_w") = 0,
+             py::arg("dilation_h") = 1, py::arg("dilation_w") = 1)        // reference python/tensor_python.c:1139-1171
         .def("op_attention", [](PyTensor& q, PyTensor& k, PyTensor& v, double scale) { return wrap(op_attention(q.t, k.t, v.t, scale), "op_attention"); },
              py::arg("k"), py::arg("v"), py::arg("scale"))
         .def("op_add", [](PyTensor& a, PyTensor& b) { return wrap(op_add(a.t, b.t), "op_add"); })

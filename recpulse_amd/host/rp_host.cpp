@@ -787,6 +787,90 @@ void backward_attention_fn(GradFn* self, Tensor* grad_output) {
     free_tensor(g); free_tensor(od); free_tensor(qd); free_tensor(kd); free_tensor(vd);
 }
 
+// ---- conv2d ----------------------------------------------------------------------------
+// The reference lowers one sample at a time: im2col, rp_matmul, and for the gradients col2im or a densified transpose
+// per sample (ops/ops.c:4759-4770, 4533-4551, 4575-4617), with the bias and its gradient done on the host.  Here a
+// chunk of the batch is lowered at once and multiplied by one strided-batched GEMM whose weight operand has batch
+// stride 0 and whose transposes are stride views; the chunk keeps the lowered matrix under a fixed budget.
+struct ConvSaved { int sh, sw, ph, pw, dh, dw, N, C, H, W, Co, kH, kW, oH, oW; };
+
+long long conv_col_budget() {                            // bytes of lowered activations held at a time
+    const char* e = getenv("RP_CONV_COL_BYTES");         // read at every call: tests shrink it to force several chunks
+    const long long v = e ? atoll(e) : 0;
+    return v > 0 ? v : (2ll << 30);
+}
+
+int conv_chunk(const ConvSaved& c, size_t esz) {
+    const long long per_sample = (long long)c.C * c.kH * c.kW * c.oH * c.oW * (long long)esz;
+    long long n = conv_col_budget() / (per_sample > 0 ? per_sample : 1);
+    return (int)(n < 1 ? 1 : (n > c.N ? c.N : n));
+}
+
+bool conv_is_pointwise(const ConvSaved& c) {              // 1x1, unit stride, no padding: the activations are the lowered matrix
+    return c.kH == 1 && c.kW == 1 && c.sh == 1 && c.sw == 1 && c.ph == 0 && c.pw == 0;
+}
+
+int conv_lower(void* col, const void* x, int nb, const ConvSaved& c, DType dt) {
+    return rp_hip_im2col_batched(col, x, nb, c.C, c.H, c.W, c.kH, c.kW, c.sh, c.sw, c.ph, c.pw, c.dh, c.dw, c.oH, c.oW, dt);
+}
+
+void backward_conv2d_fn(GradFn* self, Tensor* grad_output) {         // reference ops/ops.c:4473-4720
+    Tensor* x = self->inputs[0]; Tensor* w = self->inputs[1];
+    Tensor* bias = self->num_inputs > 2 ? self->inputs[2] : nullptr;
+    const ConvSaved& c = *(ConvSaved*)self->saved_data;
+    if (!needs_grad(x) && !needs_grad(w) && !needs_grad(bias)) return;
+    if (!on_device(x->device_id)) { dev_fail("op_conv2d backward"); return; }
+    const DType dt = x->dtype;
+    const size_t esz = dtype_size(dt);
+    const int rows = c.C * c.kH * c.kW, cols = c.oH * c.oW;
+    const long long x_n = (long long)c.C * c.H * c.W, y_n = (long long)c.Co * cols, col_n = (long long)rows * cols;
+    const bool pointwise = conv_is_pointwise(c);
+    const int chunk = conv_chunk(c, esz);
+    Tensor* g = dense(grad_output);
+    Tensor* xd = dense(x); Tensor* wd = dense(w);
+    void* col = nullptr;
+    bool ok = g && xd && wd;
+    if (ok && !pointwise && (needs_grad(x) || needs_grad(w))) ok = rp_hip_malloc(&col, (size_t)chunk * col_n * esz) == 0;
+    if (ok && needs_grad(x)) {
+        // dcol[n] = W^T . dy[n], then each input pixel gathers its taps
+        Tensor* dx = empty_tensor(dt, x->device_id, x->ndim, x->shape);
+        bool good = dx != nullptr;
+        for (int n0 = 0; good && n0 < c.N; n0 += chunk) {
+            const int nb = c.N - n0 < chunk ? c.N - n0 : chunk;
+            char* dx_n = (char*)dx->data + n0 * x_n * esz;
+            const char* g_n = (const char*)g->data + n0 * y_n * esz;
+            good = rp_hip_gemm_strided_batched(pointwise ? (void*)dx_n : col, wd->data, g_n, nullptr, nb, rows, c.Co, cols,
+                                               0, 1, rows, y_n, cols, 1, col_n, cols, 1, 0, dt) == 0 &&
+                   (pointwise || rp_hip_col2im_batched(dx_n, col, nb, c.C, c.H, c.W, c.kH, c.kW, c.sh, c.sw, c.ph, c.pw, c.dh, c.dw, c.oH, c.oW, 0, dt) == 0);
+        }
+        if (good) accumulate_grad(x, dx); else { dev_fail("op_conv2d backward (input)"); free_tensor(dx); }
+    }
+    if (ok && needs_grad(w)) {
+        // per-sample dy[n] . col[n]^T as one batched GEMM, then the sum over the batch in the accumulate type
+        Tensor* dw = empty_tensor(dt, w->device_id, w->ndim, w->shape);
+        void* per_sample = nullptr;
+        bool good = dw && rp_hip_malloc(&per_sample, (size_t)chunk * c.Co * rows * esz) == 0;
+        for (int n0 = 0; good && n0 < c.N; n0 += chunk) {
+            const int nb = c.N - n0 < chunk ? c.N - n0 : chunk;
+            const char* x_nptr = (const char*)xd->data + n0 * x_n * esz;
+            const char* g_n = (const char*)g->data + n0 * y_n * esz;
+            good = (pointwise || conv_lower(col, x_nptr, nb, c, dt) == 0) &&
+                   rp_hip_gemm_strided_batched(per_sample, g_n, pointwise ? (const void*)x_nptr : col, nullptr, nb, c.Co, cols, rows,
+                                               y_n, cols, 1, col_n, 1, cols, (long long)c.Co * rows, rows, 1, 0, dt) == 0 &&
+                   rp_hip_reduce_rows(dw->data, per_sample, nb, c.Co * rows, n0 > 0, dt) == 0;
+        }
+        if (per_sample) rp_hip_free(per_sample);
+        if (good) accumulate_grad(w, dw); else { dev_fail("op_conv2d backward (weight)"); free_tensor(dw); }
+    }
+    if (ok && needs_grad(bias)) {
+        Tensor* db = empty_tensor(dt, bias->device_id, bias->ndim, bias->shape);
+        if (db && rp_hip_channel_sums(db->data, g->data, c.N, c.Co, cols, 0, dt) == 0) accumulate_grad(bias, db);
+        else { dev_fail("op_conv2d backward (bias)"); free_tensor(db); }
+    }
+    if (col) rp_hip_free(col);
+    free_tensor(g); free_tensor(xd); free_tensor(wd);
+}
+
 void backward_reduce_all_fn(GradFn* self, Tensor* grad_output) {     // sum_all / mean_all: every element receives g (or g / size)
     Tensor* x = self->inputs[0];
     if (!needs_grad(x)) return;
@@ -932,6 +1016,50 @@ Tensor* op_attention(Tensor* q, Tensor* k, Tensor* v, double scale) {
         gf->free_saved = free_attn_saved;
     }
     free_tensor(qd); free_tensor(kd); free_tensor(vd);
+    return out;
+}
+
+// reference ops/ops.c:4723-4870.  input [N, C_in, H, W], weight [C_out, C_in, kH, kW], bias [C_out] or null.
+Tensor* op_conv2d(Tensor* input, Tensor* weight, Tensor* bias, int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h, int dilation_w) {
+    if (!input || !weight) return nullptr;
+    if (input->ndim != 4 || weight->ndim != 4 || weight->shape[1] != input->shape[1] || !same_place(input, weight)) { fail("op_conv2d: input [N, C, H, W] and weight [C_out, C, kH, kW] of one dtype and device"); return nullptr; }
+    if (stride_h <= 0 || stride_w <= 0 || pad_h < 0 || pad_w < 0 || dilation_h <= 0 || dilation_w <= 0) { fail("op_conv2d: strides and dilations must be positive, paddings non-negative"); return nullptr; }
+    if (bias && (bias->ndim != 1 || bias->shape[0] != weight->shape[0] || !same_place(input, bias) || !rp_is_contiguous(bias))) { fail("op_conv2d: bias must be a dense vector of C_out"); return nullptr; }
+    if (input->device_id == -1) { fail("op_conv2d on host tensors is not provided by this build; move the operands to a GPU"); return nullptr; }
+    ConvSaved c{stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w, input->shape[0], input->shape[1], input->shape[2], input->shape[3],
+                weight->shape[0], weight->shape[2], weight->shape[3], 0, 0};
+    c.oH = (c.H + 2 * pad_h - dilation_h * (c.kH - 1) - 1) / stride_h + 1;
+    c.oW = (c.W + 2 * pad_w - dilation_w * (c.kW - 1) - 1) / stride_w + 1;
+    if (c.oH <= 0 || c.oW <= 0 || c.H + 2 * pad_h < dilation_h * (c.kH - 1) + 1 || c.W + 2 * pad_w < dilation_w * (c.kW - 1) + 1) { fail("op_conv2d: the kernel does not fit the padded input"); return nullptr; }
+    const DType dt = input->dtype;
+    const size_t esz = dtype_size(dt);
+    const int rows = c.C * c.kH * c.kW, cols = c.oH * c.oW;
+    const long long x_n = (long long)c.C * c.H * c.W, y_n = (long long)c.Co * cols, col_n = (long long)rows * cols;
+    if (col_n >= (1ll << 31) || y_n >= (1ll << 31)) { fail("op_conv2d: one sample's lowered matrix exceeds 2^31 elements"); return nullptr; }
+    int out_shape[4] = {c.N, c.Co, c.oH, c.oW};
+    Tensor* xd = dense(input); Tensor* wd = dense(weight);
+    Tensor* out = (xd && wd) ? empty_tensor(dt, input->device_id, 4, out_shape) : nullptr;
+    const bool pointwise = conv_is_pointwise(c);
+    const int chunk = conv_chunk(c, esz);
+    void* col = nullptr;
+    bool ok = out && on_device(input->device_id) && (pointwise || rp_hip_malloc(&col, (size_t)chunk * col_n * esz) == 0);
+    for (int n0 = 0; ok && n0 < c.N; n0 += chunk) {
+        const int nb = c.N - n0 < chunk ? c.N - n0 : chunk;
+        const char* x_nptr = (const char*)xd->data + n0 * x_n * esz;
+        ok = (pointwise || conv_lower(col, x_nptr, nb, c, dt) == 0) &&
+             rp_hip_gemm_strided_batched((char*)out->data + n0 * y_n * esz, wd->data, pointwise ? (const void*)x_nptr : col, nullptr, nb, c.Co, rows, cols,
+                                         0, rows, 1, col_n, cols, 1, y_n, cols, 1, 0, dt) == 0;
+    }
+    if (ok && bias) ok = rp_hip_channel_bias_add(out->data, bias->data, c.N, c.Co, cols, dt) == 0;
+    if (col) rp_hip_free(col);
+    free_tensor(xd); free_tensor(wd);
+    if (!ok) { dev_fail("op_conv2d"); free_tensor(out); return nullptr; }
+    if (needs_grad(input) || needs_grad(weight) || needs_grad(bias)) {
+        GradFn* gf = bias ? attach(out, backward_conv2d_fn, {input, weight, bias}) : attach(out, backward_conv2d_fn, {input, weight});
+        ConvSaved* sv = (ConvSaved*)malloc(sizeof(ConvSaved));
+        *sv = c;
+        gf->saved_data = sv;
+    }
     return out;
 }
 

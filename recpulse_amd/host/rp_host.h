@@ -98,6 +98,8 @@ Tensor* rp_expand(Tensor* x, int ndim, int* shape);
 /* ---- autograd ops ---- */
 Tensor* op_matmul(Tensor* a, Tensor* b);                 /* 2-D as in the reference; >2-D operands are batched (extension) */
 Tensor* op_linear(Tensor* x, Tensor* w, Tensor* bias);   /* x·w + bias in one launch (extension; bias may be NULL) */
+Tensor* op_conv2d(Tensor* input, Tensor* weight, Tensor* bias, int stride_h, int stride_w, int pad_h, int pad_w,
+                  int dilation_h, int dilation_w);                       /* reference ops/ops.h:89-91 */
 Tensor* op_attention(Tensor* q, Tensor* k, Tensor* v, double scale);   /* softmax(scale·q·kᵀ)·v in one launch (extension; 16-bit dtypes) */
 Tensor* op_add(Tensor* x1, Tensor* x2);
 Tensor* op_relu(Tensor* x);

@@ -360,3 +360,109 @@ def test_attention_slice_vs_torch_autograd(dt, tol):
     assert oracle.rel_err(oracle.to_f64(got["O"], dt), o.detach().numpy()) < tol
     for name, t in (("dQ", tq), ("dK", tk), ("dV", tv)):
         assert oracle.rel_err(oracle.to_f64(got[name], dt), t.grad.numpy()) < tol, name
+
+
+# --------------------------------------------------------------------------- conv2d lowering
+CONV_CASES = [tuple(tuple(v) if isinstance(v, list) else v for v in c) for c in GOLD["conv2d_parity_shapes"]["cases"]]
+
+
+def _ref_lowering(name, dst, src, C, H, W, k, s, p, d, oH, oW):
+    fn = getattr(REF, name)
+    assert fn(dst.ctypes.data, src.ctypes.data, C, H, W, k[0], k[1], s[0], s[1], p[0], p[1], d[0], d[1], oH, oW) == 0
+
+
+@needs_ref
+@pytest.mark.parametrize("dt,ty", [(F32, np.float32), (F64, np.float64)])
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "x".join(map(str, c[0])))
+def test_im2col_col2im_bit_equal_to_reference_kernels(dt, ty, case):
+    (N, C, H, W), (Co, _, kH, kW), s, p, d, _ = case
+    rng = np.random.default_rng(70)
+    oH, oW = oracle.conv_out_size(H, kH, s[0], p[0], d[0]), oracle.conv_out_size(W, kW, s[1], p[1], d[1])
+    im = rng.standard_normal((C, H, W)).astype(ty)
+    col = oracle.im2col(im, (kH, kW), s, p, d, dt)
+    want = np.empty_like(col)
+    _ref_lowering("im2col_kernel_host_f32" if dt == F32 else "im2col_kernel_host_f64", want, im, C, H, W, (kH, kW), s, p, d, oH, oW)
+    assert np.array_equal(col, want)
+    # col2im adds into an image that already holds values
+    c2 = rng.standard_normal(col.shape).astype(ty)
+    base = rng.standard_normal((C, H, W)).astype(ty)
+    got = oracle.col2im(base, c2, (kH, kW), s, p, d, dt)
+    want_im = base.copy()
+    _ref_lowering("col2im_kernel_host_f32" if dt == F32 else "col2im_kernel_host_f64", want_im, c2, C, H, W, (kH, kW), s, p, d, oH, oW)
+    assert np.array_equal(got, want_im)
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "x".join(map(str, c[0])))
+def test_col2im_is_the_adjoint_of_im2col(case):
+    """<im2col(x), c> == <x, col2im(c)> for any x and c: fixes every index of the gather against the scatter."""
+    (N, C, H, W), (Co, _, kH, kW), s, p, d, _ = case
+    rng = np.random.default_rng(71)
+    x = rng.standard_normal((C, H, W))
+    col = oracle.im2col(x, (kH, kW), s, p, d, F64)
+    c = rng.standard_normal(col.shape)
+    back = oracle.col2im(np.zeros((C, H, W)), c, (kH, kW), s, p, d, F64)
+    assert abs((col * c).sum() - (x * back).sum()) <= 1e-10 * max(1.0, abs((col * c).sum()))
+
+
+@pytest.mark.parametrize("dt", [F16, BF16])
+def test_lowering_16bit_is_fp32_pivot_then_one_narrowing(dt):
+    rng = np.random.default_rng(72)
+    C, H, W, k, s, p, d = 3, 7, 6, (3, 2), (2, 1), (1, 1), (1, 2)
+    im = oracle.to_storage(rng.standard_normal((C, H, W)), dt)
+    col = oracle.im2col(im, k, s, p, d, dt)
+    assert np.array_equal(col, oracle.narrow(oracle.im2col(oracle.widen(im, dt), k, s, p, d, F32), dt))
+    c2 = oracle.to_storage(rng.standard_normal(col.shape), dt)
+    got = oracle.col2im(im, c2, k, s, p, d, dt)
+    assert np.array_equal(got, oracle.narrow(oracle.col2im(oracle.widen(im, dt), oracle.widen(c2, dt), k, s, p, d, F32), dt))
+
+
+@pytest.mark.parametrize("dt", ALL)
+def test_conv2d_reference_known_answers(dt):
+    for case in GOLD["conv2d_known_answers"]["cases"]:
+        x = _st(np.ones(case["x_shape"]), dt); w = _st(np.ones(case["w_shape"]), dt)
+        bias = _st(case["bias"], dt) if "bias" in case else None
+        s, p = tuple(case.get("stride", (1, 1))), tuple(case.get("pad", (0, 0)))
+        y = oracle.conv2d_forward(x, w, bias, s, p, (1, 1), dt)
+        assert list(y.shape) == case["out_shape"]
+        if "out_sum" in case:
+            assert oracle.to_f64(y, dt).sum() == case["out_sum"]
+        if "bias_grad_of_sum" in case:
+            _, _, db = oracle.conv2d_backward(x, w, _st(np.ones(y.shape), dt), s, p, (1, 1), dt)
+            assert list(oracle.to_f64(db, dt)) == case["bias_grad_of_sum"]
+
+
+def test_conv2d_weight_gradient_vs_central_differences():
+    g = GOLD["conv2d_known_answers"]["weight_gradcheck"]
+    x = np.array(g["x"], dtype=np.float64).reshape(g["x_shape"]); w = np.array(g["w"], dtype=np.float64).reshape(g["w_shape"])
+    y = oracle.conv2d_forward(x, w, None, (1, 1), (0, 0), (1, 1), F64)
+    _, dw, _ = oracle.conv2d_backward(x, w, np.ones_like(y), (1, 1), (0, 0), (1, 1), F64, with_bias=False)
+    eps = 1e-3
+    for i in range(9):
+        wp, wm = w.copy().reshape(-1), w.copy().reshape(-1)
+        wp[i] += eps; wm[i] -= eps
+        num = (oracle.conv2d_forward(x, wp.reshape(w.shape), None, (1, 1), (0, 0), (1, 1), F64).sum()
+               - oracle.conv2d_forward(x, wm.reshape(w.shape), None, (1, 1), (0, 0), (1, 1), F64).sum()) / (2 * eps)
+        assert abs(dw.reshape(-1)[i] - num) <= 1e-2 * max(1.0, abs(num))
+
+
+@pytest.mark.parametrize("dt,tdt,tol", [(F32, "float32", 2e-5), (F64, "float64", 1e-12), (BF16, None, 3e-2), (F16, None, 4e-3)])
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "x".join(map(str, c[0])))
+def test_conv2d_vs_torch_autograd(dt, tdt, tol, case):
+    """Forward and all three gradients against torch.nn.functional.conv2d in float64 (an independent implementation)."""
+    import torch
+    xs, ws, s, p, d, has_bias = case
+    rng = np.random.default_rng(73)
+    x, w = oracle.to_storage(rng.standard_normal(xs), dt), oracle.to_storage(rng.standard_normal(ws) * 0.3, dt)
+    b = oracle.to_storage(rng.standard_normal(ws[0]), dt) if has_bias else None
+    y = oracle.conv2d_forward(x, w, b, s, p, d, dt)
+    dy = oracle.to_storage(rng.standard_normal(y.shape), dt)
+    dx, dw, db = oracle.conv2d_backward(x, w, dy, s, p, d, dt, with_bias=has_bias)
+    xt = torch.tensor(oracle.to_f64(x, dt), requires_grad=True); wt = torch.tensor(oracle.to_f64(w, dt), requires_grad=True)
+    bt = torch.tensor(oracle.to_f64(b, dt), requires_grad=True) if has_bias else None
+    yt = torch.nn.functional.conv2d(xt, wt, bt, stride=s, padding=p, dilation=d)
+    yt.backward(torch.tensor(oracle.to_f64(dy, dt)))
+    assert oracle.rel_err(oracle.to_f64(y, dt), yt.detach().numpy()) <= tol
+    assert oracle.rel_err(oracle.to_f64(dx, dt), xt.grad.numpy()) <= tol
+    assert oracle.rel_err(oracle.to_f64(dw, dt), wt.grad.numpy()) <= tol
+    if has_bias:
+        assert oracle.rel_err(oracle.to_f64(db, dt), bt.grad.numpy()) <= tol
