@@ -244,6 +244,9 @@ def secondary(capi, quick_reps=20):
     # config 4: attention-shaped batched GEMMs on stride views
     out["attention_bf16"] = attention_times(capi, "bf16")
     out["attention_f32"] = attention_times(capi, "f32")
+    # conv2d (the next caller of the GEMM): ResNet-style 3x3 layer, every launch of forward + backward
+    out["conv2d_bf16"] = conv2d_times(capi, "bf16")
+    out["conv2d_f32"] = conv2d_times(capi, "f32")
     # config 2: fp32 MLP 784-256-128-10, batch 256, forward + backward through the C ABI (9 GEMMs + neighbours)
     out["mlp_f32_step"] = mlp_step_time(capi)
     out["mlp_f32_step"]["ms_through_python_api"] = mlp_step_time_dropin()
@@ -306,6 +309,54 @@ def attention_times(capi, dt_name="bf16"):
         chain_b = out["fwd_bwd_ms"] * 1e3 - chain
         out["fused_backward"] = {"us": round(msb * 1e3, 1), "unfused_chain_us": round(chain_b, 1), "TFLOP/s": round(10.0 * Z * S * S * D / msb / 1e9, 1)}
         out["fused_fwd_bwd_ms"] = round(ms + msb, 4)
+    return out
+
+
+def conv2d_times(capi, dt_name="bf16"):
+    """A ResNet-style 3x3 layer (N 64, 64 -> 64 channels, 56 x 56, padding 1) lowered onto the batched GEMM: every
+    launch of the forward and backward timed on its own from a HIP graph.  Lowering bytes are read + written once."""
+    rng = np.random.default_rng(4)
+    N, C, H, W, Co, k, pad = 64, 64, 56, 56, 64, 3, 1
+    dt = {"bf16": capi.BF16, "f32": capi.F32}[dt_name]
+    esz = 2 if dt == capi.BF16 else 4
+    mk = (lambda shape: _normal_bf16(rng, shape)) if dt == capi.BF16 else (lambda shape: rng.standard_normal(shape).astype(np.float32))
+    D_ = capi.DeviceBuffer
+    rows, cols = C * k * k, H * W
+    x_n, y_n, col_n = C * H * W, Co * cols, rows * cols
+    d_x, d_w, d_b, d_dy = D_.from_numpy(mk((N, C, H, W))), D_.from_numpy(mk((Co, rows))), D_.from_numpy(mk((Co,))), D_.from_numpy(mk((N, Co, cols)))
+    d_col, d_y, d_dx = D_(N * col_n * esz), D_(N * y_n * esz), D_(N * x_n * esz)
+    d_dws, d_dw, d_db = D_(N * Co * rows * esz), D_(Co * rows * esz), D_(Co * esz)
+    L = capi.lib()
+    geom = (C, H, W, k, k, 1, 1, pad, pad, 1, 1, H, W)
+    gemm_flops = 2.0 * N * Co * rows * cols
+    ops = {
+        "im2col": (lambda: capi.check(L.rp_hip_im2col_batched(d_col.ptr, d_x.ptr, N, *geom, dt), "im2col"), 0.0, N * (x_n + col_n) * esz),
+        "y=W.col": (lambda: capi.gemm(d_y.ptr, d_w.ptr, d_col.ptr, None, N, Co, rows, cols, (0, rows, 1), (col_n, cols, 1), (y_n, cols, 1), False, dt),
+                    gemm_flops, (Co * rows + N * (col_n + y_n)) * esz),
+        "bias_add": (lambda: capi.check(L.rp_hip_channel_bias_add(d_y.ptr, d_b.ptr, N, Co, cols, dt), "bias"), 0.0, 2 * N * y_n * esz),
+        "dcol=Wt.dy": (lambda: capi.gemm(d_col.ptr, d_w.ptr, d_dy.ptr, None, N, rows, Co, cols, (0, 1, rows), (y_n, cols, 1), (col_n, cols, 1), False, dt),
+                       gemm_flops, (Co * rows + N * (col_n + y_n)) * esz),
+        "col2im": (lambda: capi.check(L.rp_hip_col2im_batched(d_dx.ptr, d_col.ptr, N, *geom, 0, dt), "col2im"), 0.0, N * (x_n + col_n) * esz),
+        "dW_n=dy.colt": (lambda: capi.gemm(d_dws.ptr, d_dy.ptr, d_col.ptr, None, N, Co, cols, rows, (y_n, cols, 1), (col_n, 1, cols), (Co * rows, rows, 1), False, dt),
+                         gemm_flops, N * (col_n + y_n + Co * rows) * esz),
+        "dW=sum_n": (lambda: capi.check(L.rp_hip_reduce_rows(d_dw.ptr, d_dws.ptr, N, Co * rows, 0, dt), "reduce_rows"), 0.0, (N + 1) * Co * rows * esz),
+        "db": (lambda: capi.check(L.rp_hip_channel_sums(d_db.ptr, d_dy.ptr, N, Co, cols, 0, dt), "channel_sums"), 0.0, N * y_n * esz),
+    }
+    for fn, _, _ in ops.values():
+        fn()
+    capi.check(L.rp_hip_im2col_batched(d_col.ptr, d_x.ptr, N, *geom, dt), "im2col")       # dW reads the lowered activations, not dcol
+    out, total = {}, 0.0
+    for name, (fn, flops, nbytes) in ops.items():
+        ms = _time_graph(capi, fn, 10, 2)
+        total += ms
+        out[name] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1)}
+        if flops:
+            out[name]["TFLOP/s"] = round(flops / ms / 1e9, 1)
+    total += out["im2col"]["us"] * 1e-3                 # the backward lowers the activations again for dW
+    out["fwd_bwd_ms"] = round(total, 4)
+    out["fwd_bwd_TFLOP/s"] = round(3 * gemm_flops / total / 1e9, 1)
+    for d in (d_x, d_w, d_b, d_dy, d_col, d_y, d_dx, d_dws, d_dw, d_db):
+        d.free()
     return out
 
 

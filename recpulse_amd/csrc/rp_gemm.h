@@ -53,11 +53,15 @@ struct TileCoord { int tm, tn; bool valid; };
 
 // The XCD-aware order launches whole rounds of 8 super-tiles (one per XCD): a super-tile count that is neither a
 // multiple of 8 nor large leaves XCDs idle in the last round (with 2 super-tiles only 2 of the 8 XCDs would work,
-// for every matrix of a batch), so those cases use plain row-major order, which deals tiles evenly.
+// for every matrix of a batch), and super-tiles that hang over the edge of the output give their XCD less work
+// than the others (5 x 25 tiles make 8 super-tiles holding 32, 32, 32, 4, 8, 8, 8 and 1 tiles).  Unless at least
+// nine tenths of the launched slots hold a tile, plain row-major order is used, which deals tiles evenly.
 __host__ __device__ __forceinline__ bool schedule_by_xcd(int tiles_m, int tiles_n) {
     constexpr int XCDS = 8, GM = 4, GN = 8;
-    int sup = ((tiles_m + GM - 1) / GM) * ((tiles_n + GN - 1) / GN);
-    return sup % XCDS == 0 || sup >= 4 * XCDS;
+    const int sup = ((tiles_m + GM - 1) / GM) * ((tiles_n + GN - 1) / GN);
+    if (!(sup % XCDS == 0 || sup >= 4 * XCDS)) return false;
+    const long long slots = (long long)((sup + XCDS - 1) / XCDS) * XCDS * GM * GN;
+    return (long long)tiles_m * tiles_n * 10 >= slots * 9;
 }
 
 __device__ __forceinline__ TileCoord schedule_tile(int bid, int tiles_m, int tiles_n) {
