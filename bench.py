@@ -461,6 +461,10 @@ def main():
                     help="run only the few-row bf16 GEMMs of configuration 5a and print their figures (for profiling that kernel alone)")
     ap.add_argument("--wide-only", action="store_true",
                     help="run only the fp32 (4096) and fp64 (2048, 4096) square GEMMs and print their figures (for profiling those kernels alone)")
+    ap.add_argument("--attention-only", action="store_true",
+                    help="run only the configuration-4 attention launches in bf16, unfused and fused (for profiling those kernels alone)")
+    ap.add_argument("--conv-only", action="store_true",
+                    help="run only the conv2d layer's launches in bf16 (for profiling those kernels alone)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain copy kernel of known size (256 MiB in, 256 MiB out), the yardstick for FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
@@ -484,6 +488,12 @@ def main():
         src.free(); dst.free()
     if args.skinny_only:
         print(json.dumps({"skinny": skinny_times(capi, rows=(1, 8))}))
+        return
+    if args.attention_only:
+        print(json.dumps({"attention_bf16": attention_times(capi, "bf16")}))
+        return
+    if args.conv_only:
+        print(json.dumps({"conv2d_bf16": conv2d_times(capi, "bf16")}))
         return
     if args.wide_only:
         print(json.dumps({"wide": wide_times(capi, (("gemm_f32_4096", "f32", 4096), ("gemm_f64_2048", "f64", 2048), ("gemm_f64_4096", "f64", 4096)))}))

@@ -2,7 +2,7 @@
  * rp_oracle.c — TEST INFRASTRUCTURE, NOT PRODUCT CODE.
  *
  * A plain-C restatement of the RecPulse reference's CPU arithmetic for the
- * matmul path.  It exists to check the HIP kernels and to time a CPU baseline.
+ * matmul path and its callers' lowering (im2col / col2im of conv2d).  It exists to check the HIP kernels and to time a CPU baseline.
  * Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may
  * load it; nothing in the shipped library links, imports or calls it.
  *

@@ -209,7 +209,16 @@ __global__ void channel_sums_finish_kernel(T* out, const typename traits<T>::acc
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= channels) return;
     A s = 0;
-    for (int n = 0; n < batch; n++) s += partial[(size_t)n * channels + c];
+    int n = 0;
+    constexpr int U = 16;                       // independent loads in flight; the adds stay in batch order
+    for (; n + U <= batch; n += U) {
+        A v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) v[u] = partial[(size_t)(n + u) * channels + c];
+#pragma unroll
+        for (int u = 0; u < U; u++) s += v[u];
+    }
+    for (; n < batch; n++) s += partial[(size_t)n * channels + c];
     T r = narrow<T>(s);
     if (accumulate) r = narrow<T>(widen(out[c]) + widen(r));
     out[c] = r;
