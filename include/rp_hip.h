@@ -207,6 +207,38 @@ int rp_hip_channel_bias_add(void* y, const void* bias, int batch, int channels, 
  * that the reference sums on the host (ops/ops.c:4620-4716). */
 int rp_hip_channel_sums(void* out, const void* grad, int batch, int channels, int hw, int accumulate, int dtype);
 
+/* ---- LSTM / GRU cells (recpulse/module.py:255-351): the element-wise half of a step, fused ---- */
+
+/* LSTM: gates [batch, 4*hidden] = i | f | g | o pre-activations x.W_ih + h.W_hh (two calls of
+ * rp_hip_gemm_strided_batched, the second with accumulate = 1); b_ih, b_hh [4*hidden] or NULL are added here, in the
+ * reference's order (recpulse/module.py:285-287); c_prev [batch, hidden] with the given row stride.
+ * Writes act [batch, 4*hidden] (sigmoid / tanh of the gates, kept for the backward) and hc [batch, 2*hidden] =
+ * h_next | c_next.  Replaces the reference's chunk, 3 sigmoid, 2 tanh, 3 mul and 1 add launches
+ * (recpulse/module.py:289-299; ops/ops.c op_sigmoid, op_tanh, op_mul, op_add), with a rounding to the tensor dtype
+ * wherever the reference materialises a tensor. */
+int rp_hip_lstm_cell_forward(void* hc, void* act, const void* gates, const void* b_ih, const void* b_hh,
+                             const void* c_prev, long long c_prev_row_stride, int batch, int hidden, int dtype);
+/* dgates [batch, 4*hidden] and dc_prev [batch, hidden] from dhc [batch, 2*hidden] (gradient of h_next | c_next):
+ * the backward functions of the same ops (ops/grad_host.c:365-400 tanh, 622-660 sigmoid; mul and add in ops/ops.c). */
+int rp_hip_lstm_cell_backward(void* dgates, void* dc_prev, const void* dhc, const void* act, const void* hc,
+                              const void* c_prev, long long c_prev_row_stride, int batch, int hidden, int dtype);
+
+/* GRU: gi = x.W_ih + b_ih and gh = h.W_hh + b_hh, [batch, 3*hidden] = r | z | n; h_prev [batch, hidden] with the given
+ * row stride.  Writes h_next [batch, hidden] and act [batch, 3*hidden] = r | z | n after their nonlinearities.
+ * Replaces recpulse/module.py:343-351 (2 chunk, 5 add, 2 sigmoid, 1 tanh, 3 mul, 1 rsub_scalar launches). */
+int rp_hip_gru_cell_forward(void* h_next, void* act, const void* gi, const void* gh, const void* h_prev,
+                            long long h_prev_row_stride, int batch, int hidden, int dtype);
+/* dgi, dgh [batch, 3*hidden] and the direct part dh_next * z of dh_prev [batch, hidden] (the part through gh is the
+ * GEMM dgh . W_hh^T, to be accumulated onto it). */
+int rp_hip_gru_cell_backward(void* dgi, void* dgh, void* dh_prev, const void* dh_next, const void* act, const void* gh,
+                             const void* h_prev, long long h_prev_row_stride, int batch, int hidden, int dtype);
+
+/* dst[sum_d idx_d * dst_strides[d]] = src[dense idx]: places the gradient of a slice inside a (zeroed) tensor of the
+ * sliced shape, the device half of the reference's backward_slice_fn / backward_chunk_fn (ops/ops.c:7536-7600).
+ * shape and dst_strides are host arrays of ndim <= 8 entries. */
+int rp_hip_scatter_strided(void* dst, const void* src, int ndim, const int* shape, const long long* dst_strides,
+                           size_t size, int dtype);
+
 /* Fused attention forward for bfloat16 / float16: O[b] = softmax(scale * Q[b] * K[b]^T) * V[b], the score matrix never
  * leaves the chip.  Q, O: [batch, sq, d]; K, V: [batch, sk, d]; d in {32, 64, 128} and contiguous (unit stride);
  * *_bs / *_rs are the batch and row strides in elements (multiples of 8; operands 16-byte aligned).

@@ -65,6 +65,8 @@ _sum_all = _sig("orc_sum_all", _i, _vp, _vp, _sz, _i)
 _reduce_rows = _sig("orc_reduce_rows", _i, _vp, _vp, _i, _i, _i)
 _contig = _sig("orc_contiguous_copy", _i, _vp, _vp, _i, _ip, _llp, _i)
 _ce = _sig("orc_cross_entropy_mean", _i, _vp, _vp, _vp, _ip, _i, _i, _d, _i)
+_sigmoid = _sig("orc_sigmoid", _i, _vp, _vp, _sz, _i)
+_tanh = _sig("orc_tanh", _i, _vp, _vp, _sz, _i)
 _im2col = _sig("orc_im2col", _i, _vp, _vp, *([_i] * 14))
 _col2im = _sig("orc_col2im", _i, _vp, _vp, *([_i] * 14))
 _widen = _sig("orc_widen", None, _vp, _vp, _sz, _i)
@@ -381,6 +383,109 @@ def conv2d_backward(x, w, dy, stride, pad, dilation, dtype, with_bias=True):
     return dx, dw.reshape(w.shape), db
 
 
+# ---------------------------------------------------------------------------
+# LSTM / GRU cells: the reference's op chain (recpulse/module.py:281-300, 334-351), one rounding per op
+# ---------------------------------------------------------------------------
+def sigmoid(x, dtype):
+    x = np.ascontiguousarray(x); out = np.empty_like(x)
+    _check(_sigmoid(_ptr(out), _ptr(x), x.size, dtype), "sigmoid")
+    return out
+
+
+def tanh(x, dtype):
+    x = np.ascontiguousarray(x); out = np.empty_like(x)
+    _check(_tanh(_ptr(out), _ptr(x), x.size, dtype), "tanh")
+    return out
+
+
+def _ew(fn, dtype, *xs):
+    """One element-wise reference op: operands widened to float32 (float64 for float64), one IEEE operation chain
+    `fn` in that type, one narrowing (reference functional/functional.c:10-56 for the 16-bit pivot)."""
+    ct = np.float64 if dtype == F64 else np.float32
+    ws = [to_f64(x, dtype).astype(ct) if dtype in (F16, BF16) else np.asarray(x, dtype=ct) for x in xs]
+    y = fn(*ws).astype(ct)
+    return narrow(y, dtype) if dtype in (F16, BF16) else y
+
+
+def mul(a, b, dtype):
+    return _ew(lambda x, y: x * y, dtype, a, b)
+
+
+def sub(a, b, dtype):
+    return _ew(lambda x, y: x - y, dtype, a, b)
+
+
+def _row_add(y, bias, dtype):
+    return add(y, np.ascontiguousarray(np.broadcast_to(bias, y.shape)), dtype)
+
+
+def lstm_cell_forward(x, h, c, w_ih, w_hh, b_ih, b_hh, dtype):
+    """recpulse/module.py:281-300.  Returns (h_next, c_next, saved) with saved = the activated gates."""
+    H = h.shape[1]
+    gates = add(matmul(x, w_ih, dtype), matmul(h, w_hh, dtype), dtype)
+    if b_ih is not None:
+        gates = _row_add(_row_add(gates, b_ih, dtype), b_hh, dtype)
+    i_g, f_g, g_g, o_g = (np.ascontiguousarray(gates[:, q * H:(q + 1) * H]) for q in range(4))
+    i_g, f_g, g_g, o_g = sigmoid(i_g, dtype), sigmoid(f_g, dtype), tanh(g_g, dtype), sigmoid(o_g, dtype)
+    c_next = add(mul(f_g, c, dtype), mul(i_g, g_g, dtype), dtype)
+    tc = tanh(c_next, dtype)
+    return mul(o_g, tc, dtype), c_next, (i_g, f_g, g_g, o_g, tc)
+
+
+def lstm_cell_backward(x, h, c, w_ih, w_hh, saved, dh, dc, dtype):
+    """The chain of backward functions the reference's autograd runs for lstm_cell_forward (mul, tanh, add, sigmoid,
+    chunk, add, matmul: ops/grad_host.c:365-400, 622-660; ops/ops.c:6759-6814).  Returns dx, dh_prev, dc_prev, dw_ih,
+    dw_hh, db (= db_ih = db_hh)."""
+    i_g, f_g, g_g, o_g, tc = saved
+    one = np.ones_like(to_f64(tc, dtype))
+    d_o = mul(dh, tc, dtype)
+    d_tc = mul(dh, o_g, dtype)
+    dcn = add(dc, _ew(lambda g, t: g * (1 - t * t), dtype, d_tc, tc), dtype)
+    d_f, d_cprev, d_i, d_g = mul(dcn, c, dtype), mul(dcn, f_g, dtype), mul(dcn, g_g, dtype), mul(dcn, i_g, dtype)
+    sig_b = lambda g, y: g * y * (1 - y)
+    dgates = np.concatenate([_ew(sig_b, dtype, d_i, i_g), _ew(sig_b, dtype, d_f, f_g),
+                             _ew(lambda g, y: g * (1 - y * y), dtype, d_g, g_g), _ew(sig_b, dtype, d_o, o_g)], axis=1)
+    del one
+    dx = matmul(dgates, np.ascontiguousarray(w_ih.T), dtype)
+    dh_prev = matmul(dgates, np.ascontiguousarray(w_hh.T), dtype)
+    dw_ih = matmul(np.ascontiguousarray(x.T), dgates, dtype)
+    dw_hh = matmul(np.ascontiguousarray(h.T), dgates, dtype)
+    return dx, dh_prev, d_cprev, dw_ih, dw_hh, reduce_rows(dgates, dtype)
+
+
+def gru_cell_forward(x, h, w_ih, w_hh, b_ih, b_hh, dtype):
+    """recpulse/module.py:334-351.  Returns (h_next, saved)."""
+    H = h.shape[1]
+    gi, gh = matmul(x, w_ih, dtype), matmul(h, w_hh, dtype)
+    if b_ih is not None:
+        gi, gh = _row_add(gi, b_ih, dtype), _row_add(gh, b_hh, dtype)
+    i_r, i_z, i_n = (np.ascontiguousarray(gi[:, q * H:(q + 1) * H]) for q in range(3))
+    h_r, h_z, h_n = (np.ascontiguousarray(gh[:, q * H:(q + 1) * H]) for q in range(3))
+    r = sigmoid(add(i_r, h_r, dtype), dtype)
+    z = sigmoid(add(i_z, h_z, dtype), dtype)
+    n = tanh(add(i_n, mul(r, h_n, dtype), dtype), dtype)
+    omz = _ew(lambda v: 1 - v, dtype, z)
+    return add(mul(omz, n, dtype), mul(z, h, dtype), dtype), (r, z, n, h_n, omz)
+
+
+def gru_cell_backward(x, h, w_ih, w_hh, saved, dh, dtype):
+    """Backward chain of gru_cell_forward.  Returns dx, dh_prev, dw_ih, dw_hh, db_ih, db_hh."""
+    r, z, n, h_n, omz = saved
+    d_n = mul(dh, omz, dtype)
+    d_z = sub(mul(dh, h, dtype), mul(dh, n, dtype), dtype)
+    d_pre_n = _ew(lambda g, y: g * (1 - y * y), dtype, d_n, n)
+    d_r = mul(d_pre_n, h_n, dtype)
+    sig_b = lambda g, y: g * y * (1 - y)
+    d_pre_r, d_pre_z = _ew(sig_b, dtype, d_r, r), _ew(sig_b, dtype, d_z, z)
+    dgi = np.concatenate([d_pre_r, d_pre_z, d_pre_n], axis=1)
+    dgh = np.concatenate([d_pre_r, d_pre_z, mul(d_pre_n, r, dtype)], axis=1)
+    dx = matmul(dgi, np.ascontiguousarray(w_ih.T), dtype)
+    dh_prev = add(mul(dh, z, dtype), matmul(dgh, np.ascontiguousarray(w_hh.T), dtype), dtype)
+    dw_ih = matmul(np.ascontiguousarray(x.T), dgi, dtype)
+    dw_hh = matmul(np.ascontiguousarray(h.T), dgh, dtype)
+    return dx, dh_prev, dw_ih, dw_hh, reduce_rows(dgi, dtype), reduce_rows(dgh, dtype)
+
+
 def matmul_f64(a, b, dtype):
     """The float64 oracle: exact inputs of `dtype`, float64 numpy product."""
     return to_f64(a, dtype) @ to_f64(b, dtype)
@@ -406,6 +511,11 @@ def load_reference():
         fn = getattr(ref, name)
         fn.restype = _i
         fn.argtypes = [_vp, _vp, _vp, _i, _i, _i]
+    for name, ct in (("sigmoid_kernel_host_f32", None), ("sigmoid_kernel_host_f64", None), ("tanh_kernel_host_f32", None), ("tanh_kernel_host_f64", None)):
+        if hasattr(ref, name):
+            fn = getattr(ref, name)
+            fn.restype = _i
+            fn.argtypes = [_vp, _vp, _sz]
     for name in ("im2col_kernel_host_f32", "im2col_kernel_host_f64", "col2im_kernel_host_f32", "col2im_kernel_host_f64"):
         if hasattr(ref, name):
             fn = getattr(ref, name)

@@ -663,3 +663,27 @@ int orc_col2im(void* im, const void* col, int C, int H, int W, int kH, int kW, i
     return 0;
 }
 
+/* ---------------------------------------------------------------------------
+ * sigmoid and tanh, the nonlinearities of the LSTM / GRU cells.
+ * reference functional/functional_host.c:498-545 (tanhf / tanh; 1/(1+expf(-x)) / 1/(1+exp(-x)));
+ * 16-bit through the fp32 pivot with one narrowing (functional/functional.c, same pattern as add).
+ * ------------------------------------------------------------------------- */
+static int orc_unary(void* out, const void* x, size_t n, int dtype, int is_tanh) {
+    if (!out || !x || n == 0) return -1;
+    if (dtype == ORC_F64) {
+        const double* a = (const double*)x; double* o = (double*)out;
+        for (size_t i = 0; i < n; i++) o[i] = is_tanh ? tanh(a[i]) : 1.0 / (1.0 + exp(-a[i]));
+        return 0;
+    }
+    float* w = (float*)orc_load_as_compute(x, n, dtype);
+    const float* a = w ? w : (const float*)x;
+    float* o = (dtype == ORC_F32) ? (float*)out : (float*)malloc(n * 4);
+    if (!o || (dtype != ORC_F32 && !w)) { free(w); if (dtype != ORC_F32) free(o); return -1; }
+    for (size_t i = 0; i < n; i++) o[i] = is_tanh ? tanhf(a[i]) : 1.0f / (1.0f + expf(-a[i]));
+    if (dtype != ORC_F32) { orc_narrow(o, out, n, dtype); free(o); }
+    free(w);
+    return 0;
+}
+int orc_sigmoid(void* out, const void* x, size_t n, int dtype) { return orc_unary(out, x, n, dtype, 0); }
+int orc_tanh(void* out, const void* x, size_t n, int dtype) { return orc_unary(out, x, n, dtype, 1); }
+

@@ -73,6 +73,11 @@ SIGNATURES = {
     "rp_hip_col2im_batched": (_i, [_vp, _vp] + [_i] * 16),
     "rp_hip_channel_bias_add": (_i, [_vp, _vp, _i, _i, _i, _i]),
     "rp_hip_channel_sums": (_i, [_vp, _vp, _i, _i, _i, _i, _i]),
+    "rp_hip_lstm_cell_forward": (_i, [_vp] * 6 + [_ll, _i, _i, _i]),
+    "rp_hip_lstm_cell_backward": (_i, [_vp] * 6 + [_ll, _i, _i, _i]),
+    "rp_hip_gru_cell_forward": (_i, [_vp] * 5 + [_ll, _i, _i, _i]),
+    "rp_hip_gru_cell_backward": (_i, [_vp] * 7 + [_ll, _i, _i, _i]),
+    "rp_hip_scatter_strided": (_i, [_vp, _vp, _i, _ip, ctypes.POINTER(ctypes.c_longlong), _sz, _i]),
     "rp_hip_attention_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i] + [_ll] * 8 + [_d, _i]),
     "rp_hip_attention_backward": (_i, [_vp] * 9 + [_i] * 4 + [_ll] * 10 + [_d, _i]),
 }

@@ -1,4 +1,5 @@
-"""Parameter bookkeeping (`Module`), the affine layer (`Linear`) and the convolution layer (`Conv2d`).
+"""Parameter bookkeeping (`Module`), the affine layer (`Linear`), the convolution layer (`Conv2d`) and the
+recurrent cells (`LSTMCell`, `GRUCell`).
 
 Behaviour kept from the reference's recpulse/module.py:
   * a module records its parameters in `tracked` under their attribute names; assigning a
@@ -12,6 +13,10 @@ Behaviour kept from the reference's recpulse/module.py:
   * `Conv2d` stores its weight as [out_channels, in_channels, kH, kW], initialised
     N(0, 1/(in_channels*kH*kW)), bias zeros, and accepts ints or pairs for kernel size, stride,
     padding and dilation (:117-155).
+  * `LSTMCell` / `GRUCell` store weight_ih [input_size, G*hidden] and weight_hh [hidden, G*hidden] (G = 4: i, f, g,
+    o; G = 3: r, z, n), initialised N(0, 1/hidden), biases zeros; a missing state is zeros; LSTMCell returns
+    (h_next, c_next), GRUCell h_next (:255-351).  A step here is one autograd node (two GEMMs and one fused
+    element-wise kernel) instead of the reference's twenty-odd ops.
 The Linear forward pass issues ONE launch (GEMM with the bias add in its epilogue) through
 `Tensor.op_linear`; the two-op form the reference uses gives the same values and is kept as
 `forward_two_ops` for comparison.
@@ -145,4 +150,41 @@ class Conv2d(Module):
         return self.keep(x.op_conv2d(self.weight, bias=self.bias, stride_h=self.stride[0], stride_w=self.stride[1],
                                      pad_h=self.padding[0], pad_w=self.padding[1],
                                      dilation_h=self.dilation[0], dilation_w=self.dilation[1]))
+
+
+class _RecurrentCell(Module):
+    GATES = 0
+
+    def __init__(self, input_size, hidden_size, bias=True):
+        super().__init__()
+        self.input_size, self.hidden_size = input_size, hidden_size
+        scale = 1.0 / math.sqrt(hidden_size)
+        g = self.GATES * hidden_size
+        self.weight_ih = self.track("weight_ih", rp.randn([input_size, g]).mul_scalar(scale).requires_grad_(True))
+        self.weight_hh = self.track("weight_hh", rp.randn([hidden_size, g]).mul_scalar(scale).requires_grad_(True))
+        self.bias_ih = self.track("bias_ih", rp.zeros([g]).requires_grad_(True)) if bias else None
+        self.bias_hh = self.track("bias_hh", rp.zeros([g]).requires_grad_(True)) if bias else None
+
+    def _zero_state(self, x):
+        return rp.zeros([x.shape[0], self.hidden_size], dtype=x.dtype, device=str(x.device))
+
+
+class LSTMCell(_RecurrentCell):
+    """(h_next, c_next) = LSTM step of x [B, input_size] from state (h, c), gates in the order i, f, g, o."""
+    GATES = 4
+
+    def forward(self, x, state=None):
+        h, c = state if state is not None else (self._zero_state(x), self._zero_state(x))
+        hc = self.keep(x.op_lstm_cell(h, c, self.weight_ih, self.weight_hh, self.bias_ih, self.bias_hh))
+        batch, hid = x.shape[0], self.hidden_size
+        return self.keep(hc.slice([0, 0], [batch, hid])), self.keep(hc.slice([0, hid], [batch, 2 * hid]))
+
+
+class GRUCell(_RecurrentCell):
+    """h_next = GRU step of x [B, input_size] from h, gates in the order r, z, n."""
+    GATES = 3
+
+    def forward(self, x, h=None):
+        h = h if h is not None else self._zero_state(x)
+        return self.keep(x.op_gru_cell(h, self.weight_ih, self.weight_hh, self.bias_ih, self.bias_hh))
 

@@ -184,6 +184,14 @@ PYBIND11_MODULE(recpulse_cuda, m) {
             return wrap(op_conv2d(x.t, w.t, bias.is_none() ? nullptr : bias.cast<PyTensor&>().t, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w), "op_conv2d");
         }, py::arg("weight"), py::arg("bias") = py::none(), py::arg("stride_h") = 1, py::arg("stride_w") = 1, py::arg("pad_h") = 0, py::arg("pad_w") = 0,
              py::arg("dilation_h") = 1, py::arg("dilation_w") = 1)        // reference python/tensor_python.c:1139-1171
+        .def("op_lstm_cell", [](PyTensor& x, PyTensor& h, PyTensor& c, PyTensor& w_ih, PyTensor& w_hh, py::object b_ih, py::object b_hh) {
+            return wrap(op_lstm_cell(x.t, h.t, c.t, w_ih.t, w_hh.t, b_ih.is_none() ? nullptr : b_ih.cast<PyTensor&>().t,
+                                     b_hh.is_none() ? nullptr : b_hh.cast<PyTensor&>().t), "op_lstm_cell");
+        }, py::arg("h"), py::arg("c"), py::arg("weight_ih"), py::arg("weight_hh"), py::arg("bias_ih") = py::none(), py::arg("bias_hh") = py::none())
+        .def("op_gru_cell", [](PyTensor& x, PyTensor& h, PyTensor& w_ih, PyTensor& w_hh, py::object b_ih, py::object b_hh) {
+            return wrap(op_gru_cell(x.t, h.t, w_ih.t, w_hh.t, b_ih.is_none() ? nullptr : b_ih.cast<PyTensor&>().t,
+                                    b_hh.is_none() ? nullptr : b_hh.cast<PyTensor&>().t), "op_gru_cell");
+        }, py::arg("h"), py::arg("weight_ih"), py::arg("weight_hh"), py::arg("bias_ih") = py::none(), py::arg("bias_hh") = py::none())
         .def("op_attention", [](PyTensor& q, PyTensor& k, PyTensor& v, double scale) { return wrap(op_attention(q.t, k.t, v.t, scale), "op_attention"); },
              py::arg("k"), py::arg("v"), py::arg("scale"))
         .def("op_add", [](PyTensor& a, PyTensor& b) { return wrap(op_add(a.t, b.t), "op_add"); })
@@ -254,7 +262,7 @@ PYBIND11_MODULE(recpulse_cuda, m) {
                 return v;
             };
             std::vector<int> b = get(start, "start"), e = get(stop, "stop"), s = get(step, "step");
-            return wrap(rp_slice(a.t, b.empty() ? nullptr : b.data(), e.empty() ? nullptr : e.data(), s.empty() ? nullptr : s.data()), "slice");
+            return wrap(op_slice(a.t, b.empty() ? nullptr : b.data(), e.empty() ? nullptr : e.data(), s.empty() ? nullptr : s.data()), "slice");      // reference python/tensor_python.c:2198
         }, py::arg("start") = py::none(), py::arg("stop") = py::none(), py::arg("step") = py::none())
         .def("__repr__", [](PyTensor& s) {
             std::string r = "Tensor(shape=(";

@@ -871,6 +871,92 @@ void backward_conv2d_fn(GradFn* self, Tensor* grad_output) {         // referenc
     free_tensor(g); free_tensor(xd); free_tensor(wd);
 }
 
+// ---- slice with a gradient (reference ops/ops.c op_slice, backward_slice_fn :7536-7600) ----
+struct SliceSaved { int ndim; int start[8]; int step[8]; };
+
+void backward_slice_fn(GradFn* self, Tensor* grad_output) {
+    Tensor* x = self->inputs[0];
+    if (!needs_grad(x)) return;
+    const SliceSaved& sv = *(SliceSaved*)self->saved_data;
+    // the slice's gradient, placed inside a zeroed tensor of x's shape
+    Tensor* g = dense(grad_output);
+    Tensor* full = zeros_tensor(x->dtype, x->device_id, x->ndim, x->shape, nullptr);
+    bool ok = g && full && on_device(x->device_id);
+    if (ok) {
+        long long strides[8], off = 0;
+        for (int d = 0; d < sv.ndim; d++) { strides[d] = (long long)full->strides[d] * sv.step[d]; off += (long long)sv.start[d] * full->strides[d]; }
+        ok = rp_hip_scatter_strided((char*)full->data + off * (long long)dtype_size(x->dtype), g->data, sv.ndim, grad_output->shape, strides, g->size, x->dtype) == 0;
+    }
+    if (ok) accumulate_grad(x, full); else { dev_fail("slice backward"); free_tensor(full); }
+    free_tensor(g);
+}
+
+// ---- LSTM / GRU cells ----------------------------------------------------------------
+// One autograd node per cell step: two GEMMs into the gate pre-activations, one fused element-wise kernel, and in
+// the backward one element-wise kernel followed by the four GEMMs and the bias reductions.  The reference composes a
+// step from about twenty ops (recpulse/module.py:281-300, 334-351).
+struct CellSaved { Tensor* act; Tensor* pre; Tensor* state; };       // activated gates; gh (GRU only); the previous c (LSTM) or h (GRU), unit column stride
+
+void free_cell_saved(void* p) {
+    CellSaved* s = (CellSaved*)p;
+    free_tensor(s->act); free_tensor(s->pre); free_tensor(s->state);
+    free(s);
+}
+
+Tensor* unit_columns(Tensor* x) { return x->strides[x->ndim - 1] == 1 ? tensor_retain(x) : rp_contiguous(x); }
+
+void bias_grad(Tensor* bias, Tensor* dgates) {
+    if (bias && needs_grad(bias)) accumulate_grad(bias, reduce_grad_to_shape(dgates, bias->ndim, bias->shape));
+}
+
+void backward_lstm_cell_fn(GradFn* self, Tensor* grad_output) {
+    Tensor* x = self->inputs[0]; Tensor* h = self->inputs[1]; Tensor* c = self->inputs[2];
+    Tensor* w_ih = self->inputs[3]; Tensor* w_hh = self->inputs[4]; Tensor* b_ih = self->inputs[5]; Tensor* b_hh = self->inputs[6];
+    CellSaved* sv = (CellSaved*)self->saved_data;
+    Tensor* hc = self->owner;
+    const int batch = x->shape[0], hidden = hc->shape[1] / 2;
+    int gshape[2] = {batch, 4 * hidden}, cshape[2] = {batch, hidden};
+    Tensor* dhc = dense(grad_output);
+    Tensor* hcd = dense(hc);
+    Tensor* dgates = empty_tensor(x->dtype, x->device_id, 2, gshape);
+    Tensor* dc = empty_tensor(x->dtype, x->device_id, 2, cshape);
+    bool ok = dhc && hcd && dgates && dc && on_device(x->device_id) &&
+              rp_hip_lstm_cell_backward(dgates->data, dc->data, dhc->data, sv->act->data, hcd->data, sv->state->data, sv->state->strides[0], batch, hidden, x->dtype) == 0;
+    if (!ok) dev_fail("op_lstm_cell backward");
+    if (ok && needs_grad(c)) { accumulate_grad(c, dc); dc = nullptr; }
+    if (ok && needs_grad(x)) gemm_grad(x, dgates, false, w_ih, true);
+    if (ok && needs_grad(h)) gemm_grad(h, dgates, false, w_hh, true);
+    if (ok && needs_grad(w_ih)) gemm_grad(w_ih, x, true, dgates, false);
+    if (ok && needs_grad(w_hh)) gemm_grad(w_hh, h, true, dgates, false);
+    if (ok) { bias_grad(b_ih, dgates); bias_grad(b_hh, dgates); }
+    free_tensor(dhc); free_tensor(hcd); free_tensor(dgates); free_tensor(dc);
+}
+
+void backward_gru_cell_fn(GradFn* self, Tensor* grad_output) {
+    Tensor* x = self->inputs[0]; Tensor* h = self->inputs[1];
+    Tensor* w_ih = self->inputs[2]; Tensor* w_hh = self->inputs[3]; Tensor* b_ih = self->inputs[4]; Tensor* b_hh = self->inputs[5];
+    CellSaved* sv = (CellSaved*)self->saved_data;
+    const int batch = x->shape[0], hidden = self->owner->shape[1];
+    int gshape[2] = {batch, 3 * hidden}, hshape[2] = {batch, hidden};
+    Tensor* dh = dense(grad_output);
+    Tensor* dgi = empty_tensor(x->dtype, x->device_id, 2, gshape);
+    Tensor* dgh = empty_tensor(x->dtype, x->device_id, 2, gshape);
+    Tensor* dh_direct = empty_tensor(x->dtype, x->device_id, 2, hshape);
+    bool ok = dh && dgi && dgh && dh_direct && on_device(x->device_id) &&
+              rp_hip_gru_cell_backward(dgi->data, dgh->data, dh_direct->data, dh->data, sv->act->data, sv->pre->data, sv->state->data, sv->state->strides[0],
+                                       batch, hidden, x->dtype) == 0;
+    if (!ok) dev_fail("op_gru_cell backward");
+    if (ok && needs_grad(h)) {
+        accumulate_grad(h, dh_direct); dh_direct = nullptr;           // dh * z, then the part through gh on top of it
+        gemm_grad(h, dgh, false, w_hh, true);
+    }
+    if (ok && needs_grad(x)) gemm_grad(x, dgi, false, w_ih, true);
+    if (ok && needs_grad(w_ih)) gemm_grad(w_ih, x, true, dgi, false);
+    if (ok && needs_grad(w_hh)) gemm_grad(w_hh, h, true, dgh, false);
+    if (ok) { bias_grad(b_ih, dgi); bias_grad(b_hh, dgh); }
+    free_tensor(dh); free_tensor(dgi); free_tensor(dgh); free_tensor(dh_direct);
+}
+
 void backward_reduce_all_fn(GradFn* self, Tensor* grad_output) {     // sum_all / mean_all: every element receives g (or g / size)
     Tensor* x = self->inputs[0];
     if (!needs_grad(x)) return;
@@ -1060,6 +1146,87 @@ Tensor* op_conv2d(Tensor* input, Tensor* weight, Tensor* bias, int stride_h, int
         *sv = c;
         gf->saved_data = sv;
     }
+    return out;
+}
+
+Tensor* op_slice(Tensor* x, int* start, int* stop, int* step) {        // reference ops/ops.h:51
+    Tensor* out = rp_slice(x, start, stop, step);
+    if (out && needs_grad(x)) {
+        if (x->ndim > 8) { fail("op_slice: more than 8 dimensions"); free_tensor(out); return nullptr; }
+        GradFn* gf = attach(out, backward_slice_fn, {x});
+        SliceSaved* sv = (SliceSaved*)calloc(1, sizeof(SliceSaved));
+        sv->ndim = x->ndim;
+        for (int d = 0; d < x->ndim; d++) {
+            int b = start ? start[d] : 0;
+            sv->start[d] = b < 0 ? b + x->shape[d] : b;
+            sv->step[d] = step ? step[d] : 1;
+        }
+        gf->saved_data = sv;
+    }
+    return out;
+}
+
+static bool cell_operands_ok(const char* op, Tensor* x, Tensor* h, Tensor* w_ih, Tensor* w_hh, Tensor* b_ih, Tensor* b_hh, int gates) {
+    if (!x || !h || !w_ih || !w_hh) return false;
+    const bool shapes = x->ndim == 2 && h->ndim == 2 && w_ih->ndim == 2 && w_hh->ndim == 2 && x->shape[0] == h->shape[0] && w_ih->shape[0] == x->shape[1] &&
+                        w_hh->shape[0] == h->shape[1] && w_ih->shape[1] == gates * h->shape[1] && w_hh->shape[1] == gates * h->shape[1];
+    if (!shapes || !same_place(x, h) || !same_place(x, w_ih) || !same_place(x, w_hh)) { fail("%s: x [B, I], h [B, H], w_ih [I, %dH], w_hh [H, %dH] of one dtype and device", op, gates, gates); return false; }
+    if ((b_ih == nullptr) != (b_hh == nullptr)) { fail("%s: give both biases or neither", op); return false; }
+    for (Tensor* b : {b_ih, b_hh})
+        if (b && (b->ndim != 1 || b->shape[0] != gates * h->shape[1] || !same_place(x, b) || !rp_is_contiguous(b))) { fail("%s: biases must be dense vectors of %dH", op, gates); return false; }
+    if (x->device_id == -1) { fail("%s on host tensors is not provided by this build; move the operands to a GPU", op); return false; }
+    return true;
+}
+
+// One LSTM step (recpulse/module.py:281-300).  Returns hc [B, 2H] = h_next | c_next; the halves are taken with op_slice.
+Tensor* op_lstm_cell(Tensor* x, Tensor* h, Tensor* c, Tensor* w_ih, Tensor* w_hh, Tensor* b_ih, Tensor* b_hh) {
+    if (!cell_operands_ok("op_lstm_cell", x, h, w_ih, w_hh, b_ih, b_hh, 4)) return nullptr;
+    if (!c || c->ndim != 2 || !same_shape(c, h) || !same_place(x, c)) { fail("op_lstm_cell: c must have h's shape, dtype and device"); return nullptr; }
+    const int batch = x->shape[0], hidden = h->shape[1];
+    int gshape[2] = {batch, 4 * hidden}, oshape[2] = {batch, 2 * hidden};
+    Tensor* gates = empty_tensor(x->dtype, x->device_id, 2, gshape);
+    Tensor* act = empty_tensor(x->dtype, x->device_id, 2, gshape);
+    Tensor* hc = empty_tensor(x->dtype, x->device_id, 2, oshape);
+    Tensor* cd = unit_columns(c);
+    // x . W_ih, then h . W_hh on top of it (beta = 1): the reference's matmul, matmul, add as two launches
+    bool ok = gates && act && hc && cd && device_gemm(gates, x, false, w_ih, false, nullptr, 0) == 0 && device_gemm(gates, h, false, w_hh, false, nullptr, 1) == 0 &&
+              rp_hip_lstm_cell_forward(hc->data, act->data, gates->data, b_ih ? b_ih->data : nullptr, b_hh ? b_hh->data : nullptr, cd->data, cd->strides[0],
+                                       batch, hidden, x->dtype) == 0;
+    free_tensor(gates);
+    if (!ok) { dev_fail("op_lstm_cell"); free_tensor(act); free_tensor(hc); free_tensor(cd); return nullptr; }
+    bool track = needs_grad(x) || needs_grad(h) || needs_grad(c) || needs_grad(w_ih) || needs_grad(w_hh) || needs_grad(b_ih) || needs_grad(b_hh);
+    if (track) {
+        GradFn* gf = attach(hc, backward_lstm_cell_fn, {x, h, c, w_ih, w_hh, b_ih, b_hh});
+        CellSaved* sv = (CellSaved*)calloc(1, sizeof(CellSaved));
+        sv->act = act; sv->state = cd;
+        gf->saved_data = sv;
+        gf->free_saved = free_cell_saved;
+    } else { free_tensor(act); free_tensor(cd); }
+    return hc;
+}
+
+// One GRU step (recpulse/module.py:334-351).  Returns h_next [B, H].
+Tensor* op_gru_cell(Tensor* x, Tensor* h, Tensor* w_ih, Tensor* w_hh, Tensor* b_ih, Tensor* b_hh) {
+    if (!cell_operands_ok("op_gru_cell", x, h, w_ih, w_hh, b_ih, b_hh, 3)) return nullptr;
+    const int batch = x->shape[0], hidden = h->shape[1];
+    int gshape[2] = {batch, 3 * hidden};
+    Tensor* gi = empty_tensor(x->dtype, x->device_id, 2, gshape);
+    Tensor* gh = empty_tensor(x->dtype, x->device_id, 2, gshape);
+    Tensor* act = empty_tensor(x->dtype, x->device_id, 2, gshape);
+    Tensor* out = empty_tensor(x->dtype, x->device_id, 2, h->shape);
+    Tensor* hd = unit_columns(h);
+    bool ok = gi && gh && act && out && hd && device_gemm(gi, x, false, w_ih, false, b_ih, 0) == 0 && device_gemm(gh, h, false, w_hh, false, b_hh, 0) == 0 &&
+              rp_hip_gru_cell_forward(out->data, act->data, gi->data, gh->data, hd->data, hd->strides[0], batch, hidden, x->dtype) == 0;
+    free_tensor(gi);
+    if (!ok) { dev_fail("op_gru_cell"); free_tensor(gh); free_tensor(act); free_tensor(out); free_tensor(hd); return nullptr; }
+    bool track = needs_grad(x) || needs_grad(h) || needs_grad(w_ih) || needs_grad(w_hh) || needs_grad(b_ih) || needs_grad(b_hh);
+    if (track) {
+        GradFn* gf = attach(out, backward_gru_cell_fn, {x, h, w_ih, w_hh, b_ih, b_hh});
+        CellSaved* sv = (CellSaved*)calloc(1, sizeof(CellSaved));
+        sv->act = act; sv->pre = gh; sv->state = hd;
+        gf->saved_data = sv;
+        gf->free_saved = free_cell_saved;
+    } else { free_tensor(act); free_tensor(gh); free_tensor(hd); }
     return out;
 }
 

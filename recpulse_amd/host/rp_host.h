@@ -100,6 +100,9 @@ Tensor* op_matmul(Tensor* a, Tensor* b);                 /* 2-D as in the refere
 Tensor* op_linear(Tensor* x, Tensor* w, Tensor* bias);   /* x·w + bias in one launch (extension; bias may be NULL) */
 Tensor* op_conv2d(Tensor* input, Tensor* weight, Tensor* bias, int stride_h, int stride_w, int pad_h, int pad_w,
                   int dilation_h, int dilation_w);                       /* reference ops/ops.h:89-91 */
+Tensor* op_slice(Tensor* x, int* start, int* stop, int* step);          /* reference ops/ops.h:51 */
+Tensor* op_lstm_cell(Tensor* x, Tensor* h, Tensor* c, Tensor* w_ih, Tensor* w_hh, Tensor* b_ih, Tensor* b_hh);   /* one step as one node: [B, 2H] = h_next | c_next (extension) */
+Tensor* op_gru_cell(Tensor* x, Tensor* h, Tensor* w_ih, Tensor* w_hh, Tensor* b_ih, Tensor* b_hh);                /* one step as one node: h_next (extension) */
 Tensor* op_attention(Tensor* q, Tensor* k, Tensor* v, double scale);   /* softmax(scale·q·kᵀ)·v in one launch (extension; 16-bit dtypes) */
 Tensor* op_add(Tensor* x1, Tensor* x2);
 Tensor* op_relu(Tensor* x);

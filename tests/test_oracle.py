@@ -466,3 +466,94 @@ def test_conv2d_vs_torch_autograd(dt, tdt, tol, case):
     assert oracle.rel_err(oracle.to_f64(dw, dt), wt.grad.numpy()) <= tol
     if has_bias:
         assert oracle.rel_err(oracle.to_f64(db, dt), bt.grad.numpy()) <= tol
+
+
+# --------------------------------------------------------------------------- LSTM / GRU cells
+@needs_ref
+@pytest.mark.parametrize("dt,ty", [(F32, np.float32), (F64, np.float64)])
+def test_sigmoid_tanh_bit_equal_to_reference_kernels(dt, ty):
+    rng = np.random.default_rng(90)
+    x = np.concatenate([rng.standard_normal(4000) * 4, [0.0, -0.0, 30.0, -30.0, 100.0, -100.0, 1e-8]]).astype(ty)
+    sfx = "f32" if dt == F32 else "f64"
+    for mine, name in ((oracle.sigmoid, "sigmoid_kernel_host_" + sfx), (oracle.tanh, "tanh_kernel_host_" + sfx)):
+        want = np.empty_like(x)
+        assert getattr(REF, name)(want.ctypes.data, x.ctypes.data, x.size) == 0
+        assert np.array_equal(mine(x, dt), want), name
+
+
+@pytest.mark.parametrize("dt", [F16, BF16])
+def test_sigmoid_tanh_16bit_is_fp32_pivot_then_one_narrowing(dt):
+    rng = np.random.default_rng(91)
+    x = oracle.to_storage(rng.standard_normal(3000) * 3, dt)
+    assert np.array_equal(oracle.sigmoid(x, dt), oracle.narrow(oracle.sigmoid(oracle.widen(x, dt), F32), dt))
+    assert np.array_equal(oracle.tanh(x, dt), oracle.narrow(oracle.tanh(oracle.widen(x, dt), F32), dt))
+
+
+def _cell_inputs(rng, B, I, H, gates, dt):
+    st = lambda a: oracle.to_storage(a, dt)
+    return (st(rng.standard_normal((B, I))), st(rng.standard_normal((B, H)) * 0.5), st(rng.standard_normal((B, H)) * 0.5),
+            st(rng.standard_normal((I, gates * H)) / np.sqrt(H)), st(rng.standard_normal((H, gates * H)) / np.sqrt(H)),
+            st(rng.standard_normal(gates * H) * 0.1), st(rng.standard_normal(gates * H) * 0.1))
+
+
+@pytest.mark.parametrize("dt,tol", [(F32, 2e-6), (F64, 1e-13), (BF16, 2e-2), (F16, 3e-3)])
+@pytest.mark.parametrize("bias", [True, False])
+def test_lstm_cell_vs_torch(dt, tol, bias):
+    """torch.nn.LSTMCell in float64 (same gate order i, f, g, o; its weights are the transposes) and its autograd."""
+    import torch
+    rng = np.random.default_rng(92)
+    B, I, H = 5, 7, 6
+    x, h, c, w_ih, w_hh, b_ih, b_hh = _cell_inputs(rng, B, I, H, 4, dt)
+    if not bias:
+        b_ih = b_hh = None
+    hn, cn, saved = oracle.lstm_cell_forward(x, h, c, w_ih, w_hh, b_ih, b_hh, dt)
+    dh, dc = oracle.to_storage(rng.standard_normal((B, H)), dt), oracle.to_storage(rng.standard_normal((B, H)), dt)
+    got = oracle.lstm_cell_backward(x, h, c, w_ih, w_hh, saved, dh, dc, dt)
+    T = lambda a: torch.tensor(oracle.to_f64(a, dt), requires_grad=True)
+    tx, th, tc, tw1, tw2 = T(x), T(h), T(c), T(w_ih), T(w_hh)
+    tb1, tb2 = (T(b_ih), T(b_hh)) if bias else (None, None)
+    gates = tx @ tw1 + th @ tw2 + ((tb1 + tb2) if bias else 0)
+    i_g, f_g, g_g, o_g = gates.chunk(4, 1)
+    cn_t = torch.sigmoid(f_g) * tc + torch.sigmoid(i_g) * torch.tanh(g_g)
+    hn_t = torch.sigmoid(o_g) * torch.tanh(cn_t)
+    cell = torch.nn.LSTMCell(I, H, bias=bias, dtype=torch.float64)                    # the library's own cell agrees with the formula above
+    with torch.no_grad():
+        cell.weight_ih.copy_(tw1.T); cell.weight_hh.copy_(tw2.T)
+        if bias:
+            cell.bias_ih.copy_(tb1); cell.bias_hh.copy_(tb2)
+    lib_h, lib_c = cell(tx.detach(), (th.detach(), tc.detach()))
+    assert torch.allclose(lib_h, hn_t, atol=1e-12) and torch.allclose(lib_c, cn_t, atol=1e-12)
+    (hn_t * torch.tensor(oracle.to_f64(dh, dt))).sum().add((cn_t * torch.tensor(oracle.to_f64(dc, dt))).sum()).backward()
+    assert oracle.rel_err(oracle.to_f64(hn, dt), hn_t.detach().numpy()) <= tol
+    assert oracle.rel_err(oracle.to_f64(cn, dt), cn_t.detach().numpy()) <= tol
+    want = [tx.grad, th.grad, tc.grad, tw1.grad, tw2.grad] + ([tb1.grad] if bias else [])
+    for name, g, w in zip(("dx", "dh", "dc", "dw_ih", "dw_hh", "db"), got, want):
+        assert oracle.rel_err(oracle.to_f64(g, dt), w.numpy()) <= 3 * tol, name
+
+
+@pytest.mark.parametrize("dt,tol", [(F32, 2e-6), (F64, 1e-13), (BF16, 2e-2), (F16, 3e-3)])
+@pytest.mark.parametrize("bias", [True, False])
+def test_gru_cell_vs_torch(dt, tol, bias):
+    """torch.nn.GRUCell in float64 (gate order r, z, n; n = tanh(i_n + r * (h_n + b_hn)); h' = (1 - z) n + z h)."""
+    import torch
+    rng = np.random.default_rng(93)
+    B, I, H = 4, 6, 5
+    x, h, _, w_ih, w_hh, b_ih, b_hh = _cell_inputs(rng, B, I, H, 3, dt)
+    if not bias:
+        b_ih = b_hh = None
+    hn, saved = oracle.gru_cell_forward(x, h, w_ih, w_hh, b_ih, b_hh, dt)
+    dh = oracle.to_storage(rng.standard_normal((B, H)), dt)
+    got = oracle.gru_cell_backward(x, h, w_ih, w_hh, saved, dh, dt)
+    T = lambda a: torch.tensor(oracle.to_f64(a, dt), requires_grad=True)
+    tx, th, tw1, tw2 = T(x), T(h), T(w_ih), T(w_hh)
+    tb1, tb2 = (T(b_ih), T(b_hh)) if bias else (None, None)
+    cell = torch.nn.GRUCell(I, H, bias=bias, dtype=torch.float64)
+    params = {"weight_ih": tw1.T, "weight_hh": tw2.T}
+    if bias:
+        params.update({"bias_ih": tb1, "bias_hh": tb2})
+    hn_t = torch.func.functional_call(cell, params, (tx, th))
+    (hn_t * torch.tensor(oracle.to_f64(dh, dt))).sum().backward()
+    assert oracle.rel_err(oracle.to_f64(hn, dt), hn_t.detach().numpy()) <= tol
+    want = [tx.grad, th.grad, tw1.grad, tw2.grad] + ([tb1.grad, tb2.grad] if bias else [])
+    for name, g, w in zip(("dx", "dh", "dw_ih", "dw_hh", "db_ih", "db_hh"), got, want):
+        assert oracle.rel_err(oracle.to_f64(g, dt), w.numpy()) <= 3 * tol, name
