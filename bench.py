@@ -247,6 +247,9 @@ def secondary(capi, quick_reps=20):
     # conv2d (the next caller of the GEMM): ResNet-style 3x3 layer, every launch of forward + backward
     out["conv2d_bf16"] = conv2d_times(capi, "bf16")
     out["conv2d_f32"] = conv2d_times(capi, "f32")
+    # an LSTM step (the last caller of the GEMM on the list): small GEMMs bound by the weights' bytes and by launches
+    out["lstm_step_bf16"] = lstm_step_times(capi, "bf16")
+    out["lstm_step_f32"] = lstm_step_times(capi, "f32")
     # config 2: fp32 MLP 784-256-128-10, batch 256, forward + backward through the C ABI (9 GEMMs + neighbours)
     out["mlp_f32_step"] = mlp_step_time(capi)
     out["mlp_f32_step"]["ms_through_python_api"] = mlp_step_time_dropin()
@@ -357,6 +360,54 @@ def conv2d_times(capi, dt_name="bf16"):
     out["fwd_bwd_TFLOP/s"] = round(3 * gemm_flops / total / 1e9, 1)
     for d in (d_x, d_w, d_b, d_dy, d_col, d_y, d_dx, d_dws, d_dw, d_db):
         d.free()
+    return out
+
+
+def lstm_step_times(capi, dt_name="bf16"):
+    """One LSTM step (batch 64, input 1024, hidden 1024) forward + backward through the C ABI: 2 + 4 GEMMs, the two
+    fused element-wise kernels and the bias reduction, each launch on its own and the whole step from one HIP graph."""
+    rng = np.random.default_rng(5)
+    B, I, H = 64, 1024, 1024
+    G = 4 * H
+    dt = {"bf16": capi.BF16, "f32": capi.F32}[dt_name]
+    esz = 2 if dt == capi.BF16 else 4
+    if dt == capi.BF16:
+        mk = lambda shape, s=1.0: _bf16_bits((rng.standard_normal(shape) * s).astype(np.float32))
+    else:
+        mk = lambda shape, s=1.0: (rng.standard_normal(shape) * s).astype(np.float32)
+    D_ = capi.DeviceBuffer
+    d_x, d_h, d_c = D_.from_numpy(mk((B, I))), D_.from_numpy(mk((B, H), 0.5)), D_.from_numpy(mk((B, H), 0.5))
+    d_wi, d_wh = D_.from_numpy(mk((I, G), 1 / 32)), D_.from_numpy(mk((H, G), 1 / 32))
+    d_bi, d_bh, d_dhc = D_.from_numpy(mk((G,), 0.1)), D_.from_numpy(mk((G,), 0.1)), D_.from_numpy(mk((B, 2 * H)))
+    d_g, d_act, d_hc, d_dg = D_(B * G * esz), D_(B * G * esz), D_(B * 2 * H * esz), D_(B * G * esz)
+    d_dc, d_dx, d_dh = D_(B * H * esz), D_(B * I * esz), D_(B * H * esz)
+    d_dwi, d_dwh, d_db = D_(I * G * esz), D_(H * G * esz), D_(G * esz)
+    L = capi.lib()
+    ops = {
+        "gates=x.Wih": (lambda: capi.gemm(d_g.ptr, d_x.ptr, d_wi.ptr, None, 1, B, I, G, (0, I, 1), (0, G, 1), (0, G, 1), False, dt), 2.0 * B * I * G, (B * I + I * G + B * G) * esz),
+        "gates+=h.Whh": (lambda: capi.gemm(d_g.ptr, d_h.ptr, d_wh.ptr, None, 1, B, H, G, (0, H, 1), (0, G, 1), (0, G, 1), True, dt), 2.0 * B * H * G, (B * H + H * G + 2 * B * G) * esz),
+        "cell_fwd": (lambda: capi.check(L.rp_hip_lstm_cell_forward(d_hc.ptr, d_act.ptr, d_g.ptr, d_bi.ptr, d_bh.ptr, d_c.ptr, H, B, H, dt), "lstm fwd"), 0.0, (2 * B * G + 3 * B * H) * esz),
+        "cell_bwd": (lambda: capi.check(L.rp_hip_lstm_cell_backward(d_dg.ptr, d_dc.ptr, d_dhc.ptr, d_act.ptr, d_hc.ptr, d_c.ptr, H, B, H, dt), "lstm bwd"), 0.0, (2 * B * G + 6 * B * H) * esz),
+        "dx=dg.Wiht": (lambda: capi.gemm(d_dx.ptr, d_dg.ptr, d_wi.ptr, None, 1, B, G, I, (0, G, 1), (0, 1, G), (0, I, 1), False, dt), 2.0 * B * I * G, (B * G + I * G + B * I) * esz),
+        "dh=dg.Whht": (lambda: capi.gemm(d_dh.ptr, d_dg.ptr, d_wh.ptr, None, 1, B, G, H, (0, G, 1), (0, 1, G), (0, H, 1), False, dt), 2.0 * B * H * G, (B * G + H * G + B * H) * esz),
+        "dWih=xt.dg": (lambda: capi.gemm(d_dwi.ptr, d_x.ptr, d_dg.ptr, None, 1, I, B, G, (0, 1, I), (0, G, 1), (0, G, 1), False, dt), 2.0 * B * I * G, (B * I + B * G + I * G) * esz),
+        "dWhh=ht.dg": (lambda: capi.gemm(d_dwh.ptr, d_h.ptr, d_dg.ptr, None, 1, H, B, G, (0, 1, H), (0, G, 1), (0, G, 1), False, dt), 2.0 * B * H * G, (B * H + B * G + H * G) * esz),
+        "db": (lambda: capi.check(L.rp_hip_reduce_rows(d_db.ptr, d_dg.ptr, B, G, 0, dt), "reduce_rows"), 0.0, (B * G + G) * esz),
+    }
+    for fn, _, _ in ops.values():
+        fn()
+    out = {}
+    for name, (fn, flops, nbytes) in ops.items():
+        ms = _time_graph(capi, fn, 20, 2)
+        out[name] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1)}
+    def step():
+        for fn, _, _ in ops.values():
+            fn()
+    ms = _time_graph(capi, step, 10, 2)
+    total_bytes = sum(nb for _, _, nb in ops.values())
+    out["step_ms"] = round(ms, 4)
+    out["step_GB/s"] = round(total_bytes / ms / 1e6, 1)
+    out["launches"] = len(ops)
     return out
 
 

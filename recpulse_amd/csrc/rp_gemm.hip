@@ -32,6 +32,12 @@ static bool force_generic() {
     return v == 1;
 }
 
+static int skinny_max_rows() {                     // RP_HIP_SKINNY_MAX_M: rows up to which a deep 16-bit GEMM with few output tiles splits k
+    static int v = -1;
+    if (v < 0) { const char* e = getenv("RP_HIP_SKINNY_MAX_M"); v = e ? atoi(e) : 128; if (v < 32) v = 32; }
+    return v;
+}
+
 // Decide the kernel family and tile from shapes and strides alone (pointer
 // alignment is checked by the caller, which may still fall back to generic).
 static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long a_cs, long long b_rs, long long b_cs,
@@ -54,8 +60,12 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     const bool mfma_ok = (a_kc || a_mc) && (b_kc || b_mc) && batch_ok && strides_ok;
     const bool is16 = dtype == RP_DTYPE_FLOAT16 || dtype == RP_DTYPE_BFLOAT16;
 
-    // 16-bit, few rows, deep k: split k over many blocks so that B streams at HBM speed (output columns in whole 8s)
-    if (is16 && mfma_ok && batch == 1 && m <= 32 && n % 8 == 0 && n >= 256 && k >= 1024 && (long long)k * n >= (1ll << 22)) {
+    // 16-bit, few rows, deep k: split k over many blocks so that B streams at HBM speed (output columns in whole 8s).
+    // Up to 32 rows always; up to skinny_max_rows() when the 128 x 128 tiles of the output would occupy under half the
+    // CUs (and k is deep enough to be worth a second launch for the partial sums).
+    const long long tiles128_16 = (long long)((m + 127) / 128) * ((n + 127) / 128);
+    if (is16 && mfma_ok && batch == 1 && (m <= 32 || (m <= skinny_max_rows() && tiles128_16 < 128 && (k >= 2048 || tiles128_16 < 48))) && n % 8 == 0 && n >= 256 && k >= 1024 &&
+        (long long)k * n >= (1ll << 22)) {
         p.fam = FAM_MFMA16_SKINNY; p.bm = 32; p.bn = 128; p.edge = true; p.a_mc = !a_kc; p.b_mc = b_mc;
         p.name = (!p.a_mc && p.b_mc && m <= 16) ? "mfma16_stream_32x256" : "mfma16_skinny_32x128";
         return p;

@@ -263,9 +263,9 @@ int launch_mfma16_skinny(const GemmArgs& g, const Plan& p, int dtype) {
     // beyond 16 rows the partial tiles the streaming kernel exchanges outweigh what it saves
     if (!p.a_mc && p.b_mc && g.m <= SS_MAX_M && !tiled_skinny_forced()) return launch_stream16(g, dtype);
     constexpr int BN = 128;
-    const int tiles_n = (g.n + BN - 1) / BN;
+    const int tiles = ((g.n + BN - 1) / BN) * ((g.m + 31) / 32);
     // about three blocks per CU in flight, each split at least four slabs deep
-    int nsplit = (768 + tiles_n - 1) / tiles_n;
+    int nsplit = (768 + tiles - 1) / tiles;
     int max_split = g.k / (4 * M16_BK) > 0 ? g.k / (4 * M16_BK) : 1;
     if (nsplit > max_split) nsplit = max_split;
     int k_per_split = ((g.k + nsplit - 1) / nsplit + M16_BK - 1) / M16_BK * M16_BK;
