@@ -143,21 +143,33 @@ def headline(capi, steps, warmup, n=8192, data="normal"):
 
 
 def cpu_baseline(a, b, target_s=15.0):
-    """The oracle's restatement of the reference CPU matmul on a row slab of the 8192^3 bf16 GEMM, one core.  Two rows
-    are timed first and the slab is sized from them for about `target_s` seconds of CPU work (4 to 256 rows)."""
+    """The reference's CPU path for the bf16 GEMM (functional/functional.c:986-1000: widen A and B to float32, the
+    i-j-l loop of matmul_kernel_host_f32, narrow C) on a row slab of the 8192^3 GEMM, one core.  When the reference's
+    own host kernel was compiled into oracle/_ref the loop is that code ("reference"); otherwise the oracle's
+    restatement of it ("port").  Two rows are timed first and the slab is sized from them for about `target_s`
+    seconds of CPU work (4 to 256 rows)."""
     import oracle
     n = b.shape[0]
+    ref = oracle.load_reference()
+
+    def run(slab):
+        if ref is None:
+            return oracle.matmul(slab, b, oracle.BF16)              # widens B to fp32 once per call, as the reference does
+        c32 = oracle.reference_matmul(ref, oracle.widen(slab, oracle.BF16), oracle.widen(b, oracle.BF16), oracle.F32)
+        return oracle.narrow(c32, oracle.BF16)
+
     t0 = time.perf_counter()
-    oracle.matmul(np.ascontiguousarray(a[:2]), b, oracle.BF16)       # includes widening B to fp32 once, as every call does
+    run(np.ascontiguousarray(a[:2]))
     probe = time.perf_counter() - t0
     rows = int(min(256, max(4, round(target_s / (probe / 2)))))
     slab = np.ascontiguousarray(a[:rows])
     t0 = time.perf_counter()
-    oracle.matmul(slab, b, oracle.BF16)
+    run(slab)
     dt = time.perf_counter() - t0
     flops = 2.0 * rows * n * n
-    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
-            "sample": f"{rows} of {n} rows of the bf16 {n}^3 forward GEMM (fp32 pivot, i-j-l loop), {dt:.1f} s; "
+    what = "the reference's matmul_kernel_host_f32 compiled from its own source" if ref is not None else "the oracle's restatement of the reference loop"
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "reference" if ref is not None else "port",
+            "sample": f"{rows} of {n} rows of the bf16 {n}^3 forward GEMM ({what}; fp32 pivot, i-j-l loop), {dt:.1f} s; "
                       f"host has {os.cpu_count()} logical cores"}
 
 
