@@ -608,7 +608,6 @@ extern "C" int rp_hip_attention_backward(void* dQ, void* dK, void* dV, const voi
     }
     if (dtype != RP_DTYPE_BFLOAT16 && dtype != RP_DTYPE_FLOAT16) { set_error("rp_hip_attention_backward: bfloat16 / float16 only (dtype %d)", dtype); return -1; }
     if (d != 32 && d != 64 && d != 128) { set_error("rp_hip_attention_backward: head dimension %d (supported: 32, 64, 128)", d); return -1; }
-    if (batch > 65535) { set_error("rp_hip_attention_backward: batch %d exceeds 65535", batch); return -1; }
     const long long strides[] = {q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs, do_bs, do_rs};
     for (long long s : strides)
         if (s < 0 || s % 8) { set_error("rp_hip_attention_backward: strides must be non-negative multiples of 8 elements"); return -1; }
@@ -619,8 +618,17 @@ extern "C" int rp_hip_attention_backward(void* dQ, void* dK, void* dV, const voi
     }
     void* dots = nullptr;
     if (rp_hip_malloc(&dots, (size_t)batch * sq * sizeof(float)) != 0) return -1;
-    AttnBwdArgs g{dQ, dK, dV, Q, K, V, O, dO, lse, (float*)dots, batch, sq, sk, q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs, do_bs, do_rs, (float)scale};
-    const int rc = dtype == RP_DTYPE_BFLOAT16 ? launch_attention_bwd_t<bf16_t>(g, d) : launch_attention_bwd_t<f16_t>(g, d);
+    // the batch rides on a grid axis that holds at most 65535 blocks: longer batches go in chunks
+    constexpr int MAX_BATCH = 65535;
+    int rc = 0;
+    for (int b0 = 0; rc == 0 && b0 < batch; b0 += MAX_BATCH) {
+        const int nb = batch - b0 < MAX_BATCH ? batch - b0 : MAX_BATCH;
+        const long long q_off = (long long)b0 * sq * d * 2, k_off = (long long)b0 * sk * d * 2;        // the gradients are dense
+        AttnBwdArgs g{(char*)dQ + q_off, (char*)dK + k_off, (char*)dV + k_off, (const char*)Q + b0 * q_bs * 2, (const char*)K + b0 * k_bs * 2,
+                      (const char*)V + b0 * v_bs * 2, (const char*)O + b0 * o_bs * 2, (const char*)dO + b0 * do_bs * 2, lse + (long long)b0 * sq,
+                      (float*)dots + (long long)b0 * sq, nb, sq, sk, q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs, do_bs, do_rs, (float)scale};
+        rc = dtype == RP_DTYPE_BFLOAT16 ? launch_attention_bwd_t<bf16_t>(g, d) : launch_attention_bwd_t<f16_t>(g, d);
+    }
     rp_hip_free(dots);        // stream-ordered reuse: the pool hands it out again only to later work on this stream
     return rc;
 }

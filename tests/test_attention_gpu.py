@@ -143,3 +143,19 @@ def test_fused_attention_backward_rejects_bad_arguments():
     assert b"head dimension" in L.rp_hip_last_error()
     assert L.rp_hip_attention_backward(p, p, p, p, p, p, p, p, None, 1, 4, 4, 64, 256, 64, 256, 64, 256, 64, 256, 64, 256, 64, 1.0, BF16) == -1
     assert L.rp_hip_attention_backward(p, p, p, p, p, p, p, p, p, 1, 4, 4, 64, 256, 64, 256, 64, 256, 64, 256, 64, 256, 64, 1.0, capi.F32) == -1
+
+
+def test_fused_attention_batch_longer_than_a_grid_axis():
+    """70 000 heads of 8 x 8 x 32: forward and backward go in two chunks of the batch; checked on both sides of the seam."""
+    rng = np.random.default_rng(64)
+    Z, S, D = 70000, 8, 32
+    q, k, v, g = (rand_storage(rng, (Z, S, D), BF16) for _ in range(4))
+    scale = 1.0 / np.sqrt(D)
+    sel = [0, 65534, 65535, 65536, Z - 1]
+    out = _fused(q, k, v, BF16, scale)
+    want, _ = _f64(q[sel], k[sel], v[sel], BF16, scale)
+    assert oracle.rel_err(oracle.to_f64(out[sel], BF16), want) <= 1e-2
+    got = _fused_backward(q, k, v, g, BF16, scale)
+    wants = _f64_backward(q[sel], k[sel], v[sel], g[sel], BF16, scale)
+    for a, b in zip(got, wants):
+        assert oracle.rel_err(oracle.to_f64(a[sel], BF16), b) <= 2e-2
