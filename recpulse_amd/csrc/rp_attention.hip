@@ -14,8 +14,9 @@
 // key rows 8*(v/4) + 4*(lane/32) + v%4) is, after narrowing to 16 bits, exactly a B operand of the second product whose
 // k slots are those same keys, so the probabilities go from one MFMA to the next without leaving the lane; and O^T has
 // the same lane = query mapping, so the rescaling factor of the online softmax is a per-lane scalar too.
-// Q and K fragments are 16-byte global loads straight into MFMA operand registers (rows are d-contiguous); V is the one
-// operand that needs a transpose (k slots = keys, rows = d) and goes through LDS with ds_read_tr16_b64.
+// Q fragments are 16-byte global loads straight into MFMA operand registers, once per wave (rows are d-contiguous).
+// K and V blocks are staged in LDS by the whole workgroup with row-contiguous loads: K fragments are read back with
+// ds_read_b128, V, the one operand that needs a transpose (k slots = keys, rows = d), with ds_read_tr16_b64.
 // Probabilities are narrowed to the tensor dtype before the second product (as the reference's P is), accumulation is
 // fp32 throughout, and the scores themselves are never rounded to 16 bits (the reference rounds S and S*scale).
 #include "rp_gemm_mfma16_kernel.h"
@@ -36,6 +37,26 @@ struct AttnArgs {
 constexpr int AT_KEYS = 32;                 // keys per step
 constexpr int AT_QROWS = 128;               // query rows per workgroup (32 per wave)
 
+// Two fp32 values to a pair of T with the hardware's packed round-to-nearest-even conversion (one instruction for
+// two values).  The probabilities and the score gradients packed with it exist only inside the fused kernels, as MFMA
+// operands; tensors that leave a kernel are narrowed with the reference's rule (narrow<T>).
+template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b);
+template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float a, float b) {
+    typedef __attribute__((ext_vector_type(2))) __bf16 v2;
+    const v2 v = {(__bf16)a, (__bf16)b};
+    return __builtin_bit_cast(uint32_t, v);
+}
+template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
+    typedef __attribute__((ext_vector_type(2))) _Float16 v2;
+    const v2 v = {(_Float16)a, (_Float16)b};
+    return __builtin_bit_cast(uint32_t, v);
+}
+// slots 8t .. 8t+7 of sixteen fp32 values as one MFMA B operand
+template <typename T> __device__ __forceinline__ s16x8_t pack8(const float* x) {
+    u32x4_t w = {pack2<T>(x[0], x[1]), pack2<T>(x[2], x[3]), pack2<T>(x[4], x[5]), pack2<T>(x[6], x[7])};
+    return __builtin_bit_cast(s16x8_t, w);
+}
+
 template <typename T, int D>
 __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_fwd16_kernel(AttnArgs g) {
     static_assert(D % 32 == 0 && D <= 128, "head dimension: a multiple of 32 up to 128");
@@ -43,7 +64,9 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_fwd16_kernel(A
     constexpr int DT = D / 32;              // 32-row tiles of O^T
     constexpr int VP = m16_mc_pitch(D);     // LDS pitch of a V row in elements, the GEMM kernels' conflict-free one for this read pattern
     constexpr int VPIECES = AT_KEYS * D / 8 / 256 > 0 ? AT_KEYS * D / 8 / 256 : 1;      // 16-byte pieces of a V block per thread
+    constexpr int RP = D + 8;               // LDS pitch of a K row in elements: 16 bytes past a multiple of 128, so that ds_read_b128 of 16 rows is conflict-free
     __shared__ __attribute__((aligned(16))) uint16_t vlds[2][AT_KEYS * VP];
+    __shared__ __attribute__((aligned(16))) uint16_t klds[2][AT_KEYS * RP];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -53,7 +76,10 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_fwd16_kernel(A
     const uint16_t* Q = (const uint16_t*)g.Q + (long long)z * g.q_bs;
     const uint16_t* K = (const uint16_t*)g.K + (long long)z * g.k_bs;
     const uint16_t* V = (const uint16_t*)g.V + (long long)z * g.v_bs;
-    const float sc = g.scale * 1.44269504088896341f;                // scores are kept in units of log2 e
+    // exp(scale * s - max) = exp2(s * sc - max * sc) with sc = |scale| log2 e: one fused multiply-add per score; a
+    // negative scale flips the sign of the scores first, so that the running maximum can be kept on the raw scores
+    const float sc = fabsf(g.scale) * 1.44269504088896341f;
+    const bool flip = g.scale < 0.f;
 
     // Q^T as a B operand: lane (h, c) holds d = 16*ks + 8h .. +7 of query row q0 + c (zero beyond sq)
     const char* q_end = (const char*)(Q + ((long long)(g.sq - 1) * g.q_rs + D));
@@ -64,28 +90,32 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_fwd16_kernel(A
     for (int ks = 0; ks < KS; ks++)
         qf[ks] = __builtin_bit_cast(s16x8_t, __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, (int)(((long long)c * g.q_rs + 16 * ks + 8 * h) * 2), 0, 0));
 
-    // K as an A operand: lane (h, c) holds d = 16*ks + 8h .. +7 of key kb + c; rows past sk read zeros and are masked below
+    // K and V blocks [32 keys][D] go to LDS, 16 bytes per thread and piece, in whole rows (every cache line is
+    // requested once per workgroup; fragment loads straight from global memory would touch 32 lines per instruction
+    // and per wave, which the vector cache's tag pipeline cannot keep up with).  Rows past sk read zeros.
     const char* k_end = (const char*)(K + ((long long)(g.sk - 1) * g.k_rs + D));
-    const uint32_t k_voff = (uint32_t)(((long long)c * g.k_rs + 8 * h) * 2);
-    auto load_k = [&](s16x8_t (&kf)[KS], int kb) {
-        const char* kp = (const char*)(K + (long long)kb * g.k_rs);
-        const __amdgpu_buffer_rsrc_t k_rsrc = m16_rsrc(kp, kb < g.sk ? (long long)(k_end - kp) : 0);
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) kf[ks] = __builtin_bit_cast(s16x8_t, __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, (int)k_voff, 32 * ks, 0));
-    };
-
-    // V block [32 keys][D] into LDS, 16 bytes per thread and piece
     const char* v_end = (const char*)(V + ((long long)(g.sk - 1) * g.v_rs + D));
-    auto load_v = [&](u32x4_t (&vr)[VPIECES], int kb) {
-        const char* vp = (const char*)(V + (long long)kb * g.v_rs);
-        const __amdgpu_buffer_rsrc_t v_rsrc = m16_rsrc(vp, kb < g.sk ? (long long)(v_end - vp) : 0);
+    auto load_blk = [&](u32x4_t (&r)[VPIECES], const uint16_t* M, long long rs, const char* end, int kb) {
+        const char* mp = (const char*)(M + (long long)kb * rs);
+        const __amdgpu_buffer_rsrc_t rsrc = m16_rsrc(mp, kb < g.sk ? (long long)(end - mp) : 0);
 #pragma unroll
         for (int i = 0; i < VPIECES; i++) {
             const int id = threadIdx.x + 256 * i, key = id / (D / 8), d8 = (id % (D / 8)) * 8;
             const bool live = AT_KEYS * D / 8 >= 256 || id < AT_KEYS * D / 8;
-            vr[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, live ? (int)(((long long)key * g.v_rs + d8) * 2) : (int)M16_OOB, 0, 0);
+            r[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, live ? (int)(((long long)key * rs + d8) * 2) : (int)M16_OOB, 0, 0);
         }
     };
+    auto load_v = [&](u32x4_t (&vr)[VPIECES], int kb) { load_blk(vr, V, g.v_rs, v_end, kb); };
+    auto load_k = [&](u32x4_t (&kr)[VPIECES], int kb) { load_blk(kr, K, g.k_rs, k_end, kb); };
+    // K as an A operand of the first product: lane (h, c) reads d = 16*ks + 8h .. +7 of key row c
+    auto store_k = [&](const u32x4_t (&kr)[VPIECES], uint16_t* stage) {
+#pragma unroll
+        for (int i = 0; i < VPIECES; i++) {
+            const int id = threadIdx.x + 256 * i, key = id / (D / 8), d8 = (id % (D / 8)) * 8;
+            if (AT_KEYS * D / 8 >= 256 || id < AT_KEYS * D / 8) *(u32x4_t*)(stage + key * RP + d8) = kr[i];
+        }
+    };
+    const int k_fr0 = c * RP + 8 * h;
     auto store_v = [&](const u32x4_t (&vr)[VPIECES], uint16_t* stage) {
 #pragma unroll
         for (int i = 0; i < VPIECES; i++) {
@@ -113,31 +143,32 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_fwd16_kernel(A
     for (int dt = 0; dt < DT; dt++)
 #pragma unroll
         for (int v = 0; v < 16; v++) ot[dt][v] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;            // running maximum (log2 units) and this lane's share of the running sum
+    float m_run = -INFINITY, l_run = 0.f;            // running maximum (of the raw, sign-adjusted scores) and this lane's share of the running sum
 
     const int nblocks = (g.sk + AT_KEYS - 1) / AT_KEYS;
-    s16x8_t kf[2][KS];
-    u32x4_t vr[VPIECES];
-    load_k(kf[0], 0);
+    u32x4_t kr[VPIECES], vr[VPIECES];
+    load_k(kr, 0);
     load_v(vr, 0);
+    store_k(kr, klds[0]);
     store_v(vr, vlds[0]);
-    load_k(kf[1], AT_KEYS);
+    load_k(kr, AT_KEYS);
     load_v(vr, AT_KEYS);
     __syncthreads();
 
-    auto step = [&](int blk, auto slotc) {
-        constexpr int SLOT = decltype(slotc)::value;
+    auto step = [&](int blk) {
         const int kb = blk * AT_KEYS;
         const uint16_t* stage = vlds[blk & 1];
+        const uint16_t* kstage = klds[blk & 1];
         // scores of 32 keys x 32 queries
         f32x16_t st;
 #pragma unroll
         for (int v = 0; v < 16; v++) st[v] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) st = mfma16_ops<T>::mma(kf[SLOT][ks], qf[ks], st);
-        load_k(kf[SLOT], kb + 2 * AT_KEYS);                 // this slot's next use is two blocks on
-        // V of the next block goes to the other stage (everyone left it at the previous barrier); then request the one after
+        for (int ks = 0; ks < KS; ks++) st = mfma16_ops<T>::mma(*(const s16x8_t*)(kstage + k_fr0 + 16 * ks), qf[ks], st);
+        // the next block goes to the other stage (everyone left it at the previous barrier); then request the one after
+        store_k(kr, klds[(blk & 1) ^ 1]);
         store_v(vr, vlds[(blk & 1) ^ 1]);
+        load_k(kr, kb + 2 * AT_KEYS);
         load_v(vr, kb + 2 * AT_KEYS);
 
         // this step's V^T fragments, requested before the softmax arithmetic that hides their latency
@@ -147,9 +178,12 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_fwd16_kernel(A
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) vfr[t][dt] = read_v(stage, dt, t);
 
+        if (flip) {
 #pragma unroll
-        for (int v = 0; v < 16; v++) st[v] *= sc;
-        if (kb + AT_KEYS > g.sk) {                          // the last block of a ragged sk
+            for (int v = 0; v < 16; v++) st[v] = -st[v];
+        }
+        const bool ragged = kb + AT_KEYS > g.sk;            // the last block of a ragged sk
+        if (ragged) {
 #pragma unroll
             for (int v = 0; v < 16; v++)
                 if (kb + 8 * (v / 4) + 4 * h + (v % 4) >= g.sk) st[v] = -INFINITY;
@@ -161,15 +195,19 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_fwd16_kernel(A
         mx = fmaxf(other, mx);
         // a query row beyond sq (or a block of masked keys met first) keeps mx = -inf: exp2(-inf - -inf) must not produce NaN
         const float m_use = mx == -INFINITY ? 0.f : mx;
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+        const float msc = m_use * sc;
+        const float alpha = __builtin_amdgcn_exp2f(m_run == -INFINITY ? -INFINITY : m_run * sc - msc);
         float psum = 0.f;
-        T p[16];
+        float e[16];
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const float e = __builtin_amdgcn_exp2f(st[v] - m_use);
-            p[v] = narrow<T>(e);
-            psum += widen(p[v]);                            // the sum counts the probabilities the second product sees
+        for (int v = 0; v < 16; v++) e[v] = __builtin_amdgcn_exp2f(fmaf(st[v], sc, -msc));
+        if (ragged) {                                       // a masked score times a zero scale would be NaN, not 0
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+                if (kb + 8 * (v / 4) + 4 * h + (v % 4) >= g.sk) e[v] = 0.f;
         }
+#pragma unroll
+        for (int v = 0; v < 16; v++) psum += e[v];
         l_run = l_run * alpha + psum;
         m_run = mx;
         if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {   // once the running maxima have settled there is nothing to rescale
@@ -181,18 +219,13 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_fwd16_kernel(A
         // O^T += V^T * P^T, 16 keys per MFMA
 #pragma unroll
         for (int t = 0; t < 2; t++) {
-            s16x8_t pb;
-#pragma unroll
-            for (int e = 0; e < 8; e++) pb[e] = (short)p[8 * t + e].bits;
+            const s16x8_t pb = pack8<T>(e + 8 * t);
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) ot[dt] = mfma16_ops<T>::mma(vfr[t][dt], pb, ot[dt]);
         }
         __syncthreads();                                    // next stage is written, this one is free
     };
-    for (int blk = 0; blk < nblocks; blk += 2) {
-        step(blk, std::integral_constant<int, 0>{});
-        if (blk + 1 < nblocks) step(blk + 1, std::integral_constant<int, 1>{});
-    }
+    for (int blk = 0; blk < nblocks; blk++) step(blk);
 
     // finish: the two lanes of a query add their sums; O[q][d] = O^T[d][q] / l
     const float l_all = l_run + __shfl_xor(l_run, 32, 64);
@@ -212,7 +245,7 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_fwd16_kernel(A
                 memcpy(&w, out, 8);
                 *(uint2*)(orow + 32 * dt + 8 * v4 + 4 * h) = w;
             }
-        if (g.L && h == 0) g.L[(long long)z * g.sq + q] = (m_run + __builtin_amdgcn_logf(l_all)) * 0.693147180559945309f;   // natural log of the row sum of exp(scale * s)
+        if (g.L && h == 0) g.L[(long long)z * g.sq + q] = (m_run * sc + __builtin_amdgcn_logf(l_all)) * 0.693147180559945309f;   // natural log of the row sum of exp(scale * s)
     }
 }
 
@@ -260,6 +293,21 @@ struct AttnBlock {
             if (AT_KEYS * D / 8 >= 256 || id < AT_KEYS * D / 8) *(u32x4_t*)(stage + row * VP + d8) = r[i];
         }
     }
+    // the same block kept a second way, for operands whose fragments are 8 consecutive d of one row (ds_read_b128):
+    // the pitch is 16 bytes past a multiple of 128, which spreads 16 rows over all banks
+    static constexpr int RP = D + 8;
+    static constexpr int ROW_ELEMS = AT_KEYS * RP;
+    static __device__ __forceinline__ void store_rows(const u32x4_t (&r)[PIECES], uint16_t* stage) {
+#pragma unroll
+        for (int i = 0; i < PIECES; i++) {
+            const int id = threadIdx.x + 256 * i, row = id / (D / 8), d8 = (id % (D / 8)) * 8;
+            if (AT_KEYS * D / 8 >= 256 || id < AT_KEYS * D / 8) *(u32x4_t*)(stage + row * RP + d8) = r[i];
+        }
+    }
+    // fragment ks of block row c: d = 16*ks + 8h .. +7 (an A operand with row = lane % 32)
+    static __device__ __forceinline__ s16x8_t frag(const uint16_t* stage, int c, int h, int ks) {
+        return *(const s16x8_t*)(stage + c * RP + 16 * ks + 8 * h);
+    }
     // lane's base offset for transposed reads: k slot e of MFMA t <-> block row 16t + 8*(e/4) + 4*(lane/32) + e%4
     static __device__ __forceinline__ int tr_base(int lane) {
         const int grp = lane >> 4, s16 = lane & 15;
@@ -291,7 +339,9 @@ template <typename T, int D>
 __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_bwd_dq16_kernel(AttnBwdArgs g) {
     constexpr int KS = D / 16, DT = D / 32;
     using Blk = AttnBlock<D>;
-    __shared__ __attribute__((aligned(16))) uint16_t klds[2][Blk::ELEMS];
+    __shared__ __attribute__((aligned(16))) uint16_t klds[2][Blk::ELEMS];           // K for transposed reads (K^T of the dQ product)
+    __shared__ __attribute__((aligned(16))) uint16_t krows[2][Blk::ROW_ELEMS];       // K and V for row fragments (S^T and dP^T)
+    __shared__ __attribute__((aligned(16))) uint16_t vrows[2][Blk::ROW_ELEMS];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int h = lane >> 5, c = lane & 31;
@@ -329,6 +379,7 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_bwd_dq16_kerne
         dq_dot += __shfl_xor(dq_dot, 32, 64);
         if (q < g.sq && h == 0) g.Dq[(long long)z * g.sq + q] = dq_dot;
     }
+    const float dq_dot_scaled = dq_dot * g.scale;
 
     f32x16_t acc[DT];
 #pragma unroll
@@ -338,13 +389,14 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_bwd_dq16_kerne
 
     const int tr0 = Blk::tr_base(lane);
     const int nblocks = (g.sk + AT_KEYS - 1) / AT_KEYS;
-    s16x8_t kf[KS], vf[KS];                  // A operands: row = key kb + c; reloaded for the next block right after their last use
-    u32x4_t kr[Blk::PIECES];
-    attn_load_rows<KS>(kf, K, g.k_rs, 0, g.sk, k_end, c, h);
-    attn_load_rows<KS>(vf, V, g.v_rs, 0, g.sk, v_end, c, h);
+    // K and V blocks are staged by the whole workgroup with row-contiguous loads (fragment loads straight from
+    // global memory touch 32 cache lines per instruction and wave, more than the vector cache's tag pipeline sustains)
+    u32x4_t kr[Blk::PIECES], vr[Blk::PIECES];
     Blk::load(kr, K, g.k_rs, 0, g.sk, k_end);
-    Blk::store(kr, klds[0]);
+    Blk::load(vr, V, g.v_rs, 0, g.sk, v_end);
+    Blk::store(kr, klds[0]); Blk::store_rows(kr, krows[0]); Blk::store_rows(vr, vrows[0]);
     Blk::load(kr, K, g.k_rs, AT_KEYS, g.sk, k_end);
+    Blk::load(vr, V, g.v_rs, AT_KEYS, g.sk, v_end);
     __syncthreads();
 
     auto step = [&](int blk) {
@@ -353,36 +405,34 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_bwd_dq16_kerne
         f32x16_t st, dp;
 #pragma unroll
         for (int v = 0; v < 16; v++) { st[v] = 0.f; dp[v] = 0.f; }
+        const int cur = blk & 1;
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) st = mfma16_ops<T>::mma(kf[ks], qf[ks], st);        // S^T: keys x queries
+        for (int ks = 0; ks < KS; ks++) st = mfma16_ops<T>::mma(Blk::frag(krows[cur], c, h, ks), qf[ks], st);        // S^T: keys x queries
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) dp = mfma16_ops<T>::mma(vf[ks], dof[ks], dp);       // dP^T
-        attn_load_rows<KS>(kf, K, g.k_rs, kb + AT_KEYS, g.sk, k_end, c, h);
-        attn_load_rows<KS>(vf, V, g.v_rs, kb + AT_KEYS, g.sk, v_end, c, h);
+        for (int ks = 0; ks < KS; ks++) dp = mfma16_ops<T>::mma(Blk::frag(vrows[cur], c, h, ks), dof[ks], dp);       // dP^T
         // this step's K^T fragments, requested before the arithmetic that hides their latency
         s16x8_t ktf[2][DT];
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) ktf[t][dt] = Blk::read_tr(stage, tr0, dt, t);
-        Blk::store(kr, klds[(blk & 1) ^ 1]);
+        Blk::store(kr, klds[cur ^ 1]); Blk::store_rows(kr, krows[cur ^ 1]); Blk::store_rows(vr, vrows[cur ^ 1]);
         Blk::load(kr, K, g.k_rs, kb + 2 * AT_KEYS, g.sk, k_end);
-        T ds[16];
+        Blk::load(vr, V, g.v_rs, kb + 2 * AT_KEYS, g.sk, v_end);
+        float ds[16];
 #pragma unroll
         for (int v = 0; v < 16; v++) {
-            const float p = widen(narrow<T>(__builtin_amdgcn_exp2f(st[v] * sc - lq)));     // the P the forward multiplied with
-            ds[v] = narrow<T>(p * (dp[v] - dq_dot) * g.scale);
+            const float p = __builtin_amdgcn_exp2f(fmaf(st[v], sc, -lq));
+            ds[v] = p * fmaf(dp[v], g.scale, -dq_dot_scaled);                  // P o (dP - Dq) * scale
         }
         if (kb + AT_KEYS > g.sk) {                          // the last block of a ragged sk: keys past the end count for nothing
 #pragma unroll
             for (int v = 0; v < 16; v++)
-                if (kb + 8 * (v / 4) + 4 * h + (v % 4) >= g.sk) ds[v].bits = 0;
+                if (kb + 8 * (v / 4) + 4 * h + (v % 4) >= g.sk) ds[v] = 0.f;
         }
 #pragma unroll
         for (int t = 0; t < 2; t++) {
-            s16x8_t dsb;
-#pragma unroll
-            for (int e = 0; e < 8; e++) dsb[e] = (short)ds[8 * t + e].bits;
+            const s16x8_t dsb = pack8<T>(ds + 8 * t);
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) acc[dt] = mfma16_ops<T>::mma(ktf[t][dt], dsb, acc[dt]);      // dQ^T += K^T dS^T
         }
@@ -407,12 +457,17 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_bwd_dq16_kerne
 
 // dK and dV: a wave owns 32 keys and walks the queries.
 template <typename T, int D>
-__global__ void __launch_bounds__(256) attention_bwd_dkv16_kernel(AttnBwdArgs g) {
+__global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) attention_bwd_dkv16_kernel(AttnBwdArgs g) {
     constexpr int KS = D / 16, DT = D / 32;
     using Blk = AttnBlock<D>;
-    __shared__ __attribute__((aligned(16))) uint16_t qlds[2][Blk::ELEMS];
-    __shared__ __attribute__((aligned(16))) uint16_t dolds[2][Blk::ELEMS];
-    __shared__ __attribute__((aligned(16))) float rowlds[2][2][AT_KEYS];        // [stage][L, Dq][query of the block]
+    // dynamic LDS (above 64 KB for d = 128): Q and dO blocks, each kept for transposed reads (Q^T, dO^T of the dK and
+    // dV products) and for row fragments (S and dP), two stages; then L and Dq of the block's queries
+    extern __shared__ __attribute__((aligned(16))) uint16_t dkv_lds[];
+    uint16_t (*qlds)[Blk::ELEMS] = (uint16_t (*)[Blk::ELEMS])dkv_lds;
+    uint16_t (*dolds)[Blk::ELEMS] = (uint16_t (*)[Blk::ELEMS])(dkv_lds + 2 * Blk::ELEMS);
+    uint16_t (*qrows)[Blk::ROW_ELEMS] = (uint16_t (*)[Blk::ROW_ELEMS])(dkv_lds + 4 * Blk::ELEMS);
+    uint16_t (*dorows)[Blk::ROW_ELEMS] = (uint16_t (*)[Blk::ROW_ELEMS])(dkv_lds + 4 * Blk::ELEMS + 2 * Blk::ROW_ELEMS);
+    float (*rowlds)[2][AT_KEYS] = (float (*)[2][AT_KEYS])(dkv_lds + 4 * Blk::ELEMS + 4 * Blk::ROW_ELEMS);        // [stage][L, Dq][query of the block]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int h = lane >> 5, c = lane & 31;
@@ -442,11 +497,10 @@ __global__ void __launch_bounds__(256) attention_bwd_dkv16_kernel(AttnBwdArgs g)
 
     const int tr0 = Blk::tr_base(lane);
     const int nblocks = (g.sq + AT_KEYS - 1) / AT_KEYS;
-    s16x8_t qf[KS], dof[KS];                 // A operands: row = query qb + c; reloaded for the next block right after their last use
     u32x4_t qr[Blk::PIECES], dor[Blk::PIECES];
     // L and Dq of the block's 32 queries: every lane requests query qb + lane % 32 (buffer loads, zero past sq, so
     // that no branch surrounds them and the wait for them can be counted); wave 0 puts them in LDS: its lower half
-    // the L (in log2 units, +inf past sq, which makes those rows' probabilities exactly 0), its upper half the Dq
+    // the L (in log2 units, +inf past sq, which makes those rows' probabilities exactly 0), its upper half Dq * scale
     const __amdgpu_buffer_rsrc_t l_rsrc = m16_rsrc(Lz, (long long)g.sq * 4), d_rsrc = m16_rsrc(Dz, (long long)g.sq * 4);
     float row_l = 0.f, row_d = 0.f;
     auto load_rowv = [&](int qb) {
@@ -454,15 +508,13 @@ __global__ void __launch_bounds__(256) attention_bwd_dkv16_kernel(AttnBwdArgs g)
         row_d = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(d_rsrc, (qb + c) * 4, 0, 0));
     };
     auto store_rowv = [&](int stage, int qb) {
-        if (wave == 0) rowlds[stage][h][c] = h ? row_d : (qb + c < g.sq ? row_l * 1.44269504088896341f : INFINITY);
+        if (wave == 0) rowlds[stage][h][c] = h ? row_d * g.scale : (qb + c < g.sq ? row_l * 1.44269504088896341f : INFINITY);
     };
-    attn_load_rows<KS>(qf, Q, g.q_rs, 0, g.sq, q_end, c, h);
-    attn_load_rows<KS>(dof, dO, g.do_rs, 0, g.sq, do_end, c, h);
     Blk::load(qr, Q, g.q_rs, 0, g.sq, q_end);
     Blk::load(dor, dO, g.do_rs, 0, g.sq, do_end);
     load_rowv(0);
-    Blk::store(qr, qlds[0]);
-    Blk::store(dor, dolds[0]);
+    Blk::store(qr, qlds[0]); Blk::store_rows(qr, qrows[0]);
+    Blk::store(dor, dolds[0]); Blk::store_rows(dor, dorows[0]);
     store_rowv(0, 0);
     Blk::load(qr, Q, g.q_rs, AT_KEYS, g.sq, q_end);
     Blk::load(dor, dO, g.do_rs, AT_KEYS, g.sq, do_end);
@@ -476,35 +528,31 @@ __global__ void __launch_bounds__(256) attention_bwd_dkv16_kernel(AttnBwdArgs g)
 #pragma unroll
         for (int v = 0; v < 16; v++) { st[v] = 0.f; dp[v] = 0.f; }
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) st = mfma16_ops<T>::mma(qf[ks], kf[ks], st);        // S: queries x keys
+        for (int ks = 0; ks < KS; ks++) st = mfma16_ops<T>::mma(Blk::frag(qrows[cur], c, h, ks), kf[ks], st);        // S: queries x keys
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) dp = mfma16_ops<T>::mma(dof[ks], vf[ks], dp);       // dP
-        attn_load_rows<KS>(qf, Q, g.q_rs, qb + AT_KEYS, g.sq, q_end, c, h);
-        attn_load_rows<KS>(dof, dO, g.do_rs, qb + AT_KEYS, g.sq, do_end, c, h);
-        Blk::store(qr, qlds[cur ^ 1]);
-        Blk::store(dor, dolds[cur ^ 1]);
+        for (int ks = 0; ks < KS; ks++) dp = mfma16_ops<T>::mma(Blk::frag(dorows[cur], c, h, ks), vf[ks], dp);       // dP
+        Blk::store(qr, qlds[cur ^ 1]); Blk::store_rows(qr, qrows[cur ^ 1]);
+        Blk::store(dor, dolds[cur ^ 1]); Blk::store_rows(dor, dorows[cur ^ 1]);
         store_rowv(cur ^ 1, qb + AT_KEYS);
         Blk::load(qr, Q, g.q_rs, qb + 2 * AT_KEYS, g.sq, q_end);
         Blk::load(dor, dO, g.do_rs, qb + 2 * AT_KEYS, g.sq, do_end);
         load_rowv(qb + 2 * AT_KEYS);
-        T p[16], ds[16];
+        float p[16], ds[16];
 #pragma unroll
         for (int v4 = 0; v4 < 4; v4++) {
-            // registers 4*v4 .. 4*v4+3 are queries qb + 8*v4 + 4h + (0..3): their L and Dq are 16 contiguous bytes each
+            // registers 4*v4 .. 4*v4+3 are queries qb + 8*v4 + 4h + (0..3): their L and scaled Dq are 16 contiguous bytes each
             const f32x4_t l4 = *(const f32x4_t*)&rowlds[cur][0][8 * v4 + 4 * h];
             const f32x4_t d4 = *(const f32x4_t*)&rowlds[cur][1][8 * v4 + 4 * h];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int v = 4 * v4 + e;
-                p[v] = narrow<T>(__builtin_amdgcn_exp2f(st[v] * sc - l4[e]));          // 0 for a query past sq: its L is +inf
-                ds[v] = narrow<T>(widen(p[v]) * (dp[v] - d4[e]) * g.scale);
+                p[v] = __builtin_amdgcn_exp2f(fmaf(st[v], sc, -l4[e]));          // 0 for a query past sq: its L is +inf
+                ds[v] = p[v] * fmaf(dp[v], g.scale, -d4[e]);                      // P o (dP - Dq) * scale
             }
         }
 #pragma unroll
         for (int t = 0; t < 2; t++) {
-            s16x8_t pb, dsb;
-#pragma unroll
-            for (int e = 0; e < 8; e++) { pb[e] = (short)p[8 * t + e].bits; dsb[e] = (short)ds[8 * t + e].bits; }
+            const s16x8_t pb = pack8<T>(p + 8 * t), dsb = pack8<T>(ds + 8 * t);
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) {
                 dvt[dt] = mfma16_ops<T>::mma(Blk::read_tr(dolds[cur], tr0, dt, t), pb, dvt[dt]);      // dV^T += dO^T P
@@ -533,25 +581,28 @@ __global__ void __launch_bounds__(256) attention_bwd_dkv16_kernel(AttnBwdArgs g)
     }
 }
 
+template <int D>
+constexpr size_t attn_dkv_lds_bytes() { return (size_t)(4 * AttnBlock<D>::ELEMS + 4 * AttnBlock<D>::ROW_ELEMS) * 2 + 2 * 2 * AT_KEYS * sizeof(float); }
+
+template <typename T, int D>
+static int launch_attention_bwd_d(const AttnBwdArgs& g) {
+    dim3 gq((g.sq + AT_QROWS - 1) / AT_QROWS, g.batch), gk((g.sk + AT_QROWS - 1) / AT_QROWS, g.batch);
+    constexpr size_t smem = attn_dkv_lds_bytes<D>();
+    auto dkv = attention_bwd_dkv16_kernel<T, D>;
+    if (smem > 64 * 1024 && !check_hip(hipFuncSetAttribute((const void*)dkv, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem), "hipFuncSetAttribute")) return -1;
+    hipLaunchKernelGGL((attention_bwd_dq16_kernel<T, D>), gq, dim3(256), 0, current_stream(), g);
+    hipLaunchKernelGGL(dkv, gk, dim3(256), smem, current_stream(), g);
+    return check_launch("attention backward kernels") ? 0 : -1;
+}
+
 template <typename T>
 static int launch_attention_bwd_t(const AttnBwdArgs& g, int d) {
-    dim3 gq((g.sq + AT_QROWS - 1) / AT_QROWS, g.batch), gk((g.sk + AT_QROWS - 1) / AT_QROWS, g.batch);
     switch (d) {
-        case 32:
-            hipLaunchKernelGGL((attention_bwd_dq16_kernel<T, 32>), gq, dim3(256), 0, current_stream(), g);
-            hipLaunchKernelGGL((attention_bwd_dkv16_kernel<T, 32>), gk, dim3(256), 0, current_stream(), g);
-            break;
-        case 64:
-            hipLaunchKernelGGL((attention_bwd_dq16_kernel<T, 64>), gq, dim3(256), 0, current_stream(), g);
-            hipLaunchKernelGGL((attention_bwd_dkv16_kernel<T, 64>), gk, dim3(256), 0, current_stream(), g);
-            break;
-        case 128:
-            hipLaunchKernelGGL((attention_bwd_dq16_kernel<T, 128>), gq, dim3(256), 0, current_stream(), g);
-            hipLaunchKernelGGL((attention_bwd_dkv16_kernel<T, 128>), gk, dim3(256), 0, current_stream(), g);
-            break;
+        case 32: return launch_attention_bwd_d<T, 32>(g);
+        case 64: return launch_attention_bwd_d<T, 64>(g);
+        case 128: return launch_attention_bwd_d<T, 128>(g);
         default: set_error("rp_hip_attention_backward: head dimension %d (supported: 32, 64, 128)", d); return -1;
     }
-    return check_launch("attention backward kernels") ? 0 : -1;
 }
 
 template <typename T>
