@@ -305,25 +305,24 @@ def attention_times(capi, dt_name="bf16"):
         if flops:
             out[name]["TFLOP/s"] = round(flops / ms / 1e9, 1)
     out["fwd_bwd_ms"] = round(total + out["scale"]["us"] * 1e-3, 4)     # the scale runs twice (S/8 and dS/8)
-    if dt == capi.BF16:
-        # the same forward (S, scale, softmax, O) as one fused kernel that never writes S or P
-        fused = lambda: capi.check(L.rp_hip_attention_forward(d_o.ptr, d_q.ptr, d_k.ptr, d_v.ptr, None, Z, S, S, D,
-                                                              sd, D, sd, D, sd, D, sd, D, 0.125, dt), "rp_hip_attention_forward")
-        ms = _time_graph(capi, fused, 10, 2)
-        chain = sum(out[k]["us"] for k in ("S=Q.Kt", "scale", "softmax", "O=P.V"))
-        nbytes = 4 * sd * Z * esz
-        out["fused_forward"] = {"us": round(ms * 1e3, 1), "unfused_chain_us": round(chain, 1), "TFLOP/s": round(4.0 * Z * S * S * D / ms / 1e9, 1),
-                                "GB/s": round(nbytes / ms / 1e6, 1)}
-        # and the backward (dQ, dK, dV from Q, K, V, O, dO and the saved row statistics) as two launches
-        d_lse = D_(Z * S * 4)
-        capi.check(L.rp_hip_attention_forward(d_o.ptr, d_q.ptr, d_k.ptr, d_v.ptr, d_lse.ptr, Z, S, S, D, sd, D, sd, D, sd, D, sd, D, 0.125, dt), "rp_hip_attention_forward")
-        fused_b = lambda: capi.check(L.rp_hip_attention_backward(d_dq.ptr, d_dk.ptr, d_dv.ptr, d_q.ptr, d_k.ptr, d_v.ptr, d_o.ptr, d_do.ptr, d_lse.ptr,
-                                                                 Z, S, S, D, sd, D, sd, D, sd, D, sd, D, sd, D, 0.125, dt), "rp_hip_attention_backward")
-        fused_b()
-        msb = _time_graph(capi, fused_b, 10, 2)
-        chain_b = out["fwd_bwd_ms"] * 1e3 - chain
-        out["fused_backward"] = {"us": round(msb * 1e3, 1), "unfused_chain_us": round(chain_b, 1), "TFLOP/s": round(10.0 * Z * S * S * D / msb / 1e9, 1)}
-        out["fused_fwd_bwd_ms"] = round(ms + msb, 4)
+    # the same forward (S, scale, softmax, O) as one fused kernel that never writes S or P
+    fused = lambda: capi.check(L.rp_hip_attention_forward(d_o.ptr, d_q.ptr, d_k.ptr, d_v.ptr, None, Z, S, S, D,
+                                                          sd, D, sd, D, sd, D, sd, D, 0.125, dt), "rp_hip_attention_forward")
+    ms = _time_graph(capi, fused, 10, 2)
+    chain = sum(out[k]["us"] for k in ("S=Q.Kt", "scale", "softmax", "O=P.V"))
+    nbytes = 4 * sd * Z * esz
+    out["fused_forward"] = {"us": round(ms * 1e3, 1), "unfused_chain_us": round(chain, 1), "TFLOP/s": round(4.0 * Z * S * S * D / ms / 1e9, 1),
+                            "GB/s": round(nbytes / ms / 1e6, 1)}
+    # and the backward (dQ, dK, dV from Q, K, V, O, dO and the saved row statistics) as two launches
+    d_lse = D_(Z * S * 4)
+    capi.check(L.rp_hip_attention_forward(d_o.ptr, d_q.ptr, d_k.ptr, d_v.ptr, d_lse.ptr, Z, S, S, D, sd, D, sd, D, sd, D, sd, D, 0.125, dt), "rp_hip_attention_forward")
+    fused_b = lambda: capi.check(L.rp_hip_attention_backward(d_dq.ptr, d_dk.ptr, d_dv.ptr, d_q.ptr, d_k.ptr, d_v.ptr, d_o.ptr, d_do.ptr, d_lse.ptr,
+                                                             Z, S, S, D, sd, D, sd, D, sd, D, sd, D, sd, D, 0.125, dt), "rp_hip_attention_backward")
+    fused_b()
+    msb = _time_graph(capi, fused_b, 10, 2)
+    chain_b = out["fwd_bwd_ms"] * 1e3 - chain
+    out["fused_backward"] = {"us": round(msb * 1e3, 1), "unfused_chain_us": round(chain_b, 1), "TFLOP/s": round(10.0 * Z * S * S * D / msb / 1e9, 1)}
+    out["fused_fwd_bwd_ms"] = round(ms + msb, 4)
     return out
 
 

@@ -239,13 +239,13 @@ int rp_hip_gru_cell_backward(void* dgi, void* dgh, void* dh_prev, const void* dh
 int rp_hip_scatter_strided(void* dst, const void* src, int ndim, const int* shape, const long long* dst_strides,
                            size_t size, int dtype);
 
-/* Fused attention forward for bfloat16 / float16: O[b] = softmax(scale * Q[b] * K[b]^T) * V[b], the score matrix never
- * leaves the chip.  Q, O: [batch, sq, d]; K, V: [batch, sk, d]; d in {32, 64, 128} and contiguous (unit stride);
- * *_bs / *_rs are the batch and row strides in elements (multiples of 8; operands 16-byte aligned).
- * lse (may be NULL): float32 [batch, sq], log of the row sums of exp(scale * scores), for a backward pass.
- * No counterpart in the reference, which composes the same value from op_matmul, op_mul_scalar, op_softmax and
- * op_matmul (ops/ops.c:6816-6884, 6022-6086, 5721-5788) and rounds the scores to the tensor dtype on the way;
- * here only the probabilities are rounded (as the reference's P is), accumulation is float32. */
+/* Fused attention forward: O[b] = softmax(scale * Q[b] * K[b]^T) * V[b], the score matrix never leaves the chip.
+ * bfloat16 / float16 with d in {32, 64, 128}, float32 with d in {32, 64}.  Q, O: [batch, sq, d]; K, V: [batch, sk, d];
+ * d contiguous (unit stride); *_bs / *_rs are the batch and row strides in elements (multiples of 16 bytes; operands
+ * 16-byte aligned).  lse (may be NULL): float32 [batch, sq], log of the row sums of exp(scale * scores), for a backward
+ * pass.  No counterpart in the reference, which composes the same value from op_matmul, op_mul_scalar, op_softmax and
+ * op_matmul (ops/ops.c:6816-6884, 6022-6086, 5721-5788) and rounds the scores to the tensor dtype on the way; here
+ * only the probabilities of the 16-bit types are rounded (to 16 bits, nearest even), accumulation is float32. */
 int rp_hip_attention_forward(void* O, const void* Q, const void* K, const void* V, float* lse,
                              int batch, int sq, int sk, int d,
                              long long q_bs, long long q_rs, long long k_bs, long long k_rs,

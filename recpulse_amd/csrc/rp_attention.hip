@@ -20,22 +20,9 @@
 // Probabilities are narrowed to the tensor dtype before the second product (as the reference's P is), accumulation is
 // fp32 throughout, and the scores themselves are never rounded to 16 bits (the reference rounds S and S*scale).
 #include "rp_gemm_mfma16_kernel.h"
+#include "rp_attention.h"
 
 namespace rp {
-
-struct AttnArgs {
-    void* O;
-    const void* Q;
-    const void* K;
-    const void* V;
-    float* L;                   // optional [batch, sq] row-wise log-sum-exp of the scaled scores
-    int batch, sq, sk;
-    long long q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs;      // in elements; the head dimension is contiguous
-    float scale;
-};
-
-constexpr int AT_KEYS = 32;                 // keys per step
-constexpr int AT_QROWS = 128;               // query rows per workgroup (32 per wave)
 
 // Two fp32 values to a pair of T with the hardware's packed round-to-nearest-even conversion (one instruction for
 // two values).  The probabilities and the score gradients packed with it exist only inside the fused kernels, as MFMA
@@ -260,16 +247,6 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_fwd16_kernel(A
 // registers; the ones that must be read transposed (K^T for dQ; dO^T and Q^T for dV and dK) go through LDS and
 // ds_read_tr16_b64.
 // ============================================================================
-struct AttnBwdArgs {
-    void* dQ; void* dK; void* dV;           // dense [batch, s, d]
-    const void* Q; const void* K; const void* V; const void* O; const void* dO;
-    const float* L;                         // [batch, sq] log-sum-exp rows from the forward
-    float* Dq;                              // [batch, sq] row dots of dO and O: written by the dQ kernel, read by the dK/dV kernel
-    int batch, sq, sk;
-    long long q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs, do_bs, do_rs;
-    float scale;
-};
-
 // A [32 rows][D] block of a d-contiguous matrix, staged in LDS for transposed MFMA operand reads.
 template <int D>
 struct AttnBlock {
@@ -630,18 +607,21 @@ extern "C" int rp_hip_attention_forward(void* O, const void* Q, const void* K, c
         set_error("rp_hip_attention_forward: null operand or non-positive extent (batch=%d sq=%d sk=%d d=%d)", batch, sq, sk, d);
         return -1;
     }
-    if (dtype != RP_DTYPE_BFLOAT16 && dtype != RP_DTYPE_FLOAT16) { set_error("rp_hip_attention_forward: bfloat16 / float16 only (dtype %d)", dtype); return -1; }
+    if (dtype != RP_DTYPE_BFLOAT16 && dtype != RP_DTYPE_FLOAT16 && dtype != RP_DTYPE_FLOAT32) { set_error("rp_hip_attention_forward: bfloat16, float16 or float32 (dtype %d)", dtype); return -1; }
+    const bool f32 = dtype == RP_DTYPE_FLOAT32;
+    const long long esz = f32 ? 4 : 2, vec = 16 / esz;
+    if (f32 ? (d != 32 && d != 64) : (d != 32 && d != 64 && d != 128)) { set_error("rp_hip_attention_forward: head dimension %d (supported: 32, 64, and 128 for the 16-bit types)", d); return -1; }
     const long long strides[] = {q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs};
     for (long long s : strides)
-        if (s < 0 || s % 8) { set_error("rp_hip_attention_forward: strides must be non-negative multiples of 8 elements"); return -1; }
+        if (s < 0 || s % vec) { set_error("rp_hip_attention_forward: strides must be non-negative multiples of 16 bytes"); return -1; }
     if (q_rs >= (1ll << 22) || k_rs >= (1ll << 22) || v_rs >= (1ll << 22)) { set_error("rp_hip_attention_forward: row stride too large"); return -1; }
     if (((uintptr_t)O | (uintptr_t)Q | (uintptr_t)K | (uintptr_t)V) & 15) { set_error("rp_hip_attention_forward: operands must be 16-byte aligned"); return -1; }
     constexpr int MAX_BATCH = 65535;
     for (int b0 = 0; b0 < batch; b0 += MAX_BATCH) {
         const int nb = batch - b0 < MAX_BATCH ? batch - b0 : MAX_BATCH;
-        AttnArgs g{(char*)O + b0 * o_bs * 2, (const char*)Q + b0 * q_bs * 2, (const char*)K + b0 * k_bs * 2, (const char*)V + b0 * v_bs * 2,
+        AttnArgs g{(char*)O + b0 * o_bs * esz, (const char*)Q + b0 * q_bs * esz, (const char*)K + b0 * k_bs * esz, (const char*)V + b0 * v_bs * esz,
                    lse ? lse + (long long)b0 * sq : nullptr, nb, sq, sk, q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs, (float)scale};
-        int rc = dtype == RP_DTYPE_BFLOAT16 ? launch_attention_t<bf16_t>(g, d) : launch_attention_t<f16_t>(g, d);
+        int rc = f32 ? launch_attention_f32(g, d) : dtype == RP_DTYPE_BFLOAT16 ? launch_attention_t<bf16_t>(g, d) : launch_attention_t<f16_t>(g, d);
         if (rc != 0) return -1;
     }
     return 0;
@@ -657,11 +637,13 @@ extern "C" int rp_hip_attention_backward(void* dQ, void* dK, void* dV, const voi
         set_error("rp_hip_attention_backward: null operand or non-positive extent (batch=%d sq=%d sk=%d d=%d)", batch, sq, sk, d);
         return -1;
     }
-    if (dtype != RP_DTYPE_BFLOAT16 && dtype != RP_DTYPE_FLOAT16) { set_error("rp_hip_attention_backward: bfloat16 / float16 only (dtype %d)", dtype); return -1; }
-    if (d != 32 && d != 64 && d != 128) { set_error("rp_hip_attention_backward: head dimension %d (supported: 32, 64, 128)", d); return -1; }
+    if (dtype != RP_DTYPE_BFLOAT16 && dtype != RP_DTYPE_FLOAT16 && dtype != RP_DTYPE_FLOAT32) { set_error("rp_hip_attention_backward: bfloat16, float16 or float32 (dtype %d)", dtype); return -1; }
+    const bool f32 = dtype == RP_DTYPE_FLOAT32;
+    const long long esz = f32 ? 4 : 2, vec = 16 / esz;
+    if (f32 ? (d != 32 && d != 64) : (d != 32 && d != 64 && d != 128)) { set_error("rp_hip_attention_backward: head dimension %d (supported: 32, 64, and 128 for the 16-bit types)", d); return -1; }
     const long long strides[] = {q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs, do_bs, do_rs};
     for (long long s : strides)
-        if (s < 0 || s % 8) { set_error("rp_hip_attention_backward: strides must be non-negative multiples of 8 elements"); return -1; }
+        if (s < 0 || s % vec) { set_error("rp_hip_attention_backward: strides must be non-negative multiples of 16 bytes"); return -1; }
     if (q_rs >= (1ll << 22) || k_rs >= (1ll << 22) || v_rs >= (1ll << 22) || o_rs >= (1ll << 22) || do_rs >= (1ll << 22)) { set_error("rp_hip_attention_backward: row stride too large"); return -1; }
     if (((uintptr_t)dQ | (uintptr_t)dK | (uintptr_t)dV | (uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)O | (uintptr_t)dO) & 15) {
         set_error("rp_hip_attention_backward: operands must be 16-byte aligned");
@@ -674,11 +656,11 @@ extern "C" int rp_hip_attention_backward(void* dQ, void* dK, void* dV, const voi
     int rc = 0;
     for (int b0 = 0; rc == 0 && b0 < batch; b0 += MAX_BATCH) {
         const int nb = batch - b0 < MAX_BATCH ? batch - b0 : MAX_BATCH;
-        const long long q_off = (long long)b0 * sq * d * 2, k_off = (long long)b0 * sk * d * 2;        // the gradients are dense
-        AttnBwdArgs g{(char*)dQ + q_off, (char*)dK + k_off, (char*)dV + k_off, (const char*)Q + b0 * q_bs * 2, (const char*)K + b0 * k_bs * 2,
-                      (const char*)V + b0 * v_bs * 2, (const char*)O + b0 * o_bs * 2, (const char*)dO + b0 * do_bs * 2, lse + (long long)b0 * sq,
+        const long long q_off = (long long)b0 * sq * d * esz, k_off = (long long)b0 * sk * d * esz;        // the gradients are dense
+        AttnBwdArgs g{(char*)dQ + q_off, (char*)dK + k_off, (char*)dV + k_off, (const char*)Q + b0 * q_bs * esz, (const char*)K + b0 * k_bs * esz,
+                      (const char*)V + b0 * v_bs * esz, (const char*)O + b0 * o_bs * esz, (const char*)dO + b0 * do_bs * esz, lse + (long long)b0 * sq,
                       (float*)dots + (long long)b0 * sq, nb, sq, sk, q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs, do_bs, do_rs, (float)scale};
-        rc = dtype == RP_DTYPE_BFLOAT16 ? launch_attention_bwd_t<bf16_t>(g, d) : launch_attention_bwd_t<f16_t>(g, d);
+        rc = f32 ? launch_attention_bwd_f32(g, d) : dtype == RP_DTYPE_BFLOAT16 ? launch_attention_bwd_t<bf16_t>(g, d) : launch_attention_bwd_t<f16_t>(g, d);
     }
     rp_hip_free(dots);        // stream-ordered reuse: the pool hands it out again only to later work on this stream
     return rc;

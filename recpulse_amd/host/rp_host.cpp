@@ -1071,14 +1071,15 @@ Tensor* op_linear(Tensor* x, Tensor* w, Tensor* bias) {
     return out;
 }
 
-// O = softmax(scale · Q · Kᵀ) · V in one launch (extension; bfloat16 / float16, head dimension 32, 64 or 128).
+// O = softmax(scale · Q · Kᵀ) · V in one launch (extension; bfloat16 / float16 with head dimension 32, 64 or 128,
+// float32 with 32 or 64).
 // q: [..., sq, d], k and v: [..., sk, d] with equal leading dims.  Equals q.op_matmul(kᵀ).op_mul_scalar(scale)
 // .op_softmax(-1).op_matmul(v) up to the roundings of the score matrix that the fused kernel does not make.
 Tensor* op_attention(Tensor* q, Tensor* k, Tensor* v, double scale) {
     if (!q || !k || !v) return nullptr;
     const int nd = q->ndim;
     if (nd < 2 || k->ndim != nd || v->ndim != nd || !same_place(q, k) || !same_place(q, v)) { fail("op_attention: rank, dtype or device mismatch"); return nullptr; }
-    if (q->dtype != DTYPE_BFLOAT16 && q->dtype != DTYPE_FLOAT16) { fail("op_attention: bfloat16 or float16 tensors only"); return nullptr; }
+    if (q->dtype == DTYPE_FLOAT64) { fail("op_attention: bfloat16, float16 or float32 tensors"); return nullptr; }
     if (q->device_id == -1) { fail("op_attention on host tensors is not provided by this build; move the operands to a GPU"); return nullptr; }
     const int sq = q->shape[nd - 2], d = q->shape[nd - 1], sk = k->shape[nd - 2];
     bool shapes = k->shape[nd - 1] == d && v->shape[nd - 1] == d && v->shape[nd - 2] == sk;

@@ -103,7 +103,7 @@ Tensor* op_conv2d(Tensor* input, Tensor* weight, Tensor* bias, int stride_h, int
 Tensor* op_slice(Tensor* x, int* start, int* stop, int* step);          /* reference ops/ops.h:51 */
 Tensor* op_lstm_cell(Tensor* x, Tensor* h, Tensor* c, Tensor* w_ih, Tensor* w_hh, Tensor* b_ih, Tensor* b_hh);   /* one step as one node: [B, 2H] = h_next | c_next (extension) */
 Tensor* op_gru_cell(Tensor* x, Tensor* h, Tensor* w_ih, Tensor* w_hh, Tensor* b_ih, Tensor* b_hh);                /* one step as one node: h_next (extension) */
-Tensor* op_attention(Tensor* q, Tensor* k, Tensor* v, double scale);   /* softmax(scale·q·kᵀ)·v in one launch (extension; 16-bit dtypes) */
+Tensor* op_attention(Tensor* q, Tensor* k, Tensor* v, double scale);   /* softmax(scale·q·kᵀ)·v in one launch (extension; 16-bit dtypes and float32) */
 Tensor* op_add(Tensor* x1, Tensor* x2);
 Tensor* op_relu(Tensor* x);
 Tensor* op_softmax(Tensor* x, int dim);
