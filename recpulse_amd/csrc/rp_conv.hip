@@ -47,7 +47,8 @@ __device__ __forceinline__ void load_span(T (&v)[VEC], const T* row, int start, 
 // neighbours in memory and come in with a single (unaligned) vector load, borders included (load_span); spans that
 // wrap to the next output row, and other strides, go one by one.  The taps' loads overlap almost entirely and hit
 // in the vector cache; the stores of a wave are whole kilobytes of one col row.
-template <typename T, int VEC>
+// TAPS3: the kernel is 3 x 3 (the tap loops unroll, so that all nine loads of a thread are in flight together).
+template <typename T, int VEC, bool TAPS3>
 __global__ void __launch_bounds__(256) im2col_kernel(T* col, const T* im, ConvGeom g, unsigned total_vec) {
     const int cols = g.oH * g.oW;
     const unsigned vec_per_row = cols / VEC;
@@ -59,8 +60,7 @@ __global__ void __launch_bounds__(256) im2col_kernel(T* col, const T* im, ConvGe
     const int p = pv * VEC;
     const int oh0 = p / g.oW, ow0 = p % g.oW;
     const bool span = VEC > 1 && g.sw == 1 && ow0 + VEC <= g.oW && g.W >= VEC;
-    for (int kh = 0; kh < g.kH; kh++)
-        for (int kw = 0; kw < g.kW; kw++, dst += cols) {
+    auto tap = [&](int kh, int kw, T* dst) {
             T v[VEC];
             if constexpr (VEC > 1) {
                 if (span) {
@@ -89,7 +89,14 @@ __global__ void __launch_bounds__(256) im2col_kernel(T* col, const T* im, ConvGe
 #pragma unroll
                 for (int e = 0; e < VEC; e++) dst[e] = v[e];
             }
-        }
+    };
+    if constexpr (TAPS3) {
+#pragma unroll
+        for (int t = 0; t < 9; t++) tap(t / 3, t % 3, dst + (size_t)t * cols);
+    } else {
+        for (int kh = 0; kh < g.kH; kh++)
+            for (int kw = 0; kw < g.kW; kw++, dst += cols) tap(kh, kw, dst);
+    }
 }
 
 // One thread per VEC neighbouring input pixels of a row (VEC = 1 when W is not a whole number of vectors).
@@ -257,8 +264,10 @@ static void launch_im2col(void* col, const void* im, const ConvGeom& g) {
         const unsigned total = (unsigned)np * per_plane;
         T* c0 = (T*)((char*)col + (size_t)p0 * g.kH * g.kW * cols * esz);
         const T* i0 = (const T*)((const char*)im + (size_t)p0 * g.H * g.W * esz);
-        if (vec) hipLaunchKernelGGL((im2col_kernel<T, VEC>), dim3((total + 255) / 256), dim3(256), 0, current_stream(), c0, i0, g, total);
-        else hipLaunchKernelGGL((im2col_kernel<T, 1>), dim3((total + 255) / 256), dim3(256), 0, current_stream(), c0, i0, g, total);
+        const dim3 grid((total + 255) / 256);
+        if (vec && g.kH == 3 && g.kW == 3) hipLaunchKernelGGL((im2col_kernel<T, VEC, true>), grid, dim3(256), 0, current_stream(), c0, i0, g, total);
+        else if (vec) hipLaunchKernelGGL((im2col_kernel<T, VEC, false>), grid, dim3(256), 0, current_stream(), c0, i0, g, total);
+        else hipLaunchKernelGGL((im2col_kernel<T, 1, false>), grid, dim3(256), 0, current_stream(), c0, i0, g, total);
     }
 }
 
