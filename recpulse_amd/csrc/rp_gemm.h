@@ -20,7 +20,7 @@ struct GemmArgs {
     int accumulate;
 };
 
-enum Family { FAM_GENERIC = 0, FAM_SKINNY, FAM_MFMA16, FAM_MFMA16_SKINNY, FAM_MFMAW };
+enum Family { FAM_GENERIC = 0, FAM_SKINNY, FAM_MFMA16, FAM_MFMA16_SKINNY, FAM_MFMAW, FAM_TINY };
 
 struct Plan {
     Family fam;
@@ -125,6 +125,7 @@ int launch_generic(const GemmArgs& g, int dtype);
 int launch_skinny(const GemmArgs& g, int dtype);
 int launch_mfma16(const GemmArgs& g, const Plan& p, int dtype);
 int launch_mfmaw(const GemmArgs& g, const Plan& p, int dtype);
+int launch_tiny(const GemmArgs& g, int dtype);
 // adds k-split partials [nsplit][part_rows][n] (fp32, rows beyond g.m unused) in split order and runs the epilogue into C
 int launch_splitk_combine(const GemmArgs& g, const float* partials, int nsplit, int part_rows, int dtype);
 

@@ -16,6 +16,7 @@
 //            transposing ds_read_b64_tr_b16, so no layout needs a copy.
 //   mfmaw    fp32 (v_mfma_f32_32x32x2_f32) and fp64 (v_mfma_f64_16x16x4_f64).
 //   skinny   m <= 8 against a row-major B: a split-k streaming kernel bound by HBM.
+//   tiny     fp32 outputs of a few hundred 16 x 16 tiles: one launch, k split over the waves of a workgroup.
 //   generic  any strides, any shape; LDS-tiled scalar FMA.
 #include "rp_gemm.h"
 
@@ -29,6 +30,12 @@ static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 static bool force_generic() {
     static int v = -1;
     if (v < 0) { const char* e = getenv("RP_HIP_FORCE_GENERIC"); v = (e && e[0] == '1') ? 1 : 0; }
+    return v == 1;
+}
+
+static bool tiny_off() {                           // RP_HIP_NO_TINY=1: small fp32 GEMMs take the tiled kernels with a k split instead
+    static int v = -1;
+    if (v < 0) { const char* e = getenv("RP_HIP_NO_TINY"); v = (e && e[0] == '1') ? 1 : 0; }
     return v == 1;
 }
 
@@ -77,6 +84,12 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
         p.fam = FAM_SKINNY; p.name = "skinny"; p.b_mc = true;
         return p;
     }
+    // fp32, an output of fewer than 64 tiles of 64 x 64 and a k that one workgroup walks in a few microseconds: one launch
+    // of 16 x 16 tiles with k split over the four waves of a workgroup, any strides (no split over workgroups, no second launch)
+    if (dtype == RP_DTYPE_FLOAT32 && k <= 2048 && (long long)((m + 63) / 64) * ((n + 63) / 64) * batch < 64 && !tiny_off()) {
+        p.fam = FAM_TINY; p.bm = 16; p.bn = 16; p.name = "tiny32_16x16";
+        return p;
+    }
     if (!mfma_ok) return p;
     p.a_mc = !a_kc;             // when both qualify (extent-1 corner cases) keep the row-major reading
     p.b_mc = b_mc;
@@ -103,12 +116,13 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
 
 static int run_gemm(const GemmArgs& g, int dtype) {
     Plan p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype);
-    if (p.fam != FAM_GENERIC && !(aligned16(g.A) && aligned16(g.B))) p.fam = FAM_GENERIC;
+    if (p.fam != FAM_GENERIC && p.fam != FAM_TINY && !(aligned16(g.A) && aligned16(g.B))) p.fam = FAM_GENERIC;
     switch (p.fam) {
         case FAM_MFMA16:
         case FAM_MFMA16_SKINNY: return launch_mfma16(g, p, dtype);
         case FAM_MFMAW:  return launch_mfmaw(g, p, dtype);
         case FAM_SKINNY: return launch_skinny(g, dtype);
+        case FAM_TINY:   return launch_tiny(g, dtype);
         default:         return launch_generic(g, dtype);
     }
 }

@@ -50,8 +50,9 @@ def test_kernel_selection_names():
     assert name(1, 32, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F16) == "mfma16_skinny_32x128"
     assert name(1, 8, 8192, 8192, (8192, 1), (1, 8192), (8192, 1), capi.BF16) == "mfma16_skinny_32x128"
     assert name(1, 8, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F32) == "skinny"
-    assert name(1, 128, 784, 256, (784, 1), (256, 1), (256, 1), capi.F32) == "mfma32_64x64"          # few tiles: small tile + split-k
+    assert name(1, 128, 784, 256, (784, 1), (256, 1), (256, 1), capi.F32) == "tiny32_16x16"          # a small fp32 output: one launch of 16 x 16 tiles
+    assert name(1, 128, 4096, 256, (4096, 1), (256, 1), (256, 1), capi.F32) == "mfma32_64x64"        # deeper k: small tile + split-k over workgroups
     assert name(1, 4096, 4096, 4096, (4096, 1), (4096, 1), (4096, 1), capi.F32) == "mfma32_128x128"
     assert name(1, 2048, 2048, 2048, (2048, 1), (2048, 1), (2048, 1), capi.F64) == "mfma64_128x128"
-    assert name(1, 5, 7, 3, (7, 1), (3, 1), (3, 1), capi.F32) == "generic"                                 # odd extents
-    assert name(1, 64, 64, 64, (128, 2), (64, 1), (64, 1), capi.F32) == "generic"                          # no unit stride
+    assert name(1, 5, 7, 3, (7, 1), (3, 1), (3, 1), capi.BF16) == "generic"                                # odd extents
+    assert name(1, 64, 64, 64, (128, 2), (64, 1), (64, 1), capi.F64) == "generic"                          # no unit stride

@@ -233,14 +233,16 @@ def test_streaming_rows_single_launch_finish(m):
 
 @pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
 def test_ragged_small_outputs_deep_k(dt):
-    """Outputs that no vector kernel takes (n = 10, odd strides) with a deep k: the generic kernel splits k across
-    blocks and a scalar kernel adds the partials in split order, so results repeat bit for bit.  fp64 does not split."""
+    """Outputs that no vector kernel takes (n = 10, odd strides) with a deep k.  16-bit: the generic kernel splits k
+    across blocks and a scalar kernel adds the partials in split order.  fp32: the one-launch 16 x 16-tile kernel, whose
+    four waves add their partial tiles in wave order.  Either way results repeat bit for bit.  fp64 does not split."""
     rng = np.random.default_rng(40)
     for m, k, n, layout in [(128, 256, 10, "tn"), (256, 128, 10, "nn"), (17, 1000, 3, "nn"), (70, 333, 65, "nt"), (10, 96, 130, "tt")]:
         a, b = _operands(rng, m, k, n, dt, layout)
         es = a.itemsize
         if dt != F64:              # 2-element vectors fit some of these shapes, which then take the fp64 MFMA kernel
-            assert capi.gemm_kernel_name(1, m, k, n, (a.strides[0] // es, a.strides[1] // es), (b.strides[0] // es, b.strides[1] // es), (n, 1), dt) == "generic"
+            name = capi.gemm_kernel_name(1, m, k, n, (a.strides[0] // es, a.strides[1] // es), (b.strides[0] // es, b.strides[1] // es), (n, 1), dt)
+            assert name == ("tiny32_16x16" if dt == F32 else "generic")
         bias = rand_storage(rng, (n,), dt); c0 = rand_storage(rng, (m, n), dt)
         got = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)
         _check(got, a, b, dt, k, bias=bias, c_init=c0, accumulate=True)
@@ -284,3 +286,30 @@ def test_rejects_bad_arguments():
     assert lib.rp_hip_gemm_strided_batched(d.ptr, d.ptr, d.ptr, None, 1, 2, 2, 2, 0, 2, 1, 0, 2, 1, 0, 2, 1, 0, 7) == -1
     assert lib.matmul_kernel_device(d.ptr, d.ptr, d.ptr, 2, -1, 2, F32) == -1
     assert b"extent" in lib.rp_hip_last_error()
+
+
+def test_small_fp32_outputs_take_one_launch():
+    """fp32 outputs of fewer than 64 tiles of 64 x 64 with k <= 2048 (the layers of the configuration-2 MLP): every layout,
+    ragged extents, batches, bias and accumulation, against the oracle and float64; repeatable bit for bit."""
+    rng = np.random.default_rng(43)
+    cases = [(256, 784, 256, "nn"), (256, 256, 784, "nt"), (784, 256, 256, "tn"), (256, 128, 10, "nn"), (1, 5, 1, "nn"), (33, 2048, 47, "tt"),
+             (100, 17, 300, "nt"), (16, 16, 16, "nn"), (250, 1, 250, "tn")]
+    for m, k, n, layout in cases:
+        a, b = _operands(rng, m, k, n, F32, layout)
+        assert capi.gemm_kernel_name(1, m, k, n, (a.strides[0] // 4, a.strides[1] // 4), (b.strides[0] // 4, b.strides[1] // 4), (n, 1), F32) == "tiny32_16x16"
+        bias = rand_storage(rng, (n,), F32); c0 = rand_storage(rng, (m, n), F32)
+        for kw in ({}, {"bias": bias}, {"bias": bias, "c_init": c0, "accumulate": True}):
+            got = device_gemm(a, b, F32, **kw)
+            _check(got, a, b, F32, k, **kw)
+            assert np.array_equal(got, device_gemm(a, b, F32, **kw))
+    # beyond the limits the tiled kernels take over
+    assert capi.gemm_kernel_name(1, 256, 4096, 256, (4096, 1), (256, 1), (256, 1), F32) != "tiny32_16x16"
+    assert capi.gemm_kernel_name(1, 512, 512, 512, (512, 1), (512, 1), (512, 1), F32) != "tiny32_16x16"
+    # a small batch of small matrices on stride views
+    a3 = rand_storage(rng, (5, 40, 24), F32); b3 = rand_storage(rng, (5, 24, 56), F32)
+    assert capi.gemm_kernel_name(5, 40, 24, 56, (24, 1), (56, 1), (56, 1), F32) == "tiny32_16x16"
+    got = device_gemm(a3, b3, F32)
+    assert oracle.rel_err(got, oracle_gemm(a3, b3, F32)) <= tol(F32, 24)
+    got_t = device_gemm(a3, np.ascontiguousarray(b3.transpose(0, 2, 1)).transpose(0, 2, 1), F32)
+    assert oracle.rel_err(got_t, oracle_gemm(a3, b3, F32)) <= tol(F32, 24)
+
