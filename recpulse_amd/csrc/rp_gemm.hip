@@ -100,7 +100,9 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
         // the 256 x 256 tile runs one block per CU, so it needs a k loop long enough to hide its prologue and
         // epilogue; with fewer than four slabs the smaller tile (two blocks per CU) overlaps them instead
         if (m >= 256 && n >= 256 && tiles256 >= 128 && k >= 4 * M16_BK) { p.bm = 256; p.bn = 256; p.name = "mfma16_256x256"; }
-        else if (m > 64 || n > 64) { p.bm = 128; p.bn = 128; p.name = "mfma16_128x128"; }
+        // fewer than 128 tiles of 128 x 128 would leave over half the CUs idle: the 64 x 64 tile quadruples the workgroups
+        // (1024^3: 10.9 -> 7.3 us)
+        else if ((m > 64 || n > 64) && tiles128_16 * batch >= 128) { p.bm = 128; p.bn = 128; p.name = "mfma16_128x128"; }
         else { p.bm = 64; p.bn = 64; p.name = "mfma16_64x64"; }
         p.edge = (m % p.bm) || (n % p.bn) || (k % M16_BK);
     } else {
