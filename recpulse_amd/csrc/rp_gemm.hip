@@ -69,9 +69,10 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
 
     // 16-bit, few rows, deep k: split k over many blocks so that B streams at HBM speed (output columns in whole 8s).
     // Up to 32 rows always; up to skinny_max_rows() when the 128 x 128 tiles of the output would occupy under half the
-    // CUs (and k is deep enough to be worth a second launch for the partial sums).
+    // CUs and k is deep enough to be worth a second launch for the partial sums (64 x 1024 x 4096: 6.6 us on 64 x 64 tiles
+    // in one launch against 9.4 us split; 64 x 4096 x 1024: 16.4 against 9.1).
     const long long tiles128_16 = (long long)((m + 127) / 128) * ((n + 127) / 128);
-    if (is16 && mfma_ok && batch == 1 && (m <= 32 || (m <= skinny_max_rows() && tiles128_16 < 128 && (k >= 2048 || tiles128_16 < 48))) && n % 8 == 0 && n >= 256 && k >= 1024 &&
+    if (is16 && mfma_ok && batch == 1 && (m <= 32 || (m <= skinny_max_rows() && tiles128_16 < 128 && k >= 2048)) && n % 8 == 0 && n >= 256 && k >= 1024 &&
         (long long)k * n >= (1ll << 22)) {
         p.fam = FAM_MFMA16_SKINNY; p.bm = 32; p.bn = 128; p.edge = true; p.a_mc = !a_kc; p.b_mc = b_mc;
         p.name = (!p.a_mc && p.b_mc && m <= 16) ? "mfma16_stream_32x256" : "mfma16_skinny_32x128";
