@@ -157,6 +157,10 @@ int sum_dim_kernel_device(void* out, const void* x, size_t outer_size, size_t di
 
 /* core/tensor_device.cu:66-114 (fill_value_kernel, copy_value_kernel<Src,Dst>) */
 int rp_hip_fill(void* ptr, double value, size_t size, int dtype);
+/* ptr[i] = scalar_dev[0] * scale (product in double, narrowed once): the gradient of sum_all / mean_all
+ * (backward_sum_all_fn / backward_mean_all_fn, ops/ops.c:2059-2110: a fill with grad_output or grad_output / size) with grad_output read where it
+ * lives instead of on the host */
+int rp_hip_fill_scaled(void* ptr, const void* scalar_dev, double scale, size_t size, int dtype);
 int rp_hip_convert(void* dst, int dst_dtype, const void* src, int src_dtype, size_t size);
 
 /* Bias gradient of Linear on the device: grad [rows, cols] dense -> out [cols],
@@ -176,6 +180,12 @@ int rp_hip_reduce_rows(void* out, const void* grad, int rows, int cols, int accu
  * 5412-5543, 5545-5643). */
 int rp_hip_cross_entropy_mean(void* loss_out, void* grad_logits, const void* logits, const int* targets,
                               int batch, int classes, double upstream, int dtype);
+
+/* The grad_logits half of rp_hip_cross_entropy_mean with the upstream factor read from one device element of
+ * dtype (the gradient of the loss as autograd holds it), so that the backward pass never waits on a
+ * device-to-host copy (the reference reads it on the host, ops/ops.c:5412-5543). */
+int rp_hip_cross_entropy_backward(void* grad_logits, const void* logits, const int* targets, int batch, int classes,
+                                  const void* upstream_dev, int dtype);
 
 /* ---- conv2d lowering (the callers of the GEMM in op_conv2d, ops/ops.c:4723-4870 and 4473-4720) ---- */
 

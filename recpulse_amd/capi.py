@@ -67,6 +67,8 @@ SIGNATURES = {
     "rp_hip_convert": (_i, [_vp, _i, _vp, _i, _sz]),
     "rp_hip_reduce_rows": (_i, [_vp, _vp, _i, _i, _i, _i]),
     "rp_hip_cross_entropy_mean": (_i, [_vp, _vp, _vp, _vp, _i, _i, _d, _i]),
+    "rp_hip_cross_entropy_backward": (_i, [_vp, _vp, _vp, _i, _i, _vp, _i]),
+    "rp_hip_fill_scaled": (_i, [_vp, _vp, _d, _sz, _i]),
     "im2col_kernel_device": (_i, [_vp, _vp] + [_i] * 14),
     "col2im_kernel_device": (_i, [_vp, _vp] + [_i] * 14),
     "rp_hip_im2col_batched": (_i, [_vp, _vp] + [_i] * 15),

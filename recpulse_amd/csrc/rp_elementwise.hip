@@ -91,6 +91,14 @@ __global__ void fill_kernel(T* p, T v, size_t n) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
 }
 
+// out[i] = scalar[0] * scale, the product taken in double and narrowed once (what the host computes when it reads
+// the scalar back first)
+template <typename T>
+__global__ void fill_scaled_kernel(T* out, const T* scalar, double scale, size_t n) {
+    const T v = narrow<T>((typename traits<T>::acc)((double)widen(scalar[0]) * scale));
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) out[i] = v;
+}
+
 // dtype conversion pivots through fp32 like the reference (core/tensor_host.c:130-207),
 // except float64 <-> float64 / float32 which are direct.
 template <typename D, typename S>
@@ -477,9 +485,10 @@ __global__ void reduce_rows_kernel(T* out, const T* g, int rows, int cols, int a
 // the reference's host loop does (ops/ops.c:5342-5352).
 template <typename T>
 __global__ void cross_entropy_kernel(T* loss, T* grad, const T* logits, const int* targets,
-                                     int batch, int classes, T upstream) {
+                                     int batch, int classes, T upstream, const T* upstream_dev) {
     __shared__ double nll[kThreads];
     double total = 0.0;
+    if (upstream_dev) upstream *= upstream_dev[0];           // the upstream gradient where it lives: no host round trip
     for (int b0 = 0; b0 < batch; b0 += blockDim.x) {
         int b = b0 + threadIdx.x;
         if (b < batch) {
@@ -718,11 +727,34 @@ int rp_hip_cross_entropy_mean(void* loss_out, void* grad_logits, const void* log
     }
     if (dtype == RP_DTYPE_FLOAT32)
         hipLaunchKernelGGL(cross_entropy_kernel<float>, dim3(1), dim3(kThreads), 0, current_stream(), (float*)loss_out, (float*)grad_logits,
-                           (const float*)logits, targets, batch, classes, (float)upstream);
+                           (const float*)logits, targets, batch, classes, (float)upstream, (const float*)nullptr);
     else
         hipLaunchKernelGGL(cross_entropy_kernel<double>, dim3(1), dim3(kThreads), 0, current_stream(), (double*)loss_out, (double*)grad_logits,
-                           (const double*)logits, targets, batch, classes, upstream);
+                           (const double*)logits, targets, batch, classes, upstream, (const double*)nullptr);
     return check_launch("cross_entropy_kernel") ? 0 : -1;
+}
+
+int rp_hip_cross_entropy_backward(void* grad_logits, const void* logits, const int* targets, int batch, int classes,
+                                  const void* upstream_dev, int dtype) {
+    RP_REQUIRE(grad_logits && logits && targets && upstream_dev && batch > 0 && classes > 0, "rp_hip_cross_entropy_backward");
+    if (dtype != RP_DTYPE_FLOAT32 && dtype != RP_DTYPE_FLOAT64) {
+        set_error("rp_hip_cross_entropy_backward: float32 and float64 only");
+        return -1;
+    }
+    if (dtype == RP_DTYPE_FLOAT32)
+        hipLaunchKernelGGL(cross_entropy_kernel<float>, dim3(1), dim3(kThreads), 0, current_stream(), (float*)nullptr, (float*)grad_logits,
+                           (const float*)logits, targets, batch, classes, 1.0f, (const float*)upstream_dev);
+    else
+        hipLaunchKernelGGL(cross_entropy_kernel<double>, dim3(1), dim3(kThreads), 0, current_stream(), (double*)nullptr, (double*)grad_logits,
+                           (const double*)logits, targets, batch, classes, 1.0, (const double*)upstream_dev);
+    return check_launch("cross_entropy_kernel") ? 0 : -1;
+}
+
+int rp_hip_fill_scaled(void* ptr, const void* scalar_dev, double scale, size_t size, int dtype) {
+    RP_REQUIRE(ptr && scalar_dev && size, "rp_hip_fill_scaled");
+    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(fill_scaled_kernel<T>, dim3(grid_for(size)), dim3(kThreads), 0, current_stream(),
+                                               (T*)ptr, (const T*)scalar_dev, scale, size));
+    return check_launch("fill_scaled_kernel") ? 0 : -1;
 }
 
 }  // extern "C"

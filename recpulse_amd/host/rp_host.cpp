@@ -957,13 +957,23 @@ void backward_gru_cell_fn(GradFn* self, Tensor* grad_output) {
     free_tensor(dh); free_tensor(dgi); free_tensor(dgh); free_tensor(dh_direct);
 }
 
+// A one-element gradient that already sits on x's device in x's dtype can be read by the kernel that uses it;
+// fetching it to the host first would make every backward pass wait for the GPU to drain.
+bool scalar_beside(const Tensor* s, const Tensor* x) {
+    return s && s->size == 1 && s->device_id == x->device_id && s->dtype == x->dtype && on_device(x->device_id);
+}
+
 void backward_reduce_all_fn(GradFn* self, Tensor* grad_output) {     // sum_all / mean_all: every element receives g (or g / size)
     Tensor* x = self->inputs[0];
     if (!needs_grad(x)) return;
     double g0 = 0, scale = ((ScalarSaved*)self->saved_data)->s;
-    if (tensor_read_scalar(grad_output, &g0) != 0) return;
     Tensor* g = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
-    if (g && fill_value_tensor(g0 * scale, g)) accumulate_grad(x, g);
+    bool ok = g != nullptr;
+    if (ok && scalar_beside(grad_output, x)) {                       // the upstream scalar never visits the host
+        ok = rp_hip_fill_scaled(g->data, grad_output->data, scale, g->size, g->dtype) == 0;
+        if (!ok) dev_fail("fill scaled");
+    } else if (ok) ok = tensor_read_scalar(grad_output, &g0) == 0 && fill_value_tensor(g0 * scale, g);
+    if (ok) accumulate_grad(x, g);
     else free_tensor(g);
 }
 
@@ -981,11 +991,15 @@ void backward_cross_entropy_fn(GradFn* self, Tensor* grad_output) {
     if (!needs_grad(x)) return;
     CESaved* s = (CESaved*)self->saved_data;
     double up = 1.0;
-    if (tensor_read_scalar(grad_output, &up) != 0) return;
+    const bool beside = scalar_beside(grad_output, x);
+    if (!beside && tensor_read_scalar(grad_output, &up) != 0) return;
     Tensor* xd = dense(x);
     Tensor* g = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
-    if (g && on_device(x->device_id) &&
-        rp_hip_cross_entropy_mean(nullptr, g->data, xd->data, (const int*)s->targets_dev, s->batch, s->classes, up, x->dtype) == 0) accumulate_grad(x, g);
+    int rc = -1;
+    if (g && xd && on_device(x->device_id))
+        rc = beside ? rp_hip_cross_entropy_backward(g->data, xd->data, (const int*)s->targets_dev, s->batch, s->classes, grad_output->data, x->dtype)
+                    : rp_hip_cross_entropy_mean(nullptr, g->data, xd->data, (const int*)s->targets_dev, s->batch, s->classes, up, x->dtype);
+    if (rc == 0) accumulate_grad(x, g);
     else free_tensor(g);
     free_tensor(xd);
 }

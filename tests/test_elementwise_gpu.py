@@ -163,6 +163,34 @@ def test_cross_entropy(dt):
     assert L().rp_hip_cross_entropy_mean(ls.ptr, None, lg.ptr, bad.ptr, 3, 3, 1.0, BF16) == -1
 
 
+@pytest.mark.parametrize("dt", [F32, F64], ids=lambda d: NAMES[d])
+def test_cross_entropy_backward_reads_the_upstream_gradient_on_the_device(dt):
+    """Same gradient, bit for bit, as the entry that takes the upstream factor from the host."""
+    rng = np.random.default_rng(49)
+    for batch, classes, up in ((256, 10, 1.0), (7, 3, -0.375), (1000, 33, 2.5)):
+        logits = oracle.to_storage(rng.normal(0, 3, (batch, classes)), dt)
+        t = rng.integers(0, classes, batch).astype(np.int32)
+        dl, dtg = Dev(logits, dt), capi.DeviceBuffer.from_numpy(t)
+        dup = Dev(oracle.to_storage(np.array([up]), dt), dt)
+        want, got = Dev.empty((batch, classes), dt), Dev.empty((batch, classes), dt)
+        capi.check(L().rp_hip_cross_entropy_mean(None, want.ptr, dl.ptr, dtg.ptr, batch, classes, up, dt), "ce")
+        capi.check(L().rp_hip_cross_entropy_backward(got.ptr, dl.ptr, dtg.ptr, batch, classes, dup.ptr, dt), "ce backward")
+        assert np.array_equal(got.numpy(), want.numpy())
+        _, grad = oracle.cross_entropy_mean(logits, t, dt)
+        assert oracle.rel_err(got.numpy(), grad * up) <= (4e-6 if dt == F32 else 1e-13)
+    assert L().rp_hip_cross_entropy_backward(got.ptr, dl.ptr, dtg.ptr, batch, classes, dup.ptr, BF16) == -1
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_fill_scaled_matches_a_host_side_product(dt):
+    for value, scale, n in ((1.0, 1.0 / 777, 777), (-2.5, 1.0, 5000), (0.3, 1.0 / 3, 1)):
+        stored = oracle.to_storage(np.array([value]), dt)
+        ds, out, want = Dev(stored, dt), Dev.empty((n,), dt), Dev.empty((n,), dt)
+        capi.check(L().rp_hip_fill_scaled(out.ptr, ds.ptr, scale, n, dt), "fill scaled")
+        capi.check(L().rp_hip_fill(want.ptr, float(oracle.to_f64(stored, dt)[0]) * scale, n, dt), "fill")
+        assert np.array_equal(out.numpy(), want.numpy())
+
+
 def test_allocator_reuses_blocks_and_reports_errors():
     a = capi.DeviceBuffer(1000); p = a.ptr
     a.free()
