@@ -369,6 +369,22 @@ def conv2d_times(capi, dt_name="bf16"):
     total += out["im2col"]["us"] * 1e-3                 # the backward lowers the activations again for dW
     out["fwd_bwd_ms"] = round(total, 4)
     out["fwd_bwd_TFLOP/s"] = round(3 * gemm_flops / total / 1e9, 1)
+    if L.rp_hip_conv2d_same_supported(C, H, W, k, k, dt) == 1:
+        # forward and input gradient straight from zero-bordered planes (no lowered matrix); the weight gradient still lowers
+        direct = {
+            "y=conv(x,W)+b": (lambda: capi.check(L.rp_hip_conv2d_same_forward(d_y.ptr, d_x.ptr, d_w.ptr, d_b.ptr, N, C, H, W, Co, k, k, dt), "same forward"),
+                              gemm_flops, N * (x_n + y_n) * esz),
+            "dx=conv_t(dy,W)": (lambda: capi.check(L.rp_hip_conv2d_same_backward_input(d_dx.ptr, d_dy.ptr, d_w.ptr, N, C, H, W, Co, k, k, dt), "same backward"),
+                                gemm_flops, N * (x_n + y_n) * esz),
+        }
+        out["lowered_fwd_bwd_ms"] = out["fwd_bwd_ms"]
+        total = (out["im2col"]["us"] + out["dW_n=dy.colt"]["us"] + out["dW=sum_n"]["us"] + out["db"]["us"]) * 1e-3
+        for name, (fn, flops, nbytes) in direct.items():
+            ms = _time_graph(capi, fn, 10, 2)
+            total += ms
+            out[name] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1), "TFLOP/s": round(flops / ms / 1e9, 1)}
+        out["fwd_bwd_ms"] = round(total, 4)
+        out["fwd_bwd_TFLOP/s"] = round(3 * gemm_flops / total / 1e9, 1)
     for d in (d_x, d_w, d_b, d_dy, d_col, d_y, d_dx, d_dws, d_dw, d_db):
         d.free()
     return out

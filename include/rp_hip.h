@@ -209,6 +209,20 @@ int rp_hip_col2im_batched(void* im, const void* col, int batch, int C_in, int H,
                           int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h, int dilation_w,
                           int out_H, int out_W, int accumulate, int dtype);
 
+/* Convolution without the lowered matrix, for stride 1, no dilation, odd kernels with padding (k - 1) / 2 ("same"
+ * output size) in bfloat16 / float16 when the channel count that is summed over is a multiple of 64
+ * (rp_hip_conv2d_same_supported says whether a shape qualifies).  x [batch, C_in, H, W], w [C_out, C_in, kH, kW],
+ * y / dy [batch, C_out, H, W], all dense.  The input is copied once into zero-bordered planes and the GEMM reads
+ * every tap from that copy in place; the sum over taps and channels is kept in fp32 and rounded once, then the bias
+ * is added with its own rounding as in rp_hip_channel_bias_add.  They stand in for the per-sample
+ * im2col + matmul (+ col2im) loops of op_conv2d and backward_conv2d_fn (ops/ops.c:4759-4783, 4533-4551); the weight
+ * gradient keeps the lowered matrix. */
+int rp_hip_conv2d_same_supported(int reduced_channels, int H, int W, int kH, int kW, int dtype);
+int rp_hip_conv2d_same_forward(void* y, const void* x, const void* w, const void* bias, int batch, int C_in, int H, int W,
+                               int C_out, int kH, int kW, int dtype);
+int rp_hip_conv2d_same_backward_input(void* dx, const void* dy, const void* w, int batch, int C_in, int H, int W,
+                                      int C_out, int kH, int kW, int dtype);
+
 /* y[n, c, :] += bias[c] for y [batch, channels, hw]: the reference pulls y to the host for this loop
  * (ops/ops.c:4772-4836). */
 int rp_hip_channel_bias_add(void* y, const void* bias, int batch, int channels, int hw, int dtype);

@@ -13,11 +13,9 @@
 // sum is rounded after every add in an order that changes from run to run.  Here col2im gathers: each input pixel adds
 // its (kh, kw) contributions in ascending order in the accumulate type and rounds once, which is what the reference's
 // host path computes (functional/functional.c:885-912, functional_host.c:1291-1313) and is repeatable.
-#include "rp_common.h"
+#include "rp_gemm.h"
 
 namespace rp {
-
-typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
 
 struct ConvGeom {
     int N, C, H, W, kH, kW, sh, sw, ph, pw, dh, dw, oH, oW;
@@ -97,6 +95,102 @@ __global__ void __launch_bounds__(256) im2col_kernel(T* col, const T* im, ConvGe
         for (int kh = 0; kh < g.kH; kh++)
             for (int kw = 0; kw < g.kW; kw++, dst += cols) tap(kh, kw, dst);
     }
+}
+
+// The common case on its own: 3 x 3 taps, stride 1, padding 1, no dilation, rows a whole number of vectors (so
+// oH = H, oW = W and every vector of a row is 16-byte aligned in the image and in every col row).  The three taps of
+// one image row are the aligned vector at the thread's columns shifted by -1, 0 and +1 elements: one vector load and
+// its two neighbouring elements per image row, no per-element masks and no variable shifts (the general kernel is
+// bound by that arithmetic, not by memory).
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256) im2col_3x3_kernel(T* col, const T* im, int H, int W, unsigned total_vec) {
+    const unsigned vec_per_row = W / VEC, vec_per_plane = H * vec_per_row;
+    const unsigned gid = blockIdx.x * 256u + threadIdx.x;
+    if (gid >= total_vec) return;
+    const unsigned plane_id = gid / vec_per_plane, pv = gid % vec_per_plane;
+    const int h = pv / vec_per_row, w0 = (pv % vec_per_row) * VEC;
+    const size_t cols = (size_t)H * W;
+    const T* plane = im + plane_id * cols;
+    T* dst = col + (size_t)plane_id * 9 * cols + (size_t)pv * VEC;
+    T zero;
+    memset(&zero, 0, sizeof(T));
+#pragma unroll
+    for (int kh = 0; kh < 3; kh++) {
+        const int h_in = h + kh - 1;
+        const bool inside = h_in >= 0 && h_in < H;
+        const T* row = plane + (size_t)(inside ? h_in : h) * W;
+        T v[VEC + 2];                                          // columns w0 - 1 .. w0 + VEC of the image row
+        const u32x4_t raw = *(const u32x4_t*)(row + w0);
+        memcpy(&v[1], &raw, 16);
+        v[0] = row[w0 > 0 ? w0 - 1 : 0];
+        v[VEC + 1] = row[w0 + VEC < W ? w0 + VEC : W - 1];
+        if (!inside || w0 == 0) v[0] = zero;
+        if (!inside || w0 + VEC >= W) v[VEC + 1] = zero;
+        if (!inside) {
+#pragma unroll
+            for (int e = 1; e <= VEC; e++) v[e] = zero;
+        }
+#pragma unroll
+        for (int kw = 0; kw < 3; kw++) {
+            u32x4_t out;
+            memcpy(&out, &v[kw], 16);
+            *(u32x4_t*)(dst + (size_t)(kh * 3 + kw) * cols) = out;
+        }
+    }
+}
+
+// The adjoint of im2col_3x3_kernel, as a gather: pixel (h, w) adds col row (kh, kw) at (h + 1 - kh, w + 1 - kw), taps in
+// ascending (kh, kw) order.  Per tap one aligned vector load and one neighbouring element.
+template <typename T, int VEC, bool START_FROM_IM>
+__global__ void __launch_bounds__(256) col2im_3x3_kernel(T* im, const T* col, int H, int W, unsigned total_vec) {
+    using A = typename traits<T>::acc;
+    const unsigned vec_per_row = W / VEC, vec_per_plane = H * vec_per_row;
+    const unsigned gid = blockIdx.x * 256u + threadIdx.x;
+    if (gid >= total_vec) return;
+    const unsigned plane_id = gid / vec_per_plane, pv = gid % vec_per_plane;
+    const int h = pv / vec_per_row, w0 = (pv % vec_per_row) * VEC;
+    const size_t cols = (size_t)H * W;
+    const T* rows = col + (size_t)plane_id * 9 * cols;
+    T* dst = im + (size_t)gid * VEC;
+    A acc[VEC];
+    if (START_FROM_IM) {
+        T cur[VEC];
+        memcpy(cur, dst, 16);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[e] = widen(cur[e]);
+    } else {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[e] = (A)0;
+    }
+    const bool has_left = w0 > 0, has_right = w0 + VEC < W;
+#pragma unroll
+    for (int kh = 0; kh < 3; kh++) {
+        const int oh = h + 1 - kh;
+        const bool inside = oh >= 0 && oh < H;
+        const T* base = rows + (size_t)(kh * 3) * cols + (size_t)(inside ? oh : h) * W;
+#pragma unroll
+        for (int kw = 0; kw < 3; kw++) {
+            const T* row = base + (size_t)kw * cols;
+            T v[VEC + 2];                                      // columns w0 - 1 .. w0 + VEC of the col row; only the ones this tap uses are loaded
+            const u32x4_t raw = *(const u32x4_t*)(row + w0);
+            memcpy(&v[1], &raw, 16);
+            if (kw == 0) v[VEC + 1] = row[has_right ? w0 + VEC : W - 1];
+            if (kw == 2) v[0] = row[has_left ? w0 - 1 : 0];
+            // pixel w0 + e takes column w0 + e + 1 - kw, i.e. v[e + 2 - kw]
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                const bool there = inside && (kw != 0 || e < VEC - 1 || has_right) && (kw != 2 || e > 0 || has_left);
+                const A sum = acc[e] + widen(v[e + 2 - kw]);
+                acc[e] = there ? sum : acc[e];
+            }
+        }
+    }
+    T out[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) out[e] = narrow<T>(acc[e]);
+    u32x4_t packed;
+    memcpy(&packed, out, 16);
+    *(u32x4_t*)dst = packed;
 }
 
 // One thread per VEC neighbouring input pixels of a row (VEC = 1 when W is not a whole number of vectors).
@@ -231,6 +325,155 @@ __global__ void channel_sums_finish_kernel(T* out, const typename traits<T>::acc
     out[c] = r;
 }
 
+// ---- convolution without a lowered matrix (stride 1, "same" padding, 16-bit types) ----
+// With the image copied once into planes of pitch Wp >= W + 2 * pad with a zero border, output position f = oh * Wp + ow
+// of tap (kh, kw) reads padded element f + kh * Wp + kw: every tap is the same matrix [C, H * Wp] at a different
+// offset, which the GEMM reads in place as a segment of its k axis (GemmArgs::seg_*).  The product comes out in the
+// same pitch (columns ow >= W hold sums that nobody uses) and unpad_planes_kernel copies the valid part.
+struct PadGeom {
+    int H, W, ph, pw, Hp, Wp;
+    long long P;                  // elements per padded plane (Hp * Wp plus the slack the last tap may read)
+};
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256) pad_planes_kernel(T* out, const T* in, PadGeom g, unsigned total_vec) {
+    const unsigned vec_per_plane = (unsigned)(g.P / VEC);
+    const unsigned gid = blockIdx.x * 256u + threadIdx.x;
+    if (gid >= total_vec) return;
+    const unsigned plane = gid / vec_per_plane, pv = gid % vec_per_plane;
+    const int e0 = (int)pv * VEC, r = e0 / g.Wp, c0 = e0 % g.Wp;           // Wp is a whole number of vectors: one row per vector
+    const int h = r - g.ph;
+    T v[VEC];
+    if (h >= 0 && h < g.H && g.W >= VEC) {
+        load_span<T, VEC>(v, in + ((size_t)plane * g.H + h) * g.W, c0 - g.pw, g.W);
+    } else {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            const int w = c0 + e - g.pw;
+            if (h >= 0 && h < g.H && w >= 0 && w < g.W) v[e] = in[((size_t)plane * g.H + h) * g.W + w];
+            else memset(&v[e], 0, sizeof(T));
+        }
+    }
+    u32x4_t raw;
+    memcpy(&raw, v, 16);
+    *(u32x4_t*)(out + (size_t)plane * g.P + e0) = raw;
+}
+
+// y[plane][h][w] = yp[plane][h * Wp + w] (+ bias[channel], one rounding add as channel_bias_add_kernel does)
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256) unpad_planes_kernel(T* y, const T* yp, const T* bias, int channels, int H, int W, int Wp, unsigned total_vec) {
+    const unsigned vec_per_plane = (unsigned)(H * W / VEC);
+    const unsigned gid = blockIdx.x * 256u + threadIdx.x;
+    if (gid >= total_vec) return;
+    const unsigned plane = gid / vec_per_plane;
+    const int e0 = (int)(gid % vec_per_plane) * VEC;
+    const T* src = yp + (size_t)plane * H * Wp;
+    T v[VEC];
+    if constexpr (VEC > 1) {                               // W is a whole number of vectors: the vector stays inside one row
+        const u32x4_t raw = *(const u32x4_t*)(src + (size_t)(e0 / W) * Wp + e0 % W);
+        memcpy(v, &raw, 16);
+    } else {
+        v[0] = src[(size_t)(e0 / W) * Wp + e0 % W];
+    }
+    if (bias) {
+        const auto b = widen(bias[plane % channels]);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) v[e] = narrow<T>(widen(v[e]) + b);
+    }
+    memcpy(y + (size_t)gid * VEC, v, VEC * sizeof(T));
+}
+
+// Weights [C_out, C_in, taps] reordered for the segmented GEMM.  Forward: [C_out][tap][C_in].  Backward to the input:
+// [C_in][tap][C_out] with the taps reversed (the gradient is a correlation with the kernel turned by 180 degrees).
+template <typename T>
+__global__ void conv_weights_by_tap_kernel(T* out, const T* w, int C_out, int C_in, int taps, int for_input_grad) {
+    const int total = C_out * C_in * taps;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+        if (!for_input_grad) {
+            const int ci = i % C_in, tap = (i / C_in) % taps, co = i / (C_in * taps);
+            out[i] = w[((size_t)co * C_in + ci) * taps + tap];
+        } else {
+            const int co = i % C_out, tap = (i / C_out) % taps, ci = i / (C_out * taps);
+            out[i] = w[((size_t)co * C_in + ci) * taps + (taps - 1 - tap)];
+        }
+    }
+}
+
+static bool same_conv_ok(int reduced_channels, int H, int W, int kH, int kW, int dtype) {
+    return (dtype == RP_DTYPE_BFLOAT16 || dtype == RP_DTYPE_FLOAT16) && reduced_channels > 0 && reduced_channels % M16_BK == 0 &&
+           H > 0 && W > 0 && kH > 0 && kW > 0 && kH % 2 == 1 && kW % 2 == 1 && kH * kW > 1 && kW <= 15 && kH <= 15 &&
+           (long long)(H + kH) * (W + kW + 8) < (1ll << 21);
+}
+
+// out[batch, C_to, H, W] = sum over taps and C_from of wt . padded(in[batch, C_from, H, W]); wt as conv_weights_by_tap_kernel
+// leaves it ([C_to][tap][C_from]).  bias may be null.  The batch goes in chunks that keep the workspace under 1 GiB.
+template <typename T>
+static int same_conv_run(void* out, const void* in, const void* wt, const void* bias, int batch, int C_from, int C_to,
+                         int H, int W, int kH, int kW, int dtype) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    PadGeom pg;
+    pg.H = H; pg.W = W; pg.ph = kH / 2; pg.pw = kW / 2; pg.Hp = H + kH - 1;
+    pg.Wp = (W + kW - 1 + VEC - 1) / VEC * VEC;
+    pg.P = (long long)pg.Hp * pg.Wp + 2 * VEC;               // the last tap of the last position reads up to kW - 2 elements past Hp * Wp
+    const long long cols = (long long)H * pg.Wp;
+    const long long per_sample = ((long long)C_from * pg.P + (long long)C_to * cols) * (long long)sizeof(T);
+    long long chunk = (1ll << 30) / per_sample;
+    chunk = chunk < 1 ? 1 : (chunk > 32768 ? 32768 : chunk);
+    if (chunk > batch) chunk = batch;
+    if (chunk * (long long)C_from * (pg.P / VEC) >= (1ll << 31) || chunk * (long long)C_to * H * W >= (1ll << 31)) {
+        set_error("conv2d: one sample is too large for the padded-plane path");
+        return -1;
+    }
+    void* padded = nullptr;
+    void* product = nullptr;
+    if (rp_hip_malloc(&padded, (size_t)(chunk * C_from * pg.P) * sizeof(T)) != 0) return -1;
+    if (rp_hip_malloc(&product, (size_t)(chunk * C_to * cols) * sizeof(T)) != 0) { rp_hip_free(padded); return -1; }
+    int rc = 0;
+    for (int b0 = 0; b0 < batch && rc == 0; b0 += (int)chunk) {
+        const int nb = batch - b0 < chunk ? batch - b0 : (int)chunk;
+        const T* in0 = (const T*)in + (size_t)b0 * C_from * H * W;
+        T* out0 = (T*)out + (size_t)b0 * C_to * H * W;
+        const unsigned pad_vecs = (unsigned)((long long)nb * C_from * (pg.P / VEC));
+        hipLaunchKernelGGL((pad_planes_kernel<T, VEC>), dim3((pad_vecs + 255) / 256), dim3(256), 0, current_stream(), (T*)padded, in0, pg, pad_vecs);
+        GemmArgs g{};
+        g.C = product; g.A = wt; g.B = padded; g.bias = nullptr;
+        g.batch = nb; g.m = C_to; g.k = kH * kW * C_from; g.n = (int)cols;
+        g.a_bs = 0; g.a_rs = (long long)kH * kW * C_from; g.a_cs = 1;
+        g.b_bs = (long long)C_from * pg.P; g.b_rs = pg.P; g.b_cs = 1;
+        g.c_bs = (long long)C_to * cols; g.c_rs = cols; g.c_cs = 1;
+        g.accumulate = 0;
+        g.seg_slabs = C_from / M16_BK; g.seg_w = kW; g.seg_sh = pg.Wp; g.seg_sw = 1; g.b_extent = (long long)C_from * pg.P;
+        rc = launch_gemm_segmented_b(g, dtype);
+        if (rc != 0) break;
+        if (W % VEC == 0 && ((uintptr_t)out0 & 15) == 0) {
+            const unsigned vecs = (unsigned)((long long)nb * C_to * H * W / VEC);
+            hipLaunchKernelGGL((unpad_planes_kernel<T, VEC>), dim3((vecs + 255) / 256), dim3(256), 0, current_stream(), out0, (const T*)product, (const T*)bias, C_to, H, W, pg.Wp, vecs);
+        } else {
+            const unsigned elems = (unsigned)((long long)nb * C_to * H * W);
+            hipLaunchKernelGGL((unpad_planes_kernel<T, 1>), dim3((elems + 255) / 256), dim3(256), 0, current_stream(), out0, (const T*)product, (const T*)bias, C_to, H, W, pg.Wp, elems);
+        }
+    }
+    if (rc == 0 && !check_launch("padded-plane convolution kernels")) rc = -1;
+    rp_hip_free(product);
+    rp_hip_free(padded);
+    return rc;
+}
+
+template <typename T>
+static int same_conv(void* out, const void* in, const void* w, const void* bias, int batch, int C_from, int C_to,
+                     int H, int W, int kH, int kW, bool for_input_grad, int dtype) {
+    const int taps = kH * kW, total = C_from * C_to * taps;
+    void* wt = nullptr;
+    if (rp_hip_malloc(&wt, (size_t)total * sizeof(T)) != 0) return -1;
+    // w is [C_out, C_in, taps]: forward reduces over C_in (C_from = C_in, C_to = C_out), the input gradient over C_out
+    const int C_out = for_input_grad ? C_from : C_to, C_in = for_input_grad ? C_to : C_from;
+    hipLaunchKernelGGL(conv_weights_by_tap_kernel<T>, dim3((total + 255) / 256 > 1024 ? 1024 : (total + 255) / 256), dim3(256), 0, current_stream(),
+                       (T*)wt, (const T*)w, C_out, C_in, taps, for_input_grad ? 1 : 0);
+    const int rc = same_conv_run<T>(out, in, wt, bias, batch, C_from, C_to, H, W, kH, kW, dtype);
+    rp_hip_free(wt);
+    return rc;
+}
+
 static bool geom_ok(const ConvGeom& g) {
     if (g.N <= 0 || g.C <= 0 || g.H <= 0 || g.W <= 0 || g.kH <= 0 || g.kW <= 0 || g.sh <= 0 || g.sw <= 0 || g.ph < 0 || g.pw < 0 ||
         g.dh <= 0 || g.dw <= 0 || g.oH <= 0 || g.oW <= 0) return false;
@@ -240,6 +483,11 @@ static bool geom_ok(const ConvGeom& g) {
     if (g.oH != eh || g.oW != ew) return false;
     return (long long)g.C * g.kH * g.kW * (long long)g.oH * g.oW < (1ll << 31) && (long long)g.H * g.W < (1ll << 31) &&
            (long long)g.N * g.C < (1ll << 31) && (long long)g.H * g.W < (1ll << 30) && (long long)g.oH * g.oW < (1ll << 30);
+}
+
+// 3 x 3 taps, stride 1, padding 1, no dilation, rows a whole number of vectors: the shape the *_3x3 kernels take
+static bool same_3x3(const ConvGeom& g, int vec) {
+    return g.kH == 3 && g.kW == 3 && g.sh == 1 && g.sw == 1 && g.ph == 1 && g.pw == 1 && g.dh == 1 && g.dw == 1 && g.W % vec == 0 && g.W >= vec;
 }
 
 static unsigned conv_grid(size_t work) {
@@ -265,7 +513,8 @@ static void launch_im2col(void* col, const void* im, const ConvGeom& g) {
         T* c0 = (T*)((char*)col + (size_t)p0 * g.kH * g.kW * cols * esz);
         const T* i0 = (const T*)((const char*)im + (size_t)p0 * g.H * g.W * esz);
         const dim3 grid((total + 255) / 256);
-        if (vec && g.kH == 3 && g.kW == 3) hipLaunchKernelGGL((im2col_kernel<T, VEC, true>), grid, dim3(256), 0, current_stream(), c0, i0, g, total);
+        if (vec && same_3x3(g, VEC) && ((uintptr_t)im & 15) == 0) hipLaunchKernelGGL((im2col_3x3_kernel<T, VEC>), grid, dim3(256), 0, current_stream(), c0, i0, g.H, g.W, total);
+        else if (vec && g.kH == 3 && g.kW == 3) hipLaunchKernelGGL((im2col_kernel<T, VEC, true>), grid, dim3(256), 0, current_stream(), c0, i0, g, total);
         else if (vec) hipLaunchKernelGGL((im2col_kernel<T, VEC, false>), grid, dim3(256), 0, current_stream(), c0, i0, g, total);
         else hipLaunchKernelGGL((im2col_kernel<T, 1, false>), grid, dim3(256), 0, current_stream(), c0, i0, g, total);
     }
@@ -285,7 +534,10 @@ static void launch_col2im(void* im, const void* col, const ConvGeom& g, bool sta
         const dim3 grid((total + 255) / 256);
         const T* c0 = (const T*)((const char*)col + (size_t)p0 * g.kH * g.kW * cols * esz);
         T* i0 = (T*)((char*)im + (size_t)p0 * g.H * g.W * esz);
-        if (vec) {
+        if (vec && same_3x3(g, VEC) && ((uintptr_t)col & 15) == 0) {
+            if (start_from_im) hipLaunchKernelGGL((col2im_3x3_kernel<T, VEC, true>), grid, dim3(256), 0, current_stream(), i0, c0, g.H, g.W, total);
+            else hipLaunchKernelGGL((col2im_3x3_kernel<T, VEC, false>), grid, dim3(256), 0, current_stream(), i0, c0, g.H, g.W, total);
+        } else if (vec) {
             if (start_from_im) hipLaunchKernelGGL((col2im_gather_kernel<T, VEC, true>), grid, dim3(256), 0, current_stream(), i0, c0, g, total);
             else hipLaunchKernelGGL((col2im_gather_kernel<T, VEC, false>), grid, dim3(256), 0, current_stream(), i0, c0, g, total);
         } else {
@@ -344,6 +596,30 @@ int im2col_kernel_device(void* col, const void* im, int C_in, int H, int W, int 
 int col2im_kernel_device(void* im, const void* col, int C_in, int H, int W, int kH, int kW, int stride_h, int stride_w,
                          int pad_h, int pad_w, int dilation_h, int dilation_w, int out_H, int out_W, int dtype) {
     return rp_hip_col2im_batched(im, col, 1, C_in, H, W, kH, kW, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w, out_H, out_W, 1, dtype);
+}
+
+int rp_hip_conv2d_same_supported(int reduced_channels, int H, int W, int kH, int kW, int dtype) {
+    return same_conv_ok(reduced_channels, H, W, kH, kW, dtype) ? 1 : 0;
+}
+
+int rp_hip_conv2d_same_forward(void* y, const void* x, const void* w, const void* bias, int batch, int C_in, int H, int W,
+                               int C_out, int kH, int kW, int dtype) {
+    if (!y || !x || !w || batch <= 0 || C_out <= 0 || !same_conv_ok(C_in, H, W, kH, kW, dtype) || ((uintptr_t)x & 1) || ((uintptr_t)y & 1)) {
+        set_error("rp_hip_conv2d_same_forward: null operand or a shape outside rp_hip_conv2d_same_supported");
+        return -1;
+    }
+    if (dtype == RP_DTYPE_BFLOAT16) return same_conv<bf16_t>(y, x, w, bias, batch, C_in, C_out, H, W, kH, kW, false, dtype);
+    return same_conv<f16_t>(y, x, w, bias, batch, C_in, C_out, H, W, kH, kW, false, dtype);
+}
+
+int rp_hip_conv2d_same_backward_input(void* dx, const void* dy, const void* w, int batch, int C_in, int H, int W,
+                                      int C_out, int kH, int kW, int dtype) {
+    if (!dx || !dy || !w || batch <= 0 || C_in <= 0 || !same_conv_ok(C_out, H, W, kH, kW, dtype) || ((uintptr_t)dx & 1) || ((uintptr_t)dy & 1)) {
+        set_error("rp_hip_conv2d_same_backward_input: null operand or a shape outside rp_hip_conv2d_same_supported");
+        return -1;
+    }
+    if (dtype == RP_DTYPE_BFLOAT16) return same_conv<bf16_t>(dx, dy, w, nullptr, batch, C_out, C_in, H, W, kH, kW, true, dtype);
+    return same_conv<f16_t>(dx, dy, w, nullptr, batch, C_out, C_in, H, W, kH, kW, true, dtype);
 }
 
 int rp_hip_channel_bias_add(void* y, const void* bias, int batch, int channels, int hw, int dtype) {

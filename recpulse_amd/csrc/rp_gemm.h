@@ -18,6 +18,12 @@ struct GemmArgs {
     long long b_bs, b_rs, b_cs;
     long long c_bs, c_rs, c_cs;
     int accumulate;
+    // B's k axis in segments (16-bit MFMA kernels only; all zero = one plain matrix).  k is cut into segments of
+    // seg_slabs slabs of M16_BK; segment s = (sh, sw), sw = s % seg_w, starts at element offset sh * seg_sh + sw * seg_sw
+    // from B and runs with B's strides from there.  This is how a convolution reads its taps from one zero-bordered
+    // copy of the image instead of from a lowered matrix.  b_extent: elements of one batch entry of B that may be read.
+    int seg_slabs, seg_w;
+    long long seg_sh, seg_sw, b_extent;
 };
 
 enum Family { FAM_GENERIC = 0, FAM_SKINNY, FAM_MFMA16, FAM_MFMA16_SKINNY, FAM_MFMAW, FAM_TINY };
@@ -126,6 +132,7 @@ int launch_skinny(const GemmArgs& g, int dtype);
 int launch_mfma16(const GemmArgs& g, const Plan& p, int dtype);
 int launch_mfmaw(const GemmArgs& g, const Plan& p, int dtype);
 int launch_tiny(const GemmArgs& g, int dtype);
+int launch_gemm_segmented_b(const GemmArgs& g, int dtype);
 // adds k-split partials [nsplit][part_rows][n] (fp32, rows beyond g.m unused) in split order and runs the epilogue into C
 int launch_splitk_combine(const GemmArgs& g, const float* partials, int nsplit, int part_rows, int dtype);
 

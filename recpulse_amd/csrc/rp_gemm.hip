@@ -39,10 +39,33 @@ static bool tiny_off() {                           // RP_HIP_NO_TINY=1: small fp
     return v == 1;
 }
 
+static bool wide64() {                             // RP_HIP_NO_64X256=1: outputs of at most 64 rows keep the square tiles
+    static int v = -1;
+    if (v < 0) { const char* e = getenv("RP_HIP_NO_64X256"); v = (e && e[0] == '1') ? 0 : 1; }
+    return v == 1;
+}
+
 static int skinny_max_rows() {                     // RP_HIP_SKINNY_MAX_M: rows up to which a deep 16-bit GEMM with few output tiles splits k
     static int v = -1;
     if (v < 0) { const char* e = getenv("RP_HIP_SKINNY_MAX_M"); v = e ? atoi(e) : 128; if (v < 32) v = 32; }
     return v;
+}
+
+// Tile of the 16-bit MFMA kernel for an output of batch x m x n with reduction length k.
+static void choose_tile16(Plan& p, int batch, int m, int k, int n) {
+    p.fam = FAM_MFMA16;
+    const long long tiles256 = (long long)((m + 255) / 256) * ((n + 255) / 256) * batch;
+    const long long tiles128 = (long long)((m + 127) / 128) * ((n + 127) / 128) * batch;
+    // the 256 x 256 tile runs one block per CU, so it needs a k loop long enough to hide its prologue and
+    // epilogue; with fewer than four slabs the smaller tile (two blocks per CU) overlaps them instead
+    if (m >= 256 && n >= 256 && tiles256 >= 128 && k >= 4 * M16_BK) { p.bm = 256; p.bn = 256; p.name = "mfma16_256x256"; }
+    // fewer than 128 tiles of 128 x 128 would leave over half the CUs idle: the 64 x 64 tile quadruples the workgroups
+    // (1024^3: 10.9 -> 7.3 us)
+    // at most 64 rows: a 64 x 256 tile (the same 64 x 64 patch per wave as the 128 x 128 tile, none of it past the last row)
+    else if (m <= 64 && n >= 256 && wide64() && (long long)((n + 255) / 256) * batch >= 128) { p.bm = 64; p.bn = 256; p.name = "mfma16_64x256"; }
+    else if ((m > 64 || n > 64) && tiles128 >= 128) { p.bm = 128; p.bn = 128; p.name = "mfma16_128x128"; }
+    else { p.bm = 64; p.bn = 64; p.name = "mfma16_64x64"; }
+    p.edge = (m % p.bm) || (n % p.bn) || (k % M16_BK);
 }
 
 // Decide the kernel family and tile from shapes and strides alone (pointer
@@ -96,16 +119,7 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     p.b_mc = b_mc;
 
     if (is16) {
-        p.fam = FAM_MFMA16;
-        long long tiles256 = (long long)((m + 255) / 256) * ((n + 255) / 256) * batch;
-        // the 256 x 256 tile runs one block per CU, so it needs a k loop long enough to hide its prologue and
-        // epilogue; with fewer than four slabs the smaller tile (two blocks per CU) overlaps them instead
-        if (m >= 256 && n >= 256 && tiles256 >= 128 && k >= 4 * M16_BK) { p.bm = 256; p.bn = 256; p.name = "mfma16_256x256"; }
-        // fewer than 128 tiles of 128 x 128 would leave over half the CUs idle: the 64 x 64 tile quadruples the workgroups
-        // (1024^3: 10.9 -> 7.3 us)
-        else if ((m > 64 || n > 64) && tiles128_16 * batch >= 128) { p.bm = 128; p.bn = 128; p.name = "mfma16_128x128"; }
-        else { p.bm = 64; p.bn = 64; p.name = "mfma16_64x64"; }
-        p.edge = (m % p.bm) || (n % p.bn) || (k % M16_BK);
+        choose_tile16(p, batch, m, k, n);
     } else {
         p.fam = FAM_MFMAW;
         long long tiles128 = (long long)((m + 127) / 128) * ((n + 127) / 128) * batch;
@@ -128,6 +142,23 @@ static int run_gemm(const GemmArgs& g, int dtype) {
         case FAM_TINY:   return launch_tiny(g, dtype);
         default:         return launch_generic(g, dtype);
     }
+}
+
+// C_z = A_z . B_z with B's k axis given as segments (GemmArgs::seg_*): the 16-bit MFMA kernel reads every segment
+// in place, at any 2-byte alignment.  For callers inside the library (the convolution), which guarantee: a 16-bit
+// dtype, A in a fast layout with a 16-byte aligned base, B with unit stride along n, k a whole number of segments.
+int launch_gemm_segmented_b(const GemmArgs& g, int dtype) {
+    const bool is16 = dtype == RP_DTYPE_FLOAT16 || dtype == RP_DTYPE_BFLOAT16;
+    const bool a_kc = g.a_cs == 1 && g.a_rs % 8 == 0, a_mc = g.a_rs == 1 && g.a_cs % 8 == 0 && g.m % 8 == 0;
+    const long long max_stride = 1ll << 22;
+    if (!is16 || !(a_kc || a_mc) || !aligned16(g.A) || g.a_bs % 8 || g.b_cs != 1 || g.n % 8 || g.seg_slabs <= 0 || g.seg_w <= 0 ||
+        g.k % (g.seg_slabs * M16_BK) || g.a_rs >= max_stride || g.a_cs >= max_stride || g.b_rs >= max_stride || g.batch > 65535) {
+        set_error("segmented GEMM: operands outside what the 16-bit MFMA kernel reads in place");
+        return -1;
+    }
+    Plan p{FAM_MFMA16, 64, 64, !a_kc, true, true, "mfma16"};
+    choose_tile16(p, g.batch, g.m, g.k, g.n);
+    return launch_mfma16(g, p, dtype);
 }
 
 }  // namespace rp

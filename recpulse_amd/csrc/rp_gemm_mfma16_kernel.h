@@ -158,8 +158,24 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     const char* a_slab = (const char*)(a_mat + (long long)m0 * a_fs + (long long)kbeg * a_ks);
     const char* b_slab = (const char*)(b_mat + (long long)n0 * b_fs + (long long)kbeg * b_ks);
     const char* a_end = (const char*)(a_mat + ((long long)(g.m - 1) * a_fs + (long long)(kend - 1) * a_ks + 1));
-    const char* b_end = (const char*)(b_mat + ((long long)(g.n - 1) * b_fs + (long long)(kend - 1) * b_ks + 1));
+    const bool segmented = g.seg_slabs > 0;                 // B's k axis is a list of segments (never together with SPLITK)
+    const char* b_end = segmented ? (const char*)(b_mat + g.b_extent)
+                                  : (const char*)(b_mat + ((long long)(g.n - 1) * b_fs + (long long)(kend - 1) * b_ks + 1));
     const long long a_step = (long long)M16_BK * a_ks * 2, b_step = (long long)M16_BK * b_ks * 2;
+    // From the last slab of a segment the pointer goes back to the segment's start and on to the next one's: one
+    // step along seg_sw, or, after the seg_w-th segment of a row, to the start of the next row of segments.
+    const long long seg_next = segmented ? g.seg_sw * 2 - (long long)(g.seg_slabs - 1) * b_step : b_step;
+    const long long seg_wrap = segmented ? (g.seg_sh - (long long)g.seg_w * g.seg_sw) * 2 : 0;
+    int seg_left = segmented ? g.seg_slabs : 0x7fffffff, seg_col = 0;
+    auto advance_b = [&]() {
+        if (--seg_left == 0) {
+            seg_left = g.seg_slabs;
+            b_slab += seg_next;
+            if (++seg_col == g.seg_w) { seg_col = 0; b_slab += seg_wrap; }
+        } else {
+            b_slab += b_step;
+        }
+    };
 
     // Per-thread piece offsets (bytes from the slab pointer).  The buffer descriptor ends at the operand's last
     // element, which zero-fills rows past the free extent (KC) or k past the end (MC); the other axis of each
@@ -247,14 +263,14 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     static_for<0, NA>([&](auto ic) { store_piece_a(smem, ic); });
     static_for<0, NB>([&](auto ic) { store_piece_b(smem, ic); });
     a_slab += a_step;
-    b_slab += b_step;
+    advance_b();
     if (nslabs > 1) {
         point_at_slab(M16_BK);
         static_for<0, NA>([&](auto ic) { load_piece_a(ic); });
         static_for<0, NB>([&](auto ic) { load_piece_b(ic); });
     }
     a_slab += a_step;
-    b_slab += b_step;
+    advance_b();
     __syncthreads();
     static_for<0, RD_A + RD_B>([&](auto rc) { read_item(smem, I0{}, I0{}, rc); });
 
@@ -330,7 +346,7 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
         if constexpr (NEXT) __syncthreads();
         kstep(I1{}, I0{}, next_tag, C0{}, C0{}, std::false_type{}, std::false_type{}, other, other);
         a_slab += a_step;
-        b_slab += b_step;
+        advance_b();
         cur ^= 1;
     };
 

@@ -810,6 +810,16 @@ bool conv_is_pointwise(const ConvSaved& c) {              // 1x1, unit stride, n
     return c.kH == 1 && c.kW == 1 && c.sh == 1 && c.sw == 1 && c.ph == 0 && c.pw == 0;
 }
 
+// Stride 1, no dilation, odd kernel with padding (k - 1) / 2, a 16-bit type and `reduced` channels in whole slabs of
+// the GEMM: the convolution (reduced = C_in) or its input gradient (reduced = C_out) reads its taps from zero-bordered
+// planes and never builds the lowered matrix.  RP_CONV_NO_DIRECT=1 keeps the lowered path (read at every call).
+bool conv_direct(const ConvSaved& c, DType dt, int reduced) {
+    const char* e = getenv("RP_CONV_NO_DIRECT");
+    if (e && e[0] == '1') return false;
+    return c.sh == 1 && c.sw == 1 && c.dh == 1 && c.dw == 1 && c.kH % 2 == 1 && c.kW % 2 == 1 && c.ph == c.kH / 2 && c.pw == c.kW / 2 &&
+           rp_hip_conv2d_same_supported(reduced, c.H, c.W, c.kH, c.kW, dt) == 1;
+}
+
 int conv_lower(void* col, const void* x, int nb, const ConvSaved& c, DType dt) {
     return rp_hip_im2col_batched(col, x, nb, c.C, c.H, c.W, c.kH, c.kW, c.sh, c.sw, c.ph, c.pw, c.dh, c.dw, c.oH, c.oW, dt);
 }
@@ -830,12 +840,14 @@ void backward_conv2d_fn(GradFn* self, Tensor* grad_output) {         // referenc
     Tensor* xd = dense(x); Tensor* wd = dense(w);
     void* col = nullptr;
     bool ok = g && xd && wd;
-    if (ok && !pointwise && (needs_grad(x) || needs_grad(w))) ok = rp_hip_malloc(&col, (size_t)chunk * col_n * esz) == 0;
+    const bool direct_dx = !pointwise && conv_direct(c, dt, c.Co);
+    if (ok && !pointwise && ((needs_grad(x) && !direct_dx) || needs_grad(w))) ok = rp_hip_malloc(&col, (size_t)chunk * col_n * esz) == 0;
     if (ok && needs_grad(x)) {
-        // dcol[n] = W^T . dy[n], then each input pixel gathers its taps
+        // dcol[n] = W^T . dy[n], then each input pixel gathers its taps; or the taps straight from zero-bordered planes of dy
         Tensor* dx = empty_tensor(dt, x->device_id, x->ndim, x->shape);
         bool good = dx != nullptr;
-        for (int n0 = 0; good && n0 < c.N; n0 += chunk) {
+        if (good && direct_dx) good = rp_hip_conv2d_same_backward_input(dx->data, g->data, wd->data, c.N, c.C, c.H, c.W, c.Co, c.kH, c.kW, dt) == 0;
+        for (int n0 = 0; good && !direct_dx && n0 < c.N; n0 += chunk) {
             const int nb = c.N - n0 < chunk ? c.N - n0 : chunk;
             char* dx_n = (char*)dx->data + n0 * x_n * esz;
             const char* g_n = (const char*)g->data + n0 * y_n * esz;
@@ -1143,15 +1155,19 @@ Tensor* op_conv2d(Tensor* input, Tensor* weight, Tensor* bias, int stride_h, int
     const bool pointwise = conv_is_pointwise(c);
     const int chunk = conv_chunk(c, esz);
     void* col = nullptr;
-    bool ok = out && on_device(input->device_id) && (pointwise || rp_hip_malloc(&col, (size_t)chunk * col_n * esz) == 0);
-    for (int n0 = 0; ok && n0 < c.N; n0 += chunk) {
+    const bool direct = !pointwise && conv_direct(c, dt, c.C);
+    bool ok = out && on_device(input->device_id) && (pointwise || direct || rp_hip_malloc(&col, (size_t)chunk * col_n * esz) == 0);
+    if (ok && direct) {
+        ok = rp_hip_conv2d_same_forward(out->data, xd->data, wd->data, bias ? bias->data : nullptr, c.N, c.C, c.H, c.W, c.Co, c.kH, c.kW, dt) == 0;   // adds the bias too
+    }
+    for (int n0 = 0; ok && !direct && n0 < c.N; n0 += chunk) {
         const int nb = c.N - n0 < chunk ? c.N - n0 : chunk;
         const char* x_nptr = (const char*)xd->data + n0 * x_n * esz;
         ok = (pointwise || conv_lower(col, x_nptr, nb, c, dt) == 0) &&
              rp_hip_gemm_strided_batched((char*)out->data + n0 * y_n * esz, wd->data, pointwise ? (const void*)x_nptr : col, nullptr, nb, c.Co, rows, cols,
                                          0, rows, 1, col_n, cols, 1, y_n, cols, 1, 0, dt) == 0;
     }
-    if (ok && bias) ok = rp_hip_channel_bias_add(out->data, bias->data, c.N, c.Co, cols, dt) == 0;
+    if (ok && bias && !direct) ok = rp_hip_channel_bias_add(out->data, bias->data, c.N, c.Co, cols, dt) == 0;
     if (col) rp_hip_free(col);
     free_tensor(xd); free_tensor(wd);
     if (!ok) { dev_fail("op_conv2d"); free_tensor(out); return nullptr; }

@@ -26,7 +26,12 @@ REF_CASES = [tuple(tuple(v) if isinstance(v, list) else v for v in c) for c in G
 MORE_CASES = [((3, 4, 16, 16), (6, 4, 3, 3), (1, 1), (1, 1), (1, 1), True),
               ((2, 5, 9, 9), (3, 5, 1, 1), (2, 2), (0, 0), (1, 1), True),
               ((4, 16, 8, 8), (24, 16, 1, 1), (1, 1), (0, 0), (1, 1), True),
-              ((2, 32, 14, 14), (64, 32, 3, 3), (1, 1), (1, 1), (1, 1), False)]
+              ((2, 32, 14, 14), (64, 32, 3, 3), (1, 1), (1, 1), (1, 1), False),
+              # 3 x 3 / stride 1 / padding 1 with whole vectors per row: first, interior and last vectors of a row, and a one-row image
+              ((2, 3, 5, 24), (4, 3, 3, 3), (1, 1), (1, 1), (1, 1), True),
+              ((1, 2, 1, 8), (2, 2, 3, 3), (1, 1), (1, 1), (1, 1), False),
+              # 64 channels in and out: the 16-bit types read the taps from zero-bordered planes, forward and input gradient
+              ((2, 64, 8, 8), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), True)]
 CASES = REF_CASES + MORE_CASES
 DT_NAME = {F32: "float32", F64: "float64", F16: "float16", BF16: "bfloat16"}
 
@@ -100,6 +105,60 @@ def test_lowering_rejects_inconsistent_geometry():
     assert L.rp_hip_im2col_batched(None, d.ptr, 1, 1, 4, 4, 3, 3, 1, 1, 0, 0, 1, 1, 2, 2, F32) == -1
 
 
+SAME_CASES = [  # (batch, C_in, H, W, C_out, kH, kW): whole tiles, ragged columns, several slabs per tap, 5 x 5, one row
+    (3, 64, 8, 8, 64, 3, 3), (2, 128, 14, 14, 64, 3, 3), (2, 64, 7, 20, 192, 3, 3), (1, 64, 9, 12, 32, 5, 5),
+    (2, 64, 1, 16, 64, 3, 1), (1, 64, 56, 56, 64, 3, 3)]
+
+
+@pytest.mark.parametrize("dt", [BF16, F16], ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("case", SAME_CASES, ids=lambda c: "x".join(map(str, c)))
+def test_same_convolution_without_lowered_matrix(dt, case):
+    """rp_hip_conv2d_same_forward / _backward_input against the oracle's per-sample chain and against float64."""
+    import torch
+    N, Ci, H, W, Co, kH, kW = case
+    L = capi.lib()
+    assert L.rp_hip_conv2d_same_supported(Ci, H, W, kH, kW, dt) == 1
+    rng = np.random.default_rng(83)
+    x, w = rand_storage(rng, (N, Ci, H, W), dt), oracle.to_storage(rng.standard_normal((Co, Ci, kH, kW)) * 0.2, dt)
+    b = rand_storage(rng, (Co,), dt)
+    s, p, d = (1, 1), (kH // 2, kW // 2), (1, 1)
+    dx_, dw_, db_, dy_ = Dev(x, dt), Dev(w, dt), Dev(b, dt), Dev.empty((N, Co, H, W), dt)
+    capi.check(L.rp_hip_conv2d_same_forward(dy_.ptr, dx_.ptr, dw_.ptr, db_.ptr, N, Ci, H, W, Co, kH, kW, dt), "same forward")
+    y_ref = oracle.conv2d_forward(x, w, b, s, p, d, dt)
+    xt, wt = torch.tensor(oracle.to_f64(x, dt)), torch.tensor(oracle.to_f64(w, dt))
+    y_exact = torch.nn.functional.conv2d(xt, wt, torch.tensor(oracle.to_f64(b, dt)), padding=p).numpy()
+    got = oracle.to_f64(dy_.numpy(), dt)
+    assert oracle.rel_err(got, oracle.to_f64(y_ref, dt)) <= tol(dt, Ci * kH * kW)
+    assert oracle.rel_err(got, y_exact) <= tol(dt, Ci * kH * kW)
+    # without a bias the result is the fp32 sum rounded once: no further from float64 than one 16-bit rounding
+    capi.check(L.rp_hip_conv2d_same_forward(dy_.ptr, dx_.ptr, dw_.ptr, None, N, Ci, H, W, Co, kH, kW, dt), "same forward")
+    y_nb = torch.nn.functional.conv2d(xt, wt, None, padding=p).numpy()
+    assert oracle.rel_err(oracle.to_f64(dy_.numpy(), dt), y_nb) <= (2.0 ** -8 if dt == BF16 else 2.0 ** -11)
+    # gradient with respect to the input
+    if Co % 64 == 0:
+        g = rand_storage(rng, (N, Co, H, W), dt)
+        dg_, dgx_ = Dev(g, dt), Dev.empty((N, Ci, H, W), dt)
+        capi.check(L.rp_hip_conv2d_same_backward_input(dgx_.ptr, dg_.ptr, dw_.ptr, N, Ci, H, W, Co, kH, kW, dt), "same backward")
+        dx_ref, _, _ = oracle.conv2d_backward(x, w, g, s, p, d, dt, with_bias=False)
+        dx_exact = torch.nn.grad.conv2d_input((N, Ci, H, W), wt, torch.tensor(oracle.to_f64(g, dt)), padding=p).numpy()
+        got = oracle.to_f64(dgx_.numpy(), dt)
+        assert oracle.rel_err(got, oracle.to_f64(dx_ref, dt)) <= tol(dt, Co * kH * kW)
+        assert oracle.rel_err(got, dx_exact) <= (2.0 ** -8 if dt == BF16 else 2.0 ** -11)
+    else:
+        assert L.rp_hip_conv2d_same_supported(Co, H, W, kH, kW, dt) == 0
+
+
+def test_same_convolution_rejects_other_shapes():
+    L = capi.lib()
+    assert L.rp_hip_conv2d_same_supported(64, 8, 8, 3, 3, F32) == 0            # 16-bit types only
+    assert L.rp_hip_conv2d_same_supported(48, 8, 8, 3, 3, BF16) == 0           # channels in whole slabs of 64
+    assert L.rp_hip_conv2d_same_supported(64, 8, 8, 2, 2, BF16) == 0           # odd kernels only
+    assert L.rp_hip_conv2d_same_supported(64, 8, 8, 1, 1, BF16) == 0           # 1 x 1 needs no lowering in the first place
+    d = Dev.empty((64 * 64,), BF16)
+    assert L.rp_hip_conv2d_same_forward(d.ptr, d.ptr, d.ptr, None, 1, 48, 8, 8, 64, 3, 3, BF16) == -1
+    assert b"rp_hip_conv2d_same_supported" in L.rp_hip_last_error()
+
+
 # ---- through the drop-in module -------------------------------------------------------------------------------
 def _dev(arr, dt, grad=False):
     """storage array -> device tensor (16-bit values travel as float32, exactly)."""
@@ -155,6 +214,7 @@ def test_conv2d_forward_and_backward(dt, case, monkeypatch):
     # with the lowered matrix limited to one sample at a time the batch goes in chunks of one: the GEMMs then run
     # unbatched (a different kernel and split of k may be chosen), so the comparison is to tolerance, not to the bit
     monkeypatch.setenv("RP_CONV_COL_BYTES", "1")
+    monkeypatch.setenv("RP_CONV_NO_DIRECT", "1")           # and always through the lowered matrix
     again = _run_conv(x, w, b, dy, s, p, d, dt)
     for name, g, r, k in zip(names, again, refs, ks):
         if r is not None:
