@@ -370,15 +370,15 @@ def conv2d_times(capi, dt_name="bf16"):
     out["fwd_bwd_ms"] = round(total, 4)
     out["fwd_bwd_TFLOP/s"] = round(3 * gemm_flops / total / 1e9, 1)
     if L.rp_hip_conv2d_same_supported(C, H, W, k, k, dt) == 1:
-        # forward and input gradient straight from zero-bordered planes (no lowered matrix); the weight gradient still lowers
+        # forward and both gradients straight from zero-bordered planes (no lowered matrix)
         direct = {
             "y=conv(x,W)+b": (lambda: capi.check(L.rp_hip_conv2d_same_forward(d_y.ptr, d_x.ptr, d_w.ptr, d_b.ptr, N, C, H, W, Co, k, k, dt), "same forward"),
                               gemm_flops, N * (x_n + y_n) * esz),
-            "dx=conv_t(dy,W)": (lambda: capi.check(L.rp_hip_conv2d_same_backward_input(d_dx.ptr, d_dy.ptr, d_w.ptr, N, C, H, W, Co, k, k, dt), "same backward"),
-                                gemm_flops, N * (x_n + y_n) * esz),
+            "dx,dW=conv_bwd(dy,x,W)": (lambda: capi.check(L.rp_hip_conv2d_same_backward(d_dx.ptr, d_dw.ptr, d_dy.ptr, d_x.ptr, d_w.ptr, N, C, H, W, Co, k, k, dt), "same backward"),
+                                       2 * gemm_flops, N * (2 * x_n + y_n) * esz),
         }
         out["lowered_fwd_bwd_ms"] = out["fwd_bwd_ms"]
-        total = (out["im2col"]["us"] + out["dW_n=dy.colt"]["us"] + out["dW=sum_n"]["us"] + out["db"]["us"]) * 1e-3
+        total = out["db"]["us"] * 1e-3
         for name, (fn, flops, nbytes) in direct.items():
             ms = _time_graph(capi, fn, 10, 2)
             total += ms

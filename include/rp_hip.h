@@ -211,17 +211,23 @@ int rp_hip_col2im_batched(void* im, const void* col, int batch, int C_in, int H,
 
 /* Convolution without the lowered matrix, for stride 1, no dilation, odd kernels with padding (k - 1) / 2 ("same"
  * output size) in bfloat16 / float16 when the channel count that is summed over is a multiple of 64
- * (rp_hip_conv2d_same_supported says whether a shape qualifies).  x [batch, C_in, H, W], w [C_out, C_in, kH, kW],
+ * (rp_hip_conv2d_same_supported says whether a shape qualifies; reduced_channels 0 asks about geometry and dtype alone).  x [batch, C_in, H, W], w [C_out, C_in, kH, kW],
  * y / dy [batch, C_out, H, W], all dense.  The input is copied once into zero-bordered planes and the GEMM reads
  * every tap from that copy in place; the sum over taps and channels is kept in fp32 and rounded once, then the bias
  * is added with its own rounding as in rp_hip_channel_bias_add.  They stand in for the per-sample
- * im2col + matmul (+ col2im) loops of op_conv2d and backward_conv2d_fn (ops/ops.c:4759-4783, 4533-4551); the weight
- * gradient keeps the lowered matrix. */
+ * im2col + matmul (+ col2im) loops of op_conv2d and backward_conv2d_fn (ops/ops.c:4759-4783, 4533-4551). */
 int rp_hip_conv2d_same_supported(int reduced_channels, int H, int W, int kH, int kW, int dtype);
 int rp_hip_conv2d_same_forward(void* y, const void* x, const void* w, const void* bias, int batch, int C_in, int H, int W,
                                int C_out, int kH, int kW, int dtype);
 int rp_hip_conv2d_same_backward_input(void* dx, const void* dy, const void* w, int batch, int C_in, int H, int W,
                                       int C_out, int kH, int kW, int dtype);
+/* Both gradients from one zero-bordered copy of dy; dx or dw may be NULL (x is read only for dw, w only for dx).
+ * dx needs rp_hip_conv2d_same_supported(C_out, ...); dw [C_out, C_in, kH, kW] needs
+ * rp_hip_conv2d_same_supported(0, ...), i.e. only the geometry and the dtype: its reduction runs over the positions
+ * of a sample (every (tap, channel) column of the GEMM is a shifted plane of the padded input), the per-sample
+ * products are rounded and then summed over the batch in fp32 as in the lowered path (ops/ops.c:4575-4617). */
+int rp_hip_conv2d_same_backward(void* dx, void* dw, const void* dy, const void* x, const void* w, int batch, int C_in, int H, int W,
+                                int C_out, int kH, int kW, int dtype);
 
 /* y[n, c, :] += bias[c] for y [batch, channels, hw]: the reference pulls y to the host for this loop
  * (ops/ops.c:4772-4836). */

@@ -77,6 +77,7 @@ SIGNATURES = {
     "rp_hip_conv2d_same_supported": (_i, [_i] * 6),
     "rp_hip_conv2d_same_forward": (_i, [_vp] * 4 + [_i] * 8),
     "rp_hip_conv2d_same_backward_input": (_i, [_vp] * 3 + [_i] * 8),
+    "rp_hip_conv2d_same_backward": (_i, [_vp] * 5 + [_i] * 8),
     "rp_hip_channel_sums": (_i, [_vp, _vp, _i, _i, _i, _i, _i]),
     "rp_hip_lstm_cell_forward": (_i, [_vp] * 6 + [_ll, _i, _i, _i]),
     "rp_hip_lstm_cell_backward": (_i, [_vp] * 6 + [_ll, _i, _i, _i]),

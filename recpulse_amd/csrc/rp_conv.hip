@@ -399,8 +399,10 @@ __global__ void conv_weights_by_tap_kernel(T* out, const T* w, int C_out, int C_
     }
 }
 
+static PadGeom pad_geom(int H, int W, int kH, int kW, int vec);
+
 static bool same_conv_ok(int reduced_channels, int H, int W, int kH, int kW, int dtype) {
-    return (dtype == RP_DTYPE_BFLOAT16 || dtype == RP_DTYPE_FLOAT16) && reduced_channels > 0 && reduced_channels % M16_BK == 0 &&
+    return (dtype == RP_DTYPE_BFLOAT16 || dtype == RP_DTYPE_FLOAT16) && reduced_channels >= 0 && reduced_channels % M16_BK == 0 &&
            H > 0 && W > 0 && kH > 0 && kW > 0 && kH % 2 == 1 && kW % 2 == 1 && kH * kW > 1 && kW <= 15 && kH <= 15 &&
            (long long)(H + kH) * (W + kW + 8) < (1ll << 21);
 }
@@ -411,10 +413,7 @@ template <typename T>
 static int same_conv_run(void* out, const void* in, const void* wt, const void* bias, int batch, int C_from, int C_to,
                          int H, int W, int kH, int kW, int dtype) {
     constexpr int VEC = 16 / (int)sizeof(T);
-    PadGeom pg;
-    pg.H = H; pg.W = W; pg.ph = kH / 2; pg.pw = kW / 2; pg.Hp = H + kH - 1;
-    pg.Wp = (W + kW - 1 + VEC - 1) / VEC * VEC;
-    pg.P = (long long)pg.Hp * pg.Wp + 2 * VEC;               // the last tap of the last position reads up to kW - 2 elements past Hp * Wp
+    const PadGeom pg = pad_geom(H, W, kH, kW, VEC);
     const long long cols = (long long)H * pg.Wp;
     const long long per_sample = ((long long)C_from * pg.P + (long long)C_to * cols) * (long long)sizeof(T);
     long long chunk = (1ll << 30) / per_sample;
@@ -472,6 +471,100 @@ static int same_conv(void* out, const void* in, const void* w, const void* bias,
     const int rc = same_conv_run<T>(out, in, wt, bias, batch, C_from, C_to, H, W, kH, kW, dtype);
     rp_hip_free(wt);
     return rc;
+}
+
+// dw[co][ci][tap] = by_tap[co][tap][ci]: the weight gradient back in the weights' own order
+template <typename T>
+__global__ void conv_weights_from_tap_kernel(T* dw, const T* by_tap, int C_out, int C_in, int taps) {
+    const int total = C_out * C_in * taps;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+        const int tap = i % taps, ci = (i / taps) % C_in, co = i / (taps * C_in);
+        dw[i] = by_tap[((size_t)co * taps + tap) * C_in + ci];
+    }
+}
+
+static PadGeom pad_geom(int H, int W, int kH, int kW, int vec) {
+    PadGeom pg;
+    pg.H = H; pg.W = W; pg.ph = kH / 2; pg.pw = kW / 2; pg.Hp = H + kH - 1;
+    pg.Wp = (W + kW - 1 + vec - 1) / vec * vec;
+    pg.P = (long long)pg.Hp * pg.Wp + 2 * vec;               // the last tap of the last position reads up to kW - 2 elements past Hp * Wp
+    return pg;
+}
+
+// Both gradients of a same-padding convolution from one zero-bordered copy of dy (either output may be null).
+//   dx[n, ci]       = sum over taps and co of w[co, ci, reversed tap] . padded(dy)[n, co] shifted by the tap      (segments along k)
+//   dw[co, ci, tap] = sum over n and positions of padded(dy)[n, co] . padded(x)[n, ci] shifted by the tap          (segments along n),
+// the per-sample products rounded to T and then added over the batch in the accumulate type, as the lowered path does.
+template <typename T>
+static int same_conv_backward(void* dx, void* dw, const void* dy, const void* x, const void* w, int batch, int C_in, int H, int W,
+                              int C_out, int kH, int kW, int dtype) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    const PadGeom pg = pad_geom(H, W, kH, kW, VEC);
+    const int taps = kH * kW;
+    const long long cols = (long long)H * pg.Wp, w_n = (long long)C_out * C_in * taps;
+    const long long product_n = (dx && (long long)C_in * cols > (dw ? w_n : 0)) ? (long long)C_in * cols : (dw ? w_n : (long long)C_in * cols);
+    const long long per_sample = ((long long)C_out * pg.P + (dw ? (long long)C_in * pg.P : 0) + product_n) * (long long)sizeof(T);
+    long long chunk = (1ll << 30) / per_sample;
+    chunk = chunk < 1 ? 1 : (chunk > 32768 ? 32768 : chunk);
+    if (chunk > batch) chunk = batch;
+    const long long most_channels = C_in > C_out ? C_in : C_out;
+    if (chunk * most_channels * (pg.P / VEC) >= (1ll << 31) || chunk * (long long)C_in * H * W >= (1ll << 31) || w_n >= (1ll << 31) ||
+        most_channels * pg.P >= (1ll << 30)) {
+        set_error("conv2d backward: one sample is too large for the padded-plane path");
+        return -1;
+    }
+    void *dy_pad = nullptr, *x_pad = nullptr, *product = nullptr, *wt = nullptr, *dw_by_tap = nullptr;
+    bool ok = rp_hip_malloc(&dy_pad, (size_t)(chunk * C_out * pg.P) * sizeof(T)) == 0 &&
+              rp_hip_malloc(&product, (size_t)(chunk * product_n) * sizeof(T)) == 0 &&
+              (!dx || rp_hip_malloc(&wt, (size_t)w_n * sizeof(T)) == 0) &&
+              (!dw || (rp_hip_malloc(&x_pad, (size_t)(chunk * C_in * pg.P) * sizeof(T)) == 0 && rp_hip_malloc(&dw_by_tap, (size_t)w_n * sizeof(T)) == 0));
+    const unsigned w_grid = (unsigned)((w_n + 255) / 256 > 1024 ? 1024 : (w_n + 255) / 256);
+    if (ok && dx) hipLaunchKernelGGL(conv_weights_by_tap_kernel<T>, dim3(w_grid), dim3(256), 0, current_stream(), (T*)wt, (const T*)w, C_out, C_in, taps, 1);
+    for (int b0 = 0; ok && b0 < batch; b0 += (int)chunk) {
+        const int nb = batch - b0 < chunk ? batch - b0 : (int)chunk;
+        const T* dy0 = (const T*)dy + (size_t)b0 * C_out * H * W;
+        const unsigned dy_vecs = (unsigned)((long long)nb * C_out * (pg.P / VEC));
+        hipLaunchKernelGGL((pad_planes_kernel<T, VEC>), dim3((dy_vecs + 255) / 256), dim3(256), 0, current_stream(), (T*)dy_pad, dy0, pg, dy_vecs);
+        if (dx) {
+            T* dx0 = (T*)dx + (size_t)b0 * C_in * H * W;
+            GemmArgs g{};
+            g.C = product; g.A = wt; g.B = dy_pad;
+            g.batch = nb; g.m = C_in; g.k = taps * C_out; g.n = (int)cols;
+            g.a_bs = 0; g.a_rs = (long long)taps * C_out; g.a_cs = 1;
+            g.b_bs = (long long)C_out * pg.P; g.b_rs = pg.P; g.b_cs = 1;
+            g.c_bs = (long long)C_in * cols; g.c_rs = cols; g.c_cs = 1;
+            g.seg_slabs = C_out / M16_BK; g.seg_w = kW; g.seg_sh = pg.Wp; g.seg_sw = 1; g.b_extent = (long long)C_out * pg.P;
+            ok = launch_gemm_segmented_b(g, dtype) == 0;
+            if (!ok) break;
+            if (W % VEC == 0 && ((uintptr_t)dx0 & 15) == 0) {
+                const unsigned vecs = (unsigned)((long long)nb * C_in * H * W / VEC);
+                hipLaunchKernelGGL((unpad_planes_kernel<T, VEC>), dim3((vecs + 255) / 256), dim3(256), 0, current_stream(), dx0, (const T*)product, (const T*)nullptr, C_in, H, W, pg.Wp, vecs);
+            } else {
+                const unsigned elems = (unsigned)((long long)nb * C_in * H * W);
+                hipLaunchKernelGGL((unpad_planes_kernel<T, 1>), dim3((elems + 255) / 256), dim3(256), 0, current_stream(), dx0, (const T*)product, (const T*)nullptr, C_in, H, W, pg.Wp, elems);
+            }
+        }
+        if (dw) {
+            const T* x0 = (const T*)x + (size_t)b0 * C_in * H * W;
+            const unsigned x_vecs = (unsigned)((long long)nb * C_in * (pg.P / VEC));
+            hipLaunchKernelGGL((pad_planes_kernel<T, VEC>), dim3((x_vecs + 255) / 256), dim3(256), 0, current_stream(), (T*)x_pad, x0, pg, x_vecs);
+            GemmArgs g{};
+            g.C = product;
+            g.A = (const T*)dy_pad + (size_t)pg.ph * pg.Wp + pg.pw;          // dy in the pitch of the padded planes, zeros in the columns past W
+            g.B = x_pad;
+            g.batch = nb; g.m = C_out; g.k = (int)cols; g.n = taps * C_in;
+            g.a_bs = (long long)C_out * pg.P; g.a_rs = pg.P; g.a_cs = 1;
+            g.b_bs = (long long)C_in * pg.P; g.b_rs = 1; g.b_cs = pg.P;
+            g.c_bs = w_n; g.c_rs = (long long)taps * C_in; g.c_cs = 1;
+            g.seg_n = C_in; g.seg_w = kW; g.seg_sh = pg.Wp; g.seg_sw = 1; g.b_extent = (long long)C_in * pg.P;
+            ok = launch_gemm_segmented_b(g, dtype) == 0 && rp_hip_reduce_rows(dw_by_tap, product, nb, (int)w_n, b0 > 0 ? 1 : 0, dtype) == 0;
+        }
+    }
+    if (ok && dw) hipLaunchKernelGGL(conv_weights_from_tap_kernel<T>, dim3(w_grid), dim3(256), 0, current_stream(), (T*)dw, (const T*)dw_by_tap, C_out, C_in, taps);
+    if (ok && !check_launch("padded-plane convolution kernels")) ok = false;
+    for (void* p : {dy_pad, x_pad, product, wt, dw_by_tap})
+        if (p) rp_hip_free(p);
+    return ok ? 0 : -1;
 }
 
 static bool geom_ok(const ConvGeom& g) {
@@ -618,8 +711,19 @@ int rp_hip_conv2d_same_backward_input(void* dx, const void* dy, const void* w, i
         set_error("rp_hip_conv2d_same_backward_input: null operand or a shape outside rp_hip_conv2d_same_supported");
         return -1;
     }
-    if (dtype == RP_DTYPE_BFLOAT16) return same_conv<bf16_t>(dx, dy, w, nullptr, batch, C_out, C_in, H, W, kH, kW, true, dtype);
-    return same_conv<f16_t>(dx, dy, w, nullptr, batch, C_out, C_in, H, W, kH, kW, true, dtype);
+    if (dtype == RP_DTYPE_BFLOAT16) return same_conv_backward<bf16_t>(dx, nullptr, dy, nullptr, w, batch, C_in, H, W, C_out, kH, kW, dtype);
+    return same_conv_backward<f16_t>(dx, nullptr, dy, nullptr, w, batch, C_in, H, W, C_out, kH, kW, dtype);
+}
+
+int rp_hip_conv2d_same_backward(void* dx, void* dw, const void* dy, const void* x, const void* w, int batch, int C_in, int H, int W,
+                                int C_out, int kH, int kW, int dtype) {
+    const bool shapes = batch > 0 && C_in > 0 && C_out > 0 && same_conv_ok(dx ? C_out : 0, H, W, kH, kW, dtype);
+    if ((!dx && !dw) || !dy || (dx && !w) || (dw && !x) || !shapes) {
+        set_error("rp_hip_conv2d_same_backward: null operand or a shape outside rp_hip_conv2d_same_supported");
+        return -1;
+    }
+    if (dtype == RP_DTYPE_BFLOAT16) return same_conv_backward<bf16_t>(dx, dw, dy, x, w, batch, C_in, H, W, C_out, kH, kW, dtype);
+    return same_conv_backward<f16_t>(dx, dw, dy, x, w, batch, C_in, H, W, C_out, kH, kW, dtype);
 }
 
 int rp_hip_channel_bias_add(void* y, const void* bias, int batch, int channels, int hw, int dtype) {

@@ -24,6 +24,10 @@ struct GemmArgs {
     // copy of the image instead of from a lowered matrix.  b_extent: elements of one batch entry of B that may be read.
     int seg_slabs, seg_w;
     long long seg_sh, seg_sw, b_extent;
+    // Or B's n axis in segments of seg_n columns (B with unit stride along k): column j = (s, c) sits at the
+    // segment's offset (same formula) plus c * b_cs.  This is the weight gradient: the reduction runs over positions
+    // and every (tap, channel) column is a shifted plane of the padded image.
+    int seg_n;
 };
 
 enum Family { FAM_GENERIC = 0, FAM_SKINNY, FAM_MFMA16, FAM_MFMA16_SKINNY, FAM_MFMAW, FAM_TINY };

@@ -146,17 +146,21 @@ static int run_gemm(const GemmArgs& g, int dtype) {
 
 // C_z = A_z . B_z with B's k axis given as segments (GemmArgs::seg_*): the 16-bit MFMA kernel reads every segment
 // in place, at any 2-byte alignment.  For callers inside the library (the convolution), which guarantee: a 16-bit
-// dtype, A in a fast layout with a 16-byte aligned base, B with unit stride along n, k a whole number of segments.
+// dtype, A with unit stride along k or m (any 2-byte alignment), B with unit stride along n and k a whole number of
+// segments, or B with unit stride along k and n a whole number of segments.
 int launch_gemm_segmented_b(const GemmArgs& g, int dtype) {
     const bool is16 = dtype == RP_DTYPE_FLOAT16 || dtype == RP_DTYPE_BFLOAT16;
-    const bool a_kc = g.a_cs == 1 && g.a_rs % 8 == 0, a_mc = g.a_rs == 1 && g.a_cs % 8 == 0 && g.m % 8 == 0;
+    const bool a_kc = g.a_cs == 1, a_mc = g.a_rs == 1 && g.m % 8 == 0;
     const long long max_stride = 1ll << 22;
-    if (!is16 || !(a_kc || a_mc) || !aligned16(g.A) || g.a_bs % 8 || g.b_cs != 1 || g.n % 8 || g.seg_slabs <= 0 || g.seg_w <= 0 ||
-        g.k % (g.seg_slabs * M16_BK) || g.a_rs >= max_stride || g.a_cs >= max_stride || g.b_rs >= max_stride || g.batch > 65535) {
+    bool ok = is16 && (a_kc || a_mc) && g.seg_w > 0 && g.a_rs < max_stride && g.a_cs < max_stride && g.b_rs < max_stride && g.b_cs < max_stride &&
+              g.batch <= 65535 && g.b_extent > 0 && g.b_extent < (1ll << 30);
+    if (g.seg_slabs > 0) ok = ok && g.seg_n == 0 && g.b_cs == 1 && g.n % 8 == 0 && g.k % (g.seg_slabs * M16_BK) == 0;      // segments along k
+    else ok = ok && g.seg_n > 0 && g.b_rs == 1 && g.k % 8 == 0 && g.n % g.seg_n == 0;                                       // segments along n
+    if (!ok) {
         set_error("segmented GEMM: operands outside what the 16-bit MFMA kernel reads in place");
         return -1;
     }
-    Plan p{FAM_MFMA16, 64, 64, !a_kc, true, true, "mfma16"};
+    Plan p{FAM_MFMA16, 64, 64, !a_kc, g.seg_slabs > 0, true, "mfma16"};
     choose_tile16(p, g.batch, g.m, g.k, g.n);
     return launch_mfma16(g, p, dtype);
 }

@@ -156,10 +156,11 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     const uint16_t* b_mat = (const uint16_t*)g.B + (long long)z * g.b_bs;
     // uniform pointers to the tile's current slab and one past the operand's last valid element
     const char* a_slab = (const char*)(a_mat + (long long)m0 * a_fs + (long long)kbeg * a_ks);
-    const char* b_slab = (const char*)(b_mat + (long long)n0 * b_fs + (long long)kbeg * b_ks);
+    const bool n_segmented = !B_MC && g.seg_n > 0;           // B's columns are a list of segments: offsets are taken from B itself, not from the tile
+    const char* b_slab = (const char*)(b_mat + (n_segmented ? 0ll : (long long)n0 * b_fs) + (long long)kbeg * b_ks);
     const char* a_end = (const char*)(a_mat + ((long long)(g.m - 1) * a_fs + (long long)(kend - 1) * a_ks + 1));
     const bool segmented = g.seg_slabs > 0;                 // B's k axis is a list of segments (never together with SPLITK)
-    const char* b_end = segmented ? (const char*)(b_mat + g.b_extent)
+    const char* b_end = (segmented || n_segmented) ? (const char*)(b_mat + g.b_extent)
                                   : (const char*)(b_mat + ((long long)(g.n - 1) * b_fs + (long long)(kend - 1) * b_ks + 1));
     const long long a_step = (long long)M16_BK * a_ks * 2, b_step = (long long)M16_BK * b_ks * 2;
     // From the last slab of a segment the pointer goes back to the segment's start and on to the next one's: one
@@ -195,6 +196,11 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
         int r = b_r0 + (B_MC ? 0 : i * MapB::PIECE_ROWS), kk = b_kk0 + (B_MC ? i * MapB::PIECE_ROWS : 0);
         b_goff[i] = (uint32_t)(((long long)r * b_fs + (long long)kk * b_ks) * 2);
         if (EDGE && B_MC && n0 + r >= g.n) b_goff[i] = M16_OOB;
+        if (n_segmented) {
+            const int j = n0 + r, seg = j / g.seg_n, c = j - seg * g.seg_n;
+            const long long at = (long long)(seg / g.seg_w) * g.seg_sh + (long long)(seg % g.seg_w) * g.seg_sw + (long long)c * b_fs + (long long)kk * b_ks;
+            b_goff[i] = (EDGE && j >= g.n) ? M16_OOB : (uint32_t)(at * 2);        // the descriptor's end no longer stands for "past the last column"
+        }
     }
     const int a_wr0 = MapA::lds_off(a_r0, a_kk0), b_wr0 = A_ELEMS + MapB::lds_off(b_r0, b_kk0);     // LDS element offsets of piece 0
     const int a_fr0 = FragA::base(wm0, lane), b_fr0 = A_ELEMS + FragB::base(wn0, lane);

@@ -840,14 +840,22 @@ void backward_conv2d_fn(GradFn* self, Tensor* grad_output) {         // referenc
     Tensor* xd = dense(x); Tensor* wd = dense(w);
     void* col = nullptr;
     bool ok = g && xd && wd;
-    const bool direct_dx = !pointwise && conv_direct(c, dt, c.Co);
-    if (ok && !pointwise && ((needs_grad(x) && !direct_dx) || needs_grad(w))) ok = rp_hip_malloc(&col, (size_t)chunk * col_n * esz) == 0;
-    if (ok && needs_grad(x)) {
-        // dcol[n] = W^T . dy[n], then each input pixel gathers its taps; or the taps straight from zero-bordered planes of dy
+    const bool direct_dx = !pointwise && conv_direct(c, dt, c.Co), direct_dw = !pointwise && conv_direct(c, dt, 0);
+    if (ok && !pointwise && ((needs_grad(x) && !direct_dx) || (needs_grad(w) && !direct_dw))) ok = rp_hip_malloc(&col, (size_t)chunk * col_n * esz) == 0;
+    if (ok && ((needs_grad(x) && direct_dx) || (needs_grad(w) && direct_dw))) {
+        // both gradients from one zero-bordered copy of dy, no lowered matrix
+        Tensor* dx = (needs_grad(x) && direct_dx) ? empty_tensor(dt, x->device_id, x->ndim, x->shape) : nullptr;
+        Tensor* dw = (needs_grad(w) && direct_dw) ? empty_tensor(dt, w->device_id, w->ndim, w->shape) : nullptr;
+        const bool good = (dx || dw) && rp_hip_conv2d_same_backward(dx ? dx->data : nullptr, dw ? dw->data : nullptr, g->data, xd->data, wd->data,
+                                                                    c.N, c.C, c.H, c.W, c.Co, c.kH, c.kW, dt) == 0;
+        if (good) { if (dx) accumulate_grad(x, dx); if (dw) accumulate_grad(w, dw); }
+        else { dev_fail("op_conv2d backward (padded planes)"); free_tensor(dx); free_tensor(dw); ok = false; }
+    }
+    if (ok && needs_grad(x) && !direct_dx) {
+        // dcol[n] = W^T . dy[n], then each input pixel gathers its taps
         Tensor* dx = empty_tensor(dt, x->device_id, x->ndim, x->shape);
         bool good = dx != nullptr;
-        if (good && direct_dx) good = rp_hip_conv2d_same_backward_input(dx->data, g->data, wd->data, c.N, c.C, c.H, c.W, c.Co, c.kH, c.kW, dt) == 0;
-        for (int n0 = 0; good && !direct_dx && n0 < c.N; n0 += chunk) {
+        for (int n0 = 0; good && n0 < c.N; n0 += chunk) {
             const int nb = c.N - n0 < chunk ? c.N - n0 : chunk;
             char* dx_n = (char*)dx->data + n0 * x_n * esz;
             const char* g_n = (const char*)g->data + n0 * y_n * esz;
@@ -857,7 +865,7 @@ void backward_conv2d_fn(GradFn* self, Tensor* grad_output) {         // referenc
         }
         if (good) accumulate_grad(x, dx); else { dev_fail("op_conv2d backward (input)"); free_tensor(dx); }
     }
-    if (ok && needs_grad(w)) {
+    if (ok && needs_grad(w) && !direct_dw) {
         // per-sample dy[n] . col[n]^T as one batched GEMM, then the sum over the batch in the accumulate type
         Tensor* dw = empty_tensor(dt, w->device_id, w->ndim, w->shape);
         void* per_sample = nullptr;

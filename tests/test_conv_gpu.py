@@ -107,7 +107,7 @@ def test_lowering_rejects_inconsistent_geometry():
 
 SAME_CASES = [  # (batch, C_in, H, W, C_out, kH, kW): whole tiles, ragged columns, several slabs per tap, 5 x 5, one row
     (3, 64, 8, 8, 64, 3, 3), (2, 128, 14, 14, 64, 3, 3), (2, 64, 7, 20, 192, 3, 3), (1, 64, 9, 12, 32, 5, 5),
-    (2, 64, 1, 16, 64, 3, 1), (1, 64, 56, 56, 64, 3, 3)]
+    (2, 64, 1, 16, 64, 3, 1), (1, 64, 56, 56, 64, 3, 3), (5, 64, 10, 10, 24, 3, 3)]
 
 
 @pytest.mark.parametrize("dt", [BF16, F16], ids=lambda d: NAMES[d])
@@ -146,6 +146,21 @@ def test_same_convolution_without_lowered_matrix(dt, case):
         assert oracle.rel_err(got, dx_exact) <= (2.0 ** -8 if dt == BF16 else 2.0 ** -11)
     else:
         assert L.rp_hip_conv2d_same_supported(Co, H, W, kH, kW, dt) == 0
+        g = rand_storage(rng, (N, Co, H, W), dt)
+        dg_ = Dev(g, dt)
+    # gradient with respect to the weights (any channel counts), alone and together with the input gradient
+    assert L.rp_hip_conv2d_same_supported(0, H, W, kH, kW, dt) == 1
+    dgw_ = Dev.empty((Co, Ci, kH, kW), dt)
+    capi.check(L.rp_hip_conv2d_same_backward(None, dgw_.ptr, dg_.ptr, dx_.ptr, None, N, Ci, H, W, Co, kH, kW, dt), "same backward (weights)")
+    _, dw_ref, _ = oracle.conv2d_backward(x, w, g, s, p, d, dt, with_bias=False)
+    dw_exact = torch.nn.grad.conv2d_weight(xt, (Co, Ci, kH, kW), torch.tensor(oracle.to_f64(g, dt)), padding=p).numpy()
+    got_w = oracle.to_f64(dgw_.numpy(), dt)
+    assert oracle.rel_err(got_w, oracle.to_f64(dw_ref, dt).reshape(got_w.shape)) <= tol(dt, N * H * W)
+    assert oracle.rel_err(got_w, dw_exact) <= tol(dt, N * H * W)
+    if Co % 64 == 0:
+        both_x, both_w = Dev.empty((N, Ci, H, W), dt), Dev.empty((Co, Ci, kH, kW), dt)
+        capi.check(L.rp_hip_conv2d_same_backward(both_x.ptr, both_w.ptr, dg_.ptr, dx_.ptr, dw_.ptr, N, Ci, H, W, Co, kH, kW, dt), "same backward (both)")
+        assert np.array_equal(both_x.numpy(), dgx_.numpy()) and np.array_equal(both_w.numpy(), dgw_.numpy())
 
 
 def test_same_convolution_rejects_other_shapes():
