@@ -62,7 +62,10 @@ static void choose_tile16(Plan& p, int batch, int m, int k, int n) {
     // fewer than 128 tiles of 128 x 128 would leave over half the CUs idle: the 64 x 64 tile quadruples the workgroups
     // (1024^3: 10.9 -> 7.3 us)
     // at most 64 rows: a 64 x 256 tile (the same 64 x 64 patch per wave as the 128 x 128 tile, none of it past the last row)
-    else if (m <= 64 && n >= 256 && wide64() && (long long)((n + 255) / 256) * batch >= 128) { p.bm = 64; p.bn = 256; p.name = "mfma16_64x256"; }
+    // (64 x 128 while k is short: two blocks share a CU and one's loads and stores overlap the other's few slabs)
+    else if (m <= 64 && n >= 256 && wide64() && (long long)((n + 255) / 256) * batch >= 128) {
+        p.bm = 64; p.bn = k <= 1024 ? 128 : 256; p.name = k <= 1024 ? "mfma16_64x128" : "mfma16_64x256";
+    }
     else if ((m > 64 || n > 64) && tiles128 >= 128) { p.bm = 128; p.bn = 128; p.name = "mfma16_128x128"; }
     else { p.bm = 64; p.bn = 64; p.name = "mfma16_64x64"; }
     p.edge = (m % p.bm) || (n % p.bn) || (k % M16_BK);

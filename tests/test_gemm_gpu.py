@@ -264,6 +264,26 @@ def test_large_tile_kernel_multi_slab():
         assert oracle.rel_err(oracle.to_f64(got[rows], dt), oracle.to_f64(want, dt)) <= tol(dt, k)
 
 
+def test_wide_tiles_for_outputs_of_at_most_64_rows():
+    """Up to 64 rows and many columns: 64 x 128 tiles while k is short, 64 x 256 beyond (one row of waves, no MFMA
+    spent on rows past m).  Full tiles and ragged ones, every layout, bias and accumulation; checked against float64
+    everywhere and against the oracle on a slab of columns."""
+    rng = np.random.default_rng(41)
+    cases = [(64, 192, 32768, BF16, "nn", "mfma16_64x128", False), (33, 64, 32776, F16, "nt", "mfma16_64x128", True),
+             (64, 1088, 32768, BF16, "tn", "mfma16_64x256", True), (40, 1096, 32776, F16, "nn", "mfma16_64x256", False)]
+    for m, k, n, dt, layout, kernel, epilogue in cases:
+        a, b = _operands(rng, m, k, n, dt, layout)
+        es = a.itemsize
+        assert capi.gemm_kernel_name(1, m, k, n, (a.strides[0] // es, a.strides[1] // es), (b.strides[0] // es, b.strides[1] // es), (n, 1), dt) == kernel
+        bias = rand_storage(rng, (n,), dt) if epilogue else None
+        c0 = rand_storage(rng, (m, n), dt) if epilogue else None
+        got = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=epilogue)
+        assert oracle.rel_err(oracle.to_f64(got, dt), f64_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=epilogue)) <= tol(dt, k)
+        cols = np.r_[0:8, 250:262, n - 9:n]
+        _check(got[:, cols], a, np.ascontiguousarray(b[:, cols]), dt, k, bias=None if bias is None else bias[cols],
+               c_init=None if c0 is None else np.ascontiguousarray(c0[:, cols]), accumulate=epilogue)
+
+
 def test_batch_longer_than_a_grid_axis():
     """70 000 tiny matrices in one call (the batch index rides on a grid axis of at most 65 535 blocks), A shared by
     all of them through a zero batch stride."""
