@@ -86,9 +86,30 @@ static void launch_map(T* out, const T* x1, const T* x2, Op op, size_t n) {
         hipLaunchKernelGGL((map_scalar_kernel<T, TWO, Op>), dim3(grid_for(n - done)), dim3(kThreads), 0, current_stream(), out, x1, x2, op, done, n);
 }
 
+// p[0 .. n) = v with 16-byte stores over the aligned middle (a store of one element per lane fills half a cache line
+// per wave and runs at a third of the bandwidth); the elements before and after it go one by one.
+template <typename T>
+__device__ __forceinline__ void fill_span(T* p, T v, size_t n) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+    size_t head = ((16 - ((uintptr_t)p & 15)) & 15) / sizeof(T);
+    head = head < n ? head : n;
+    const size_t nvec = (n - head) / VEC, tail0 = head + nvec * VEC;
+    T lanes[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) lanes[e] = v;
+    u32x4 pattern;
+    __builtin_memcpy(&pattern, lanes, 16);
+    u32x4* body = (u32x4*)(p + head);
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = tid; i < nvec; i += stride) body[i] = pattern;
+    if (tid < head) p[tid] = v;
+    if (tid < n - tail0) p[tail0 + tid] = v;
+}
+
 template <typename T>
 __global__ void fill_kernel(T* p, T v, size_t n) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+    fill_span(p, v, n);
 }
 
 // out[i] = scalar[0] * scale, the product taken in double and narrowed once (what the host computes when it reads
@@ -96,17 +117,27 @@ __global__ void fill_kernel(T* p, T v, size_t n) {
 template <typename T>
 __global__ void fill_scaled_kernel(T* out, const T* scalar, double scale, size_t n) {
     const T v = narrow<T>((typename traits<T>::acc)((double)widen(scalar[0]) * scale));
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) out[i] = v;
+    fill_span(out, v, n);
 }
 
 // dtype conversion pivots through fp32 like the reference (core/tensor_host.c:130-207),
 // except float64 <-> float64 / float32 which are direct.
+// GROUP elements per thread (the whole groups of the array; the rest go one by one), read and written as one
+// vector each when `vectors` says both arrays are aligned for that.
 template <typename D, typename S>
-__global__ void convert_kernel(D* dst, const S* src, size_t n) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
-        auto w = widen(src[i]);
-        dst[i] = narrow<D>((typename traits<D>::acc)w);
+__global__ void convert_kernel(D* dst, const S* src, size_t n, int vectors) {
+    constexpr int GROUP = 16 / (int)(sizeof(D) < sizeof(S) ? sizeof(D) : sizeof(S));      // the narrower side moves 16 bytes
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (size_t)gridDim.x * blockDim.x;
+    const size_t groups = vectors ? n / GROUP : 0;
+    for (size_t i = tid; i < groups; i += stride) {
+        S in[GROUP];
+        D out[GROUP];
+        __builtin_memcpy(in, __builtin_assume_aligned(src + i * GROUP, 16), sizeof(in));
+#pragma unroll
+        for (int e = 0; e < GROUP; e++) out[e] = narrow<D>((typename traits<D>::acc)widen(in[e]));
+        __builtin_memcpy(__builtin_assume_aligned(dst + i * GROUP, 16), out, sizeof(out));
     }
+    for (size_t i = groups * GROUP + tid; i < n; i += stride) dst[i] = narrow<D>((typename traits<D>::acc)widen(src[i]));
 }
 
 // ---- broadcasting add ------------------------------------------------------------
@@ -561,12 +592,14 @@ template <> f16_t host_narrow<f16_t>(double value) {
 
 template <typename D>
 static int convert_from(void* dst, const void* src, int src_dtype, size_t size) {
-    unsigned blocks = grid_for(size);
+    // every group of elements is at least 16 bytes on either side, so 16-byte aligned bases keep every group aligned
+    const int vectors = (((uintptr_t)dst | (uintptr_t)src) & 15) == 0 ? 1 : 0;
+    unsigned blocks = grid_for(vectors ? size / 2 + 1 : size);
     switch (src_dtype) {
-        case RP_DTYPE_FLOAT32:  hipLaunchKernelGGL((convert_kernel<D, float>), dim3(blocks), dim3(kThreads), 0, current_stream(), (D*)dst, (const float*)src, size); break;
-        case RP_DTYPE_FLOAT64:  hipLaunchKernelGGL((convert_kernel<D, double>), dim3(blocks), dim3(kThreads), 0, current_stream(), (D*)dst, (const double*)src, size); break;
-        case RP_DTYPE_FLOAT16:  hipLaunchKernelGGL((convert_kernel<D, f16_t>), dim3(blocks), dim3(kThreads), 0, current_stream(), (D*)dst, (const f16_t*)src, size); break;
-        case RP_DTYPE_BFLOAT16: hipLaunchKernelGGL((convert_kernel<D, bf16_t>), dim3(blocks), dim3(kThreads), 0, current_stream(), (D*)dst, (const bf16_t*)src, size); break;
+        case RP_DTYPE_FLOAT32:  hipLaunchKernelGGL((convert_kernel<D, float>), dim3(blocks), dim3(kThreads), 0, current_stream(), (D*)dst, (const float*)src, size, vectors); break;
+        case RP_DTYPE_FLOAT64:  hipLaunchKernelGGL((convert_kernel<D, double>), dim3(blocks), dim3(kThreads), 0, current_stream(), (D*)dst, (const double*)src, size, vectors); break;
+        case RP_DTYPE_FLOAT16:  hipLaunchKernelGGL((convert_kernel<D, f16_t>), dim3(blocks), dim3(kThreads), 0, current_stream(), (D*)dst, (const f16_t*)src, size, vectors); break;
+        case RP_DTYPE_BFLOAT16: hipLaunchKernelGGL((convert_kernel<D, bf16_t>), dim3(blocks), dim3(kThreads), 0, current_stream(), (D*)dst, (const bf16_t*)src, size, vectors); break;
         default: set_error("rp_hip_convert: unsupported source dtype %d", src_dtype); return -1;
     }
     return check_launch("convert_kernel") ? 0 : -1;
@@ -699,7 +732,7 @@ int sum_dim_kernel_device(void* out, const void* x, size_t outer_size, size_t di
 
 int rp_hip_fill(void* ptr, double value, size_t size, int dtype) {
     RP_REQUIRE(ptr && size, "rp_hip_fill");
-    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(fill_kernel<T>, dim3(grid_for(size)), dim3(kThreads), 0, current_stream(),
+    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(fill_kernel<T>, dim3(grid_for(size * sizeof(T) / 16 + 16)), dim3(kThreads), 0, current_stream(),
                                                (T*)ptr, host_narrow<T>(value), size));
     return check_launch("fill_kernel") ? 0 : -1;
 }
@@ -752,7 +785,7 @@ int rp_hip_cross_entropy_backward(void* grad_logits, const void* logits, const i
 
 int rp_hip_fill_scaled(void* ptr, const void* scalar_dev, double scale, size_t size, int dtype) {
     RP_REQUIRE(ptr && scalar_dev && size, "rp_hip_fill_scaled");
-    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(fill_scaled_kernel<T>, dim3(grid_for(size)), dim3(kThreads), 0, current_stream(),
+    RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(fill_scaled_kernel<T>, dim3(grid_for(size * sizeof(T) / 16 + 16)), dim3(kThreads), 0, current_stream(),
                                                (T*)ptr, (const T*)scalar_dev, scale, size));
     return check_launch("fill_scaled_kernel") ? 0 : -1;
 }

@@ -135,6 +135,20 @@ def test_fill_and_convert(dt):
         capi.check(L().rp_hip_convert(do.ptr, dst, dx.ptr, dt, 777), "convert")
         want = oracle.to_storage(oracle.to_f64(x, dt), dst)
         assert np.array_equal(do.numpy(), want), (dt, dst)
+    # bases that are not 16-byte aligned: the elements before the first boundary and after the last whole vector go one by one
+    es = x.itemsize
+    canvas = Dev(np.zeros(1100, dtype=x.dtype), dt)
+    for first, count in ((3, 1000), (1, 5), (7, 1), (5, 64)):
+        capi.check(L().rp_hip_fill(canvas.ptr, 0.0, 1100, dt), "fill")
+        capi.check(L().rp_hip_fill(canvas.ptr + first * es, 2.0, count, dt), "fill")
+        got = oracle.to_f64(canvas.numpy(), dt)
+        assert (got[first:first + count] == 2.0).all() and not got[:first].any() and not got[first + count:].any(), (first, count)
+    for dst in ALL:
+        do = Dev(np.zeros(800, dtype=oracle.to_storage(np.zeros(1), dst).dtype), dst)
+        capi.check(L().rp_hip_convert(do.ptr + do.numpy().itemsize, dst, dx.ptr + es, dt, 776), "convert")
+        want = oracle.to_storage(oracle.to_f64(x[1:], dt), dst)
+        got = do.numpy()
+        assert np.array_equal(got[1:777], want) and not oracle.to_f64(got[:1], dst).any() and not oracle.to_f64(got[777:], dst).any(), (dt, dst)
     buf = Dev.empty((1001,), F32)
     capi.check(L().rp_hip_fill(buf.ptr, 5.0, 1001, F32), "fill")
     capi.check(L().rp_hip_memset(buf.ptr + 4, 0, 4 * 999), "memset")
