@@ -335,7 +335,7 @@ struct PadGeom {
     long long P;                  // elements per padded plane (Hp * Wp plus the slack the last tap may read)
 };
 
-template <typename T, int VEC>
+template <typename T, int VEC, bool ALIGNED_ROWS>
 __global__ void __launch_bounds__(256) pad_planes_kernel(T* out, const T* in, PadGeom g, unsigned total_vec) {
     const unsigned vec_per_plane = (unsigned)(g.P / VEC);
     const unsigned gid = blockIdx.x * 256u + threadIdx.x;
@@ -344,7 +344,20 @@ __global__ void __launch_bounds__(256) pad_planes_kernel(T* out, const T* in, Pa
     const int e0 = (int)pv * VEC, r = e0 / g.Wp, c0 = e0 % g.Wp;           // Wp is a whole number of vectors: one row per vector
     const int h = r - g.ph;
     T v[VEC];
-    if (h >= 0 && h < g.H && g.W >= VEC) {
+    if (ALIGNED_ROWS && g.pw == 1) {
+        // W a whole number of vectors and one column of border: the aligned vector at c0 moved up one element, with
+        // the element before it in front
+        const bool row_inside = h >= 0 && h < g.H;
+        const T* row = in + ((size_t)plane * g.H + (row_inside ? h : 0)) * g.W;
+        T w[VEC + 1];
+        const bool have_vec = row_inside && c0 < g.W, have_left = row_inside && c0 >= 1 && c0 <= g.W;
+        const u32x4_t raw = *(const u32x4_t*)(row + (have_vec ? c0 : 0));
+        memcpy(&w[1], &raw, 16);
+        w[0] = row[have_left ? c0 - 1 : 0];
+        if (!have_left) memset(&w[0], 0, sizeof(T));
+        if (!have_vec) memset(&w[1], 0, VEC * sizeof(T));
+        memcpy(v, w, VEC * sizeof(T));
+    } else if (h >= 0 && h < g.H && g.W >= VEC) {
         load_span<T, VEC>(v, in + ((size_t)plane * g.H + h) * g.W, c0 - g.pw, g.W);
     } else {
 #pragma unroll
@@ -357,6 +370,14 @@ __global__ void __launch_bounds__(256) pad_planes_kernel(T* out, const T* in, Pa
     u32x4_t raw;
     memcpy(&raw, v, 16);
     *(u32x4_t*)(out + (size_t)plane * g.P + e0) = raw;
+}
+
+template <typename T>
+static void launch_pad(T* out, const T* in, const PadGeom& pg, unsigned vecs) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    const dim3 grid((vecs + 255) / 256);
+    if (pg.W % VEC == 0 && ((uintptr_t)in & 15) == 0) hipLaunchKernelGGL((pad_planes_kernel<T, VEC, true>), grid, dim3(256), 0, current_stream(), out, in, pg, vecs);
+    else hipLaunchKernelGGL((pad_planes_kernel<T, VEC, false>), grid, dim3(256), 0, current_stream(), out, in, pg, vecs);
 }
 
 // y[plane][h][w] = yp[plane][h * Wp + w] (+ bias[channel], one rounding add as channel_bias_add_kernel does)
@@ -433,7 +454,7 @@ static int same_conv_run(void* out, const void* in, const void* wt, const void* 
         const T* in0 = (const T*)in + (size_t)b0 * C_from * H * W;
         T* out0 = (T*)out + (size_t)b0 * C_to * H * W;
         const unsigned pad_vecs = (unsigned)((long long)nb * C_from * (pg.P / VEC));
-        hipLaunchKernelGGL((pad_planes_kernel<T, VEC>), dim3((pad_vecs + 255) / 256), dim3(256), 0, current_stream(), (T*)padded, in0, pg, pad_vecs);
+        launch_pad<T>((T*)padded, in0, pg, pad_vecs);
         GemmArgs g{};
         g.C = product; g.A = wt; g.B = padded; g.bias = nullptr;
         g.batch = nb; g.m = C_to; g.k = kH * kW * C_from; g.n = (int)cols;
@@ -524,7 +545,7 @@ static int same_conv_backward(void* dx, void* dw, const void* dy, const void* x,
         const int nb = batch - b0 < chunk ? batch - b0 : (int)chunk;
         const T* dy0 = (const T*)dy + (size_t)b0 * C_out * H * W;
         const unsigned dy_vecs = (unsigned)((long long)nb * C_out * (pg.P / VEC));
-        hipLaunchKernelGGL((pad_planes_kernel<T, VEC>), dim3((dy_vecs + 255) / 256), dim3(256), 0, current_stream(), (T*)dy_pad, dy0, pg, dy_vecs);
+        launch_pad<T>((T*)dy_pad, dy0, pg, dy_vecs);
         if (dx) {
             T* dx0 = (T*)dx + (size_t)b0 * C_in * H * W;
             GemmArgs g{};
@@ -547,7 +568,7 @@ static int same_conv_backward(void* dx, void* dw, const void* dy, const void* x,
         if (dw) {
             const T* x0 = (const T*)x + (size_t)b0 * C_in * H * W;
             const unsigned x_vecs = (unsigned)((long long)nb * C_in * (pg.P / VEC));
-            hipLaunchKernelGGL((pad_planes_kernel<T, VEC>), dim3((x_vecs + 255) / 256), dim3(256), 0, current_stream(), (T*)x_pad, x0, pg, x_vecs);
+            launch_pad<T>((T*)x_pad, x0, pg, x_vecs);
             GemmArgs g{};
             g.C = product;
             g.A = (const T*)dy_pad + (size_t)pg.ph * pg.Wp + pg.pw;          // dy in the pitch of the padded planes, zeros in the columns past W
