@@ -422,6 +422,14 @@ __global__ void conv_weights_by_tap_kernel(T* out, const T* w, int C_out, int C_
 
 static PadGeom pad_geom(int H, int W, int kH, int kW, int vec);
 
+// Bytes of padded planes and products held at a time (the batch goes in chunks).  RP_CONV_WORKSPACE_BYTES overrides the
+// 1 GiB default; it is read at every call so that tests can force several chunks.
+static long long same_conv_workspace() {
+    const char* e = getenv("RP_CONV_WORKSPACE_BYTES");
+    const long long v = e ? atoll(e) : 0;
+    return v > 0 ? v : (1ll << 30);
+}
+
 static bool same_conv_ok(int reduced_channels, int H, int W, int kH, int kW, int dtype) {
     return (dtype == RP_DTYPE_BFLOAT16 || dtype == RP_DTYPE_FLOAT16) && reduced_channels >= 0 && reduced_channels % M16_BK == 0 &&
            H > 0 && W > 0 && kH > 0 && kW > 0 && kH % 2 == 1 && kW % 2 == 1 && kH * kW > 1 && kW <= 15 && kH <= 15 &&
@@ -429,7 +437,7 @@ static bool same_conv_ok(int reduced_channels, int H, int W, int kH, int kW, int
 }
 
 // out[batch, C_to, H, W] = sum over taps and C_from of wt . padded(in[batch, C_from, H, W]); wt as conv_weights_by_tap_kernel
-// leaves it ([C_to][tap][C_from]).  bias may be null.  The batch goes in chunks that keep the workspace under 1 GiB.
+// leaves it ([C_to][tap][C_from]).  bias may be null.  The batch goes in chunks that keep the workspace under same_conv_workspace().
 template <typename T>
 static int same_conv_run(void* out, const void* in, const void* wt, const void* bias, int batch, int C_from, int C_to,
                          int H, int W, int kH, int kW, int dtype) {
@@ -437,7 +445,7 @@ static int same_conv_run(void* out, const void* in, const void* wt, const void* 
     const PadGeom pg = pad_geom(H, W, kH, kW, VEC);
     const long long cols = (long long)H * pg.Wp;
     const long long per_sample = ((long long)C_from * pg.P + (long long)C_to * cols) * (long long)sizeof(T);
-    long long chunk = (1ll << 30) / per_sample;
+    long long chunk = same_conv_workspace() / per_sample;
     chunk = chunk < 1 ? 1 : (chunk > 32768 ? 32768 : chunk);
     if (chunk > batch) chunk = batch;
     if (chunk * (long long)C_from * (pg.P / VEC) >= (1ll << 31) || chunk * (long long)C_to * H * W >= (1ll << 31)) {
@@ -525,7 +533,7 @@ static int same_conv_backward(void* dx, void* dw, const void* dy, const void* x,
     const long long cols = (long long)H * pg.Wp, w_n = (long long)C_out * C_in * taps;
     const long long product_n = (dx && (long long)C_in * cols > (dw ? w_n : 0)) ? (long long)C_in * cols : (dw ? w_n : (long long)C_in * cols);
     const long long per_sample = ((long long)C_out * pg.P + (dw ? (long long)C_in * pg.P : 0) + product_n) * (long long)sizeof(T);
-    long long chunk = (1ll << 30) / per_sample;
+    long long chunk = same_conv_workspace() / per_sample;
     chunk = chunk < 1 ? 1 : (chunk > 32768 ? 32768 : chunk);
     if (chunk > batch) chunk = batch;
     const long long most_channels = C_in > C_out ? C_in : C_out;

@@ -163,6 +163,32 @@ def test_same_convolution_without_lowered_matrix(dt, case):
         assert np.array_equal(both_x.numpy(), dgx_.numpy()) and np.array_equal(both_w.numpy(), dgw_.numpy())
 
 
+def test_same_convolution_in_chunks_of_the_batch(monkeypatch):
+    """With room for two samples at a time a batch of five goes in three chunks: same bits as in one piece (the weight
+    gradient adds its chunks in fp32 and rounds after each, so it is compared to tolerance)."""
+    dt, (N, Ci, H, W, Co, kH, kW) = BF16, (5, 64, 6, 8, 64, 3, 3)
+    L = capi.lib()
+    rng = np.random.default_rng(84)
+    x, w, g = rand_storage(rng, (N, Ci, H, W), dt), oracle.to_storage(rng.standard_normal((Co, Ci, kH, kW)) * 0.2, dt), rand_storage(rng, (N, Co, H, W), dt)
+    dx_, dw_, dg_ = Dev(x, dt), Dev(w, dt), Dev(g, dt)
+
+    def run():
+        y, gx, gw = Dev.empty((N, Co, H, W), dt), Dev.empty((N, Ci, H, W), dt), Dev.empty((Co, Ci, kH, kW), dt)
+        capi.check(L.rp_hip_conv2d_same_forward(y.ptr, dx_.ptr, dw_.ptr, None, N, Ci, H, W, Co, kH, kW, dt), "same forward")
+        capi.check(L.rp_hip_conv2d_same_backward(gx.ptr, gw.ptr, dg_.ptr, dx_.ptr, dw_.ptr, N, Ci, H, W, Co, kH, kW, dt), "same backward")
+        return y.numpy(), gx.numpy(), gw.numpy()
+
+    whole = run()
+    per_sample = (2 * 64 * (8 * 16 + 16) + 64 * 64 * 9) * 2          # padded dy and x planes plus the larger product, bytes
+    monkeypatch.setenv("RP_CONV_WORKSPACE_BYTES", str(2 * per_sample + 64))
+    parts = run()
+    assert np.array_equal(whole[0], parts[0]) and np.array_equal(whole[1], parts[1])
+    assert oracle.rel_err(oracle.to_f64(parts[2], dt), oracle.to_f64(whole[2], dt)) <= 2.0 ** -7
+    forward_per_sample = (64 * (8 * 16 + 16) + 64 * 6 * 16) * 2      # the forward holds less per sample: give it room for two as well
+    monkeypatch.setenv("RP_CONV_WORKSPACE_BYTES", str(2 * forward_per_sample + 64))
+    assert np.array_equal(whole[0], run()[0])
+
+
 def test_same_convolution_rejects_other_shapes():
     L = capi.lib()
     assert L.rp_hip_conv2d_same_supported(64, 8, 8, 3, 3, F32) == 0            # 16-bit types only
