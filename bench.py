@@ -173,6 +173,47 @@ def cpu_baseline(a, b, target_s=15.0):
                       f"host has {os.cpu_count()} logical cores"}
 
 
+def cpu_baseline_configs():
+    """The same CPU path on the smaller configurations, one core, each bounded to a second or two: configuration 1
+    (fp32 Linear forward), configuration 2 (the nine fp32 GEMMs of the MLP step), configuration 3 at N = 1024 (bf16,
+    a 256-row slab), 5a (bf16, m = 1 against the 8192 x 8192 matrix) and 5b (fp64 2048^2, a 32-row slab).
+    fp32 / fp64 products run in the reference's own matmul_kernel_host_* when oracle/_ref holds it, 16-bit ones
+    and everything else in the oracle's restatement."""
+    import oracle
+    ref = oracle.load_reference()
+    rng = np.random.default_rng(6)
+
+    def mm(a, b, dt):
+        if ref is not None and dt in (oracle.F32, oracle.F64):
+            return oracle.reference_matmul(ref, a, b, dt)
+        return oracle.matmul(a, b, dt)
+
+    def timed(shapes, dt, npdt):
+        if dt == oracle.BF16:
+            ops = [(_normal_bf16(rng, (m, k)), _normal_bf16(rng, (k, n))) for m, k, n in shapes]
+        else:
+            ops = [(rng.standard_normal((m, k)).astype(npdt), rng.standard_normal((k, n)).astype(npdt)) for m, k, n in shapes]
+        t0 = time.perf_counter()
+        for x, y in ops:
+            mm(x, y, dt)
+        sec = time.perf_counter() - t0
+        return {"ms": round(sec * 1e3, 2), "GFLOP/s": round(sum(2.0 * m * k * n for m, k, n in shapes) / sec / 1e9, 3)}
+
+    mlp = []
+    for rows, fan_in, fan_out in ((256, 784, 256), (256, 256, 128), (256, 128, 10)):
+        mlp += [(rows, fan_in, fan_out), (rows, fan_out, fan_in), (fan_in, rows, fan_out)]          # forward, dX, dW
+    out = {
+        "config1_linear_fwd_f32": timed([(128, 784, 256)], oracle.F32, np.float32),
+        "config2_mlp_9_gemms_f32": timed(mlp, oracle.F32, np.float32),
+        "config3_bf16_1024_rows_0_255": timed([(256, 1024, 1024)], oracle.BF16, np.float32),
+        "config5a_bf16_m1": timed([(1, 8192, 8192)], oracle.BF16, np.float32),           # the loop is linear in m: m = 8 and 32 take 8 and 32 times as long
+        "config5b_f64_2048_rows_0_31": timed([(32, 2048, 2048)], oracle.F64, np.float64),
+    }
+    out["kind"] = "reference for fp32/fp64, port for bf16" if ref is not None else "port"
+    out["cores"] = 1
+    return out
+
+
 def skinny_times(capi, quick_reps=20, rows=(1, 8, 32)):
     """Config 5a: bf16 A[m, 8192] x W[8192, 8192], replayed from a HIP graph; bytes are A, W and the output once."""
     out = {}
@@ -599,6 +640,8 @@ def main():
     del a, b
     if not args.no_secondary:
         line["secondary"] = secondary(capi)
+        if not args.no_cpu:
+            line["secondary"]["cpu_one_core"] = cpu_baseline_configs()
     print(json.dumps(line))
 
 
