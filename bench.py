@@ -584,6 +584,8 @@ def main():
                     help="run only the configuration-4 attention launches in bf16, unfused and fused (for profiling those kernels alone)")
     ap.add_argument("--conv-only", action="store_true",
                     help="run only the conv2d layer's launches in bf16 (for profiling those kernels alone)")
+    ap.add_argument("--mlp-only", action="store_true",
+                    help="run only the configuration-2 MLP step (C ABI from a HIP graph, eager, and through the drop-in Python API)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain copy kernel of known size (256 MiB in, 256 MiB out), the yardstick for FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
@@ -610,6 +612,11 @@ def main():
         return
     if args.attention_only:
         print(json.dumps({"attention_bf16": attention_times(capi, "bf16")}))
+        return
+    if args.mlp_only:
+        out = mlp_step_time(capi)
+        out["ms_through_python_api"] = mlp_step_time_dropin()
+        print(json.dumps({"mlp_f32_step": out}))
         return
     if args.conv_only:
         print(json.dumps({"conv2d_bf16": conv2d_times(capi, "bf16")}))
