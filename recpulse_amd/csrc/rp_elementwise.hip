@@ -542,10 +542,19 @@ __global__ void cross_entropy_kernel(T* loss, T* grad, const T* logits, const in
                 }
             }
         }
+        if (!loss) continue;                           // gradient only: nobody needs the sum (uniform: no thread reaches the barriers)
         __syncthreads();
         if (threadIdx.x == 0) {
-            int lim = batch - b0 < (int)blockDim.x ? batch - b0 : (int)blockDim.x;
-            for (int i = 0; i < lim; i++) total += nll[i];
+            const int lim = batch - b0 < (int)blockDim.x ? batch - b0 : (int)blockDim.x;
+            int i = 0;
+            for (; i + 16 <= lim; i += 16) {             // sixteen LDS reads in flight, the adds still one by one in batch order
+                double v[16];
+#pragma unroll
+                for (int u = 0; u < 16; u++) v[u] = nll[i + u];
+#pragma unroll
+                for (int u = 0; u < 16; u++) total += v[u];
+            }
+            for (; i < lim; i++) total += nll[i];
         }
         __syncthreads();
     }
