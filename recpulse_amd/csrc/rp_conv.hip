@@ -329,7 +329,9 @@ __global__ void channel_sums_finish_kernel(T* out, const typename traits<T>::acc
 // With the image copied once into planes of pitch Wp >= W + 2 * pad with a zero border, output position f = oh * Wp + ow
 // of tap (kh, kw) reads padded element f + kh * Wp + kw: every tap is the same matrix [C, H * Wp] at a different
 // offset, which the GEMM reads in place as a segment of its k axis (GemmArgs::seg_*).  The product comes out in the
-// same pitch (columns ow >= W hold sums that nobody uses) and unpad_planes_kernel copies the valid part.
+// same pitch (columns ow >= W hold sums that nobody uses): the GEMM's epilogue stores only the valid columns, folded
+// into dense planes, and adds the bias per output channel (GemmArgs::c_fold_*, bias_by_row) when image rows are whole
+// 16-byte vectors; otherwise the product stays in the planes' pitch and unpad_planes_kernel copies the valid part.
 struct PadGeom {
     int H, W, ph, pw, Hp, Wp;
     long long P;                  // elements per padded plane (Hp * Wp plus the slack the last tap may read)
@@ -471,15 +473,18 @@ static int same_conv_run(void* out, const void* in, const void* wt, const void* 
         g.c_bs = (long long)C_to * cols; g.c_rs = cols; g.c_cs = 1;
         g.accumulate = 0;
         g.seg_slabs = C_from / M16_BK; g.seg_w = kW; g.seg_sh = pg.Wp; g.seg_sw = 1; g.b_extent = (long long)C_from * pg.P;
+        if (W % VEC == 0 && ((uintptr_t)out0 & 15) == 0) {
+            // whole vectors per image row: the GEMM's epilogue drops the columns past W and adds the bias itself
+            g.C = out0; g.c_bs = (long long)C_to * H * W; g.c_rs = (long long)H * W;
+            g.c_fold_from = pg.Wp; g.c_fold_to = W; g.bias = bias; g.bias_by_row = 1;
+            rc = launch_gemm_segmented_b(g, dtype);
+            continue;
+        }
+        // rows that are not whole vectors: the product stays in the planes' pitch and a copy kernel drops the unused columns
         rc = launch_gemm_segmented_b(g, dtype);
         if (rc != 0) break;
-        if (W % VEC == 0 && ((uintptr_t)out0 & 15) == 0) {
-            const unsigned vecs = (unsigned)((long long)nb * C_to * H * W / VEC);
-            hipLaunchKernelGGL((unpad_planes_kernel<T, VEC>), dim3((vecs + 255) / 256), dim3(256), 0, current_stream(), out0, (const T*)product, (const T*)bias, C_to, H, W, pg.Wp, vecs);
-        } else {
-            const unsigned elems = (unsigned)((long long)nb * C_to * H * W);
-            hipLaunchKernelGGL((unpad_planes_kernel<T, 1>), dim3((elems + 255) / 256), dim3(256), 0, current_stream(), out0, (const T*)product, (const T*)bias, C_to, H, W, pg.Wp, elems);
-        }
+        const unsigned elems = (unsigned)((long long)nb * C_to * H * W);
+        hipLaunchKernelGGL((unpad_planes_kernel<T, 1>), dim3((elems + 255) / 256), dim3(256), 0, current_stream(), out0, (const T*)product, (const T*)bias, C_to, H, W, pg.Wp, elems);
     }
     if (rc == 0 && !check_launch("padded-plane convolution kernels")) rc = -1;
     rp_hip_free(product);
@@ -563,12 +568,11 @@ static int same_conv_backward(void* dx, void* dw, const void* dy, const void* x,
             g.b_bs = (long long)C_out * pg.P; g.b_rs = pg.P; g.b_cs = 1;
             g.c_bs = (long long)C_in * cols; g.c_rs = cols; g.c_cs = 1;
             g.seg_slabs = C_out / M16_BK; g.seg_w = kW; g.seg_sh = pg.Wp; g.seg_sw = 1; g.b_extent = (long long)C_out * pg.P;
+            const bool fold = W % VEC == 0 && ((uintptr_t)dx0 & 15) == 0;     // the epilogue stores dense planes itself
+            if (fold) { g.C = dx0; g.c_bs = (long long)C_in * H * W; g.c_rs = (long long)H * W; g.c_fold_from = pg.Wp; g.c_fold_to = W; }
             ok = launch_gemm_segmented_b(g, dtype) == 0;
             if (!ok) break;
-            if (W % VEC == 0 && ((uintptr_t)dx0 & 15) == 0) {
-                const unsigned vecs = (unsigned)((long long)nb * C_in * H * W / VEC);
-                hipLaunchKernelGGL((unpad_planes_kernel<T, VEC>), dim3((vecs + 255) / 256), dim3(256), 0, current_stream(), dx0, (const T*)product, (const T*)nullptr, C_in, H, W, pg.Wp, vecs);
-            } else {
+            if (!fold) {
                 const unsigned elems = (unsigned)((long long)nb * C_in * H * W);
                 hipLaunchKernelGGL((unpad_planes_kernel<T, 1>), dim3((elems + 255) / 256), dim3(256), 0, current_stream(), dx0, (const T*)product, (const T*)nullptr, C_in, H, W, pg.Wp, elems);
             }

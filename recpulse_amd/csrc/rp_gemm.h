@@ -28,6 +28,11 @@ struct GemmArgs {
     // segment's offset (same formula) plus c * b_cs.  This is the weight gradient: the reduction runs over positions
     // and every (tap, channel) column is a shifted plane of the padded image.
     int seg_n;
+    // Epilogue options of the 16-bit MFMA kernels (non-split path, C with unit column stride in whole 16-byte vectors).
+    // bias_by_row: bias[m] is added to row m instead of bias[n] to column n.  c_fold_from / c_fold_to: output column
+    // f = r * c_fold_from + c is stored at column r * c_fold_to + c when c < c_fold_to and dropped otherwise (both
+    // multiples of 8): a product computed in the pitch of zero-bordered planes lands in dense planes.
+    int bias_by_row, c_fold_from, c_fold_to;
 };
 
 enum Family { FAM_GENERIC = 0, FAM_SKINNY, FAM_MFMA16, FAM_MFMA16_SKINNY, FAM_MFMAW, FAM_TINY };

@@ -159,6 +159,10 @@ int launch_gemm_segmented_b(const GemmArgs& g, int dtype) {
               g.batch <= 65535 && g.b_extent > 0 && g.b_extent < (1ll << 30);
     if (g.seg_slabs > 0) ok = ok && g.seg_n == 0 && g.b_cs == 1 && g.n % 8 == 0 && g.k % (g.seg_slabs * M16_BK) == 0;      // segments along k
     else ok = ok && g.seg_n > 0 && g.b_rs == 1 && g.k % 8 == 0 && g.n % g.seg_n == 0;                                       // segments along n
+    // the folded store and the per-row bias exist on the vector path of the epilogue only
+    if (g.c_fold_from > 0)
+        ok = ok && g.c_cs == 1 && g.c_rs % 8 == 0 && g.c_bs % 8 == 0 && aligned16(g.C) && g.c_fold_from % 8 == 0 && g.c_fold_to % 8 == 0 &&
+             g.c_fold_to <= g.c_fold_from && g.n % g.c_fold_from == 0;
     if (!ok) {
         set_error("segmented GEMM: operands outside what the 16-bit MFMA kernel reads in place");
         return -1;

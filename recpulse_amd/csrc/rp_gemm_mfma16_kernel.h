@@ -379,24 +379,40 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
 #pragma unroll
         for (int j = 0; j < TNI; j++) {
             const int col = j * 32 + (lane & 31), gnl = n0 + wn0 + col;
-            const float bcol = (has_bias && (!EDGE || gnl < g.n)) ? widen(bias[gnl]) : 0.f;
-            auto stage = [&](auto with_bias) {
+            const bool by_row = g.bias_by_row != 0;
+            const float bcol = (has_bias && !by_row && (!EDGE || gnl < g.n)) ? widen(bias[gnl]) : 0.f;
+            auto stage = [&](auto with_bias, auto row_bias) {
 #pragma unroll
                 for (int i = 0; i < TMI; i++)
 #pragma unroll
                     for (int v = 0; v < 16; v++) {
                         const int row = i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
                         T y = narrow<T>(acc[i][j][v]);
-                        if constexpr (decltype(with_bias)::value) y = narrow<T>(widen(y) + bcol);
+                        if constexpr (decltype(row_bias)::value) {
+                            const int gmr = m0 + wm0 + row;
+                            y = narrow<T>(widen(y) + ((!EDGE || gmr < g.m) ? widen(bias[gmr]) : 0.f));
+                        } else if constexpr (decltype(with_bias)::value) {
+                            y = narrow<T>(widen(y) + bcol);
+                        }
                         region[row * EP + col] = y.bits;
                     }
             };
-            if (has_bias) stage(std::true_type{});
-            else stage(std::false_type{});
+            if (has_bias && by_row) stage(std::true_type{}, std::true_type{});
+            else if (has_bias) stage(std::true_type{}, std::false_type{});
+            else stage(std::false_type{}, std::false_type{});
         }
         __syncthreads();
         const int ecol = (lane % LPR) * 8, erow = lane / LPR;
         const int gn = n0 + wn0 + ecol;
+        // folded output: this lane's 8 columns keep their place inside a run of c_fold_from columns, the runs
+        // move together to c_fold_to columns each, and the columns past c_fold_to of a run are not stored
+        int gn_out = gn;
+        bool live = true;
+        if (g.c_fold_from > 0) {
+            const int run = gn / g.c_fold_from, within = gn - run * g.c_fold_from;
+            live = within < g.c_fold_to;
+            gn_out = run * g.c_fold_to + within;
+        }
 #pragma unroll 4
         for (int r = erow; r < WM; r += RPS) {
             const int gm = m0 + wm0 + r;
@@ -404,17 +420,18 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
             const u32x4_t staged = *(const u32x4_t*)(region + r * EP + ecol);
             T* crow = C + (long long)gm * g.c_rs;
             if (c_vec && (!EDGE || gn + 8 <= g.n)) {
+                if (!live) continue;
                 u32x4_t o = staged;
                 if (accum) {
                     T y[8], old[8], out[8];
-                    const u32x4_t was = *(const u32x4_t*)(crow + gn);
+                    const u32x4_t was = *(const u32x4_t*)(crow + gn_out);
                     memcpy(y, &staged, 16);
                     memcpy(old, &was, 16);
 #pragma unroll
                     for (int e = 0; e < 8; e++) out[e] = narrow<T>(widen(old[e]) + widen(y[e]));
                     memcpy(&o, out, 16);
                 }
-                __builtin_nontemporal_store(o, (u32x4_t*)(crow + gn));      // written once, never re-read: keep it out of the way of the operand panels in L2
+                __builtin_nontemporal_store(o, (u32x4_t*)(crow + gn_out));  // written once, never re-read: keep it out of the way of the operand panels in L2
             } else {
                 T y[8];
                 memcpy(y, &staged, 16);
