@@ -438,6 +438,38 @@ static bool same_conv_ok(int reduced_channels, int H, int W, int kH, int kW, int
            (long long)(H + kH) * (W + kW + 8) < (1ll << 21);
 }
 
+// out[nb, C_to, H, W] (dense) = sum over taps and C_from of wt[C_to][tap][C_from] . padded[nb, C_from, planes of pg], (+ bias per
+// channel): the GEMM whose k axis walks the taps as segments.  When image rows are whole 16-byte vectors its epilogue
+// stores only the valid columns, folded into dense planes, and adds the bias; otherwise the product goes to `product`
+// ([nb, C_to, H * Wp]) and a copy kernel drops the unused columns.
+template <typename T>
+static int taps_gemm(T* out, void* product, const void* wt, const void* padded, const void* bias, int nb, int C_from, int C_to,
+                     const PadGeom& pg, int kH, int kW, int dtype) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    const int H = pg.H, W = pg.W;
+    const long long cols = (long long)H * pg.Wp;
+    const bool fold = W % VEC == 0 && ((uintptr_t)out & 15) == 0;
+    GemmArgs g{};
+    g.A = wt; g.B = padded;
+    g.batch = nb; g.m = C_to; g.k = kH * kW * C_from; g.n = (int)cols;
+    g.a_bs = 0; g.a_rs = (long long)kH * kW * C_from; g.a_cs = 1;
+    g.b_bs = (long long)C_from * pg.P; g.b_rs = pg.P; g.b_cs = 1;
+    g.seg_slabs = C_from / M16_BK; g.seg_w = kW; g.seg_sh = pg.Wp; g.seg_sw = 1; g.b_extent = (long long)C_from * pg.P;
+    g.c_cs = 1;
+    if (fold) {
+        g.C = out; g.c_bs = (long long)C_to * H * W; g.c_rs = (long long)H * W;
+        g.c_fold_from = pg.Wp; g.c_fold_to = W; g.bias = bias; g.bias_by_row = 1;
+    } else {
+        g.C = product; g.c_bs = (long long)C_to * cols; g.c_rs = cols;
+    }
+    if (launch_gemm_segmented_b(g, dtype) != 0) return -1;
+    if (!fold) {
+        const unsigned elems = (unsigned)((long long)nb * C_to * H * W);
+        hipLaunchKernelGGL((unpad_planes_kernel<T, 1>), dim3((elems + 255) / 256), dim3(256), 0, current_stream(), out, (const T*)product, (const T*)bias, C_to, H, W, pg.Wp, elems);
+    }
+    return 0;
+}
+
 // out[batch, C_to, H, W] = sum over taps and C_from of wt . padded(in[batch, C_from, H, W]); wt as conv_weights_by_tap_kernel
 // leaves it ([C_to][tap][C_from]).  bias may be null.  The batch goes in chunks that keep the workspace under same_conv_workspace().
 template <typename T>
@@ -465,26 +497,7 @@ static int same_conv_run(void* out, const void* in, const void* wt, const void* 
         T* out0 = (T*)out + (size_t)b0 * C_to * H * W;
         const unsigned pad_vecs = (unsigned)((long long)nb * C_from * (pg.P / VEC));
         launch_pad<T>((T*)padded, in0, pg, pad_vecs);
-        GemmArgs g{};
-        g.C = product; g.A = wt; g.B = padded; g.bias = nullptr;
-        g.batch = nb; g.m = C_to; g.k = kH * kW * C_from; g.n = (int)cols;
-        g.a_bs = 0; g.a_rs = (long long)kH * kW * C_from; g.a_cs = 1;
-        g.b_bs = (long long)C_from * pg.P; g.b_rs = pg.P; g.b_cs = 1;
-        g.c_bs = (long long)C_to * cols; g.c_rs = cols; g.c_cs = 1;
-        g.accumulate = 0;
-        g.seg_slabs = C_from / M16_BK; g.seg_w = kW; g.seg_sh = pg.Wp; g.seg_sw = 1; g.b_extent = (long long)C_from * pg.P;
-        if (W % VEC == 0 && ((uintptr_t)out0 & 15) == 0) {
-            // whole vectors per image row: the GEMM's epilogue drops the columns past W and adds the bias itself
-            g.C = out0; g.c_bs = (long long)C_to * H * W; g.c_rs = (long long)H * W;
-            g.c_fold_from = pg.Wp; g.c_fold_to = W; g.bias = bias; g.bias_by_row = 1;
-            rc = launch_gemm_segmented_b(g, dtype);
-            continue;
-        }
-        // rows that are not whole vectors: the product stays in the planes' pitch and a copy kernel drops the unused columns
-        rc = launch_gemm_segmented_b(g, dtype);
-        if (rc != 0) break;
-        const unsigned elems = (unsigned)((long long)nb * C_to * H * W);
-        hipLaunchKernelGGL((unpad_planes_kernel<T, 1>), dim3((elems + 255) / 256), dim3(256), 0, current_stream(), out0, (const T*)product, (const T*)bias, C_to, H, W, pg.Wp, elems);
+        rc = taps_gemm<T>(out0, product, wt, padded, bias, nb, C_from, C_to, pg, kH, kW, dtype);
     }
     if (rc == 0 && !check_launch("padded-plane convolution kernels")) rc = -1;
     rp_hip_free(product);
@@ -561,21 +574,8 @@ static int same_conv_backward(void* dx, void* dw, const void* dy, const void* x,
         launch_pad<T>((T*)dy_pad, dy0, pg, dy_vecs);
         if (dx) {
             T* dx0 = (T*)dx + (size_t)b0 * C_in * H * W;
-            GemmArgs g{};
-            g.C = product; g.A = wt; g.B = dy_pad;
-            g.batch = nb; g.m = C_in; g.k = taps * C_out; g.n = (int)cols;
-            g.a_bs = 0; g.a_rs = (long long)taps * C_out; g.a_cs = 1;
-            g.b_bs = (long long)C_out * pg.P; g.b_rs = pg.P; g.b_cs = 1;
-            g.c_bs = (long long)C_in * cols; g.c_rs = cols; g.c_cs = 1;
-            g.seg_slabs = C_out / M16_BK; g.seg_w = kW; g.seg_sh = pg.Wp; g.seg_sw = 1; g.b_extent = (long long)C_out * pg.P;
-            const bool fold = W % VEC == 0 && ((uintptr_t)dx0 & 15) == 0;     // the epilogue stores dense planes itself
-            if (fold) { g.C = dx0; g.c_bs = (long long)C_in * H * W; g.c_rs = (long long)H * W; g.c_fold_from = pg.Wp; g.c_fold_to = W; }
-            ok = launch_gemm_segmented_b(g, dtype) == 0;
+            ok = taps_gemm<T>(dx0, product, wt, dy_pad, nullptr, nb, C_out, C_in, pg, kH, kW, dtype) == 0;
             if (!ok) break;
-            if (!fold) {
-                const unsigned elems = (unsigned)((long long)nb * C_in * H * W);
-                hipLaunchKernelGGL((unpad_planes_kernel<T, 1>), dim3((elems + 255) / 256), dim3(256), 0, current_stream(), dx0, (const T*)product, (const T*)nullptr, C_in, H, W, pg.Wp, elems);
-            }
         }
         if (dw) {
             const T* x0 = (const T*)x + (size_t)b0 * C_in * H * W;
