@@ -54,5 +54,8 @@ def test_kernel_selection_names():
     assert name(1, 128, 4096, 256, (4096, 1), (256, 1), (256, 1), capi.F32) == "mfma32_64x64"        # deeper k: small tile + split-k over workgroups
     assert name(1, 4096, 4096, 4096, (4096, 1), (4096, 1), (4096, 1), capi.F32) == "mfma32_128x128"
     assert name(1, 2048, 2048, 2048, (2048, 1), (2048, 1), (2048, 1), capi.F64) == "mfma64_128x128"
+    assert name(64, 64, 576, 3136, (576, 1), (3136, 1), (3136, 1), capi.BF16) == "mfma16_64x128"           # at most 64 rows, short k (a lowered convolution)
+    assert name(64, 64, 3136, 576, (3136, 1), (1, 3136), (576, 1), capi.F16) == "mfma16_64x256"            # at most 64 rows, long k (its weight gradient)
+    assert name(1, 64, 1024, 4096, (1024, 1), (4096, 1), (4096, 1), capi.BF16) == "mfma16_64x64"           # too few column tiles for the wide ones
     assert name(1, 5, 7, 3, (7, 1), (3, 1), (3, 1), capi.BF16) == "generic"                                # odd extents
     assert name(1, 64, 64, 64, (128, 2), (64, 1), (64, 1), capi.F64) == "generic"                          # no unit stride
