@@ -433,7 +433,9 @@ static long long same_conv_workspace() {
 }
 
 static bool same_conv_ok(int reduced_channels, int H, int W, int kH, int kW, int dtype) {
-    return (dtype == RP_DTYPE_BFLOAT16 || dtype == RP_DTYPE_FLOAT16) && reduced_channels >= 0 && reduced_channels % M16_BK == 0 &&
+    // the channels summed over come in whole k slabs of the GEMM kernel that runs: 64 (16-bit), 32 (float32), 16 (float64)
+    const int slab = (dtype == RP_DTYPE_BFLOAT16 || dtype == RP_DTYPE_FLOAT16) ? M16_BK : (dtype == RP_DTYPE_FLOAT32 ? 32 : 16);
+    return dtype_size(dtype) != 0 && reduced_channels >= 0 && reduced_channels % slab == 0 &&
            H > 0 && W > 0 && kH > 0 && kW > 0 && kH % 2 == 1 && kW % 2 == 1 && kH * kW > 1 && kW <= 15 && kH <= 15 &&
            (long long)(H + kH) * (W + kW + 8) < (1ll << 21);
 }
@@ -454,7 +456,7 @@ static int taps_gemm(T* out, void* product, const void* wt, const void* padded, 
     g.batch = nb; g.m = C_to; g.k = kH * kW * C_from; g.n = (int)cols;
     g.a_bs = 0; g.a_rs = (long long)kH * kW * C_from; g.a_cs = 1;
     g.b_bs = (long long)C_from * pg.P; g.b_rs = pg.P; g.b_cs = 1;
-    g.seg_slabs = C_from / M16_BK; g.seg_w = kW; g.seg_sh = pg.Wp; g.seg_sw = 1; g.b_extent = (long long)C_from * pg.P;
+    g.seg_k = C_from; g.seg_w = kW; g.seg_sh = pg.Wp; g.seg_sw = 1; g.b_extent = (long long)C_from * pg.P;
     g.c_cs = 1;
     if (fold) {
         g.C = out; g.c_bs = (long long)C_to * H * W; g.c_rs = (long long)H * W;
@@ -534,7 +536,7 @@ static PadGeom pad_geom(int H, int W, int kH, int kW, int vec) {
     PadGeom pg;
     pg.H = H; pg.W = W; pg.ph = kH / 2; pg.pw = kW / 2; pg.Hp = H + kH - 1;
     pg.Wp = (W + kW - 1 + vec - 1) / vec * vec;
-    pg.P = (long long)pg.Hp * pg.Wp + 2 * vec;               // the last tap of the last position reads up to kW - 2 elements past Hp * Wp
+    pg.P = (long long)pg.Hp * pg.Wp + 16;                    // the last tap of the last position reads up to kW - 2 <= 13 elements past Hp * Wp
     return pg;
 }
 
@@ -734,8 +736,10 @@ int rp_hip_conv2d_same_forward(void* y, const void* x, const void* w, const void
         set_error("rp_hip_conv2d_same_forward: null operand or a shape outside rp_hip_conv2d_same_supported");
         return -1;
     }
-    if (dtype == RP_DTYPE_BFLOAT16) return same_conv<bf16_t>(y, x, w, bias, batch, C_in, C_out, H, W, kH, kW, false, dtype);
-    return same_conv<f16_t>(y, x, w, bias, batch, C_in, C_out, H, W, kH, kW, false, dtype);
+    const size_t esz = dtype_size(dtype);
+    if (((uintptr_t)x | (uintptr_t)y) & (esz - 1)) { set_error("rp_hip_conv2d_same_forward: misaligned operand"); return -1; }
+    RP_DISPATCH_DTYPE(dtype, return same_conv<T>(y, x, w, bias, batch, C_in, C_out, H, W, kH, kW, false, dtype));
+    return -1;
 }
 
 int rp_hip_conv2d_same_backward_input(void* dx, const void* dy, const void* w, int batch, int C_in, int H, int W,
@@ -744,8 +748,8 @@ int rp_hip_conv2d_same_backward_input(void* dx, const void* dy, const void* w, i
         set_error("rp_hip_conv2d_same_backward_input: null operand or a shape outside rp_hip_conv2d_same_supported");
         return -1;
     }
-    if (dtype == RP_DTYPE_BFLOAT16) return same_conv_backward<bf16_t>(dx, nullptr, dy, nullptr, w, batch, C_in, H, W, C_out, kH, kW, dtype);
-    return same_conv_backward<f16_t>(dx, nullptr, dy, nullptr, w, batch, C_in, H, W, C_out, kH, kW, dtype);
+    RP_DISPATCH_DTYPE(dtype, return same_conv_backward<T>(dx, nullptr, dy, nullptr, w, batch, C_in, H, W, C_out, kH, kW, dtype));
+    return -1;
 }
 
 int rp_hip_conv2d_same_backward(void* dx, void* dw, const void* dy, const void* x, const void* w, int batch, int C_in, int H, int W,
@@ -755,8 +759,8 @@ int rp_hip_conv2d_same_backward(void* dx, void* dw, const void* dy, const void* 
         set_error("rp_hip_conv2d_same_backward: null operand or a shape outside rp_hip_conv2d_same_supported");
         return -1;
     }
-    if (dtype == RP_DTYPE_BFLOAT16) return same_conv_backward<bf16_t>(dx, dw, dy, x, w, batch, C_in, H, W, C_out, kH, kW, dtype);
-    return same_conv_backward<f16_t>(dx, dw, dy, x, w, batch, C_in, H, W, C_out, kH, kW, dtype);
+    RP_DISPATCH_DTYPE(dtype, return same_conv_backward<T>(dx, dw, dy, x, w, batch, C_in, H, W, C_out, kH, kW, dtype));
+    return -1;
 }
 
 int rp_hip_channel_bias_add(void* y, const void* bias, int batch, int channels, int hw, int dtype) {

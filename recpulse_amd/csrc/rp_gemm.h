@@ -18,20 +18,20 @@ struct GemmArgs {
     long long b_bs, b_rs, b_cs;
     long long c_bs, c_rs, c_cs;
     int accumulate;
-    // B's k axis in segments (16-bit MFMA kernels only; all zero = one plain matrix).  k is cut into segments of
-    // seg_slabs slabs of M16_BK; segment s = (sh, sw), sw = s % seg_w, starts at element offset sh * seg_sh + sw * seg_sw
+    // B's k axis in segments (MFMA kernels only; all zero = one plain matrix).  k is cut into segments of seg_k
+    // elements (whole k slabs of the kernel); segment s = (sh, sw), sw = s % seg_w, starts at element offset sh * seg_sh + sw * seg_sw
     // from B and runs with B's strides from there.  This is how a convolution reads its taps from one zero-bordered
     // copy of the image instead of from a lowered matrix.  b_extent: elements of one batch entry of B that may be read.
-    int seg_slabs, seg_w;
+    int seg_k, seg_w;
     long long seg_sh, seg_sw, b_extent;
     // Or B's n axis in segments of seg_n columns (B with unit stride along k): column j = (s, c) sits at the
     // segment's offset (same formula) plus c * b_cs.  This is the weight gradient: the reduction runs over positions
     // and every (tap, channel) column is a shifted plane of the padded image.
     int seg_n;
-    // Epilogue options of the 16-bit MFMA kernels (non-split path, C with unit column stride in whole 16-byte vectors).
+    // Epilogue options of the MFMA kernels (non-split path, C with unit column stride in whole 16-byte vectors).
     // bias_by_row: bias[m] is added to row m instead of bias[n] to column n.  c_fold_from / c_fold_to: output column
     // f = r * c_fold_from + c is stored at column r * c_fold_to + c when c < c_fold_to and dropped otherwise (both
-    // multiples of 8): a product computed in the pitch of zero-bordered planes lands in dense planes.
+    // whole 16-byte vectors): a product computed in the pitch of zero-bordered planes lands in dense planes.
     int bias_by_row, c_fold_from, c_fold_to;
 };
 

@@ -147,29 +147,39 @@ static int run_gemm(const GemmArgs& g, int dtype) {
     }
 }
 
-// C_z = A_z . B_z with B's k axis given as segments (GemmArgs::seg_*): the 16-bit MFMA kernel reads every segment
-// in place, at any 2-byte alignment.  For callers inside the library (the convolution), which guarantee: a 16-bit
-// dtype, A with unit stride along k or m (any 2-byte alignment), B with unit stride along n and k a whole number of
-// segments, or B with unit stride along k and n a whole number of segments.
+// C_z = A_z . B_z with B's k axis or its n axis given as segments (GemmArgs::seg_*): the MFMA kernels read every
+// segment in place, at any alignment of whole elements.  For callers inside the library (the convolution), which
+// guarantee: A with unit stride along k or m, B with unit stride along n and k a whole number of segments of whole
+// slabs, or B with unit stride along k and n a whole number of segments.
 int launch_gemm_segmented_b(const GemmArgs& g, int dtype) {
     const bool is16 = dtype == RP_DTYPE_FLOAT16 || dtype == RP_DTYPE_BFLOAT16;
-    const bool a_kc = g.a_cs == 1, a_mc = g.a_rs == 1 && g.m % 8 == 0;
+    const int vec = 16 / (int)dtype_size(dtype);
+    const int bk = is16 ? M16_BK : (dtype == RP_DTYPE_FLOAT32 ? 32 : 16);           // k slab of the kernel that will run
+    const bool a_kc = g.a_cs == 1, a_mc = g.a_rs == 1 && g.m % vec == 0;
     const long long max_stride = 1ll << 22;
-    bool ok = is16 && (a_kc || a_mc) && g.seg_w > 0 && g.a_rs < max_stride && g.a_cs < max_stride && g.b_rs < max_stride && g.b_cs < max_stride &&
+    bool ok = dtype_size(dtype) && (a_kc || a_mc) && g.seg_w > 0 && g.a_rs < max_stride && g.a_cs < max_stride && g.b_rs < max_stride && g.b_cs < max_stride &&
               g.batch <= 65535 && g.b_extent > 0 && g.b_extent < (1ll << 30);
-    if (g.seg_slabs > 0) ok = ok && g.seg_n == 0 && g.b_cs == 1 && g.n % 8 == 0 && g.k % (g.seg_slabs * M16_BK) == 0;      // segments along k
-    else ok = ok && g.seg_n > 0 && g.b_rs == 1 && g.k % 8 == 0 && g.n % g.seg_n == 0;                                       // segments along n
+    if (!is16) ok = ok && (a_kc ? g.a_rs % vec == 0 && g.k % vec == 0 : g.a_cs % vec == 0) && g.a_bs % vec == 0;     // the fp32 / fp64 kernel loads A with plain vector loads
+    if (g.seg_k > 0) ok = ok && g.seg_n == 0 && g.b_cs == 1 && g.n % vec == 0 && g.seg_k % bk == 0 && g.k % g.seg_k == 0;    // segments along k
+    else ok = ok && g.seg_n > 0 && g.b_rs == 1 && g.k % vec == 0 && g.n % g.seg_n == 0;                                     // segments along n
     // the folded store and the per-row bias exist on the vector path of the epilogue only
     if (g.c_fold_from > 0)
-        ok = ok && g.c_cs == 1 && g.c_rs % 8 == 0 && g.c_bs % 8 == 0 && aligned16(g.C) && g.c_fold_from % 8 == 0 && g.c_fold_to % 8 == 0 &&
+        ok = ok && g.c_cs == 1 && g.c_rs % vec == 0 && g.c_bs % vec == 0 && aligned16(g.C) && g.c_fold_from % vec == 0 && g.c_fold_to % vec == 0 &&
              g.c_fold_to <= g.c_fold_from && g.n % g.c_fold_from == 0;
     if (!ok) {
-        set_error("segmented GEMM: operands outside what the 16-bit MFMA kernel reads in place");
+        set_error("segmented GEMM: operands outside what the MFMA kernels read in place");
         return -1;
     }
-    Plan p{FAM_MFMA16, 64, 64, !a_kc, g.seg_slabs > 0, true, "mfma16"};
-    choose_tile16(p, g.batch, g.m, g.k, g.n);
-    return launch_mfma16(g, p, dtype);
+    if (is16) {
+        Plan p{FAM_MFMA16, 64, 64, !a_kc, g.seg_k > 0, true, "mfma16"};
+        choose_tile16(p, g.batch, g.m, g.k, g.n);
+        return launch_mfma16(g, p, dtype);
+    }
+    Plan p{FAM_MFMAW, 64, 64, !a_kc, g.seg_k > 0, true, "mfmaw"};
+    const long long tiles128 = (long long)((g.m + 127) / 128) * ((g.n + 127) / 128) * g.batch;
+    if (g.m > 64 && g.n > 64 && tiles128 >= 128) { p.bm = 128; p.bn = 128; }
+    p.edge = (g.m % p.bm) || (g.n % p.bn) || (g.k % bk);
+    return launch_mfmaw(g, p, dtype);
 }
 
 }  // namespace rp

@@ -159,18 +159,19 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     const bool n_segmented = !B_MC && g.seg_n > 0;           // B's columns are a list of segments: offsets are taken from B itself, not from the tile
     const char* b_slab = (const char*)(b_mat + (n_segmented ? 0ll : (long long)n0 * b_fs) + (long long)kbeg * b_ks);
     const char* a_end = (const char*)(a_mat + ((long long)(g.m - 1) * a_fs + (long long)(kend - 1) * a_ks + 1));
-    const bool segmented = g.seg_slabs > 0;                 // B's k axis is a list of segments (never together with SPLITK)
+    const int seg_slabs = g.seg_k / M16_BK;
+    const bool segmented = seg_slabs > 0;                 // B's k axis is a list of segments (never together with SPLITK)
     const char* b_end = (segmented || n_segmented) ? (const char*)(b_mat + g.b_extent)
                                   : (const char*)(b_mat + ((long long)(g.n - 1) * b_fs + (long long)(kend - 1) * b_ks + 1));
     const long long a_step = (long long)M16_BK * a_ks * 2, b_step = (long long)M16_BK * b_ks * 2;
     // From the last slab of a segment the pointer goes back to the segment's start and on to the next one's: one
     // step along seg_sw, or, after the seg_w-th segment of a row, to the start of the next row of segments.
-    const long long seg_next = segmented ? g.seg_sw * 2 - (long long)(g.seg_slabs - 1) * b_step : b_step;
+    const long long seg_next = segmented ? g.seg_sw * 2 - (long long)(seg_slabs - 1) * b_step : b_step;
     const long long seg_wrap = segmented ? (g.seg_sh - (long long)g.seg_w * g.seg_sw) * 2 : 0;
-    int seg_left = segmented ? g.seg_slabs : 0x7fffffff, seg_col = 0;
+    int seg_left = segmented ? seg_slabs : 0x7fffffff, seg_col = 0;
     auto advance_b = [&]() {
         if (--seg_left == 0) {
-            seg_left = g.seg_slabs;
+            seg_left = seg_slabs;
             b_slab += seg_next;
             if (++seg_col == g.seg_w) { seg_col = 0; b_slab += seg_wrap; }
         } else {

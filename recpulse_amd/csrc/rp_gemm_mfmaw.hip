@@ -54,7 +54,21 @@ struct MwSlab {
         int r, kk;
         coords(t, i, r, kk);
         if (EDGE && !((row0 + r < free_extent) && (k0 + kk < k_extent))) return uint4{0u, 0u, 0u, 0u};
-        return *(const uint4*)(base + (long long)(row0 + r) * free_stride + (long long)(k0 + kk) * k_stride);
+        return load_at(base + (long long)(row0 + r) * free_stride + (long long)(k0 + kk) * k_stride);
+    }
+    // the same piece with the offset of its free index given (a free axis that is a list of segments)
+    static __device__ __forceinline__ uint4 load_free_at(const T* base, long long free_offset, long long k_stride, int row0, int k0,
+                                                         int free_extent, int k_extent, int t, int i) {
+        int r, kk;
+        coords(t, i, r, kk);
+        if (EDGE && !((row0 + r < free_extent) && (k0 + kk < k_extent))) return uint4{0u, 0u, 0u, 0u};
+        return load_at(base + free_offset + (long long)(k0 + kk) * k_stride);
+    }
+    // 16 bytes from an address that is a multiple of the element size only (segment offsets shift whole elements)
+    static __device__ __forceinline__ uint4 load_at(const T* p) {
+        uint4 v;
+        __builtin_memcpy(&v, p, 16);
+        return v;
     }
     static __device__ __forceinline__ void store(T* lds, uint4 raw, int t, int i) {
         int r, kk;
@@ -127,10 +141,34 @@ __global__ void __launch_bounds__(256, 2) gemm_mfmaw_kernel(GemmArgs g, int tile
 
     uint4 regs[NP_ALL];                        // pieces 0 .. NA-1 are A's, the rest B's
     const int nslabs = (klen + BK - 1) / BK;
+    // B as a list of segments (GemmArgs::seg_*; never with SPLITK).  Along k (B_MC): every slab lies inside one segment,
+    // whose start replaces B's for that slab.  Along n (!B_MC): each piece's column has its own offset, fixed for
+    // the whole loop.
+    const bool k_segmented = B_MC && g.seg_k > 0, n_segmented = !B_MC && g.seg_n > 0;
+    long long b_free_off[NB];
+    if (n_segmented) {
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            int r, kk;
+            SlabB::coords(t, i, r, kk);
+            const int j = n0 + r < g.n ? n0 + r : g.n - 1, seg = j / g.seg_n;
+            b_free_off[i] = (long long)(seg / g.seg_w) * g.seg_sh + (long long)(seg % g.seg_w) * g.seg_sw + (long long)(j - seg * g.seg_n) * b_fs;
+        }
+    }
     auto load_piece = [&](auto pc, int k0) {
         constexpr int p = decltype(pc)::value;
-        if constexpr (p < NA) regs[p] = SlabA::load(A, a_fs, a_ks, m0, k0, g.m, klen, t, p);
-        else regs[p] = SlabB::load(B, b_fs, b_ks, n0, k0, g.n, klen, t, p - NA);
+        if constexpr (p < NA) {
+            regs[p] = SlabA::load(A, a_fs, a_ks, m0, k0, g.m, klen, t, p);
+        } else if (n_segmented) {
+            regs[p] = SlabB::load_free_at(B, b_free_off[p - NA], b_ks, n0, k0, g.n, klen, t, p - NA);
+        } else {
+            const T* base = B;
+            if (k_segmented) {
+                const int seg = k0 / g.seg_k;
+                base = B + (long long)(seg / g.seg_w) * g.seg_sh + (long long)(seg % g.seg_w) * g.seg_sw - (long long)seg * g.seg_k * b_ks;
+            }
+            regs[p] = SlabB::load(base, b_fs, b_ks, n0, k0, g.n, klen, t, p - NA);
+        }
     };
     auto store_piece = [&](auto pc, T* stage) {
         constexpr int p = decltype(pc)::value;
@@ -212,9 +250,19 @@ __global__ void __launch_bounds__(256, 2) gemm_mfmaw_kernel(GemmArgs g, int tile
                     region[(i * MT + cfg::acc_row(v, lane)) * EP + jj * MT + lf] = acc[i][p * TJ + jj][v];
         __syncthreads();
         const int gn = n0 + wn0 + p * CN + ecol;
+        const bool by_row = g.bias_by_row != 0;
         T bv[V];
 #pragma unroll
-        for (int e = 0; e < V; e++) bv[e] = (has_bias && (!EDGE || gn + e < g.n)) ? bias[gn + e] : (T)0;
+        for (int e = 0; e < V; e++) bv[e] = (has_bias && !by_row && (!EDGE || gn + e < g.n)) ? bias[gn + e] : (T)0;
+        // folded output (GemmArgs::c_fold_*): the vector keeps its place inside a run of c_fold_from columns, the runs
+        // move together to c_fold_to columns each, vectors past c_fold_to of a run are not stored
+        int gn_out = gn;
+        bool live = true;
+        if (g.c_fold_from > 0) {
+            const int run = gn / g.c_fold_from, within = gn - run * g.c_fold_from;
+            live = within < g.c_fold_to;
+            gn_out = run * g.c_fold_to + within;
+        }
 #pragma unroll 2
         for (int r = erow; r < WM; r += RPS) {
             const int gm = m0 + wm0 + r;
@@ -228,14 +276,19 @@ __global__ void __launch_bounds__(256, 2) gemm_mfmaw_kernel(GemmArgs g, int tile
                 continue;
             }
             T* crow = C + (long long)gm * g.c_rs;
+            if (has_bias && by_row) {
+#pragma unroll
+                for (int e = 0; e < V; e++) bv[e] = bias[gm];
+            }
             if (c_vec && (!EDGE || gn + V <= g.n)) {
+                if (!live) continue;
                 T old[V], out[V];
-                if (accum) { uint4 o = *(const uint4*)(crow + gn); memcpy(old, &o, 16); }
+                if (accum) { uint4 o = *(const uint4*)(crow + gn_out); memcpy(old, &o, 16); }
 #pragma unroll
                 for (int e = 0; e < V; e++) out[e] = finish<T>(vals[e], has_bias, bv[e], accum, accum ? old[e] : (T)0);
                 uint4 o;
                 memcpy(&o, out, 16);
-                *(uint4*)(crow + gn) = o;
+                *(uint4*)(crow + gn_out) = o;
             } else {
 #pragma unroll
                 for (int e = 0; e < V; e++) {
@@ -288,7 +341,7 @@ static int launch_mfmaw_t(const GemmArgs& g, const Plan& p) {
     // least two slabs deep), and add the partials in split order afterwards.  fp32 only, one matrix at a time.
     int nsplit = 1, k_per_split = 0;
     constexpr int BK = mfmaw_cfg<T>::BK;
-    if (sizeof(T) == 4 && g.batch == 1 && p.bm == 64 && g.n % 4 == 0) {
+    if (sizeof(T) == 4 && g.batch == 1 && p.bm == 64 && g.n % 4 == 0 && g.seg_k == 0 && g.seg_n == 0 && g.c_fold_from == 0 && !g.bias_by_row) {   // (segments and the folded store: never split)
         int tiles = ((g.m + 63) / 64) * ((g.n + 63) / 64);
         int want = (256 + tiles - 1) / tiles, deep = g.k / (2 * BK);
         nsplit = want < deep ? want : deep;

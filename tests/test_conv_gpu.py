@@ -110,7 +110,12 @@ SAME_CASES = [  # (batch, C_in, H, W, C_out, kH, kW): whole tiles, ragged column
     (2, 64, 1, 16, 64, 3, 1), (1, 64, 56, 56, 64, 3, 3), (5, 64, 10, 10, 24, 3, 3)]
 
 
-@pytest.mark.parametrize("dt", [BF16, F16], ids=lambda d: NAMES[d])
+def _one_rounding(dt, k):
+    """Distance from float64 of a sum kept in the accumulate type and rounded once to dt."""
+    return {BF16: 2.0 ** -8, F16: 2.0 ** -11}.get(dt, tol(dt, k))
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
 @pytest.mark.parametrize("case", SAME_CASES, ids=lambda c: "x".join(map(str, c)))
 def test_same_convolution_without_lowered_matrix(dt, case):
     """rp_hip_conv2d_same_forward / _backward_input against the oracle's per-sample chain and against float64."""
@@ -130,12 +135,14 @@ def test_same_convolution_without_lowered_matrix(dt, case):
     got = oracle.to_f64(dy_.numpy(), dt)
     assert oracle.rel_err(got, oracle.to_f64(y_ref, dt)) <= tol(dt, Ci * kH * kW)
     assert oracle.rel_err(got, y_exact) <= tol(dt, Ci * kH * kW)
-    # without a bias the result is the fp32 sum rounded once: no further from float64 than one 16-bit rounding
+    # without a bias the result is the sum in the accumulate type rounded once: no further from float64 than one rounding of dt
     capi.check(L.rp_hip_conv2d_same_forward(dy_.ptr, dx_.ptr, dw_.ptr, None, N, Ci, H, W, Co, kH, kW, dt), "same forward")
     y_nb = torch.nn.functional.conv2d(xt, wt, None, padding=p).numpy()
-    assert oracle.rel_err(oracle.to_f64(dy_.numpy(), dt), y_nb) <= (2.0 ** -8 if dt == BF16 else 2.0 ** -11)
-    # gradient with respect to the input
-    if Co % 64 == 0:
+    assert oracle.rel_err(oracle.to_f64(dy_.numpy(), dt), y_nb) <= _one_rounding(dt, Ci * kH * kW)
+    # gradient with respect to the input (C_out in whole k slabs of the dtype's kernel)
+    dx_ok = L.rp_hip_conv2d_same_supported(Co, H, W, kH, kW, dt) == 1
+    assert dx_ok == (Co % {BF16: 64, F16: 64, F32: 32, F64: 16}[dt] == 0)
+    if dx_ok:
         g = rand_storage(rng, (N, Co, H, W), dt)
         dg_, dgx_ = Dev(g, dt), Dev.empty((N, Ci, H, W), dt)
         capi.check(L.rp_hip_conv2d_same_backward_input(dgx_.ptr, dg_.ptr, dw_.ptr, N, Ci, H, W, Co, kH, kW, dt), "same backward")
@@ -143,9 +150,8 @@ def test_same_convolution_without_lowered_matrix(dt, case):
         dx_exact = torch.nn.grad.conv2d_input((N, Ci, H, W), wt, torch.tensor(oracle.to_f64(g, dt)), padding=p).numpy()
         got = oracle.to_f64(dgx_.numpy(), dt)
         assert oracle.rel_err(got, oracle.to_f64(dx_ref, dt)) <= tol(dt, Co * kH * kW)
-        assert oracle.rel_err(got, dx_exact) <= (2.0 ** -8 if dt == BF16 else 2.0 ** -11)
+        assert oracle.rel_err(got, dx_exact) <= _one_rounding(dt, Co * kH * kW)
     else:
-        assert L.rp_hip_conv2d_same_supported(Co, H, W, kH, kW, dt) == 0
         g = rand_storage(rng, (N, Co, H, W), dt)
         dg_ = Dev(g, dt)
     # gradient with respect to the weights (any channel counts), alone and together with the input gradient
@@ -157,7 +163,7 @@ def test_same_convolution_without_lowered_matrix(dt, case):
     got_w = oracle.to_f64(dgw_.numpy(), dt)
     assert oracle.rel_err(got_w, oracle.to_f64(dw_ref, dt).reshape(got_w.shape)) <= tol(dt, N * H * W)
     assert oracle.rel_err(got_w, dw_exact) <= tol(dt, N * H * W)
-    if Co % 64 == 0:
+    if dx_ok:
         both_x, both_w = Dev.empty((N, Ci, H, W), dt), Dev.empty((Co, Ci, kH, kW), dt)
         capi.check(L.rp_hip_conv2d_same_backward(both_x.ptr, both_w.ptr, dg_.ptr, dx_.ptr, dw_.ptr, N, Ci, H, W, Co, kH, kW, dt), "same backward (both)")
         assert np.array_equal(both_x.numpy(), dgx_.numpy()) and np.array_equal(both_w.numpy(), dgw_.numpy())
@@ -191,8 +197,12 @@ def test_same_convolution_in_chunks_of_the_batch(monkeypatch):
 
 def test_same_convolution_rejects_other_shapes():
     L = capi.lib()
-    assert L.rp_hip_conv2d_same_supported(64, 8, 8, 3, 3, F32) == 0            # 16-bit types only
-    assert L.rp_hip_conv2d_same_supported(48, 8, 8, 3, 3, BF16) == 0           # channels in whole slabs of 64
+    assert L.rp_hip_conv2d_same_supported(48, 8, 8, 3, 3, BF16) == 0           # channels in whole k slabs: 64 for 16-bit types,
+    assert L.rp_hip_conv2d_same_supported(48, 8, 8, 3, 3, F32) == 0            # 32 for float32,
+    assert L.rp_hip_conv2d_same_supported(32, 8, 8, 3, 3, F32) == 1
+    assert L.rp_hip_conv2d_same_supported(24, 8, 8, 3, 3, F64) == 0            # 16 for float64
+    assert L.rp_hip_conv2d_same_supported(48, 8, 8, 3, 3, F64) == 1
+    assert L.rp_hip_conv2d_same_supported(64, 8, 8, 3, 3, 99) == 0             # no such dtype
     assert L.rp_hip_conv2d_same_supported(64, 8, 8, 2, 2, BF16) == 0           # odd kernels only
     assert L.rp_hip_conv2d_same_supported(64, 8, 8, 1, 1, BF16) == 0           # 1 x 1 needs no lowering in the first place
     d = Dev.empty((64 * 64,), BF16)
