@@ -210,10 +210,11 @@ int rp_hip_col2im_batched(void* im, const void* col, int batch, int C_in, int H,
                           int out_H, int out_W, int accumulate, int dtype);
 
 /* Convolution without the lowered matrix, for stride 1, no dilation, odd kernels with padding (k - 1) / 2 ("same"
- * output size) in bfloat16 / float16 when the channel count that is summed over is a multiple of 64
- * (rp_hip_conv2d_same_supported says whether a shape qualifies; reduced_channels 0 asks about geometry and dtype alone).  x [batch, C_in, H, W], w [C_out, C_in, kH, kW],
- * y / dy [batch, C_out, H, W], all dense.  The input is copied once into zero-bordered planes and the GEMM reads
- * every tap from that copy in place; the sum over taps and channels is kept in fp32 and rounded once, then the bias
+ * output size) when the channel count that is summed over is a multiple of 64 (bfloat16 / float16), 32 (float32)
+ * or 16 (float64); rp_hip_conv2d_same_supported says whether a shape qualifies, reduced_channels 0 asks about
+ * geometry and dtype alone.  x [batch, C_in, H, W], w [C_out, C_in, kH, kW], y / dy [batch, C_out, H, W], all dense.
+ * The input is copied once into zero-bordered planes and the GEMM reads every tap from that copy in place; the sum
+ * over taps and channels is kept in the accumulate type (fp32; fp64 for float64) and rounded once, then the bias
  * is added with its own rounding as in rp_hip_channel_bias_add.  They stand in for the per-sample
  * im2col + matmul (+ col2im) loops of op_conv2d and backward_conv2d_fn (ops/ops.c:4759-4783, 4533-4551). */
 int rp_hip_conv2d_same_supported(int reduced_channels, int H, int W, int kH, int kW, int dtype);

@@ -325,7 +325,7 @@ __global__ void channel_sums_finish_kernel(T* out, const typename traits<T>::acc
     out[c] = r;
 }
 
-// ---- convolution without a lowered matrix (stride 1, "same" padding, 16-bit types) ----
+// ---- convolution without a lowered matrix (stride 1, "same" padding) ----
 // With the image copied once into planes of pitch Wp >= W + 2 * pad with a zero border, output position f = oh * Wp + ow
 // of tap (kh, kw) reads padded element f + kh * Wp + kw: every tap is the same matrix [C, H * Wp] at a different
 // offset, which the GEMM reads in place as a segment of its k axis (GemmArgs::seg_*).  The product comes out in the

@@ -810,7 +810,7 @@ bool conv_is_pointwise(const ConvSaved& c) {              // 1x1, unit stride, n
     return c.kH == 1 && c.kW == 1 && c.sh == 1 && c.sw == 1 && c.ph == 0 && c.pw == 0;
 }
 
-// Stride 1, no dilation, odd kernel with padding (k - 1) / 2, a 16-bit type and `reduced` channels in whole slabs of
+// Stride 1, no dilation, odd kernel with padding (k - 1) / 2 and `reduced` channels in whole k slabs of
 // the GEMM: the convolution (reduced = C_in) or its input gradient (reduced = C_out) reads its taps from zero-bordered
 // planes and never builds the lowered matrix.  RP_CONV_NO_DIRECT=1 keeps the lowered path (read at every call).
 bool conv_direct(const ConvSaved& c, DType dt, int reduced) {
