@@ -305,6 +305,7 @@ def secondary(capi, quick_reps=20):
     out["lstm_step_f32"] = lstm_step_times(capi, "f32")
     # config 2: fp32 MLP 784-256-128-10, batch 256, forward + backward through the C ABI (9 GEMMs + neighbours)
     out["mlp_f32_step"] = mlp_step_time(capi)
+    out["mlp_f32_step"]["ms_separate_launches"] = mlp_step_time(capi, fused_backward=False)["ms"]
     out["mlp_f32_step"]["ms_through_python_api"] = mlp_step_time_dropin()
     return out
 
@@ -479,7 +480,10 @@ def lstm_step_times(capi, dt_name="bf16"):
     return out
 
 
-def mlp_step_time(capi, reps=50):
+def mlp_step_time(capi, reps=50, fused_backward=True):
+    """Configuration 2 through the C ABI.  fused_backward: each layer's three gradients (dX, dW, db) come from one
+    rp_hip_linear_backward call, which runs them as one launch for layers this small; False issues the two GEMMs and
+    the bias reduction separately (the same bits, 18 launches instead of 12)."""
     import ctypes
     rng = np.random.default_rng(1)
     dims = [784, 256, 128, 10]; batch = 256
@@ -508,19 +512,25 @@ def mlp_step_time(capi, reps=50):
         for i in (2, 1, 0):
             m, k, n = batch, dims[i], dims[i + 1]
             inp = d_x if i == 0 else d_h[i - 1]
-            L.rp_hip_reduce_rows(d_db[i].ptr, d_g[i].ptr, m, n, 0, F)
-            # dW[k,n] = inpᵀ[k,m] · g[m,n]
-            capi.gemm(d_dw[i].ptr, inp.ptr, d_g[i].ptr, None, 1, k, m, n, (0, 1, k), (0, n, 1), (0, n, 1), False, F)
-            # dIn[m,k] = g[m,n] · Wᵀ[n,k]
             dst = d_dx if i == 0 else d_gh[i - 1]
-            capi.gemm(dst.ptr, d_g[i].ptr, d_w[i].ptr, None, 1, m, n, k, (0, n, 1), (0, 1, n), (0, k, 1), False, F)
+            if fused_backward:
+                L.rp_hip_linear_backward(dst.ptr, d_dw[i].ptr, d_db[i].ptr, d_g[i].ptr, inp.ptr, d_w[i].ptr, m, k, n,
+                                         k, 1, n, 1, k, 1, n, 1, 0, 0, 0, F)
+            else:
+                L.rp_hip_reduce_rows(d_db[i].ptr, d_g[i].ptr, m, n, 0, F)
+                # dW[k,n] = inpᵀ[k,m] · g[m,n]
+                capi.gemm(d_dw[i].ptr, inp.ptr, d_g[i].ptr, None, 1, k, m, n, (0, 1, k), (0, n, 1), (0, n, 1), False, F)
+                # dIn[m,k] = g[m,n] · Wᵀ[n,k]
+                capi.gemm(dst.ptr, d_g[i].ptr, d_w[i].ptr, None, 1, m, n, k, (0, n, 1), (0, 1, n), (0, k, 1), False, F)
             if i > 0:
                 L.backwards_relu_device(d_gh[i - 1].ptr, d_z[i - 1].ptr, d_g[i - 1].ptr, m * k, F)
 
     ms = _time_launches(capi, step, reps, 5)
     ms_graph = _time_graph(capi, step, 10, 2)
-    return {"ms": ms_graph, "ms_eager_from_python": ms, "launches": 18, "note": "9 GEMMs (bias fused into the 3 forward ones), 2 relu, 2 relu-backward, "
-            "cross-entropy fwd+bwd, 3 bias-gradient reductions; `ms` replays the step from a HIP graph, "
+    return {"ms": ms_graph, "ms_eager_from_python": ms, "launches": 12 if fused_backward else 18,
+            "note": "9 GEMMs (bias fused into the 3 forward ones), 2 relu, 2 relu-backward, "
+            "cross-entropy fwd+bwd, 3 bias-gradient reductions; with each layer's dX, dW and db in one launch (rp_hip_linear_backward) "
+            "that is 12 launches, issued separately 18 (`ms_separate_launches`); `ms` replays the step from a HIP graph, "
             "`ms_eager_from_python` launches it call by call through ctypes, `ms_through_python_api` is the same step through "
             "the drop-in recpulse_cuda tensors, recpulse.module.Linear and autograd (wall clock, allocation and graph bookkeeping included)"}
 
@@ -615,6 +625,7 @@ def main():
         return
     if args.mlp_only:
         out = mlp_step_time(capi)
+        out["ms_separate_launches"] = mlp_step_time(capi, fused_backward=False)["ms"]
         out["ms_through_python_api"] = mlp_step_time_dropin()
         print(json.dumps({"mlp_f32_step": out}))
         return

@@ -163,6 +163,17 @@ int rp_hip_fill(void* ptr, double value, size_t size, int dtype);
 int rp_hip_fill_scaled(void* ptr, const void* scalar_dev, double scale, size_t size, int dtype);
 int rp_hip_convert(void* dst, int dst_dtype, const void* src, int src_dtype, size_t size);
 
+/* The backward of y = x . w + b for 2-D operands in one call: dx [m, k] = dy . w^T, dw [k, n] = x^T . dy,
+ * db [n] = column sums of dy (rows added top to bottom, as rp_hip_reduce_rows).  dy [m, n] is dense; x [m, k], w [k, n],
+ * dx and dw carry (row, column) strides in elements; any of dx, dw, db may be NULL; accumulate_* = 1 adds to what the
+ * output holds.  Same values, bit for bit, as two rp_hip_gemm_strided_batched calls with the transposes as swapped
+ * strides (backward_matmul_fn, ops/ops.c:6759-6814) and rp_hip_reduce_rows; for small float32 layers (the
+ * one-launch 16 x 16-tile kernel's range) the three run as ONE launch, which is most of such a layer's time. */
+int rp_hip_linear_backward(void* dx, void* dw, void* db, const void* dy, const void* x, const void* w, int m, int k, int n,
+                           long long x_rs, long long x_cs, long long w_rs, long long w_cs,
+                           long long dx_rs, long long dx_cs, long long dw_rs, long long dw_cs,
+                           int accumulate_dx, int accumulate_dw, int accumulate_db, int dtype);
+
 /* Bias gradient of Linear on the device: grad [rows, cols] dense -> out [cols],
  * each column summed top to bottom in fp32 (fp64 for float64).  Stands in for
  * the device->host->device round trip of reduce_grad_to_shape

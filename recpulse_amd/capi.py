@@ -66,6 +66,7 @@ SIGNATURES = {
     "rp_hip_fill": (_i, [_vp, _d, _sz, _i]),
     "rp_hip_convert": (_i, [_vp, _i, _vp, _i, _sz]),
     "rp_hip_reduce_rows": (_i, [_vp, _vp, _i, _i, _i, _i]),
+    "rp_hip_linear_backward": (_i, [_vp] * 6 + [_i] * 3 + [_ll] * 8 + [_i] * 4),
     "rp_hip_cross_entropy_mean": (_i, [_vp, _vp, _vp, _vp, _i, _i, _d, _i]),
     "rp_hip_cross_entropy_backward": (_i, [_vp, _vp, _vp, _i, _i, _vp, _i]),
     "rp_hip_fill_scaled": (_i, [_vp, _vp, _d, _sz, _i]),

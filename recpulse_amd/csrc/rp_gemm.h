@@ -142,6 +142,7 @@ int launch_mfma16(const GemmArgs& g, const Plan& p, int dtype);
 int launch_mfmaw(const GemmArgs& g, const Plan& p, int dtype);
 int launch_tiny(const GemmArgs& g, int dtype);
 int launch_gemm_segmented_b(const GemmArgs& g, int dtype);
+int launch_linear_backward_tiny(const GemmArgs& gx, const GemmArgs& gw, void* db, const void* dy, int rows, int cols, int accumulate_db);
 // adds k-split partials [nsplit][part_rows][n] (fp32, rows beyond g.m unused) in split order and runs the epilogue into C
 int launch_splitk_combine(const GemmArgs& g, const float* partials, int nsplit, int part_rows, int dtype);
 

@@ -219,6 +219,33 @@ int matmul_kernel_device(void* C, const void* A, const void* B, int m, int k, in
     return rp_hip_gemm_strided_batched(C, A, B, nullptr, 1, m, k, n, 0, k, 1, 0, n, 1, 0, n, 1, 0, dtype);
 }
 
+int rp_hip_linear_backward(void* dx, void* dw, void* db, const void* dy, const void* x, const void* w, int m, int k, int n,
+                           long long x_rs, long long x_cs, long long w_rs, long long w_cs,
+                           long long dx_rs, long long dx_cs, long long dw_rs, long long dw_cs,
+                           int accumulate_dx, int accumulate_dw, int accumulate_db, int dtype) {
+    if (!dy || (dx && !w) || (dw && !x) || m <= 0 || k <= 0 || n <= 0 || !dtype_size(dtype)) {
+        set_error("rp_hip_linear_backward: null operand, non-positive extent or unsupported dtype (m=%d k=%d n=%d)", m, k, n);
+        return -1;
+    }
+    if (x_rs < 0 || x_cs < 0 || w_rs < 0 || w_cs < 0 || dx_rs < 0 || dx_cs < 0 || dw_rs < 0 || dw_cs < 0) { set_error("rp_hip_linear_backward: negative stride"); return -1; }
+    // dx[m, k] = dy[m, n] . w^T (w [k, n] read with its strides swapped); dw[k, n] = x^T . dy (x [m, k] likewise)
+    GemmArgs gx{dx, dy, w, nullptr, 1, m, n, k, 0, n, 1, 0, w_cs, w_rs, 0, dx_rs, dx_cs, accumulate_dx};
+    GemmArgs gw{dw, x, dy, nullptr, 1, k, m, n, 0, x_cs, x_rs, 0, n, 1, 0, dw_rs, dw_cs, accumulate_dw};
+    bool fused = dtype == RP_DTYPE_FLOAT32 && (dx || dw);
+    if (fused && dx) fused = make_plan(1, gx.m, gx.k, gx.n, gx.a_rs, gx.a_cs, gx.b_rs, gx.b_cs, gx.c_rs, gx.c_cs, 0, 0, dtype).fam == FAM_TINY;
+    if (fused && dw) fused = make_plan(1, gw.m, gw.k, gw.n, gw.a_rs, gw.a_cs, gw.b_rs, gw.b_cs, gw.c_rs, gw.c_cs, 0, 0, dtype).fam == FAM_TINY;
+    if (fused) {
+        // small layer: one launch does all three, block for block what the separate launches would do
+        if (!dx) gx.m = 0;
+        if (!dw) gw.m = 0;
+        return launch_linear_backward_tiny(gx, gw, db, dy, m, n, accumulate_db);
+    }
+    if (dx && run_gemm(gx, dtype) != 0) return -1;
+    if (dw && run_gemm(gw, dtype) != 0) return -1;
+    if (db && rp_hip_reduce_rows(db, dy, m, n, accumulate_db, dtype) != 0) return -1;
+    return 0;
+}
+
 const char* rp_hip_gemm_kernel_name(int batch, int m, int k, int n, long long a_rs, long long a_cs,
                                     long long b_rs, long long b_cs, long long c_rs, long long c_cs, int dtype) {
     if (batch <= 0 || m <= 0 || k <= 0 || n <= 0 || !dtype_size(dtype)) return "invalid";

@@ -698,8 +698,42 @@ void backward_add_fn(GradFn* self, Tensor* grad_output) {            // referenc
     }
 }
 
+// Where a gradient of `target` is to be written: its existing dense gradient (accumulate = 1) or a fresh tensor that
+// the caller hands to accumulate_grad afterwards.  Null when the target needs no gradient or the tensor could not be made.
+struct GradSlot { Tensor* into; Tensor* fresh; int accumulate; };
+
+GradSlot grad_slot(Tensor* target) {
+    GradSlot s{nullptr, nullptr, 0};
+    if (!target || !needs_grad(target)) return s;
+    Meta* m = ensure_meta(target);
+    if (m->grad && rp_is_contiguous(m->grad)) { s.into = m->grad; s.accumulate = 1; return s; }
+    s.fresh = empty_tensor(target->dtype, target->device_id, target->ndim, target->shape);
+    s.into = s.fresh;
+    return s;
+}
+
 void backward_linear_fn(GradFn* self, Tensor* grad_output) {
+    Tensor* x = self->inputs[0]; Tensor* w = self->inputs[1];
     Tensor* bias = self->num_inputs > 2 ? self->inputs[2] : nullptr;
+    if (x->ndim == 2 && w->ndim == 2 && on_device(x->device_id)) {
+        // one call for the three gradients: a single launch for layers as small as an MLP's
+        Tensor* g = dense(grad_output);
+        GradSlot sx = grad_slot(x), sw = grad_slot(w), sb = grad_slot(bias);
+        const int m = x->shape[0], k = x->shape[1], n = w->shape[1];
+        const bool ok = g && rp_hip_linear_backward(sx.into ? sx.into->data : nullptr, sw.into ? sw.into->data : nullptr, sb.into ? sb.into->data : nullptr,
+                                                    g->data, x->data, w->data, m, k, n, x->strides[0], x->strides[1], w->strides[0], w->strides[1],
+                                                    k, 1, n, 1, sx.accumulate, sw.accumulate, sb.accumulate, x->dtype) == 0;
+        Tensor* targets[3] = {x, w, bias};
+        GradSlot* slots[3] = {&sx, &sw, &sb};
+        for (int i = 0; i < 3; i++) {
+            if (!slots[i]->fresh) continue;
+            if (ok) accumulate_grad(targets[i], slots[i]->fresh);
+            else free_tensor(slots[i]->fresh);
+        }
+        if (!ok) dev_fail("op_linear backward");
+        free_tensor(g);
+        return;
+    }
     if (bias && needs_grad(bias)) accumulate_grad(bias, reduce_grad_to_shape(grad_output, bias->ndim, bias->shape));
     backward_matmul_fn(self, grad_output);
 }

@@ -12,7 +12,7 @@ import pytest
 
 import oracle
 from recpulse_amd import capi
-from devhelp import ALL, BF16, F16, F32, F64, NAMES, device_gemm, f64_gemm, oracle_gemm, rand_storage, tol
+from devhelp import Dev, ALL, BF16, F16, F32, F64, NAMES, device_gemm, f64_gemm, oracle_gemm, rand_storage, tol
 
 pytestmark = pytest.mark.gpu
 GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")))
@@ -282,6 +282,43 @@ def test_wide_tiles_for_outputs_of_at_most_64_rows():
         cols = np.r_[0:8, 250:262, n - 9:n]
         _check(got[:, cols], a, np.ascontiguousarray(b[:, cols]), dt, k, bias=None if bias is None else bias[cols],
                c_init=None if c0 is None else np.ascontiguousarray(c0[:, cols]), accumulate=epilogue)
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_linear_backward_in_one_call(dt):
+    """rp_hip_linear_backward against two GEMM calls with swapped strides and rp_hip_reduce_rows: the same bits,
+    whether the three run as one launch (small float32 layers) or one after the other; outputs that are absent,
+    accumulated into, and a transposed x view."""
+    rng = np.random.default_rng(42)
+    L = capi.lib()
+    for m, k, n in ((256, 784, 256), (256, 128, 10), (37, 50, 21), (512, 1024, 512)):
+        x, w, dy = rand_storage(rng, (m, k), dt), rand_storage(rng, (k, n), dt), rand_storage(rng, (m, n), dt)
+        dx0, dw0, db0 = rand_storage(rng, (m, k), dt), rand_storage(rng, (k, n), dt), rand_storage(rng, (n,), dt)
+        d_x, d_w, d_dy = Dev(x, dt), Dev(w, dt), Dev(dy, dt)
+        for acc in (0, 1):
+            want_dx, want_dw, want_db = Dev(dx0, dt), Dev(dw0, dt), Dev(db0, dt)
+            capi.gemm(want_dx.ptr, d_dy.ptr, d_w.ptr, None, 1, m, n, k, (0, n, 1), (0, 1, n), (0, k, 1), bool(acc), dt)
+            capi.gemm(want_dw.ptr, d_x.ptr, d_dy.ptr, None, 1, k, m, n, (0, 1, k), (0, n, 1), (0, n, 1), bool(acc), dt)
+            capi.check(L.rp_hip_reduce_rows(want_db.ptr, d_dy.ptr, m, n, acc, dt), "reduce_rows")
+            got_dx, got_dw, got_db = Dev(dx0, dt), Dev(dw0, dt), Dev(db0, dt)
+            capi.check(L.rp_hip_linear_backward(got_dx.ptr, got_dw.ptr, got_db.ptr, d_dy.ptr, d_x.ptr, d_w.ptr, m, k, n,
+                                                k, 1, n, 1, k, 1, n, 1, acc, acc, acc, dt), "linear_backward")
+            assert np.array_equal(got_dx.numpy(), want_dx.numpy()) and np.array_equal(got_dw.numpy(), want_dw.numpy())
+            assert np.array_equal(got_db.numpy(), want_db.numpy())
+        # only some of the outputs, and x given as the transpose of a [k, m] array
+        xt = Dev(np.ascontiguousarray(x.T), dt)
+        only_w, only_b = Dev(dw0, dt), Dev(db0, dt)
+        capi.check(L.rp_hip_linear_backward(None, only_w.ptr, None, d_dy.ptr, xt.ptr, None, m, k, n, 1, m, n, 1, k, 1, n, 1, 0, 0, 0, dt), "dw only")
+        capi.check(L.rp_hip_linear_backward(None, None, only_b.ptr, d_dy.ptr, None, None, m, k, n, k, 1, n, 1, k, 1, n, 1, 0, 0, 0, dt), "db only")
+        ref_w = Dev(dw0, dt)
+        capi.gemm(ref_w.ptr, d_x.ptr, d_dy.ptr, None, 1, k, m, n, (0, 1, k), (0, n, 1), (0, n, 1), False, dt)
+        assert oracle.rel_err(oracle.to_f64(only_w.numpy(), dt), oracle.to_f64(ref_w.numpy(), dt)) <= tol(dt, m)     # another layout may take another kernel
+        ref_b = Dev(db0, dt)
+        capi.check(L.rp_hip_reduce_rows(ref_b.ptr, d_dy.ptr, m, n, 0, dt), "reduce_rows")
+        assert np.array_equal(only_b.numpy(), ref_b.numpy())
+        _, dwant = oracle.matmul_backward(x, w, dy, dt)
+        assert oracle.rel_err(oracle.to_f64(only_w.numpy(), dt), oracle.to_f64(dwant, dt)) <= tol(dt, m)
+    assert L.rp_hip_linear_backward(None, None, None, None, None, None, 4, 4, 4, 4, 1, 4, 1, 4, 1, 4, 1, 0, 0, 0, dt) == -1
 
 
 def test_batch_longer_than_a_grid_axis():
