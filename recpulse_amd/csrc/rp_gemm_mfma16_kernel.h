@@ -38,12 +38,30 @@ template <> struct mfma16_ops<bf16_t> {
     static __device__ __forceinline__ f32x16_t mma(s16x8_t a, s16x8_t b, f32x16_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
     }
+    // 16 x 16 x 32, accumulating in place.  Written as an instruction with the accumulator tied to the result: through the
+    // builtin the register allocator gives the result another register than the accumulator it came from and moves all
+    // 256 accumulator registers around the loop (three copies per MFMA).
+    static __device__ __forceinline__ f32x4_t mma(s16x8_t a, s16x8_t b, f32x4_t c) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+        return c;
+    }
 };
 template <> struct mfma16_ops<f16_t> {
     static __device__ __forceinline__ f32x16_t mma(s16x8_t a, s16x8_t b, f32x16_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
     }
+    static __device__ __forceinline__ f32x4_t mma(s16x8_t a, s16x8_t b, f32x4_t c) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+        return c;
+    }
 };
+
+// MFMA shape of a block tile: the 256 x 256 tile multiplies with 16 x 16 x 32 (k-steps of 32), the others with 32 x 32 x 16.
+// Both run 512 multiply-adds per cycle, but the deeper instruction moves fewer register bytes per multiply-add
+// (2 KB of operands and 2 KB of accumulators per 8 192 against 2 KB and 8 KB per 16 384), and under the power limit
+// that governs a large GEMM the chip sustains a higher clock on it: a loop of nothing but MFMAs on N(0,1) operands
+// measured 1.84 PFLOP/s at 2.16 GHz against 1.65 PFLOP/s at 1.83 GHz.
+__host__ __device__ constexpr int m16_mfma_tile(int bm, int bn) { return (bm == 256 && bn == 256) ? 16 : 32; }
 
 constexpr int M16_KC_PITCH = M16_BK + 8;                       // elements
 __host__ __device__ constexpr int m16_mc_pitch(int cols) { return cols + 32; }
@@ -98,19 +116,23 @@ struct SlabMap {
 
 // Lane's base element offset for MFMA fragments of an operand tile whose wave patch starts at free index w0.
 // Fragment (tile i, k-step ks, read h) then sits at base + step(i, ks, h), a compile-time constant.
-template <int ROWS, bool MC>
+// MT: the MFMA's tile edge, 32 (k-step 16: a lane holds free index lane % 32, k octet lane / 32) or 16 (k-step 32:
+// free index lane % 16, k octet lane / 16).
+template <int ROWS, bool MC, int MT>
 struct FragMap {
+    static constexpr int KSTEP = MT == 32 ? 16 : 32;
     static __device__ __forceinline__ int base(int w0, int lane) {
-        if (!MC) return (w0 + (lane & 31)) * M16_KC_PITCH + (lane >> 5) * 8;
+        if (!MC) return (w0 + (lane % MT)) * M16_KC_PITCH + (lane / MT) * 8;
         // ds_read_b64_tr_b16: inside each 16-lane group, source lane s points at 4 consecutive free
         // indices of k-row s/4; destination lane j receives free index j of k-rows 0..3.
         int grp = lane >> 4, s = lane & 15;
-        return (8 * (grp >> 1) + (s >> 2)) * m16_mc_pitch(ROWS) + w0 + 16 * (grp & 1) + 4 * (s & 3);
+        if (MT == 32) return (8 * (grp >> 1) + (s >> 2)) * m16_mc_pitch(ROWS) + w0 + 16 * (grp & 1) + 4 * (s & 3);
+        return (8 * grp + (s >> 2)) * m16_mc_pitch(ROWS) + w0 + 4 * (s & 3);          // the four groups are the four k octets of the same 16 free indices
     }
     static constexpr int READS = MC ? 2 : 1;                 // DS instructions per fragment
     static constexpr int step(int i, int ks, int h) {
-        return MC ? ks * 16 * m16_mc_pitch(ROWS) + i * 32 + h * 4 * m16_mc_pitch(ROWS)
-                  : i * 32 * M16_KC_PITCH + ks * 16;
+        return MC ? ks * KSTEP * m16_mc_pitch(ROWS) + i * MT + h * 4 * m16_mc_pitch(ROWS)
+                  : i * MT * M16_KC_PITCH + ks * KSTEP;
     }
     // DS read H of the fragment into v (KC: the whole fragment; MC: k values 4H .. 4H+3)
     template <int H>
@@ -128,13 +150,17 @@ template <typename T, int BM, int BN, int WGM, bool A_MC, bool B_MC, bool EDGE, 
 __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_m, int tiles_n, float* partials, int k_per_split) {
     constexpr int WGN = 4 / WGM;
     constexpr int WM = BM / WGM, WN = BN / WGN;       // wave patch
-    constexpr int TMI = WM / 32, TNI = WN / 32;       // MFMA tiles per wave
+    constexpr int MT = SPLITK ? 32 : m16_mfma_tile(BM, BN);      // MFMA tile edge; k-steps of 16 (MT 32) or 32 (MT 16)
+    constexpr int NKS = MT == 32 ? 4 : 2;             // k-steps per slab
+    constexpr int NV = MT == 32 ? 16 : 4;             // accumulator registers per MFMA tile
+    using acc_t = std::conditional_t<MT == 32, f32x16_t, f32x4_t>;
+    constexpr int TMI = WM / MT, TNI = WN / MT;       // MFMA tiles per wave
     constexpr int A_ELEMS = m16_tile_elems(BM, A_MC), B_ELEMS = m16_tile_elems(BN, B_MC);
     constexpr int STAGE = A_ELEMS + B_ELEMS;          // stage s: A at smem + s*STAGE, B right after it
     using MapA = SlabMap<BM, A_MC>;
     using MapB = SlabMap<BN, B_MC>;
-    using FragA = FragMap<BM, A_MC>;
-    using FragB = FragMap<BN, B_MC>;
+    using FragA = FragMap<BM, A_MC, MT>;
+    using FragB = FragMap<BN, B_MC, MT>;
     constexpr int NA = MapA::NL, NB = MapB::NL;
     constexpr int RD_A = TMI * FragA::READS, RD_B = TNI * FragB::READS;      // DS read instructions per k-step
     constexpr int NMFMA = TMI * TNI;
@@ -206,13 +232,13 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     const int a_wr0 = MapA::lds_off(a_r0, a_kk0), b_wr0 = A_ELEMS + MapB::lds_off(b_r0, b_kk0);     // LDS element offsets of piece 0
     const int a_fr0 = FragA::base(wm0, lane), b_fr0 = A_ELEMS + FragB::base(wn0, lane);
 
-    f32x16_t acc[TMI][TNI];
+    acc_t acc[TMI][TNI];
 #pragma unroll
     for (int i = 0; i < TMI; i++)
 #pragma unroll
         for (int j = 0; j < TNI; j++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+            for (int v = 0; v < NV; v++) acc[i][j][v] = 0.f;
 
     u32x4_t ra[NA], rb[NB];
     const int nslabs = (kend - kbeg + M16_BK - 1) / M16_BK;
@@ -224,17 +250,29 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
         b_rsrc = m16_rsrc(b_slab, EDGE ? (long long)(b_end - b_slab) : 0x7fffffffll);
         kleft = kend - kbeg - k0;
     };
+    // Without edges piece i sits a uniform number of bytes after piece 0: one lane offset per operand plus a scalar
+    // offset per piece, instead of a register per piece.
+    const int a_piece_step = (int)((long long)MapA::PIECE_ROWS * (A_MC ? a_ks : a_fs) * 2);
+    const int b_piece_step = (int)((long long)MapB::PIECE_ROWS * (B_MC ? b_ks : b_fs) * 2);
     auto load_piece_a = [&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        uint32_t off = a_goff[i];
-        if (EDGE && !A_MC && a_kk0 >= kleft) off = M16_OOB;
-        ra[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)off, 0, 0);
+        if constexpr (!EDGE) {
+            ra[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)a_goff[0], i * a_piece_step, 0);
+        } else {
+            uint32_t off = a_goff[i];
+            if (!A_MC && a_kk0 >= kleft) off = M16_OOB;
+            ra[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)off, 0, 0);
+        }
     };
     auto load_piece_b = [&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        uint32_t off = b_goff[i];
-        if (EDGE && !B_MC && b_kk0 >= kleft) off = M16_OOB;
-        rb[i] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, (int)off, 0, 0);
+        if constexpr (!EDGE) {
+            rb[i] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, n_segmented ? (int)b_goff[i] : (int)b_goff[0], n_segmented ? 0 : i * b_piece_step, 0);
+        } else {
+            uint32_t off = b_goff[i];
+            if (!B_MC && b_kk0 >= kleft) off = M16_OOB;
+            rb[i] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, (int)off, 0, 0);
+        }
     };
     auto store_piece_a = [&](uint16_t* stage, auto ic) {
         constexpr int i = decltype(ic)::value;
@@ -245,13 +283,18 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
         *(u32x4_t*)(stage + b_wr0 + i * MapB::LDS_STEP) = rb[i];
     };
 
-    s16x8_t af[2][TMI], bf[2][TNI];
+    // B fragments have two slots (the next k-step's are read while this one's are multiplied).  With 32 x 32 tiles
+    // so have A's.  With 16 x 16 tiles (8 x 8 of them per wave) that would be 128 registers: A's have ONE slot, and
+    // since the MFMAs run A-tile-major, tile i's register is refilled for the next k-step as soon as its row of MFMAs
+    // has been issued.
+    constexpr int A_SLOTS = MT == 32 ? 2 : 1;
+    s16x8_t af[A_SLOTS][TMI], bf[2][TNI];
     // DS read number r (0 .. RD_A+RD_B-1) of the fragments for k-step KS into fragment slot SLOT
     auto read_item = [&](const uint16_t* stage, auto ksc, auto slotc, auto rc) {
         constexpr int KS = decltype(ksc)::value, SLOT = decltype(slotc)::value, r = decltype(rc)::value;
         if constexpr (r < RD_A) {
             constexpr int i = r / FragA::READS, h = r % FragA::READS;
-            FragA::template read<h>(af[SLOT][i], stage + a_fr0 + FragA::step(i, KS, h));
+            FragA::template read<h>(af[SLOT % A_SLOTS][i], stage + a_fr0 + FragA::step(i, KS, h));
         } else {
             constexpr int q = r - RD_A, j = q / FragB::READS, h = q % FragB::READS;
             FragB::template read<h>(bf[SLOT][j], stage + b_fr0 + FragB::step(j, KS, h));
@@ -305,11 +348,41 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
         constexpr int NR = DO_READ ? RD_A + RD_B : 0;
         static_for<0, NMFMA>([&](auto qc) {
             constexpr int q = decltype(qc)::value, i = q / TNI, j = q % TNI;
-            acc[i][j] = mfma16_ops<T>::mma(af[MSLOT][i], bf[MSLOT][j], acc[i][j]);
-            static_for<(NR * q) / NMFMA, (NR * (q + 1)) / NMFMA>([&](auto rc) {
-                read_item(rd_stage, rksc, std::integral_constant<int, MSLOT ^ 1>{}, rc);
-            });
-            if constexpr (NMFMA >= 4) {
+            acc[i][j] = mfma16_ops<T>::mma(af[MSLOT % A_SLOTS][i], bf[MSLOT][j], acc[i][j]);
+            if constexpr (A_SLOTS == 2) {
+                static_for<(NR * q) / NMFMA, (NR * (q + 1)) / NMFMA>([&](auto rc) {
+                    read_item(rd_stage, rksc, std::integral_constant<int, MSLOT ^ 1>{}, rc);
+                });
+            } else {
+                // 16 x 16 x 32: an MFMA lasts 16 cycles, about what one LDS or buffer instruction takes to issue, so a
+                // micro-step carries at most one of them (two at a row's end).  Row i of MFMAs (j = 0 .. 7): B reads at
+                // j = 0, 2; LDS stores of pieces 2i, 2i+1 at j = 1, 3; the loads that refill those registers at
+                // j = 4, 5; A tile i's read for the next k-step after the row's last MFMA, j = 7.
+                static_assert(TNI == 8 && TMI == 8, "the 16 x 16 x 32 schedule is written for 8 x 8 tiles per wave");
+                constexpr int BPR = RD_B / TMI;                       // B reads per row: 1 or 2
+                constexpr int PPR = (NP + TMI - 1) / TMI;             // pieces per row (all of the slab's traffic sits in one k-step): 2
+                static_assert(BPR <= 2 && PPR <= 2, "row schedule");
+                if constexpr (DO_READ) {
+                    if constexpr (j == 0) read_item(rd_stage, rksc, std::integral_constant<int, MSLOT ^ 1>{}, std::integral_constant<int, RD_A + i * BPR>{});
+                    if constexpr (j == 2 && BPR == 2) read_item(rd_stage, rksc, std::integral_constant<int, MSLOT ^ 1>{}, std::integral_constant<int, RD_A + i * BPR + 1>{});
+                    if constexpr (j == TNI - 1) {
+                        static_for<i * FragA::READS, (i + 1) * FragA::READS>([&](auto rc) {
+                            read_item(rd_stage, rksc, std::integral_constant<int, MSLOT ^ 1>{}, rc);
+                        });
+                    }
+                }
+                if constexpr (j == 1 || j == 3) {
+                    constexpr int p = P0 + i * PPR + (j == 3 ? 1 : 0);
+                    if constexpr (WR && (j == 1 || PPR == 2) && p < P0 + NP) store_piece(wr_stage, std::integral_constant<int, p>{});
+                }
+                if constexpr (j == 4 || j == 5) {
+                    constexpr int p = P0 + i * PPR + (j == 5 ? 1 : 0);
+                    if constexpr (LD && (j == 4 || PPR == 2) && p < P0 + NP) load_piece(std::integral_constant<int, p>{});
+                }
+            }
+            if constexpr (A_SLOTS == 1) {
+                // (slab traffic placed above)
+            } else if constexpr (NMFMA >= 4) {
                 // a piece's LDS store and the global load that refills its register go to neighbouring micro-steps,
                 // so no MFMA has both (and a fragment read) to wait behind
                 constexpr int D = NMFMA - 1;
@@ -347,9 +420,14 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
         const uint16_t* stage = smem + cur * STAGE;
         uint16_t* other = smem + (cur ^ 1) * STAGE;
         if constexpr (decltype(next2_tag)::value) point_at_slab((s + 2) * M16_BK);
-        kstep(I0{}, I1{}, std::true_type{}, C0{}, C1{}, next_tag, next2_tag, stage, other);
-        kstep(I1{}, I2{}, std::true_type{}, C1{}, C2{}, next_tag, next2_tag, stage, other);
-        kstep(I0{}, I3{}, std::true_type{}, C2{}, C3{}, next_tag, next2_tag, stage, other);
+        if constexpr (NKS == 4) {
+            kstep(I0{}, I1{}, std::true_type{}, C0{}, C1{}, next_tag, next2_tag, stage, other);
+            kstep(I1{}, I2{}, std::true_type{}, C1{}, C2{}, next_tag, next2_tag, stage, other);
+            kstep(I0{}, I3{}, std::true_type{}, C2{}, C3{}, next_tag, next2_tag, stage, other);
+        } else {
+            // two k-steps of 32: the first carries all of the slab traffic (it is as long as two of the others)
+            kstep(I0{}, I1{}, std::true_type{}, C0{}, C3{}, next_tag, next2_tag, stage, other);
+        }
         if constexpr (NEXT) __syncthreads();
         kstep(I1{}, I0{}, next_tag, C0{}, C0{}, std::false_type{}, std::false_type{}, other, other);
         a_slab += a_step;
@@ -364,6 +442,7 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     if (s + 1 < nslabs) { slab_step(s, yes{}, no{}); s++; }
     slab_step(s, no{}, no{});
 
+    if constexpr (MT == 16) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");      // the in-place MFMAs above are opaque to the compiler: let the last ones drain before their results are read
     // ---- epilogue ----
     T* C = (T*)g.C + (long long)z * g.c_bs;
     const T* bias = (const T*)g.bias;
@@ -379,15 +458,16 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
         __syncthreads();                                 // every wave is done with the main loop's LDS
 #pragma unroll
         for (int j = 0; j < TNI; j++) {
-            const int col = j * 32 + (lane & 31), gnl = n0 + wn0 + col;
+            const int col = j * MT + (lane % MT), gnl = n0 + wn0 + col;
             const bool by_row = g.bias_by_row != 0;
             const float bcol = (has_bias && !by_row && (!EDGE || gnl < g.n)) ? widen(bias[gnl]) : 0.f;
             auto stage = [&](auto with_bias, auto row_bias) {
 #pragma unroll
                 for (int i = 0; i < TMI; i++)
 #pragma unroll
-                    for (int v = 0; v < 16; v++) {
-                        const int row = i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                    for (int v = 0; v < NV; v++) {
+                        // accumulator register v: 32 x 32 tiles hold rows 8 * (v / 4) + 4 * (lane / 32) + v % 4, 16 x 16 tiles rows 4 * (lane / 16) + v
+                        const int row = MT == 32 ? i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4) : i * 16 + 4 * (lane >> 4) + v;
                         T y = narrow<T>(acc[i][j][v]);
                         if constexpr (decltype(row_bias)::value) {
                             const int gmr = m0 + wm0 + row;
