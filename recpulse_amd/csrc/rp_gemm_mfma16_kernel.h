@@ -456,16 +456,17 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
         uint16_t* region = smem + wave * (WM * EP);
         const bool c_vec = (g.c_cs == 1) && (g.c_rs % 8 == 0) && (((uintptr_t)C & 15) == 0);
         __syncthreads();                                 // every wave is done with the main loop's LDS
-#pragma unroll
-        for (int j = 0; j < TNI; j++) {
+        // (compile-time tile indices: a loop that the compiler declines to unroll would index the accumulators at run
+        // time and move all of them to scratch memory for the whole kernel)
+        static_for<0, TNI>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
             const int col = j * MT + (lane % MT), gnl = n0 + wn0 + col;
             const bool by_row = g.bias_by_row != 0;
             const float bcol = (has_bias && !by_row && (!EDGE || gnl < g.n)) ? widen(bias[gnl]) : 0.f;
             auto stage = [&](auto with_bias, auto row_bias) {
-#pragma unroll
-                for (int i = 0; i < TMI; i++)
-#pragma unroll
-                    for (int v = 0; v < NV; v++) {
+                static_for<0, TMI * NV>([&](auto ivc) {
+                    {
+                        constexpr int i = decltype(ivc)::value / NV, v = decltype(ivc)::value % NV;
                         // accumulator register v: 32 x 32 tiles hold rows 8 * (v / 4) + 4 * (lane / 32) + v % 4, 16 x 16 tiles rows 4 * (lane / 16) + v
                         const int row = MT == 32 ? i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4) : i * 16 + 4 * (lane >> 4) + v;
                         T y = narrow<T>(acc[i][j][v]);
@@ -477,11 +478,12 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
                         }
                         region[row * EP + col] = y.bits;
                     }
+                });
             };
             if (has_bias && by_row) stage(std::true_type{}, std::true_type{});
             else if (has_bias) stage(std::true_type{}, std::false_type{});
             else stage(std::false_type{}, std::false_type{});
-        }
+        });
         __syncthreads();
         const int ecol = (lane % LPR) * 8, erow = lane / LPR;
         const int gn = n0 + wn0 + ecol;
