@@ -24,6 +24,10 @@ namespace rp {
 // have a full slab of MFMA time to land, and the single barrier per slab sits
 // where only one MFMA group is left to issue.  Every MFMA is followed by its
 // share of DS / VMEM work and a scheduling barrier, which pins the interleaving.
+// The 256 x 256 tile multiplies with 16x16x32 MFMAs instead (m16_mfma_tile): two
+// k-steps of 32 per slab, 8 x 8 tiles per wave, the slab traffic all in the first
+// k-step, one DS / VMEM instruction per MFMA, A fragments in a single slot that is
+// refilled row by row.
 //
 // LDS layouts (16-bit elements):
 //   KC operand: [rows][64 + 8]   row pitch 144 B -> the 16 rows a quarter-wave
