@@ -337,8 +337,36 @@ struct PadGeom {
     long long P;                  // elements per padded plane (Hp * Wp plus the slack the last tap may read)
 };
 
+// Weights [C_out, C_in, taps] reordered for the segmented GEMM.  Forward: [C_out][tap][C_in].  Backward to the input:
+// [C_in][tap][C_out] with the taps reversed (the gradient is a correlation with the kernel turned by 180 degrees).
+// The job rides on the launch that pads the planes (its last `blocks` workgroups): the GEMM that needs both comes next
+// anyway, and a launch of its own costs more than the 70 KB it moves.
+struct WeightJob {
+    void* out;
+    const void* w;
+    int C_out, C_in, taps, for_input_grad, blocks;       // blocks == 0: no job
+};
+
+template <typename T>
+__device__ __forceinline__ void weights_by_tap(const WeightJob& j, int block, int nblocks) {
+    T* out = (T*)j.out;
+    const T* w = (const T*)j.w;
+    const int total = j.C_out * j.C_in * j.taps;
+    for (int i = block * 256 + threadIdx.x; i < total; i += nblocks * 256) {
+        if (!j.for_input_grad) {
+            const int ci = i % j.C_in, tap = (i / j.C_in) % j.taps, co = i / (j.C_in * j.taps);
+            out[i] = w[((size_t)co * j.C_in + ci) * j.taps + tap];
+        } else {
+            const int co = i % j.C_out, tap = (i / j.C_out) % j.taps, ci = i / (j.C_out * j.taps);
+            out[i] = w[((size_t)co * j.C_in + ci) * j.taps + (j.taps - 1 - tap)];
+        }
+    }
+}
+
 template <typename T, int VEC, bool ALIGNED_ROWS>
-__global__ void __launch_bounds__(256) pad_planes_kernel(T* out, const T* in, PadGeom g, unsigned total_vec) {
+__global__ void __launch_bounds__(256) pad_planes_kernel(T* out, const T* in, PadGeom g, unsigned total_vec, WeightJob job) {
+    const unsigned pad_blocks = gridDim.x - job.blocks;
+    if (blockIdx.x >= pad_blocks) { weights_by_tap<T>(job, blockIdx.x - pad_blocks, job.blocks); return; }
     const unsigned vec_per_plane = (unsigned)(g.P / VEC);
     const unsigned gid = blockIdx.x * 256u + threadIdx.x;
     if (gid >= total_vec) return;
@@ -375,11 +403,16 @@ __global__ void __launch_bounds__(256) pad_planes_kernel(T* out, const T* in, Pa
 }
 
 template <typename T>
-static void launch_pad(T* out, const T* in, const PadGeom& pg, unsigned vecs) {
+static void launch_pad(T* out, const T* in, const PadGeom& pg, unsigned vecs, WeightJob job = WeightJob{nullptr, nullptr, 0, 0, 0, 0, 0}) {
     constexpr int VEC = 16 / (int)sizeof(T);
-    const dim3 grid((vecs + 255) / 256);
-    if (pg.W % VEC == 0 && ((uintptr_t)in & 15) == 0) hipLaunchKernelGGL((pad_planes_kernel<T, VEC, true>), grid, dim3(256), 0, current_stream(), out, in, pg, vecs);
-    else hipLaunchKernelGGL((pad_planes_kernel<T, VEC, false>), grid, dim3(256), 0, current_stream(), out, in, pg, vecs);
+    const dim3 grid((vecs + 255) / 256 + job.blocks);
+    if (pg.W % VEC == 0 && ((uintptr_t)in & 15) == 0) hipLaunchKernelGGL((pad_planes_kernel<T, VEC, true>), grid, dim3(256), 0, current_stream(), out, in, pg, vecs, job);
+    else hipLaunchKernelGGL((pad_planes_kernel<T, VEC, false>), grid, dim3(256), 0, current_stream(), out, in, pg, vecs, job);
+}
+
+static WeightJob weight_job(void* out, const void* w, int C_out, int C_in, int taps, bool for_input_grad) {
+    const int total = C_out * C_in * taps;
+    return WeightJob{out, w, C_out, C_in, taps, for_input_grad ? 1 : 0, (total + 255) / 256 > 64 ? 64 : (total + 255) / 256};
 }
 
 // y[plane][h][w] = yp[plane][h * Wp + w] (+ bias[channel], one rounding add as channel_bias_add_kernel does)
@@ -404,22 +437,6 @@ __global__ void __launch_bounds__(256) unpad_planes_kernel(T* y, const T* yp, co
         for (int e = 0; e < VEC; e++) v[e] = narrow<T>(widen(v[e]) + b);
     }
     memcpy(y + (size_t)gid * VEC, v, VEC * sizeof(T));
-}
-
-// Weights [C_out, C_in, taps] reordered for the segmented GEMM.  Forward: [C_out][tap][C_in].  Backward to the input:
-// [C_in][tap][C_out] with the taps reversed (the gradient is a correlation with the kernel turned by 180 degrees).
-template <typename T>
-__global__ void conv_weights_by_tap_kernel(T* out, const T* w, int C_out, int C_in, int taps, int for_input_grad) {
-    const int total = C_out * C_in * taps;
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
-        if (!for_input_grad) {
-            const int ci = i % C_in, tap = (i / C_in) % taps, co = i / (C_in * taps);
-            out[i] = w[((size_t)co * C_in + ci) * taps + tap];
-        } else {
-            const int co = i % C_out, tap = (i / C_out) % taps, ci = i / (C_out * taps);
-            out[i] = w[((size_t)co * C_in + ci) * taps + (taps - 1 - tap)];
-        }
-    }
 }
 
 static PadGeom pad_geom(int H, int W, int kH, int kW, int vec);
@@ -472,11 +489,11 @@ static int taps_gemm(T* out, void* product, const void* wt, const void* padded, 
     return 0;
 }
 
-// out[batch, C_to, H, W] = sum over taps and C_from of wt . padded(in[batch, C_from, H, W]); wt as conv_weights_by_tap_kernel
+// out[batch, C_to, H, W] = sum over taps and C_from of wt . padded(in[batch, C_from, H, W]); wt as weights_by_tap
 // leaves it ([C_to][tap][C_from]).  bias may be null.  The batch goes in chunks that keep the workspace under same_conv_workspace().
 template <typename T>
 static int same_conv_run(void* out, const void* in, const void* wt, const void* bias, int batch, int C_from, int C_to,
-                         int H, int W, int kH, int kW, int dtype) {
+                         int H, int W, int kH, int kW, int dtype, WeightJob job) {
     constexpr int VEC = 16 / (int)sizeof(T);
     const PadGeom pg = pad_geom(H, W, kH, kW, VEC);
     const long long cols = (long long)H * pg.Wp;
@@ -498,7 +515,8 @@ static int same_conv_run(void* out, const void* in, const void* wt, const void* 
         const T* in0 = (const T*)in + (size_t)b0 * C_from * H * W;
         T* out0 = (T*)out + (size_t)b0 * C_to * H * W;
         const unsigned pad_vecs = (unsigned)((long long)nb * C_from * (pg.P / VEC));
-        launch_pad<T>((T*)padded, in0, pg, pad_vecs);
+        launch_pad<T>((T*)padded, in0, pg, pad_vecs, job);          // the first chunk's launch reorders the weights too
+        job.blocks = 0;
         rc = taps_gemm<T>(out0, product, wt, padded, bias, nb, C_from, C_to, pg, kH, kW, dtype);
     }
     if (rc == 0 && !check_launch("padded-plane convolution kernels")) rc = -1;
@@ -515,21 +533,36 @@ static int same_conv(void* out, const void* in, const void* w, const void* bias,
     if (rp_hip_malloc(&wt, (size_t)total * sizeof(T)) != 0) return -1;
     // w is [C_out, C_in, taps]: forward reduces over C_in (C_from = C_in, C_to = C_out), the input gradient over C_out
     const int C_out = for_input_grad ? C_from : C_to, C_in = for_input_grad ? C_to : C_from;
-    hipLaunchKernelGGL(conv_weights_by_tap_kernel<T>, dim3((total + 255) / 256 > 1024 ? 1024 : (total + 255) / 256), dim3(256), 0, current_stream(),
-                       (T*)wt, (const T*)w, C_out, C_in, taps, for_input_grad ? 1 : 0);
-    const int rc = same_conv_run<T>(out, in, wt, bias, batch, C_from, C_to, H, W, kH, kW, dtype);
+    const int rc = same_conv_run<T>(out, in, wt, bias, batch, C_from, C_to, H, W, kH, kW, dtype, weight_job(wt, w, C_out, C_in, taps, for_input_grad));
     rp_hip_free(wt);
     return rc;
 }
 
-// dw[co][ci][tap] = by_tap[co][tap][ci]: the weight gradient back in the weights' own order
+// dw[co][ci][tap] (+)= sum over the nb samples of per_sample[n][co][tap][ci]: the per-sample products added top to bottom in
+// the accumulate type and rounded once (what rp_hip_reduce_rows does), written back in the weights' own order.
+// accumulate: a later chunk of the batch adds to what the earlier ones left, with a rounding of its own.
 template <typename T>
-__global__ void conv_weights_from_tap_kernel(T* dw, const T* by_tap, int C_out, int C_in, int taps) {
+__global__ void conv_dw_from_samples_kernel(T* dw, const T* per_sample, int nb, int C_out, int C_in, int taps, int accumulate) {
+    using A = typename traits<T>::acc;
     const int total = C_out * C_in * taps;
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
-        const int tap = i % taps, ci = (i / taps) % C_in, co = i / (taps * C_in);
-        dw[i] = by_tap[((size_t)co * taps + tap) * C_in + ci];
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;             // index in [co][tap][ci] order: neighbouring threads read neighbouring elements
+    if (i >= total) return;
+    const int ci = i % C_in, tap = (i / C_in) % taps, co = i / (C_in * taps);
+    A s = 0;
+    int n = 0;
+    constexpr int U = 16;                                            // independent loads in flight; the adds stay in sample order
+    for (; n + U <= nb; n += U) {
+        A v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) v[u] = widen(per_sample[(size_t)(n + u) * total + i]);
+#pragma unroll
+        for (int u = 0; u < U; u++) s += v[u];
     }
+    for (; n < nb; n++) s += widen(per_sample[(size_t)n * total + i]);
+    T r = narrow<T>(s);
+    T* dst = dw + ((size_t)co * C_in + ci) * taps + tap;
+    if (accumulate) r = narrow<T>(widen(*dst) + widen(r));
+    *dst = r;
 }
 
 static PadGeom pad_geom(int H, int W, int kH, int kW, int vec) {
@@ -562,18 +595,18 @@ static int same_conv_backward(void* dx, void* dw, const void* dy, const void* x,
         set_error("conv2d backward: one sample is too large for the padded-plane path");
         return -1;
     }
-    void *dy_pad = nullptr, *x_pad = nullptr, *product = nullptr, *wt = nullptr, *dw_by_tap = nullptr;
+    void *dy_pad = nullptr, *x_pad = nullptr, *product = nullptr, *wt = nullptr;
     bool ok = rp_hip_malloc(&dy_pad, (size_t)(chunk * C_out * pg.P) * sizeof(T)) == 0 &&
               rp_hip_malloc(&product, (size_t)(chunk * product_n) * sizeof(T)) == 0 &&
               (!dx || rp_hip_malloc(&wt, (size_t)w_n * sizeof(T)) == 0) &&
-              (!dw || (rp_hip_malloc(&x_pad, (size_t)(chunk * C_in * pg.P) * sizeof(T)) == 0 && rp_hip_malloc(&dw_by_tap, (size_t)w_n * sizeof(T)) == 0));
-    const unsigned w_grid = (unsigned)((w_n + 255) / 256 > 1024 ? 1024 : (w_n + 255) / 256);
-    if (ok && dx) hipLaunchKernelGGL(conv_weights_by_tap_kernel<T>, dim3(w_grid), dim3(256), 0, current_stream(), (T*)wt, (const T*)w, C_out, C_in, taps, 1);
+              (!dw || rp_hip_malloc(&x_pad, (size_t)(chunk * C_in * pg.P) * sizeof(T)) == 0);
+    WeightJob job = dx ? weight_job(wt, w, C_out, C_in, taps, true) : WeightJob{nullptr, nullptr, 0, 0, 0, 0, 0};
     for (int b0 = 0; ok && b0 < batch; b0 += (int)chunk) {
         const int nb = batch - b0 < chunk ? batch - b0 : (int)chunk;
         const T* dy0 = (const T*)dy + (size_t)b0 * C_out * H * W;
         const unsigned dy_vecs = (unsigned)((long long)nb * C_out * (pg.P / VEC));
-        launch_pad<T>((T*)dy_pad, dy0, pg, dy_vecs);
+        launch_pad<T>((T*)dy_pad, dy0, pg, dy_vecs, job);          // the first chunk's launch reorders the weights for dx too
+        job.blocks = 0;
         if (dx) {
             T* dx0 = (T*)dx + (size_t)b0 * C_in * H * W;
             ok = taps_gemm<T>(dx0, product, wt, dy_pad, nullptr, nb, C_out, C_in, pg, kH, kW, dtype) == 0;
@@ -592,12 +625,13 @@ static int same_conv_backward(void* dx, void* dw, const void* dy, const void* x,
             g.b_bs = (long long)C_in * pg.P; g.b_rs = 1; g.b_cs = pg.P;
             g.c_bs = w_n; g.c_rs = (long long)taps * C_in; g.c_cs = 1;
             g.seg_n = C_in; g.seg_w = kW; g.seg_sh = pg.Wp; g.seg_sw = 1; g.b_extent = (long long)C_in * pg.P;
-            ok = launch_gemm_segmented_b(g, dtype) == 0 && rp_hip_reduce_rows(dw_by_tap, product, nb, (int)w_n, b0 > 0 ? 1 : 0, dtype) == 0;
+            ok = launch_gemm_segmented_b(g, dtype) == 0;
+            if (ok) hipLaunchKernelGGL(conv_dw_from_samples_kernel<T>, dim3((unsigned)((w_n + 255) / 256)), dim3(256), 0, current_stream(),
+                                       (T*)dw, (const T*)product, nb, C_out, C_in, taps, b0 > 0 ? 1 : 0);
         }
     }
-    if (ok && dw) hipLaunchKernelGGL(conv_weights_from_tap_kernel<T>, dim3(w_grid), dim3(256), 0, current_stream(), (T*)dw, (const T*)dw_by_tap, C_out, C_in, taps);
     if (ok && !check_launch("padded-plane convolution kernels")) ok = false;
-    for (void* p : {dy_pad, x_pad, product, wt, dw_by_tap})
+    for (void* p : {dy_pad, x_pad, product, wt})
         if (p) rp_hip_free(p);
     return ok ? 0 : -1;
 }
