@@ -264,6 +264,24 @@ def test_large_tile_kernel_multi_slab():
         assert oracle.rel_err(oracle.to_f64(got[rows], dt), oracle.to_f64(want, dt)) <= tol(dt, k)
 
 
+def test_large_tile_kernel_with_ragged_edges():
+    """The 256 x 256 tile (16 x 16 x 32 MFMAs) on extents that are whole vectors but not whole tiles or slabs: rows and
+    columns past the edge, a last slab of 8, every layout, bias and accumulation.  Float64 everywhere, the oracle on
+    sampled rows (first and last of tiles, the ragged last tile)."""
+    rng = np.random.default_rng(43)
+    m, k, n = 2856, 264, 3080
+    for dt, layout, epilogue in [(BF16, "nn", True), (F16, "nt", False), (BF16, "tn", False), (F16, "tt", True)]:
+        a, b = _operands(rng, m, k, n, dt, layout)
+        es = a.itemsize
+        assert capi.gemm_kernel_name(1, m, k, n, (a.strides[0] // es, a.strides[1] // es), (b.strides[0] // es, b.strides[1] // es), (n, 1), dt) == "mfma16_256x256"
+        bias = rand_storage(rng, (n,), dt) if epilogue else None
+        c0 = rand_storage(rng, (m, n), dt) if epilogue else None
+        got = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=epilogue)
+        assert oracle.rel_err(oracle.to_f64(got, dt), f64_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=epilogue)) <= tol(dt, k)
+        rows = np.array([0, 15, 16, 255, 256, 2559, 2560, 2815, 2816, 2855])
+        _check(got[rows], np.ascontiguousarray(a[rows]), b, dt, k, bias=bias, c_init=None if c0 is None else np.ascontiguousarray(c0[rows]), accumulate=epilogue)
+
+
 def test_wide_tiles_for_outputs_of_at_most_64_rows():
     """Up to 64 rows and many columns: 64 x 128 tiles while k is short, 64 x 256 beyond (one row of waves, no MFMA
     spent on rows past m).  Full tiles and ragged ones, every layout, bias and accumulation; checked against float64
