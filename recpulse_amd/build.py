@@ -21,8 +21,20 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-u
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
-def _compile(src, extra):
+def _fresh(obj, src):
+    """True when obj is newer than its source and every header under csrc/ and include/."""
+    if not os.path.exists(obj):
+        return False
+    t = os.path.getmtime(obj)
+    deps = [os.path.join(CSRC, src)] + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
+    deps.append(os.path.join(HERE, "..", "include", "rp_hip.h"))
+    return all(os.path.getmtime(d) < t for d in deps)
+
+
+def _compile(src, extra, force=True):
     obj = os.path.join(BUILD_DIR, src.replace(".hip", ".o"))
+    if not force and not extra and _fresh(obj, src):
+        return obj
     cmd = [HIPCC] + FLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
@@ -34,12 +46,13 @@ def _compile(src, extra):
     return obj
 
 
-def build(extra_flags=(), verbose=True):
+def build(extra_flags=(), verbose=True, force=True):
+    """Compile and link.  force=False recompiles only the translation units older than their sources (development loop)."""
     os.makedirs(LIB_DIR, exist_ok=True)
     os.makedirs(BUILD_DIR, exist_ok=True)
     extra = list(extra_flags)
     with ThreadPoolExecutor(max_workers=8) as ex:
-        objs = list(ex.map(lambda s: _compile(s, extra), SOURCES))
+        objs = list(ex.map(lambda s: _compile(s, extra, force), SOURCES))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
@@ -76,5 +89,7 @@ def build_host(verbose=True):
 
 
 if __name__ == "__main__":
-    build(sys.argv[1:])
+    args = sys.argv[1:]
+    incremental = "--incremental" in args
+    build([a for a in args if a != "--incremental"], force=not incremental)
     build_host()

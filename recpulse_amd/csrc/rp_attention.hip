@@ -662,7 +662,7 @@ extern "C" int rp_hip_attention_backward(void* dQ, void* dK, void* dV, const voi
                       (float*)dots + (long long)b0 * sq, nb, sq, sk, q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs, do_bs, do_rs, (float)scale};
         rc = f32 ? launch_attention_bwd_f32(g, d) : dtype == RP_DTYPE_BFLOAT16 ? launch_attention_bwd_t<bf16_t>(g, d) : launch_attention_bwd_t<f16_t>(g, d);
     }
-    rp_hip_free(dots);        // stream-ordered reuse: the pool hands it out again only to later work on this stream
+    rp_hip_free(dots);        // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
     return rc;
 }
 

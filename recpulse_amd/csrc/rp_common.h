@@ -14,6 +14,7 @@ void set_error(const char* fmt, ...);
 hipStream_t current_stream();
 bool check_hip(hipError_t e, const char* what);          // false (and error text) on failure
 bool check_launch(const char* what);                     // hipGetLastError after a launch
+bool stream_is_capturing();                              // the calling thread's stream is recording a graph
 
 inline size_t dtype_size(int dtype) {                    // reference core/half_precision.h:10-18
     switch (dtype) {

@@ -111,9 +111,10 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g, float* pa
 // k range; they combine through LDS in a fixed tree.  The grid's second axis
 // splits k further: split partials go to a workspace and a small second kernel
 // adds them in split order (so the result does not depend on scheduling) and
-// runs the epilogue.  (A single-kernel "last block reduces" scheme needs
-// device-scope fences, which write back and invalidate the whole per-XCD L2
-// and cost far more than the second launch.)
+// runs the epilogue.  (For these few-microsecond launches the second kernel
+// is cheaper than the three device-scope round trips of a single-launch
+// "last block reduces" finish; the long streaming kernel of the 16-bit
+// few-row path uses that finish, see splitk_arrival_counters.)
 // ============================================================================
 constexpr int SK_THREADS = 512, SK_WAVES = SK_THREADS / 64;
 
@@ -279,9 +280,14 @@ int* splitk_arrival_counters(long long tiles, size_t partial_bytes, bool* failed
     if (dev < 0 || dev >= MAX_DEVICES) return nullptr;
     std::lock_guard<std::mutex> lock(mu);
     if (blocks[dev]) return blocks[dev];
+    // First use on this device.  The counters must read zero for every stream that will ever use them, so they are
+    // created outside any recording and cleared with a blocking fill; a first use that happens while a graph is being
+    // recorded takes the two-launch path instead (the next eager call creates the block).
+    if (stream_is_capturing()) return nullptr;
     void* p = nullptr;
-    if (rp_hip_malloc(&p, SPLITK_MAX_TILES * sizeof(int)) != 0) { *failed = true; return nullptr; }
-    if (rp_hip_memset(p, 0, SPLITK_MAX_TILES * sizeof(int)) != 0) { rp_hip_free(p); *failed = true; return nullptr; }      // a fill kernel on the current stream
+    if (!check_hip(hipMalloc(&p, SPLITK_MAX_TILES * sizeof(int)), "hipMalloc (split-k counters)")) { *failed = true; return nullptr; }
+    if (!check_hip(hipMemset(p, 0, SPLITK_MAX_TILES * sizeof(int)), "hipMemset (split-k counters)") ||
+        !check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize (split-k counters)")) { (void)hipFree(p); *failed = true; return nullptr; }
     blocks[dev] = (int*)p;
     return blocks[dev];
 }
@@ -351,7 +357,7 @@ static int launch_generic_t(const GemmArgs& g) {
             hipLaunchKernelGGL((gemm_generic_kernel<T, true>), grid, dim3(256), 0, current_stream(), g, (float*)ws, k_per_split);
             int rc = check_launch("gemm_generic_kernel") ? 0 : -1;
             if (rc == 0) rc = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, traits<T>::code);
-            rp_hip_free(ws);      // stream-ordered reuse: the pool hands it out again only to later work on this stream
+            rp_hip_free(ws);      // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
             return rc;
         }
     }
@@ -399,7 +405,7 @@ static int launch_skinny_t(const GemmArgs& g) {
     }
     bool ok = check_hip(attr, "hipFuncSetAttribute") && check_launch("gemm_skinny_kernel");
     if (ok && nsplit > 1) ok = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, traits<T>::code) == 0;
-    if (ws) rp_hip_free(ws);      // stream-ordered reuse: the pool hands it out again only to later work on this stream
+    if (ws) rp_hip_free(ws);      // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
     return ok ? 0 : -1;
 }
 

@@ -238,7 +238,7 @@ static int launch_stream16(const GemmArgs& g, int dtype) {
     if (dtype == RP_DTYPE_BFLOAT16) rc = launch_stream16_t<bf16_t>(g, (float*)ws, nsplit, k_per_split, arrivals);
     else rc = launch_stream16_t<f16_t>(g, (float*)ws, nsplit, k_per_split, arrivals);
     if (rc == 0 && nsplit > 1 && !arrivals) rc = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, dtype);
-    if (ws) rp_hip_free(ws);          // stream-ordered reuse: the pool hands it out again only to later work on this stream
+    if (ws) rp_hip_free(ws);          // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
     return rc;
 }
 
@@ -276,7 +276,7 @@ int launch_mfma16_skinny(const GemmArgs& g, const Plan& p, int dtype) {
     if (dtype == RP_DTYPE_BFLOAT16) rc = launch_skinny16_t<bf16_t>(g, p, (float*)ws, nsplit, k_per_split);
     else rc = launch_skinny16_t<f16_t>(g, p, (float*)ws, nsplit, k_per_split);
     if (rc == 0) rc = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, dtype);
-    rp_hip_free(ws);          // stream-ordered reuse: the pool hands it out again only to later work on this stream
+    rp_hip_free(ws);          // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
     return rc;
 }
 

@@ -39,7 +39,11 @@ bool check_launch(const char* what) { return check_hip(hipGetLastError(), what);
 // (core/tensor_device.cu:44-46) and frees it when the tensor dies; hipMalloc /
 // hipFree cost tens of microseconds and hipFree synchronises the device, which
 // would dominate the small-GEMM configs.  Freed blocks are therefore kept per
-// device in size-keyed lists and reused.
+// device in size-keyed lists and reused.  The lists are shared by every thread
+// and stream of the process: a block freed while kernels that use it are still
+// queued may be handed to the very next rp_hip_malloc of its size, which is safe
+// for work issued afterwards on the same stream only.  Callers that run several
+// streams at once wait for a block's last user before freeing it.
 struct Pool {
     std::mutex mu;
     std::unordered_map<void*, std::pair<int, size_t>> live;       // ptr -> (device, rounded size)
@@ -49,6 +53,37 @@ struct Pool {
 };
 
 static Pool& pool() { static Pool* p = new Pool(); return *p; }   // leaked on purpose: outlives HIP teardown
+
+// Blocks and graph capture.  A kernel recorded into a graph keeps the addresses it was recorded with, so a block
+// that is freed while the calling thread records (a split-k workspace, an intermediate tensor) must not be handed
+// to anyone else for as long as the graph can be replayed: every replay writes there.  While a capture that this
+// library began is active, freed blocks therefore go to a list of the capture (later allocations of the same
+// capture may take them again, which is the stream-ordered reuse the recording itself has); at the capture's end
+// the list is tied to the executable graph, and rp_hip_graph_destroy gives the blocks back to the pool.
+// rp_hip_empty_cache only sees the pool's own lists, so it never releases such a block.
+struct HeldBlock { void* ptr; int dev; size_t size; };
+struct CaptureState { bool active = false; std::vector<HeldBlock> freed; };
+static thread_local CaptureState g_capture;
+static std::mutex g_graph_mu;
+static std::unordered_map<void*, std::vector<HeldBlock>>& graph_blocks() { static auto* m = new std::unordered_map<void*, std::vector<HeldBlock>>(); return *m; }
+
+static void release_to_pool(const std::vector<HeldBlock>& blocks) {
+    Pool& p = pool();
+    for (const HeldBlock& b : blocks) {
+        if (p.enabled) { std::lock_guard<std::mutex> lk(p.mu); p.free_lists[{b.dev, b.size}].push_back(b.ptr); }
+        else (void)hipFree(b.ptr);
+    }
+}
+
+// true when the calling thread's stream is recording a graph that was not begun through this library
+static bool foreign_capture() {
+    if (!g_stream || g_capture.active) return false;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(g_stream, &st) != hipSuccess) { (void)hipGetLastError(); return false; }
+    return st != hipStreamCaptureStatusNone;
+}
+
+bool stream_is_capturing() { return g_capture.active || foreign_capture(); }
 
 static size_t round_size(size_t bytes) {
     if (bytes == 0) bytes = 1;
@@ -109,6 +144,17 @@ int rp_hip_malloc(void** ptr, size_t bytes) {
     if (!check_hip(hipGetDevice(&dev), "hipGetDevice")) return -1;
     Pool& p = pool();
     size_t sz = round_size(bytes);
+    if (g_capture.active) {                          // a block this recording has already let go of
+        for (size_t i = g_capture.freed.size(); i-- > 0;) {
+            const HeldBlock b = g_capture.freed[i];
+            if (b.dev != dev || b.size != sz) continue;
+            g_capture.freed.erase(g_capture.freed.begin() + (long)i);
+            std::lock_guard<std::mutex> lk(p.mu);
+            p.live[b.ptr] = {dev, sz};
+            *ptr = b.ptr;
+            return 0;
+        }
+    }
     if (p.enabled) {
         std::lock_guard<std::mutex> lk(p.mu);
         auto it = p.free_lists.find({dev, sz});
@@ -144,6 +190,13 @@ int rp_hip_free(void* ptr) {
         if (it == p.live.end()) { set_error("rp_hip_free: pointer %p was not allocated by rp_hip_malloc", ptr); return -1; }
         auto key = it->second;
         p.live.erase(it);
+        if (g_capture.active) { g_capture.freed.push_back({ptr, key.first, key.second}); return 0; }    // stays with the graph being recorded
+        if (foreign_capture()) {
+            // recorded by a graph this library knows nothing about: the block is never handed out again
+            std::lock_guard<std::mutex> gl(g_graph_mu);
+            graph_blocks()[nullptr].push_back({ptr, key.first, key.second});
+            return 0;
+        }
         if (p.enabled) { p.free_lists[key].push_back(ptr); return 0; }
     }
     return check_hip(hipFree(ptr), "hipFree") ? 0 : -1;
@@ -240,17 +293,25 @@ int rp_hip_stream_synchronize(void) {
 // not memset nodes), so a recorded sequence replays exactly; host-blocking copies must stay outside.
 int rp_hip_graph_capture_begin(void) {
     if (!g_stream) { set_error("rp_hip_graph_capture_begin: set a created stream first (the null stream cannot be captured)"); return -1; }
-    return check_hip(hipStreamBeginCapture(g_stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture") ? 0 : -1;
+    if (g_capture.active) { set_error("rp_hip_graph_capture_begin: this thread is already recording"); return -1; }
+    if (!check_hip(hipStreamBeginCapture(g_stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture")) return -1;
+    g_capture.active = true;
+    g_capture.freed.clear();
+    return 0;
 }
 
 int rp_hip_graph_capture_end(void** graph_exec) {
     if (!graph_exec) { set_error("rp_hip_graph_capture_end: null argument"); return -1; }
     hipGraph_t graph = nullptr;
-    if (!check_hip(hipStreamEndCapture(g_stream, &graph), "hipStreamEndCapture")) return -1;
+    std::vector<HeldBlock> held;
+    held.swap(g_capture.freed);
+    g_capture.active = false;
+    if (!check_hip(hipStreamEndCapture(g_stream, &graph), "hipStreamEndCapture")) { release_to_pool(held); return -1; }
     hipGraphExec_t exec = nullptr;
     bool ok = check_hip(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate");
     (void)hipGraphDestroy(graph);
-    if (!ok) return -1;
+    if (!ok) { release_to_pool(held); return -1; }       // nothing can replay the recording
+    if (!held.empty()) { std::lock_guard<std::mutex> gl(g_graph_mu); graph_blocks()[(void*)exec] = std::move(held); }
     *graph_exec = (void*)exec;
     return 0;
 }
@@ -260,7 +321,16 @@ int rp_hip_graph_launch(void* graph_exec) {
 }
 
 int rp_hip_graph_destroy(void* graph_exec) {
-    return check_hip(hipGraphExecDestroy((hipGraphExec_t)graph_exec), "hipGraphExecDestroy") ? 0 : -1;
+    if (!graph_exec) return 0;
+    const bool ok = check_hip(hipGraphExecDestroy((hipGraphExec_t)graph_exec), "hipGraphExecDestroy");
+    std::vector<HeldBlock> held;
+    {
+        std::lock_guard<std::mutex> gl(g_graph_mu);
+        auto it = graph_blocks().find(graph_exec);
+        if (it != graph_blocks().end()) { held = std::move(it->second); graph_blocks().erase(it); }
+    }
+    release_to_pool(held);          // the caller has waited for the last replay, as before any free
+    return ok ? 0 : -1;
 }
 
 int rp_hip_event_create(void** event) {

@@ -172,7 +172,7 @@ PYBIND11_MODULE(recpulse_cuda, m) {
             return self;
         }, py::arg("flag") = true)
         .def("backward", [](PyTensor& s) {
-            if (tensor_backward(s.t) != 0) throw std::runtime_error(std::string("backward failed: ") + rp_last_error());
+            if (tensor_backward(s.t) != 0) throw std::runtime_error(std::string("backward operation failed: ") + rp_last_error());
         })
         .def("zero_grad", [](PyTensor& s) { tensor_zero_grad(s.t); })
         // ---- autograd ops ----
@@ -294,6 +294,7 @@ PYBIND11_MODULE(recpulse_cuda, m) {
         auto s = to_shape(shape);
         return wrap(rp_rand(parse_dtype(dtype), parse_device(device), (int)s.size(), s.data()), "rand");
     }, py::arg("shape"), py::arg("dtype") = "float32", py::arg("device") = "cpu");
+    m.def("_fail_gemm_after", [](int n) { rp_debug_fail_gemm_after(n); }, py::arg("n"));      // fault injection for tests of the error paths
     m.def("manual_seed", [](unsigned long long seed) { rp_manual_seed(seed); });
     m.def("device_count", []() { int n = 0; for (int i = 0; i < 64 && validate_device_id(i); i++) n = i + 1; return n; });
 }

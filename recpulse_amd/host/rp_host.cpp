@@ -21,12 +21,18 @@
 namespace {
 
 thread_local char g_err[512] = "";
+// While tensor_backward runs, the first failure of any backward function is kept here: backward functions return
+// nothing, so this is how the driver learns that a gradient is missing (reference convention: tensor_backward
+// returns -1 and the binding raises, python/tensor_python.c:400-414).
+thread_local bool g_in_backward = false;
+thread_local char g_backward_err[512] = "";
 
 void fail(const char* fmt, ...) {
     va_list ap;
     va_start(ap, fmt);
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
+    if (g_in_backward && !g_backward_err[0]) snprintf(g_backward_err, sizeof(g_backward_err), "%s", g_err[0] ? g_err : "unknown failure");
 }
 
 // a device call failed: keep the device layer's own text
@@ -205,7 +211,7 @@ Tensor* dense(Tensor* x) { return rp_is_contiguous(x) ? tensor_retain(x) : rp_co
 // Accumulate rule of every backward function (reference ops/ops.c:6781-6788): the first gradient is stored,
 // later ones are added in place.  `g` is consumed.
 void accumulate_grad(Tensor* x, Tensor* g) {
-    if (!g) return;
+    if (!g) { if (g_in_backward && !g_backward_err[0]) fail("a gradient could not be computed"); return; }
     Meta* m = ensure_meta(x);
     if (!m->grad) { m->grad = g; return; }
     if (m->grad->device_id >= 0) {
@@ -231,6 +237,11 @@ size_t dtype_size(DType dtype) {
 }
 
 const char* rp_last_error(void) { return g_err; }
+
+// Fault injection for tests of the error paths: the n-th GEMM issued by the host layer from now on (n = 1 is the next
+// one) fails before anything is launched; n <= 0 switches it off.  Nothing else reads this counter.
+static thread_local int g_fail_gemm_in = 0;
+void rp_debug_fail_gemm_after(int n) { g_fail_gemm_in = n > 0 ? n : 0; }
 
 // ======================================================================== core
 bool validate_device_id(int device_id) {              // reference core/tensor.c:10-16
@@ -424,16 +435,21 @@ int tensor_backward(Tensor* root) {
             stack.pop_back();
         }
     }
+    g_in_backward = true;
+    g_backward_err[0] = 0;
     for (auto it = order.rbegin(); it != order.rend(); ++it) {
         Tensor* t = *it;
         GradFn* gf = t->metadata->grad_fn;
         if (gf && t->metadata->grad) gf->backward(gf, t->metadata->grad);
     }
+    g_in_backward = false;
     for (Tensor* t : order) {
         GradFn* gf = t->metadata->grad_fn;
         t->metadata->grad_fn = nullptr;
         free_grad_fn(gf);                                   // may drop the last reference to intermediates; `order` is not touched again
     }
+    // the walk always finishes (the graph is freed either way); the first failure of a backward function decides the result
+    if (g_backward_err[0]) { fail("%s", g_backward_err); return -1; }
     return 0;
 }
 
@@ -611,19 +627,35 @@ int device_gemm(Tensor* c, Tensor* a, bool a_t, Tensor* b, bool b_t, Tensor* bia
     if (ba == 1) a_bs = 0;
     if (bb == 1) b_bs = 0;
     if (!on_device(c->device_id)) return dev_fail("set device");
+    if (g_fail_gemm_in > 0 && --g_fail_gemm_in == 0) { fail("matmul: failure injected by rp_debug_fail_gemm_after"); return -1; }
     int rc = rp_hip_gemm_strided_batched(c->data, a->data, b->data, bias ? bias->data : nullptr, batch, m, k, n,
                                          a_bs, a_rs, a_cs, b_bs, b_rs, b_cs, c_bs, c->strides[cn - 2], c->strides[cn - 1], accumulate, c->dtype);
     return rc == 0 ? 0 : dev_fail("matmul");
 }
 
-// gradient of a GEMM operand: writes into a fresh tensor, or straight into the existing gradient (beta = 1)
+// An operand as the strided GEMM entry can read it: itself when its leading dims collapse into one batch stride,
+// a dense copy otherwise (the forward's rule in op_matmul).  The result is owned by the caller.
+Tensor* gemm_operand(Tensor* x) {
+    int bt; long long bs;
+    return batch_layout(x, &bt, &bs) ? tensor_retain(x) : rp_contiguous(x);
+}
+
+// gradient of a GEMM operand: writes into a fresh tensor, or straight into the existing gradient (beta = 1).
+// A failure is recorded (fail / dev_fail) and surfaces from tensor_backward.
 void gemm_grad(Tensor* target, Tensor* a, bool a_t, Tensor* b, bool b_t) {
     Meta* m = ensure_meta(target);
-    if (m->grad && rp_is_contiguous(m->grad)) { device_gemm(m->grad, a, a_t, b, b_t, nullptr, 1); return; }
-    Tensor* g = empty_tensor(target->dtype, target->device_id, target->ndim, target->shape);
-    if (!g) return;
-    if (device_gemm(g, a, a_t, b, b_t, nullptr, 0) != 0) { free_tensor(g); return; }
-    accumulate_grad(target, g);
+    Tensor* aa = gemm_operand(a);
+    Tensor* bb = gemm_operand(b);
+    if (!aa || !bb) { fail("matmul backward: an operand could not be made dense"); free_tensor(aa); free_tensor(bb); return; }
+    if (m->grad && rp_is_contiguous(m->grad)) {
+        device_gemm(m->grad, aa, a_t, bb, b_t, nullptr, 1);
+    } else {
+        Tensor* g = empty_tensor(target->dtype, target->device_id, target->ndim, target->shape);
+        if (!g) fail("matmul backward: gradient allocation failed");
+        else if (device_gemm(g, aa, a_t, bb, b_t, nullptr, 0) != 0) free_tensor(g);
+        else accumulate_grad(target, g);
+    }
+    free_tensor(aa); free_tensor(bb);
 }
 
 // dA = dC · Bᵀ and dB = Aᵀ · dC (reference ops/ops.c:6759-6814), with the transposes passed as stride views
@@ -639,10 +671,12 @@ void backward_matmul_fn(GradFn* self, Tensor* grad_output) {
         else {
             // shared 2-D weight under a batched activation: fold the batch into the rows, dB = A2dᵀ · dC2d
             Tensor* a2 = dense(a); Tensor* g2 = dense(grad_output);
+            if (!a2 || !g2) { fail("matmul backward: an operand could not be made dense"); free_tensor(a2); free_tensor(g2); return; }
             int sa[2] = {(int)(a2->size / a2->shape[a2->ndim - 1]), a2->shape[a2->ndim - 1]};
             int sg[2] = {(int)(g2->size / g2->shape[g2->ndim - 1]), g2->shape[g2->ndim - 1]};
             Tensor* av = rp_reshape(a2, 2, sa); Tensor* gv = rp_reshape(g2, 2, sg);
             if (av && gv) gemm_grad(b, av, true, gv, false);
+            else fail("matmul backward: operands could not be folded to two dimensions");
             free_tensor(av); free_tensor(gv); free_tensor(a2); free_tensor(g2);
         }
     }
@@ -743,8 +777,8 @@ void backward_relu_fn(GradFn* self, Tensor* grad_output) {           // referenc
     if (!needs_grad(x)) return;
     Tensor* xd = dense(x); Tensor* gd = dense(grad_output);
     Tensor* g = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
-    if (g && on_device(x->device_id) && backwards_relu_device(gd->data, xd->data, g->data, x->size, x->dtype) == 0) accumulate_grad(x, g);
-    else free_tensor(g);
+    if (g && xd && gd && on_device(x->device_id) && backwards_relu_device(gd->data, xd->data, g->data, x->size, x->dtype) == 0) accumulate_grad(x, g);
+    else { dev_fail("relu backward"); free_tensor(g); }
     free_tensor(xd); free_tensor(gd);
 }
 
@@ -766,8 +800,8 @@ void backward_softmax_fn(GradFn* self, Tensor* grad_output) {        // referenc
     split_dims(y, dim, &outer, &d, &inner);
     Tensor* gd = dense(grad_output);
     Tensor* g = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
-    if (g && on_device(x->device_id) && backwards_softmax_device(gd->data, y->data, g->data, outer, d, inner, x->dtype) == 0) accumulate_grad(x, g);
-    else free_tensor(g);
+    if (g && gd && on_device(x->device_id) && backwards_softmax_device(gd->data, y->data, g->data, outer, d, inner, x->dtype) == 0) accumulate_grad(x, g);
+    else { dev_fail("softmax backward"); free_tensor(g); }
     free_tensor(gd);
 }
 
@@ -780,8 +814,8 @@ void backward_mul_scalar_fn(GradFn* self, Tensor* grad_output) {     // referenc
     float sf = (float)s;
     Tensor* gd = dense(grad_output);
     Tensor* g = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
-    if (g && rp_mul_scalar(g->data, gd->data, x->dtype == DTYPE_FLOAT64 ? (const void*)&s : (const void*)&sf, x->size, x->dtype, x->device_id) == 0) accumulate_grad(x, g);
-    else free_tensor(g);
+    if (g && gd && rp_mul_scalar(g->data, gd->data, x->dtype == DTYPE_FLOAT64 ? (const void*)&s : (const void*)&sf, x->size, x->dtype, x->device_id) == 0) accumulate_grad(x, g);
+    else { fail("mul_scalar backward failed: %s", rp_hip_last_error()); free_tensor(g); }
     free_tensor(gd);
 }
 
@@ -1028,7 +1062,7 @@ void backward_reduce_all_fn(GradFn* self, Tensor* grad_output) {     // sum_all 
         if (!ok) dev_fail("fill scaled");
     } else if (ok) ok = tensor_read_scalar(grad_output, &g0) == 0 && fill_value_tensor(g0 * scale, g);
     if (ok) accumulate_grad(x, g);
-    else free_tensor(g);
+    else { if (!g_backward_err[0]) fail("sum_all / mean_all backward failed"); free_tensor(g); }
 }
 
 struct CESaved { int batch, classes; void* targets_dev; int device_id; };
@@ -1046,7 +1080,7 @@ void backward_cross_entropy_fn(GradFn* self, Tensor* grad_output) {
     CESaved* s = (CESaved*)self->saved_data;
     double up = 1.0;
     const bool beside = scalar_beside(grad_output, x);
-    if (!beside && tensor_read_scalar(grad_output, &up) != 0) return;
+    if (!beside && tensor_read_scalar(grad_output, &up) != 0) { fail("cross-entropy backward: upstream gradient could not be read"); return; }
     Tensor* xd = dense(x);
     Tensor* g = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
     int rc = -1;
@@ -1054,7 +1088,7 @@ void backward_cross_entropy_fn(GradFn* self, Tensor* grad_output) {
         rc = beside ? rp_hip_cross_entropy_backward(g->data, xd->data, (const int*)s->targets_dev, s->batch, s->classes, grad_output->data, x->dtype)
                     : rp_hip_cross_entropy_mean(nullptr, g->data, xd->data, (const int*)s->targets_dev, s->batch, s->classes, up, x->dtype);
     if (rc == 0) accumulate_grad(x, g);
-    else free_tensor(g);
+    else { dev_fail("cross-entropy backward"); free_tensor(g); }
     free_tensor(xd);
 }
 

@@ -66,6 +66,7 @@ struct GradFn {                                     /* reference ops/ops.h:14-20
 
 size_t dtype_size(DType dtype);
 const char* rp_last_error(void);
+void rp_debug_fail_gemm_after(int n);      /* tests of the error paths: the n-th GEMM from now on fails; n <= 0 switches it off */
 
 /* ---- core ---- */
 bool validate_device_id(int device_id);

@@ -319,3 +319,58 @@ def test_training_halves_the_loss_and_is_deterministic():
     assert losses == losses2
     for p, q in zip(params, params2):
         assert np.array_equal(p, q)
+
+
+# ---- the usual head split x.reshape(B, S, H, D).permute(0, 2, 1, 3): its leading dims do not collapse into one batch
+# stride, so forward AND backward take a dense copy of that operand; both gradients must exist and match the oracle
+@pytest.mark.parametrize("dtype,tol", [("float64", 1e-12), ("float32", 1e-5 * 8), ("bfloat16", 2e-2)])
+def test_batched_matmul_backward_on_head_split_views(dtype, tol):
+    rng = np.random.default_rng(57)
+    B, S, H, D = 2, 48, 3, 32
+    code = {"float64": oracle.F64, "float32": oracle.F32, "bfloat16": oracle.BF16}[dtype]
+    xq, xk = (oracle.to_f64(oracle.to_storage(rng.normal(0, 1, (B, S, H * D)), code), code) for _ in range(2))
+    dq = dev(xq, dtype, grad=True); dk = dev(xk, dtype, grad=True)
+    q = dq.reshape([B, S, H, D]).permute([0, 2, 1, 3])                # strides (S*H*D, D, H*D, 1)
+    kT = dk.reshape([B, S, H, D]).permute([0, 2, 3, 1])               # K^T per head, a view as well
+    assert not q.is_contiguous and not kT.is_contiguous
+    s = q.op_matmul(kT)
+    assert s.shape == (B, H, S, S)
+    s.backward()                                                       # upstream of ones
+    # oracle: per (b, h) slice, the reference's CPU matmul and its backward GEMMs on dense copies
+    q4 = xq.reshape(B, S, H, D).transpose(0, 2, 1, 3); k4 = xk.reshape(B, S, H, D).transpose(0, 2, 1, 3)
+    want_s = np.zeros((B, H, S, S)); want_dq = np.zeros((B, H, S, D)); want_dkT = np.zeros((B, H, D, S))
+    ones = oracle.to_storage(np.ones((S, S)), code)
+    for b in range(B):
+        for h in range(H):
+            a_ = oracle.to_storage(q4[b, h], code); b_ = oracle.to_storage(np.ascontiguousarray(k4[b, h].T), code)
+            want_s[b, h] = oracle.to_f64(oracle.matmul(a_, b_, code), code)
+            da, db = oracle.matmul_backward(a_, b_, ones, code)
+            want_dq[b, h] = oracle.to_f64(da, code); want_dkT[b, h] = oracle.to_f64(db, code)
+    assert oracle.rel_err(host(s), want_s) <= tol
+    assert dq.has_grad and dk.has_grad
+    got_dq = host(dq.grad).reshape(B, S, H, D).transpose(0, 2, 1, 3)
+    got_dkT = host(dk.grad).reshape(B, S, H, D).transpose(0, 2, 3, 1)
+    assert oracle.rel_err(got_dq, want_dq) <= tol
+    assert oracle.rel_err(got_dkT, want_dkT) <= tol
+
+
+# ---- a GEMM that fails inside backward() must surface (reference python/tensor_python.c:400-414 raises
+# "backward operation failed"); the failure is forced from the host, nothing faulty reaches the device
+def test_failure_inside_backward_raises_and_leaves_no_stale_grad():
+    a = dev(np.arange(6.0).reshape(2, 3), "float32", grad=True)
+    b = dev(np.arange(12.0).reshape(3, 4), "float32", grad=True)
+    s = a.op_matmul(b).op_sum_all()
+    rp._fail_gemm_after(1)                      # the next GEMM the host layer issues is dA = dC . B^T
+    try:
+        with pytest.raises(RuntimeError, match="backward"):
+            s.backward()
+    finally:
+        rp._fail_gemm_after(0)
+    assert not a.has_grad                        # the failed gradient is absent, not stale
+    assert b.has_grad                            # the walk went on: dB = A^T . dC was computed
+    b.zero_grad()
+    # the graph was freed all the same and the tensors stay usable
+    s2 = a.op_matmul(b).op_sum_all()
+    s2.backward()
+    assert np.array_equal(host(a.grad), np.tile(np.arange(12.0).reshape(3, 4).sum(1), (2, 1)))
+    assert np.array_equal(host(b.grad), np.tile(np.arange(6.0).reshape(2, 3).sum(0)[:, None], (1, 4)))

@@ -251,6 +251,39 @@ def test_graph_replay_matches_eager():
                 assert np.array_equal(g_, w_)
 
 
+def test_workspace_recorded_into_a_graph_is_not_handed_out_while_the_graph_lives():
+    """A split-k GEMM recorded into a graph keeps writing its partial sums to the workspace it was recorded with.
+    Until the graph is destroyed that block must not be given to anyone else: buffers allocated after the recording,
+    of every size the workspace could have, keep their contents across replays."""
+    rng = np.random.default_rng(52)
+    w = rand_storage(rng, (1, 2048), BF16); x = rand_storage(rng, (2048, 1024), BF16)
+    dw, dxx, dz = Dev(w, BF16), Dev(x, BF16), Dev.empty((1, 1024), BF16)
+
+    def skinny():
+        capi.gemm(dz.ptr, dw.ptr, dxx.ptr, None, 1, 1, 2048, 1024, (0, 2048, 1), (0, 1024, 1), (0, 1024, 1), False, BF16)
+
+    skinny()                                        # eager once: the workspace block now sits in the pool
+    capi.synchronize()
+    want = dz.numpy().copy()
+    stream = capi.Stream()
+    with stream:
+        with capi.Graph.capture() as graph:
+            skinny()
+        # whatever size the workspace had (nsplit x 1 x 1024 floats, rounded to 512 bytes), one of these would get its block
+        guards = [capi.DeviceBuffer(nsplit * 1024 * 4) for nsplit in range(1, 33)]
+        for gbuf in guards:
+            capi.check(L().rp_hip_memset(gbuf.ptr, 0x5A, gbuf.nbytes), "memset")
+        for _ in range(3):
+            capi.check(L().rp_hip_fill(dz.ptr, -1.0, 1024, BF16), "fill")
+            graph.launch()
+            capi.check(L().rp_hip_stream_synchronize(), "sync")
+            assert np.array_equal(dz.numpy(), want)
+            for gbuf in guards:
+                assert np.all(gbuf.to_numpy(np.uint8, (gbuf.nbytes,)) == 0x5A)
+        for gbuf in guards:
+            gbuf.free()
+
+
 def test_narrowing_to_fp16_every_exponent_and_rounding_case():
     """fp32 -> fp16 on the device against the oracle, bit for bit: every sign and exponent with mantissas that sit
     on, just below and just above every rounding boundary (ties, carries into the next binade, the subnormal range,
