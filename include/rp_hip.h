@@ -116,6 +116,22 @@ int rp_hip_gemm_strided_batched(void* C, const void* A, const void* B, const voi
                                 long long c_bs, long long c_rs, long long c_cs,
                                 int accumulate, int dtype);
 
+/* The same product from a caller that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Arguments, results and errors are those
+ * of rp_hip_gemm_strided_batched, bit for bit; the difference is that the split-k kernels take their partial sums and
+ * arrival counters from a fixed device array of RP_HIP_NOALLOC_WORKSPACE_BYTES (+ 4 KiB) that every GPU the library
+ * runs on holds until the process ends, and that no hipMalloc, hipFree or pool call is made.  A shape whose split-k
+ * workspace would exceed the array returns -1 with a message that names both sizes.  All calls on one GPU share that
+ * GPU's array: calls that overlap in time on one GPU (different streams or threads) race on it and must be serialised
+ * by the caller.  The first call on a device resolves the array's address and should be made outside a recording. */
+#define RP_HIP_NOALLOC_WORKSPACE_BYTES 16777216 /* 16 MiB */
+int rp_hip_gemm_strided_batched_noalloc(void* C, const void* A, const void* B, const void* bias,
+                                        int batch, int m, int k, int n,
+                                        long long a_bs, long long a_rs, long long a_cs,
+                                        long long b_bs, long long b_rs, long long b_cs,
+                                        long long c_bs, long long c_rs, long long c_cs,
+                                        int accumulate, int dtype);
+
 /* Name of the kernel family the dispatcher picks for a problem, for logs and
  * tests ("mfma16_256x256", "skinny", "generic", ...).  No device work. */
 const char* rp_hip_gemm_kernel_name(int batch, int m, int k, int n,

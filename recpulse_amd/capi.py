@@ -50,6 +50,7 @@ SIGNATURES = {
     "rp_hip_event_destroy": (_i, [_vp]),
     "matmul_kernel_device": (_i, [_vp, _vp, _vp, _i, _i, _i, _i]),
     "rp_hip_gemm_strided_batched": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i] + [_ll] * 9 + [_i, _i]),
+    "rp_hip_gemm_strided_batched_noalloc": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i] + [_ll] * 9 + [_i, _i]),
     "rp_hip_gemm_kernel_name": (ctypes.c_char_p, [_i, _i, _i, _i] + [_ll] * 6 + [_i]),
     "add_kernel_device": (_i, [_vp, _vp, _vp, _sz, _i]),
     "add_strided_kernel_device": (_i, [_vp, _vp, _vp, _i, _ip, _ip, _ip, _sz, _i]),

@@ -135,6 +135,13 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t splitk_rsrc(const float* parti
 // streams of one device must be serialised by the caller.
 int* splitk_arrival_counters(long long tiles, size_t partial_bytes, bool* failed);
 
+// Workspace of a GEMM launcher (split-k partial sums): a pool block, or, inside the entry point that allocates
+// nothing, a piece of that entry point's fixed device array (then -1 with an error when it is too small).
+int gemm_workspace(void** ws, size_t bytes);
+void gemm_workspace_release(void* ws);
+// Inside the entry point that allocates nothing: its arrival counters (already zero); nullptr elsewhere.
+int* noalloc_arrival_counters();
+
 // per-family launchers (dtype is one of the RP_DTYPE_* codes the family supports)
 int launch_generic(const GemmArgs& g, int dtype);
 int launch_skinny(const GemmArgs& g, int dtype);

@@ -20,6 +20,8 @@
 //   generic  any strides, any shape; LDS-tiled scalar FMA.
 #include "rp_gemm.h"
 
+#include <mutex>
+
 namespace rp {
 
 // ============================================================================
@@ -182,6 +184,64 @@ int launch_gemm_segmented_b(const GemmArgs& g, int dtype) {
     return launch_mfmaw(g, p, dtype);
 }
 
+// ============================================================================
+// The entry point that allocates nothing (rp_hip_gemm_strided_batched_noalloc).
+// Its split-k launchers take their workspace and arrival counters from one fixed
+// device array instead of the pool.  Every GPU the library runs on holds its own
+// copy of the array at its own address for the life of the process; host code
+// never uses the array's name as an address, only the pointer that
+// hipGetSymbolAddress returned for the device that was current.
+// ============================================================================
+constexpr size_t NOALLOC_COUNTER_BYTES = (size_t)SPLITK_MAX_TILES * sizeof(int);      // arrival counters, then the partial sums
+constexpr size_t NOALLOC_WORKSPACE_BYTES = (size_t)RP_HIP_NOALLOC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_COUNTER_BYTES + NOALLOC_WORKSPACE_BYTES];
+
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static std::mutex g_scratch_mu;
+static unsigned char* g_scratch_ptr[NOALLOC_MAX_DEVICES] = {};      // per device: where that device's copy of `scratch` lives
+static thread_local unsigned char* g_noalloc_base = nullptr;        // non-null while the calling thread is inside the entry point
+static thread_local bool g_noalloc_busy = false;                    // its workspace is handed out (one launcher at a time)
+
+// Address of the current device's copy of the array, resolved once per device.
+static unsigned char* noalloc_scratch_of_current_device() {
+    int dev = 0;
+    if (!check_hip(hipGetDevice(&dev), "hipGetDevice")) return nullptr;
+    if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) { set_error("rp_hip_gemm_strided_batched_noalloc: device ordinal %d is beyond the %d this entry point tracks", dev, NOALLOC_MAX_DEVICES); return nullptr; }
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (!check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return nullptr;
+        g_scratch_ptr[dev] = (unsigned char*)p;
+    }
+    return g_scratch_ptr[dev];
+}
+
+int gemm_workspace(void** ws, size_t bytes) {
+    if (!g_noalloc_base) return rp_hip_malloc(ws, bytes);
+    *ws = nullptr;
+    if (bytes > NOALLOC_WORKSPACE_BYTES) {
+        set_error("rp_hip_gemm_strided_batched_noalloc: this shape needs %zu bytes of split-k workspace, the fixed array holds %zu", bytes, NOALLOC_WORKSPACE_BYTES);
+        return -1;
+    }
+    if (g_noalloc_busy) { set_error("rp_hip_gemm_strided_batched_noalloc: workspace requested twice"); return -1; }
+    g_noalloc_busy = true;
+    *ws = g_noalloc_base + NOALLOC_COUNTER_BYTES;
+    return 0;
+}
+
+void gemm_workspace_release(void* ws) {
+    if (!ws) return;
+    if (g_noalloc_base && ws == g_noalloc_base + NOALLOC_COUNTER_BYTES) { g_noalloc_busy = false; return; }
+    rp_hip_free(ws);
+}
+
+int* noalloc_arrival_counters() { return (int*)g_noalloc_base; }
+
+__global__ void __launch_bounds__(256) clear_counters_kernel(int* counters, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) counters[i] = 0;
+}
+
 }  // namespace rp
 
 using namespace rp;
@@ -213,6 +273,28 @@ int rp_hip_gemm_strided_batched(void* C, const void* A, const void* B, const voi
         if (run_gemm(g, dtype) != 0) return -1;
     }
     return 0;
+}
+
+int rp_hip_gemm_strided_batched_noalloc(void* C, const void* A, const void* B, const void* bias,
+                                        int batch, int m, int k, int n,
+                                        long long a_bs, long long a_rs, long long a_cs,
+                                        long long b_bs, long long b_rs, long long b_cs,
+                                        long long c_bs, long long c_rs, long long c_cs,
+                                        int accumulate, int dtype) {
+    if (g_noalloc_base) { set_error("rp_hip_gemm_strided_batched_noalloc: re-entered"); return -1; }
+    unsigned char* base = noalloc_scratch_of_current_device();
+    if (!base) return -1;
+    // The array keeps what the last call left.  The partial sums are fully overwritten before they are read; the
+    // arrival counters must read zero, and a launch that was cut short could have left some standing: clear them
+    // with a kernel (stream-ordered before the GEMM; not a memset node, so the call can be recorded into a graph).
+    hipLaunchKernelGGL(clear_counters_kernel, dim3((SPLITK_MAX_TILES + 255) / 256), dim3(256), 0, current_stream(), (int*)base, SPLITK_MAX_TILES);
+    if (!check_launch("clear_counters_kernel")) return -1;
+    g_noalloc_base = base;
+    g_noalloc_busy = false;
+    const int rc = rp_hip_gemm_strided_batched(C, A, B, bias, batch, m, k, n, a_bs, a_rs, a_cs, b_bs, b_rs, b_cs, c_bs, c_rs, c_cs, accumulate, dtype);
+    g_noalloc_base = nullptr;
+    g_noalloc_busy = false;
+    return rc;
 }
 
 int matmul_kernel_device(void* C, const void* A, const void* B, int m, int k, int n, int dtype) {

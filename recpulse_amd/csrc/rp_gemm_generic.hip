@@ -273,6 +273,7 @@ int* splitk_arrival_counters(long long tiles, size_t partial_bytes, bool* failed
     static int* blocks[MAX_DEVICES] = {};
     static int two_launch = -1;
     *failed = false;
+    if (int* fixed = noalloc_arrival_counters()) return (tiles > SPLITK_MAX_TILES || partial_bytes >= (1ull << 31)) ? nullptr : fixed;
     if (two_launch < 0) { const char* e = getenv("RP_HIP_SPLITK_TWO_LAUNCH"); two_launch = (e && e[0] == '1') ? 1 : 0; }
     if (two_launch == 1 || tiles > SPLITK_MAX_TILES || partial_bytes >= (1ull << 31)) return nullptr;
     int dev = 0;
@@ -352,12 +353,12 @@ static int launch_generic_t(const GemmArgs& g) {
         nsplit = (g.k + k_per_split - 1) / k_per_split;
         if (nsplit > 1) {
             void* ws = nullptr;
-            if (rp_hip_malloc(&ws, (size_t)nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
+            if (gemm_workspace(&ws, (size_t)nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
             dim3 grid((g.n + 63) / 64, (g.m + 63) / 64, nsplit);
             hipLaunchKernelGGL((gemm_generic_kernel<T, true>), grid, dim3(256), 0, current_stream(), g, (float*)ws, k_per_split);
             int rc = check_launch("gemm_generic_kernel") ? 0 : -1;
             if (rc == 0) rc = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, traits<T>::code);
-            rp_hip_free(ws);      // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
+            gemm_workspace_release(ws);      // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
             return rc;
         }
     }
@@ -388,7 +389,7 @@ static int launch_skinny_t(const GemmArgs& g) {
     int nsplit = (g.k + k_per_block - 1) / k_per_block;
     if (nsplit > 65535) { set_error("gemm skinny: k too large"); return -1; }
     void* ws = nullptr;
-    if (nsplit > 1 && rp_hip_malloc(&ws, (size_t)nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
+    if (nsplit > 1 && gemm_workspace(&ws, (size_t)nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
     dim3 grid(groups, nsplit);
     auto smem = [&](int mrows) {
         size_t a_slice = (size_t)k_per_block * mrows * 4, combine = (size_t)(SK_WAVES / 2) * mrows * VEC * 64 * 4;
@@ -405,7 +406,7 @@ static int launch_skinny_t(const GemmArgs& g) {
     }
     bool ok = check_hip(attr, "hipFuncSetAttribute") && check_launch("gemm_skinny_kernel");
     if (ok && nsplit > 1) ok = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, traits<T>::code) == 0;
-    if (ws) rp_hip_free(ws);      // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
+    if (ws) gemm_workspace_release(ws);      // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
     return ok ? 0 : -1;
 }
 

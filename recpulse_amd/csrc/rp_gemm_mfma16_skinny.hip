@@ -227,18 +227,18 @@ static int launch_stream16(const GemmArgs& g, int dtype) {
     nsplit = (g.k + k_per_split - 1) / k_per_split;
     const size_t part_bytes = (size_t)nsplit * g.m * g.n * sizeof(float);
     void* ws = nullptr;
-    if (nsplit > 1 && rp_hip_malloc(&ws, part_bytes) != 0) return -1;
+    if (nsplit > 1 && gemm_workspace(&ws, part_bytes) != 0) return -1;
     int* arrivals = nullptr;
     if (nsplit > 1) {
         bool failed = false;
         arrivals = splitk_arrival_counters(groups, part_bytes, &failed);
-        if (failed) { rp_hip_free(ws); return -1; }
+        if (failed) { gemm_workspace_release(ws); return -1; }
     }
     int rc;
     if (dtype == RP_DTYPE_BFLOAT16) rc = launch_stream16_t<bf16_t>(g, (float*)ws, nsplit, k_per_split, arrivals);
     else rc = launch_stream16_t<f16_t>(g, (float*)ws, nsplit, k_per_split, arrivals);
     if (rc == 0 && nsplit > 1 && !arrivals) rc = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, dtype);
-    if (ws) rp_hip_free(ws);          // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
+    if (ws) gemm_workspace_release(ws);          // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
     return rc;
 }
 
@@ -271,12 +271,12 @@ int launch_mfma16_skinny(const GemmArgs& g, const Plan& p, int dtype) {
     int k_per_split = ((g.k + nsplit - 1) / nsplit + M16_BK - 1) / M16_BK * M16_BK;
     nsplit = (g.k + k_per_split - 1) / k_per_split;
     void* ws = nullptr;
-    if (rp_hip_malloc(&ws, (size_t)nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
+    if (gemm_workspace(&ws, (size_t)nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
     int rc;
     if (dtype == RP_DTYPE_BFLOAT16) rc = launch_skinny16_t<bf16_t>(g, p, (float*)ws, nsplit, k_per_split);
     else rc = launch_skinny16_t<f16_t>(g, p, (float*)ws, nsplit, k_per_split);
     if (rc == 0) rc = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, dtype);
-    rp_hip_free(ws);          // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
+    gemm_workspace_release(ws);          // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
     return rc;
 }
 

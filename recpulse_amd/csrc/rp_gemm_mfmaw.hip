@@ -352,11 +352,11 @@ static int launch_mfmaw_t(const GemmArgs& g, const Plan& p) {
         if (nsplit < 2) nsplit = 1;
     }
     void* ws = nullptr;
-    if (nsplit > 1 && rp_hip_malloc(&ws, (size_t)nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
+    if (nsplit > 1 && gemm_workspace(&ws, (size_t)nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
     int rc = (p.bm == 128) ? launch_mfmaw_layout<T, 128, 128>(g, p, (float*)ws, nsplit, k_per_split)
                            : launch_mfmaw_layout<T, 64, 64>(g, p, (float*)ws, nsplit, k_per_split);
     if (rc == 0 && nsplit > 1) rc = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, traits<T>::code);
-    if (ws) rp_hip_free(ws);          // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
+    if (ws) gemm_workspace_release(ws);          // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
     return rc;
 }
 
