@@ -15,6 +15,7 @@ hipStream_t current_stream();
 bool check_hip(hipError_t e, const char* what);          // false (and error text) on failure
 bool check_launch(const char* what);                     // hipGetLastError after a launch
 bool stream_is_capturing();                              // the calling thread's stream is recording a graph
+int device_cu_count();                                   // compute units of the current device (0 when it cannot be read)
 
 inline size_t dtype_size(int dtype) {                    // reference core/half_precision.h:10-18
     switch (dtype) {

@@ -151,7 +151,7 @@ struct FragMap {
 };
 
 template <typename T, int BM, int BN, int WGM, bool A_MC, bool B_MC, bool EDGE, bool SPLITK>
-__global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_m, int tiles_n, float* partials, int k_per_split) {
+__global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_m, int tiles_n, float* partials, int k_per_split, int sched_total) {
     constexpr int WGN = 4 / WGM;
     constexpr int WM = BM / WGM, WN = BN / WGN;       // wave patch
     constexpr int MT = SPLITK ? 32 : m16_mfma_tile(BM, BN);      // MFMA tile edge; k-steps of 16 (MT 32) or 32 (MT 16)
@@ -170,9 +170,15 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     constexpr int NMFMA = TMI * TNI;
     extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
 
-    TileCoord tc = schedule_tile(blockIdx.x, tiles_m, tiles_n);
-    if (!tc.valid) return;
     const int z = blockIdx.y;
+    // A workgroup walks the schedule with the grid's stride.  The launcher starts one workgroup per slot of the schedule,
+    // except for the 256 x 256 tile, which fills a CU by itself: there one workgroup per CU stays resident and takes its
+    // tiles one after the other, so that a tile's output stores drain, and the next tile's first loads fly, while MFMAs
+    // run; a workgroup per tile would hold the CU idle until its last store was acknowledged.  A stride that is a
+    // multiple of 8 keeps a workgroup's tiles on the XCD the schedule assigned them to.
+    for (int tile_id = blockIdx.x; tile_id < sched_total; tile_id += gridDim.x) {
+    TileCoord tc = schedule_tile(tile_id, tiles_m, tiles_n);
+    if (!tc.valid) continue;
     const int m0 = tc.tm * BM, n0 = tc.tn * BN;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
@@ -314,6 +320,7 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     point_at_slab(0);
     static_for<0, NA>([&](auto ic) { load_piece_a(ic); });
     static_for<0, NB>([&](auto ic) { load_piece_b(ic); });
+    if (tile_id != (int)blockIdx.x) __syncthreads();       // the previous tile's epilogue has read its staged rows out of LDS
     static_for<0, NA>([&](auto ic) { store_piece_a(smem, ic); });
     static_for<0, NB>([&](auto ic) { store_piece_b(smem, ic); });
     a_slab += a_step;
@@ -565,17 +572,25 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
             }
         }
     }
+    }   // tiles of this workgroup
 }
 
 // Launch one instantiation.  nsplit > 1 selects the split-k variant: partials must hold nsplit * m * n floats.
 template <typename T, int BM, int BN, int WGM, bool A_MC, bool B_MC, bool EDGE, bool SPLITK>
 static int m16_launch(const GemmArgs& g, float* partials, int nsplit, int k_per_split) {
     int tiles_m = (g.m + BM - 1) / BM, tiles_n = (g.n + BN - 1) / BN;
-    dim3 grid(scheduled_grid(tiles_m, tiles_n), g.batch, SPLITK ? nsplit : 1);
+    const int sched_total = scheduled_grid(tiles_m, tiles_n);
+    int blocks = sched_total;
+    if (BM == 256 && BN == 256 && !SPLITK && g.batch == 1) {
+        // one resident workgroup per CU (rounded down to whole rounds of the 8 XCDs)
+        const int cus = device_cu_count() / 8 * 8;
+        if (cus >= 8 && blocks > cus) blocks = cus;
+    }
+    dim3 grid(blocks, g.batch, SPLITK ? nsplit : 1);
     size_t smem = m16_smem_bytes(BM, BN, WGM, A_MC, B_MC, (!SPLITK && g.k <= M16_BK) ? 1 : 2);
     auto kern = gemm_mfma16_kernel<T, BM, BN, WGM, A_MC, B_MC, EDGE, SPLITK>;
     if (smem > 64 * 1024 && !check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem), "hipFuncSetAttribute")) return -1;
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, current_stream(), g, tiles_m, tiles_n, partials, k_per_split);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, current_stream(), g, tiles_m, tiles_n, partials, k_per_split, sched_total);
     return check_launch("gemm_mfma16_kernel") ? 0 : -1;
 }
 

@@ -2,6 +2,7 @@
 // copies, streams, events and the error text.
 #include "rp_common.h"
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -33,6 +34,21 @@ bool check_hip(hipError_t e, const char* what) {
 }
 
 bool check_launch(const char* what) { return check_hip(hipGetLastError(), what); }
+
+int device_cu_count() {
+    constexpr int MAX_DEVICES = 64;
+    static std::atomic<int> cached[MAX_DEVICES] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) { (void)hipGetLastError(); return 0; }
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) { (void)hipGetLastError(); n = 0; }
+        const char* e = getenv("RP_HIP_CU_COUNT");           // measurement aid: pretend the device has this many CUs
+        if (e && atoi(e) > 0) n = atoi(e);
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
 
 // ---- caching allocator ------------------------------------------------------
 // The reference allocates and zero-fills device memory for every op output
