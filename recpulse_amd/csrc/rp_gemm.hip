@@ -75,8 +75,14 @@ static void choose_tile16(Plan& p, int batch, int m, int k, int n) {
 
 // Decide the kernel family and tile from shapes and strides alone (pointer
 // alignment is checked by the caller, which may still fall back to generic).
+static bool direct32_off() {                       // RP_HIP_NO_DIRECT32=1: short-k fp32 GEMMs keep the LDS-tiled kernel
+    static int v = -1;
+    if (v < 0) { const char* e = getenv("RP_HIP_NO_DIRECT32"); v = (e && e[0] == '1') ? 1 : 0; }
+    return v == 1;
+}
+
 static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long a_cs, long long b_rs, long long b_cs,
-                      long long c_rs, long long c_cs, long long a_bs, long long b_bs, int dtype) {
+                      long long c_rs, long long c_cs, long long a_bs, long long b_bs, int dtype, bool allow_direct = true) {
     Plan p{FAM_GENERIC, 64, 64, false, false, true, "generic"};
     if (force_generic()) return p;
     const int vec = 16 / (int)dtype_size(dtype);                // elements per 16-byte vector
@@ -119,6 +125,16 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
         p.fam = FAM_TINY; p.bm = 16; p.bn = 16; p.name = "tiny32_16x16";
         return p;
     }
+    // fp32 with 32 < k <= 64, both operands with unit stride along their free index and an output of at least 128 tiles of
+    // 128 x 128: no k loop to pipeline, so every wave multiplies a 64 x 64 patch straight out of registers (no LDS, no
+    // barrier).  (With unit stride along k a lane's loads touch 64 cache lines per instruction and the vector cache's
+    // tag lookups take longer than the MFMAs: those layouts keep LDS.)
+    if (dtype == RP_DTYPE_FLOAT32 && allow_direct && !direct32_off() && k > 32 && k <= 64 && a_rs == 1 && a_cs != 1 && b_cs == 1 && b_rs != 1 &&
+        (a_cs != 1 || (k % 4 == 0 && a_rs % 4 == 0 && a_bs % 4 == 0)) && (b_rs != 1 || (k % 4 == 0 && b_cs % 4 == 0 && b_bs % 4 == 0)) &&
+        m >= 64 && n >= 64 && (long long)((m + 127) / 128) * ((n + 127) / 128) * batch >= 128) {
+        p.fam = FAM_DIRECT32; p.bm = 128; p.bn = 128; p.a_mc = a_cs != 1; p.b_mc = b_rs != 1; p.name = "direct32_128x128";
+        return p;
+    }
     if (!mfma_ok) return p;
     p.a_mc = !a_kc;             // when both qualify (extent-1 corner cases) keep the row-major reading
     p.b_mc = b_mc;
@@ -138,6 +154,10 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
 
 static int run_gemm(const GemmArgs& g, int dtype) {
     Plan p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype);
+    if (p.fam == FAM_DIRECT32) {
+        if (direct32_takes(g)) return launch_direct32(g);
+        p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype, false);     // base pointers or spans it cannot address
+    }
     if (p.fam != FAM_GENERIC && p.fam != FAM_TINY && !(aligned16(g.A) && aligned16(g.B))) p.fam = FAM_GENERIC;
     switch (p.fam) {
         case FAM_MFMA16:

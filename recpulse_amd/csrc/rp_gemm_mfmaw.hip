@@ -302,6 +302,150 @@ __global__ void __launch_bounds__(256, 2) gemm_mfmaw_kernel(GemmArgs g, int tile
     }
 }
 
+// ============================================================================
+// Short reductions (k of at most two slabs: 64 for fp32), many tiles.
+// A tile of such a product has no k loop to pipeline: load, wait, multiply for a few microseconds, store.  In the
+// kernel above those phases follow one another inside a workgroup, and the 64 KB a tile writes wait at the end of
+// it for a write path that takes about 8 bytes per clock from a CU: the epilogue costs more than the multiplies
+// (S = Q.K^T of 192 x 512 x 64 x 512: prologue 4.5 K, MFMAs 12.5 K, epilogue 17 K cycles per tile).  Here the
+// workgroups are resident and walk the tiles (of all batch entries): the whole k of the NEXT tile is loaded into
+// registers while this tile is multiplied, and the accumulators are stored straight from registers (register v of a
+// 32 x 32 MFMA tile is 32 adjacent columns of one row across 32 lanes, a full 128-byte line), so the stores of a
+// tile drain while the next one is multiplied and no tile waits for memory at its start or its end.
+// ============================================================================
+template <typename T, int BM, int BN, bool A_MC, bool B_MC, bool EDGE>
+__global__ void __launch_bounds__(256, (BM <= 64 ? 4 : 2)) gemm_mfmaw_shortk_kernel(GemmArgs g, int tiles_m, int tiles_n, long long total) {
+    using cfg = mfmaw_cfg<T>;
+    constexpr int MT = cfg::MT, BK = cfg::BK, NKS = BK / cfg::KS;
+    constexpr int WM = BM / 2, WN = BN / 2, TMI = WM / MT, TNI = WN / MT;
+    constexpr int PA = BM + cfg::PAD, PB = BN + cfg::PAD;
+    constexpr int A_ELEMS = BK * PA, B_ELEMS = BK * PB, STAGE = A_ELEMS + B_ELEMS;
+    using SlabA = MwSlab<T, BM, A_MC, EDGE>;
+    using SlabB = MwSlab<T, BN, B_MC, EDGE>;
+    constexpr int NA = SlabA::NP, NB = SlabB::NP, NP_ALL = NA + NB;
+    extern __shared__ __attribute__((aligned(16))) unsigned char mw_smem_raw[];
+    T* smem = (T*)mw_smem_raw;                 // stage 0: k [0, BK), stage 1: k [BK, 2 BK)
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
+    const long long a_fs = g.a_rs, a_ks = g.a_cs, b_fs = g.b_cs, b_ks = g.b_rs;
+    const int slabs = g.k > BK ? 2 : 1;
+    const int per_matrix = tiles_m * tiles_n;
+    const int lf = lane % MT, lk = lane / MT;
+
+    uint4 regs[2][NP_ALL];
+    auto load_tile = [&](long long id) {
+        const int z = (int)(id / per_matrix), tile = (int)(id % per_matrix);
+        const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN;
+        const T* A = (const T*)g.A + (long long)z * g.a_bs;
+        const T* B = (const T*)g.B + (long long)z * g.b_bs;
+        mw_static_for<0, 2>([&](auto sc) {
+            constexpr int sl = decltype(sc)::value;
+            if (sl < slabs) {
+                mw_static_for<0, NP_ALL>([&](auto pc) {
+                    constexpr int p = decltype(pc)::value;
+                    if constexpr (p < NA) regs[sl][p] = SlabA::load(A, a_fs, a_ks, m0, sl * BK, g.m, g.k, t, p);
+                    else regs[sl][p] = SlabB::load(B, b_fs, b_ks, n0, sl * BK, g.n, g.k, t, p - NA);
+                });
+            }
+        });
+    };
+
+    long long id = blockIdx.x;
+    if (id < total) load_tile(id);
+    for (; id < total; id += gridDim.x) {
+        const int z = (int)(id / per_matrix), tile = (int)(id % per_matrix);
+        const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN;
+        // this tile's operands: registers -> LDS (every wave has finished reading the previous tile: barrier at the loop's end)
+        mw_static_for<0, 2>([&](auto sc) {
+            constexpr int sl = decltype(sc)::value;
+            if (sl < slabs) {
+                mw_static_for<0, NP_ALL>([&](auto pc) {
+                    constexpr int p = decltype(pc)::value;
+                    if constexpr (p < NA) SlabA::store(smem + sl * STAGE, regs[sl][p], t, p);
+                    else SlabB::store(smem + sl * STAGE + A_ELEMS, regs[sl][p], t, p - NA);
+                });
+            }
+        });
+        __syncthreads();
+        if (id + gridDim.x < total) load_tile(id + gridDim.x);       // lands while this tile is multiplied
+
+        typename cfg::acc_t acc[TMI][TNI];
+#pragma unroll
+        for (int i = 0; i < TMI; i++)
+#pragma unroll
+            for (int j = 0; j < TNI; j++)
+#pragma unroll
+                for (int v = 0; v < cfg::NV; v++) acc[i][j][v] = (T)0;
+        T af[2][TMI], bf[2][TNI];
+        auto read_frags = [&](const T* stage, int ks, int slot) {
+            const int kk = ks * cfg::KS + lk;
+#pragma unroll
+            for (int i = 0; i < TMI; i++) af[slot][i] = stage[kk * PA + wm0 + i * MT + lf];
+#pragma unroll
+            for (int j = 0; j < TNI; j++) bf[slot][j] = stage[A_ELEMS + kk * PB + wn0 + j * MT + lf];
+        };
+        read_frags(smem, 0, 0);
+        for (int sl = 0; sl < slabs; sl++) {
+            const T* stage = smem + sl * STAGE;
+            mw_static_for<0, NKS>([&](auto ksc) {
+                constexpr int ks = decltype(ksc)::value, slot = ks & 1;
+                if constexpr (ks + 1 < NKS) read_frags(stage, ks + 1, slot ^ 1);
+                else if (sl + 1 < slabs) read_frags(stage + STAGE, 0, slot ^ 1);
+#pragma unroll
+                for (int i = 0; i < TMI; i++)
+#pragma unroll
+                    for (int j = 0; j < TNI; j++) acc[i][j] = cfg::mma(af[slot][i], bf[slot][j], acc[i][j]);
+            });
+        }
+
+        // epilogue straight from the accumulators: one store instruction is MT adjacent columns of 64 / MT rows
+        T* C = (T*)g.C + (long long)z * g.c_bs;
+        const T* bias = (const T*)g.bias;
+        const bool has_bias = bias != nullptr, accum = g.accumulate != 0;
+#pragma unroll
+        for (int j = 0; j < TNI; j++) {
+            const int gn = n0 + wn0 + j * MT + lf;
+            const bool col_ok = !EDGE || gn < g.n;
+            const T bv = (has_bias && col_ok) ? bias[gn] : (T)0;
+#pragma unroll
+            for (int i = 0; i < TMI; i++)
+#pragma unroll
+                for (int v = 0; v < cfg::NV; v++) {
+                    const int gm = m0 + wm0 + i * MT + cfg::acc_row(v, lane);
+                    if (EDGE && !(col_ok && gm < g.m)) continue;
+                    T* pc = C + (long long)gm * g.c_rs + (long long)gn * g.c_cs;
+                    if (accum) *pc = finish<T>(acc[i][j][v], has_bias, bv, true, *pc);
+                    else *pc = finish<T>(acc[i][j][v], has_bias, bv, false, (T)0);
+                }
+        }
+        __syncthreads();                       // every wave is done with this tile's LDS
+    }
+}
+
+template <typename T, int BM, int BN, bool A_MC, bool B_MC>
+static int mw_launch_shortk(const GemmArgs& g, bool edge) {
+    const int tiles_m = (g.m + BM - 1) / BM, tiles_n = (g.n + BN - 1) / BN;
+    const long long total = (long long)tiles_m * tiles_n * g.batch;
+    constexpr size_t smem = 2 * (size_t)mfmaw_cfg<T>::BK * (BM + BN + 2 * mfmaw_cfg<T>::PAD) * sizeof(T);
+    int cus = device_cu_count();
+    if (cus <= 0) cus = 256;
+    const long long blocks = total < 2ll * cus ? total : 2ll * cus;         // two resident workgroups per CU
+    auto launch = [&](auto kern) {
+        if (smem > 64 * 1024 && !check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem), "hipFuncSetAttribute")) return -1;
+        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), smem, current_stream(), g, tiles_m, tiles_n, total);
+        return check_launch("gemm_mfmaw_shortk_kernel") ? 0 : -1;
+    };
+    if (edge) return launch(gemm_mfmaw_shortk_kernel<T, BM, BN, A_MC, B_MC, true>);
+    return launch(gemm_mfmaw_shortk_kernel<T, BM, BN, A_MC, B_MC, false>);
+}
+
+// fp32, k of at most two slabs, at least 128 tiles of 128 x 128: the resident, cross-tile pipelined kernel
+static bool shortk_off() {                        // RP_HIP_NO_SHORTK=1 keeps the general kernel
+    static int v = -1;
+    if (v < 0) { const char* e = getenv("RP_HIP_NO_SHORTK"); v = (e && e[0] == '1') ? 1 : 0; }
+    return v == 1;
+}
+
 template <typename T, int BM, int BN, bool A_MC, bool B_MC, bool EDGE, bool SPLITK>
 static int mw_launch(const GemmArgs& g, dim3 grid, int tiles_m, int tiles_n, float* partials, int k_per_split) {
     constexpr size_t smem = mw_smem_bytes<T>(BM, BN);
@@ -361,6 +505,13 @@ static int launch_mfmaw_t(const GemmArgs& g, const Plan& p) {
 }
 
 int launch_mfmaw(const GemmArgs& g, const Plan& p, int dtype) {
+    if (dtype == RP_DTYPE_FLOAT32 && p.bm == 128 && g.k <= 2 * mfmaw_cfg<float>::BK && !shortk_off() && g.seg_k == 0 && g.seg_n == 0 && g.c_fold_from == 0 && !g.bias_by_row) {
+        const bool edge = p.edge || g.k != 2 * mfmaw_cfg<float>::BK;
+        if (!p.a_mc && p.b_mc) return mw_launch_shortk<float, 128, 128, false, true>(g, edge);
+        if (!p.a_mc && !p.b_mc) return mw_launch_shortk<float, 128, 128, false, false>(g, edge);
+        if (p.a_mc && p.b_mc) return mw_launch_shortk<float, 128, 128, true, true>(g, edge);
+        return mw_launch_shortk<float, 128, 128, true, false>(g, edge);
+    }
     if (dtype == RP_DTYPE_FLOAT32) return launch_mfmaw_t<float>(g, p);
     if (dtype == RP_DTYPE_FLOAT64) return launch_mfmaw_t<double>(g, p);
     set_error("mfmaw GEMM: unsupported dtype %d", dtype);

@@ -388,3 +388,39 @@ def test_small_fp32_outputs_take_one_launch():
     got_t = device_gemm(a3, np.ascontiguousarray(b3.transpose(0, 2, 1)).transpose(0, 2, 1), F32)
     assert oracle.rel_err(got_t, oracle_gemm(a3, b3, F32)) <= tol(F32, 24)
 
+
+
+# ---- fp32 products with a short reduction (k <= 64) and many tiles: the resident cross-tile kernel (every layout, ragged
+# extents, k below a whole slab, bias, accumulation) and, for operands with unit stride along their free index, the
+# kernel that multiplies straight out of registers
+@pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("batch,m,k,n", [(8, 512, 64, 512), (9, 500, 64, 456), (33, 250, 44, 300), (16, 384, 36, 512), (40, 256, 20, 256)])
+def test_fp32_short_reduction_batched(layout, batch, m, k, n):
+    rng = np.random.default_rng(61)
+    a = rand_storage(rng, (batch, m, k), F32) if layout[0] == "n" else rand_storage(rng, (batch, k, m), F32).transpose(0, 2, 1)
+    b = rand_storage(rng, (batch, k, n), F32) if layout[1] == "n" else rand_storage(rng, (batch, n, k), F32).transpose(0, 2, 1)
+    a_rc, b_rc = [s // 4 for s in a.strides[1:]], [s // 4 for s in b.strides[1:]]
+    kernel = capi.gemm_kernel_name(batch, m, k, n, a_rc, b_rc, (n, 1), F32)
+    if layout == "tn" and k > 32:
+        assert kernel == "direct32_128x128"
+    elif m % 4 == 0 and n % 4 == 0 and k % 4 == 0:
+        assert kernel == "mfma32_128x128"
+    got = device_gemm(a, b, F32)
+    _check(got, a, b, F32, k)
+    bias = rand_storage(rng, (n,), F32)
+    c0 = rand_storage(rng, (batch, m, n), F32)
+    got = device_gemm(a, b, F32, bias=bias, c_init=c0, accumulate=True)
+    _check(got, a, b, F32, k, bias=bias, c_init=c0, accumulate=True)
+
+
+def test_fp32_short_reduction_integers_bit_exact():
+    """Small integers: every partial sum is exact, so the product must equal the oracle's bit for bit in any summation order."""
+    rng = np.random.default_rng(62)
+    batch, m, k, n = 8, 512, 64, 512
+    for layout in LAYOUTS:
+        a = rng.integers(-3, 4, (batch, m, k) if layout[0] == "n" else (batch, k, m)).astype(np.float32)
+        b = rng.integers(-3, 4, (batch, k, n) if layout[1] == "n" else (batch, n, k)).astype(np.float32)
+        a = a if layout[0] == "n" else a.transpose(0, 2, 1)
+        b = b if layout[1] == "n" else b.transpose(0, 2, 1)
+        got = device_gemm(a, b, F32)
+        assert np.array_equal(got, np.matmul(a.astype(np.float64), b.astype(np.float64)).astype(np.float32)), layout
