@@ -374,3 +374,43 @@ def test_failure_inside_backward_raises_and_leaves_no_stale_grad():
     s2.backward()
     assert np.array_equal(host(a.grad), np.tile(np.arange(12.0).reshape(3, 4).sum(1), (2, 1)))
     assert np.array_equal(host(b.grad), np.tile(np.arange(6.0).reshape(2, 3).sum(0)[:, None], (1, 4)))
+
+
+# ---- benchmark configuration 4 at full size through the drop-in tensors: Q, K, V [16, 12, 512, 64], K^T as the 4-D
+# permuted view (reference ops/ops.c:8639-8697: shape and strides permuted, data shared), forward and backward.  The two
+# leading dims collapse into one batch stride inside the host layer; nothing is copied.
+@pytest.mark.parametrize("dtype,tol_gemm,tol_chain", [("bfloat16", 2e-2, 3e-2), ("float32", 1e-5 * np.sqrt(512), 1e-5 * np.sqrt(512))])
+def test_config4_full_size_on_4d_permuted_view(dtype, tol_gemm, tol_chain):
+    import torch
+    rng = np.random.default_rng(3)
+    B, H, S, D = 16, 12, 512, 64
+    code = {"float32": oracle.F32, "bfloat16": oracle.BF16}[dtype]
+    q, k, v = (oracle.to_f64(oracle.to_storage(rng.normal(0, 1, (B, H, S, D)), code), code) for _ in range(3))
+    qt, kt, vt = (dev(a, dtype, grad=True) for a in (q, k, v))
+    kT = kt.permute([0, 1, 3, 2])
+    assert kT.shape == (B, H, D, S) and not kT.is_contiguous
+    s = qt.op_matmul(kT)
+    assert s.shape == (B, H, S, S)
+    # S alone against float64 at one GEMM's tolerance
+    assert oracle.rel_err(host(s), np.matmul(q, k.transpose(0, 1, 3, 2))) <= tol_gemm
+    o = s.op_mul_scalar(0.125).op_softmax(dim=-1).op_matmul(vt)
+    assert o.shape == (B, H, S, D) and o.dtype == dtype
+    o.backward()                                     # upstream of ones (reference core/tensor.c:223-228)
+    for t in (qt, kt, vt):
+        assert t.has_grad and t.grad.shape == (B, H, S, D)
+    # the whole chain against float64 autograd
+    tq, tk, tv = (torch.tensor(x, requires_grad=True) for x in (q, k, v))
+    to = torch.softmax(tq @ tk.transpose(2, 3) * 0.125, -1) @ tv
+    to.sum().backward()
+    assert oracle.rel_err(host(o), to.detach().numpy()) <= tol_chain
+    grads = {"dQ": host(qt.grad), "dK": host(kt.grad), "dV": host(vt.grad)}
+    for name, want in (("dQ", tq.grad), ("dK", tk.grad), ("dV", tv.grad)):
+        assert oracle.rel_err(grads[name], want.numpy()) <= tol_chain, name
+    # and the CPU oracle (the reference's op chain, one rounding per op) on two (batch, head) slices
+    ones = oracle.to_storage(np.ones((S, D)), code)
+    o_host = host(o)
+    for b, h in ((0, 0), (B - 1, H - 1)):
+        want = oracle.attention(oracle.to_storage(q[b, h], code), oracle.to_storage(k[b, h], code), oracle.to_storage(v[b, h], code), code, scale=0.125, d_out=ones)
+        assert oracle.rel_err(o_host[b, h], oracle.to_f64(want["O"], code)) <= tol_gemm, (b, h)
+        for name in ("dQ", "dK", "dV"):
+            assert oracle.rel_err(grads[name][b, h], oracle.to_f64(want[name], code)) <= tol_gemm, (name, b, h)
