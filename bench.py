@@ -174,9 +174,11 @@ def cpu_baseline(a, b, target_s=15.0):
 
 
 def cpu_baseline_configs():
-    """The same CPU path on the smaller configurations, one core, each bounded to a second or two: configuration 1
+    """The same CPU path on the other configurations, one core, each bounded to a second or two: configuration 1
     (fp32 Linear forward), configuration 2 (the nine fp32 GEMMs of the MLP step), configuration 3 at N = 1024 (bf16,
-    a 256-row slab), 5a (bf16, m = 1 against the 8192 x 8192 matrix) and 5b (fp64 2048^2, a 32-row slab).
+    a 256-row slab) and at N = 4096 (bf16 and fp32, an 8-row slab, the whole GEMM extrapolated), configuration 4 as a
+    loop of per-head 2-D products (2 of the 192 heads, extrapolated), 5a (bf16, m = 1 against the 8192 x 8192 matrix)
+    and 5b (fp64 2048^2, a 32-row slab).
     fp32 / fp64 products run in the reference's own matmul_kernel_host_* when oracle/_ref holds it, 16-bit ones
     and everything else in the oracle's restatement."""
     import oracle
@@ -188,7 +190,9 @@ def cpu_baseline_configs():
             return oracle.reference_matmul(ref, a, b, dt)
         return oracle.matmul(a, b, dt)
 
-    def timed(shapes, dt, npdt):
+    def timed(shapes, dt, npdt, whole=1.0):
+        """`whole`: how many times the timed slab fits into the configuration; above 1 the full time is an extrapolation
+        (the loop's cost is linear in the rows of A and in the number of per-head products)."""
         if dt == oracle.BF16:
             ops = [(_normal_bf16(rng, (m, k)), _normal_bf16(rng, (k, n))) for m, k, n in shapes]
         else:
@@ -197,7 +201,10 @@ def cpu_baseline_configs():
         for x, y in ops:
             mm(x, y, dt)
         sec = time.perf_counter() - t0
-        return {"ms": round(sec * 1e3, 2), "GFLOP/s": round(sum(2.0 * m * k * n for m, k, n in shapes) / sec / 1e9, 3)}
+        out = {"ms": round(sec * 1e3, 2), "GFLOP/s": round(sum(2.0 * m * k * n for m, k, n in shapes) / sec / 1e9, 3)}
+        if whole != 1.0:
+            out["extrapolated_whole_config_ms"] = round(sec * 1e3 * whole, 1)
+        return out
 
     mlp = []
     for rows, fan_in, fan_out in ((256, 784, 256), (256, 256, 128), (256, 128, 10)):
@@ -206,6 +213,13 @@ def cpu_baseline_configs():
         "config1_linear_fwd_f32": timed([(128, 784, 256)], oracle.F32, np.float32),
         "config2_mlp_9_gemms_f32": timed(mlp, oracle.F32, np.float32),
         "config3_bf16_1024_rows_0_255": timed([(256, 1024, 1024)], oracle.BF16, np.float32),
+        # N = 4096: 8 of the 4096 rows of one GEMM (forward; dA and dB cost the same)
+        "config3_bf16_4096_rows_0_7": timed([(8, 4096, 4096)], oracle.BF16, np.float32, whole=512.0),
+        "config3_f32_4096_rows_0_7": timed([(8, 4096, 4096)], oracle.F32, np.float32, whole=512.0),
+        # configuration 4 as the reference would run it: op_matmul is 2-D only (ops/ops.c:6818), so a loop of per-head
+        # products; 2 of the 192 heads, S = Q.K^T on a densified K^T and O = P.V (the four backward GEMMs cost twice that again)
+        "config4_bf16_2_heads_fwd": timed([(512, 64, 512), (512, 512, 64)] * 2, oracle.BF16, np.float32, whole=96.0),
+        "config4_f32_2_heads_fwd": timed([(512, 64, 512), (512, 512, 64)] * 2, oracle.F32, np.float32, whole=96.0),
         "config5a_bf16_m1": timed([(1, 8192, 8192)], oracle.BF16, np.float32),           # the loop is linear in m: m = 8 and 32 take 8 and 32 times as long
         "config5b_f64_2048_rows_0_31": timed([(32, 2048, 2048)], oracle.F64, np.float64),
     }
@@ -266,7 +280,7 @@ def f16_time(capi, n=8192):
 
 def square_sweep(capi, sizes=(1024, 4096)):
     """Config 3 below the headline size: C = A.B, dA = dC.Bt, dB = At.dC (transposes as stride views) in bf16 and
-    fp16 at N = 1024 and 4096, each replayed from a HIP graph; microseconds and TFLOP/s."""
+    fp16 at N = 1024 and 4096, each replayed from a HIP graph; microseconds, TFLOP/s and the fraction of the MFMA peak."""
     out = {}
     rng = np.random.default_rng(2)
     for n in sizes:
@@ -282,7 +296,8 @@ def square_sweep(capi, sizes=(1024, 4096)):
             row = {}
             for op, fn in ops.items():
                 ms = _time_graph(capi, fn, 10, 2)
-                row[op] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(2.0 * n ** 3 / ms / 1e9, 1)}
+                tf = 2.0 * n ** 3 / ms / 1e9
+                row[op] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(tf, 1), "frac_mfma": round(tf / PEAK_TFLOPS[name], 3)}
             out[f"{name}_{n}"] = row
             for d in (d_a, d_b, d_dc, d_c):
                 d.free()
@@ -346,6 +361,7 @@ def attention_times(capi, dt_name="bf16"):
         out[name] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1), "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 3)}
         if flops:
             out[name]["TFLOP/s"] = round(flops / ms / 1e9, 1)
+            out[name]["frac_mfma"] = round(flops / ms / 1e9 / PEAK_TFLOPS[dt_name], 3)       # these GEMMs sit near the ridge: both fractions are given
     out["fwd_bwd_ms"] = round(total + out["scale"]["us"] * 1e-3, 4)     # the scale runs twice (S/8 and dS/8)
     # the same forward (S, scale, softmax, O) as one fused kernel that never writes S or P
     fused = lambda: capi.check(L.rp_hip_attention_forward(d_o.ptr, d_q.ptr, d_k.ptr, d_v.ptr, None, Z, S, S, D,
