@@ -163,6 +163,10 @@ int log_softmax_kernel_device(void* out, const void* x, size_t outer_size, size_
 /* ops/grad_device.cu:1236-1291 */
 int backwards_softmax_device(const void* grad_c, const void* softmax_out, void* grad_x,
                              size_t outer_size, size_t dim_size, size_t inner_size, int dtype);
+/* ops/ops.h:260, ops/grad_device.cu:1256-1310 (values of ops/grad_host.c:1428-1500): grad_x = grad_c - exp(y) * sum over
+ * the axis of grad_c, with y the output of log_softmax; the gradient of op_log_softmax (ops/ops.c:5693-5719). */
+int backwards_log_softmax_device(const void* grad_c, const void* log_softmax_out, void* grad_x,
+                                 size_t outer_size, size_t dim_size, size_t inner_size, int dtype);
 /* functional/functional_device.cu:1197-1266: gather a strided view (element strides) into dense memory */
 int contiguous_copy_kernel_device(void* out, const void* in, int ndim, int* shape, int* strides, size_t size, int dtype);
 /* functional/functional_device.cu:756-989: out is a one-element device buffer */
@@ -213,6 +217,19 @@ int rp_hip_cross_entropy_mean(void* loss_out, void* grad_logits, const void* log
  * device-to-host copy (the reference reads it on the host, ops/ops.c:5412-5543). */
 int rp_hip_cross_entropy_backward(void* grad_logits, const void* logits, const int* targets, int batch, int classes,
                                   const void* upstream_dev, int dtype);
+
+/* Cross-entropy with every reduction (0 none, 1 mean, 2 sum: ops/ops.h:109-111) on logits (from_logits != 0:
+ * log_softmax + softmax inside) or on probabilities (from_logits == 0: log(x), as op_cross_entropy_loss does when its
+ * input came out of op_softmax, ops/ops.c:5553-5585).  x [batch, classes], float32 / float64; targets: device
+ * int32[batch].  loss_out: batch elements for 'none', one otherwise (the NLL terms summed in batch order in double,
+ * ops/ops.c:5342-5352). */
+int rp_hip_cross_entropy_forward(void* loss_out, const void* x, const int* targets, int batch, int classes,
+                                 int reduction, int from_logits, int dtype);
+/* Its gradient (backward_cross_entropy_loss_fn, ops/ops.c:5412-5543, which the reference builds on the host):
+ * softmax - onehot, or -1 / p at the target for probabilities; times 1 / batch for 'mean'; times the upstream
+ * gradient read on the device (batch elements for 'none', one otherwise). */
+int rp_hip_cross_entropy_grad(void* grad_x, const void* x, const int* targets, int batch, int classes,
+                              int reduction, int from_logits, const void* upstream_dev, int dtype);
 
 /* ---- conv2d lowering (the callers of the GEMM in op_conv2d, ops/ops.c:4723-4870 and 4473-4720) ---- */
 

@@ -65,6 +65,8 @@ _sum_all = _sig("orc_sum_all", _i, _vp, _vp, _sz, _i)
 _reduce_rows = _sig("orc_reduce_rows", _i, _vp, _vp, _i, _i, _i)
 _contig = _sig("orc_contiguous_copy", _i, _vp, _vp, _i, _ip, _llp, _i)
 _ce = _sig("orc_cross_entropy_mean", _i, _vp, _vp, _vp, _ip, _i, _i, _d, _i)
+_ce_any = _sig("orc_cross_entropy", _i, _vp, _vp, _vp, _ip, _i, _i, _i, _i, _vp, _i)
+_bw_log_softmax = _sig("orc_backwards_log_softmax", _i, _vp, _vp, _vp, _sz, _sz, _sz, _i)
 _sigmoid = _sig("orc_sigmoid", _i, _vp, _vp, _sz, _i)
 _tanh = _sig("orc_tanh", _i, _vp, _vp, _sz, _i)
 _im2col = _sig("orc_im2col", _i, _vp, _vp, *([_i] * 14))
@@ -239,6 +241,36 @@ def cross_entropy_mean(logits, targets, dtype, upstream=1.0):
     _check(_ce(_ptr(loss), _ptr(grad), _ptr(logits), t.ctypes.data_as(_ip), b, c, float(upstream), dtype),
            "cross_entropy_mean")
     return loss, grad
+
+
+REDUCTIONS = {"none": 0, "mean": 1, "sum": 2}          # reference ops/ops.h:109-111
+
+
+def cross_entropy(x, targets, dtype, reduction="mean", from_logits=True, upstream=None):
+    """reference ops/ops.c:5545-5643 with every reduction, on logits or on probabilities (from_logits=False).
+    Returns (loss, dx): loss has shape [batch] for 'none' and [1] otherwise; dx is None unless `upstream` (the
+    gradient of the loss: [batch] for 'none', one element otherwise) is given.  f32 / f64 only."""
+    x = np.ascontiguousarray(x)
+    b, c = x.shape
+    t = np.ascontiguousarray(targets, dtype=np.int32)
+    red = REDUCTIONS[reduction]
+    loss = np.empty((b if red == 0 else 1,), dtype=NP_STORAGE[dtype])
+    grad, up = None, None
+    if upstream is not None:
+        grad = np.empty_like(x)
+        up = np.ascontiguousarray(np.broadcast_to(np.asarray(upstream, dtype=NP_STORAGE[dtype]).reshape(-1), (b if red == 0 else 1,)))
+    _check(_ce_any(_ptr(loss), _ptr(grad) if grad is not None else None, _ptr(x), t.ctypes.data_as(_ip), b, c, red, int(bool(from_logits)),
+                   _ptr(up) if up is not None else None, dtype), "cross_entropy")
+    return loss, grad
+
+
+def backwards_log_softmax(grad_c, y, dtype, dim=-1):
+    """reference ops/grad_host.c:1428-1500: y is the log-softmax output."""
+    grad_c = np.ascontiguousarray(grad_c); y = np.ascontiguousarray(y)
+    out = np.empty_like(y)
+    o, d, i = _split(y.shape, dim)
+    _check(_bw_log_softmax(_ptr(grad_c), _ptr(y), _ptr(out), o, d, i, dtype), "backwards_log_softmax")
+    return out
 
 
 # ---------------------------------------------------------------------------

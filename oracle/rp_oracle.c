@@ -582,6 +582,125 @@ done:
 }
 
 /* ---------------------------------------------------------------------------
+ * Cross-entropy with every reduction and both input kinds.
+ * reference ops/ops.c:5545-5643 (op_cross_entropy_loss), 5318-5400 (op_nll_loss),
+ * 5412-5543 (backward_cross_entropy_loss_fn); reduction codes ops/ops.h:109-111
+ * (0 none, 1 mean, 2 sum).
+ *   from_logits != 0: log_probs = log_softmax(x), the saved probabilities = softmax(x);
+ *   from_logits == 0: x already holds probabilities, log_probs = log(x) (rp_log, element-wise).
+ * Forward: NLL terms -log_probs[b, target_b]; 'none' returns them, otherwise they are
+ * summed in batch order in double, narrowed to float for float32, and 'mean' then divides
+ * by (float)batch in the tensor's type.
+ * Backward: grad = p - onehot (logits) or -1 / p at the target and 0 elsewhere
+ * (probabilities); 'mean' multiplies by 1 / batch; then by the upstream gradient, one
+ * element for 'mean' / 'sum', one per row for 'none' (rp_mul_strided with strides {1, 0}).
+ * float32 / float64 only, as orc_cross_entropy_mean.
+ * ------------------------------------------------------------------------- */
+int orc_cross_entropy(void* loss_out, void* grad_x, const void* x, const int* targets, int batch, int classes,
+                      int reduction, int from_logits, const void* upstream, int dtype) {
+    if (!x || !targets || batch <= 0 || classes <= 0 || reduction < 0 || reduction > 2) return -1;
+    if (dtype != ORC_F32 && dtype != ORC_F64) return -1;
+    for (int b = 0; b < batch; b++) if (targets[b] < 0 || targets[b] >= classes) return -1;
+    size_t n = (size_t)batch * classes, es = orc_elem_size(dtype);
+    void* lp = malloc(n * es);
+    void* sm = malloc(n * es);
+    int rc = -1;
+    if (!lp || !sm) goto done;
+    if (from_logits) {
+        orc_log_softmax(lp, x, (size_t)batch, (size_t)classes, 1, dtype);
+        orc_softmax(sm, x, (size_t)batch, (size_t)classes, 1, dtype);
+    } else {
+        if (dtype == ORC_F64) for (size_t i = 0; i < n; i++) ((double*)lp)[i] = log(((const double*)x)[i]);
+        else for (size_t i = 0; i < n; i++) ((float*)lp)[i] = logf(((const float*)x)[i]);
+        memcpy(sm, x, n * es);
+    }
+    if (loss_out) {
+        if (reduction == 0) {
+            for (int b = 0; b < batch; b++) {
+                size_t off = (size_t)b * classes + targets[b];
+                if (dtype == ORC_F64) ((double*)loss_out)[b] = -((const double*)lp)[off];
+                else ((float*)loss_out)[b] = -((const float*)lp)[off];
+            }
+        } else {
+            double s64 = 0.0;
+            for (int b = 0; b < batch; b++) {
+                size_t off = (size_t)b * classes + targets[b];
+                if (dtype == ORC_F64) s64 -= ((const double*)lp)[off];
+                else s64 -= (double)((const float*)lp)[off];
+            }
+            float s32 = (float)s64;
+            if (reduction == 1) { s32 /= (float)batch; s64 /= (double)batch; }
+            if (dtype == ORC_F64) *(double*)loss_out = s64; else *(float*)loss_out = s32;
+        }
+    }
+    if (grad_x) {
+        if (!upstream) goto done;
+        if (dtype == ORC_F64) {
+            double* g = (double*)grad_x; const double* s = (const double*)sm; const double* up = (const double*)upstream;
+            if (from_logits) {
+                for (size_t i = 0; i < n; i++) g[i] = s[i];
+                for (int b = 0; b < batch; b++) g[(size_t)b * classes + targets[b]] -= 1.0;
+            } else {
+                for (size_t i = 0; i < n; i++) g[i] = 0.0;
+                for (int b = 0; b < batch; b++) { size_t ti = (size_t)b * classes + targets[b]; g[ti] = -1.0 / s[ti]; }
+            }
+            if (reduction == 1) { double sc = 1.0 / (double)batch; for (size_t i = 0; i < n; i++) g[i] *= sc; }
+            for (size_t i = 0; i < n; i++) g[i] = g[i] * (reduction == 0 ? up[i / (size_t)classes] : up[0]);
+        } else {
+            float* g = (float*)grad_x; const float* s = (const float*)sm; const float* up = (const float*)upstream;
+            if (from_logits) {
+                for (size_t i = 0; i < n; i++) g[i] = s[i];
+                for (int b = 0; b < batch; b++) g[(size_t)b * classes + targets[b]] -= 1.0f;
+            } else {
+                for (size_t i = 0; i < n; i++) g[i] = 0.0f;
+                for (int b = 0; b < batch; b++) { size_t ti = (size_t)b * classes + targets[b]; g[ti] = -1.0f / s[ti]; }
+            }
+            if (reduction == 1) { float sc = 1.0f / (float)batch; for (size_t i = 0; i < n; i++) g[i] *= sc; }
+            for (size_t i = 0; i < n; i++) g[i] = g[i] * (reduction == 0 ? up[i / (size_t)classes] : up[0]);
+        }
+    }
+    rc = 0;
+done:
+    free(lp); free(sm);
+    return rc;
+}
+
+/* gradient of log_softmax: gx = g - exp(y) * sum_d g, the sum in index order in the compute type.
+ * reference ops/grad_host.c:1428-1500 (16-bit through the fp32 pivot, one narrowing). */
+int orc_backwards_log_softmax(const void* grad_c, const void* y, void* grad_x,
+                              size_t outer, size_t dim, size_t inner, int dtype) {
+    if (!grad_c || !y || !grad_x) return -1;
+    size_t n = outer * dim * inner;
+    if (dtype == ORC_F64) {
+        const double* g = (const double*)grad_c; const double* l = (const double*)y; double* r = (double*)grad_x;
+        for (size_t o = 0; o < outer; o++) for (size_t i = 0; i < inner; i++) {
+            size_t base = o * dim * inner + i;
+            double sum = 0.0;
+            for (size_t d = 0; d < dim; d++) sum += g[base + d * inner];
+            for (size_t d = 0; d < dim; d++) r[base + d * inner] = g[base + d * inner] - exp(l[base + d * inner]) * sum;
+        }
+        return 0;
+    }
+    float* gw = (float*)orc_load_as_compute(grad_c, n, dtype);
+    float* lw = (float*)orc_load_as_compute(y, n, dtype);
+    int half = (dtype == ORC_F16 || dtype == ORC_BF16);
+    if (half && (!gw || !lw)) { free(gw); free(lw); return -1; }
+    const float* g = half ? gw : (const float*)grad_c;
+    const float* l = half ? lw : (const float*)y;
+    float* r = half ? (float*)malloc((n ? n : 1) * 4) : (float*)grad_x;
+    if (!r) { free(gw); free(lw); return -1; }
+    for (size_t o = 0; o < outer; o++) for (size_t i = 0; i < inner; i++) {
+        size_t base = o * dim * inner + i;
+        float sum = 0.0f;
+        for (size_t d = 0; d < dim; d++) sum += g[base + d * inner];
+        for (size_t d = 0; d < dim; d++) r[base + d * inner] = g[base + d * inner] - expf(l[base + d * inner]) * sum;
+    }
+    if (half) { orc_narrow(r, grad_x, n, dtype); free(r); }
+    free(gw); free(lw);
+    return 0;
+}
+
+/* ---------------------------------------------------------------------------
  * conv2d lowering.  reference functional/functional_host.c:1237-1262 (im2col)
  * and 1291-1313 (col2im, which ADDS into im); 16-bit through the fp32 pivot with
  * one narrowing at the end (functional/functional.c:866-879, 896-911).

@@ -60,6 +60,7 @@ SIGNATURES = {
     "softmax_kernel_device": (_i, [_vp, _vp, _sz, _sz, _sz, _i]),
     "log_softmax_kernel_device": (_i, [_vp, _vp, _sz, _sz, _sz, _i]),
     "backwards_softmax_device": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _i]),
+    "backwards_log_softmax_device": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _i]),
     "contiguous_copy_kernel_device": (_i, [_vp, _vp, _i, _ip, _ip, _sz, _i]),
     "sum_all_kernel_device": (_i, [_vp, _vp, _sz, _i]),
     "mean_all_kernel_device": (_i, [_vp, _vp, _sz, _i]),
@@ -70,6 +71,8 @@ SIGNATURES = {
     "rp_hip_linear_backward": (_i, [_vp] * 6 + [_i] * 3 + [_ll] * 8 + [_i] * 4),
     "rp_hip_cross_entropy_mean": (_i, [_vp, _vp, _vp, _vp, _i, _i, _d, _i]),
     "rp_hip_cross_entropy_backward": (_i, [_vp, _vp, _vp, _i, _i, _vp, _i]),
+    "rp_hip_cross_entropy_forward": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i]),
+    "rp_hip_cross_entropy_grad": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _i]),
     "rp_hip_fill_scaled": (_i, [_vp, _vp, _d, _sz, _i]),
     "im2col_kernel_device": (_i, [_vp, _vp] + [_i] * 14),
     "col2im_kernel_device": (_i, [_vp, _vp] + [_i] * 14),

@@ -434,6 +434,38 @@ __global__ void backwards_softmax_strided_kernel(const T* gc, const T* y, T* gx,
     }
 }
 
+// gradient of log_softmax (reference ops/grad_host.c:1428-1500): gx = g - exp(y) * sum_d g, with y the op's output.
+// One thread per (outer, inner) pair, the sum in index order as the reference's host loop runs it; for rows that
+// are contiguous (inner == 1) a wave per row with the partial sums of the lanes added by wave_sum.
+template <typename T>
+__global__ void backwards_log_softmax_rows_kernel(const T* gc, const T* y, T* gx, size_t rows, size_t dim) {
+    using A = typename traits<T>::acc;
+    int lane = threadIdx.x & 63;
+    size_t wave = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    size_t nwaves = ((size_t)gridDim.x * blockDim.x) >> 6;
+    for (size_t r = wave; r < rows; r += nwaves) {
+        const T* g = gc + r * dim;
+        const T* l = y + r * dim;
+        A sum = 0;
+        for (size_t d = lane; d < dim; d += 64) sum += widen(g[d]);
+        sum = wave_sum(sum);
+        for (size_t d = lane; d < dim; d += 64) gx[r * dim + d] = narrow<T>(widen(g[d]) - rp_exp(widen(l[d])) * sum);
+    }
+}
+
+template <typename T>
+__global__ void backwards_log_softmax_strided_kernel(const T* gc, const T* y, T* gx, size_t outer, size_t dim, size_t inner) {
+    using A = typename traits<T>::acc;
+    size_t n = outer * inner;
+    for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (size_t)gridDim.x * blockDim.x) {
+        size_t base = (t / inner) * dim * inner + (t % inner);
+        A sum = 0;
+        for (size_t d = 0; d < dim; d++) sum += widen(gc[base + d * inner]);
+        for (size_t d = 0; d < dim; d++)
+            gx[base + d * inner] = narrow<T>(widen(gc[base + d * inner]) - rp_exp(widen(y[base + d * inner])) * sum);
+    }
+}
+
 // ---- reductions ----------------------------------------------------------------------
 // Deterministic two-level sum in two launches: each block sums a contiguous slab
 // (threads stride it, then a fixed-order LDS tree) into a file-scope partials
@@ -561,6 +593,66 @@ __global__ void cross_entropy_kernel(T* loss, T* grad, const T* logits, const in
     if (threadIdx.x == 0 && loss) {
         if (sizeof(T) == 8) loss[0] = (T)(total / (double)batch);
         else { float f = (float)total; f /= (float)batch; loss[0] = (T)f; }
+    }
+}
+
+// The same with every reduction (0 none, 1 mean, 2 sum: reference ops/ops.h:109-111) and on probabilities as well as on
+// logits (reference ops/ops.c:5545-5643, 5412-5543).  loss: batch elements for 'none', one otherwise.  upstream_dev: the
+// gradient of the loss on the device, batch elements for 'none', one otherwise (grad only).
+template <typename T>
+__global__ void cross_entropy_any_kernel(T* loss, T* grad, const T* x, const int* targets, int batch, int classes,
+                                         int reduction, int from_logits, const T* upstream_dev) {
+    __shared__ double nll[kThreads];
+    double total = 0.0;
+    for (int b0 = 0; b0 < batch; b0 += blockDim.x) {
+        int b = b0 + threadIdx.x;
+        if (b < batch) {
+            const T* row = x + (size_t)b * classes;
+            int t = targets[b];
+            bool valid = (t >= 0 && t < classes);      // callers validate; a bad index poisons the loss instead of reading out of bounds
+            T mx = 0, sum = 1, logp = 0;
+            if (from_logits) {
+                mx = lowest<T>();
+                for (int c = 0; c < classes; c++) mx = row[c] > mx ? row[c] : mx;
+                sum = 0;
+                for (int c = 0; c < classes; c++) sum += rp_exp(row[c] - mx);
+                if (valid) logp = row[t] - mx - rp_log(sum);
+            } else if (valid) {
+                logp = rp_log(row[t]);
+            }
+            nll[threadIdx.x] = valid ? -(double)logp : (double)NAN;
+            if (loss && reduction == 0) loss[b] = valid ? -logp : (T)NAN;
+            if (grad) {
+                const T up = upstream_dev[reduction == 0 ? b : 0];
+                const T sc = (T)1 / (T)batch;
+                for (int c = 0; c < classes; c++) {
+                    T g;
+                    if (from_logits) { g = rp_exp(row[c] - mx) / sum; if (c == t) g -= (T)1; }
+                    else g = (c == t) ? (T)-1 / row[c] : (T)0;
+                    if (reduction == 1) g *= sc;
+                    grad[(size_t)b * classes + c] = g * up;
+                }
+            }
+        }
+        if (!loss || reduction == 0) continue;         // uniform: no thread reaches the barriers
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const int lim = batch - b0 < (int)blockDim.x ? batch - b0 : (int)blockDim.x;
+            int i = 0;
+            for (; i + 16 <= lim; i += 16) {             // sixteen LDS reads in flight, the adds one by one in batch order, in double (reference ops/ops.c:5342-5352)
+                double v[16];
+#pragma unroll
+                for (int u = 0; u < 16; u++) v[u] = nll[i + u];
+#pragma unroll
+                for (int u = 0; u < 16; u++) total += v[u];
+            }
+            for (; i < lim; i++) total += nll[i];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0 && loss && reduction != 0) {
+        if (sizeof(T) == 8) loss[0] = (T)(reduction == 1 ? total / (double)batch : total);
+        else { float f = (float)total; if (reduction == 1) f /= (float)batch; loss[0] = (T)f; }
     }
 }
 
@@ -707,6 +799,20 @@ int backwards_softmax_device(const void* grad_c, const void* softmax_out, void* 
     return check_launch("backwards_softmax kernel") ? 0 : -1;
 }
 
+int backwards_log_softmax_device(const void* grad_c, const void* log_softmax_out, void* grad_x,
+                                 size_t outer_size, size_t dim_size, size_t inner_size, int dtype) {
+    RP_REQUIRE(grad_c && log_softmax_out && grad_x && outer_size && dim_size && inner_size, "backwards_log_softmax_device");
+    if (inner_size == 1) {
+        unsigned blocks = grid_for(outer_size * 64, kThreads, 1u << 16);       // a wave per row
+        RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(backwards_log_softmax_rows_kernel<T>, dim3(blocks), dim3(kThreads), 0, current_stream(),
+                                                    (const T*)grad_c, (const T*)log_softmax_out, (T*)grad_x, outer_size, dim_size));
+    } else {
+        RP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(backwards_log_softmax_strided_kernel<T>, dim3(grid_for(outer_size * inner_size)), dim3(kThreads), 0,
+                                                    current_stream(), (const T*)grad_c, (const T*)log_softmax_out, (T*)grad_x, outer_size, dim_size, inner_size));
+    }
+    return check_launch("backwards_log_softmax kernel") ? 0 : -1;
+}
+
 int contiguous_copy_kernel_device(void* out, const void* in, int ndim, int* shape, int* strides, size_t size, int dtype) {
     RP_REQUIRE(out && in && shape && strides && size && ndim > 0, "contiguous_copy_kernel_device");
     if (ndim > kMaxDims) { set_error("contiguous_copy_kernel_device: more than %d dimensions", kMaxDims); return -1; }
@@ -790,6 +896,32 @@ int rp_hip_cross_entropy_backward(void* grad_logits, const void* logits, const i
         hipLaunchKernelGGL(cross_entropy_kernel<double>, dim3(1), dim3(kThreads), 0, current_stream(), (double*)nullptr, (double*)grad_logits,
                            (const double*)logits, targets, batch, classes, 1.0, (const double*)upstream_dev);
     return check_launch("cross_entropy_kernel") ? 0 : -1;
+}
+
+int rp_hip_cross_entropy_forward(void* loss_out, const void* x, const int* targets, int batch, int classes,
+                                 int reduction, int from_logits, int dtype) {
+    RP_REQUIRE(loss_out && x && targets && batch > 0 && classes > 0 && reduction >= 0 && reduction <= 2, "rp_hip_cross_entropy_forward");
+    if (dtype != RP_DTYPE_FLOAT32 && dtype != RP_DTYPE_FLOAT64) { set_error("rp_hip_cross_entropy_forward: float32 and float64 only"); return -1; }
+    if (dtype == RP_DTYPE_FLOAT32)
+        hipLaunchKernelGGL(cross_entropy_any_kernel<float>, dim3(1), dim3(kThreads), 0, current_stream(), (float*)loss_out, (float*)nullptr,
+                           (const float*)x, targets, batch, classes, reduction, from_logits ? 1 : 0, (const float*)nullptr);
+    else
+        hipLaunchKernelGGL(cross_entropy_any_kernel<double>, dim3(1), dim3(kThreads), 0, current_stream(), (double*)loss_out, (double*)nullptr,
+                           (const double*)x, targets, batch, classes, reduction, from_logits ? 1 : 0, (const double*)nullptr);
+    return check_launch("cross_entropy_any_kernel") ? 0 : -1;
+}
+
+int rp_hip_cross_entropy_grad(void* grad_x, const void* x, const int* targets, int batch, int classes,
+                              int reduction, int from_logits, const void* upstream_dev, int dtype) {
+    RP_REQUIRE(grad_x && x && targets && upstream_dev && batch > 0 && classes > 0 && reduction >= 0 && reduction <= 2, "rp_hip_cross_entropy_grad");
+    if (dtype != RP_DTYPE_FLOAT32 && dtype != RP_DTYPE_FLOAT64) { set_error("rp_hip_cross_entropy_grad: float32 and float64 only"); return -1; }
+    if (dtype == RP_DTYPE_FLOAT32)
+        hipLaunchKernelGGL(cross_entropy_any_kernel<float>, dim3(1), dim3(kThreads), 0, current_stream(), (float*)nullptr, (float*)grad_x,
+                           (const float*)x, targets, batch, classes, reduction, from_logits ? 1 : 0, (const float*)upstream_dev);
+    else
+        hipLaunchKernelGGL(cross_entropy_any_kernel<double>, dim3(1), dim3(kThreads), 0, current_stream(), (double*)nullptr, (double*)grad_x,
+                           (const double*)x, targets, batch, classes, reduction, from_logits ? 1 : 0, (const double*)upstream_dev);
+    return check_launch("cross_entropy_any_kernel") ? 0 : -1;
 }
 
 int rp_hip_fill_scaled(void* ptr, const void* scalar_dev, double scale, size_t size, int dtype) {

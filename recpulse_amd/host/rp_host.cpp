@@ -805,6 +805,20 @@ void backward_softmax_fn(GradFn* self, Tensor* grad_output) {        // referenc
     free_tensor(gd);
 }
 
+void backward_log_softmax_fn(GradFn* self, Tensor* grad_output) {    // reference ops/ops.c:5693-5719; y is the op's own output
+    Tensor* x = self->inputs[0];
+    if (!needs_grad(x)) return;
+    Tensor* y = self->owner;
+    int dim = ((DimSaved*)self->saved_data)->dim;
+    size_t outer, d, inner;
+    split_dims(y, dim, &outer, &d, &inner);
+    Tensor* gd = dense(grad_output);
+    Tensor* g = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
+    if (g && gd && on_device(x->device_id) && backwards_log_softmax_device(gd->data, y->data, g->data, outer, d, inner, x->dtype) == 0) accumulate_grad(x, g);
+    else { dev_fail("log_softmax backward"); free_tensor(g); }
+    free_tensor(gd);
+}
+
 struct ScalarSaved { double s; };
 
 void backward_mul_scalar_fn(GradFn* self, Tensor* grad_output) {     // reference ops/ops.c:5966-6020
@@ -1065,7 +1079,7 @@ void backward_reduce_all_fn(GradFn* self, Tensor* grad_output) {     // sum_all 
     else { if (!g_backward_err[0]) fail("sum_all / mean_all backward failed"); free_tensor(g); }
 }
 
-struct CESaved { int batch, classes; void* targets_dev; int device_id; };
+struct CESaved { int batch, classes; void* targets_dev; int device_id; int reduction, from_logits; };
 
 void free_ce_saved(void* p) {
     CESaved* s = (CESaved*)p;
@@ -1078,18 +1092,19 @@ void backward_cross_entropy_fn(GradFn* self, Tensor* grad_output) {
     Tensor* x = self->inputs[0];
     if (!needs_grad(x)) return;
     CESaved* s = (CESaved*)self->saved_data;
-    double up = 1.0;
-    const bool beside = scalar_beside(grad_output, x);
-    if (!beside && tensor_read_scalar(grad_output, &up) != 0) { fail("cross-entropy backward: upstream gradient could not be read"); return; }
+    // the upstream gradient is read where it lives: one element for 'mean' / 'sum', one per row for 'none'
+    Tensor* up = nullptr;
+    const size_t want = s->reduction == 0 ? (size_t)s->batch : 1;
+    if (grad_output->size == want && grad_output->device_id == x->device_id && grad_output->dtype == x->dtype) up = dense(grad_output);
+    else if (grad_output->size == want) up = tensor_to(grad_output, x->device_id, x->dtype, false);
     Tensor* xd = dense(x);
     Tensor* g = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
     int rc = -1;
-    if (g && xd && on_device(x->device_id))
-        rc = beside ? rp_hip_cross_entropy_backward(g->data, xd->data, (const int*)s->targets_dev, s->batch, s->classes, grad_output->data, x->dtype)
-                    : rp_hip_cross_entropy_mean(nullptr, g->data, xd->data, (const int*)s->targets_dev, s->batch, s->classes, up, x->dtype);
+    if (g && xd && up && on_device(x->device_id))
+        rc = rp_hip_cross_entropy_grad(g->data, xd->data, (const int*)s->targets_dev, s->batch, s->classes, s->reduction, s->from_logits, up->data, x->dtype);
     if (rc == 0) accumulate_grad(x, g);
-    else { dev_fail("cross-entropy backward"); free_tensor(g); }
-    free_tensor(xd);
+    else { if (up) dev_fail("cross-entropy backward"); else fail("cross-entropy backward: upstream gradient has the wrong size"); free_tensor(g); }
+    free_tensor(xd); free_tensor(up);
 }
 
 struct PermSaved { int ndim; int dims[8]; };
@@ -1387,8 +1402,8 @@ static Tensor* softmax_any(Tensor* x, int dim, bool take_log) {
                                                           : softmax_kernel_device(out->data, xd->data, outer, d, inner, x->dtype)) : -1;
     free_tensor(xd);
     if (rc != 0) { dev_fail("softmax"); free_tensor(out); return nullptr; }
-    if (!take_log && needs_grad(x)) {
-        GradFn* gf = attach(out, backward_softmax_fn, {x});
+    if (needs_grad(x)) {
+        GradFn* gf = attach(out, take_log ? backward_log_softmax_fn : backward_softmax_fn, {x});
         DimSaved* s = (DimSaved*)malloc(sizeof(DimSaved));
         s->dim = dim;
         gf->saved_data = s;
@@ -1444,22 +1459,25 @@ Tensor* op_cross_entropy_loss(Tensor* input, const int* targets, int batch_size,
     if (!input || !targets) return nullptr;
     for (int b = 0; b < batch_size; b++) if (targets[b] < 0 || targets[b] >= num_classes) { fail("op_cross_entropy_loss: target out of range"); return nullptr; }
     if (input->ndim != 2 || input->shape[0] != batch_size || input->shape[1] != num_classes) { fail("op_cross_entropy_loss: input must be [batch, classes]"); return nullptr; }
-    if (reduction != 1 || from_logits == 0) { fail("op_cross_entropy_loss: this build provides reduction='mean' on logits"); return nullptr; }
+    if (reduction < 0 || reduction > 2) { fail("op_cross_entropy_loss: reduction must be none (0), mean (1) or sum (2)"); return nullptr; }
+    // -1: an input that came out of op_softmax holds probabilities, anything else logits (reference ops/ops.c:5553-5557)
+    if (from_logits == -1) from_logits = !(input->metadata && input->metadata->grad_fn && input->metadata->grad_fn->backward == backward_softmax_fn);
     if (input->dtype != DTYPE_FLOAT32 && input->dtype != DTYPE_FLOAT64) { fail("op_cross_entropy_loss: float32 / float64 only"); return nullptr; }
     if (input->device_id == -1) { fail("op_cross_entropy_loss on host tensors is not provided by this build"); return nullptr; }
     if (!on_device(input->device_id)) { dev_fail("set device"); return nullptr; }
     void* tdev = nullptr;
     if (rp_hip_malloc(&tdev, sizeof(int) * batch_size) != 0 || rp_hip_memcpy_h2d(tdev, targets, sizeof(int) * batch_size) != 0) { dev_fail("targets upload"); if (tdev) rp_hip_free(tdev); return nullptr; }
     Tensor* xd = dense(input);
-    int one = 1;
-    Tensor* out = xd ? empty_tensor(input->dtype, input->device_id, 1, &one) : nullptr;
-    int rc = out ? rp_hip_cross_entropy_mean(out->data, nullptr, xd->data, (const int*)tdev, batch_size, num_classes, 1.0, input->dtype) : -1;
+    int out_len = reduction == 0 ? batch_size : 1;                   // 'none' keeps one loss per row (reference ops/ops.c:5356-5360)
+    Tensor* out = xd ? empty_tensor(input->dtype, input->device_id, 1, &out_len) : nullptr;
+    int rc = out ? rp_hip_cross_entropy_forward(out->data, xd->data, (const int*)tdev, batch_size, num_classes, reduction, from_logits, input->dtype) : -1;
     free_tensor(xd);
     if (rc != 0) { dev_fail("cross entropy"); rp_hip_free(tdev); free_tensor(out); return nullptr; }
     if (needs_grad(input)) {
         GradFn* gf = attach(out, backward_cross_entropy_fn, {input});
         CESaved* s = (CESaved*)calloc(1, sizeof(CESaved));
         s->batch = batch_size; s->classes = num_classes; s->targets_dev = tdev; s->device_id = input->device_id;
+        s->reduction = reduction; s->from_logits = from_logits;
         gf->saved_data = s;
         gf->free_saved = free_ce_saved;
     } else {

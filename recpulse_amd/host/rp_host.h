@@ -108,7 +108,7 @@ Tensor* op_attention(Tensor* q, Tensor* k, Tensor* v, double scale);   /* softma
 Tensor* op_add(Tensor* x1, Tensor* x2);
 Tensor* op_relu(Tensor* x);
 Tensor* op_softmax(Tensor* x, int dim);
-Tensor* op_log_softmax(Tensor* x, int dim);              /* forward only */
+Tensor* op_log_softmax(Tensor* x, int dim);
 Tensor* op_mul_scalar(Tensor* x, double scalar);
 Tensor* op_sum_all(Tensor* x);
 Tensor* op_mean_all(Tensor* x);

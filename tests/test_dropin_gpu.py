@@ -414,3 +414,57 @@ def test_config4_full_size_on_4d_permuted_view(dtype, tol_gemm, tol_chain):
         assert oracle.rel_err(o_host[b, h], oracle.to_f64(want["O"], code)) <= tol_gemm, (b, h)
         for name in ("dQ", "dK", "dV"):
             assert oracle.rel_err(grads[name][b, h], oracle.to_f64(want[name], code)) <= tol_gemm, (name, b, h)
+
+
+# ---- op_cross_entropy_loss with every reduction, on logits and on the output of op_softmax (which the op detects and
+# treats as probabilities, reference ops/ops.c:5553-5585), and op_log_softmax with its backward (ops/ops.c:5693-5719,
+# 5790-5860): values and gradients against torch in float64
+@pytest.mark.parametrize("dtype,tol", [("float32", 4e-6), ("float64", 1e-12)])
+@pytest.mark.parametrize("reduction", ["none", "sum", "mean"])
+def test_cross_entropy_reductions_and_probability_inputs(dtype, tol, reduction):
+    import torch
+    rng = np.random.default_rng(58)
+    batch, classes = 48, 10
+    x = rng.normal(0, 2, (batch, classes)); w = rng.normal(0, 1, batch)
+    targets = rng.integers(0, classes, batch).tolist()
+    for through_softmax in (False, True):
+        xt = dev(x, dtype, grad=True)
+        src = xt.op_softmax(dim=-1) if through_softmax else xt
+        loss = src.op_cross_entropy_loss(targets, reduction=reduction)
+        assert loss.shape == ((batch,) if reduction == "none" else (1,))
+        tx = torch.tensor(host(xt), requires_grad=True)
+        tl = torch.nn.functional.cross_entropy(tx, torch.tensor(targets), reduction=reduction)
+        np.testing.assert_allclose(host(loss), tl.detach().numpy().reshape(loss.shape), rtol=tol * 10, atol=tol)
+        if reduction == "none":                       # weight the rows so that the per-row upstream gradient is exercised
+            wt = dev(w.reshape(1, batch), dtype)
+            wt.op_matmul(loss.reshape([batch, 1])).backward()
+            (tl * torch.tensor(host(wt)[0])).sum().backward()
+        else:
+            loss.backward()
+            tl.backward()
+        assert oracle.rel_err(host(xt.grad), tx.grad.numpy()) <= tol * 20, (reduction, through_softmax)
+    # explicit from_logits overrides the detection; an unknown reduction is refused
+    xt = dev(x, dtype)
+    a = xt.op_cross_entropy_loss(targets, reduction=reduction, from_logits=1)
+    b = xt.op_cross_entropy_loss(targets, reduction=reduction)
+    assert np.array_equal(host(a), host(b))
+    with pytest.raises(ValueError):
+        xt.op_cross_entropy_loss(targets, reduction="median")
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 4e-6), ("float64", 1e-12), ("bfloat16", 3e-2)])
+def test_log_softmax_backward(dtype, tol):
+    import torch
+    rng = np.random.default_rng(59)
+    x = rng.normal(0, 2, (6, 9, 5)); w = rng.normal(0, 1, (6, 9, 5))
+    for dim in (-1, 1):
+        xt = dev(x, dtype, grad=True)
+        y = xt.op_log_softmax(dim=dim)
+        assert y.requires_grad
+        # loss = sum(y * w) written with the ops at hand: flatten and multiply by w as a column
+        wt = dev(w.reshape(-1, 1), dtype)
+        y.reshape([1, x.size]).op_matmul(wt).backward()
+        tx = torch.tensor(host(xt), requires_grad=True)
+        (torch.log_softmax(tx, dim) * torch.tensor(host(wt).reshape(x.shape))).sum().backward()
+        np.testing.assert_allclose(host(y), torch.log_softmax(tx, dim).detach().numpy(), rtol=tol * 5, atol=tol * 5)
+        assert oracle.rel_err(host(xt.grad), tx.grad.numpy()) <= tol * 10, dim

@@ -195,6 +195,51 @@ def test_cross_entropy_backward_reads_the_upstream_gradient_on_the_device(dt):
     assert L().rp_hip_cross_entropy_backward(got.ptr, dl.ptr, dtg.ptr, batch, classes, dup.ptr, BF16) == -1
 
 
+@pytest.mark.parametrize("dt", [F32, F64], ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("from_logits", [True, False], ids=["logits", "probabilities"])
+@pytest.mark.parametrize("reduction", ["none", "sum", "mean"])
+def test_cross_entropy_every_reduction_on_logits_and_probabilities(dt, from_logits, reduction):
+    """rp_hip_cross_entropy_forward / _grad against the oracle's restatement of op_cross_entropy_loss and its backward
+    (reference ops/ops.c:5545-5643, 5412-5543)."""
+    rng = np.random.default_rng(50)
+    red = oracle.REDUCTIONS[reduction]
+    tolv = 4e-6 if dt == F32 else 1e-13
+    for batch, classes in ((256, 10), (7, 3), (1000, 33)):
+        x = oracle.to_storage(rng.normal(0, 3, (batch, classes)), dt)
+        if not from_logits:
+            x = oracle.softmax(x, dt)
+        t = rng.integers(0, classes, batch).astype(np.int32)
+        up = oracle.to_storage(rng.normal(0, 1, batch if red == 0 else 1), dt)
+        dx, dtg, dup = Dev(x, dt), capi.DeviceBuffer.from_numpy(t), Dev(up, dt)
+        dloss, dgrad = Dev.empty((batch if red == 0 else 1,), dt), Dev.empty((batch, classes), dt)
+        capi.check(L().rp_hip_cross_entropy_forward(dloss.ptr, dx.ptr, dtg.ptr, batch, classes, red, int(from_logits), dt), "ce forward")
+        capi.check(L().rp_hip_cross_entropy_grad(dgrad.ptr, dx.ptr, dtg.ptr, batch, classes, red, int(from_logits), dup.ptr, dt), "ce grad")
+        loss, grad = oracle.cross_entropy(x, t, dt, reduction, from_logits, upstream=up)
+        assert oracle.rel_err(dloss.numpy(), loss) <= tolv
+        assert oracle.rel_err(dgrad.numpy(), grad) <= tolv
+        if reduction == "mean" and from_logits:              # the older mean-on-logits entry gives the same bits
+            old = Dev.empty((1,), dt)
+            capi.check(L().rp_hip_cross_entropy_mean(old.ptr, None, dx.ptr, dtg.ptr, batch, classes, 1.0, dt), "ce")
+            assert np.array_equal(old.numpy(), dloss.numpy())
+    assert L().rp_hip_cross_entropy_forward(dloss.ptr, dx.ptr, dtg.ptr, batch, classes, 3, 1, dt) == -1
+    assert L().rp_hip_cross_entropy_forward(dloss.ptr, dx.ptr, dtg.ptr, batch, classes, red, 1, BF16) == -1
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_backwards_log_softmax(dt):
+    """Gradient of log_softmax (reference ops/grad_host.c:1428-1500) over the last and over a middle axis."""
+    rng = np.random.default_rng(51)
+    for shape, dim in (((7, 33), -1), ((1000, 10), -1), ((3, 600), -1), ((3, 5, 4), 1), ((2, 70, 3), 1)):
+        x = rand_storage(rng, shape, dt); g = rand_storage(rng, shape, dt)
+        y = oracle.softmax(x, dt, dim=dim, log=True)
+        o, d, i = oracle._split(shape, dim)
+        dg, dy, dgx = Dev(g, dt), Dev(y, dt), Dev.empty(shape, dt)
+        capi.check(L().backwards_log_softmax_device(dg.ptr, dy.ptr, dgx.ptr, o, d, i, dt), "backwards_log_softmax")
+        want = oracle.backwards_log_softmax(g, y, dt, dim=dim)
+        assert oracle.rel_err(oracle.to_f64(dgx.numpy(), dt), oracle.to_f64(want, dt)) <= _tol(dt), (shape, dim)
+    assert L().backwards_log_softmax_device(None, dy.ptr, dgx.ptr, o, d, i, dt) == -1
+
+
 @pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
 def test_fill_scaled_matches_a_host_side_product(dt):
     for value, scale, n in ((1.0, 1.0 / 777, 777), (-2.5, 1.0, 5000), (0.3, 1.0 / 3, 1)):

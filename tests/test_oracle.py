@@ -257,6 +257,12 @@ def test_elementwise_bit_equal_to_reference_kernels():
         o = np.empty_like(ys)
         assert REF.backwards_softmax_host(oracle._ptr(gs), oracle._ptr(ys), oracle._ptr(o), 7, 33, 1, dt) == 0
         assert np.array_equal(o, oracle.backwards_softmax(gs, ys, dt)), dt
+    REF.backwards_log_softmax_host.argtypes = [vp, vp, vp, sz, sz, sz, ctypes.c_int]
+    for dt in ALL:
+        ls = oracle.softmax(oracle.to_storage(x, dt), dt, log=True); gs = oracle.to_storage(g, dt)
+        o = np.empty_like(ls)
+        assert REF.backwards_log_softmax_host(oracle._ptr(gs), oracle._ptr(ls), oracle._ptr(o), 7, 33, 1, dt) == 0
+        assert np.array_equal(o, oracle.backwards_log_softmax(gs, ls, dt)), dt
     # broadcasting add, the Linear bias case
     y = rng.normal(0, 1, (6, 9)).astype(np.float32); b = rng.normal(0, 1, (9,)).astype(np.float32)
     o = np.empty_like(y)
@@ -557,3 +563,55 @@ def test_gru_cell_vs_torch(dt, tol, bias):
     want = [tx.grad, th.grad, tw1.grad, tw2.grad] + ([tb1.grad, tb2.grad] if bias else [])
     for name, g, w in zip(("dx", "dh", "dw_ih", "dw_hh", "db_ih", "db_hh"), got, want):
         assert oracle.rel_err(oracle.to_f64(g, dt), w.numpy()) <= 3 * tol, name
+
+
+# ---- cross-entropy with every reduction, on logits and on probabilities (reference ops/ops.c:5545-5643, 5412-5543),
+# and the gradient of log_softmax (ops/grad_host.c:1428-1500): against torch in float64 and against closed forms
+@pytest.mark.parametrize("dt,tdt,tol", [(F32, "float32", 2e-6), (F64, "float64", 1e-13)])
+@pytest.mark.parametrize("reduction", ["none", "sum", "mean"])
+def test_cross_entropy_every_reduction_vs_torch(dt, tdt, tol, reduction):
+    import torch
+    rng = np.random.default_rng(29)
+    batch, classes = 37, 11
+    logits = rng.normal(0, 2, (batch, classes)).astype(oracle.NP_STORAGE[dt])
+    targets = rng.integers(0, classes, batch)
+    up = rng.normal(0, 1, batch if reduction == "none" else 1).astype(oracle.NP_STORAGE[dt])
+    t = torch.tensor(logits.astype(np.float64), requires_grad=True)
+    l = torch.nn.functional.cross_entropy(t, torch.tensor(targets), reduction=reduction)
+    (l * torch.tensor(up.astype(np.float64))).sum().backward()
+    loss, grad = oracle.cross_entropy(logits, targets, dt, reduction, True, upstream=up)
+    assert loss.shape == ((batch,) if reduction == "none" else (1,))
+    np.testing.assert_allclose(loss, l.detach().numpy().reshape(loss.shape), rtol=tol * 10, atol=tol)
+    np.testing.assert_allclose(grad, t.grad.numpy(), rtol=tol * 50, atol=tol * 5)
+    # the same loss from probabilities: log(p) instead of log_softmax(x), gradient -1 / p at the target only
+    probs = oracle.softmax(logits, dt)
+    tp = torch.tensor(probs.astype(np.float64), requires_grad=True)
+    lp = torch.nn.functional.nll_loss(torch.log(tp), torch.tensor(targets), reduction=reduction)
+    (lp * torch.tensor(up.astype(np.float64))).sum().backward()
+    loss_p, grad_p = oracle.cross_entropy(probs, targets, dt, reduction, False, upstream=up)
+    np.testing.assert_allclose(loss_p, lp.detach().numpy().reshape(loss_p.shape), rtol=tol * 10, atol=tol)
+    np.testing.assert_allclose(grad_p, tp.grad.numpy(), rtol=tol * 50, atol=tol * 5)
+    assert np.count_nonzero(grad_p) <= batch                 # one entry per row
+    if reduction == "mean":                                     # the mean-on-logits path is the older entry, bit for bit
+        l0, g0 = oracle.cross_entropy_mean(logits, targets, dt, upstream=float(up[0]))
+        assert np.array_equal(l0, loss) and np.array_equal(g0, grad)
+    with pytest.raises(RuntimeError):
+        oracle.cross_entropy(logits, np.full(batch, classes), dt, reduction)
+
+
+@pytest.mark.parametrize("dt", ALL)
+def test_backwards_log_softmax_vs_torch_and_closed_form(dt):
+    import torch
+    rng = np.random.default_rng(31)
+    x = oracle.to_storage(rng.normal(0, 2, (3, 9, 4)), dt); g = oracle.to_storage(rng.normal(0, 1, (3, 9, 4)), dt)
+    for dim in (1, 2, -1):
+        y = oracle.softmax(x, dt, dim=dim, log=True)
+        got = oracle.to_f64(oracle.backwards_log_softmax(g, y, dt, dim=dim), dt)
+        t = torch.tensor(oracle.to_f64(x, dt), requires_grad=True)
+        torch.log_softmax(t, dim).backward(torch.tensor(oracle.to_f64(g, dt)))
+        tol = {F32: 2e-6, F64: 1e-13, F16: 4e-3, BF16: 3e-2}[dt]
+        np.testing.assert_allclose(got, t.grad.numpy(), rtol=tol * 10, atol=tol * 4)
+    # a gradient that is constant along the axis: gx = g (1 - n p), and the rows of gx sum to 0 when g sums against p... closed form on one row
+    yrow = oracle.softmax(oracle.to_storage(np.array([[0.0, np.log(3.0)]]), dt), dt, log=True)          # p = (1/4, 3/4)
+    gx = oracle.to_f64(oracle.backwards_log_softmax(oracle.to_storage(np.array([[1.0, 1.0]]), dt), yrow, dt), dt)
+    np.testing.assert_allclose(gx, [[1 - 2 * 0.25, 1 - 2 * 0.75]], rtol=2e-2 if dt in (F16, BF16) else 1e-6)
