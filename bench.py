@@ -142,6 +142,80 @@ def headline(capi, steps, warmup, n=8192, data="normal"):
     }
 
 
+def sustained(capi, seconds, data="normal", n=8192, period=0.2, dtype="bf16"):
+    """The forward 8192^3 bf16 GEMM launched back to back for `seconds` while a second thread polls the machine's SMI
+    tool (amd-smi, a separate process that opens no compute context) for the shader clock and the socket power: the figures that say whether
+    the part runs against its power limit on these operand values.  Returns TFLOP/s over the whole interval with the
+    mean / min / max of every quantity sampled."""
+    import subprocess
+    import threading
+    rng = np.random.default_rng(2)
+    dt = capi.BF16 if dtype == "bf16" else capi.F16
+    to_bits = _bf16_bits if dtype == "bf16" else (lambda x: x.astype(np.float16).view(np.uint16))
+    if data == "normal":
+        a, b = (to_bits(rng.standard_normal((n, n)).astype(np.float32)) for _ in range(2))
+    elif data == "ints":
+        a, b = (to_bits(rng.integers(-3, 4, (n, n)).astype(np.float32)) for _ in range(2))
+    else:
+        a, b = (to_bits(np.full((n, n), 1.0 if data == "ones" else 0.0, dtype=np.float32)) for _ in range(2))
+    d_a, d_b = (capi.DeviceBuffer.from_numpy(t) for t in (a, b))
+    d_c = capi.DeviceBuffer(n * n * 2)
+    rm = (0, n, 1)
+    fwd = lambda: capi.gemm(d_c.ptr, d_a.ptr, d_b.ptr, None, 1, n, n, n, rm, rm, rm, False, dt)
+    samples, stop = [], threading.Event()
+
+    def poll():
+        while not stop.is_set():
+            try:
+                txt = subprocess.run(["amd-smi", "metric", "-g", "0", "--power", "--clock", "--json"], capture_output=True, text=True, timeout=10).stdout
+                doc = json.loads(txt)
+                gpu = (doc.get("gpu_data") if isinstance(doc, dict) else doc)[0]
+                row = {}
+                power = gpu.get("power", {}).get("socket_power", {})
+                if isinstance(power, dict) and isinstance(power.get("value"), (int, float)):
+                    row["power_w"] = float(power["value"])
+                clocks = [c["clk"]["value"] for name, c in gpu.get("clock", {}).items()
+                          if name.startswith("gfx_") and isinstance(c, dict) and isinstance(c.get("clk", {}).get("value"), (int, float))]
+                if clocks:
+                    row["sclk_mhz"] = sum(clocks) / len(clocks)          # mean over the XCDs
+                if row:
+                    samples.append(row)
+            except Exception:
+                pass
+            stop.wait(period)
+
+    fwd(); capi.synchronize()
+    stream = capi.Stream()
+    reps = 25
+    with stream:
+        with capi.Graph.capture() as graph:
+            for _ in range(reps):
+                fwd()
+        graph.launch(); capi.check(capi.lib().rp_hip_stream_synchronize(), "sync")
+        th = threading.Thread(target=poll, daemon=True)
+        th.start()
+        time.sleep(0.3)
+        e0, e1 = capi.Event(), capi.Event()
+        launched, t0 = 0, time.perf_counter()
+        e0.record()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(4):
+                graph.launch()
+            launched += 4 * reps
+            capi.check(capi.lib().rp_hip_stream_synchronize(), "sync")      # keeps the queue a few graphs deep, not unbounded
+        e1.record(); e1.synchronize()
+        ms = e0.elapsed_ms(e1)
+        stop.set(); th.join(timeout=6)
+    out = {"dtype": dtype, "data": data, "seconds": round(ms * 1e-3, 2), "gemms": launched, "ms_per_gemm": ms / launched,
+           "TFLOP/s": 2.0 * n ** 3 * launched / ms / 1e9, "smi_samples": len(samples)}
+    busy = samples[2:] if len(samples) > 4 else samples               # the first polls may predate the clock ramp
+    for key in ("sclk_mhz", "power_w"):
+        vals = [r[key] for r in busy if key in r]
+        if vals:
+            out[key] = {"mean": round(sum(vals) / len(vals), 1), "min": min(vals), "max": max(vals)}
+    return out
+
+
 def cpu_baseline(a, b, target_s=15.0):
     """The reference's CPU path for the bf16 GEMM (functional/functional.c:986-1000: widen A and B to float32, the
     i-j-l loop of matmul_kernel_host_f32, narrow C) on a row slab of the 8192^3 GEMM, one core.  When the reference's
@@ -612,6 +686,12 @@ def main():
                     help="run only the conv2d layer's launches in bf16 (for profiling those kernels alone)")
     ap.add_argument("--mlp-only", action="store_true",
                     help="run only the configuration-2 MLP step (C ABI from a HIP graph, eager, and through the drop-in Python API)")
+    ap.add_argument("--sustain", type=float, default=0.0,
+                    help="run the forward 8192^3 bf16 GEMM back to back for this many seconds on --data operands while polling amd-smi "
+                         "for shader clock and socket power, and print those figures (evidence for the power-limit reading of the headline)")
+    ap.add_argument("--sustain-dtype", choices=["bf16", "f16"], default="bf16", help="16-bit type of the --sustain run")
+    ap.add_argument("--f16-only", action="store_true",
+                    help="run only the fp16 8192^3 forward GEMM (for profiling that kernel alone)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain copy kernel of known size (256 MiB in, 256 MiB out), the yardstick for FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
@@ -633,8 +713,14 @@ def main():
             capi.check(capi.lib().rp_hip_convert(dst.ptr, capi.F32, src.ptr, capi.F32, n), "copy")
         capi.synchronize()
         src.free(); dst.free()
+    if args.sustain > 0:
+        print(json.dumps({"sustained_gemm_8192": sustained(capi, args.sustain, args.data, dtype=args.sustain_dtype)}))
+        return
     if args.skinny_only:
-        print(json.dumps({"skinny": skinny_times(capi, rows=(1, 8))}))
+        print(json.dumps({"skinny": skinny_times(capi, rows=(1, 8, 32))}))
+        return
+    if args.f16_only:
+        print(json.dumps({"gemm_f16_8192": f16_time(capi)}))
         return
     if args.attention_only:
         print(json.dumps({"attention_bf16": attention_times(capi, "bf16")}))
