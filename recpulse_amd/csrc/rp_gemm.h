@@ -35,7 +35,7 @@ struct GemmArgs {
     int bias_by_row, c_fold_from, c_fold_to;
 };
 
-enum Family { FAM_GENERIC = 0, FAM_SKINNY, FAM_MFMA16, FAM_MFMA16_SKINNY, FAM_MFMAW, FAM_TINY, FAM_DIRECT32 };
+enum Family { FAM_GENERIC = 0, FAM_SKINNY, FAM_MFMA16, FAM_MFMA16_SKINNY, FAM_MFMAW, FAM_TINY, FAM_DIRECT32, FAM_STREAM32 };
 
 struct Plan {
     Family fam;
@@ -150,6 +150,8 @@ int launch_mfmaw(const GemmArgs& g, const Plan& p, int dtype);
 int launch_tiny(const GemmArgs& g, int dtype);
 bool direct32_takes(const GemmArgs& g);          // pointer alignment and spans the short-k fp32 kernel can address
 int launch_direct32(const GemmArgs& g);
+bool stream32_takes(const GemmArgs& g);          // options, alignment and spans the k-contiguous short-k fp32 kernel can address
+int launch_stream32(const GemmArgs& g);
 int launch_gemm_segmented_b(const GemmArgs& g, int dtype);
 int launch_linear_backward_tiny(const GemmArgs& gx, const GemmArgs& gw, void* db, const void* dy, int rows, int cols, int accumulate_db);
 // adds k-split partials [nsplit][part_rows][n] (fp32, rows beyond g.m unused) in split order and runs the epilogue into C

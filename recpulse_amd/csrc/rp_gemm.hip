@@ -81,6 +81,12 @@ static bool direct32_off() {                       // RP_HIP_NO_DIRECT32=1: shor
     return v == 1;
 }
 
+static bool stream32_off() {                       // RP_HIP_NO_STREAM32=1: k-contiguous short-k fp32 GEMMs keep the kernel that stages through registers
+    static int v = -1;
+    if (v < 0) { const char* e = getenv("RP_HIP_NO_STREAM32"); v = (e && e[0] == '1') ? 1 : 0; }
+    return v == 1;
+}
+
 static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long a_cs, long long b_rs, long long b_cs,
                       long long c_rs, long long c_cs, long long a_bs, long long b_bs, int dtype, bool allow_direct = true) {
     Plan p{FAM_GENERIC, 64, 64, false, false, true, "generic"};
@@ -135,6 +141,13 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
         p.fam = FAM_DIRECT32; p.bm = 128; p.bn = 128; p.a_mc = a_cs != 1; p.b_mc = b_rs != 1; p.name = "direct32_128x128";
         return p;
     }
+    // fp32 with k <= 64, both operands contiguous along k and at least one 128 x 128 tile per CU: one resident workgroup per
+    // CU whose fetching waves fill LDS directly and whose multiplying waves store the previous tile between the MFMAs
+    if (dtype == RP_DTYPE_FLOAT32 && allow_direct && !stream32_off() && k <= 64 && k % 4 == 0 && a_cs == 1 && b_rs == 1 && a_rs % 4 == 0 && b_cs % 4 == 0 &&
+        batch_ok && m > 64 && n > 64 && (long long)((m + 127) / 128) * ((n + 127) / 128) * batch >= 256) {
+        p.fam = FAM_STREAM32; p.bm = 128; p.bn = 128; p.a_mc = false; p.b_mc = false; p.edge = (m % 128) || (n % 128); p.name = "stream32_128x128";
+        return p;
+    }
     if (!mfma_ok) return p;
     p.a_mc = !a_kc;             // when both qualify (extent-1 corner cases) keep the row-major reading
     p.b_mc = b_mc;
@@ -154,6 +167,10 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
 
 static int run_gemm(const GemmArgs& g, int dtype) {
     Plan p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype);
+    if (p.fam == FAM_STREAM32) {
+        if (stream32_takes(g)) return launch_stream32(g);
+        p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype, false);     // options, base pointers or spans it does not take
+    }
     if (p.fam == FAM_DIRECT32) {
         if (direct32_takes(g)) return launch_direct32(g);
         p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype, false);     // base pointers or spans it cannot address

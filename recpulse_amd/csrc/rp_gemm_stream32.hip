@@ -1,0 +1,238 @@
+// fp32 GEMM with a short reduction (k <= 64) and both operands contiguous along k, e.g. S = Q.K^T per head.
+//
+// Such a product writes far more than it reads (512 x 512 outputs from 2 x 512 x 64 inputs), and per 128 x 128
+// tile the 64 KB of stores take about as long as the 128 MFMAs of a wave.  A block that multiplies, then stores,
+// then loads leaves the matrix pipe idle for more than half of the time, and a second block on the CU only fills
+// part of that.  Here one block of eight waves stays on each CU and walks its tiles with every phase overlapped:
+//
+//  - waves 4..7 only fetch.  A tile's rows of A and B (256 bytes each, zero-filled past k) go from memory straight
+//    into LDS (buffer loads with the LDS bit: no registers, 1 KB per instruction), two tiles of LDS in rotation, so
+//    tile t + 1 lands while tile t is multiplied.  A wave instruction fills four consecutive LDS rows; which 16-byte
+//    piece of the global row a lane fetches is the piece index XOR the row's low four bits, so that the 16 lanes
+//    that later read one piece index of 16 consecutive rows hit 16 different bank groups.
+//  - waves 0..3 only multiply and store.  Each owns a 64 x 64 patch (2 x 2 MFMA tiles of v_mfma_f32_32x32x2_f32)
+//    and two sets of accumulators: while tile t is accumulated into one set, the other set, tile t - 1, is stored,
+//    one store behind every second MFMA.  Lane (r, h) = (lane % 32, lane / 32) reads 16 bytes of its row from LDS
+//    for four MFMA steps: step (u, e) pairs k = 8u + e from the lanes with h = 0 and k = 8u + 4 + e from h = 1; A and
+//    B use the same pairing, and a sum over k does not care about the order.
+//
+// The two roles never wait for each other's memory operations: the fetching waves wait for loads only, the
+// multiplying waves issue stores only and never wait for them (a wave's loads and stores share one counter, and a
+// wait for a load would also wait for every younger store).  One block-wide barrier per tile hands a filled LDS tile
+// to the multipliers and an emptied one back.
+#include "rp_gemm.h"
+
+#include <type_traits>
+
+namespace rp {
+
+constexpr int S32_BM = 128, S32_BN = 128, S32_MAXK = 64;
+constexpr int S32_ROW_BYTES = 256;                                   // one LDS row: 64 floats
+constexpr int S32_TILE_BYTES = (S32_BM + S32_BN) * S32_ROW_BYTES;    // 64 KB: A rows, then B rows
+constexpr uint32_t S32_OOB = 0x80000000u;
+
+typedef __attribute__((address_space(3))) void* s32_lds_t;
+
+template <int I, int N, typename F>
+__device__ __forceinline__ void s32_static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        s32_static_for<I + 1, N>(f);
+    }
+}
+
+struct S32Tile {
+    int z, m0, n0;
+};
+
+__device__ __forceinline__ S32Tile s32_tile(long long id, int per_matrix, int tiles_n) {
+    S32Tile t;
+    t.z = (int)(id / per_matrix);
+    const int tile = (int)(id % per_matrix);
+    t.m0 = (tile / tiles_n) * S32_BM;
+    t.n0 = (tile % tiles_n) * S32_BN;
+    return t;
+}
+
+// (a bit cast applied directly to one element of a vector reads the wrong element with this compiler: pass the element by value)
+__device__ __forceinline__ uint32_t s32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t s32_rsrc(const void* base, long long span_bytes) {
+    const int n = span_bytes <= 0 ? 0 : (span_bytes > 0x7fffffffll ? 0x7fffffff : (int)span_bytes);
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, n, 0x00020000);
+}
+
+// KCH: 16-byte pieces of k per lane pair that are multiplied (8 for k <= 64, 4 for k <= 32); EDGE: m or n not whole tiles.
+template <int KCH, bool EDGE>
+__global__ void __launch_bounds__(512) gemm_stream32_kernel(GemmArgs g, int tiles_m, int tiles_n, long long total) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char s32_smem[];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int per_matrix = tiles_m * tiles_n;
+    const long long first = blockIdx.x, stride = gridDim.x;
+    const long long a_span = ((long long)(g.m - 1) * g.a_rs + g.k) * 4, b_span = ((long long)(g.n - 1) * g.b_cs + g.k) * 4;
+
+    if (wave >= 4) {
+        // ---- fetch: this wave brings rows [32p, 32p + 32) of A and of B for every tile ----
+        const int p = wave - 4;
+        uint32_t a_off[8], b_off[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const int row = 4 * q + (lane >> 4);                        // row within the wave's 32
+            const int piece = (lane & 15) ^ (row & 15);                 // which 16 bytes of the global row land in this lane's LDS slot
+            const bool in = piece * 4 < g.k;
+            a_off[q] = in ? (uint32_t)(((long long)row * g.a_rs + piece * 4) * 4) : S32_OOB;
+            b_off[q] = in ? (uint32_t)(((long long)row * g.b_cs + piece * 4) * 4) : S32_OOB;
+        }
+        auto fetch = [&](long long id, int buf) {
+            const S32Tile t = s32_tile(id, per_matrix, tiles_n);
+            const __amdgpu_buffer_rsrc_t ra = s32_rsrc((const float*)g.A + (long long)t.z * g.a_bs, a_span);
+            const __amdgpu_buffer_rsrc_t rb = s32_rsrc((const float*)g.B + (long long)t.z * g.b_bs, b_span);
+            const int sa = (int)((long long)(t.m0 + 32 * p) * g.a_rs * 4), sb = (int)((long long)(t.n0 + 32 * p) * g.b_cs * 4);
+            unsigned char* dst = s32_smem + buf * S32_TILE_BYTES + 32 * p * S32_ROW_BYTES;
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (s32_lds_t)(dst + q * 1024), 16, (int)a_off[q], sa, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (s32_lds_t)(dst + S32_BM * S32_ROW_BYTES + q * 1024), 16, (int)b_off[q], sb, 0, 0);
+            }
+        };
+        if (first < total) fetch(first, 0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        int buf = 0;
+        for (long long id = first; id < total; id += stride) {
+            if (id + stride < total) fetch(id + stride, buf ^ 1);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            buf ^= 1;
+        }
+        return;
+    }
+
+    // ---- multiply and store ----
+    const int r = lane & 31, h = lane >> 5;
+    const int wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * 64;
+    // LDS byte address of piece 2u + h of this lane's row: lane_a ^ (32 u) (rows are 256-byte aligned, so the XOR only
+    // touches the piece bits)
+    const uint32_t lane_a = (uint32_t)((wm0 + r) * S32_ROW_BYTES + ((h ^ (r & 15)) * 16));
+    const uint32_t lane_b = (uint32_t)(S32_BM * S32_ROW_BYTES + (wn0 + r) * S32_ROW_BYTES + ((h ^ (r & 15)) * 16));
+    const uint32_t c_lane = (uint32_t)(((long long)(4 * h) * g.c_rs + (long long)r * g.c_cs) * 4);
+    const long long c_span = ((long long)(g.m - 1) * g.c_rs + (long long)(g.n - 1) * g.c_cs + 1) * 4;
+
+    f32x16_t acc[2][2][2];              // [set][i][j]
+    f32x4_t af[2][2], bf[2][2];         // [slot][i or j]: four k values of the lane's row
+
+    // store number n (0..63) of accumulator set SET: register v of MFMA tile (i, j), i.e. columns 32j + r of rows 32i + 8(v / 4) + 4h + v % 4
+    auto store_one = [&](auto set_c, auto n_c, const S32Tile& t, const __amdgpu_buffer_rsrc_t& rc) {
+        constexpr int SET = decltype(set_c)::value, n = decltype(n_c)::value;
+        constexpr int sj = n >> 5, si = (n >> 4) & 1, v = n & 15;
+        constexpr int row = 32 * si + 8 * (v / 4) + (v % 4);
+        const int gm = t.m0 + wm0 + row, gn = t.n0 + wn0 + 32 * sj;
+        const int soff = (int)(((long long)gm * g.c_rs + (long long)gn * g.c_cs) * 4);
+        uint32_t voff = c_lane;
+        if constexpr (EDGE) voff = (gm + 4 * h < g.m && gn + r < g.n) ? c_lane : S32_OOB;
+        const float val = acc[SET][si][sj][v];
+        __builtin_amdgcn_raw_buffer_store_b32(s32_bits(val), rc, (int)voff, soff, 0);
+    };
+
+    // one tile: accumulate into set CUR from LDS tile `buf`; if STORE, write set CUR ^ 1 (the tile `prev`) meanwhile
+    auto tile_pass = [&](auto cur_c, auto store_c, int buf, const S32Tile& prev) {
+        constexpr int CUR = decltype(cur_c)::value;
+        constexpr bool STORE = decltype(store_c)::value;
+        const unsigned char* base = s32_smem + buf * S32_TILE_BYTES;
+        const __amdgpu_buffer_rsrc_t rc = s32_rsrc((float*)g.C + (long long)prev.z * g.c_bs, c_span);
+        auto read_frags = [&](int u, int slot) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) af[slot][i] = *(const f32x4_t*)(base + ((lane_a ^ (uint32_t)(32 * u)) + i * 32 * S32_ROW_BYTES));
+#pragma unroll
+            for (int j = 0; j < 2; j++) bf[slot][j] = *(const f32x4_t*)(base + ((lane_b ^ (uint32_t)(32 * u)) + j * 32 * S32_ROW_BYTES));
+        };
+        read_frags(0, 0);
+        s32_static_for<0, KCH>([&](auto uc) {
+            constexpr int u = decltype(uc)::value, slot = u & 1;
+            if constexpr (u + 1 < KCH) read_frags(u + 1, slot ^ 1);
+            s32_static_for<0, 16>([&](auto sc) {
+                constexpr int s = decltype(sc)::value, e = s >> 2, i = (s >> 1) & 1, j = s & 1;
+                if constexpr (u == 0 && e == 0) {
+                    const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                    acc[CUR][i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[slot][i][e], bf[slot][j][e], zero, 0, 0, 0);
+                } else {
+                    acc[CUR][i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[slot][i][e], bf[slot][j][e], acc[CUR][i][j], 0, 0, 0);
+                }
+                if constexpr (STORE) {
+                    // 64 stores over 16 * KCH MFMAs
+                    constexpr int PER = 64 / KCH;                        // stores per u: 8 or 16
+                    constexpr int EVERY = 16 / PER;                      // an MFMA in every EVERY carries one
+                    if constexpr (s % EVERY == EVERY - 1) store_one(std::integral_constant<int, CUR ^ 1>{}, std::integral_constant<int, u * PER + s / EVERY>{}, prev, rc);
+                    if constexpr (s % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+                }
+            });
+        });
+    };
+
+    __syncthreads();                                   // the first tile is in LDS
+    S32Tile prev = {0, 0, 0};
+    int buf = 0, last = 0;
+    long long id = first;
+    if (id >= total) return;
+    tile_pass(std::integral_constant<int, 0>{}, std::false_type{}, buf, prev);
+    prev = s32_tile(id, per_matrix, tiles_n);
+    __syncthreads();
+    buf ^= 1;
+    id += stride;
+    // two tiles per round, so that the accumulator sets are fixed registers
+    while (id < total) {
+        tile_pass(std::integral_constant<int, 1>{}, std::true_type{}, buf, prev);
+        prev = s32_tile(id, per_matrix, tiles_n);
+        __syncthreads();
+        buf ^= 1;
+        id += stride;
+        last = 1;
+        if (id >= total) break;
+        tile_pass(std::integral_constant<int, 0>{}, std::true_type{}, buf, prev);
+        prev = s32_tile(id, per_matrix, tiles_n);
+        __syncthreads();
+        buf ^= 1;
+        id += stride;
+        last = 0;
+    }
+    // the last tile's accumulators
+    const __amdgpu_buffer_rsrc_t rc = s32_rsrc((float*)g.C + (long long)prev.z * g.c_bs, c_span);
+    if (last == 0) s32_static_for<0, 64>([&](auto nc) { store_one(std::integral_constant<int, 0>{}, nc, prev, rc); });
+    else s32_static_for<0, 64>([&](auto nc) { store_one(std::integral_constant<int, 1>{}, nc, prev, rc); });
+}
+
+// ---- host side ----
+
+// Whether this kernel takes the product: fp32, k <= 64 in whole 16-byte pieces, both operands contiguous along k with
+// 16-byte aligned rows, C overwritten (no accumulation, bias, segments or folded store), and every byte offset the
+// kernel forms from a batch entry's base within the 32-bit range of buffer addressing.
+bool stream32_takes(const GemmArgs& g) {
+    if (g.k > S32_MAXK || g.k < 4 || g.k % 4 || g.m < 1 || g.n < 1 || g.batch < 1) return false;
+    if (g.bias || g.accumulate || g.seg_k || g.seg_n || g.c_fold_from || g.bias_by_row) return false;
+    if (g.a_cs != 1 || g.b_rs != 1 || g.a_rs % 4 || g.b_cs % 4 || g.a_bs % 4 || g.b_bs % 4 || g.a_rs < 0 || g.b_cs < 0 || g.c_rs < 0 || g.c_cs < 0) return false;
+    if (((uintptr_t)g.A & 15) || ((uintptr_t)g.B & 15) || ((uintptr_t)g.C & 3)) return false;
+    const long long lim = 1ll << 30;
+    // rows up to a whole tile past the last one are addressed (and read as zero or dropped by the range check)
+    const long long a_reach = ((long long)(g.m + S32_BM) * g.a_rs + S32_MAXK) * 4, b_reach = ((long long)(g.n + S32_BN) * g.b_cs + S32_MAXK) * 4;
+    const long long c_reach = ((long long)(g.m + S32_BM) * g.c_rs + (long long)(g.n + S32_BN) * g.c_cs) * 4;
+    return a_reach < lim && b_reach < lim && c_reach < lim;
+}
+
+int launch_stream32(const GemmArgs& g) {
+    const int tiles_m = (g.m + S32_BM - 1) / S32_BM, tiles_n = (g.n + S32_BN - 1) / S32_BN;
+    const long long total = (long long)tiles_m * tiles_n * g.batch;
+    int cus = device_cu_count();
+    if (cus <= 0) cus = 256;
+    const unsigned blocks = (unsigned)(total < cus ? total : cus);          // one resident workgroup per CU walks its tiles
+    const bool edge = (g.m % S32_BM) || (g.n % S32_BN);
+    constexpr int smem = 2 * S32_TILE_BYTES;
+    auto launch = [&](auto kern) {
+        if (!check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem), "hipFuncSetAttribute")) return -1;
+        hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), smem, current_stream(), g, tiles_m, tiles_n, total);
+        return check_launch("gemm_stream32_kernel") ? 0 : -1;
+    };
+    if (g.k <= 32) return edge ? launch(gemm_stream32_kernel<4, true>) : launch(gemm_stream32_kernel<4, false>);
+    return edge ? launch(gemm_stream32_kernel<8, true>) : launch(gemm_stream32_kernel<8, false>);
+}
+
+}  // namespace rp

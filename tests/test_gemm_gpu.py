@@ -413,10 +413,57 @@ def test_fp32_short_reduction_batched(layout, batch, m, k, n):
     _check(got, a, b, F32, k, bias=bias, c_init=c0, accumulate=True)
 
 
+# ---- fp32, k <= 64, both operands contiguous along k, at least one 128 x 128 tile per CU: the resident kernel whose
+# fetching waves fill LDS directly and whose multiplying waves store the previous tile between the MFMAs
+STREAM32_SHAPES = [(16, 512, 64, 512), (20, 500, 64, 456), (48, 250, 44, 300), (32, 384, 36, 512), (70, 256, 20, 256), (300, 130, 8, 129), (260, 128, 32, 128),
+                   (1, 2048, 64, 2048), (3, 1100, 60, 1300)]
+
+
+@pytest.mark.parametrize("batch,m,k,n", STREAM32_SHAPES)
+def test_fp32_stream_kernel_k_contiguous(batch, m, k, n):
+    rng = np.random.default_rng(63)
+    a = rand_storage(rng, (batch, m, k), F32)
+    b = rand_storage(rng, (batch, n, k), F32).transpose(0, 2, 1)
+    assert capi.gemm_kernel_name(batch, m, k, n, (k, 1), (1, k), (n, 1), F32) == "stream32_128x128"
+    got = device_gemm(a, b, F32)
+    _check(got, a, b, F32, k)
+    # a bias or an accumulated C is not this kernel's: the same call must still be right through the one that takes over
+    bias = rand_storage(rng, (n,), F32)
+    c0 = rand_storage(rng, (batch, m, n), F32)
+    got = device_gemm(a, b, F32, bias=bias, c_init=c0, accumulate=True)
+    _check(got, a, b, F32, k, bias=bias, c_init=c0, accumulate=True)
+
+
+def test_fp32_stream_kernel_views_and_strided_output():
+    """Rows that are slices of wider arrays (row pitch above k), a batch stride that skips entries, and C written through
+    row / column strides of a transposed, padded output: nothing outside the addressed elements may change."""
+    rng = np.random.default_rng(64)
+    batch, m, k, n = 24, 384, 48, 512
+    wide_a = rand_storage(rng, (2 * batch, m, 80), F32)
+    wide_b = rand_storage(rng, (batch, n, 96), F32)
+    a = wide_a[::2, :, 16:16 + k]                              # every other batch entry, columns 16..63 of 80
+    b = wide_b[:, :, 32:32 + k].transpose(0, 2, 1)
+    assert capi.gemm_kernel_name(batch, m, k, n, (80, 1), (1, 96), (n, 1), F32) == "stream32_128x128"
+    got = device_gemm(a, b, F32)
+    _check(got, a, b, F32, k)
+    # C[z] stored transposed inside a padded [n + 3, m + 5] plane
+    pitch = m + 5
+    plane = (n + 3) * pitch
+    c0 = rand_storage(rng, (batch, n + 3, pitch), F32)
+    da, db, dc = capi.DeviceBuffer.from_numpy(wide_a), capi.DeviceBuffer.from_numpy(wide_b), capi.DeviceBuffer.from_numpy(c0)
+    capi.gemm(dc.ptr, da.at(16 * 4), db.at(32 * 4), None, batch, m, k, n, (2 * m * 80, 80, 1), (n * 96, 1, 96), (plane, 1, pitch), False, F32)
+    capi.synchronize()
+    out = dc.to_numpy(np.float32, (batch, n + 3, pitch))
+    for d in (da, db, dc):
+        d.free()
+    assert np.array_equal(out[:, :n, :m], got.transpose(0, 2, 1))
+    assert np.array_equal(out[:, n:, :], c0[:, n:, :]) and np.array_equal(out[:, :, m:], c0[:, :, m:])
+
+
 def test_fp32_short_reduction_integers_bit_exact():
     """Small integers: every partial sum is exact, so the product must equal the oracle's bit for bit in any summation order."""
     rng = np.random.default_rng(62)
-    batch, m, k, n = 8, 512, 64, 512
+    batch, m, k, n = 16, 512, 64, 512
     for layout in LAYOUTS:
         a = rng.integers(-3, 4, (batch, m, k) if layout[0] == "n" else (batch, k, m)).astype(np.float32)
         b = rng.integers(-3, 4, (batch, k, n) if layout[1] == "n" else (batch, n, k)).astype(np.float32)
