@@ -35,7 +35,7 @@ struct GemmArgs {
     int bias_by_row, c_fold_from, c_fold_to;
 };
 
-enum Family { FAM_GENERIC = 0, FAM_SKINNY, FAM_MFMA16, FAM_MFMA16_SKINNY, FAM_MFMAW, FAM_TINY, FAM_DIRECT32, FAM_STREAM32 };
+enum Family { FAM_GENERIC = 0, FAM_SKINNY, FAM_MFMA16, FAM_MFMA16_SKINNY, FAM_MFMAW, FAM_TINY, FAM_DIRECT32, FAM_PIPE32, FAM_PIPE16 };
 
 struct Plan {
     Family fam;
@@ -56,6 +56,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(4))) double f64x4_t;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2_t;
 
 // Tile scheduling shared by the MFMA kernels.
 // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2), so a
@@ -150,8 +151,10 @@ int launch_mfmaw(const GemmArgs& g, const Plan& p, int dtype);
 int launch_tiny(const GemmArgs& g, int dtype);
 bool direct32_takes(const GemmArgs& g);          // pointer alignment and spans the short-k fp32 kernel can address
 int launch_direct32(const GemmArgs& g);
-bool stream32_takes(const GemmArgs& g);          // options, alignment and spans the k-contiguous short-k fp32 kernel can address
-int launch_stream32(const GemmArgs& g);
+bool pipe32_takes(const GemmArgs& g);          // options, alignment and spans the k-contiguous short-k fp32 kernel can address
+int launch_pipe32(const GemmArgs& g);
+bool pipe16_takes(const GemmArgs& g);          // the same for the 16-bit kernel (C row-major in whole 8-byte quads)
+int launch_pipe16(const GemmArgs& g, int dtype);
 int launch_gemm_segmented_b(const GemmArgs& g, int dtype);
 int launch_linear_backward_tiny(const GemmArgs& gx, const GemmArgs& gw, void* db, const void* dy, int rows, int cols, int accumulate_db);
 // adds k-split partials [nsplit][part_rows][n] (fp32, rows beyond g.m unused) in split order and runs the epilogue into C

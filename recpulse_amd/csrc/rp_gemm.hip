@@ -81,9 +81,15 @@ static bool direct32_off() {                       // RP_HIP_NO_DIRECT32=1: shor
     return v == 1;
 }
 
-static bool stream32_off() {                       // RP_HIP_NO_STREAM32=1: k-contiguous short-k fp32 GEMMs keep the kernel that stages through registers
+static bool pipe32_off() {                       // RP_HIP_NO_PIPE32=1: k-contiguous short-k fp32 GEMMs keep the kernel that stages through registers
     static int v = -1;
-    if (v < 0) { const char* e = getenv("RP_HIP_NO_STREAM32"); v = (e && e[0] == '1') ? 1 : 0; }
+    if (v < 0) { const char* e = getenv("RP_HIP_NO_PIPE32"); v = (e && e[0] == '1') ? 1 : 0; }
+    return v == 1;
+}
+
+static bool pipe16_off() {                       // RP_HIP_NO_PIPE16=1: the same for the 16-bit kernel
+    static int v = -1;
+    if (v < 0) { const char* e = getenv("RP_HIP_NO_PIPE16"); v = (e && e[0] == '1') ? 1 : 0; }
     return v == 1;
 }
 
@@ -99,7 +105,6 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     bool b_mc = (b_cs == 1) && (b_rs % vec == 0) && (n % vec == 0);
     bool b_kc = (b_rs == 1) && (b_cs % vec == 0) && (k % vec == 0);
     bool batch_ok = (batch == 1) || ((a_bs % vec == 0) && (b_bs % vec == 0));
-    (void)c_rs; (void)c_cs;
 
     // the MFMA kernels address a tile with 32-bit byte offsets from a 64-bit tile pointer
     const long long max_stride = 1ll << 22;
@@ -143,9 +148,15 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     }
     // fp32 with k <= 64, both operands contiguous along k and at least one 128 x 128 tile per CU: one resident workgroup per
     // CU whose fetching waves fill LDS directly and whose multiplying waves store the previous tile between the MFMAs
-    if (dtype == RP_DTYPE_FLOAT32 && allow_direct && !stream32_off() && k <= 64 && k % 4 == 0 && a_cs == 1 && b_rs == 1 && a_rs % 4 == 0 && b_cs % 4 == 0 &&
+    if (dtype == RP_DTYPE_FLOAT32 && allow_direct && !pipe32_off() && k <= 64 && k % 4 == 0 && a_cs == 1 && b_rs == 1 && a_rs % 4 == 0 && b_cs % 4 == 0 &&
         batch_ok && m > 64 && n > 64 && (long long)((m + 127) / 128) * ((n + 127) / 128) * batch >= 256) {
-        p.fam = FAM_STREAM32; p.bm = 128; p.bn = 128; p.a_mc = false; p.b_mc = false; p.edge = (m % 128) || (n % 128); p.name = "stream32_128x128";
+        p.fam = FAM_PIPE32; p.bm = 128; p.bn = 128; p.a_mc = false; p.b_mc = false; p.edge = (m % 128) || (n % 128); p.name = "pipe32_128x128";
+        return p;
+    }
+    // the same for bf16 / fp16 (C row-major): there the stores and the narrowing are what takes time
+    if (is16 && allow_direct && !pipe16_off() && k <= 64 && k % 8 == 0 && a_cs == 1 && b_rs == 1 && a_rs % 8 == 0 && b_cs % 8 == 0 && batch_ok &&
+        c_cs == 1 && c_rs % 8 == 0 && n % 8 == 0 && m > 64 && n > 64 && (long long)((m + 127) / 128) * ((n + 127) / 128) * batch >= 256) {
+        p.fam = FAM_PIPE16; p.bm = 128; p.bn = 128; p.a_mc = false; p.b_mc = false; p.edge = (m % 128) || (n % 128); p.name = "pipe16_128x128";
         return p;
     }
     if (!mfma_ok) return p;
@@ -167,9 +178,13 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
 
 static int run_gemm(const GemmArgs& g, int dtype) {
     Plan p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype);
-    if (p.fam == FAM_STREAM32) {
-        if (stream32_takes(g)) return launch_stream32(g);
+    if (p.fam == FAM_PIPE32) {
+        if (pipe32_takes(g)) return launch_pipe32(g);
         p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype, false);     // options, base pointers or spans it does not take
+    }
+    if (p.fam == FAM_PIPE16) {
+        if (pipe16_takes(g)) return launch_pipe16(g, dtype);
+        p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype, false);
     }
     if (p.fam == FAM_DIRECT32) {
         if (direct32_takes(g)) return launch_direct32(g);

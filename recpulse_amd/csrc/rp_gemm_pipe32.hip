@@ -45,12 +45,12 @@ struct S32Tile {
     int z, m0, n0;
 };
 
-__device__ __forceinline__ S32Tile s32_tile(long long id, int per_matrix, int tiles_n) {
+__device__ __forceinline__ S32Tile s32_tile(unsigned id, unsigned per_matrix, unsigned tiles_n) {
     S32Tile t;
-    t.z = (int)(id / per_matrix);
-    const int tile = (int)(id % per_matrix);
-    t.m0 = (tile / tiles_n) * S32_BM;
-    t.n0 = (tile % tiles_n) * S32_BN;
+    const unsigned z = id / per_matrix, tile = id - z * per_matrix, tm = tile / tiles_n;
+    t.z = (int)z;
+    t.m0 = (int)tm * S32_BM;
+    t.n0 = (int)(tile - tm * tiles_n) * S32_BN;
     return t;
 }
 
@@ -64,11 +64,11 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t s32_rsrc(const void* base, lon
 
 // KCH: 16-byte pieces of k per lane pair that are multiplied (8 for k <= 64, 4 for k <= 32); EDGE: m or n not whole tiles.
 template <int KCH, bool EDGE>
-__global__ void __launch_bounds__(512) gemm_stream32_kernel(GemmArgs g, int tiles_m, int tiles_n, long long total) {
-    extern __shared__ __attribute__((aligned(1024))) unsigned char s32_smem[];
+__global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_m, int tiles_n, unsigned total) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char p32_smem[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int per_matrix = tiles_m * tiles_n;
-    const long long first = blockIdx.x, stride = gridDim.x;
+    const unsigned per_matrix = (unsigned)(tiles_m * tiles_n);
+    const unsigned first = blockIdx.x, stride = gridDim.x;          // (tile numbers stay below 2^31: first + stride cannot wrap)
     const long long a_span = ((long long)(g.m - 1) * g.a_rs + g.k) * 4, b_span = ((long long)(g.n - 1) * g.b_cs + g.k) * 4;
 
     if (wave >= 4) {
@@ -83,12 +83,12 @@ __global__ void __launch_bounds__(512) gemm_stream32_kernel(GemmArgs g, int tile
             a_off[q] = in ? (uint32_t)(((long long)row * g.a_rs + piece * 4) * 4) : S32_OOB;
             b_off[q] = in ? (uint32_t)(((long long)row * g.b_cs + piece * 4) * 4) : S32_OOB;
         }
-        auto fetch = [&](long long id, int buf) {
+        auto fetch = [&](unsigned id, int buf) {
             const S32Tile t = s32_tile(id, per_matrix, tiles_n);
             const __amdgpu_buffer_rsrc_t ra = s32_rsrc((const float*)g.A + (long long)t.z * g.a_bs, a_span);
             const __amdgpu_buffer_rsrc_t rb = s32_rsrc((const float*)g.B + (long long)t.z * g.b_bs, b_span);
             const int sa = (int)((long long)(t.m0 + 32 * p) * g.a_rs * 4), sb = (int)((long long)(t.n0 + 32 * p) * g.b_cs * 4);
-            unsigned char* dst = s32_smem + buf * S32_TILE_BYTES + 32 * p * S32_ROW_BYTES;
+            unsigned char* dst = p32_smem + buf * S32_TILE_BYTES + 32 * p * S32_ROW_BYTES;
 #pragma unroll
             for (int q = 0; q < 8; q++) {
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (s32_lds_t)(dst + q * 1024), 16, (int)a_off[q], sa, 0, 0);
@@ -99,7 +99,7 @@ __global__ void __launch_bounds__(512) gemm_stream32_kernel(GemmArgs g, int tile
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         int buf = 0;
-        for (long long id = first; id < total; id += stride) {
+        for (unsigned id = first; id < total; id += stride) {
             if (id + stride < total) fetch(id + stride, buf ^ 1);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
@@ -134,22 +134,31 @@ __global__ void __launch_bounds__(512) gemm_stream32_kernel(GemmArgs g, int tile
         __builtin_amdgcn_raw_buffer_store_b32(s32_bits(val), rc, (int)voff, soff, 0);
     };
 
-    // one tile: accumulate into set CUR from LDS tile `buf`; if STORE, write set CUR ^ 1 (the tile `prev`) meanwhile
+    auto read_frags = [&](const unsigned char* base, int u, int slot) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) af[slot][i] = *(const f32x4_t*)(base + ((lane_a ^ (uint32_t)(32 * u)) + i * 32 * S32_ROW_BYTES));
+#pragma unroll
+        for (int j = 0; j < 2; j++) bf[slot][j] = *(const f32x4_t*)(base + ((lane_b ^ (uint32_t)(32 * u)) + j * 32 * S32_ROW_BYTES));
+    };
+
+    // One tile: accumulate into set CUR from LDS tile `buf` (whose first pieces are already in fragment slot 0); if STORE,
+    // write set CUR ^ 1 (the tile `prev`) meanwhile.  The block's barrier sits before the last piece's MFMAs, when every
+    // LDS read of this tile has returned: behind it the other LDS tile holds the next tile, whose first pieces are read
+    // under those MFMAs, and the fetching waves may overwrite this one.
     auto tile_pass = [&](auto cur_c, auto store_c, int buf, const S32Tile& prev) {
         constexpr int CUR = decltype(cur_c)::value;
         constexpr bool STORE = decltype(store_c)::value;
-        const unsigned char* base = s32_smem + buf * S32_TILE_BYTES;
+        const unsigned char* base = p32_smem + buf * S32_TILE_BYTES;
+        const unsigned char* next_base = p32_smem + (buf ^ 1) * S32_TILE_BYTES;
         const __amdgpu_buffer_rsrc_t rc = s32_rsrc((float*)g.C + (long long)prev.z * g.c_bs, c_span);
-        auto read_frags = [&](int u, int slot) {
-#pragma unroll
-            for (int i = 0; i < 2; i++) af[slot][i] = *(const f32x4_t*)(base + ((lane_a ^ (uint32_t)(32 * u)) + i * 32 * S32_ROW_BYTES));
-#pragma unroll
-            for (int j = 0; j < 2; j++) bf[slot][j] = *(const f32x4_t*)(base + ((lane_b ^ (uint32_t)(32 * u)) + j * 32 * S32_ROW_BYTES));
-        };
-        read_frags(0, 0);
         s32_static_for<0, KCH>([&](auto uc) {
             constexpr int u = decltype(uc)::value, slot = u & 1;
-            if constexpr (u + 1 < KCH) read_frags(u + 1, slot ^ 1);
+            if constexpr (u + 1 < KCH) {
+                read_frags(base, u + 1, slot ^ 1);
+            } else {
+                __syncthreads();
+                read_frags(next_base, 0, slot ^ 1);
+            }
             s32_static_for<0, 16>([&](auto sc) {
                 constexpr int s = decltype(sc)::value, e = s >> 2, i = (s >> 1) & 1, j = s & 1;
                 if constexpr (u == 0 && e == 0) {
@@ -172,25 +181,23 @@ __global__ void __launch_bounds__(512) gemm_stream32_kernel(GemmArgs g, int tile
     __syncthreads();                                   // the first tile is in LDS
     S32Tile prev = {0, 0, 0};
     int buf = 0, last = 0;
-    long long id = first;
+    unsigned id = first;
     if (id >= total) return;
+    read_frags(p32_smem, 0, 0);
     tile_pass(std::integral_constant<int, 0>{}, std::false_type{}, buf, prev);
     prev = s32_tile(id, per_matrix, tiles_n);
-    __syncthreads();
     buf ^= 1;
     id += stride;
     // two tiles per round, so that the accumulator sets are fixed registers
     while (id < total) {
         tile_pass(std::integral_constant<int, 1>{}, std::true_type{}, buf, prev);
         prev = s32_tile(id, per_matrix, tiles_n);
-        __syncthreads();
         buf ^= 1;
         id += stride;
         last = 1;
         if (id >= total) break;
         tile_pass(std::integral_constant<int, 0>{}, std::true_type{}, buf, prev);
         prev = s32_tile(id, per_matrix, tiles_n);
-        __syncthreads();
         buf ^= 1;
         id += stride;
         last = 0;
@@ -206,8 +213,9 @@ __global__ void __launch_bounds__(512) gemm_stream32_kernel(GemmArgs g, int tile
 // Whether this kernel takes the product: fp32, k <= 64 in whole 16-byte pieces, both operands contiguous along k with
 // 16-byte aligned rows, C overwritten (no accumulation, bias, segments or folded store), and every byte offset the
 // kernel forms from a batch entry's base within the 32-bit range of buffer addressing.
-bool stream32_takes(const GemmArgs& g) {
+bool pipe32_takes(const GemmArgs& g) {
     if (g.k > S32_MAXK || g.k < 4 || g.k % 4 || g.m < 1 || g.n < 1 || g.batch < 1) return false;
+    if ((long long)((g.m + S32_BM - 1) / S32_BM) * ((g.n + S32_BN - 1) / S32_BN) * g.batch >= (1ll << 30)) return false;
     if (g.bias || g.accumulate || g.seg_k || g.seg_n || g.c_fold_from || g.bias_by_row) return false;
     if (g.a_cs != 1 || g.b_rs != 1 || g.a_rs % 4 || g.b_cs % 4 || g.a_bs % 4 || g.b_bs % 4 || g.a_rs < 0 || g.b_cs < 0 || g.c_rs < 0 || g.c_cs < 0) return false;
     if (((uintptr_t)g.A & 15) || ((uintptr_t)g.B & 15) || ((uintptr_t)g.C & 3)) return false;
@@ -218,7 +226,7 @@ bool stream32_takes(const GemmArgs& g) {
     return a_reach < lim && b_reach < lim && c_reach < lim;
 }
 
-int launch_stream32(const GemmArgs& g) {
+int launch_pipe32(const GemmArgs& g) {
     const int tiles_m = (g.m + S32_BM - 1) / S32_BM, tiles_n = (g.n + S32_BN - 1) / S32_BN;
     const long long total = (long long)tiles_m * tiles_n * g.batch;
     int cus = device_cu_count();
@@ -228,11 +236,11 @@ int launch_stream32(const GemmArgs& g) {
     constexpr int smem = 2 * S32_TILE_BYTES;
     auto launch = [&](auto kern) {
         if (!check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem), "hipFuncSetAttribute")) return -1;
-        hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), smem, current_stream(), g, tiles_m, tiles_n, total);
-        return check_launch("gemm_stream32_kernel") ? 0 : -1;
+        hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), smem, current_stream(), g, tiles_m, tiles_n, (unsigned)total);
+        return check_launch("gemm_pipe32_kernel") ? 0 : -1;
     };
-    if (g.k <= 32) return edge ? launch(gemm_stream32_kernel<4, true>) : launch(gemm_stream32_kernel<4, false>);
-    return edge ? launch(gemm_stream32_kernel<8, true>) : launch(gemm_stream32_kernel<8, false>);
+    if (g.k <= 32) return edge ? launch(gemm_pipe32_kernel<4, true>) : launch(gemm_pipe32_kernel<4, false>);
+    return edge ? launch(gemm_pipe32_kernel<8, true>) : launch(gemm_pipe32_kernel<8, false>);
 }
 
 }  // namespace rp

@@ -60,6 +60,7 @@ def test_matmul_kernel_device_seam_f64_parity_shapes():
 
 
 LAYOUTS = ["nn", "nt", "tn", "tt"]
+HALF = [F16, BF16]
 
 
 def _operands(rng, m, k, n, dt, layout, dist="normal"):
@@ -415,16 +416,16 @@ def test_fp32_short_reduction_batched(layout, batch, m, k, n):
 
 # ---- fp32, k <= 64, both operands contiguous along k, at least one 128 x 128 tile per CU: the resident kernel whose
 # fetching waves fill LDS directly and whose multiplying waves store the previous tile between the MFMAs
-STREAM32_SHAPES = [(16, 512, 64, 512), (20, 500, 64, 456), (48, 250, 44, 300), (32, 384, 36, 512), (70, 256, 20, 256), (300, 130, 8, 129), (260, 128, 32, 128),
+PIPE32_SHAPES = [(16, 512, 64, 512), (20, 500, 64, 456), (48, 250, 44, 300), (32, 384, 36, 512), (70, 256, 20, 256), (300, 130, 8, 129), (260, 128, 32, 128),
                    (1, 2048, 64, 2048), (3, 1100, 60, 1300)]
 
 
-@pytest.mark.parametrize("batch,m,k,n", STREAM32_SHAPES)
-def test_fp32_stream_kernel_k_contiguous(batch, m, k, n):
+@pytest.mark.parametrize("batch,m,k,n", PIPE32_SHAPES)
+def test_fp32_pipelined_kernel_k_contiguous(batch, m, k, n):
     rng = np.random.default_rng(63)
     a = rand_storage(rng, (batch, m, k), F32)
     b = rand_storage(rng, (batch, n, k), F32).transpose(0, 2, 1)
-    assert capi.gemm_kernel_name(batch, m, k, n, (k, 1), (1, k), (n, 1), F32) == "stream32_128x128"
+    assert capi.gemm_kernel_name(batch, m, k, n, (k, 1), (1, k), (n, 1), F32) == "pipe32_128x128"
     got = device_gemm(a, b, F32)
     _check(got, a, b, F32, k)
     # a bias or an accumulated C is not this kernel's: the same call must still be right through the one that takes over
@@ -434,7 +435,7 @@ def test_fp32_stream_kernel_k_contiguous(batch, m, k, n):
     _check(got, a, b, F32, k, bias=bias, c_init=c0, accumulate=True)
 
 
-def test_fp32_stream_kernel_views_and_strided_output():
+def test_fp32_pipelined_kernel_views_and_strided_output():
     """Rows that are slices of wider arrays (row pitch above k), a batch stride that skips entries, and C written through
     row / column strides of a transposed, padded output: nothing outside the addressed elements may change."""
     rng = np.random.default_rng(64)
@@ -443,7 +444,7 @@ def test_fp32_stream_kernel_views_and_strided_output():
     wide_b = rand_storage(rng, (batch, n, 96), F32)
     a = wide_a[::2, :, 16:16 + k]                              # every other batch entry, columns 16..63 of 80
     b = wide_b[:, :, 32:32 + k].transpose(0, 2, 1)
-    assert capi.gemm_kernel_name(batch, m, k, n, (80, 1), (1, 96), (n, 1), F32) == "stream32_128x128"
+    assert capi.gemm_kernel_name(batch, m, k, n, (80, 1), (1, 96), (n, 1), F32) == "pipe32_128x128"
     got = device_gemm(a, b, F32)
     _check(got, a, b, F32, k)
     # C[z] stored transposed inside a padded [n + 3, m + 5] plane
@@ -458,6 +459,49 @@ def test_fp32_stream_kernel_views_and_strided_output():
         d.free()
     assert np.array_equal(out[:, :n, :m], got.transpose(0, 2, 1))
     assert np.array_equal(out[:, n:, :], c0[:, n:, :]) and np.array_equal(out[:, :, m:], c0[:, :, m:])
+
+
+# ---- the same for bf16 / fp16 (C row-major, n in whole eights): narrowing and stores between the MFMAs of the next tile
+PIPE16_SHAPES = [(16, 512, 64, 512), (20, 500, 64, 456), (48, 250, 40, 296), (32, 384, 32, 512), (70, 256, 16, 256), (300, 130, 8, 136), (3, 1100, 56, 1304)]
+
+
+@pytest.mark.parametrize("dt", HALF, ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("batch,m,k,n", PIPE16_SHAPES)
+def test_16bit_pipelined_kernel_k_contiguous(batch, m, k, n, dt):
+    rng = np.random.default_rng(65)
+    a = rand_storage(rng, (batch, m, k), dt)
+    b = rand_storage(rng, (batch, n, k), dt).transpose(0, 2, 1)
+    assert capi.gemm_kernel_name(batch, m, k, n, (k, 1), (1, k), (n, 1), dt) == "pipe16_128x128"
+    got = device_gemm(a, b, dt)
+    _check(got, a, b, dt, k)
+    bias = rand_storage(rng, (n,), dt)
+    c0 = rand_storage(rng, (batch, m, n), dt)
+    got = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)          # not this kernel's: through the one that takes over
+    _check(got, a, b, dt, k, bias=bias, c_init=c0, accumulate=True)
+
+
+@pytest.mark.parametrize("dt", HALF, ids=lambda d: NAMES[d])
+def test_16bit_pipelined_kernel_bit_exact_and_padded_rows(dt):
+    """Small integers (every sum exact, so any order gives the oracle's bits), operands that are slices of wider arrays,
+    and C with a row pitch above n: nothing outside the addressed elements may change."""
+    rng = np.random.default_rng(66)
+    batch, m, k, n = 24, 384, 48, 504
+    wide_a = oracle.to_storage(rng.integers(-3, 4, (2 * batch, m, 80)).astype(np.float64), dt)
+    wide_b = oracle.to_storage(rng.integers(-3, 4, (batch, n, 96)).astype(np.float64), dt)
+    a = wide_a[::2, :, 16:16 + k]
+    b = wide_b[:, :, 32:32 + k].transpose(0, 2, 1)
+    want = np.matmul(oracle.to_f64(np.ascontiguousarray(a), dt), oracle.to_f64(np.ascontiguousarray(b), dt))
+    pitch = n + 16
+    c0 = rand_storage(rng, (batch, m + 2, pitch), dt)
+    da, db, dc = capi.DeviceBuffer.from_numpy(wide_a), capi.DeviceBuffer.from_numpy(wide_b), capi.DeviceBuffer.from_numpy(c0)
+    assert capi.gemm_kernel_name(batch, m, k, n, (80, 1), (1, 96), (pitch, 1), dt) == "pipe16_128x128"
+    capi.gemm(dc.ptr, da.at(16 * 2), db.at(32 * 2), None, batch, m, k, n, (2 * m * 80, 80, 1), (n * 96, 1, 96), ((m + 2) * pitch, pitch, 1), False, dt)
+    capi.synchronize()
+    out = dc.to_numpy(capi.NP_STORAGE[dt], (batch, m + 2, pitch))
+    for d in (da, db, dc):
+        d.free()
+    assert np.array_equal(oracle.to_f64(out[:, :m, :n], dt), want)
+    assert np.array_equal(out[:, m:, :], c0[:, m:, :]) and np.array_equal(out[:, :, n:], c0[:, :, n:])
 
 
 def test_fp32_short_reduction_integers_bit_exact():
