@@ -93,6 +93,12 @@ static bool pipe16_off() {                       // RP_HIP_NO_PIPE16=1: the same
     return v == 1;
 }
 
+static bool pipe16k_off() {                        // RP_HIP_NO_PIPE16K=1: narrow 16-bit outputs keep the general tiled kernel
+    static int v = -1;
+    if (v < 0) { const char* e = getenv("RP_HIP_NO_PIPE16K"); v = (e && e[0] == '1') ? 1 : 0; }
+    return v == 1;
+}
+
 static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long a_cs, long long b_rs, long long b_cs,
                       long long c_rs, long long c_cs, long long a_bs, long long b_bs, int dtype, bool allow_direct = true) {
     Plan p{FAM_GENERIC, 64, 64, false, false, true, "generic"};
@@ -159,6 +165,13 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
         p.fam = FAM_PIPE16; p.bm = 128; p.bn = 128; p.a_mc = false; p.b_mc = false; p.edge = (m % 128) || (n % 128); p.name = "pipe16_128x128";
         return p;
     }
+    // bf16 / fp16, at most 64 output columns, at least one 128-row tile per CU (O = P.V per head, a tall matrix times a narrow
+    // one): bound by reading A; the resident kernel whose fetching waves keep three k slabs in flight into LDS
+    if (is16 && allow_direct && !pipe16k_off() && n <= 64 && n % 8 == 0 && k % 8 == 0 && k >= 64 && (a_kc || a_mc) && (b_kc || b_mc) && batch_ok &&
+        c_cs == 1 && c_rs % 8 == 0 && m > 64 && (long long)((m + 127) / 128) * batch >= 256) {
+        p.fam = FAM_PIPE16K; p.bm = 128; p.bn = 64; p.a_mc = !a_kc; p.b_mc = !b_kc; p.edge = (m % 128) || n != 64; p.name = "pipe16k_128x64";
+        return p;
+    }
     if (!mfma_ok) return p;
     p.a_mc = !a_kc;             // when both qualify (extent-1 corner cases) keep the row-major reading
     p.b_mc = b_mc;
@@ -184,6 +197,10 @@ static int run_gemm(const GemmArgs& g, int dtype) {
     }
     if (p.fam == FAM_PIPE16) {
         if (pipe16_takes(g)) return launch_pipe16(g, dtype);
+        p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype, false);
+    }
+    if (p.fam == FAM_PIPE16K) {
+        if (pipe16k_takes(g)) return launch_pipe16k(g, dtype);
         p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype, false);
     }
     if (p.fam == FAM_DIRECT32) {

@@ -504,6 +504,57 @@ def test_16bit_pipelined_kernel_bit_exact_and_padded_rows(dt):
     assert np.array_equal(out[:, m:, :], c0[:, m:, :]) and np.array_equal(out[:, :, n:], c0[:, :, n:])
 
 
+# ---- bf16 / fp16 outputs of at most 64 columns with at least one 128-row tile per CU: the resident kernel that streams k
+# slabs of A and B into LDS, every operand layout, ragged m, n below 64, k that ends inside a slab
+PIPE16K_SHAPES = [(64, 512, 512, 64), (70, 504, 200, 40), (300, 136, 72, 64), (1, 32768, 96, 56), (130, 256, 64, 64), (33, 1000, 328, 8)]
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("dt", HALF, ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("batch,m,k,n", PIPE16K_SHAPES)
+def test_16bit_narrow_output_kernel(batch, m, k, n, dt, layout):
+    rng = np.random.default_rng(67)
+    a = rand_storage(rng, (batch, m, k), dt) if layout[0] == "n" else rand_storage(rng, (batch, k, m), dt).transpose(0, 2, 1)
+    b = rand_storage(rng, (batch, k, n), dt) if layout[1] == "n" else rand_storage(rng, (batch, n, k), dt).transpose(0, 2, 1)
+    es = a.itemsize
+    a_rc, b_rc = [x // es for x in a.strides[1:]], [x // es for x in b.strides[1:]]
+    assert capi.gemm_kernel_name(batch, m, k, n, a_rc, b_rc, (n, 1), dt) == "pipe16k_128x64"
+    got = device_gemm(a, b, dt)
+    _check(got, a, b, dt, k)
+    bias = rand_storage(rng, (n,), dt)
+    c0 = rand_storage(rng, (batch, m, n), dt)
+    got = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)          # not this kernel's: through the one that takes over
+    _check(got, a, b, dt, k, bias=bias, c_init=c0, accumulate=True)
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_16bit_narrow_output_kernel_bit_exact(layout):
+    """Small integers: every partial sum is exact in fp32, so the product must equal the oracle's bits in any summation
+    order; C rows with a pitch above n must keep what lies between them."""
+    rng = np.random.default_rng(68)
+    batch, m, k, n, dt = 40, 1024, 448, 48, BF16
+    a64 = rng.integers(-2, 3, (batch, m, k) if layout[0] == "n" else (batch, k, m)).astype(np.float64)
+    b64 = rng.integers(-2, 3, (batch, k, n) if layout[1] == "n" else (batch, n, k)).astype(np.float64)
+    a_st, b_st = oracle.to_storage(a64, dt), oracle.to_storage(b64, dt)
+    a = a_st if layout[0] == "n" else a_st.transpose(0, 2, 1)
+    b = b_st if layout[1] == "n" else b_st.transpose(0, 2, 1)
+    want = np.matmul(a64 if layout[0] == "n" else a64.transpose(0, 2, 1), b64 if layout[1] == "n" else b64.transpose(0, 2, 1))
+    pitch = 64
+    c0 = rand_storage(rng, (batch, m, pitch), dt)
+    da, db, dc = capi.DeviceBuffer.from_numpy(a_st), capi.DeviceBuffer.from_numpy(b_st), capi.DeviceBuffer.from_numpy(c0)
+    es = 2
+    a_str = (m * k,) + tuple(x // es for x in a.strides[1:])
+    b_str = (k * n,) + tuple(x // es for x in b.strides[1:])
+    assert capi.gemm_kernel_name(batch, m, k, n, a_str[1:], b_str[1:], (pitch, 1), dt) == "pipe16k_128x64"
+    capi.gemm(dc.ptr, da.ptr, db.ptr, None, batch, m, k, n, a_str, b_str, (m * pitch, pitch, 1), False, dt)
+    capi.synchronize()
+    out = dc.to_numpy(capi.NP_STORAGE[dt], (batch, m, pitch))
+    for d in (da, db, dc):
+        d.free()
+    assert np.array_equal(oracle.to_f64(out[:, :, :n], dt), want)
+    assert np.array_equal(out[:, :, n:], c0[:, :, n:])
+
+
 def test_fp32_short_reduction_integers_bit_exact():
     """Small integers: every partial sum is exact, so the product must equal the oracle's bit for bit in any summation order."""
     rng = np.random.default_rng(62)
