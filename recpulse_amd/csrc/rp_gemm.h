@@ -149,6 +149,17 @@ int launch_skinny(const GemmArgs& g, int dtype);
 int launch_mfma16(const GemmArgs& g, const Plan& p, int dtype);
 int launch_mfmaw(const GemmArgs& g, const Plan& p, int dtype);
 int launch_tiny(const GemmArgs& g, int dtype);
+// Tiles [first, last) of `total` for this workgroup of a grid of resident workgroups (one per CU): a contiguous run, so
+// that a workgroup's consecutive tiles share operand rows, and runs that are neighbours in tile order on the same XCD
+// (workgroups go to the XCDs round robin), so that what they share is fetched into one L2 only.
+__device__ __forceinline__ void resident_tile_run(unsigned total, unsigned& first, unsigned& last) {
+    const unsigned grid = gridDim.x, b = blockIdx.x;
+    const unsigned w = (grid % 8 == 0) ? (b % 8) * (grid / 8) + b / 8 : b;
+    const unsigned run = (total + grid - 1) / grid;
+    first = w * run < total ? w * run : total;
+    last = first + run < total ? first + run : total;
+}
+
 bool direct32_takes(const GemmArgs& g);          // pointer alignment and spans the short-k fp32 kernel can address
 int launch_direct32(const GemmArgs& g);
 bool pipe32_takes(const GemmArgs& g);          // options, alignment and spans the k-contiguous short-k fp32 kernel can address

@@ -84,7 +84,10 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     extern __shared__ __attribute__((aligned(1024))) unsigned char p16_smem[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const unsigned per_matrix = (unsigned)(tiles_m * tiles_n);
-    const unsigned first = blockIdx.x, stride = gridDim.x;          // (tile numbers stay below 2^30: first + stride cannot wrap)
+    unsigned first, last;
+    resident_tile_run(total, first, last);
+    total = last;                                                   // this workgroup's tiles are [first, total)
+    constexpr unsigned stride = 1;
     const long long a_span = ((long long)(g.m - 1) * g.a_rs + g.k) * 2, b_span = ((long long)(g.n - 1) * g.b_cs + g.k) * 2;
 
     if (wave >= 4) {
