@@ -399,6 +399,27 @@ def secondary(capi, quick_reps=20):
     return out
 
 
+def memory_ceilings(capi, sizes_mb=(64, 128, 200, 256, 384, 512, 1024, 2048)):
+    """What the memory system gives plain streaming kernels of this library at a given footprint: rp_hip_fill (stores
+    only), rp_hip_channel_sums over 1024 contiguous runs (loads only) and rp_hip_convert fp32 -> fp32 (one load per store).
+    Up to the 256 MB of the memory-side cache repeated passes over the same buffer never reach HBM; beyond it they do."""
+    L = capi.lib()
+    out = {}
+    for mb in sizes_mb:
+        n = mb * (1 << 20) // 4
+        a, b, red = capi.DeviceBuffer(n * 4), capi.DeviceBuffer(n * 4), capi.DeviceBuffer(1024 * 4)
+        capi.check(L.rp_hip_fill(a.ptr, 1.0, n, capi.F32), "fill")
+        reps = max(3, min(20, 4096 // mb))
+        t_fill = _time_launches(capi, lambda: capi.check(L.rp_hip_fill(b.ptr, 2.0, n, capi.F32), "fill"), reps, 2)
+        t_read = _time_launches(capi, lambda: capi.check(L.rp_hip_channel_sums(red.ptr, a.ptr, 1, 1024, n // 1024, 0, capi.F32), "channel_sums"), reps, 2)
+        t_copy = _time_launches(capi, lambda: capi.check(L.rp_hip_convert(b.ptr, capi.F32, a.ptr, capi.F32, n), "convert"), reps, 2)
+        out[f"{mb}MB"] = {"store_us": round(t_fill * 1e3, 1), "store_GB/s": round(n * 4 / t_fill / 1e6), "load_us": round(t_read * 1e3, 1),
+                          "load_GB/s": round(n * 4 / t_read / 1e6), "copy_us": round(t_copy * 1e3, 1), "copy_GB/s_load_plus_store": round(2 * n * 4 / t_copy / 1e6)}
+        for d in (a, b, red):
+            d.free()
+    return out
+
+
 def attention_times(capi, dt_name="bf16"):
     """Config 4: Q, K, V [16*12, 512, 64]; S = Q·Kᵀ (Kᵀ a stride view), P = softmax(S/8), O = P·V, and the four
     backward GEMMs, each timed on its own from a HIP graph.  GEMM bytes are A, B and C once."""
@@ -680,6 +701,8 @@ def main():
                     help="run only the few-row bf16 GEMMs of configuration 5a and print their figures (for profiling that kernel alone)")
     ap.add_argument("--wide-only", action="store_true",
                     help="run only the fp32 (4096) and fp64 (2048, 4096) square GEMMs and print their figures (for profiling those kernels alone)")
+    ap.add_argument("--memory-ceilings", action="store_true",
+                    help="only the store / load / copy rates of the library's streaming kernels at footprints from 64 MB to 2 GB")
     ap.add_argument("--attention-only", action="store_true",
                     help="run only the configuration-4 attention launches in bf16, unfused and fused (for profiling those kernels alone)")
     ap.add_argument("--conv-only", action="store_true",
@@ -722,8 +745,11 @@ def main():
     if args.f16_only:
         print(json.dumps({"gemm_f16_8192": f16_time(capi)}))
         return
+    if args.memory_ceilings:
+        print(json.dumps({"memory_ceilings": memory_ceilings(capi)}))
+        return
     if args.attention_only:
-        print(json.dumps({"attention_bf16": attention_times(capi, "bf16")}))
+        print(json.dumps({"attention_bf16": attention_times(capi, "bf16"), "attention_f32": attention_times(capi, "f32")}))
         return
     if args.mlp_only:
         out = mlp_step_time(capi)

@@ -254,7 +254,7 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
         const int soff = (int)((long long)gm * g.c_rs * 2);
         uint32_t voff = c_lane;
         if constexpr (EDGE) voff = (gm + rr < g.m && 8 * rp < g.n) ? c_lane : K16_OOB;      // (n is a multiple of 8: a piece is inside or outside as a whole)
-        __builtin_amdgcn_raw_buffer_store_b128(rows[e], rc, (int)voff, soff, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(rows[e], rc, (int)voff, soff, 2);          // (streaming store: the output is not read again by this kernel)
     };
 
     // One slab, whose fragments are already in registers: behind each k step's MFMAs the same fragments of the NEXT slab

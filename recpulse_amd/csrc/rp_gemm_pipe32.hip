@@ -134,7 +134,7 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
         uint32_t voff = c_lane;
         if constexpr (EDGE) voff = (gm + 4 * h < g.m && gn + r < g.n) ? c_lane : S32_OOB;
         const float val = acc[SET][si][sj][v];
-        __builtin_amdgcn_raw_buffer_store_b32(s32_bits(val), rc, (int)voff, soff, 0);
+        __builtin_amdgcn_raw_buffer_store_b32(s32_bits(val), rc, (int)voff, soff, 2);          // (streaming store: the output is not read again by this kernel)
     };
 
     auto read_frags = [&](const unsigned char* base, int u, int slot) {
