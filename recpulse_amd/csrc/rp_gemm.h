@@ -35,7 +35,7 @@ struct GemmArgs {
     int bias_by_row, c_fold_from, c_fold_to;
 };
 
-enum Family { FAM_GENERIC = 0, FAM_SKINNY, FAM_MFMA16, FAM_MFMA16_SKINNY, FAM_MFMAW, FAM_TINY, FAM_DIRECT32, FAM_PIPE32, FAM_PIPE16, FAM_PIPE16K };
+enum Family { FAM_GENERIC = 0, FAM_SKINNY, FAM_MFMA16, FAM_MFMA16_SKINNY, FAM_MFMAW, FAM_TINY, FAM_DIRECT32, FAM_PIPE32, FAM_PIPE16, FAM_PIPE16K, FAM_PIPE32K };
 
 struct Plan {
     Family fam;
@@ -168,6 +168,8 @@ bool pipe16_takes(const GemmArgs& g);          // the same for the 16-bit kernel
 int launch_pipe16(const GemmArgs& g, int dtype);
 bool pipe16k_takes(const GemmArgs& g);         // the 16-bit kernel for outputs of at most 64 columns and any k
 int launch_pipe16k(const GemmArgs& g, int dtype);
+bool pipe32k_takes(const GemmArgs& g);         // and its fp32 twin
+int launch_pipe32k(const GemmArgs& g);
 int launch_gemm_segmented_b(const GemmArgs& g, int dtype);
 int launch_linear_backward_tiny(const GemmArgs& gx, const GemmArgs& gw, void* db, const void* dy, int rows, int cols, int accumulate_db);
 // adds k-split partials [nsplit][part_rows][n] (fp32, rows beyond g.m unused) in split order and runs the epilogue into C

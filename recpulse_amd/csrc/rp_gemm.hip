@@ -99,6 +99,12 @@ static bool pipe16k_off() {                        // RP_HIP_NO_PIPE16K=1: narro
     return v == 1;
 }
 
+static bool pipe32k_off() {                        // RP_HIP_NO_PIPE32K=1: narrow fp32 outputs keep the general tiled kernel
+    static int v = -1;
+    if (v < 0) { const char* e = getenv("RP_HIP_NO_PIPE32K"); v = (e && e[0] == '1') ? 1 : 0; }
+    return v == 1;
+}
+
 static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long a_cs, long long b_rs, long long b_cs,
                       long long c_rs, long long c_cs, long long a_bs, long long b_bs, int dtype, bool allow_direct = true) {
     Plan p{FAM_GENERIC, 64, 64, false, false, true, "generic"};
@@ -172,6 +178,12 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
         p.fam = FAM_PIPE16K; p.bm = 128; p.bn = 64; p.a_mc = !a_kc; p.b_mc = !b_kc; p.edge = (m % 128) || n != 64; p.name = "pipe16k_128x64";
         return p;
     }
+    // the same in fp32 (any C strides): bound by the MFMAs, which the resident kernel keeps fed without a wait per slab
+    if (dtype == RP_DTYPE_FLOAT32 && allow_direct && !pipe32k_off() && n <= 64 && k % 4 == 0 && k >= 32 && (a_kc || (a_rs == 1 && a_cs % 4 == 0)) &&
+        (b_kc || (b_cs == 1 && b_rs % 4 == 0)) && batch_ok && m > 64 && (long long)((m + 127) / 128) * batch >= 256) {
+        p.fam = FAM_PIPE32K; p.bm = 128; p.bn = 64; p.a_mc = !a_kc; p.b_mc = !b_kc; p.edge = (m % 128) || n != 64; p.name = "pipe32k_128x64";
+        return p;
+    }
     if (!mfma_ok) return p;
     p.a_mc = !a_kc;             // when both qualify (extent-1 corner cases) keep the row-major reading
     p.b_mc = b_mc;
@@ -201,6 +213,10 @@ static int run_gemm(const GemmArgs& g, int dtype) {
     }
     if (p.fam == FAM_PIPE16K) {
         if (pipe16k_takes(g)) return launch_pipe16k(g, dtype);
+        p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype, false);
+    }
+    if (p.fam == FAM_PIPE32K) {
+        if (pipe32k_takes(g)) return launch_pipe32k(g);
         p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype, false);
     }
     if (p.fam == FAM_DIRECT32) {

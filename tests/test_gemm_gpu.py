@@ -555,6 +555,53 @@ def test_16bit_narrow_output_kernel_bit_exact(layout):
     assert np.array_equal(out[:, :, n:], c0[:, :, n:])
 
 
+# ---- and its fp32 twin (any n up to 64, any C strides)
+PIPE32K_SHAPES = [(64, 512, 512, 64), (70, 500, 200, 40), (300, 130, 72, 64), (1, 32768, 96, 50), (130, 256, 32, 64), (33, 1000, 324, 7)]
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("batch,m,k,n", PIPE32K_SHAPES)
+def test_fp32_narrow_output_kernel(batch, m, k, n, layout):
+    rng = np.random.default_rng(69)
+    # free-index-major operands need 16-byte aligned k rows: pad the storage, view the first m (n) entries
+    mp, npad = (m + 3) // 4 * 4, (n + 3) // 4 * 4
+    a = rand_storage(rng, (batch, m, k), F32) if layout[0] == "n" else rand_storage(rng, (batch, k, mp), F32)[:, :, :m].transpose(0, 2, 1)
+    b = rand_storage(rng, (batch, k, npad), F32)[:, :, :n] if layout[1] == "n" else rand_storage(rng, (batch, n, k), F32).transpose(0, 2, 1)
+    a_rc, b_rc = [x // 4 for x in a.strides[1:]], [x // 4 for x in b.strides[1:]]
+    assert capi.gemm_kernel_name(batch, m, k, n, a_rc, b_rc, (n, 1), F32) == "pipe32k_128x64"
+    got = device_gemm(a, b, F32)
+    _check(got, a, b, F32, k)
+    bias = rand_storage(rng, (n,), F32)
+    c0 = rand_storage(rng, (batch, m, n), F32)
+    got = device_gemm(a, b, F32, bias=bias, c_init=c0, accumulate=True)          # not this kernel's: through the one that takes over
+    _check(got, a, b, F32, k, bias=bias, c_init=c0, accumulate=True)
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_fp32_narrow_output_kernel_bit_exact_strided_c(layout):
+    """Small integers (every partial sum exact: the oracle's bits in any order) into a transposed, padded C."""
+    rng = np.random.default_rng(70)
+    batch, m, k, n = 40, 1024, 448, 48
+    a64 = rng.integers(-3, 4, (batch, m, k) if layout[0] == "n" else (batch, k, m)).astype(np.float32)
+    b64 = rng.integers(-3, 4, (batch, k, n) if layout[1] == "n" else (batch, n, k)).astype(np.float32)
+    a = a64 if layout[0] == "n" else a64.transpose(0, 2, 1)
+    b = b64 if layout[1] == "n" else b64.transpose(0, 2, 1)
+    want = np.matmul(a.astype(np.float64), b.astype(np.float64)).astype(np.float32)
+    pitch = m + 3
+    c0 = rand_storage(rng, (batch, n + 1, pitch), F32)
+    da, db, dc = capi.DeviceBuffer.from_numpy(a64), capi.DeviceBuffer.from_numpy(b64), capi.DeviceBuffer.from_numpy(c0)
+    a_str = (m * k,) + tuple(x // 4 for x in a.strides[1:])
+    b_str = (k * n,) + tuple(x // 4 for x in b.strides[1:])
+    assert capi.gemm_kernel_name(batch, m, k, n, a_str[1:], b_str[1:], (1, pitch), F32) == "pipe32k_128x64"
+    capi.gemm(dc.ptr, da.ptr, db.ptr, None, batch, m, k, n, a_str, b_str, ((n + 1) * pitch, 1, pitch), False, F32)
+    capi.synchronize()
+    out = dc.to_numpy(np.float32, (batch, n + 1, pitch))
+    for d in (da, db, dc):
+        d.free()
+    assert np.array_equal(out[:, :n, :m], want.transpose(0, 2, 1))
+    assert np.array_equal(out[:, n:, :], c0[:, n:, :]) and np.array_equal(out[:, :, m:], c0[:, :, m:])
+
+
 def test_fp32_short_reduction_integers_bit_exact():
     """Small integers: every partial sum is exact, so the product must equal the oracle's bit for bit in any summation order."""
     rng = np.random.default_rng(62)
