@@ -515,8 +515,6 @@ def conv2d_times(capi, dt_name="bf16"):
         fn()
     capi.check(L.rp_hip_im2col_batched(d_col.ptr, d_x.ptr, N, *geom, dt), "im2col")       # dW reads the lowered activations, not dcol
     out, total = {}, 0.0
-    for _ in range(300):                 # the clock the power management grants settles within some tens of milliseconds of load
-        ops["S=Q.Kt"][0]()
     for name, (fn, flops, nbytes) in ops.items():
         ms = _time_graph(capi, fn, 10, 2)
         total += ms
