@@ -166,9 +166,9 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
         return p;
     }
     // the same for bf16 / fp16 (C row-major): there the stores and the narrowing are what takes time
-    if (is16 && allow_direct && !pipe16_off() && k <= 64 && k % 8 == 0 && a_cs == 1 && b_rs == 1 && a_rs % 8 == 0 && b_cs % 8 == 0 && batch_ok &&
+    if (is16 && allow_direct && !pipe16_off() && k <= 64 && k % 8 == 0 && (a_kc || a_mc) && (b_kc || b_mc) && batch_ok &&
         c_cs == 1 && c_rs % 8 == 0 && n % 8 == 0 && m > 64 && n > 64 && (long long)((m + 127) / 128) * ((n + 127) / 128) * batch >= 256) {
-        p.fam = FAM_PIPE16; p.bm = 128; p.bn = 128; p.a_mc = false; p.b_mc = false; p.edge = (m % 128) || (n % 128); p.name = "pipe16_128x128";
+        p.fam = FAM_PIPE16; p.bm = 128; p.bn = 128; p.a_mc = !a_kc; p.b_mc = !b_kc; p.edge = (m % 128) || (n % 128); p.name = "pipe16_128x128";
         return p;
     }
     // bf16 / fp16, at most 64 output columns, at least one 128-row tile per CU (O = P.V per head, a tall matrix times a narrow

@@ -1,4 +1,5 @@
-// bf16 / fp16 GEMM with a short reduction (k <= 64) and both operands contiguous along k, e.g. S = Q.K^T per head.
+// bf16 / fp16 GEMM with a short reduction (k <= 64), e.g. S = Q.K^T per head (both operands contiguous along k) or the
+// lowered convolution's dcol = W^T.dy (both contiguous along their free index); every combination is taken.
 //
 // 128 x 128 outputs per tile from 2 x 128 x 64 inputs: the product is bound by what it writes.  The arithmetic of a tile
 // is 16 MFMAs per wave; what takes time is narrowing 64 accumulators per lane and getting 32 KB of stores out.  As in the
@@ -78,8 +79,20 @@ template <> struct s16_ops<f16_t> {
     }
 };
 
-// KST: k steps of 16 that are multiplied (4 for k <= 64, 2 for k <= 32); EDGE: m or n not whole tiles.
-template <typename T, int KST, bool EDGE>
+typedef __attribute__((ext_vector_type(4))) short s16_s16x4_t;
+
+// half H (k values 4H .. 4H + 3 of the lane's eight) of a fragment of an operand that lies in LDS as k rows
+template <int H>
+__device__ __forceinline__ void s16_read_tr(s16x8_t& v, const unsigned char* p) {
+    const s16_s16x4_t q = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16_s16x4_t __attribute__((address_space(3)))*)(p));
+    v[4 * H + 0] = q[0]; v[4 * H + 1] = q[1]; v[4 * H + 2] = q[2]; v[4 * H + 3] = q[3];
+}
+
+// KST: k steps of 16 that are multiplied (4 for k <= 64, 2 for k <= 32); A_MC / B_MC: the operand has unit stride along
+// its free index (m, n) instead of along k: it lies in LDS as 64 k rows of 128 free indices (256 bytes) whose 32-byte
+// pieces are XORed with the low three bits of the k row, and its fragments are transposing reads (ds_read_b64_tr_b16);
+// EDGE: m or n not whole tiles.
+template <typename T, int KST, bool A_MC, bool B_MC, bool EDGE>
 __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_m, int tiles_n, unsigned total) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char p16_smem[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -88,25 +101,34 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     resident_tile_run(total, first, last);
     total = last;                                                   // this workgroup's tiles are [first, total)
     constexpr unsigned stride = 1;
-    const long long a_span = ((long long)(g.m - 1) * g.a_rs + g.k) * 2, b_span = ((long long)(g.n - 1) * g.b_cs + g.k) * 2;
+    const long long a_fs = g.a_rs, a_ks = g.a_cs, b_fs = g.b_cs, b_ks = g.b_rs;      // strides of the free index and of k
+    const long long a_span = (A_MC ? ((long long)(g.k - 1) * a_ks + g.m) : ((long long)(g.m - 1) * a_fs + g.k)) * 2;
+    const long long b_span = (B_MC ? ((long long)(g.k - 1) * b_ks + g.n) : ((long long)(g.n - 1) * b_fs + g.k)) * 2;
 
     if (wave >= 4) {
-        // ---- fetch: this wave brings rows [32p, 32p + 32) of A and of B for every tile ----
+        // ---- fetch: this wave brings rows [32p, 32p + 32) (k-contiguous operand) or k rows [16p, 16p + 16) (the other
+        // layout) of A and of B for every tile; a wave instruction fills 1 KB of LDS: 8 rows, or 4 k rows ----
         const int p = wave - 4;
         uint32_t a_off[4], b_off[4];
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             const int row = 8 * q + (lane >> 3);                        // row within the wave's 32
             const int piece = (lane & 7) ^ ((row >> 1) & 7);            // which 16 bytes of the global row land in this lane's LDS slot
-            const bool in = piece * 8 < g.k;
-            a_off[q] = in ? (uint32_t)(((long long)row * g.a_rs + piece * 8) * 2) : S16_OOB;
-            b_off[q] = in ? (uint32_t)(((long long)row * g.b_cs + piece * 8) * 2) : S16_OOB;
+            const int krow = 4 * q + (lane >> 4);                       // k row within the wave's 16
+            const int c32 = ((lane & 15) >> 1) ^ (krow & 7);            // which 32 bytes of the global k row (its half: lane & 1)
+            const int free = (c32 * 2 + (lane & 1)) * 8;
+            a_off[q] = A_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * a_ks + free) * 2) : S16_OOB)
+                            : (piece * 8 < g.k ? (uint32_t)(((long long)row * a_fs + piece * 8) * 2) : S16_OOB);
+            b_off[q] = B_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * b_ks + free) * 2) : S16_OOB)
+                            : (piece * 8 < g.k ? (uint32_t)(((long long)row * b_fs + piece * 8) * 2) : S16_OOB);
         }
         auto fetch = [&](unsigned id, int buf) {
             const S16Tile t = s16_tile(id, per_matrix, tiles_n);
             const __amdgpu_buffer_rsrc_t ra = s16_rsrc((const uint16_t*)g.A + (long long)t.z * g.a_bs, a_span);
             const __amdgpu_buffer_rsrc_t rb = s16_rsrc((const uint16_t*)g.B + (long long)t.z * g.b_bs, b_span);
-            const int sa = (int)((long long)(t.m0 + 32 * p) * g.a_rs * 2), sb = (int)((long long)(t.n0 + 32 * p) * g.b_cs * 2);
+            const int sa = A_MC ? (int)(((long long)(16 * p) * a_ks + t.m0) * 2) : (int)((long long)(t.m0 + 32 * p) * a_fs * 2);
+            const int sb = B_MC ? (int)(((long long)(16 * p) * b_ks + t.n0) * 2) : (int)((long long)(t.n0 + 32 * p) * b_fs * 2);
+            // (both layouts put the wave's share at the same place: 32 rows of 128 bytes = 16 k rows of 256 bytes = 4 KB)
             unsigned char* dst = p16_smem + buf * S16_TILE_BYTES + 32 * p * S16_ROW_BYTES;
 #pragma unroll
             for (int q = 0; q < 4; q++) {
@@ -146,9 +168,35 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     // ---- multiply and store ----
     const int r = lane & 31, h = lane >> 5;
     const int wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * 64;
-    // LDS byte address of piece 2s + h of this lane's row: lane_x ^ (32 s) (rows are 128-byte aligned, so the XOR only touches the piece bits)
-    const uint32_t lane_a = (uint32_t)((wm0 + r) * S16_ROW_BYTES + ((h ^ ((r >> 1) & 7)) * 16));
-    const uint32_t lane_b = (uint32_t)(S16_BM * S16_ROW_BYTES + (wn0 + r) * S16_ROW_BYTES + ((h ^ ((r >> 1) & 7)) * 16));
+    // LDS byte addresses of the fragments of k step 0.  k-contiguous operand: piece 2s + h of the lane's row is at
+    // base ^ (32 s) (rows are 128-byte aligned, so the XOR only touches the piece bits).  Other layout: the transposing read
+    // of a 16-lane group covers 4 k rows x 16 free indices; source lane s points at free indices 4(s % 4) .. + 3 of k row
+    // s / 4; the groups are (k octet, free half) = (grp / 2, grp % 2); k step s is 16 k rows further.
+    const int grp = lane >> 4, s16 = lane & 15;
+    uint32_t a_fr[2][2], b_fr[2][2];                                // [H][tile] (k-contiguous: only [0][tile] is used)
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        if (!A_MC) {
+            a_fr[0][i] = (uint32_t)((wm0 + 32 * i + r) * S16_ROW_BYTES + ((h ^ ((r >> 1) & 7)) * 16));
+            a_fr[1][i] = 0;
+        } else {
+#pragma unroll
+            for (int H = 0; H < 2; H++) {
+                const int krow = 8 * (grp >> 1) + 4 * H + (s16 >> 2), free = wm0 + 32 * i + 16 * (grp & 1) + 4 * (s16 & 3);
+                a_fr[H][i] = (uint32_t)(krow * 256 + (((free >> 4) ^ (krow & 7)) * 32) + (free & 15) * 2);
+            }
+        }
+        if (!B_MC) {
+            b_fr[0][i] = (uint32_t)(S16_BM * S16_ROW_BYTES + (wn0 + 32 * i + r) * S16_ROW_BYTES + ((h ^ ((r >> 1) & 7)) * 16));
+            b_fr[1][i] = 0;
+        } else {
+#pragma unroll
+            for (int H = 0; H < 2; H++) {
+                const int krow = 8 * (grp >> 1) + 4 * H + (s16 >> 2), free = wn0 + 32 * i + 16 * (grp & 1) + 4 * (s16 & 3);
+                b_fr[H][i] = (uint32_t)(S16_BM * S16_ROW_BYTES + krow * 256 + (((free >> 4) ^ (krow & 7)) * 32) + (free & 15) * 2);
+            }
+        }
+    }
     // The wave's own 64 x 64 staging patch (rows of 128 bytes, 16-byte pieces XORed like the operand tiles).  After the
     // swapped MFMA a lane holds row r of C and four adjacent columns per accumulator quad: 8 bytes, written at piece
     // 4 in + q, half h.  Read back, a lane holds 16 bytes of row lane / 8 (+ 8 per instruction), piece lane % 8: eight
@@ -196,9 +244,15 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     auto read_frags = [&](const unsigned char* base, auto s_c) {
         constexpr int s = decltype(s_c)::value;
 #pragma unroll
-        for (int i = 0; i < 2; i++) af[s][i] = *(const s16x8_t*)(base + ((lane_a ^ (uint32_t)(32 * s)) + i * 32 * S16_ROW_BYTES));
+        for (int i = 0; i < 2; i++) {
+            if constexpr (!A_MC) af[s][i] = *(const s16x8_t*)(base + (a_fr[0][i] ^ (uint32_t)(32 * s)));
+            else { s16_read_tr<0>(af[s][i], base + a_fr[0][i] + 16 * s * 256); s16_read_tr<1>(af[s][i], base + a_fr[1][i] + 16 * s * 256); }
+        }
 #pragma unroll
-        for (int j = 0; j < 2; j++) bf[s][j] = *(const s16x8_t*)(base + ((lane_b ^ (uint32_t)(32 * s)) + j * 32 * S16_ROW_BYTES));
+        for (int j = 0; j < 2; j++) {
+            if constexpr (!B_MC) bf[s][j] = *(const s16x8_t*)(base + (b_fr[0][j] ^ (uint32_t)(32 * s)));
+            else { s16_read_tr<0>(bf[s][j], base + b_fr[0][j] + 16 * s * 256); s16_read_tr<1>(bf[s][j], base + b_fr[1][j] + 16 * s * 256); }
+        }
     };
 
     // One tile, whose operand pieces are already in registers: behind each k step's MFMAs the same pieces of the NEXT tile
@@ -266,7 +320,7 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
 
 // ---- host side ----
 
-// Whether this kernel takes the product: k <= 64 in whole 16-byte pieces, both operands contiguous along k with
+// Whether this kernel takes the product: k <= 64 in whole 16-byte pieces, both operands with a unit stride and
 // 16-byte aligned rows, C row-major with 16-byte aligned rows and n in whole eights, overwritten (no accumulation, bias,
 // segments or folded store), and every byte offset the kernel forms from a batch entry's base within the 32-bit range
 // of buffer addressing.
@@ -274,12 +328,16 @@ bool pipe16_takes(const GemmArgs& g) {
     if (g.k > S16_MAXK || g.k < 8 || g.k % 8 || g.m < 1 || g.n < 8 || g.n % 8 || g.batch < 1) return false;
     if ((long long)((g.m + S16_BM - 1) / S16_BM) * ((g.n + S16_BN - 1) / S16_BN) * g.batch >= (1ll << 30)) return false;
     if (g.bias || g.accumulate || g.seg_k || g.seg_n || g.c_fold_from || g.bias_by_row) return false;
-    if (g.a_cs != 1 || g.b_rs != 1 || g.a_rs % 8 || g.b_cs % 8 || g.a_bs % 8 || g.b_bs % 8 || g.a_rs < 0 || g.b_cs < 0) return false;
+    const bool a_kc = g.a_cs == 1 && g.a_rs % 8 == 0, a_mc = g.a_rs == 1 && g.a_cs % 8 == 0;
+    const bool b_kc = g.b_rs == 1 && g.b_cs % 8 == 0, b_mc = g.b_cs == 1 && g.b_rs % 8 == 0;
+    if (!(a_kc || a_mc) || !(b_kc || b_mc) || g.a_bs % 8 || g.b_bs % 8 || g.a_rs < 0 || g.a_cs < 0 || g.b_rs < 0 || g.b_cs < 0) return false;
     if (g.c_cs != 1 || g.c_rs % 8 || g.c_bs % 8 || g.c_rs < 0) return false;
     if (((uintptr_t)g.A & 15) || ((uintptr_t)g.B & 15) || ((uintptr_t)g.C & 15)) return false;
     const long long lim = 1ll << 30;
-    // rows up to a whole tile past the last one are addressed (and read as zero or dropped by the range check)
-    const long long a_reach = ((long long)(g.m + S16_BM) * g.a_rs + S16_MAXK) * 2, b_reach = ((long long)(g.n + S16_BN) * g.b_cs + S16_MAXK) * 2;
+    // free indices up to a whole tile past the last one are addressed (and read as zero, or as values that only reach
+    // outputs which are not stored)
+    const long long a_reach = (a_kc ? (long long)(g.m + S16_BM) * g.a_rs + S16_MAXK : (long long)S16_MAXK * g.a_cs + g.m + S16_BM) * 2;
+    const long long b_reach = (b_kc ? (long long)(g.n + S16_BN) * g.b_cs + S16_MAXK : (long long)S16_MAXK * g.b_rs + g.n + S16_BN) * 2;
     const long long c_reach = ((long long)(g.m + S16_BM) * g.c_rs + g.n + S16_BN) * 2;
     return a_reach < lim && b_reach < lim && c_reach < lim;
 }
@@ -298,8 +356,16 @@ static int launch_pipe16_t(const GemmArgs& g) {
         hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), smem, current_stream(), g, tiles_m, tiles_n, (unsigned)total);
         return check_launch("gemm_pipe16_kernel") ? 0 : -1;
     };
-    if (g.k <= 32) return edge ? launch(gemm_pipe16_kernel<T, 2, true>) : launch(gemm_pipe16_kernel<T, 2, false>);
-    return edge ? launch(gemm_pipe16_kernel<T, 4, true>) : launch(gemm_pipe16_kernel<T, 4, false>);
+    const bool a_mc = !(g.a_cs == 1 && g.a_rs % 8 == 0), b_mc = !(g.b_rs == 1 && g.b_cs % 8 == 0);
+    auto pick = [&](auto kst_c) {
+        constexpr int KST = decltype(kst_c)::value;
+        if (!a_mc && !b_mc) return edge ? launch(gemm_pipe16_kernel<T, KST, false, false, true>) : launch(gemm_pipe16_kernel<T, KST, false, false, false>);
+        if (!a_mc && b_mc) return edge ? launch(gemm_pipe16_kernel<T, KST, false, true, true>) : launch(gemm_pipe16_kernel<T, KST, false, true, false>);
+        if (a_mc && !b_mc) return edge ? launch(gemm_pipe16_kernel<T, KST, true, false, true>) : launch(gemm_pipe16_kernel<T, KST, true, false, false>);
+        return edge ? launch(gemm_pipe16_kernel<T, KST, true, true, true>) : launch(gemm_pipe16_kernel<T, KST, true, true, false>);
+    };
+    if (g.k <= 32) return pick(std::integral_constant<int, 2>{});
+    return pick(std::integral_constant<int, 4>{});
 }
 
 int launch_pipe16(const GemmArgs& g, int dtype) {

@@ -465,19 +465,43 @@ def test_fp32_pipelined_kernel_views_and_strided_output():
 PIPE16_SHAPES = [(16, 512, 64, 512), (20, 500, 64, 456), (48, 250, 40, 296), (32, 384, 32, 512), (70, 256, 16, 256), (300, 130, 8, 136), (3, 1100, 56, 1304)]
 
 
+@pytest.mark.parametrize("layout", LAYOUTS)
 @pytest.mark.parametrize("dt", HALF, ids=lambda d: NAMES[d])
 @pytest.mark.parametrize("batch,m,k,n", PIPE16_SHAPES)
-def test_16bit_pipelined_kernel_k_contiguous(batch, m, k, n, dt):
+def test_16bit_pipelined_kernel(batch, m, k, n, dt, layout):
     rng = np.random.default_rng(65)
-    a = rand_storage(rng, (batch, m, k), dt)
-    b = rand_storage(rng, (batch, n, k), dt).transpose(0, 2, 1)
-    assert capi.gemm_kernel_name(batch, m, k, n, (k, 1), (1, k), (n, 1), dt) == "pipe16_128x128"
+    mp = (m + 7) // 8 * 8                                   # m-major A needs 16-byte aligned k rows: pad the storage
+    a = rand_storage(rng, (batch, m, k), dt) if layout[0] == "n" else rand_storage(rng, (batch, k, mp), dt)[:, :, :m].transpose(0, 2, 1)
+    b = rand_storage(rng, (batch, k, n), dt) if layout[1] == "n" else rand_storage(rng, (batch, n, k), dt).transpose(0, 2, 1)
+    es = a.itemsize
+    a_rc, b_rc = [x // es for x in a.strides[1:]], [x // es for x in b.strides[1:]]
+    if layout[0] == "n" or m % 8 == 0:
+        assert capi.gemm_kernel_name(batch, m, k, n, a_rc, b_rc, (n, 1), dt) == "pipe16_128x128"
     got = device_gemm(a, b, dt)
     _check(got, a, b, dt, k)
     bias = rand_storage(rng, (n,), dt)
     c0 = rand_storage(rng, (batch, m, n), dt)
     got = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)          # not this kernel's: through the one that takes over
     _check(got, a, b, dt, k, bias=bias, c_init=c0, accumulate=True)
+
+
+def test_16bit_pipelined_kernel_free_index_major_bit_exact():
+    """The lowered convolution's dcol = W^T.dy shape (both operands with unit stride along their free index), small
+    integers: every sum is exact, so the product must equal the oracle's bits."""
+    rng = np.random.default_rng(73)
+    batch, m, k, n = 8, 576, 64, 3136
+    for dt in HALF:
+        w64 = rng.integers(-2, 3, (k, m)).astype(np.float64)            # shared by the batch (batch stride 0)
+        dy64 = rng.integers(-2, 3, (batch, k, n)).astype(np.float64)
+        w_st, dy_st = oracle.to_storage(w64, dt), oracle.to_storage(dy64, dt)
+        dw, ddy, dc = capi.DeviceBuffer.from_numpy(w_st), capi.DeviceBuffer.from_numpy(dy_st), capi.DeviceBuffer(batch * m * n * 2)
+        assert capi.gemm_kernel_name(batch, m, k, n, (1, m), (n, 1), (n, 1), dt) == "pipe16_128x128"
+        capi.gemm(dc.ptr, dw.ptr, ddy.ptr, None, batch, m, k, n, (0, 1, m), (k * n, n, 1), (m * n, n, 1), False, dt)
+        capi.synchronize()
+        out = dc.to_numpy(capi.NP_STORAGE[dt], (batch, m, n))
+        for d in (dw, ddy, dc):
+            d.free()
+        assert np.array_equal(out, oracle.to_storage(np.matmul(w64.T[None], dy64), dt)), dt
 
 
 @pytest.mark.parametrize("dt", HALF, ids=lambda d: NAMES[d])
