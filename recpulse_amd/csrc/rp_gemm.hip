@@ -148,6 +148,14 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
         p.fam = FAM_TINY; p.bm = 16; p.bn = 16; p.name = "tiny32_16x16";
         return p;
     }
+    // fp32 with k <= 64, any operand layout with a unit stride and at least one 128 x 128 tile per CU: one resident workgroup per
+    // CU whose fetching waves fill LDS directly and whose multiplying waves store the previous tile between the MFMAs
+    if (dtype == RP_DTYPE_FLOAT32 && allow_direct && !pipe32_off() && k <= 64 && k % 4 == 0 && ((a_cs == 1 && a_rs % 4 == 0) || (a_rs == 1 && a_cs % 4 == 0)) &&
+        ((b_rs == 1 && b_cs % 4 == 0) || (b_cs == 1 && b_rs % 4 == 0)) &&
+        batch_ok && m > 64 && n > 64 && (long long)((m + 127) / 128) * ((n + 127) / 128) * batch >= 256) {
+        p.fam = FAM_PIPE32; p.bm = 128; p.bn = 128; p.a_mc = !(a_cs == 1 && a_rs % 4 == 0); p.b_mc = !(b_rs == 1 && b_cs % 4 == 0); p.edge = (m % 128) || (n % 128); p.name = "pipe32_128x128";
+        return p;
+    }
     // fp32 with 32 < k <= 64, both operands with unit stride along their free index and an output of at least 128 tiles of
     // 128 x 128: no k loop to pipeline, so every wave multiplies a 64 x 64 patch straight out of registers (no LDS, no
     // barrier).  (With unit stride along k a lane's loads touch 64 cache lines per instruction and the vector cache's
@@ -156,13 +164,6 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
         (a_cs != 1 || (k % 4 == 0 && a_rs % 4 == 0 && a_bs % 4 == 0)) && (b_rs != 1 || (k % 4 == 0 && b_cs % 4 == 0 && b_bs % 4 == 0)) &&
         m >= 64 && n >= 64 && (long long)((m + 127) / 128) * ((n + 127) / 128) * batch >= 128) {
         p.fam = FAM_DIRECT32; p.bm = 128; p.bn = 128; p.a_mc = a_cs != 1; p.b_mc = b_rs != 1; p.name = "direct32_128x128";
-        return p;
-    }
-    // fp32 with k <= 64, both operands contiguous along k and at least one 128 x 128 tile per CU: one resident workgroup per
-    // CU whose fetching waves fill LDS directly and whose multiplying waves store the previous tile between the MFMAs
-    if (dtype == RP_DTYPE_FLOAT32 && allow_direct && !pipe32_off() && k <= 64 && k % 4 == 0 && a_cs == 1 && b_rs == 1 && a_rs % 4 == 0 && b_cs % 4 == 0 &&
-        batch_ok && m > 64 && n > 64 && (long long)((m + 127) / 128) * ((n + 127) / 128) * batch >= 256) {
-        p.fam = FAM_PIPE32; p.bm = 128; p.bn = 128; p.a_mc = false; p.b_mc = false; p.edge = (m % 128) || (n % 128); p.name = "pipe32_128x128";
         return p;
     }
     // the same for bf16 / fp16 (C row-major): there the stores and the narrowing are what takes time

@@ -1,4 +1,5 @@
-// fp32 GEMM with a short reduction (k <= 64) and both operands contiguous along k, e.g. S = Q.K^T per head.
+// fp32 GEMM with a short reduction (k <= 64), e.g. S = Q.K^T per head (both operands contiguous along k); operands with
+// unit stride along their free index are taken as well.
 //
 // Such a product writes far more than it reads (512 x 512 outputs from 2 x 512 x 64 inputs), and per 128 x 128
 // tile the 64 KB of stores take about as long as the 128 MFMAs of a wave.  A block that multiplies, then stores,
@@ -63,7 +64,10 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t s32_rsrc(const void* base, lon
 }
 
 // KCH: 16-byte pieces of k per lane pair that are multiplied (8 for k <= 64, 4 for k <= 32); EDGE: m or n not whole tiles.
-template <int KCH, bool EDGE>
+// A_MC / B_MC: the operand has unit stride along its free index (m, n) instead of along k: it lies in LDS as 64 k rows of
+// 128 free indices (512 bytes) whose 128-byte pieces are XORed with (k row / 4) % 4, so that the two halves of a wave, which
+// read k rows four apart, use different banks; its values are read one at a time.
+template <int KCH, bool A_MC, bool B_MC, bool EDGE>
 __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_m, int tiles_n, unsigned total) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char p32_smem[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -72,25 +76,34 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
     resident_tile_run(total, first, run_end);
     total = run_end;                                                   // this workgroup's tiles are [first, total)
     constexpr unsigned stride = 1;
-    const long long a_span = ((long long)(g.m - 1) * g.a_rs + g.k) * 4, b_span = ((long long)(g.n - 1) * g.b_cs + g.k) * 4;
+    const long long a_fs = g.a_rs, a_ks = g.a_cs, b_fs = g.b_cs, b_ks = g.b_rs;      // strides of the free index and of k
+    const long long a_span = (A_MC ? ((long long)(g.k - 1) * a_ks + g.m) : ((long long)(g.m - 1) * a_fs + g.k)) * 4;
+    const long long b_span = (B_MC ? ((long long)(g.k - 1) * b_ks + g.n) : ((long long)(g.n - 1) * b_fs + g.k)) * 4;
 
     if (wave >= 4) {
-        // ---- fetch: this wave brings rows [32p, 32p + 32) of A and of B for every tile ----
+        // ---- fetch: this wave brings rows [32p, 32p + 32) (k-contiguous operand) or k rows [16p, 16p + 16) (the other
+        // layout) of A and of B for every tile; a wave instruction fills 1 KB of LDS: 4 rows, or 2 k rows ----
         const int p = wave - 4;
         uint32_t a_off[8], b_off[8];
 #pragma unroll
         for (int q = 0; q < 8; q++) {
             const int row = 4 * q + (lane >> 4);                        // row within the wave's 32
             const int piece = (lane & 15) ^ (row & 15);                 // which 16 bytes of the global row land in this lane's LDS slot
-            const bool in = piece * 4 < g.k;
-            a_off[q] = in ? (uint32_t)(((long long)row * g.a_rs + piece * 4) * 4) : S32_OOB;
-            b_off[q] = in ? (uint32_t)(((long long)row * g.b_cs + piece * 4) * 4) : S32_OOB;
+            const int krow = 2 * q + (lane >> 5);                       // k row within the wave's 16
+            const int c128 = ((lane & 31) >> 3) ^ ((krow >> 2) & 3);    // which 128 bytes of the global k row (its 16-byte piece: lane & 7)
+            const int free = c128 * 32 + (lane & 7) * 4;
+            a_off[q] = A_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * a_ks + free) * 4) : S32_OOB)
+                            : (piece * 4 < g.k ? (uint32_t)(((long long)row * a_fs + piece * 4) * 4) : S32_OOB);
+            b_off[q] = B_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * b_ks + free) * 4) : S32_OOB)
+                            : (piece * 4 < g.k ? (uint32_t)(((long long)row * b_fs + piece * 4) * 4) : S32_OOB);
         }
         auto fetch = [&](unsigned id, int buf) {
             const S32Tile t = s32_tile(id, per_matrix, tiles_n);
             const __amdgpu_buffer_rsrc_t ra = s32_rsrc((const float*)g.A + (long long)t.z * g.a_bs, a_span);
             const __amdgpu_buffer_rsrc_t rb = s32_rsrc((const float*)g.B + (long long)t.z * g.b_bs, b_span);
-            const int sa = (int)((long long)(t.m0 + 32 * p) * g.a_rs * 4), sb = (int)((long long)(t.n0 + 32 * p) * g.b_cs * 4);
+            const int sa = A_MC ? (int)(((long long)(16 * p) * a_ks + t.m0) * 4) : (int)((long long)(t.m0 + 32 * p) * a_fs * 4);
+            const int sb = B_MC ? (int)(((long long)(16 * p) * b_ks + t.n0) * 4) : (int)((long long)(t.n0 + 32 * p) * b_fs * 4);
+            // (both layouts put the wave's share at the same place: 32 rows of 256 bytes = 16 k rows of 512 bytes = 8 KB)
             unsigned char* dst = p32_smem + buf * S32_TILE_BYTES + 32 * p * S32_ROW_BYTES;
 #pragma unroll
             for (int q = 0; q < 8; q++) {
@@ -114,10 +127,12 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
     // ---- multiply and store ----
     const int r = lane & 31, h = lane >> 5;
     const int wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * 64;
-    // LDS byte address of piece 2u + h of this lane's row: lane_a ^ (32 u) (rows are 256-byte aligned, so the XOR only
-    // touches the piece bits)
+    // k-contiguous operand: the LDS byte address of piece 2u + h of this lane's row is lane_x ^ (32 u) (rows are 256-byte
+    // aligned, so the XOR only touches the piece bits).  Other layout: the value of step (u, e), k row 8u + 4h + e, free
+    // index w0 + 32 i + r, is at mc_x + (8u + e) k rows, in the 128-byte piece (w0 / 32 + i) ^ ((2u + h) % 4).
     const uint32_t lane_a = (uint32_t)((wm0 + r) * S32_ROW_BYTES + ((h ^ (r & 15)) * 16));
     const uint32_t lane_b = (uint32_t)(S32_BM * S32_ROW_BYTES + (wn0 + r) * S32_ROW_BYTES + ((h ^ (r & 15)) * 16));
+    const uint32_t mc_a = (uint32_t)(4 * h * 512 + r * 4), mc_b = (uint32_t)(S32_BM * S32_ROW_BYTES + 4 * h * 512 + r * 4);
     const uint32_t c_lane = (uint32_t)(((long long)(4 * h) * g.c_rs + (long long)r * g.c_cs) * 4);
     const long long c_span = ((long long)(g.m - 1) * g.c_rs + (long long)(g.n - 1) * g.c_cs + 1) * 4;
 
@@ -139,9 +154,25 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
 
     auto read_frags = [&](const unsigned char* base, int u, int slot) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) af[slot][i] = *(const f32x4_t*)(base + ((lane_a ^ (uint32_t)(32 * u)) + i * 32 * S32_ROW_BYTES));
+        for (int i = 0; i < 2; i++) {
+            if constexpr (!A_MC) {
+                af[slot][i] = *(const f32x4_t*)(base + ((lane_a ^ (uint32_t)(32 * u)) + i * 32 * S32_ROW_BYTES));
+            } else {
+                const uint32_t at = mc_a + (uint32_t)(8 * u * 512) + ((((uint32_t)(wm0 >> 5) + i) ^ (uint32_t)((2 * u + h) & 3)) * 128);
 #pragma unroll
-        for (int j = 0; j < 2; j++) bf[slot][j] = *(const f32x4_t*)(base + ((lane_b ^ (uint32_t)(32 * u)) + j * 32 * S32_ROW_BYTES));
+                for (int e = 0; e < 4; e++) af[slot][i][e] = *(const float*)(base + at + e * 512);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            if constexpr (!B_MC) {
+                bf[slot][j] = *(const f32x4_t*)(base + ((lane_b ^ (uint32_t)(32 * u)) + j * 32 * S32_ROW_BYTES));
+            } else {
+                const uint32_t at = mc_b + (uint32_t)(8 * u * 512) + ((((uint32_t)(wn0 >> 5) + j) ^ (uint32_t)((2 * u + h) & 3)) * 128);
+#pragma unroll
+                for (int e = 0; e < 4; e++) bf[slot][j][e] = *(const float*)(base + at + e * 512);
+            }
+        }
     };
 
     // One tile: accumulate into set CUR from LDS tile `buf` (whose first pieces are already in fragment slot 0); if STORE,
@@ -213,18 +244,22 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
 
 // ---- host side ----
 
-// Whether this kernel takes the product: fp32, k <= 64 in whole 16-byte pieces, both operands contiguous along k with
+// Whether this kernel takes the product: fp32, k <= 64 in whole 16-byte pieces, both operands with a unit stride and
 // 16-byte aligned rows, C overwritten (no accumulation, bias, segments or folded store), and every byte offset the
 // kernel forms from a batch entry's base within the 32-bit range of buffer addressing.
 bool pipe32_takes(const GemmArgs& g) {
     if (g.k > S32_MAXK || g.k < 4 || g.k % 4 || g.m < 1 || g.n < 1 || g.batch < 1) return false;
     if ((long long)((g.m + S32_BM - 1) / S32_BM) * ((g.n + S32_BN - 1) / S32_BN) * g.batch >= (1ll << 30)) return false;
     if (g.bias || g.accumulate || g.seg_k || g.seg_n || g.c_fold_from || g.bias_by_row) return false;
-    if (g.a_cs != 1 || g.b_rs != 1 || g.a_rs % 4 || g.b_cs % 4 || g.a_bs % 4 || g.b_bs % 4 || g.a_rs < 0 || g.b_cs < 0 || g.c_rs < 0 || g.c_cs < 0) return false;
+    const bool a_kc = g.a_cs == 1 && g.a_rs % 4 == 0, a_mc = g.a_rs == 1 && g.a_cs % 4 == 0;
+    const bool b_kc = g.b_rs == 1 && g.b_cs % 4 == 0, b_mc = g.b_cs == 1 && g.b_rs % 4 == 0;
+    if (!(a_kc || a_mc) || !(b_kc || b_mc) || g.a_bs % 4 || g.b_bs % 4 || g.a_rs < 0 || g.a_cs < 0 || g.b_rs < 0 || g.b_cs < 0 || g.c_rs < 0 || g.c_cs < 0) return false;
     if (((uintptr_t)g.A & 15) || ((uintptr_t)g.B & 15) || ((uintptr_t)g.C & 3)) return false;
     const long long lim = 1ll << 30;
-    // rows up to a whole tile past the last one are addressed (and read as zero or dropped by the range check)
-    const long long a_reach = ((long long)(g.m + S32_BM) * g.a_rs + S32_MAXK) * 4, b_reach = ((long long)(g.n + S32_BN) * g.b_cs + S32_MAXK) * 4;
+    // free indices up to a whole tile past the last one are addressed (and read as zero, or as values that only reach
+    // outputs which are not stored)
+    const long long a_reach = (a_kc ? (long long)(g.m + S32_BM) * g.a_rs + S32_MAXK : (long long)S32_MAXK * g.a_cs + g.m + S32_BM) * 4;
+    const long long b_reach = (b_kc ? (long long)(g.n + S32_BN) * g.b_cs + S32_MAXK : (long long)S32_MAXK * g.b_rs + g.n + S32_BN) * 4;
     const long long c_reach = ((long long)(g.m + S32_BM) * g.c_rs + (long long)(g.n + S32_BN) * g.c_cs) * 4;
     return a_reach < lim && b_reach < lim && c_reach < lim;
 }
@@ -242,8 +277,16 @@ int launch_pipe32(const GemmArgs& g) {
         hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), smem, current_stream(), g, tiles_m, tiles_n, (unsigned)total);
         return check_launch("gemm_pipe32_kernel") ? 0 : -1;
     };
-    if (g.k <= 32) return edge ? launch(gemm_pipe32_kernel<4, true>) : launch(gemm_pipe32_kernel<4, false>);
-    return edge ? launch(gemm_pipe32_kernel<8, true>) : launch(gemm_pipe32_kernel<8, false>);
+    const bool a_mc = !(g.a_cs == 1 && g.a_rs % 4 == 0), b_mc = !(g.b_rs == 1 && g.b_cs % 4 == 0);
+    auto pick = [&](auto kch_c) {
+        constexpr int KCH = decltype(kch_c)::value;
+        if (!a_mc && !b_mc) return edge ? launch(gemm_pipe32_kernel<KCH, false, false, true>) : launch(gemm_pipe32_kernel<KCH, false, false, false>);
+        if (!a_mc && b_mc) return edge ? launch(gemm_pipe32_kernel<KCH, false, true, true>) : launch(gemm_pipe32_kernel<KCH, false, true, false>);
+        if (a_mc && !b_mc) return edge ? launch(gemm_pipe32_kernel<KCH, true, false, true>) : launch(gemm_pipe32_kernel<KCH, true, false, false>);
+        return edge ? launch(gemm_pipe32_kernel<KCH, true, true, true>) : launch(gemm_pipe32_kernel<KCH, true, true, false>);
+    };
+    if (g.k <= 32) return pick(std::integral_constant<int, 4>{});
+    return pick(std::integral_constant<int, 8>{});
 }
 
 }  // namespace rp

@@ -402,7 +402,7 @@ def test_fp32_short_reduction_batched(layout, batch, m, k, n):
     b = rand_storage(rng, (batch, k, n), F32) if layout[1] == "n" else rand_storage(rng, (batch, n, k), F32).transpose(0, 2, 1)
     a_rc, b_rc = [s // 4 for s in a.strides[1:]], [s // 4 for s in b.strides[1:]]
     kernel = capi.gemm_kernel_name(batch, m, k, n, a_rc, b_rc, (n, 1), F32)
-    if layout == "tn" and k > 32:
+    if layout == "tn" and k > 32 and m % 4 == 0 and n % 4 == 0:
         assert kernel == "direct32_128x128"
     elif m % 4 == 0 and n % 4 == 0 and k % 4 == 0:
         assert kernel == "mfma32_128x128"
@@ -420,12 +420,16 @@ PIPE32_SHAPES = [(16, 512, 64, 512), (20, 500, 64, 456), (48, 250, 44, 300), (32
                    (1, 2048, 64, 2048), (3, 1100, 60, 1300)]
 
 
+@pytest.mark.parametrize("layout", LAYOUTS)
 @pytest.mark.parametrize("batch,m,k,n", PIPE32_SHAPES)
-def test_fp32_pipelined_kernel_k_contiguous(batch, m, k, n):
+def test_fp32_pipelined_kernel(batch, m, k, n, layout):
     rng = np.random.default_rng(63)
-    a = rand_storage(rng, (batch, m, k), F32)
-    b = rand_storage(rng, (batch, n, k), F32).transpose(0, 2, 1)
-    assert capi.gemm_kernel_name(batch, m, k, n, (k, 1), (1, k), (n, 1), F32) == "pipe32_128x128"
+    # free-index-major operands need 16-byte aligned k rows: pad the storage, view the first m (n) entries
+    mp, npad = (m + 3) // 4 * 4, (n + 3) // 4 * 4
+    a = rand_storage(rng, (batch, m, k), F32) if layout[0] == "n" else rand_storage(rng, (batch, k, mp), F32)[:, :, :m].transpose(0, 2, 1)
+    b = rand_storage(rng, (batch, k, npad), F32)[:, :, :n] if layout[1] == "n" else rand_storage(rng, (batch, n, k), F32).transpose(0, 2, 1)
+    a_rc, b_rc = [x // 4 for x in a.strides[1:]], [x // 4 for x in b.strides[1:]]
+    assert capi.gemm_kernel_name(batch, m, k, n, a_rc, b_rc, (n, 1), F32) == "pipe32_128x128"
     got = device_gemm(a, b, F32)
     _check(got, a, b, F32, k)
     # a bias or an accumulated C is not this kernel's: the same call must still be right through the one that takes over
