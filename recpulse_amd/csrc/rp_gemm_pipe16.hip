@@ -26,42 +26,42 @@
 
 namespace rp {
 
-constexpr int S16_BM = 128, S16_BN = 128, S16_MAXK = 64;
-constexpr int S16_ROW_BYTES = 128;                                   // one LDS row: 64 16-bit values
-constexpr int S16_TILE_BYTES = (S16_BM + S16_BN) * S16_ROW_BYTES;    // 32 KB: A rows, then B rows
-constexpr int S16_NBUF = 3;                                          // LDS tiles in rotation
-constexpr uint32_t S16_OOB = 0x80000000u;
+constexpr int P16_BM = 128, P16_BN = 128, P16_MAXK = 64;
+constexpr int P16_ROW_BYTES = 128;                                   // one LDS row: 64 16-bit values
+constexpr int P16_TILE_BYTES = (P16_BM + P16_BN) * P16_ROW_BYTES;    // 32 KB: A rows, then B rows
+constexpr int P16_NBUF = 3;                                          // LDS tiles in rotation
+constexpr uint32_t P16_OOB = 0x80000000u;
 
-typedef __attribute__((address_space(3))) void* s16_lds_t;
+typedef __attribute__((address_space(3))) void* p16_lds_t;
 
 template <int I, int N, typename F>
-__device__ __forceinline__ void s16_static_for(F&& f) {
+__device__ __forceinline__ void p16_static_for(F&& f) {
     if constexpr (I < N) {
         f(std::integral_constant<int, I>{});
-        s16_static_for<I + 1, N>(f);
+        p16_static_for<I + 1, N>(f);
     }
 }
 
-struct S16Tile {
+struct P16Tile {
     int z, m0, n0;
 };
 
-__device__ __forceinline__ S16Tile s16_tile(unsigned id, unsigned per_matrix, unsigned tiles_n) {
-    S16Tile t;
+__device__ __forceinline__ P16Tile p16_tile(unsigned id, unsigned per_matrix, unsigned tiles_n) {
+    P16Tile t;
     const unsigned z = id / per_matrix, tile = id - z * per_matrix, tm = tile / tiles_n;
     t.z = (int)z;
-    t.m0 = (int)tm * S16_BM;
-    t.n0 = (int)(tile - tm * tiles_n) * S16_BN;
+    t.m0 = (int)tm * P16_BM;
+    t.n0 = (int)(tile - tm * tiles_n) * P16_BN;
     return t;
 }
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t s16_rsrc(const void* base, long long span_bytes) {
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t p16_rsrc(const void* base, long long span_bytes) {
     const int n = span_bytes <= 0 ? 0 : (span_bytes > 0x7fffffffll ? 0x7fffffff : (int)span_bytes);
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, n, 0x00020000);
 }
 
-template <typename T> struct s16_ops;
-template <> struct s16_ops<bf16_t> {
+template <typename T> struct p16_ops;
+template <> struct p16_ops<bf16_t> {
     static __device__ __forceinline__ f32x16_t mma(s16x8_t a, s16x8_t b, f32x16_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
     }
@@ -70,7 +70,7 @@ template <> struct s16_ops<bf16_t> {
         return __builtin_amdgcn_perm(__float_as_uint(hi) + 0x8000u, __float_as_uint(lo) + 0x8000u, 0x07060302u);
     }
 };
-template <> struct s16_ops<f16_t> {
+template <> struct p16_ops<f16_t> {
     static __device__ __forceinline__ f32x16_t mma(s16x8_t a, s16x8_t b, f32x16_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
     }
@@ -79,12 +79,12 @@ template <> struct s16_ops<f16_t> {
     }
 };
 
-typedef __attribute__((ext_vector_type(4))) short s16_s16x4_t;
+typedef __attribute__((ext_vector_type(4))) short p16_s16x4_t;
 
 // half H (k values 4H .. 4H + 3 of the lane's eight) of a fragment of an operand that lies in LDS as k rows
 template <int H>
-__device__ __forceinline__ void s16_read_tr(s16x8_t& v, const unsigned char* p) {
-    const s16_s16x4_t q = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16_s16x4_t __attribute__((address_space(3)))*)(p));
+__device__ __forceinline__ void p16_read_tr(s16x8_t& v, const unsigned char* p) {
+    const p16_s16x4_t q = __builtin_amdgcn_ds_read_tr16_b64_v4i16((p16_s16x4_t __attribute__((address_space(3)))*)(p));
     v[4 * H + 0] = q[0]; v[4 * H + 1] = q[1]; v[4 * H + 2] = q[2]; v[4 * H + 3] = q[3];
 }
 
@@ -117,49 +117,49 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
             const int krow = 4 * q + (lane >> 4);                       // k row within the wave's 16
             const int c32 = ((lane & 15) >> 1) ^ (krow & 7);            // which 32 bytes of the global k row (its half: lane & 1)
             const int free = (c32 * 2 + (lane & 1)) * 8;
-            a_off[q] = A_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * a_ks + free) * 2) : S16_OOB)
-                            : (piece * 8 < g.k ? (uint32_t)(((long long)row * a_fs + piece * 8) * 2) : S16_OOB);
-            b_off[q] = B_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * b_ks + free) * 2) : S16_OOB)
-                            : (piece * 8 < g.k ? (uint32_t)(((long long)row * b_fs + piece * 8) * 2) : S16_OOB);
+            a_off[q] = A_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * a_ks + free) * 2) : P16_OOB)
+                            : (piece * 8 < g.k ? (uint32_t)(((long long)row * a_fs + piece * 8) * 2) : P16_OOB);
+            b_off[q] = B_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * b_ks + free) * 2) : P16_OOB)
+                            : (piece * 8 < g.k ? (uint32_t)(((long long)row * b_fs + piece * 8) * 2) : P16_OOB);
         }
         auto fetch = [&](unsigned id, int buf) {
-            const S16Tile t = s16_tile(id, per_matrix, tiles_n);
-            const __amdgpu_buffer_rsrc_t ra = s16_rsrc((const uint16_t*)g.A + (long long)t.z * g.a_bs, a_span);
-            const __amdgpu_buffer_rsrc_t rb = s16_rsrc((const uint16_t*)g.B + (long long)t.z * g.b_bs, b_span);
+            const P16Tile t = p16_tile(id, per_matrix, tiles_n);
+            const __amdgpu_buffer_rsrc_t ra = p16_rsrc((const uint16_t*)g.A + (long long)t.z * g.a_bs, a_span);
+            const __amdgpu_buffer_rsrc_t rb = p16_rsrc((const uint16_t*)g.B + (long long)t.z * g.b_bs, b_span);
             const int sa = A_MC ? (int)(((long long)(16 * p) * a_ks + t.m0) * 2) : (int)((long long)(t.m0 + 32 * p) * a_fs * 2);
             const int sb = B_MC ? (int)(((long long)(16 * p) * b_ks + t.n0) * 2) : (int)((long long)(t.n0 + 32 * p) * b_fs * 2);
             // (both layouts put the wave's share at the same place: 32 rows of 128 bytes = 16 k rows of 256 bytes = 4 KB)
-            unsigned char* dst = p16_smem + buf * S16_TILE_BYTES + 32 * p * S16_ROW_BYTES;
+            unsigned char* dst = p16_smem + buf * P16_TILE_BYTES + 32 * p * P16_ROW_BYTES;
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (s16_lds_t)(dst + q * 1024), 16, (int)a_off[q], sa, 0, 0);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (s16_lds_t)(dst + S16_BM * S16_ROW_BYTES + q * 1024), 16, (int)b_off[q], sb, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (p16_lds_t)(dst + q * 1024), 16, (int)a_off[q], sa, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (p16_lds_t)(dst + P16_BM * P16_ROW_BYTES + q * 1024), 16, (int)b_off[q], sb, 0, 0);
             }
         };
         // The multipliers read tile t + 1 out of LDS while they multiply tile t, so at the barrier that starts tile t the
-        // loads of tile t + 1 must have landed and the LDS tile of tile t is free again: it takes tile t + S16_NBUF.  Loads
+        // loads of tile t + 1 must have landed and the LDS tile of tile t is free again: it takes tile t + P16_NBUF.  Loads
         // return in order, so "tile x has landed" is "at most the loads of the younger fetches are outstanding" (8
         // instructions per fetch); where a fetch was skipped because the tiles ran out, the wait is for everything.
         unsigned ahead = first;
         int fbuf = 0;
 #pragma unroll
-        for (int i = 0; i < S16_NBUF; i++) {
+        for (int i = 0; i < P16_NBUF; i++) {
             if (ahead < total) fetch(ahead, i);
             ahead += stride;
         }
         const bool full = ahead - stride < total;                      // every fetch above was issued
-        if (full) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(8 * (S16_NBUF - 1)) : "memory");
+        if (full) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(8 * (P16_NBUF - 1)) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();                                               // tile 0 is in LDS
-        if (full) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(8 * (S16_NBUF - 2)) : "memory");
+        if (full) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(8 * (P16_NBUF - 2)) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         for (unsigned id = first; id < total; id += stride) {
             __syncthreads();                                           // tile id + stride is in LDS; the LDS tile of tile id is free
             const bool more = ahead < total;
             if (more) fetch(ahead, fbuf);
             ahead += stride;
-            fbuf = fbuf + 1 == S16_NBUF ? 0 : fbuf + 1;
-            if (more) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(8 * (S16_NBUF - 2)) : "memory");
+            fbuf = fbuf + 1 == P16_NBUF ? 0 : fbuf + 1;
+            if (more) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(8 * (P16_NBUF - 2)) : "memory");
             else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
         return;
@@ -177,7 +177,7 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
 #pragma unroll
     for (int i = 0; i < 2; i++) {
         if (!A_MC) {
-            a_fr[0][i] = (uint32_t)((wm0 + 32 * i + r) * S16_ROW_BYTES + ((h ^ ((r >> 1) & 7)) * 16));
+            a_fr[0][i] = (uint32_t)((wm0 + 32 * i + r) * P16_ROW_BYTES + ((h ^ ((r >> 1) & 7)) * 16));
             a_fr[1][i] = 0;
         } else {
 #pragma unroll
@@ -187,13 +187,13 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
             }
         }
         if (!B_MC) {
-            b_fr[0][i] = (uint32_t)(S16_BM * S16_ROW_BYTES + (wn0 + 32 * i + r) * S16_ROW_BYTES + ((h ^ ((r >> 1) & 7)) * 16));
+            b_fr[0][i] = (uint32_t)(P16_BM * P16_ROW_BYTES + (wn0 + 32 * i + r) * P16_ROW_BYTES + ((h ^ ((r >> 1) & 7)) * 16));
             b_fr[1][i] = 0;
         } else {
 #pragma unroll
             for (int H = 0; H < 2; H++) {
                 const int krow = 8 * (grp >> 1) + 4 * H + (s16 >> 2), free = wn0 + 32 * i + 16 * (grp & 1) + 4 * (s16 & 3);
-                b_fr[H][i] = (uint32_t)(S16_BM * S16_ROW_BYTES + krow * 256 + (((free >> 4) ^ (krow & 7)) * 32) + (free & 15) * 2);
+                b_fr[H][i] = (uint32_t)(P16_BM * P16_ROW_BYTES + krow * 256 + (((free >> 4) ^ (krow & 7)) * 32) + (free & 15) * 2);
             }
         }
     }
@@ -201,8 +201,8 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     // swapped MFMA a lane holds row r of C and four adjacent columns per accumulator quad: 8 bytes, written at piece
     // 4 in + q, half h.  Read back, a lane holds 16 bytes of row lane / 8 (+ 8 per instruction), piece lane % 8: eight
     // whole 128-byte row segments per store instruction.
-    unsigned char* stage = p16_smem + S16_NBUF * S16_TILE_BYTES + wave * (64 * S16_ROW_BYTES);
-    const uint32_t st_write = (uint32_t)(r * S16_ROW_BYTES + 8 * h), st_swz = (uint32_t)((r >> 1) & 7);
+    unsigned char* stage = p16_smem + P16_NBUF * P16_TILE_BYTES + wave * (64 * P16_ROW_BYTES);
+    const uint32_t st_write = (uint32_t)(r * P16_ROW_BYTES + 8 * h), st_swz = (uint32_t)((r >> 1) & 7);
     const int rr = lane >> 3, rp = lane & 7;
     const uint32_t c_lane = (uint32_t)(((long long)rr * g.c_rs + 8 * rp) * 2);
     const long long c_span = ((long long)(g.m - 1) * g.c_rs + g.n) * 2;
@@ -213,31 +213,31 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     s16x8_t af[KST][2], bf[KST][2];     // [k step][tile]: eight k values of the lane's row
 
     auto pack_all = [&]() {
-        s16_static_for<0, 16>([&](auto nc) {
+        p16_static_for<0, 16>([&](auto nc) {
             constexpr int n = decltype(nc)::value, jm = n >> 3, in = (n >> 2) & 1, q = n & 3;
             const float v0 = acc[jm][in][4 * q], v1 = acc[jm][in][4 * q + 1], v2 = acc[jm][in][4 * q + 2], v3 = acc[jm][in][4 * q + 3];
-            packed[n][0] = s16_ops<T>::pack(v0, v1);
-            packed[n][1] = s16_ops<T>::pack(v2, v3);
+            packed[n][0] = p16_ops<T>::pack(v0, v1);
+            packed[n][1] = p16_ops<T>::pack(v2, v3);
         });
     };
     // staging write n (0..15): quad q of MFMA tile (jm, in)
     auto stage_write = [&](auto n_c) {
         constexpr int n = decltype(n_c)::value, jm = n >> 3, in = (n >> 2) & 1, q = n & 3;
-        *(u32x2_t*)(stage + st_write + 32 * jm * S16_ROW_BYTES + (((uint32_t)(4 * in + q) ^ st_swz) * 16)) = packed[n];
+        *(u32x2_t*)(stage + st_write + 32 * jm * P16_ROW_BYTES + (((uint32_t)(4 * in + q) ^ st_swz) * 16)) = packed[n];
     };
     // rows 8e .. 8e + 7 of the patch (e = 0..7): out of the staging patch (rows below 32 need staging writes 0..7 only) ...
     auto row_read = [&](auto e_c) {
         constexpr int e = decltype(e_c)::value;
         const int row = 8 * e + rr;
-        rows[e] = *(const u32x4_t*)(stage + row * S16_ROW_BYTES + (((uint32_t)rp ^ (uint32_t)((row >> 1) & 7)) * 16));
+        rows[e] = *(const u32x4_t*)(stage + row * P16_ROW_BYTES + (((uint32_t)rp ^ (uint32_t)((row >> 1) & 7)) * 16));
     };
     // ... and to memory
-    auto row_store = [&](auto e_c, const S16Tile& t, const __amdgpu_buffer_rsrc_t& rc) {
+    auto row_store = [&](auto e_c, const P16Tile& t, const __amdgpu_buffer_rsrc_t& rc) {
         constexpr int e = decltype(e_c)::value;
         const int gm = t.m0 + wm0 + 8 * e, gn = t.n0 + wn0;
         const int soff = (int)(((long long)gm * g.c_rs + gn) * 2);
         uint32_t voff = c_lane;
-        if constexpr (EDGE) voff = (gm + rr < g.m && gn + 8 * rp < g.n) ? c_lane : S16_OOB;      // (n is a multiple of 8: a piece is inside or outside as a whole)
+        if constexpr (EDGE) voff = (gm + rr < g.m && gn + 8 * rp < g.n) ? c_lane : P16_OOB;      // (n is a multiple of 8: a piece is inside or outside as a whole)
         __builtin_amdgcn_raw_buffer_store_b128(rows[e], rc, (int)voff, soff, 2);          // (streaming store: the output is not read again by this kernel)
     };
 
@@ -246,12 +246,12 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             if constexpr (!A_MC) af[s][i] = *(const s16x8_t*)(base + (a_fr[0][i] ^ (uint32_t)(32 * s)));
-            else { s16_read_tr<0>(af[s][i], base + a_fr[0][i] + 16 * s * 256); s16_read_tr<1>(af[s][i], base + a_fr[1][i] + 16 * s * 256); }
+            else { p16_read_tr<0>(af[s][i], base + a_fr[0][i] + 16 * s * 256); p16_read_tr<1>(af[s][i], base + a_fr[1][i] + 16 * s * 256); }
         }
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             if constexpr (!B_MC) bf[s][j] = *(const s16x8_t*)(base + (b_fr[0][j] ^ (uint32_t)(32 * s)));
-            else { s16_read_tr<0>(bf[s][j], base + b_fr[0][j] + 16 * s * 256); s16_read_tr<1>(bf[s][j], base + b_fr[1][j] + 16 * s * 256); }
+            else { p16_read_tr<0>(bf[s][j], base + b_fr[0][j] + 16 * s * 256); p16_read_tr<1>(bf[s][j], base + b_fr[1][j] + 16 * s * 256); }
         }
     };
 
@@ -259,35 +259,35 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     // are read (LDS tile `next`), so no MFMA ever waits for LDS.  If STORE, the previous tile (narrowed, in `packed`) goes
     // through the staging patch to memory meanwhile, in quarters of the MFMAs: staging writes 0..7 | writes 8..15 and row
     // reads 0..3 | row stores 0..3 and row reads 4..7 | row stores 4..7, so that no instruction waits for the one before it.
-    auto tile_pass = [&](auto store_c, int next, const S16Tile& prev) {
+    auto tile_pass = [&](auto store_c, int next, const P16Tile& prev) {
         constexpr bool STORE = decltype(store_c)::value;
         constexpr int NM = 4 * KST, Q = NM / 4;                    // MFMAs per tile and per quarter
         constexpr int WR = 8 / Q, RD = 4 / Q;                       // staging writes and row reads / stores per MFMA in their quarters
-        const unsigned char* next_base = p16_smem + next * S16_TILE_BYTES;
-        const __amdgpu_buffer_rsrc_t rc = s16_rsrc((uint16_t*)g.C + (long long)prev.z * g.c_bs, c_span);
+        const unsigned char* next_base = p16_smem + next * P16_TILE_BYTES;
+        const __amdgpu_buffer_rsrc_t rc = p16_rsrc((uint16_t*)g.C + (long long)prev.z * g.c_bs, c_span);
         __syncthreads();                                   // the next tile is in LDS; this tile's pieces have all arrived in registers
-        s16_static_for<0, KST>([&](auto sc) {
+        p16_static_for<0, KST>([&](auto sc) {
             constexpr int s = decltype(sc)::value;
-            s16_static_for<0, 4>([&](auto tc) {
+            p16_static_for<0, 4>([&](auto tc) {
                 constexpr int t4 = decltype(tc)::value, jm = t4 >> 1, in = t4 & 1, mi = s * 4 + t4, phase = mi / Q, idx = mi % Q;
                 // operands swapped: the MFMA's rows are columns of C
                 if constexpr (s == 0) {
                     const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                    acc[jm][in] = s16_ops<T>::mma(bf[s][in], af[s][jm], zero);
+                    acc[jm][in] = p16_ops<T>::mma(bf[s][in], af[s][jm], zero);
                 } else {
-                    acc[jm][in] = s16_ops<T>::mma(bf[s][in], af[s][jm], acc[jm][in]);
+                    acc[jm][in] = p16_ops<T>::mma(bf[s][in], af[s][jm], acc[jm][in]);
                 }
                 if constexpr (STORE) {
-                    if constexpr (phase == 0) s16_static_for<0, WR>([&](auto ec) { stage_write(std::integral_constant<int, idx * WR + decltype(ec)::value>{}); });
+                    if constexpr (phase == 0) p16_static_for<0, WR>([&](auto ec) { stage_write(std::integral_constant<int, idx * WR + decltype(ec)::value>{}); });
                     if constexpr (phase == 1) {
-                        s16_static_for<0, WR>([&](auto ec) { stage_write(std::integral_constant<int, 8 + idx * WR + decltype(ec)::value>{}); });
-                        s16_static_for<0, RD>([&](auto ec) { row_read(std::integral_constant<int, idx * RD + decltype(ec)::value>{}); });
+                        p16_static_for<0, WR>([&](auto ec) { stage_write(std::integral_constant<int, 8 + idx * WR + decltype(ec)::value>{}); });
+                        p16_static_for<0, RD>([&](auto ec) { row_read(std::integral_constant<int, idx * RD + decltype(ec)::value>{}); });
                     }
                     if constexpr (phase == 2) {
-                        s16_static_for<0, RD>([&](auto ec) { row_store(std::integral_constant<int, idx * RD + decltype(ec)::value>{}, prev, rc); });
-                        s16_static_for<0, RD>([&](auto ec) { row_read(std::integral_constant<int, 4 + idx * RD + decltype(ec)::value>{}); });
+                        p16_static_for<0, RD>([&](auto ec) { row_store(std::integral_constant<int, idx * RD + decltype(ec)::value>{}, prev, rc); });
+                        p16_static_for<0, RD>([&](auto ec) { row_read(std::integral_constant<int, 4 + idx * RD + decltype(ec)::value>{}); });
                     }
-                    if constexpr (phase == 3) s16_static_for<0, RD>([&](auto ec) { row_store(std::integral_constant<int, 4 + idx * RD + decltype(ec)::value>{}, prev, rc); });
+                    if constexpr (phase == 3) p16_static_for<0, RD>([&](auto ec) { row_store(std::integral_constant<int, 4 + idx * RD + decltype(ec)::value>{}, prev, rc); });
                     __builtin_amdgcn_sched_barrier(0);
                 }
             });
@@ -297,25 +297,25 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     };
 
     __syncthreads();                                   // the first tile is in LDS
-    S16Tile prev = {0, 0, 0};
+    P16Tile prev = {0, 0, 0};
     int next = 1;                                      // LDS tile of the tile after the current one
     unsigned id = first;
     if (id >= total) return;
-    s16_static_for<0, KST>([&](auto sc) { read_frags(p16_smem, sc); });
+    p16_static_for<0, KST>([&](auto sc) { read_frags(p16_smem, sc); });
     tile_pass(std::false_type{}, next, prev);
-    prev = s16_tile(id, per_matrix, tiles_n);
-    next = next + 1 == S16_NBUF ? 0 : next + 1;
+    prev = p16_tile(id, per_matrix, tiles_n);
+    next = next + 1 == P16_NBUF ? 0 : next + 1;
     id += stride;
     for (; id < total; id += stride) {
         tile_pass(std::true_type{}, next, prev);
-        prev = s16_tile(id, per_matrix, tiles_n);
-        next = next + 1 == S16_NBUF ? 0 : next + 1;
+        prev = p16_tile(id, per_matrix, tiles_n);
+        next = next + 1 == P16_NBUF ? 0 : next + 1;
     }
     // the last tile
-    const __amdgpu_buffer_rsrc_t rc = s16_rsrc((uint16_t*)g.C + (long long)prev.z * g.c_bs, c_span);
-    s16_static_for<0, 16>([&](auto nc) { stage_write(nc); });
-    s16_static_for<0, 8>([&](auto ec) { row_read(ec); });
-    s16_static_for<0, 8>([&](auto ec) { row_store(ec, prev, rc); });
+    const __amdgpu_buffer_rsrc_t rc = p16_rsrc((uint16_t*)g.C + (long long)prev.z * g.c_bs, c_span);
+    p16_static_for<0, 16>([&](auto nc) { stage_write(nc); });
+    p16_static_for<0, 8>([&](auto ec) { row_read(ec); });
+    p16_static_for<0, 8>([&](auto ec) { row_store(ec, prev, rc); });
 }
 
 // ---- host side ----
@@ -325,8 +325,8 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
 // segments or folded store), and every byte offset the kernel forms from a batch entry's base within the 32-bit range
 // of buffer addressing.
 bool pipe16_takes(const GemmArgs& g) {
-    if (g.k > S16_MAXK || g.k < 8 || g.k % 8 || g.m < 1 || g.n < 8 || g.n % 8 || g.batch < 1) return false;
-    if ((long long)((g.m + S16_BM - 1) / S16_BM) * ((g.n + S16_BN - 1) / S16_BN) * g.batch >= (1ll << 30)) return false;
+    if (g.k > P16_MAXK || g.k < 8 || g.k % 8 || g.m < 1 || g.n < 8 || g.n % 8 || g.batch < 1) return false;
+    if ((long long)((g.m + P16_BM - 1) / P16_BM) * ((g.n + P16_BN - 1) / P16_BN) * g.batch >= (1ll << 30)) return false;
     if (g.bias || g.accumulate || g.seg_k || g.seg_n || g.c_fold_from || g.bias_by_row) return false;
     const bool a_kc = g.a_cs == 1 && g.a_rs % 8 == 0, a_mc = g.a_rs == 1 && g.a_cs % 8 == 0;
     const bool b_kc = g.b_rs == 1 && g.b_cs % 8 == 0, b_mc = g.b_cs == 1 && g.b_rs % 8 == 0;
@@ -336,21 +336,21 @@ bool pipe16_takes(const GemmArgs& g) {
     const long long lim = 1ll << 30;
     // free indices up to a whole tile past the last one are addressed (and read as zero, or as values that only reach
     // outputs which are not stored)
-    const long long a_reach = (a_kc ? (long long)(g.m + S16_BM) * g.a_rs + S16_MAXK : (long long)S16_MAXK * g.a_cs + g.m + S16_BM) * 2;
-    const long long b_reach = (b_kc ? (long long)(g.n + S16_BN) * g.b_cs + S16_MAXK : (long long)S16_MAXK * g.b_rs + g.n + S16_BN) * 2;
-    const long long c_reach = ((long long)(g.m + S16_BM) * g.c_rs + g.n + S16_BN) * 2;
+    const long long a_reach = (a_kc ? (long long)(g.m + P16_BM) * g.a_rs + P16_MAXK : (long long)P16_MAXK * g.a_cs + g.m + P16_BM) * 2;
+    const long long b_reach = (b_kc ? (long long)(g.n + P16_BN) * g.b_cs + P16_MAXK : (long long)P16_MAXK * g.b_rs + g.n + P16_BN) * 2;
+    const long long c_reach = ((long long)(g.m + P16_BM) * g.c_rs + g.n + P16_BN) * 2;
     return a_reach < lim && b_reach < lim && c_reach < lim;
 }
 
 template <typename T>
 static int launch_pipe16_t(const GemmArgs& g) {
-    const int tiles_m = (g.m + S16_BM - 1) / S16_BM, tiles_n = (g.n + S16_BN - 1) / S16_BN;
+    const int tiles_m = (g.m + P16_BM - 1) / P16_BM, tiles_n = (g.n + P16_BN - 1) / P16_BN;
     const long long total = (long long)tiles_m * tiles_n * g.batch;
     int cus = device_cu_count();
     if (cus <= 0) cus = 256;
     const unsigned blocks = (unsigned)(total < cus ? total : cus);          // one resident workgroup per CU walks its tiles
-    const bool edge = (g.m % S16_BM) || (g.n % S16_BN);
-    constexpr int smem = S16_NBUF * S16_TILE_BYTES + 4 * 64 * S16_ROW_BYTES;          // the operand tiles and a staging patch per multiplying wave
+    const bool edge = (g.m % P16_BM) || (g.n % P16_BN);
+    constexpr int smem = P16_NBUF * P16_TILE_BYTES + 4 * 64 * P16_ROW_BYTES;          // the operand tiles and a staging patch per multiplying wave
     auto launch = [&](auto kern) {
         if (!check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem), "hipFuncSetAttribute")) return -1;
         hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), smem, current_stream(), g, tiles_m, tiles_n, (unsigned)total);

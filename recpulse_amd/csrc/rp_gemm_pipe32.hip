@@ -27,38 +27,38 @@
 
 namespace rp {
 
-constexpr int S32_BM = 128, S32_BN = 128, S32_MAXK = 64;
-constexpr int S32_ROW_BYTES = 256;                                   // one LDS row: 64 floats
-constexpr int S32_TILE_BYTES = (S32_BM + S32_BN) * S32_ROW_BYTES;    // 64 KB: A rows, then B rows
-constexpr uint32_t S32_OOB = 0x80000000u;
+constexpr int P32_BM = 128, P32_BN = 128, P32_MAXK = 64;
+constexpr int P32_ROW_BYTES = 256;                                   // one LDS row: 64 floats
+constexpr int P32_TILE_BYTES = (P32_BM + P32_BN) * P32_ROW_BYTES;    // 64 KB: A rows, then B rows
+constexpr uint32_t P32_OOB = 0x80000000u;
 
-typedef __attribute__((address_space(3))) void* s32_lds_t;
+typedef __attribute__((address_space(3))) void* p32_lds_t;
 
 template <int I, int N, typename F>
-__device__ __forceinline__ void s32_static_for(F&& f) {
+__device__ __forceinline__ void p32_static_for(F&& f) {
     if constexpr (I < N) {
         f(std::integral_constant<int, I>{});
-        s32_static_for<I + 1, N>(f);
+        p32_static_for<I + 1, N>(f);
     }
 }
 
-struct S32Tile {
+struct P32Tile {
     int z, m0, n0;
 };
 
-__device__ __forceinline__ S32Tile s32_tile(unsigned id, unsigned per_matrix, unsigned tiles_n) {
-    S32Tile t;
+__device__ __forceinline__ P32Tile p32_tile(unsigned id, unsigned per_matrix, unsigned tiles_n) {
+    P32Tile t;
     const unsigned z = id / per_matrix, tile = id - z * per_matrix, tm = tile / tiles_n;
     t.z = (int)z;
-    t.m0 = (int)tm * S32_BM;
-    t.n0 = (int)(tile - tm * tiles_n) * S32_BN;
+    t.m0 = (int)tm * P32_BM;
+    t.n0 = (int)(tile - tm * tiles_n) * P32_BN;
     return t;
 }
 
 // (a bit cast applied directly to one element of a vector reads the wrong element with this compiler: pass the element by value)
-__device__ __forceinline__ uint32_t s32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+__device__ __forceinline__ uint32_t p32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t s32_rsrc(const void* base, long long span_bytes) {
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t p32_rsrc(const void* base, long long span_bytes) {
     const int n = span_bytes <= 0 ? 0 : (span_bytes > 0x7fffffffll ? 0x7fffffff : (int)span_bytes);
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, n, 0x00020000);
 }
@@ -92,23 +92,23 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
             const int krow = 2 * q + (lane >> 5);                       // k row within the wave's 16
             const int c128 = ((lane & 31) >> 3) ^ ((krow >> 2) & 3);    // which 128 bytes of the global k row (its 16-byte piece: lane & 7)
             const int free = c128 * 32 + (lane & 7) * 4;
-            a_off[q] = A_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * a_ks + free) * 4) : S32_OOB)
-                            : (piece * 4 < g.k ? (uint32_t)(((long long)row * a_fs + piece * 4) * 4) : S32_OOB);
-            b_off[q] = B_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * b_ks + free) * 4) : S32_OOB)
-                            : (piece * 4 < g.k ? (uint32_t)(((long long)row * b_fs + piece * 4) * 4) : S32_OOB);
+            a_off[q] = A_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * a_ks + free) * 4) : P32_OOB)
+                            : (piece * 4 < g.k ? (uint32_t)(((long long)row * a_fs + piece * 4) * 4) : P32_OOB);
+            b_off[q] = B_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * b_ks + free) * 4) : P32_OOB)
+                            : (piece * 4 < g.k ? (uint32_t)(((long long)row * b_fs + piece * 4) * 4) : P32_OOB);
         }
         auto fetch = [&](unsigned id, int buf) {
-            const S32Tile t = s32_tile(id, per_matrix, tiles_n);
-            const __amdgpu_buffer_rsrc_t ra = s32_rsrc((const float*)g.A + (long long)t.z * g.a_bs, a_span);
-            const __amdgpu_buffer_rsrc_t rb = s32_rsrc((const float*)g.B + (long long)t.z * g.b_bs, b_span);
+            const P32Tile t = p32_tile(id, per_matrix, tiles_n);
+            const __amdgpu_buffer_rsrc_t ra = p32_rsrc((const float*)g.A + (long long)t.z * g.a_bs, a_span);
+            const __amdgpu_buffer_rsrc_t rb = p32_rsrc((const float*)g.B + (long long)t.z * g.b_bs, b_span);
             const int sa = A_MC ? (int)(((long long)(16 * p) * a_ks + t.m0) * 4) : (int)((long long)(t.m0 + 32 * p) * a_fs * 4);
             const int sb = B_MC ? (int)(((long long)(16 * p) * b_ks + t.n0) * 4) : (int)((long long)(t.n0 + 32 * p) * b_fs * 4);
             // (both layouts put the wave's share at the same place: 32 rows of 256 bytes = 16 k rows of 512 bytes = 8 KB)
-            unsigned char* dst = p32_smem + buf * S32_TILE_BYTES + 32 * p * S32_ROW_BYTES;
+            unsigned char* dst = p32_smem + buf * P32_TILE_BYTES + 32 * p * P32_ROW_BYTES;
 #pragma unroll
             for (int q = 0; q < 8; q++) {
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (s32_lds_t)(dst + q * 1024), 16, (int)a_off[q], sa, 0, 0);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (s32_lds_t)(dst + S32_BM * S32_ROW_BYTES + q * 1024), 16, (int)b_off[q], sb, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (p32_lds_t)(dst + q * 1024), 16, (int)a_off[q], sa, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (p32_lds_t)(dst + P32_BM * P32_ROW_BYTES + q * 1024), 16, (int)b_off[q], sb, 0, 0);
             }
         };
         if (first < total) fetch(first, 0);
@@ -130,9 +130,9 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
     // k-contiguous operand: the LDS byte address of piece 2u + h of this lane's row is lane_x ^ (32 u) (rows are 256-byte
     // aligned, so the XOR only touches the piece bits).  Other layout: the value of step (u, e), k row 8u + 4h + e, free
     // index w0 + 32 i + r, is at mc_x + (8u + e) k rows, in the 128-byte piece (w0 / 32 + i) ^ ((2u + h) % 4).
-    const uint32_t lane_a = (uint32_t)((wm0 + r) * S32_ROW_BYTES + ((h ^ (r & 15)) * 16));
-    const uint32_t lane_b = (uint32_t)(S32_BM * S32_ROW_BYTES + (wn0 + r) * S32_ROW_BYTES + ((h ^ (r & 15)) * 16));
-    const uint32_t mc_a = (uint32_t)(4 * h * 512 + r * 4), mc_b = (uint32_t)(S32_BM * S32_ROW_BYTES + 4 * h * 512 + r * 4);
+    const uint32_t lane_a = (uint32_t)((wm0 + r) * P32_ROW_BYTES + ((h ^ (r & 15)) * 16));
+    const uint32_t lane_b = (uint32_t)(P32_BM * P32_ROW_BYTES + (wn0 + r) * P32_ROW_BYTES + ((h ^ (r & 15)) * 16));
+    const uint32_t mc_a = (uint32_t)(4 * h * 512 + r * 4), mc_b = (uint32_t)(P32_BM * P32_ROW_BYTES + 4 * h * 512 + r * 4);
     const uint32_t c_lane = (uint32_t)(((long long)(4 * h) * g.c_rs + (long long)r * g.c_cs) * 4);
     const long long c_span = ((long long)(g.m - 1) * g.c_rs + (long long)(g.n - 1) * g.c_cs + 1) * 4;
 
@@ -140,23 +140,23 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
     f32x4_t af[2][2], bf[2][2];         // [slot][i or j]: four k values of the lane's row
 
     // store number n (0..63) of accumulator set SET: register v of MFMA tile (i, j), i.e. columns 32j + r of rows 32i + 8(v / 4) + 4h + v % 4
-    auto store_one = [&](auto set_c, auto n_c, const S32Tile& t, const __amdgpu_buffer_rsrc_t& rc) {
+    auto store_one = [&](auto set_c, auto n_c, const P32Tile& t, const __amdgpu_buffer_rsrc_t& rc) {
         constexpr int SET = decltype(set_c)::value, n = decltype(n_c)::value;
         constexpr int sj = n >> 5, si = (n >> 4) & 1, v = n & 15;
         constexpr int row = 32 * si + 8 * (v / 4) + (v % 4);
         const int gm = t.m0 + wm0 + row, gn = t.n0 + wn0 + 32 * sj;
         const int soff = (int)(((long long)gm * g.c_rs + (long long)gn * g.c_cs) * 4);
         uint32_t voff = c_lane;
-        if constexpr (EDGE) voff = (gm + 4 * h < g.m && gn + r < g.n) ? c_lane : S32_OOB;
+        if constexpr (EDGE) voff = (gm + 4 * h < g.m && gn + r < g.n) ? c_lane : P32_OOB;
         const float val = acc[SET][si][sj][v];
-        __builtin_amdgcn_raw_buffer_store_b32(s32_bits(val), rc, (int)voff, soff, 2);          // (streaming store: the output is not read again by this kernel)
+        __builtin_amdgcn_raw_buffer_store_b32(p32_bits(val), rc, (int)voff, soff, 2);          // (streaming store: the output is not read again by this kernel)
     };
 
     auto read_frags = [&](const unsigned char* base, int u, int slot) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             if constexpr (!A_MC) {
-                af[slot][i] = *(const f32x4_t*)(base + ((lane_a ^ (uint32_t)(32 * u)) + i * 32 * S32_ROW_BYTES));
+                af[slot][i] = *(const f32x4_t*)(base + ((lane_a ^ (uint32_t)(32 * u)) + i * 32 * P32_ROW_BYTES));
             } else {
                 const uint32_t at = mc_a + (uint32_t)(8 * u * 512) + ((((uint32_t)(wm0 >> 5) + i) ^ (uint32_t)((2 * u + h) & 3)) * 128);
 #pragma unroll
@@ -166,7 +166,7 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             if constexpr (!B_MC) {
-                bf[slot][j] = *(const f32x4_t*)(base + ((lane_b ^ (uint32_t)(32 * u)) + j * 32 * S32_ROW_BYTES));
+                bf[slot][j] = *(const f32x4_t*)(base + ((lane_b ^ (uint32_t)(32 * u)) + j * 32 * P32_ROW_BYTES));
             } else {
                 const uint32_t at = mc_b + (uint32_t)(8 * u * 512) + ((((uint32_t)(wn0 >> 5) + j) ^ (uint32_t)((2 * u + h) & 3)) * 128);
 #pragma unroll
@@ -179,13 +179,13 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
     // write set CUR ^ 1 (the tile `prev`) meanwhile.  The block's barrier sits before the last piece's MFMAs, when every
     // LDS read of this tile has returned: behind it the other LDS tile holds the next tile, whose first pieces are read
     // under those MFMAs, and the fetching waves may overwrite this one.
-    auto tile_pass = [&](auto cur_c, auto store_c, int buf, const S32Tile& prev) {
+    auto tile_pass = [&](auto cur_c, auto store_c, int buf, const P32Tile& prev) {
         constexpr int CUR = decltype(cur_c)::value;
         constexpr bool STORE = decltype(store_c)::value;
-        const unsigned char* base = p32_smem + buf * S32_TILE_BYTES;
-        const unsigned char* next_base = p32_smem + (buf ^ 1) * S32_TILE_BYTES;
-        const __amdgpu_buffer_rsrc_t rc = s32_rsrc((float*)g.C + (long long)prev.z * g.c_bs, c_span);
-        s32_static_for<0, KCH>([&](auto uc) {
+        const unsigned char* base = p32_smem + buf * P32_TILE_BYTES;
+        const unsigned char* next_base = p32_smem + (buf ^ 1) * P32_TILE_BYTES;
+        const __amdgpu_buffer_rsrc_t rc = p32_rsrc((float*)g.C + (long long)prev.z * g.c_bs, c_span);
+        p32_static_for<0, KCH>([&](auto uc) {
             constexpr int u = decltype(uc)::value, slot = u & 1;
             if constexpr (u + 1 < KCH) {
                 read_frags(base, u + 1, slot ^ 1);
@@ -193,7 +193,7 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
                 __syncthreads();
                 read_frags(next_base, 0, slot ^ 1);
             }
-            s32_static_for<0, 16>([&](auto sc) {
+            p32_static_for<0, 16>([&](auto sc) {
                 constexpr int s = decltype(sc)::value, e = s >> 2, i = (s >> 1) & 1, j = s & 1;
                 if constexpr (u == 0 && e == 0) {
                     const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -213,33 +213,33 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
     };
 
     __syncthreads();                                   // the first tile is in LDS
-    S32Tile prev = {0, 0, 0};
+    P32Tile prev = {0, 0, 0};
     int buf = 0, last = 0;
     unsigned id = first;
     if (id >= total) return;
     read_frags(p32_smem, 0, 0);
     tile_pass(std::integral_constant<int, 0>{}, std::false_type{}, buf, prev);
-    prev = s32_tile(id, per_matrix, tiles_n);
+    prev = p32_tile(id, per_matrix, tiles_n);
     buf ^= 1;
     id += stride;
     // two tiles per round, so that the accumulator sets are fixed registers
     while (id < total) {
         tile_pass(std::integral_constant<int, 1>{}, std::true_type{}, buf, prev);
-        prev = s32_tile(id, per_matrix, tiles_n);
+        prev = p32_tile(id, per_matrix, tiles_n);
         buf ^= 1;
         id += stride;
         last = 1;
         if (id >= total) break;
         tile_pass(std::integral_constant<int, 0>{}, std::true_type{}, buf, prev);
-        prev = s32_tile(id, per_matrix, tiles_n);
+        prev = p32_tile(id, per_matrix, tiles_n);
         buf ^= 1;
         id += stride;
         last = 0;
     }
     // the last tile's accumulators
-    const __amdgpu_buffer_rsrc_t rc = s32_rsrc((float*)g.C + (long long)prev.z * g.c_bs, c_span);
-    if (last == 0) s32_static_for<0, 64>([&](auto nc) { store_one(std::integral_constant<int, 0>{}, nc, prev, rc); });
-    else s32_static_for<0, 64>([&](auto nc) { store_one(std::integral_constant<int, 1>{}, nc, prev, rc); });
+    const __amdgpu_buffer_rsrc_t rc = p32_rsrc((float*)g.C + (long long)prev.z * g.c_bs, c_span);
+    if (last == 0) p32_static_for<0, 64>([&](auto nc) { store_one(std::integral_constant<int, 0>{}, nc, prev, rc); });
+    else p32_static_for<0, 64>([&](auto nc) { store_one(std::integral_constant<int, 1>{}, nc, prev, rc); });
 }
 
 // ---- host side ----
@@ -248,8 +248,8 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
 // 16-byte aligned rows, C overwritten (no accumulation, bias, segments or folded store), and every byte offset the
 // kernel forms from a batch entry's base within the 32-bit range of buffer addressing.
 bool pipe32_takes(const GemmArgs& g) {
-    if (g.k > S32_MAXK || g.k < 4 || g.k % 4 || g.m < 1 || g.n < 1 || g.batch < 1) return false;
-    if ((long long)((g.m + S32_BM - 1) / S32_BM) * ((g.n + S32_BN - 1) / S32_BN) * g.batch >= (1ll << 30)) return false;
+    if (g.k > P32_MAXK || g.k < 4 || g.k % 4 || g.m < 1 || g.n < 1 || g.batch < 1) return false;
+    if ((long long)((g.m + P32_BM - 1) / P32_BM) * ((g.n + P32_BN - 1) / P32_BN) * g.batch >= (1ll << 30)) return false;
     if (g.bias || g.accumulate || g.seg_k || g.seg_n || g.c_fold_from || g.bias_by_row) return false;
     const bool a_kc = g.a_cs == 1 && g.a_rs % 4 == 0, a_mc = g.a_rs == 1 && g.a_cs % 4 == 0;
     const bool b_kc = g.b_rs == 1 && g.b_cs % 4 == 0, b_mc = g.b_cs == 1 && g.b_rs % 4 == 0;
@@ -258,20 +258,20 @@ bool pipe32_takes(const GemmArgs& g) {
     const long long lim = 1ll << 30;
     // free indices up to a whole tile past the last one are addressed (and read as zero, or as values that only reach
     // outputs which are not stored)
-    const long long a_reach = (a_kc ? (long long)(g.m + S32_BM) * g.a_rs + S32_MAXK : (long long)S32_MAXK * g.a_cs + g.m + S32_BM) * 4;
-    const long long b_reach = (b_kc ? (long long)(g.n + S32_BN) * g.b_cs + S32_MAXK : (long long)S32_MAXK * g.b_rs + g.n + S32_BN) * 4;
-    const long long c_reach = ((long long)(g.m + S32_BM) * g.c_rs + (long long)(g.n + S32_BN) * g.c_cs) * 4;
+    const long long a_reach = (a_kc ? (long long)(g.m + P32_BM) * g.a_rs + P32_MAXK : (long long)P32_MAXK * g.a_cs + g.m + P32_BM) * 4;
+    const long long b_reach = (b_kc ? (long long)(g.n + P32_BN) * g.b_cs + P32_MAXK : (long long)P32_MAXK * g.b_rs + g.n + P32_BN) * 4;
+    const long long c_reach = ((long long)(g.m + P32_BM) * g.c_rs + (long long)(g.n + P32_BN) * g.c_cs) * 4;
     return a_reach < lim && b_reach < lim && c_reach < lim;
 }
 
 int launch_pipe32(const GemmArgs& g) {
-    const int tiles_m = (g.m + S32_BM - 1) / S32_BM, tiles_n = (g.n + S32_BN - 1) / S32_BN;
+    const int tiles_m = (g.m + P32_BM - 1) / P32_BM, tiles_n = (g.n + P32_BN - 1) / P32_BN;
     const long long total = (long long)tiles_m * tiles_n * g.batch;
     int cus = device_cu_count();
     if (cus <= 0) cus = 256;
     const unsigned blocks = (unsigned)(total < cus ? total : cus);          // one resident workgroup per CU walks its tiles
-    const bool edge = (g.m % S32_BM) || (g.n % S32_BN);
-    constexpr int smem = 2 * S32_TILE_BYTES;
+    const bool edge = (g.m % P32_BM) || (g.n % P32_BN);
+    constexpr int smem = 2 * P32_TILE_BYTES;
     auto launch = [&](auto kern) {
         if (!check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem), "hipFuncSetAttribute")) return -1;
         hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), smem, current_stream(), g, tiles_m, tiles_n, (unsigned)total);
