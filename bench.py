@@ -345,7 +345,7 @@ def f16_time(capi, n=8192):
     d_a, d_b = capi.DeviceBuffer.from_numpy(a), capi.DeviceBuffer.from_numpy(b)
     d_c = capi.DeviceBuffer(a.nbytes)
     s = (0, n, 1)
-    ms = _time_launches(capi, lambda: capi.gemm(d_c.ptr, d_a.ptr, d_b.ptr, None, 1, n, n, n, s, s, s, False, capi.F16), 10, 5)
+    ms = _time_launches(capi, lambda: capi.gemm(d_c.ptr, d_a.ptr, d_b.ptr, None, 1, n, n, n, s, s, s, False, capi.F16), 60, 15)       # as many launches as the headline times
     tf = 2.0 * n ** 3 / (ms * 1e-3) / 1e12
     for d in (d_a, d_b, d_c):
         d.free()
