@@ -315,7 +315,7 @@ int rp_hip_scatter_strided(void* dst, const void* src, int ndim, const int* shap
                            size_t size, int dtype);
 
 /* Fused attention forward: O[b] = softmax(scale * Q[b] * K[b]^T) * V[b], the score matrix never leaves the chip.
- * bfloat16 / float16 with d in {32, 64, 128}, float32 with d in {32, 64}.  Q, O: [batch, sq, d]; K, V: [batch, sk, d];
+ * bfloat16 / float16 / float32 with d in {32, 64, 128}.  Q, O: [batch, sq, d]; K, V: [batch, sk, d];
  * d contiguous (unit stride); *_bs / *_rs are the batch and row strides in elements (multiples of 16 bytes; operands
  * 16-byte aligned).  lse (may be NULL): float32 [batch, sq], log of the row sums of exp(scale * scores), for a backward
  * pass.  No counterpart in the reference, which composes the same value from op_matmul, op_mul_scalar, op_softmax and

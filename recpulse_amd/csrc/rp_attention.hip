@@ -610,7 +610,7 @@ extern "C" int rp_hip_attention_forward(void* O, const void* Q, const void* K, c
     if (dtype != RP_DTYPE_BFLOAT16 && dtype != RP_DTYPE_FLOAT16 && dtype != RP_DTYPE_FLOAT32) { set_error("rp_hip_attention_forward: bfloat16, float16 or float32 (dtype %d)", dtype); return -1; }
     const bool f32 = dtype == RP_DTYPE_FLOAT32;
     const long long esz = f32 ? 4 : 2, vec = 16 / esz;
-    if (f32 ? (d != 32 && d != 64) : (d != 32 && d != 64 && d != 128)) { set_error("rp_hip_attention_forward: head dimension %d (supported: 32, 64, and 128 for the 16-bit types)", d); return -1; }
+    if (d != 32 && d != 64 && d != 128) { set_error("rp_hip_attention_forward: head dimension %d (supported: 32, 64, 128)", d); return -1; }
     const long long strides[] = {q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs};
     for (long long s : strides)
         if (s < 0 || s % vec) { set_error("rp_hip_attention_forward: strides must be non-negative multiples of 16 bytes"); return -1; }
@@ -640,7 +640,7 @@ extern "C" int rp_hip_attention_backward(void* dQ, void* dK, void* dV, const voi
     if (dtype != RP_DTYPE_BFLOAT16 && dtype != RP_DTYPE_FLOAT16 && dtype != RP_DTYPE_FLOAT32) { set_error("rp_hip_attention_backward: bfloat16, float16 or float32 (dtype %d)", dtype); return -1; }
     const bool f32 = dtype == RP_DTYPE_FLOAT32;
     const long long esz = f32 ? 4 : 2, vec = 16 / esz;
-    if (f32 ? (d != 32 && d != 64) : (d != 32 && d != 64 && d != 128)) { set_error("rp_hip_attention_backward: head dimension %d (supported: 32, 64, and 128 for the 16-bit types)", d); return -1; }
+    if (d != 32 && d != 64 && d != 128) { set_error("rp_hip_attention_backward: head dimension %d (supported: 32, 64, 128)", d); return -1; }
     const long long strides[] = {q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, o_bs, o_rs, do_bs, do_rs};
     for (long long s : strides)
         if (s < 0 || s % vec) { set_error("rp_hip_attention_backward: strides must be non-negative multiples of 16 bytes"); return -1; }

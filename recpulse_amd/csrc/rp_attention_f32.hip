@@ -1,4 +1,4 @@
-// Fused attention for float32 (head dimension 32 or 64): forward, and the dQ and dK/dV kernels of the backward.
+// Fused attention for float32 (head dimension 32, 64 or 128): forward, and the dQ and dK/dV kernels of the backward.
 //
 // Same decomposition as the 16-bit kernels (a workgroup owns 128 queries or keys, a wave 32 of them; S^T, P^T, O^T are
 // kept transposed so that a lane owns one query of the forward and of the dQ kernel, one key of the dK/dV kernel), on
@@ -98,7 +98,7 @@ __device__ __forceinline__ void write_rows_t(float* row, const f32x16_t (&acc)[D
 }
 
 template <int D>
-__global__ void __launch_bounds__(256, 2) attention_fwd32_kernel(AttnArgs g) {
+__global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) attention_fwd32_kernel(AttnArgs g) {
     constexpr int KJ = D / 2, DT = D / 32;
     using Blk = Blk32<D>;
     __shared__ __attribute__((aligned(16))) float klds[2][Blk::ELEMS];
@@ -197,7 +197,7 @@ __global__ void __launch_bounds__(256, 2) attention_fwd32_kernel(AttnArgs g) {
 
 // dQ: a wave owns 32 queries and walks the keys.
 template <int D>
-__global__ void __launch_bounds__(256, 2) attention_bwd_dq32_kernel(AttnBwdArgs g) {
+__global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) attention_bwd_dq32_kernel(AttnBwdArgs g) {
     constexpr int KJ = D / 2, DT = D / 32;
     using Blk = Blk32<D>;
     __shared__ __attribute__((aligned(16))) float klds[2][Blk::ELEMS];
@@ -377,7 +377,8 @@ int launch_attention_f32(const AttnArgs& g, int d) {
     switch (d) {
         case 32: hipLaunchKernelGGL((attention_fwd32_kernel<32>), grid, dim3(256), 0, current_stream(), g); break;
         case 64: hipLaunchKernelGGL((attention_fwd32_kernel<64>), grid, dim3(256), 0, current_stream(), g); break;
-        default: set_error("rp_hip_attention_forward: float32 head dimension %d (supported: 32, 64)", d); return -1;
+        case 128: hipLaunchKernelGGL((attention_fwd32_kernel<128>), grid, dim3(256), 0, current_stream(), g); break;      // (68 KB of static LDS: one workgroup per CU)
+        default: set_error("rp_hip_attention_forward: float32 head dimension %d (supported: 32, 64, 128)", d); return -1;
     }
     return check_launch("attention_fwd32_kernel") ? 0 : -1;
 }
@@ -393,7 +394,11 @@ int launch_attention_bwd_f32(const AttnBwdArgs& g, int d) {
             hipLaunchKernelGGL((attention_bwd_dq32_kernel<64>), gq, dim3(256), 0, current_stream(), g);
             hipLaunchKernelGGL((attention_bwd_dkv32_kernel<64>), gk, dim3(256), 0, current_stream(), g);
             break;
-        default: set_error("rp_hip_attention_backward: float32 head dimension %d (supported: 32, 64)", d); return -1;
+        case 128:
+            hipLaunchKernelGGL((attention_bwd_dq32_kernel<128>), gq, dim3(256), 0, current_stream(), g);
+            hipLaunchKernelGGL((attention_bwd_dkv32_kernel<128>), gk, dim3(256), 0, current_stream(), g);
+            break;
+        default: set_error("rp_hip_attention_backward: float32 head dimension %d (supported: 32, 64, 128)", d); return -1;
     }
     return check_launch("attention backward kernels (float32)") ? 0 : -1;
 }

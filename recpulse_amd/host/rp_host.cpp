@@ -1188,8 +1188,8 @@ Tensor* op_linear(Tensor* x, Tensor* w, Tensor* bias) {
     return out;
 }
 
-// O = softmax(scale · Q · Kᵀ) · V in one launch (extension; bfloat16 / float16 with head dimension 32, 64 or 128,
-// float32 with 32 or 64).
+// O = softmax(scale · Q · Kᵀ) · V in one launch (extension; bfloat16, float16 or float32 with head dimension 32, 64 or
+// 128).
 // q: [..., sq, d], k and v: [..., sk, d] with equal leading dims.  Equals q.op_matmul(kᵀ).op_mul_scalar(scale)
 // .op_softmax(-1).op_matmul(v) up to the roundings of the score matrix that the fused kernel does not make.
 Tensor* op_attention(Tensor* q, Tensor* k, Tensor* v, double scale) {

@@ -43,8 +43,6 @@ BWD_TOL = {BF16: 2e-2, F16: 4e-3, F32: 1e-5}
                          ids=lambda s: "x".join(map(str, s)))
 def test_fused_attention_forward(dt, shape):
     Z, sq, sk, d = shape
-    if dt == F32 and d == 128:
-        pytest.skip("float32 kernels cover head dimensions 32 and 64 (the call is rejected: see the argument test)")
     rng = np.random.default_rng(60)
     q, k, v = rand_storage(rng, (Z, sq, d), dt), rand_storage(rng, (Z, sk, d), dt), rand_storage(rng, (Z, sk, d), dt)
     scale = 1.0 / np.sqrt(d)
@@ -79,7 +77,7 @@ def test_fused_attention_rejects_bad_arguments():
     assert L.rp_hip_attention_forward(d.ptr, d.ptr, d.ptr, d.ptr, None, 1, 4, 4, 48, 192, 48, 192, 48, 192, 48, 192, 48, 1.0, BF16) == -1
     assert b"head dimension" in L.rp_hip_last_error()
     assert L.rp_hip_attention_forward(d.ptr, d.ptr, d.ptr, d.ptr, None, 1, 4, 4, 64, 256, 64, 256, 64, 256, 64, 256, 64, 1.0, capi.F64) == -1
-    assert L.rp_hip_attention_forward(d.ptr, d.ptr, d.ptr, d.ptr, None, 1, 4, 4, 128, 512, 128, 512, 128, 512, 128, 512, 128, 1.0, capi.F32) == -1
+    assert L.rp_hip_attention_forward(d.ptr, d.ptr, d.ptr, d.ptr, None, 1, 4, 4, 96, 384, 96, 384, 96, 384, 96, 384, 96, 1.0, capi.F32) == -1
     assert L.rp_hip_attention_forward(d.ptr, d.ptr, d.ptr, d.ptr, None, 1, 4, 4, 64, 256, 66, 256, 64, 256, 64, 256, 64, 1.0, capi.F32) == -1      # row stride not a multiple of 16 bytes
     assert L.rp_hip_attention_forward(d.ptr, d.ptr, d.ptr, d.ptr, None, 1, 4, 4, 64, 256, 60, 256, 64, 256, 64, 256, 64, 1.0, BF16) == -1
 
@@ -116,8 +114,6 @@ def _fused_backward(q, k, v, g, dt, scale):
                          ids=lambda s: "x".join(map(str, s)))
 def test_fused_attention_backward(dt, shape):
     Z, sq, sk, d = shape
-    if dt == F32 and d == 128:
-        pytest.skip("float32 kernels cover head dimensions 32 and 64")
     rng = np.random.default_rng(62)
     q, k, v = rand_storage(rng, (Z, sq, d), dt), rand_storage(rng, (Z, sk, d), dt), rand_storage(rng, (Z, sk, d), dt)
     g = rand_storage(rng, (Z, sq, d), dt)
@@ -153,7 +149,7 @@ def test_fused_attention_backward_rejects_bad_arguments():
     assert b"head dimension" in L.rp_hip_last_error()
     assert L.rp_hip_attention_backward(p, p, p, p, p, p, p, p, None, 1, 4, 4, 64, 256, 64, 256, 64, 256, 64, 256, 64, 256, 64, 1.0, BF16) == -1
     assert L.rp_hip_attention_backward(p, p, p, p, p, p, p, p, p, 1, 4, 4, 64, 256, 64, 256, 64, 256, 64, 256, 64, 256, 64, 1.0, capi.F64) == -1
-    assert L.rp_hip_attention_backward(p, p, p, p, p, p, p, p, p, 1, 4, 4, 128, 512, 128, 512, 128, 512, 128, 512, 128, 512, 128, 1.0, capi.F32) == -1
+    assert L.rp_hip_attention_backward(p, p, p, p, p, p, p, p, p, 1, 4, 4, 96, 384, 96, 384, 96, 384, 96, 384, 96, 384, 96, 1.0, capi.F32) == -1
 
 
 def test_fused_attention_batch_longer_than_a_grid_axis():
