@@ -449,6 +449,9 @@ def attention_times(capi, dt_name="bf16"):
     }
     for fn, _, _ in ops.values():        # eager once, in dependency order, so every buffer holds finite values
         fn()
+    kn = lambda m, k, n, a_rc, b_rc: capi.gemm_kernel_name(Z, m, k, n, a_rc, b_rc, (n, 1), dt)
+    gemm_names = {"S=Q.Kt": kn(S, D, S, (D, 1), (1, D)), "dP=dO.Vt": kn(S, D, S, (D, 1), (1, D)), "O=P.V": kn(S, S, D, (S, 1), (D, 1)),
+                  "dQ=dS.K": kn(S, S, D, (S, 1), (D, 1)), "dV=Pt.dO": kn(S, S, D, (1, S), (D, 1)), "dK=dSt.Q": kn(S, S, D, (1, S), (D, 1))}
     out, total = {}, 0.0
     for _ in range(300):                 # the clock the power management grants settles within some tens of milliseconds of load
         ops["S=Q.Kt"][0]()
@@ -459,6 +462,7 @@ def attention_times(capi, dt_name="bf16"):
         if flops:
             out[name]["TFLOP/s"] = round(flops / ms / 1e9, 1)
             out[name]["frac_mfma"] = round(flops / ms / 1e9 / PEAK_TFLOPS[dt_name], 3)       # these GEMMs sit near the ridge: both fractions are given
+            out[name]["kernel"] = gemm_names[name]
     out["fwd_bwd_ms"] = round(total + out["scale"]["us"] * 1e-3, 4)     # the scale runs twice (S/8 and dS/8)
     # the same forward (S, scale, softmax, O) as one fused kernel that never writes S or P
     fused = lambda: capi.check(L.rp_hip_attention_forward(d_o.ptr, d_q.ptr, d_k.ptr, d_v.ptr, None, Z, S, S, D,
