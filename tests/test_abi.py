@@ -57,5 +57,17 @@ def test_kernel_selection_names():
     assert name(64, 64, 576, 3136, (576, 1), (3136, 1), (3136, 1), capi.BF16) == "mfma16_64x128"           # at most 64 rows, short k (a lowered convolution)
     assert name(64, 64, 3136, 576, (3136, 1), (1, 3136), (576, 1), capi.F16) == "mfma16_64x256"            # at most 64 rows, long k (its weight gradient)
     assert name(1, 64, 1024, 4096, (1024, 1), (4096, 1), (4096, 1), capi.BF16) == "mfma16_64x64"           # too few column tiles for the wide ones
+    # configuration 4 per head, and shapes like it: the resident kernels
+    Z, S, D = 192, 512, 64
+    for dt, short_k, narrow in ((capi.BF16, "pipe16_128x128", "pipe16k_128x64"), (capi.F16, "pipe16_128x128", "pipe16k_128x64"), (capi.F32, "pipe32_128x128", "pipe32k_128x64")):
+        assert name(Z, S, D, S, (D, 1), (1, D), (S, 1), dt) == short_k                 # S = Q.K^T, K^T a stride view
+        assert name(Z, S, S, D, (S, 1), (D, 1), (D, 1), dt) == narrow                  # O = P.V
+        assert name(Z, S, S, D, (1, S), (D, 1), (D, 1), dt) == narrow                  # dV = P^T.dO
+        assert name(64, 576, D, 3136, (1, 576), (3136, 1), (3136, 1), dt) == short_k   # the lowered convolution's dcol = W^T.dy
+    assert name(8, S, D, S, (D, 1), (1, D), (S, 1), capi.BF16) == "mfma16_128x128"       # fewer tiles than CUs: the tiled kernels
+    assert name(8, S, D, S, (D, 1), (1, D), (S, 1), capi.F32) == "mfma32_128x128"
+    assert name(Z, S, 128, S, (128, 1), (1, 128), (S, 1), capi.BF16) == "mfma16_128x128"  # k above 64
+    assert name(Z, S, S, 128, (S, 1), (128, 1), (128, 1), capi.F32) == "mfma32_128x128"   # more than 64 columns
+    assert name(Z, S, D, S, (D, 1), (1, D), (1, S), capi.BF16) == "mfma16_128x128"        # 16-bit C not row-major
     assert name(1, 5, 7, 3, (7, 1), (3, 1), (3, 1), capi.BF16) == "generic"                                # odd extents
     assert name(1, 64, 64, 64, (128, 2), (64, 1), (64, 1), capi.F64) == "generic"                          # no unit stride
