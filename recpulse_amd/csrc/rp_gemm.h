@@ -149,15 +149,20 @@ int launch_skinny(const GemmArgs& g, int dtype);
 int launch_mfma16(const GemmArgs& g, const Plan& p, int dtype);
 int launch_mfmaw(const GemmArgs& g, const Plan& p, int dtype);
 int launch_tiny(const GemmArgs& g, int dtype);
-// Tiles [first, last) of `total` for this workgroup of a grid of resident workgroups (one per CU): a contiguous run, so
-// that a workgroup's consecutive tiles share operand rows, and runs that are neighbours in tile order on the same XCD
-// (workgroups go to the XCDs round robin), so that what they share is fetched into one L2 only.
-__device__ __forceinline__ void resident_tile_run(unsigned total, unsigned& first, unsigned& last) {
+// The tiles of this workgroup in a grid of resident workgroups (one per CU): first, first + stride, ... below last.
+// Workgroups go to the XCDs round robin, so workgroup b sits on XCD b % 8.  Every XCD gets a contiguous eighth of the
+// tiles, and its workgroups walk that range side by side: at any time the CUs of an XCD work on neighbouring tiles,
+// and what those share (the rows of Q and K of a batch entry, the whole of V) is fetched into that XCD's L2 once, while
+// it is still needed.  (A contiguous run per workgroup shares as much in total, but at different times: by the time
+// the second tile of a batch entry comes up on another CU, the first one's operands have left the L2.)
+__device__ __forceinline__ void resident_tile_walk(unsigned total, unsigned& first, unsigned& last, unsigned& stride) {
     const unsigned grid = gridDim.x, b = blockIdx.x;
-    const unsigned w = (grid % 8 == 0) ? (b % 8) * (grid / 8) + b / 8 : b;
-    const unsigned run = (total + grid - 1) / grid;
-    first = w * run < total ? w * run : total;
-    last = first + run < total ? first + run : total;
+    if (grid % 8 != 0) { first = b; last = total; stride = grid; return; }
+    const unsigned xcd = b % 8, slot = b / 8, per_xcd = (total + 7) / 8;
+    const unsigned begin = xcd * per_xcd < total ? xcd * per_xcd : total;
+    last = begin + per_xcd < total ? begin + per_xcd : total;
+    first = begin + slot < last ? begin + slot : last;
+    stride = grid / 8;
 }
 
 bool direct32_takes(const GemmArgs& g);          // pointer alignment and spans the short-k fp32 kernel can address

@@ -97,10 +97,9 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     extern __shared__ __attribute__((aligned(1024))) unsigned char p16_smem[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const unsigned per_matrix = (unsigned)(tiles_m * tiles_n);
-    unsigned first, last;
-    resident_tile_run(total, first, last);
-    total = last;                                                   // this workgroup's tiles are [first, total)
-    constexpr unsigned stride = 1;
+    unsigned first, walk_end, stride;
+    resident_tile_walk(total, first, walk_end, stride);
+    total = walk_end;                                               // this workgroup's tiles: first, first + stride, ... below total
     const long long a_fs = g.a_rs, a_ks = g.a_cs, b_fs = g.b_cs, b_ks = g.b_rs;      // strides of the free index and of k
     const long long a_span = (A_MC ? ((long long)(g.k - 1) * a_ks + g.m) : ((long long)(g.m - 1) * a_fs + g.k)) * 2;
     const long long b_span = (B_MC ? ((long long)(g.k - 1) * b_ks + g.n) : ((long long)(g.n - 1) * b_fs + g.k)) * 2;

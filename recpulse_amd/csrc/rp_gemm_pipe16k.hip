@@ -82,10 +82,9 @@ template <typename T, bool A_MC, bool B_MC, bool EDGE>
 __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles_m, unsigned total) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char k16_smem[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    unsigned first, last;
-    resident_tile_run(total, first, last);
-    total = last;                                                   // this workgroup's tiles are [first, total)
-    constexpr unsigned stride = 1;
+    unsigned first, walk_end, stride;
+    resident_tile_walk(total, first, walk_end, stride);
+    total = walk_end;                                               // this workgroup's tiles: first, first + stride, ... below total
     const int nslab = (g.k + K16_BK - 1) / K16_BK;
     const long long a_fs = g.a_rs, a_ks = g.a_cs, b_fs = g.b_cs, b_ks = g.b_rs;      // strides of the free index and of k
 

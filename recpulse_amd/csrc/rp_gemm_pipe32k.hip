@@ -54,9 +54,9 @@ template <bool A_MC, bool B_MC, bool EDGE>
 __global__ void __launch_bounds__(512) gemm_pipe32k_kernel(GemmArgs g, int tiles_m, unsigned total) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char k32_smem[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    unsigned first, run_end;
-    resident_tile_run(total, first, run_end);
-    total = run_end;                                                // this workgroup's tiles are [first, total)
+    unsigned first, walk_end, stride;
+    resident_tile_walk(total, first, walk_end, stride);
+    total = walk_end;                                               // this workgroup's tiles: first, first + stride, ... below total
     const int nslab = (g.k + K32_BK - 1) / K32_BK;
     const long long a_fs = g.a_rs, a_ks = g.a_cs, b_fs = g.b_cs, b_ks = g.b_rs;      // strides of the free index and of k
 
@@ -117,7 +117,7 @@ __global__ void __launch_bounds__(512) gemm_pipe32k_kernel(GemmArgs g, int tiles
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (k32_lds_t)(dst + K32_A_BYTES + (B_MC ? 8 * p * 256 : 16 * p * 128) + q * 1024), 16,
                                                          b_k[q] < kleft ? (int)b_off[q] : (int)K32_OOB, sb, 0, 0);
             f_stage = f_stage + 1 == K32_NBUF ? 0 : f_stage + 1;
-            if (++f_s == nslab) { f_s = 0; f_id += 1; }
+            if (++f_s == nslab) { f_s = 0; f_id += stride; }
             return true;
         };
         // Loads return in order, so "slab x has landed" is "at most the loads of the younger fetches are outstanding";
@@ -130,7 +130,7 @@ __global__ void __launch_bounds__(512) gemm_pipe32k_kernel(GemmArgs g, int tiles
         __syncthreads();                                               // slab 0 is in LDS
         if (full) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(K32_FETCH * (K32_NBUF - 2)) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        for (unsigned id = first; id < total; id += 1) {
+        for (unsigned id = first; id < total; id += stride) {
             for (int s = 0; s < nslab; s++) {
                 __syncthreads();                                       // the next slab is in LDS; the stage of this one is free
                 if (fetch_next()) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(K32_FETCH * (K32_NBUF - 2)) : "memory");
@@ -199,7 +199,7 @@ __global__ void __launch_bounds__(512) gemm_pipe32k_kernel(GemmArgs g, int tiles
     if (first >= total) return;
     k32_static_for<0, 4>([&](auto uc) { read_group(k32_smem, uc); });
     int next = 1;
-    for (unsigned id = first; id < total; id += 1) {
+    for (unsigned id = first; id < total; id += stride) {
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
