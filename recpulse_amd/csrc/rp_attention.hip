@@ -58,8 +58,9 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_fwd16_kernel(A
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int h = lane >> 5, c = lane & 31;
-    const int z = blockIdx.y;
-    const int q0 = blockIdx.x * AT_QROWS + wave * 32;               // this wave's first query row
+    int row_tile, z;
+    attn_block(row_tile, z);
+    const int q0 = row_tile * AT_QROWS + wave * 32;               // this wave's first query row
     const uint16_t* Q = (const uint16_t*)g.Q + (long long)z * g.q_bs;
     const uint16_t* K = (const uint16_t*)g.K + (long long)z * g.k_bs;
     const uint16_t* V = (const uint16_t*)g.V + (long long)z * g.v_bs;
@@ -322,8 +323,9 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_bwd_dq16_kerne
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int h = lane >> 5, c = lane & 31;
-    const int z = blockIdx.y;
-    const int q0 = blockIdx.x * AT_QROWS + wave * 32;
+    int row_tile, z;
+    attn_block(row_tile, z);
+    const int q0 = row_tile * AT_QROWS + wave * 32;
     const uint16_t* Q = (const uint16_t*)g.Q + (long long)z * g.q_bs;
     const uint16_t* K = (const uint16_t*)g.K + (long long)z * g.k_bs;
     const uint16_t* V = (const uint16_t*)g.V + (long long)z * g.v_bs;
@@ -448,8 +450,9 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) attention_bwd_dkv16_kern
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int h = lane >> 5, c = lane & 31;
-    const int z = blockIdx.y;
-    const int k0 = blockIdx.x * AT_QROWS + wave * 32;               // this wave's first key
+    int row_tile, z;
+    attn_block(row_tile, z);
+    const int k0 = row_tile * AT_QROWS + wave * 32;               // this wave's first key
     const uint16_t* Q = (const uint16_t*)g.Q + (long long)z * g.q_bs;
     const uint16_t* K = (const uint16_t*)g.K + (long long)z * g.k_bs;
     const uint16_t* V = (const uint16_t*)g.V + (long long)z * g.v_bs;

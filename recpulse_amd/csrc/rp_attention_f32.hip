@@ -106,8 +106,9 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) attention_fwd32_kernel(A
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int h = lane >> 5, c = lane & 31;
-    const int z = blockIdx.y;
-    const int q0 = blockIdx.x * AT_QROWS + wave * 32;
+    int row_tile, z;
+    attn_block(row_tile, z);
+    const int q0 = row_tile * AT_QROWS + wave * 32;
     const float* Q = (const float*)g.Q + (long long)z * g.q_bs;
     const float* K = (const float*)g.K + (long long)z * g.k_bs;
     const float* V = (const float*)g.V + (long long)z * g.v_bs;
@@ -205,8 +206,9 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) attention_bwd_dq32_kerne
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int h = lane >> 5, c = lane & 31;
-    const int z = blockIdx.y;
-    const int q0 = blockIdx.x * AT_QROWS + wave * 32;
+    int row_tile, z;
+    attn_block(row_tile, z);
+    const int q0 = row_tile * AT_QROWS + wave * 32;
     const float* Q = (const float*)g.Q + (long long)z * g.q_bs;
     const float* K = (const float*)g.K + (long long)z * g.k_bs;
     const float* V = (const float*)g.V + (long long)z * g.v_bs;
@@ -289,8 +291,9 @@ __global__ void __launch_bounds__(256, D <= 32 ? 2 : 1) attention_bwd_dkv32_kern
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int h = lane >> 5, c = lane & 31;
-    const int z = blockIdx.y;
-    const int k0 = blockIdx.x * AT_QROWS + wave * 32;
+    int row_tile, z;
+    attn_block(row_tile, z);
+    const int k0 = row_tile * AT_QROWS + wave * 32;
     const float* Q = (const float*)g.Q + (long long)z * g.q_bs;
     const float* K = (const float*)g.K + (long long)z * g.k_bs;
     const float* V = (const float*)g.V + (long long)z * g.v_bs;
