@@ -170,13 +170,14 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     constexpr int NMFMA = TMI * TNI;
     extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
 
-    const int z = blockIdx.y;
+    int first_slot, z;
+    batched_block(tiles_m, tiles_n, first_slot, z);
     // A workgroup walks the schedule with the grid's stride.  The launcher starts one workgroup per slot of the schedule,
     // except for the 256 x 256 tile, which fills a CU by itself: there one workgroup per CU stays resident and takes its
     // tiles one after the other, so that a tile's output stores drain, and the next tile's first loads fly, while MFMAs
     // run; a workgroup per tile would hold the CU idle until its last store was acknowledged.  A stride that is a
     // multiple of 8 keeps a workgroup's tiles on the XCD the schedule assigned them to.
-    for (int tile_id = blockIdx.x; tile_id < sched_total; tile_id += gridDim.x) {
+    for (int tile_id = first_slot; tile_id < sched_total; tile_id += gridDim.x) {
     TileCoord tc = schedule_tile(tile_id, tiles_m, tiles_n);
     if (!tc.valid) continue;
     const int m0 = tc.tm * BM, n0 = tc.tn * BN;
@@ -320,7 +321,7 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     point_at_slab(0);
     static_for<0, NA>([&](auto ic) { load_piece_a(ic); });
     static_for<0, NB>([&](auto ic) { load_piece_b(ic); });
-    if (tile_id != (int)blockIdx.x) __syncthreads();       // the previous tile's epilogue has read its staged rows out of LDS
+    if (tile_id != first_slot) __syncthreads();            // the previous tile's epilogue has read its staged rows out of LDS
     static_for<0, NA>([&](auto ic) { store_piece_a(smem, ic); });
     static_for<0, NB>([&](auto ic) { store_piece_b(smem, ic); });
     a_slab += a_step;

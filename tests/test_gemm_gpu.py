@@ -163,6 +163,24 @@ def test_batched_strided_views(dt):
     _check(dv, p2.transpose(0, 2, 1), do, dt, 9)
 
 
+@pytest.mark.parametrize("dt", HALF, ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("batch,m,k,n", [(3, 256, 128, 384), (13, 200, 96, 136), (37, 128, 192, 128), (192, 512, 128, 128)])
+def test_batched_tiled_16bit_every_matrix_and_tile_once(dt, batch, m, k, n):
+    """Batched products on the 16-bit tiled kernel, whose workgroups are re-dealt so that an XCD takes a contiguous
+    share of the (matrix, tile) pairs: batch sizes that are no multiple of 8, ragged tiles, integer data so that a
+    tile computed twice, skipped or taken from another matrix shows as a wrong value (every matrix has its own sum)."""
+    rng = np.random.default_rng(36)
+    assert capi.gemm_kernel_name(batch, m, k, n, (k, 1), (n, 1), (n, 1), dt).startswith("mfma16_")
+    a64 = rng.integers(-2, 3, (batch, m, k)).astype(np.float64)
+    b64 = rng.integers(-2, 3, (batch, k, n)).astype(np.float64)
+    b64[:, 0, :] = 1.0
+    a64[:, :, 0] = (np.arange(batch) % 5 - 2)[:, None]                   # a per-matrix constant added to every output
+    a = oracle.to_storage(a64, dt); b = oracle.to_storage(b64, dt)
+    got = device_gemm(a, b, dt)
+    want = oracle.to_storage(np.einsum("zik,zkj->zij", a64, b64), dt)
+    assert np.array_equal(got, want)
+
+
 def test_sliced_operand_with_offset_and_padding():
     rng = np.random.default_rng(35)
     big_a = rand_storage(rng, (96, 200), F32); big_b = rand_storage(rng, (200, 160), F32)
