@@ -30,8 +30,9 @@ namespace rp {
 // refilled row by row.
 //
 // LDS layouts (16-bit elements):
-//   KC operand: [rows][64 + 8]   row pitch 144 B -> the 16 rows a quarter-wave
-//               reads with ds_read_b128 land in 16 different 16-byte bank groups
+//   KC operand: [rows][64 + 8]   row pitch 144 B: a ds_read_b128 whose lanes hold row lane % 32, k octet lane / 32
+//               (32 x 32 tiles) runs at the full rate of one instruction per 16 cycles and wave.  With 16 x 16 tiles
+//               (row lane % 16, octet lane / 16) that pitch takes twice as long (measured: 32 cycles); 160 B does not.
 //   MC operand: [64][cols + 32]  row pitch 2*cols + 64 B -> the 4 k-rows a
 //               16-lane group reads with ds_read_b64_tr_b16 start 16 banks apart
 // The epilogue narrows the accumulators, stages them through the (now idle) LDS
@@ -67,16 +68,16 @@ template <> struct mfma16_ops<f16_t> {
 // measured 1.84 PFLOP/s at 2.16 GHz against 1.65 PFLOP/s at 1.83 GHz.
 __host__ __device__ constexpr int m16_mfma_tile(int bm, int bn) { return (bm == 256 && bn == 256) ? 16 : 32; }
 
-constexpr int M16_KC_PITCH = M16_BK + 8;                       // elements
+__host__ __device__ constexpr int m16_kc_pitch(int mt) { return mt == 16 ? M16_BK + 16 : M16_BK + 8; }    // elements, by MFMA tile edge
 __host__ __device__ constexpr int m16_mc_pitch(int cols) { return cols + 32; }
-__host__ __device__ constexpr int m16_tile_elems(int rows, bool mc) {
-    return mc ? M16_BK * m16_mc_pitch(rows) : rows * M16_KC_PITCH;
+__host__ __device__ constexpr int m16_tile_elems(int rows, bool mc, int mt) {
+    return mc ? M16_BK * m16_mc_pitch(rows) : rows * m16_kc_pitch(mt);
 }
 __host__ __device__ constexpr int m16_epi_cols(int wn) { return wn >= 64 ? 64 : wn; }      // columns staged per epilogue pass
 // `stages` is 2, or 1 when k fits a single slab (the loop then never touches the second stage), which lets twice
 // as many blocks of a short-k batched GEMM share a CU and overlap their load, multiply and store phases.
-__host__ __device__ constexpr size_t m16_smem_bytes(int bm, int bn, int wgm, bool a_mc, bool b_mc, int stages = 2) {
-    size_t loop = stages * (size_t)(m16_tile_elems(bm, a_mc) + m16_tile_elems(bn, b_mc)) * 2;
+__host__ __device__ constexpr size_t m16_smem_bytes(int bm, int bn, int wgm, bool a_mc, bool b_mc, int stages, int mt) {
+    size_t loop = stages * (size_t)(m16_tile_elems(bm, a_mc, mt) + m16_tile_elems(bn, b_mc, mt)) * 2;
     size_t epi = 4 * (size_t)(bm / wgm) * (m16_epi_cols(bn / (4 / wgm)) + 4) * 4;      // split-k: fp32, 64 columns per pass
     size_t epi16 = 4 * (size_t)(bm / wgm) * (bn / (4 / wgm) + 8) * 2;                  // otherwise: the whole patch as 16-bit values
     if (epi16 > epi) epi = epi16;
@@ -103,18 +104,19 @@ constexpr uint32_t M16_OOB = 0x80000000u;        // an offset no descriptor cove
 
 // Per-thread constants of one operand's slab traffic: NL 16-byte pieces per slab; piece i sits a fixed
 // number of rows (KC) or k-rows (MC) after piece 0, so LDS offsets are piece 0's plus a compile-time step.
-template <int ROWS, bool MC>
+template <int ROWS, bool MC, int MT>
 struct SlabMap {
+    static constexpr int KCP = m16_kc_pitch(MT);
     static constexpr int NL = ROWS * 8 / 256;
     static constexpr int PIECE_ROWS = MC ? 256 / (ROWS / 8) : 32;        // k-rows (MC) or free rows (KC) between consecutive pieces
-    static constexpr int LDS_STEP = MC ? PIECE_ROWS * m16_mc_pitch(ROWS) : PIECE_ROWS * M16_KC_PITCH;   // elements
+    static constexpr int LDS_STEP = MC ? PIECE_ROWS * m16_mc_pitch(ROWS) : PIECE_ROWS * KCP;   // elements
     // piece 0 of thread t: free index r (first of 8 for MC) and slab-local k (first of 8 for KC)
     static __device__ __forceinline__ void coords0(int t, int& r, int& kk) {
         if (MC) { kk = t / (ROWS / 8); r = (t % (ROWS / 8)) * 8; }
         else    { r = t / 8; kk = (t % 8) * 8; }
     }
     static __device__ __forceinline__ int lds_off(int r, int kk) {          // element offset inside the operand's LDS tile
-        return MC ? kk * m16_mc_pitch(ROWS) + r : r * M16_KC_PITCH + kk;
+        return MC ? kk * m16_mc_pitch(ROWS) + r : r * KCP + kk;
     }
 };
 
@@ -125,8 +127,9 @@ struct SlabMap {
 template <int ROWS, bool MC, int MT>
 struct FragMap {
     static constexpr int KSTEP = MT == 32 ? 16 : 32;
+    static constexpr int KCP = m16_kc_pitch(MT);
     static __device__ __forceinline__ int base(int w0, int lane) {
-        if (!MC) return (w0 + (lane % MT)) * M16_KC_PITCH + (lane / MT) * 8;
+        if (!MC) return (w0 + (lane % MT)) * KCP + (lane / MT) * 8;
         // ds_read_b64_tr_b16: inside each 16-lane group, source lane s points at 4 consecutive free
         // indices of k-row s/4; destination lane j receives free index j of k-rows 0..3.
         int grp = lane >> 4, s = lane & 15;
@@ -136,7 +139,7 @@ struct FragMap {
     static constexpr int READS = MC ? 2 : 1;                 // DS instructions per fragment
     static constexpr int step(int i, int ks, int h) {
         return MC ? ks * KSTEP * m16_mc_pitch(ROWS) + i * MT + h * 4 * m16_mc_pitch(ROWS)
-                  : i * MT * M16_KC_PITCH + ks * KSTEP;
+                  : i * MT * KCP + ks * KSTEP;
     }
     // DS read H of the fragment into v (KC: the whole fragment; MC: k values 4H .. 4H+3)
     template <int H>
@@ -159,10 +162,10 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     constexpr int NV = MT == 32 ? 16 : 4;             // accumulator registers per MFMA tile
     using acc_t = std::conditional_t<MT == 32, f32x16_t, f32x4_t>;
     constexpr int TMI = WM / MT, TNI = WN / MT;       // MFMA tiles per wave
-    constexpr int A_ELEMS = m16_tile_elems(BM, A_MC), B_ELEMS = m16_tile_elems(BN, B_MC);
+    constexpr int A_ELEMS = m16_tile_elems(BM, A_MC, MT), B_ELEMS = m16_tile_elems(BN, B_MC, MT);
     constexpr int STAGE = A_ELEMS + B_ELEMS;          // stage s: A at smem + s*STAGE, B right after it
-    using MapA = SlabMap<BM, A_MC>;
-    using MapB = SlabMap<BN, B_MC>;
+    using MapA = SlabMap<BM, A_MC, MT>;
+    using MapB = SlabMap<BN, B_MC, MT>;
     using FragA = FragMap<BM, A_MC, MT>;
     using FragB = FragMap<BN, B_MC, MT>;
     constexpr int NA = MapA::NL, NB = MapB::NL;
@@ -588,7 +591,7 @@ static int m16_launch(const GemmArgs& g, float* partials, int nsplit, int k_per_
         if (cus >= 8 && blocks > cus) blocks = cus;
     }
     dim3 grid(blocks, g.batch, SPLITK ? nsplit : 1);
-    size_t smem = m16_smem_bytes(BM, BN, WGM, A_MC, B_MC, (!SPLITK && g.k <= M16_BK) ? 1 : 2);
+    size_t smem = m16_smem_bytes(BM, BN, WGM, A_MC, B_MC, (!SPLITK && g.k <= M16_BK) ? 1 : 2, SPLITK ? 32 : m16_mfma_tile(BM, BN));
     auto kern = gemm_mfma16_kernel<T, BM, BN, WGM, A_MC, B_MC, EDGE, SPLITK>;
     if (smem > 64 * 1024 && !check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem), "hipFuncSetAttribute")) return -1;
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, current_stream(), g, tiles_m, tiles_n, partials, k_per_split, sched_total);
