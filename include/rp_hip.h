@@ -51,6 +51,11 @@ int rp_hip_get_device(int* device_id);
 int rp_hip_malloc(void** ptr, size_t bytes);
 int rp_hip_free(void* ptr);
 int rp_hip_empty_cache(void);
+/* Allocator counters of the process (no counterpart in the reference, which calls cudaMalloc / cudaFree directly):
+ * calls to rp_hip_malloc so far, how many of them reached hipMalloc, blocks handed out and not yet freed, blocks
+ * cached for reuse.  Any pointer may be NULL.  A caller that must not allocate (a serving loop, a graph recording)
+ * checks that the first two stand still across the calls it makes. */
+int rp_hip_memory_stats(long long* malloc_requests, long long* device_mallocs, long long* live_blocks, long long* cached_blocks);
 int rp_hip_memset(void* ptr, int value, size_t bytes);
 int rp_hip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes);
 int rp_hip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes);

@@ -28,6 +28,7 @@ SIGNATURES = {
     "rp_hip_malloc": (_i, [ctypes.POINTER(_vp), _sz]),
     "rp_hip_free": (_i, [_vp]),
     "rp_hip_empty_cache": (_i, []),
+    "rp_hip_memory_stats": (_i, [ctypes.POINTER(_ll)] * 4),
     "rp_hip_memset": (_i, [_vp, _i, _sz]),
     "rp_hip_memcpy_h2d": (_i, [_vp, _vp, _sz]),
     "rp_hip_memcpy_d2h": (_i, [_vp, _vp, _sz]),

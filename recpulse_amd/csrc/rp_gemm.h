@@ -140,7 +140,9 @@ int* splitk_arrival_counters(long long tiles, size_t partial_bytes, bool* failed
 // nothing, a piece of that entry point's fixed device array (then -1 with an error when it is too small).
 int gemm_workspace(void** ws, size_t bytes);
 void gemm_workspace_release(void* ws);
-// Inside the entry point that allocates nothing: its arrival counters (already zero); nullptr elsewhere.
+// Inside the entry point that allocates nothing: its arrival counters, cleared by a kernel on the current stream the
+// first time a call asks for them (nullptr with an error when that launch fails).
+bool noalloc_active();
 int* noalloc_arrival_counters();
 
 // per-family launchers (dtype is one of the RP_DTYPE_* codes the family supports)

@@ -287,6 +287,7 @@ static std::mutex g_scratch_mu;
 static unsigned char* g_scratch_ptr[NOALLOC_MAX_DEVICES] = {};      // per device: where that device's copy of `scratch` lives
 static thread_local unsigned char* g_noalloc_base = nullptr;        // non-null while the calling thread is inside the entry point
 static thread_local bool g_noalloc_busy = false;                    // its workspace is handed out (one launcher at a time)
+static thread_local bool g_noalloc_cleared = false;                 // this call has cleared the arrival counters
 
 // Address of the current device's copy of the array, resolved once per device.
 static unsigned char* noalloc_scratch_of_current_device() {
@@ -321,11 +322,25 @@ void gemm_workspace_release(void* ws) {
     rp_hip_free(ws);
 }
 
-int* noalloc_arrival_counters() { return (int*)g_noalloc_base; }
-
 __global__ void __launch_bounds__(256) clear_counters_kernel(int* counters, int n) {
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i < n) counters[i] = 0;
+}
+
+bool noalloc_active() { return g_noalloc_base != nullptr; }
+
+// The array keeps what the last call left.  The partial sums are fully overwritten before they are read; the arrival
+// counters must read zero, and a launch that was cut short could have left some standing: the first launcher of a call
+// that wants them has them cleared by a kernel (stream-ordered before the GEMM; not a memset node, so the call can be
+// recorded into a graph).  Calls whose kernels use no counters launch nothing extra.
+int* noalloc_arrival_counters() {
+    if (!g_noalloc_base) return nullptr;
+    if (!g_noalloc_cleared) {
+        hipLaunchKernelGGL(clear_counters_kernel, dim3((SPLITK_MAX_TILES + 255) / 256), dim3(256), 0, current_stream(), (int*)g_noalloc_base, SPLITK_MAX_TILES);
+        if (!check_launch("clear_counters_kernel")) return nullptr;
+        g_noalloc_cleared = true;
+    }
+    return (int*)g_noalloc_base;
 }
 
 }  // namespace rp
@@ -370,13 +385,9 @@ int rp_hip_gemm_strided_batched_noalloc(void* C, const void* A, const void* B, c
     if (g_noalloc_base) { set_error("rp_hip_gemm_strided_batched_noalloc: re-entered"); return -1; }
     unsigned char* base = noalloc_scratch_of_current_device();
     if (!base) return -1;
-    // The array keeps what the last call left.  The partial sums are fully overwritten before they are read; the
-    // arrival counters must read zero, and a launch that was cut short could have left some standing: clear them
-    // with a kernel (stream-ordered before the GEMM; not a memset node, so the call can be recorded into a graph).
-    hipLaunchKernelGGL(clear_counters_kernel, dim3((SPLITK_MAX_TILES + 255) / 256), dim3(256), 0, current_stream(), (int*)base, SPLITK_MAX_TILES);
-    if (!check_launch("clear_counters_kernel")) return -1;
     g_noalloc_base = base;
     g_noalloc_busy = false;
+    g_noalloc_cleared = false;
     const int rc = rp_hip_gemm_strided_batched(C, A, B, bias, batch, m, k, n, a_bs, a_rs, a_cs, b_bs, b_rs, b_cs, c_bs, c_rs, c_cs, accumulate, dtype);
     g_noalloc_base = nullptr;
     g_noalloc_busy = false;

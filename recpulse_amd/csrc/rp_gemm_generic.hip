@@ -273,9 +273,13 @@ int* splitk_arrival_counters(long long tiles, size_t partial_bytes, bool* failed
     static int* blocks[MAX_DEVICES] = {};
     static int two_launch = -1;
     *failed = false;
-    if (int* fixed = noalloc_arrival_counters()) return (tiles > SPLITK_MAX_TILES || partial_bytes >= (1ull << 31)) ? nullptr : fixed;
     if (two_launch < 0) { const char* e = getenv("RP_HIP_SPLITK_TWO_LAUNCH"); two_launch = (e && e[0] == '1') ? 1 : 0; }
     if (two_launch == 1 || tiles > SPLITK_MAX_TILES || partial_bytes >= (1ull << 31)) return nullptr;
+    if (noalloc_active()) {                              // inside the entry point that allocates nothing: its fixed counters
+        int* fixed = noalloc_arrival_counters();
+        if (!fixed) *failed = true;
+        return fixed;
+    }
     int dev = 0;
     if (rp_hip_get_device(&dev) != 0) { *failed = true; return nullptr; }
     if (dev < 0 || dev >= MAX_DEVICES) return nullptr;

@@ -23,29 +23,46 @@ namespace rp {
 // Loads for four rounds are always in flight per wave and are issued
 // unconditionally (out-of-range rounds get an empty buffer descriptor and read
 // zeros), so the waits the compiler inserts count loads exactly.
-// The block's 4 waves take interleaved rounds; they add their tiles through
-// LDS in wave order, 8 rows at a time, and the block writes one fp32 partial
-// (or, without a k split, the finished output).  With `arrivals` the block
-// then counts itself in, and the last block of its column group to do so adds
-// the group's partials and writes the output (otherwise a second kernel does).
+//
+// Rounds are dealt cyclically: round q of k belongs to split q % nsplit, and
+// inside a block to wave (q / nsplit) % 4.  At any moment the grid as a whole
+// therefore reads one contiguous window of B (nsplit * 4 rounds of whole rows),
+// which the memory system serves 5 - 8 % faster than the same blocks each
+// walking a range of k of its own (the ranges lie a power of two apart).
+//
+// The block's 4 waves add their tiles through LDS in wave order, 8 rows at a
+// time, and the block writes one fp32 partial (or, without a k split, the
+// finished output).  With `arrivals` the block then counts itself in, and the
+// last block of its column group to do so adds the group's partials in split
+// order and writes the output (otherwise a second kernel does).
+//
+// Placement.  The grid is one-dimensional and block b stands for (XCD x = b % 8,
+// slot b / 8): workgroups are dealt to the XCDs round robin, so all splits of
+// column group 8i + x are given slots of XCD x.  When the host has verified that
+// rule on the device (`local`), the partials and the arrival count never leave
+// that XCD's L2: plain stores (complete when the L2 has them), an atomic that the
+// L2 executes, and loads behind an invalidate of the finishing CU's vector cache.
+// Otherwise they are exchanged at device scope (written through to memory and
+// read back from there), which costs about 1.5 us more per launch.
 // ============================================================================
 constexpr int SS_WAVES = 4, SS_COLS = 256, SS_ROUND = 16, SS_RED_PITCH = SS_COLS + 8;
 constexpr int SS_MAX_M = 16;
 constexpr int SS_DEPTH = 4;            // rounds a wave keeps in flight (register slots)
 
 template <typename T, int MT>          // MT: rows the epilogue keeps (8 or 16; m <= MT)
-__global__ void __launch_bounds__(256) gemm_stream16_kernel(GemmArgs g, float* partials, int k_per_split, int* arrivals) {
-    __shared__ __attribute__((aligned(16))) float red[SS_WAVES * 8 * SS_RED_PITCH];
+__global__ void __launch_bounds__(256) gemm_stream16_kernel(GemmArgs g, float* partials, int groups, int nsplit, int* arrivals, int local) {
+    extern __shared__ __attribute__((aligned(16))) float red[];          // [SS_WAVES][MT][SS_RED_PITCH]
     __shared__ bool arrived_last;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);       // scalar, so that buffer descriptors built from it are too
     const int h = lane >> 5, j = lane & 31;
-    const int n0 = blockIdx.x * SS_COLS;
-    const int split = blockIdx.y, nsplit = gridDim.y;
-    const int kb = split * k_per_split;                                   // a multiple of SS_WAVES * SS_ROUND
-    const int ke = kb + k_per_split < g.k ? kb + k_per_split : g.k;
-    const int rounds = (ke - kb + SS_ROUND - 1) / SS_ROUND;               // in this block
-    const int my_rounds = rounds > wave ? (rounds - wave + SS_WAVES - 1) / SS_WAVES : 0;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int group = (slot / nsplit) * 8 + xcd, split = slot % nsplit;
+    if (group >= groups) return;                                           // (whole blocks, before any barrier)
+    const int n0 = group * SS_COLS;
+    const int total_rounds = (g.k + SS_ROUND - 1) / SS_ROUND;
+    const int mine = total_rounds > split ? (total_rounds - split + nsplit - 1) / nsplit : 0;      // rounds of this block
+    const int my_rounds = mine > wave ? (mine - wave + SS_WAVES - 1) / SS_WAVES : 0;               // and of this wave
 
     const uint16_t* Bm = (const uint16_t*)g.B;
     const uint16_t* Am = (const uint16_t*)g.A;
@@ -63,7 +80,7 @@ __global__ void __launch_bounds__(256) gemm_stream16_kernel(GemmArgs g, float* p
     // request round r of this wave into register slot SLOT (r beyond the wave's share reads zeros)
     auto request = [&](auto slotc, int r) {
         constexpr int SLOT = decltype(slotc)::value;
-        const int kr = kb + (wave + SS_WAVES * r) * SS_ROUND;
+        const int kr = ((r * SS_WAVES + wave) * nsplit + split) * SS_ROUND;
         const bool live = r < my_rounds;
         const char* bb = (const char*)(Bm + (long long)kr * b_rs + n0);
         const char* ab = (const char*)(Am + kr);
@@ -111,109 +128,134 @@ __global__ void __launch_bounds__(256) gemm_stream16_kernel(GemmArgs g, float* p
     static_for<0, SS_DEPTH>([&](auto sc) { request(sc, decltype(sc)::value); __builtin_amdgcn_sched_barrier(0); });
     for (int r = 0; r < my_rounds; r += SS_DEPTH)
         static_for<0, SS_DEPTH>([&](auto sc) { consume(sc, r + decltype(sc)::value); });
-
-    // ---- the block's waves add their tiles through LDS, 8 rows per pass ----
+    // ---- the block's waves add their tiles through LDS ----
     // accumulator register v of a 32x32 tile holds row 8*(v/4) + 4*h + v%4 at column j (of residue c)
     T* C = (T*)g.C;
     const T* bias = (const T*)g.bias;
     const bool has_bias = bias != nullptr, accum = g.accumulate != 0;
+    const bool c_vec = g.c_cs == 1 && g.c_rs % 4 == 0 && ((uintptr_t)C & 7) == 0;       // a quad of outputs is one aligned 8-byte store
     const __amdgpu_buffer_rsrc_t part_rsrc = m16_rsrc(partials, partials ? (long long)nsplit * g.m * g.n * 4 : 0);
+    // four outputs of one row: the epilogue of each, stored as one vector where the layout allows
+    auto store_quad = [&](int row, int col, f32x4_t sum) {
+        T y[4];
 #pragma unroll
-    for (int p = 0; p < MT / 8; p++) {
-        if (8 * p >= g.m) break;
-        __syncthreads();
+        for (int e = 0; e < 4; e++) {
+            T* pc = C + (long long)row * g.c_rs + (long long)(col + e) * g.c_cs;
+            T old = accum ? *pc : T{};
+            y[e] = finish<T>(sum[e], has_bias, has_bias ? bias[col + e] : T{}, accum, old);
+        }
+        if (c_vec) {
+            u32x2_t w = {(uint32_t)y[0].bits | ((uint32_t)y[1].bits << 16), (uint32_t)y[2].bits | ((uint32_t)y[3].bits << 16)};
+            *(u32x2_t*)(C + (long long)row * g.c_rs + col) = w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) C[(long long)row * g.c_rs + (long long)(col + e) * g.c_cs] = y[e];
+        }
+    };
+    // A lane holds columns 8j .. 8j+7 of its rows.  In LDS a row is two planes of 128 floats, columns 8j .. 8j+3 at
+    // float 4j of the first and columns 8j+4 .. 8j+7 at float 4j of the second, so that both the waves' stores and
+    // the block's reads below are 16 bytes per lane at consecutive addresses.
+#pragma unroll
+    for (int p = 0; p < MT / 8; p++)
 #pragma unroll
         for (int vv = 0; vv < 4; vv++) {
-            float* dst = red + (wave * 8 + 4 * h + vv) * SS_RED_PITCH + 8 * j;
+            const int r = 8 * p + 4 * h + vv;
+            if (r >= g.m) continue;
+            float* dst = red + (wave * MT + r) * SS_RED_PITCH + 4 * j;
             *(f32x4_t*)dst = f32x4_t{acc[0][4 * p + vv], acc[1][4 * p + vv], acc[2][4 * p + vv], acc[3][4 * p + vv]};
-            *(f32x4_t*)(dst + 4) = f32x4_t{acc[4][4 * p + vv], acc[5][4 * p + vv], acc[6][4 * p + vv], acc[7][4 * p + vv]};
+            *(f32x4_t*)(dst + 128) = f32x4_t{acc[4][4 * p + vv], acc[5][4 * p + vv], acc[6][4 * p + vv], acc[7][4 * p + vv]};
         }
-        __syncthreads();
+    __syncthreads();
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const int idx = threadIdx.x + 256 * i, r = idx / 64, c4 = (idx % 64) * 4;
-            const int gm = 8 * p + r, gn = n0 + c4;
-            if (gm >= g.m || gn >= g.n) continue;                        // n is a multiple of 4, so a quad is wholly in or out
-            f32x4_t sum = *(const f32x4_t*)(red + r * SS_RED_PITCH + c4);
+    for (int i = 0; i < MT / 4; i++) {
+        const int idx = threadIdx.x + 256 * i, r = idx / 64, plane = (idx % 64) / 32, jj = idx % 32;
+        const int at_lds = r * SS_RED_PITCH + 128 * plane + 4 * jj;
+        const int gn = n0 + 8 * jj + 4 * plane;
+        if (r >= g.m || gn >= g.n) continue;                             // n is a multiple of 4, so a quad is wholly in or out
+        f32x4_t sum = *(const f32x4_t*)(red + at_lds);
 #pragma unroll
-            for (int w = 1; w < SS_WAVES; w++) sum += *(const f32x4_t*)(red + (w * 8 + r) * SS_RED_PITCH + c4);
-            if (nsplit > 1) {
-                const long long at = ((long long)split * g.m + gm) * g.n + gn;
-                if (arrivals) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sum), part_rsrc, (int)(at * 4), 0, SPLITK_DEVICE_SCOPE);
-                else *(f32x4_t*)(partials + at) = sum;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    T* pc = C + (long long)gm * g.c_rs + (long long)(gn + e) * g.c_cs;
-                    T old = accum ? *pc : T{};
-                    *pc = finish<T>(sum[e], has_bias, has_bias ? bias[gn + e] : T{}, accum, old);
-                }
-            }
-        }
+        for (int w = 1; w < SS_WAVES; w++) sum += *(const f32x4_t*)(red + w * MT * SS_RED_PITCH + at_lds);
+        if (nsplit > 1) {
+            const long long at = ((long long)split * g.m + r) * g.n + gn;
+            if (!arrivals) *(f32x4_t*)(partials + at) = sum;
+            else if (local) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sum), part_rsrc, (int)(at * 4), 0, 0);
+            else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sum), part_rsrc, (int)(at * 4), 0, SPLITK_DEVICE_SCOPE);
+        } else store_quad(r, gn, sum);
     }
     if (nsplit == 1 || !arrivals) return;
 
     // ---- single-launch finish: the last block of this column group to arrive adds all splits ----
-    // Partials are written and read at device scope (they bypass the per-XCD L2s, which are not coherent
-    // with each other), every thread waits for its own stores to be acknowledged before the block's arrival
-    // is counted, and the count is a device-scope atomic.  No cache-wide write-back or invalidate is needed.
+    // Every thread waits until its own partial stores are acknowledged (by the XCD's L2, or by memory for
+    // device-scope stores) before the block's arrival is counted.  No cache-wide write-back is needed.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
-        int before = __hip_atomic_fetch_add(arrivals + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        int before;
+        if (local) before = __hip_atomic_fetch_add(arrivals + group, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);    // executed by this XCD's L2
+        else before = __hip_atomic_fetch_add(arrivals + group, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         arrived_last = before == nsplit - 1;
     }
     __syncthreads();
     if (!arrived_last) return;
+    // (Loads of the partials miss this CU's vector cache, which fills on the CU's own loads only and starts every
+    // launch empty: the one block of a launch that reads a group's partials reads them here for the first time.)
     const long long split_stride = (long long)g.m * g.n;
     constexpr int QPR = SS_COLS / 4;                     // quads per row of the block's columns
-    // two quads per thread and pass (one pass covers 8 rows), the loads of eight splits of both in flight together
-    for (int r0 = 0; r0 < g.m; r0 += 8) {
-        long long at[2];
-        bool live[2];
-        int row[2], col[2];
+    constexpr int QN = MT >= 16 ? 4 : 2;                 // quads per thread and pass: a pass covers 4 * QN rows
+    // the loads of eight splits of all of a thread's quads are in flight together
+    for (int r0 = 0; r0 < g.m; r0 += 4 * QN) {
+        long long at[QN];
+        bool live[QN];
+        int row[QN], col[QN];
 #pragma unroll
-        for (int q = 0; q < 2; q++) {
+        for (int q = 0; q < QN; q++) {
             const int idx = threadIdx.x + 256 * q;
             row[q] = r0 + idx / QPR; col[q] = n0 + (idx % QPR) * 4;
             live[q] = row[q] < g.m && col[q] < g.n;
             at[q] = live[q] ? ((long long)row[q] * g.n + col[q]) * 4 : (long long)M16_OOB;      // bytes; dead quads read zeros
         }
-        f32x4_t sum[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+        f32x4_t sum[QN];
+#pragma unroll
+        for (int q = 0; q < QN; q++) sum[q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         for (int sp = 0; sp < nsplit; sp += 8) {
-            u32x4_t v[2][8];
+            u32x4_t v[QN][8];
 #pragma unroll
             for (int u = 0; u < 8; u++)
 #pragma unroll
-                for (int q = 0; q < 2; q++) {
+                for (int q = 0; q < QN; q++) {
                     const bool in = live[q] && sp + u < nsplit;
-                    v[q][u] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, in ? (int)(at[q] + (sp + u) * split_stride * 4) : (int)M16_OOB, 0, SPLITK_DEVICE_SCOPE);
+                    const int off = in ? (int)(at[q] + (sp + u) * split_stride * 4) : (int)M16_OOB;
+                    if (local) v[q][u] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, off, 0, 0);
+                    else v[q][u] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, off, 0, SPLITK_DEVICE_SCOPE);
                 }
 #pragma unroll
             for (int u = 0; u < 8; u++)
 #pragma unroll
-                for (int q = 0; q < 2; q++) sum[q] += __builtin_bit_cast(f32x4_t, v[q][u]);       // split order; absent splits add +0
+                for (int q = 0; q < QN; q++) sum[q] += __builtin_bit_cast(f32x4_t, v[q][u]);       // split order; absent splits add +0
         }
 #pragma unroll
-        for (int q = 0; q < 2; q++) {
-            if (!live[q]) continue;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                T* pc = C + (long long)row[q] * g.c_rs + (long long)(col[q] + e) * g.c_cs;
-                T old = accum ? *pc : T{};
-                *pc = finish<T>(sum[q][e], has_bias, has_bias ? bias[col[q] + e] : T{}, accum, old);
-            }
-        }
+        for (int q = 0; q < QN; q++)
+            if (live[q]) store_quad(row[q], col[q], sum[q]);
     }
-    if (threadIdx.x == 0) __hip_atomic_store(arrivals + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
+    if (threadIdx.x == 0) {                                          // ready for the next launch
+        if (local) __hip_atomic_store(arrivals + group, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        else __hip_atomic_store(arrivals + group, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+template <typename T, int MT>
+static int launch_stream16_mt(const GemmArgs& g, float* partials, int groups, int nsplit, int* arrivals, int local) {
+    constexpr size_t smem = (size_t)SS_WAVES * MT * SS_RED_PITCH * sizeof(float);
+    auto kern = gemm_stream16_kernel<T, MT>;
+    if (smem > 64 * 1024 && !check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem), "hipFuncSetAttribute")) return -1;
+    hipLaunchKernelGGL(kern, dim3(8 * ((groups + 7) / 8) * nsplit), dim3(256), smem, current_stream(), g, partials, groups, nsplit, arrivals, local);
+    return check_launch("gemm_stream16_kernel") ? 0 : -1;
 }
 
 template <typename T>
-static int launch_stream16_t(const GemmArgs& g, float* partials, int nsplit, int k_per_split, int* arrivals) {
-    dim3 grid((g.n + SS_COLS - 1) / SS_COLS, nsplit);
-    if (g.m <= 8) hipLaunchKernelGGL((gemm_stream16_kernel<T, 8>), grid, dim3(256), 0, current_stream(), g, partials, k_per_split, arrivals);
-    else          hipLaunchKernelGGL((gemm_stream16_kernel<T, 16>), grid, dim3(256), 0, current_stream(), g, partials, k_per_split, arrivals);
-    return check_launch("gemm_stream16_kernel") ? 0 : -1;
+static int launch_stream16_t(const GemmArgs& g, float* partials, int groups, int nsplit, int* arrivals, int local) {
+    if (g.m <= 8) return launch_stream16_mt<T, 8>(g, partials, groups, nsplit, arrivals, local);
+    return launch_stream16_mt<T, 16>(g, partials, groups, nsplit, arrivals, local);
 }
 
 static int launch_stream16(const GemmArgs& g, int dtype) {
@@ -223,8 +265,6 @@ static int launch_stream16(const GemmArgs& g, int dtype) {
     int nsplit = (256 + groups - 1) / groups;
     int max_split = g.k / (4 * QUANTUM) > 0 ? g.k / (4 * QUANTUM) : 1;
     if (nsplit > max_split) nsplit = max_split;
-    int k_per_split = ((g.k + nsplit - 1) / nsplit + QUANTUM - 1) / QUANTUM * QUANTUM;
-    nsplit = (g.k + k_per_split - 1) / k_per_split;
     const size_t part_bytes = (size_t)nsplit * g.m * g.n * sizeof(float);
     void* ws = nullptr;
     if (nsplit > 1 && gemm_workspace(&ws, part_bytes) != 0) return -1;
@@ -234,9 +274,13 @@ static int launch_stream16(const GemmArgs& g, int dtype) {
         arrivals = splitk_arrival_counters(groups, part_bytes, &failed);
         if (failed) { gemm_workspace_release(ws); return -1; }
     }
+    // The arrival counters of a device serve launches of both kinds of exchange.  That is safe because launches
+    // on one stream follow each other and every launch leaves its counters at zero: whatever copy of a counter an
+    // L2 still holds from an earlier launch reads zero, like memory.
+    const int local = arrivals && workgroups_share_xcd_by_residue() ? 1 : 0;
     int rc;
-    if (dtype == RP_DTYPE_BFLOAT16) rc = launch_stream16_t<bf16_t>(g, (float*)ws, nsplit, k_per_split, arrivals);
-    else rc = launch_stream16_t<f16_t>(g, (float*)ws, nsplit, k_per_split, arrivals);
+    if (dtype == RP_DTYPE_BFLOAT16) rc = launch_stream16_t<bf16_t>(g, (float*)ws, groups, nsplit, arrivals, local);
+    else rc = launch_stream16_t<f16_t>(g, (float*)ws, groups, nsplit, arrivals, local);
     if (rc == 0 && nsplit > 1 && !arrivals) rc = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, dtype);
     if (ws) gemm_workspace_release(ws);          // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
     return rc;
@@ -260,7 +304,6 @@ static int launch_skinny16_t(const GemmArgs& g, const Plan& p, float* partials, 
 
 int launch_mfma16_skinny(const GemmArgs& g, const Plan& p, int dtype) {
     if (dtype != RP_DTYPE_BFLOAT16 && dtype != RP_DTYPE_FLOAT16) { set_error("mfma16 skinny GEMM: unsupported dtype %d", dtype); return -1; }
-    // beyond 16 rows the partial tiles the streaming kernel exchanges outweigh what it saves
     if (!p.a_mc && p.b_mc && g.m <= SS_MAX_M && !tiled_skinny_forced()) return launch_stream16(g, dtype);
     constexpr int BN = 128;
     const int tiles = ((g.n + BN - 1) / BN) * ((g.m + 31) / 32);

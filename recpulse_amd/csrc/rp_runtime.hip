@@ -50,6 +50,48 @@ int device_cu_count() {
     return n;
 }
 
+// ---- workgroup placement -----------------------------------------------------
+// The dispatcher deals the workgroups of a grid to the XCDs round robin, so workgroups b and b + 8 share an L2.
+// Kernels that exchange data between workgroups through that L2 rely on it, so it is observed rather than assumed:
+// every workgroup of a 1 024-block grid records the XCC it runs on, three launches in a row, and the rule must
+// hold for all of them.  (A device with a single XCD passes trivially.)  The record lives in a device array of the
+// library, so the check allocates nothing.
+constexpr int PLACEMENT_BLOCKS = 1024;
+static __device__ int g_xcc_of_block[PLACEMENT_BLOCKS];
+
+__global__ void __launch_bounds__(256) record_xcc_kernel() {
+    if (threadIdx.x == 0) {
+        unsigned xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        g_xcc_of_block[blockIdx.x] = (int)(xcc & 15u);
+    }
+}
+
+bool workgroups_share_xcd_by_residue() {
+    constexpr int MAX_DEVICES = 64;
+    static std::atomic<int> state[MAX_DEVICES] = {};          // 0 unknown, 1 holds, 2 does not
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) { (void)hipGetLastError(); return false; }
+    int st = state[dev].load(std::memory_order_acquire);
+    if (st != 0) return st == 1;
+    if (stream_is_capturing()) return false;
+    static std::mutex mu;
+    std::lock_guard<std::mutex> lock(mu);
+    st = state[dev].load(std::memory_order_acquire);
+    if (st != 0) return st == 1;
+    const char* off = getenv("RP_HIP_NO_L2_EXCHANGE");
+    bool holds = !(off && off[0] == '1');
+    static int seen[PLACEMENT_BLOCKS];
+    for (int rep = 0; rep < 3 && holds; rep++) {
+        hipLaunchKernelGGL(record_xcc_kernel, dim3(PLACEMENT_BLOCKS), dim3(256), 0, current_stream());
+        if (hipGetLastError() != hipSuccess || hipStreamSynchronize(current_stream()) != hipSuccess ||
+            hipMemcpyFromSymbol(seen, HIP_SYMBOL(g_xcc_of_block), sizeof(seen)) != hipSuccess) { (void)hipGetLastError(); return false; }   // not decided: ask again later
+        for (int b = 8; b < PLACEMENT_BLOCKS; b++) holds = holds && seen[b] == seen[b % 8];
+    }
+    state[dev].store(holds ? 1 : 2, std::memory_order_release);
+    return holds;
+}
+
 // ---- caching allocator ------------------------------------------------------
 // The reference allocates and zero-fills device memory for every op output
 // (core/tensor_device.cu:44-46) and frees it when the tensor dies; hipMalloc /
@@ -69,6 +111,9 @@ struct Pool {
 };
 
 static Pool& pool() { static Pool* p = new Pool(); return *p; }   // leaked on purpose: outlives HIP teardown
+
+// what rp_hip_memory_stats reports: requests to rp_hip_malloc, and how many of them reached hipMalloc
+static std::atomic<long long> g_malloc_requests{0}, g_device_mallocs{0};
 
 // Blocks and graph capture.  A kernel recorded into a graph keeps the addresses it was recorded with, so a block
 // that is freed while the calling thread records (a split-k workspace, an intermediate tensor) must not be handed
@@ -156,6 +201,7 @@ int rp_hip_get_device(int* device_id) {
 int rp_hip_malloc(void** ptr, size_t bytes) {
     if (!ptr) { set_error("rp_hip_malloc: null argument"); return -1; }
     *ptr = nullptr;
+    g_malloc_requests.fetch_add(1, std::memory_order_relaxed);
     int dev = 0;
     if (!check_hip(hipGetDevice(&dev), "hipGetDevice")) return -1;
     Pool& p = pool();
@@ -182,6 +228,7 @@ int rp_hip_malloc(void** ptr, size_t bytes) {
         }
     }
     void* d = nullptr;
+    g_device_mallocs.fetch_add(1, std::memory_order_relaxed);
     hipError_t e = hipMalloc(&d, sz);
     if (e != hipSuccess && p.enabled) {            // out of memory: give cached blocks back and retry once
         (void)hipGetLastError();
@@ -216,6 +263,16 @@ int rp_hip_free(void* ptr) {
         if (p.enabled) { p.free_lists[key].push_back(ptr); return 0; }
     }
     return check_hip(hipFree(ptr), "hipFree") ? 0 : -1;
+}
+
+int rp_hip_memory_stats(long long* malloc_requests, long long* device_mallocs, long long* live_blocks, long long* cached_blocks) {
+    Pool& p = pool();
+    if (malloc_requests) *malloc_requests = g_malloc_requests.load(std::memory_order_relaxed);
+    if (device_mallocs) *device_mallocs = g_device_mallocs.load(std::memory_order_relaxed);
+    std::lock_guard<std::mutex> lk(p.mu);
+    if (live_blocks) *live_blocks = (long long)p.live.size();
+    if (cached_blocks) { long long n = 0; for (auto& kv : p.free_lists) n += (long long)kv.second.size(); *cached_blocks = n; }
+    return 0;
 }
 
 int rp_hip_empty_cache(void) {

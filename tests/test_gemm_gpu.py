@@ -250,6 +250,56 @@ def test_streaming_rows_single_launch_finish(m):
     assert np.array_equal(device_gemm(a, b, BF16), oracle_gemm(a, b, BF16))
 
 
+@pytest.mark.parametrize("m", [1, 8, 16])
+def test_streaming_rows_finish_repeats_bit_for_bit_over_hundreds_of_launches(m):
+    """The finish exchanges partial sums between the workgroups of a column group while other groups still stream:
+    launched back to back a few hundred times on resident operands (no synchronisation in between), every launch
+    must leave the bits of the first one, and the fp64 product stays inside the tolerance."""
+    rng = np.random.default_rng(41)
+    k = n = 8192
+    dt = BF16
+    a = rand_storage(rng, (m, k), dt); b = rand_storage(rng, (k, n), dt)
+    assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == "mfma16_stream_32x256"
+    da, db = capi.DeviceBuffer.from_numpy(a), capi.DeviceBuffer.from_numpy(b)
+    launches = 300
+    outs = [capi.DeviceBuffer(m * n * 2) for _ in range(launches)]
+    for dc in outs:
+        capi.gemm(dc.ptr, da.ptr, db.ptr, None, 1, m, k, n, (0, k, 1), (0, n, 1), (0, n, 1), False, dt)
+    capi.synchronize()
+    first = outs[0].to_numpy(np.uint16, (m, n))
+    for i, dc in enumerate(outs[1:], 1):
+        assert np.array_equal(first, dc.to_numpy(np.uint16, (m, n))), f"launch {i} differs from launch 0"
+    want = oracle.to_f64(a, dt) @ oracle.to_f64(b, dt)
+    assert oracle.rel_err(oracle.to_f64(first, dt), want) <= tol(dt, k)
+
+
+def test_streaming_rows_both_exchanges_give_the_same_bits(tmp_path):
+    """The k-split finish goes through the XCD's own L2 when workgroup placement was verified, and through memory at
+    device scope otherwise (RP_HIP_NO_L2_EXCHANGE=1 forces that, read once per process): a child process computes
+    the same products the other way, and the bits must agree (same partial sums, same order)."""
+    import subprocess
+    import sys
+    code = (
+        "import sys, numpy as np\n"
+        "sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
+        "from devhelp import device_gemm, rand_storage, BF16, F16\n"
+        "rng = np.random.default_rng(42)\n"
+        "out = {}\n"
+        "for i, (dt, m, k, n) in enumerate([(BF16, 1, 8192, 8192), (BF16, 8, 8192, 8192), (F16, 16, 4104, 1288), (BF16, 11, 2048, 2048)]):\n"
+        "    a = rand_storage(rng, (m, k), dt); b = rand_storage(rng, (k, n), dt)\n"
+        "    out[str(i)] = device_gemm(a, b, dt)\n"
+        "np.savez(sys.argv[1], **out)\n"
+    ) % (os.path.dirname(os.path.abspath(__file__)), os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    results = []
+    for flag in ("0", "1"):
+        path = str(tmp_path / f"exchange{flag}.npz")
+        env = dict(os.environ, RP_HIP_NO_L2_EXCHANGE=flag)
+        subprocess.run([sys.executable, "-c", code, path], check=True, env=env, timeout=300)
+        results.append(np.load(path))
+    for key in results[0].files:
+        assert np.array_equal(results[0][key], results[1][key]), f"case {key}: the two exchanges disagree"
+
+
 @pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
 def test_ragged_small_outputs_deep_k(dt):
     """Outputs that no vector kernel takes (n = 10, odd strides) with a deep k.  16-bit: the generic kernel splits k

@@ -11,8 +11,17 @@ import pytest
 from recpulse_amd import capi
 from devhelp import BF16, F16, F32, rand_storage
 
+import ctypes
+
 pytestmark = pytest.mark.gpu
 WORKSPACE = 16 << 20            # RP_HIP_NOALLOC_WORKSPACE_BYTES
+
+
+def _alloc_counters():
+    """(calls to rp_hip_malloc, calls that reached hipMalloc, live blocks, cached blocks) of the process so far."""
+    v = [ctypes.c_longlong(0) for _ in range(4)]
+    capi.check(capi.lib().rp_hip_memory_stats(*[ctypes.byref(x) for x in v]), "rp_hip_memory_stats")
+    return tuple(x.value for x in v)
 
 
 def _both(rng, m, k, n, dtype, bias=False, accumulate=False, b_transposed=False):
@@ -28,7 +37,10 @@ def _both(rng, m, k, n, dtype, bias=False, accumulate=False, b_transposed=False)
     for entry in ("rp_hip_gemm_strided_batched", "rp_hip_gemm_strided_batched_noalloc"):
         dc = capi.DeviceBuffer.from_numpy(c0)
         fn = getattr(capi.lib(), entry)
+        before = _alloc_counters()
         capi.check(fn(dc.ptr, da.ptr, db.ptr, dbias.ptr if dbias else None, 1, m, k, n, 0, k, 1, *b_st, 0, n, 1, int(accumulate), dtype), entry)
+        if entry.endswith("_noalloc"):              # the contract itself: no request to the pool, no hipMalloc, nothing held or parked
+            assert _alloc_counters() == before, (entry, before, _alloc_counters())
         capi.synchronize()
         outs.append(dc.to_numpy(capi.NP_STORAGE[dtype], (m, n)).copy())
         dc.free()
@@ -74,10 +86,47 @@ def test_noalloc_rejects_a_workspace_beyond_the_fixed_array():
     a, b = rand_storage(rng, (m, k), BF16), rand_storage(rng, (k, n), BF16)
     da, db, dc = capi.DeviceBuffer.from_numpy(a), capi.DeviceBuffer.from_numpy(b), capi.DeviceBuffer(m * n * 2)
     L = capi.lib()
+    before = _alloc_counters()
     rc = L.rp_hip_gemm_strided_batched_noalloc(dc.ptr, da.ptr, db.ptr, None, 1, m, k, n, 0, k, 1, 0, n, 1, 0, n, 1, 0, BF16)
     assert rc == -1
+    assert _alloc_counters() == before              # the refusal allocates nothing either
     msg = L.rp_hip_last_error().decode()
     assert "workspace" in msg and str(WORKSPACE) in msg, msg
     capi.synchronize()
     want, got = _both(rng, 8, 2048, 1024, BF16)
     assert np.array_equal(want, got)
+
+
+@pytest.mark.parametrize("m,k,n", [(8, 4096, 4096), (32, 4096, 4096)])
+def test_noalloc_recorded_into_a_graph_replays_like_the_eager_call(m, k, n):
+    """The callers the entry point is for include code under HIP graph capture.  After a warm eager call the entry is
+    recorded on a created stream (single-launch k-split finish at 8 rows, partial sums + combine launch at 32), the
+    graph is replayed three times with other work and a synchronisation in between, and every replay must leave the
+    eager result; neither the recording nor the replays may touch the allocator."""
+    rng = np.random.default_rng(74)
+    a, b = rand_storage(rng, (m, k), BF16), rand_storage(rng, (k, n), BF16)
+    da, db = capi.DeviceBuffer.from_numpy(a), capi.DeviceBuffer.from_numpy(b)
+    d_eager, d_graph, d_other = (capi.DeviceBuffer(m * n * 2) for _ in range(3))
+    L = capi.lib()
+
+    def call(dst):
+        capi.check(L.rp_hip_gemm_strided_batched_noalloc(dst.ptr, da.ptr, db.ptr, None, 1, m, k, n, 0, k, 1, 0, n, 1, 0, n, 1, 0, BF16), "noalloc")
+
+    call(d_eager)                                   # warm: resolves the fixed array's address, measures workgroup placement
+    capi.synchronize()
+    want = d_eager.to_numpy(np.uint16, (m, n)).copy()
+    stream = capi.Stream()
+    with stream:
+        before = _alloc_counters()
+        with capi.Graph.capture() as graph:
+            call(d_graph)
+        assert _alloc_counters() == before
+        for replay in range(3):
+            capi.check(L.rp_hip_memset(d_graph.ptr, 0xff, m * n * 2), "memset")
+            graph.launch()
+            capi.check(L.rp_hip_stream_synchronize(), "sync")
+            assert np.array_equal(d_graph.to_numpy(np.uint16, (m, n)), want), f"replay {replay}"
+            # the program's own eager work between replays: another product through the allocating entry, on this stream
+            capi.gemm(d_other.ptr, da.ptr, db.ptr, None, 1, m, k, n, (0, k, 1), (0, n, 1), (0, n, 1), False, BF16)
+            capi.check(L.rp_hip_stream_synchronize(), "sync")
+        assert _alloc_counters()[2] == before[2]    # no block of the recording stays handed out
