@@ -22,7 +22,21 @@ sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3, "f64": 78.6}     # MI355X dense MFMA
 PEAK_HBM_GBS = 8000.0
-FWD_TRAFFIC_BYTES = 1.745e9      # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the forward GEMM, see profiles/pmc_traffic_gemm_bf16_8192.md
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "pmc_traffic_gemm_bf16_8192.md")
+
+
+def forward_traffic(kernel):
+    """HBM-side bytes per launch of the forward GEMM as the committed counter summary records them (its line
+    `roofline.traffic: <bytes> (<kernel>)`), or None when the summary is absent or was taken from another kernel than
+    the one this run dispatched: the figure is a counter reading, never a constant of this script."""
+    try:
+        import re
+        m = re.search(r"roofline\.traffic:\s*([0-9.eE+]+)\s*\(([^)]+)\)", open(TRAFFIC_PROFILE).read())
+    except OSError:
+        return None
+    if not m or m.group(2).strip() != kernel:
+        return None
+    return float(m.group(1))
 
 
 def _bf16_bits(x32):
@@ -719,6 +733,9 @@ def main():
                     help="run the forward 8192^3 bf16 GEMM back to back for this many seconds on --data operands while polling amd-smi "
                          "for shader clock and socket power, and print those figures (evidence for the power-limit reading of the headline)")
     ap.add_argument("--sustain-dtype", choices=["bf16", "f16"], default="bf16", help="16-bit type of the --sustain run")
+    ap.add_argument("--sweep-only", action="store_true",
+                    help="run only the configuration-3 sweep below the headline size: N = 1024 and 4096, bf16 and fp16, forward, dA, dB "
+                         "(for profiling those kernels alone)")
     ap.add_argument("--f16-only", action="store_true",
                     help="run only the fp16 8192^3 forward GEMM (for profiling that kernel alone)")
     ap.add_argument("--calibrate", action="store_true",
@@ -747,6 +764,9 @@ def main():
         return
     if args.skinny_only:
         print(json.dumps({"skinny": skinny_times(capi, rows=(1, 8, 32))}))
+        return
+    if args.sweep_only:
+        print(json.dumps({"square_sweep": square_sweep(capi)}))
         return
     if args.f16_only:
         print(json.dumps({"gemm_f16_8192": f16_time(capi)}))
@@ -780,9 +800,10 @@ def main():
                                "C=A·B, dA=dC·Bᵀ, dB=Aᵀ·dC with transposes as stride views; A,B,dC ~ N(0,1) seed 2",
                    "m": 8192, "n": 8192, "k": 8192, "gemms_per_step": 3},
         "roofline": {"bound": "mfma", "achieved": h["fwd_tflops"], "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
-                     "frac": h["fwd_tflops"] / PEAK_TFLOPS["bf16"], "traffic": FWD_TRAFFIC_BYTES,
+                     "frac": h["fwd_tflops"] / PEAK_TFLOPS["bf16"], "traffic": forward_traffic(h["kernel"]),
                      "traffic_note": "bytes per launch below the L2s (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, scaled by a copy kernel), "
-                                     "from profiles/pmc_traffic_gemm_bf16_8192.md; algorithmic bytes are 4.027e8",
+                                     "read from profiles/pmc_traffic_gemm_bf16_8192.md (null if that summary is of another kernel); "
+                                     "algorithmic bytes are 4.027e8",
                      "kernel": h["kernel"] + " (forward, A row-major x B row-major)",
                      "avg_launch_ms": h["kernel_ms"]["fwd_nn"]},
         "kernel_ms": h["kernel_ms"], "sampled_rel_err": h["sampled_rel_err"],

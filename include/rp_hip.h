@@ -143,6 +143,10 @@ const char* rp_hip_gemm_kernel_name(int batch, int m, int k, int n,
                                     long long a_rs, long long a_cs,
                                     long long b_rs, long long b_cs,
                                     long long c_rs, long long c_cs, int dtype);
+/* Name of the kernel family and tile that the calling thread's most recent GEMM entry-point call dispatched ("none"
+ * before the first): unlike rp_hip_gemm_kernel_name it reflects the bias, the accumulate flag and the pointers of that
+ * call.  No counterpart in the reference (whose device GEMM is one cuBLAS call). */
+const char* rp_hip_last_gemm_kernel(void);
 
 /* ------------------------------------------------------------------------
  * The other device entry points the benchmark configurations touch.  Names and

@@ -53,6 +53,7 @@ SIGNATURES = {
     "rp_hip_gemm_strided_batched": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i] + [_ll] * 9 + [_i, _i]),
     "rp_hip_gemm_strided_batched_noalloc": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i] + [_ll] * 9 + [_i, _i]),
     "rp_hip_gemm_kernel_name": (ctypes.c_char_p, [_i, _i, _i, _i] + [_ll] * 6 + [_i]),
+    "rp_hip_last_gemm_kernel": (ctypes.c_char_p, []),
     "add_kernel_device": (_i, [_vp, _vp, _vp, _sz, _i]),
     "add_strided_kernel_device": (_i, [_vp, _vp, _vp, _i, _ip, _ip, _ip, _sz, _i]),
     "mul_scalar_kernel_device": (_i, [_vp, _vp, _vp, _sz, _i]),
@@ -175,6 +176,11 @@ def gemm(c_ptr, a_ptr, b_ptr, bias_ptr, batch, m, k, n, a_st, b_st, c_st, accumu
     check(lib().rp_hip_gemm_strided_batched(c_ptr, a_ptr, b_ptr, bias_ptr, batch, m, k, n,
                                             *[int(s) for s in a_st], *[int(s) for s in b_st], *[int(s) for s in c_st],
                                             int(bool(accumulate)), dtype), "rp_hip_gemm_strided_batched")
+
+
+def last_gemm_kernel():
+    """Kernel that the calling thread's most recent GEMM call dispatched (reflects bias, accumulation and pointers)."""
+    return lib().rp_hip_last_gemm_kernel().decode()
 
 
 def gemm_kernel_name(batch, m, k, n, a_rc, b_rc, c_rc, dtype):

@@ -81,6 +81,18 @@ __device__ __forceinline__ uint16_t narrow_f16_bits(float x) {
     return (uint16_t)(bits | ((w >> 16) & 0x8000u));
 }
 
+// The same narrowing for values whose result is a normal fp16 number (2^-14 <= |x| < 65520): there the first dropped
+// bit is bit 12 of the fp32 pattern, adding it to the pattern carries into the kept bits exactly when it is set (into
+// the exponent too, which is the next power of two), and the hardware's truncating conversion drops the rest: two
+// instructions instead of twelve.  f16_range_key(x) is below F16_NORMAL_SPAN exactly for those values (NaN, infinities,
+// zeros and subnormal results are not), so a wave takes this path for a tile after one unsigned maximum over its keys.
+constexpr uint32_t F16_NORMAL_SPAN = (0x477FF000u << 1) - (0x38800000u << 1);
+__device__ __forceinline__ uint32_t f16_range_key(float x) { return (__float_as_uint(x) << 1) - (0x38800000u << 1); }
+__device__ __forceinline__ uint16_t narrow_f16_normal_bits(float x) {
+    const float bumped = __uint_as_float(__float_as_uint(x) + 0x1000u);
+    return (uint16_t)__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bumped, 0.f));
+}
+
 template <typename T> __device__ __forceinline__ T narrow(typename traits<T>::acc v);
 template <> __device__ __forceinline__ float narrow<float>(float v) { return v; }
 template <> __device__ __forceinline__ double narrow<double>(double v) { return v; }

@@ -202,29 +202,32 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     return p;
 }
 
+static thread_local const char* g_last_kernel = "none";      // what rp_hip_last_gemm_kernel reports
+
 static int run_gemm(const GemmArgs& g, int dtype) {
     Plan p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype);
     if (p.fam == FAM_PIPE32) {
-        if (pipe32_takes(g)) return launch_pipe32(g);
+        if (pipe32_takes(g)) { g_last_kernel = p.name; return launch_pipe32(g); }
         p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype, false);     // options, base pointers or spans it does not take
     }
     if (p.fam == FAM_PIPE16) {
-        if (pipe16_takes(g)) return launch_pipe16(g, dtype);
+        if (pipe16_takes(g)) { g_last_kernel = p.name; return launch_pipe16(g, dtype); }
         p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype, false);
     }
     if (p.fam == FAM_PIPE16K) {
-        if (pipe16k_takes(g)) return launch_pipe16k(g, dtype);
+        if (pipe16k_takes(g)) { g_last_kernel = p.name; return launch_pipe16k(g, dtype); }
         p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype, false);
     }
     if (p.fam == FAM_PIPE32K) {
-        if (pipe32k_takes(g)) return launch_pipe32k(g);
+        if (pipe32k_takes(g)) { g_last_kernel = p.name; return launch_pipe32k(g); }
         p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype, false);
     }
     if (p.fam == FAM_DIRECT32) {
-        if (direct32_takes(g)) return launch_direct32(g);
+        if (direct32_takes(g)) { g_last_kernel = p.name; return launch_direct32(g); }
         p = make_plan(g.batch, g.m, g.k, g.n, g.a_rs, g.a_cs, g.b_rs, g.b_cs, g.c_rs, g.c_cs, g.a_bs, g.b_bs, dtype, false);     // base pointers or spans it cannot address
     }
-    if (p.fam != FAM_GENERIC && p.fam != FAM_TINY && !(aligned16(g.A) && aligned16(g.B))) p.fam = FAM_GENERIC;
+    if (p.fam != FAM_GENERIC && p.fam != FAM_TINY && !(aligned16(g.A) && aligned16(g.B))) { p.fam = FAM_GENERIC; p.name = "generic"; }
+    g_last_kernel = p.name;
     switch (p.fam) {
         case FAM_MFMA16:
         case FAM_MFMA16_SKINNY: return launch_mfma16(g, p, dtype);
@@ -424,6 +427,8 @@ int rp_hip_linear_backward(void* dx, void* dw, void* db, const void* dy, const v
     if (db && rp_hip_reduce_rows(db, dy, m, n, accumulate_db, dtype) != 0) return -1;
     return 0;
 }
+
+const char* rp_hip_last_gemm_kernel(void) { return g_last_kernel; }
 
 const char* rp_hip_gemm_kernel_name(int batch, int m, int k, int n, long long a_rs, long long a_cs,
                                     long long b_rs, long long b_cs, long long c_rs, long long c_cs, int dtype) {

@@ -479,6 +479,24 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
             const bool by_row = g.bias_by_row != 0;
             const float bcol = (has_bias && !by_row && (!EDGE || gnl < g.n)) ? widen(bias[gnl]) : 0.f;
             auto stage = [&](auto with_bias, auto row_bias) {
+                if constexpr (std::is_same<T, f16_t>::value && !decltype(with_bias)::value) {
+                    // fp16 without a bias: when every value of this column of tiles narrows to a normal number (one
+                    // unsigned maximum per value to find out, wave-uniform), the two-instruction narrowing is exact
+                    uint32_t worst = 0;
+                    static_for<0, TMI * NV>([&](auto ivc) {
+                        constexpr int i = decltype(ivc)::value / NV, v = decltype(ivc)::value % NV;
+                        const uint32_t key = f16_range_key(acc[i][j][v]);
+                        worst = key > worst ? key : worst;
+                    });
+                    if (__builtin_amdgcn_ballot_w64(worst >= F16_NORMAL_SPAN) == 0) {
+                        static_for<0, TMI * NV>([&](auto ivc) {
+                            constexpr int i = decltype(ivc)::value / NV, v = decltype(ivc)::value % NV;
+                            const int row = MT == 32 ? i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4) : i * 16 + 4 * (lane >> 4) + v;
+                            region[row * EP + col] = narrow_f16_normal_bits(acc[i][j][v]);
+                        });
+                        return;
+                    }
+                }
                 static_for<0, TMI * NV>([&](auto ivc) {
                     {
                         constexpr int i = decltype(ivc)::value / NV, v = decltype(ivc)::value % NV;

@@ -92,7 +92,10 @@ __device__ __forceinline__ void p16_read_tr(s16x8_t& v, const unsigned char* p) 
 // its free index (m, n) instead of along k: it lies in LDS as 64 k rows of 128 free indices (256 bytes) whose 32-byte
 // pieces are XORed with the low three bits of the k row, and its fragments are transposing reads (ds_read_b64_tr_b16);
 // EDGE: m or n not whole tiles.
-template <typename T, int KST, bool A_MC, bool B_MC, bool EDGE>
+// BIAS: g.bias[n] is added to every row after the product has been rounded to the tensor type (the reference's two ops):
+// on the 16-bit row pieces between the staging patch and memory, with the lane's eight bias values of a tile loaded
+// while that tile is multiplied, one tile before its stores.
+template <typename T, int KST, bool A_MC, bool B_MC, bool EDGE, bool BIAS>
 __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_m, int tiles_n, unsigned total) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char p16_smem[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -210,6 +213,13 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     u32x2_t packed[16];                 // the previous tile, narrowed: [jm][in][q]
     u32x4_t rows[8];                    // the previous tile's row segments on their way from the staging patch to memory
     s16x8_t af[KST][2], bf[KST][2];     // [k step][tile]: eight k values of the lane's row
+    u32x4_t bias_prev = {0u, 0u, 0u, 0u}, bias_cur = {0u, 0u, 0u, 0u};      // BIAS: of columns n0 + wn0 + 8 rp .. + 7 of the tile being stored / multiplied
+    auto load_bias = [&](const P16Tile& t) {
+        const int gn = t.n0 + wn0 + 8 * rp;
+        bias_cur = gn < g.n ? *(const u32x4_t*)((const uint16_t*)g.bias + gn) : u32x4_t{0u, 0u, 0u, 0u};       // (n is a multiple of 8)
+    };
+    auto widen_lo = [](uint32_t w) { T x; x.bits = (uint16_t)w; return widen(x); };
+    auto widen_hi = [](uint32_t w) { T x; x.bits = (uint16_t)(w >> 16); return widen(x); };
 
     auto pack_all = [&]() {
         p16_static_for<0, 16>([&](auto nc) {
@@ -229,6 +239,11 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
         constexpr int e = decltype(e_c)::value;
         const int row = 8 * e + rr;
         rows[e] = *(const u32x4_t*)(stage + row * P16_ROW_BYTES + (((uint32_t)rp ^ (uint32_t)((row >> 1) & 7)) * 16));
+        if constexpr (BIAS) {
+#pragma unroll
+            for (int d = 0; d < 4; d++)
+                rows[e][d] = p16_ops<T>::pack(widen_lo(rows[e][d]) + widen_lo(bias_prev[d]), widen_hi(rows[e][d]) + widen_hi(bias_prev[d]));
+        }
     };
     // ... and to memory
     auto row_store = [&](auto e_c, const P16Tile& t, const __amdgpu_buffer_rsrc_t& rc) {
@@ -301,13 +316,17 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     unsigned id = first;
     if (id >= total) return;
     p16_static_for<0, KST>([&](auto sc) { read_frags(p16_smem, sc); });
+    if constexpr (BIAS) load_bias(p16_tile(id, per_matrix, tiles_n));
     tile_pass(std::false_type{}, next, prev);
     prev = p16_tile(id, per_matrix, tiles_n);
+    if constexpr (BIAS) bias_prev = bias_cur;
     next = next + 1 == P16_NBUF ? 0 : next + 1;
     id += stride;
     for (; id < total; id += stride) {
+        if constexpr (BIAS) load_bias(p16_tile(id, per_matrix, tiles_n));
         tile_pass(std::true_type{}, next, prev);
         prev = p16_tile(id, per_matrix, tiles_n);
+        if constexpr (BIAS) bias_prev = bias_cur;
         next = next + 1 == P16_NBUF ? 0 : next + 1;
     }
     // the last tile
@@ -320,13 +339,14 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
 // ---- host side ----
 
 // Whether this kernel takes the product: k <= 64 in whole 16-byte pieces, both operands with a unit stride and
-// 16-byte aligned rows, C row-major with 16-byte aligned rows and n in whole eights, overwritten (no accumulation, bias,
-// segments or folded store), and every byte offset the kernel forms from a batch entry's base within the 32-bit range
-// of buffer addressing.
+// 16-byte aligned rows, C row-major with 16-byte aligned rows and n in whole eights, overwritten (a bias per column,
+// 16-byte aligned, is taken; no accumulation, whose extra read of C leaves the product bound by memory at the tiled
+// kernel's speed; no segments or folded store), and every byte offset the kernel forms from a batch entry's base within
+// the 32-bit range of buffer addressing.
 bool pipe16_takes(const GemmArgs& g) {
     if (g.k > P16_MAXK || g.k < 8 || g.k % 8 || g.m < 1 || g.n < 8 || g.n % 8 || g.batch < 1) return false;
     if ((long long)((g.m + P16_BM - 1) / P16_BM) * ((g.n + P16_BN - 1) / P16_BN) * g.batch >= (1ll << 30)) return false;
-    if (g.bias || g.accumulate || g.seg_k || g.seg_n || g.c_fold_from || g.bias_by_row) return false;
+    if (g.accumulate || g.seg_k || g.seg_n || g.c_fold_from || g.bias_by_row || ((uintptr_t)g.bias & 15)) return false;
     const bool a_kc = g.a_cs == 1 && g.a_rs % 8 == 0, a_mc = g.a_rs == 1 && g.a_cs % 8 == 0;
     const bool b_kc = g.b_rs == 1 && g.b_cs % 8 == 0, b_mc = g.b_cs == 1 && g.b_rs % 8 == 0;
     if (!(a_kc || a_mc) || !(b_kc || b_mc) || g.a_bs % 8 || g.b_bs % 8 || g.a_rs < 0 || g.a_cs < 0 || g.b_rs < 0 || g.b_cs < 0) return false;
@@ -356,15 +376,16 @@ static int launch_pipe16_t(const GemmArgs& g) {
         return check_launch("gemm_pipe16_kernel") ? 0 : -1;
     };
     const bool a_mc = !(g.a_cs == 1 && g.a_rs % 8 == 0), b_mc = !(g.b_rs == 1 && g.b_cs % 8 == 0);
-    auto pick = [&](auto kst_c) {
+    auto pick = [&](auto kst_c, auto bias_c) {
         constexpr int KST = decltype(kst_c)::value;
-        if (!a_mc && !b_mc) return edge ? launch(gemm_pipe16_kernel<T, KST, false, false, true>) : launch(gemm_pipe16_kernel<T, KST, false, false, false>);
-        if (!a_mc && b_mc) return edge ? launch(gemm_pipe16_kernel<T, KST, false, true, true>) : launch(gemm_pipe16_kernel<T, KST, false, true, false>);
-        if (a_mc && !b_mc) return edge ? launch(gemm_pipe16_kernel<T, KST, true, false, true>) : launch(gemm_pipe16_kernel<T, KST, true, false, false>);
-        return edge ? launch(gemm_pipe16_kernel<T, KST, true, true, true>) : launch(gemm_pipe16_kernel<T, KST, true, true, false>);
+        constexpr bool BIAS = decltype(bias_c)::value;
+        if (!a_mc && !b_mc) return edge ? launch(gemm_pipe16_kernel<T, KST, false, false, true, BIAS>) : launch(gemm_pipe16_kernel<T, KST, false, false, false, BIAS>);
+        if (!a_mc && b_mc) return edge ? launch(gemm_pipe16_kernel<T, KST, false, true, true, BIAS>) : launch(gemm_pipe16_kernel<T, KST, false, true, false, BIAS>);
+        if (a_mc && !b_mc) return edge ? launch(gemm_pipe16_kernel<T, KST, true, false, true, BIAS>) : launch(gemm_pipe16_kernel<T, KST, true, false, false, BIAS>);
+        return edge ? launch(gemm_pipe16_kernel<T, KST, true, true, true, BIAS>) : launch(gemm_pipe16_kernel<T, KST, true, true, false, BIAS>);
     };
-    if (g.k <= 32) return pick(std::integral_constant<int, 2>{});
-    return pick(std::integral_constant<int, 4>{});
+    if (g.k <= 32) return g.bias ? pick(std::integral_constant<int, 2>{}, std::true_type{}) : pick(std::integral_constant<int, 2>{}, std::false_type{});
+    return g.bias ? pick(std::integral_constant<int, 4>{}, std::true_type{}) : pick(std::integral_constant<int, 4>{}, std::false_type{});
 }
 
 int launch_pipe16(const GemmArgs& g, int dtype) {

@@ -77,8 +77,18 @@ __device__ __forceinline__ void k16_read_tr(s16x8_t& v, const unsigned char* p) 
     v[4 * H + 0] = q[0]; v[4 * H + 1] = q[1]; v[4 * H + 2] = q[2]; v[4 * H + 3] = q[3];
 }
 
+// 16-bit storage -> fp32 and back for the epilogue's additions (one rounding per reference op, like finish<T>)
+template <typename T> __device__ __forceinline__ float k16_widen_lo(uint32_t w);
+template <typename T> __device__ __forceinline__ float k16_widen_hi(uint32_t w);
+template <> __device__ __forceinline__ float k16_widen_lo<bf16_t>(uint32_t w) { return __uint_as_float(w << 16); }
+template <> __device__ __forceinline__ float k16_widen_hi<bf16_t>(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
+template <> __device__ __forceinline__ float k16_widen_lo<f16_t>(uint32_t w) { f16_t x; x.bits = (uint16_t)w; return widen(x); }
+template <> __device__ __forceinline__ float k16_widen_hi<f16_t>(uint32_t w) { f16_t x; x.bits = (uint16_t)(w >> 16); return widen(x); }
+
 // A_MC / B_MC: the operand has unit stride along its free index (m, n) instead of along k.  EDGE: m not in whole tiles or n below 64.
-template <typename T, bool A_MC, bool B_MC, bool EDGE>
+// EPI: a bias per column and / or accumulation into C (g.bias, g.accumulate): the tile is then stored right after its
+// last slab instead of between the MFMAs of the next tile, the old rows of C having been requested when the tile began.
+template <typename T, bool A_MC, bool B_MC, bool EDGE, bool EPI>
 __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles_m, unsigned total) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char k16_smem[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -211,6 +221,21 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
     u32x2_t packed[8];                  // the previous tile, narrowed: [in][q]
     u32x4_t rows[4];                    // its rows on their way from the staging patch to memory
     s16x8_t af[4], bf[4][2];            // [k step]([in]): eight k values of the lane's row / column
+    // EPI: the bias of the lane's columns 32 in + 8 q + 4 h + e as fp32 (the same for every tile: n <= 64), and the old
+    // rows of C of the current tile (pieces like `rows`)
+    float bias_f[EPI ? 32 : 1];
+    u32x4_t old[EPI ? 4 : 1];
+    const bool has_bias = EPI && g.bias != nullptr, accum = EPI && g.accumulate != 0;
+    if constexpr (EPI) {
+#pragma unroll
+        for (int n = 0; n < 8; n++) {
+            const int col = 32 * (n >> 2) + 8 * (n & 3) + 4 * h;
+            u32x2_t w = {0u, 0u};
+            if (has_bias && col < g.n) w = *(const u32x2_t*)((const uint16_t*)g.bias + col);          // (n is a multiple of 8: four columns are inside or outside together)
+            bias_f[4 * n + 0] = k16_widen_lo<T>(w[0]); bias_f[4 * n + 1] = k16_widen_hi<T>(w[0]);
+            bias_f[4 * n + 2] = k16_widen_lo<T>(w[1]); bias_f[4 * n + 3] = k16_widen_hi<T>(w[1]);
+        }
+    }
 
     auto read_frags = [&](const unsigned char* stage, auto ks_c) {
         constexpr int ks = decltype(ks_c)::value;
@@ -233,7 +258,14 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
     auto pack_all = [&]() {
         k16_static_for<0, 8>([&](auto nc) {
             constexpr int n = decltype(nc)::value, in = n >> 2, q = n & 3;
-            const float v0 = acc[in][4 * q], v1 = acc[in][4 * q + 1], v2 = acc[in][4 * q + 2], v3 = acc[in][4 * q + 3];
+            float v0 = acc[in][4 * q], v1 = acc[in][4 * q + 1], v2 = acc[in][4 * q + 2], v3 = acc[in][4 * q + 3];
+            if constexpr (EPI) {
+                if (has_bias) {                        // the product is rounded to the tensor type first, like the reference's matmul output
+                    const uint32_t p01 = k16_ops<T>::pack(v0, v1), p23 = k16_ops<T>::pack(v2, v3);
+                    v0 = k16_widen_lo<T>(p01) + bias_f[4 * n + 0]; v1 = k16_widen_hi<T>(p01) + bias_f[4 * n + 1];
+                    v2 = k16_widen_lo<T>(p23) + bias_f[4 * n + 2]; v3 = k16_widen_hi<T>(p23) + bias_f[4 * n + 3];
+                }
+            }
             packed[n][0] = k16_ops<T>::pack(v0, v1);
             packed[n][1] = k16_ops<T>::pack(v2, v3);
         });
@@ -254,6 +286,22 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
         uint32_t voff = c_lane;
         if constexpr (EDGE) voff = (gm + rr < g.m && 8 * rp < g.n) ? c_lane : K16_OOB;      // (n is a multiple of 8: a piece is inside or outside as a whole)
         __builtin_amdgcn_raw_buffer_store_b128(rows[e], rc, (int)voff, soff, 2);          // (streaming store: the output is not read again by this kernel)
+    };
+
+    // EPI: request the rows of C that tile (pm0, rc) will be added to; add them to the finished rows
+    auto old_load = [&](auto e_c, int pm0, const __amdgpu_buffer_rsrc_t& rc) {
+        constexpr int e = decltype(e_c)::value;
+        const int gm = pm0 + 32 * wave + 8 * e;
+        const int soff = (int)((long long)gm * g.c_rs * 2);
+        uint32_t voff = c_lane;
+        if constexpr (EDGE) voff = (gm + rr < g.m && 8 * rp < g.n) ? c_lane : K16_OOB;
+        old[e] = __builtin_amdgcn_raw_buffer_load_b128(rc, (int)voff, soff, 0);
+    };
+    auto row_add_old = [&](auto e_c) {
+        constexpr int e = decltype(e_c)::value;
+#pragma unroll
+        for (int d = 0; d < 4; d++)
+            rows[e][d] = k16_ops<T>::pack(k16_widen_lo<T>(old[e][d]) + k16_widen_lo<T>(rows[e][d]), k16_widen_hi<T>(old[e][d]) + k16_widen_hi<T>(rows[e][d]));
     };
 
     // One slab, whose fragments are already in registers: behind each k step's MFMAs the same fragments of the NEXT slab
@@ -290,6 +338,23 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
         for (int in = 0; in < 2; in++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[in][v] = 0.f;
+        if constexpr (EPI) {
+            // this tile's place in C is known from the start: its old rows travel while the tile is multiplied
+            const unsigned z = id / (unsigned)tiles_m;
+            pm0 = (int)(id - z * (unsigned)tiles_m) * K16_BM;
+            rc = k16_rsrc((uint16_t*)g.C + (long long)z * g.c_bs, c_span);
+            if (accum) k16_static_for<0, 4>([&](auto ec) { old_load(ec, pm0, rc); });
+            for (int s = 0; s < nslab; s++) {
+                slab_pass(std::false_type{}, next, pm0, rc);
+                next = next + 1 == K16_NBUF ? 0 : next + 1;
+            }
+            pack_all();
+            k16_static_for<0, 8>([&](auto nc) { stage_write(nc); });
+            k16_static_for<0, 4>([&](auto ec) { row_read(ec); });
+            if (accum) k16_static_for<0, 4>([&](auto ec) { row_add_old(ec); });
+            k16_static_for<0, 4>([&](auto ec) { row_store(ec, pm0, rc); });
+            continue;
+        }
         for (int s = 0; s < nslab; s++) {
             if (pending) slab_pass(std::true_type{}, next, pm0, rc);
             else slab_pass(std::false_type{}, next, pm0, rc);
@@ -302,6 +367,7 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
         rc = k16_rsrc((uint16_t*)g.C + (long long)z * g.c_bs, c_span);
         pending = true;
     }
+    if constexpr (EPI) return;
     // the last tile
     k16_static_for<0, 8>([&](auto nc) { stage_write(nc); });
     k16_static_for<0, 4>([&](auto ec) { row_read(ec); });
@@ -311,12 +377,13 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
 // ---- host side ----
 
 // Whether this kernel takes the product: n <= 64 in whole eights, k in whole eights, both operands with a unit stride and
-// 16-byte aligned rows, C row-major with 16-byte aligned rows, overwritten (no accumulation, bias, segments or folded
-// store), and every byte offset the kernel forms from a batch entry's base within the 32-bit range of buffer addressing.
+// 16-byte aligned rows, C row-major with 16-byte aligned rows (no segments or folded store; a bias per column, 8-byte
+// aligned, and accumulation into C are taken), and every byte offset the kernel forms from a batch entry's base within
+// the 32-bit range of buffer addressing.
 bool pipe16k_takes(const GemmArgs& g) {
     if (g.n > K16_BN || g.n < 8 || g.n % 8 || g.k < 8 || g.k % 8 || g.m < 1 || g.batch < 1) return false;
     if ((long long)((g.m + K16_BM - 1) / K16_BM) * g.batch >= (1ll << 30)) return false;
-    if (g.bias || g.accumulate || g.seg_k || g.seg_n || g.c_fold_from || g.bias_by_row) return false;
+    if (g.seg_k || g.seg_n || g.c_fold_from || g.bias_by_row || ((uintptr_t)g.bias & 7)) return false;
     const bool a_kc = g.a_cs == 1 && g.a_rs % 8 == 0, a_mc = g.a_rs == 1 && g.a_cs % 8 == 0 && g.m % 8 == 0;
     const bool b_kc = g.b_rs == 1 && g.b_cs % 8 == 0, b_mc = g.b_cs == 1 && g.b_rs % 8 == 0;
     if (!(a_kc || a_mc) || !(b_kc || b_mc) || g.a_bs % 8 || g.b_bs % 8 || g.a_rs < 0 || g.a_cs < 0 || g.b_rs < 0 || g.b_cs < 0) return false;
@@ -346,10 +413,14 @@ static int launch_pipe16k_t(const GemmArgs& g) {
         hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), K16_SMEM_BYTES, current_stream(), g, tiles_m, (unsigned)total);
         return check_launch("gemm_pipe16k_kernel") ? 0 : -1;
     };
-    if (!a_mc && !b_mc) return edge ? launch(gemm_pipe16k_kernel<T, false, false, true>) : launch(gemm_pipe16k_kernel<T, false, false, false>);
-    if (!a_mc && b_mc) return edge ? launch(gemm_pipe16k_kernel<T, false, true, true>) : launch(gemm_pipe16k_kernel<T, false, true, false>);
-    if (a_mc && !b_mc) return edge ? launch(gemm_pipe16k_kernel<T, true, false, true>) : launch(gemm_pipe16k_kernel<T, true, false, false>);
-    return edge ? launch(gemm_pipe16k_kernel<T, true, true, true>) : launch(gemm_pipe16k_kernel<T, true, true, false>);
+    auto pick = [&](auto epi_c) {
+        constexpr bool EPI = decltype(epi_c)::value;
+        if (!a_mc && !b_mc) return edge ? launch(gemm_pipe16k_kernel<T, false, false, true, EPI>) : launch(gemm_pipe16k_kernel<T, false, false, false, EPI>);
+        if (!a_mc && b_mc) return edge ? launch(gemm_pipe16k_kernel<T, false, true, true, EPI>) : launch(gemm_pipe16k_kernel<T, false, true, false, EPI>);
+        if (a_mc && !b_mc) return edge ? launch(gemm_pipe16k_kernel<T, true, false, true, EPI>) : launch(gemm_pipe16k_kernel<T, true, false, false, EPI>);
+        return edge ? launch(gemm_pipe16k_kernel<T, true, true, true, EPI>) : launch(gemm_pipe16k_kernel<T, true, true, false, EPI>);
+    };
+    return (g.bias || g.accumulate) ? pick(std::true_type{}) : pick(std::false_type{});
 }
 
 int launch_pipe16k(const GemmArgs& g, int dtype) {

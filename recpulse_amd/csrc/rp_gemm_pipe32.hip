@@ -67,7 +67,9 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t p32_rsrc(const void* base, lon
 // A_MC / B_MC: the operand has unit stride along its free index (m, n) instead of along k: it lies in LDS as 64 k rows of
 // 128 free indices (512 bytes) whose 128-byte pieces are XORed with (k row / 4) % 4, so that the two halves of a wave, which
 // read k rows four apart, use different banks; its values are read one at a time.
-template <int KCH, bool A_MC, bool B_MC, bool EDGE>
+// BIAS: g.bias[n] is added to every row (the lane's two bias values of a tile are loaded while that tile is multiplied,
+// one tile before its stores).
+template <int KCH, bool A_MC, bool B_MC, bool EDGE, bool BIAS>
 __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_m, int tiles_n, unsigned total) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char p32_smem[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -137,6 +139,14 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
 
     f32x16_t acc[2][2][2];              // [set][i][j]
     f32x4_t af[2][2], bf[2][2];         // [slot][i or j]: four k values of the lane's row
+    float bias_prev[2] = {0.f, 0.f}, bias_cur[2] = {0.f, 0.f};      // BIAS: of columns n0 + wn0 + 32 j + r of the tile being stored / multiplied
+    auto load_bias = [&](const P32Tile& t) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int gn = t.n0 + wn0 + 32 * j + r;
+            bias_cur[j] = gn < g.n ? ((const float*)g.bias)[gn] : 0.f;
+        }
+    };
 
     // store number n (0..63) of accumulator set SET: register v of MFMA tile (i, j), i.e. columns 32j + r of rows 32i + 8(v / 4) + 4h + v % 4
     auto store_one = [&](auto set_c, auto n_c, const P32Tile& t, const __amdgpu_buffer_rsrc_t& rc) {
@@ -147,7 +157,8 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
         const int soff = (int)(((long long)gm * g.c_rs + (long long)gn * g.c_cs) * 4);
         uint32_t voff = c_lane;
         if constexpr (EDGE) voff = (gm + 4 * h < g.m && gn + r < g.n) ? c_lane : P32_OOB;
-        const float val = acc[SET][si][sj][v];
+        float val = acc[SET][si][sj][v];
+        if constexpr (BIAS) val = val + bias_prev[sj];
         __builtin_amdgcn_raw_buffer_store_b32(p32_bits(val), rc, (int)voff, soff, 2);          // (streaming store: the output is not read again by this kernel)
     };
 
@@ -217,20 +228,26 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
     unsigned id = first;
     if (id >= total) return;
     read_frags(p32_smem, 0, 0);
+    if constexpr (BIAS) load_bias(p32_tile(id, per_matrix, tiles_n));
     tile_pass(std::integral_constant<int, 0>{}, std::false_type{}, buf, prev);
     prev = p32_tile(id, per_matrix, tiles_n);
+    if constexpr (BIAS) { bias_prev[0] = bias_cur[0]; bias_prev[1] = bias_cur[1]; }
     buf ^= 1;
     id += stride;
     // two tiles per round, so that the accumulator sets are fixed registers
     while (id < total) {
+        if constexpr (BIAS) load_bias(p32_tile(id, per_matrix, tiles_n));
         tile_pass(std::integral_constant<int, 1>{}, std::true_type{}, buf, prev);
         prev = p32_tile(id, per_matrix, tiles_n);
+        if constexpr (BIAS) { bias_prev[0] = bias_cur[0]; bias_prev[1] = bias_cur[1]; }
         buf ^= 1;
         id += stride;
         last = 1;
         if (id >= total) break;
+        if constexpr (BIAS) load_bias(p32_tile(id, per_matrix, tiles_n));
         tile_pass(std::integral_constant<int, 0>{}, std::true_type{}, buf, prev);
         prev = p32_tile(id, per_matrix, tiles_n);
+        if constexpr (BIAS) { bias_prev[0] = bias_cur[0]; bias_prev[1] = bias_cur[1]; }
         buf ^= 1;
         id += stride;
         last = 0;
@@ -244,12 +261,13 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
 // ---- host side ----
 
 // Whether this kernel takes the product: fp32, k <= 64 in whole 16-byte pieces, both operands with a unit stride and
-// 16-byte aligned rows, C overwritten (no accumulation, bias, segments or folded store), and every byte offset the
-// kernel forms from a batch entry's base within the 32-bit range of buffer addressing.
+// 16-byte aligned rows, C overwritten (a bias per column is taken; no accumulation, whose extra read of C leaves the
+// product bound by memory at the tiled kernel's speed; no segments or folded store), and every byte offset the kernel
+// forms from a batch entry's base within the 32-bit range of buffer addressing.
 bool pipe32_takes(const GemmArgs& g) {
     if (g.k > P32_MAXK || g.k < 4 || g.k % 4 || g.m < 1 || g.n < 1 || g.batch < 1) return false;
     if ((long long)((g.m + P32_BM - 1) / P32_BM) * ((g.n + P32_BN - 1) / P32_BN) * g.batch >= (1ll << 30)) return false;
-    if (g.bias || g.accumulate || g.seg_k || g.seg_n || g.c_fold_from || g.bias_by_row) return false;
+    if (g.accumulate || g.seg_k || g.seg_n || g.c_fold_from || g.bias_by_row || ((uintptr_t)g.bias & 3)) return false;
     const bool a_kc = g.a_cs == 1 && g.a_rs % 4 == 0, a_mc = g.a_rs == 1 && g.a_cs % 4 == 0;
     const bool b_kc = g.b_rs == 1 && g.b_cs % 4 == 0, b_mc = g.b_cs == 1 && g.b_rs % 4 == 0;
     if (!(a_kc || a_mc) || !(b_kc || b_mc) || g.a_bs % 4 || g.b_bs % 4 || g.a_rs < 0 || g.a_cs < 0 || g.b_rs < 0 || g.b_cs < 0 || g.c_rs < 0 || g.c_cs < 0) return false;
@@ -277,15 +295,16 @@ int launch_pipe32(const GemmArgs& g) {
         return check_launch("gemm_pipe32_kernel") ? 0 : -1;
     };
     const bool a_mc = !(g.a_cs == 1 && g.a_rs % 4 == 0), b_mc = !(g.b_rs == 1 && g.b_cs % 4 == 0);
-    auto pick = [&](auto kch_c) {
+    auto pick = [&](auto kch_c, auto bias_c) {
         constexpr int KCH = decltype(kch_c)::value;
-        if (!a_mc && !b_mc) return edge ? launch(gemm_pipe32_kernel<KCH, false, false, true>) : launch(gemm_pipe32_kernel<KCH, false, false, false>);
-        if (!a_mc && b_mc) return edge ? launch(gemm_pipe32_kernel<KCH, false, true, true>) : launch(gemm_pipe32_kernel<KCH, false, true, false>);
-        if (a_mc && !b_mc) return edge ? launch(gemm_pipe32_kernel<KCH, true, false, true>) : launch(gemm_pipe32_kernel<KCH, true, false, false>);
-        return edge ? launch(gemm_pipe32_kernel<KCH, true, true, true>) : launch(gemm_pipe32_kernel<KCH, true, true, false>);
+        constexpr bool BIAS = decltype(bias_c)::value;
+        if (!a_mc && !b_mc) return edge ? launch(gemm_pipe32_kernel<KCH, false, false, true, BIAS>) : launch(gemm_pipe32_kernel<KCH, false, false, false, BIAS>);
+        if (!a_mc && b_mc) return edge ? launch(gemm_pipe32_kernel<KCH, false, true, true, BIAS>) : launch(gemm_pipe32_kernel<KCH, false, true, false, BIAS>);
+        if (a_mc && !b_mc) return edge ? launch(gemm_pipe32_kernel<KCH, true, false, true, BIAS>) : launch(gemm_pipe32_kernel<KCH, true, false, false, BIAS>);
+        return edge ? launch(gemm_pipe32_kernel<KCH, true, true, true, BIAS>) : launch(gemm_pipe32_kernel<KCH, true, true, false, BIAS>);
     };
-    if (g.k <= 32) return pick(std::integral_constant<int, 4>{});
-    return pick(std::integral_constant<int, 8>{});
+    if (g.k <= 32) return g.bias ? pick(std::integral_constant<int, 4>{}, std::true_type{}) : pick(std::integral_constant<int, 4>{}, std::false_type{});
+    return g.bias ? pick(std::integral_constant<int, 8>{}, std::true_type{}) : pick(std::integral_constant<int, 8>{}, std::false_type{});
 }
 
 }  // namespace rp

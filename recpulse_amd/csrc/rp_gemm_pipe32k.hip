@@ -50,7 +50,9 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t k32_rsrc(const void* base, lon
 __device__ __forceinline__ uint32_t k32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
 
 // A_MC / B_MC: the operand has unit stride along its free index (m, n) instead of along k.  EDGE: m not in whole tiles or n below 64.
-template <bool A_MC, bool B_MC, bool EDGE>
+// EPI: a bias per column and / or accumulation into C (g.bias, g.accumulate), with finish<float>'s order of additions;
+// the old values of C are requested when the tile begins, so they have arrived when its last slab is done.
+template <bool A_MC, bool B_MC, bool EDGE, bool EPI>
 __global__ void __launch_bounds__(512) gemm_pipe32k_kernel(GemmArgs g, int tiles_m, unsigned total) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char k32_smem[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -158,6 +160,14 @@ __global__ void __launch_bounds__(512) gemm_pipe32k_kernel(GemmArgs g, int tiles
 
     f32x16_t acc[2];                    // [j: columns 32 j .. 32 j + 31]
     float af[16], bf[2][16];            // [4u + e]: the lane's value for MFMA step (u, e)
+    const bool has_bias = EPI && g.bias != nullptr, accum = EPI && g.accumulate != 0;
+    float bias_v[2] = {0.f, 0.f};       // EPI: the bias of the lane's columns 32 j + r (the same for every tile: n <= 64)
+    float old[EPI ? 32 : 1];            // EPI: the current tile's old values of C, [16 j + v]
+    if constexpr (EPI) {
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+            if (has_bias && 32 * j + r < g.n) bias_v[j] = ((const float*)g.bias)[32 * j + r];
+    }
 
     auto read_group = [&](const unsigned char* stage, auto u_c) {
         constexpr int u = decltype(u_c)::value;
@@ -204,21 +214,38 @@ __global__ void __launch_bounds__(512) gemm_pipe32k_kernel(GemmArgs g, int tiles
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[j][v] = 0.f;
+        // register v of tile j is row 8(v / 4) + 4h + v % 4, columns 32 j + r
+        const unsigned z = id / (unsigned)tiles_m;
+        const int gm0 = (int)(id - z * (unsigned)tiles_m) * K32_BM + 32 * wave;
+        const __amdgpu_buffer_rsrc_t rc = k32_rsrc((float*)g.C + (long long)z * g.c_bs, c_span);
+        auto place = [&](auto nc, int& soff, uint32_t& voff) {
+            constexpr int n = decltype(nc)::value, j = n >> 4, v = n & 15, row = 8 * (v / 4) + (v % 4);
+            const int gm = gm0 + row;
+            soff = (int)(((long long)gm * g.c_rs + (long long)(32 * j) * g.c_cs) * 4);
+            voff = c_lane;
+            if constexpr (EDGE) voff = (gm + 4 * h < g.m && 32 * j + r < g.n) ? c_lane : K32_OOB;
+        };
+        if constexpr (EPI) {
+            if (accum) k32_static_for<0, 32>([&](auto nc) {
+                int soff; uint32_t voff;
+                place(nc, soff, voff);
+                old[decltype(nc)::value] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rc, (int)voff, soff, 0));
+            });
+        }
         for (int s = 0; s < nslab; s++) {
             slab_pass(next);
             next = next + 1 == K32_NBUF ? 0 : next + 1;
         }
-        // the tile's stores: register v of tile j is row 8(v / 4) + 4h + v % 4, columns 32 j + r
-        const unsigned z = id / (unsigned)tiles_m;
-        const int gm0 = (int)(id - z * (unsigned)tiles_m) * K32_BM + 32 * wave;
-        const __amdgpu_buffer_rsrc_t rc = k32_rsrc((float*)g.C + (long long)z * g.c_bs, c_span);
+        // the tile's stores
         k32_static_for<0, 32>([&](auto nc) {
-            constexpr int n = decltype(nc)::value, j = n >> 4, v = n & 15, row = 8 * (v / 4) + (v % 4);
-            const int gm = gm0 + row;
-            const int soff = (int)(((long long)gm * g.c_rs + (long long)(32 * j) * g.c_cs) * 4);
-            uint32_t voff = c_lane;
-            if constexpr (EDGE) voff = (gm + 4 * h < g.m && 32 * j + r < g.n) ? c_lane : K32_OOB;
-            const float val = acc[j][v];
+            constexpr int n = decltype(nc)::value, j = n >> 4, v = n & 15;
+            int soff; uint32_t voff;
+            place(nc, soff, voff);
+            float val = acc[j][v];
+            if constexpr (EPI) {
+                if (has_bias) val = val + bias_v[j];
+                if (accum) val = old[n] + val;
+            }
             __builtin_amdgcn_raw_buffer_store_b32(k32_bits(val), rc, (int)voff, soff, 2);          // (streaming store)
         });
     }
@@ -227,12 +254,12 @@ __global__ void __launch_bounds__(512) gemm_pipe32k_kernel(GemmArgs g, int tiles
 // ---- host side ----
 
 // Whether this kernel takes the product: fp32, n <= 64, k in whole fours, both operands with a unit stride and 16-byte
-// aligned rows, C overwritten (no accumulation, bias, segments or folded store), and every byte offset the kernel forms
-// from a batch entry's base within the 32-bit range of buffer addressing.
+// aligned rows (no segments or folded store; a bias per column and accumulation into C are taken), and every byte offset
+// the kernel forms from a batch entry's base within the 32-bit range of buffer addressing.
 bool pipe32k_takes(const GemmArgs& g) {
     if (g.n > K32_BN || g.n < 1 || g.k < 4 || g.k % 4 || g.m < 1 || g.batch < 1) return false;
     if ((long long)((g.m + K32_BM - 1) / K32_BM) * g.batch >= (1ll << 30)) return false;
-    if (g.bias || g.accumulate || g.seg_k || g.seg_n || g.c_fold_from || g.bias_by_row) return false;
+    if (g.seg_k || g.seg_n || g.c_fold_from || g.bias_by_row || ((uintptr_t)g.bias & 3)) return false;
     const bool a_kc = g.a_cs == 1 && g.a_rs % 4 == 0, a_mc = g.a_rs == 1 && g.a_cs % 4 == 0;
     const bool b_kc = g.b_rs == 1 && g.b_cs % 4 == 0, b_mc = g.b_cs == 1 && g.b_rs % 4 == 0;
     if (!(a_kc || a_mc) || !(b_kc || b_mc) || g.a_bs % 4 || g.b_bs % 4 || g.a_rs < 0 || g.a_cs < 0 || g.b_rs < 0 || g.b_cs < 0) return false;
@@ -261,10 +288,14 @@ int launch_pipe32k(const GemmArgs& g) {
         hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), K32_SMEM_BYTES, current_stream(), g, tiles_m, (unsigned)total);
         return check_launch("gemm_pipe32k_kernel") ? 0 : -1;
     };
-    if (!a_mc && !b_mc) return edge ? launch(gemm_pipe32k_kernel<false, false, true>) : launch(gemm_pipe32k_kernel<false, false, false>);
-    if (!a_mc && b_mc) return edge ? launch(gemm_pipe32k_kernel<false, true, true>) : launch(gemm_pipe32k_kernel<false, true, false>);
-    if (a_mc && !b_mc) return edge ? launch(gemm_pipe32k_kernel<true, false, true>) : launch(gemm_pipe32k_kernel<true, false, false>);
-    return edge ? launch(gemm_pipe32k_kernel<true, true, true>) : launch(gemm_pipe32k_kernel<true, true, false>);
+    auto pick = [&](auto epi_c) {
+        constexpr bool EPI = decltype(epi_c)::value;
+        if (!a_mc && !b_mc) return edge ? launch(gemm_pipe32k_kernel<false, false, true, EPI>) : launch(gemm_pipe32k_kernel<false, false, false, EPI>);
+        if (!a_mc && b_mc) return edge ? launch(gemm_pipe32k_kernel<false, true, true, EPI>) : launch(gemm_pipe32k_kernel<false, true, false, EPI>);
+        if (a_mc && !b_mc) return edge ? launch(gemm_pipe32k_kernel<true, false, true, EPI>) : launch(gemm_pipe32k_kernel<true, false, false, EPI>);
+        return edge ? launch(gemm_pipe32k_kernel<true, true, true, EPI>) : launch(gemm_pipe32k_kernel<true, true, false, EPI>);
+    };
+    return (g.bias || g.accumulate) ? pick(std::true_type{}) : pick(std::false_type{});
 }
 
 }  // namespace rp

@@ -146,6 +146,37 @@ def test_16bit_rounding_is_the_references_half_away_from_zero(dt):
     assert got_all[2] == (-258.0 if dt == BF16 else -2050.0)
 
 
+@pytest.mark.parametrize("m,n,k", [(256, 128, 64), (512, 512, 256)])
+def test_fp16_epilogue_rounding_at_the_tile_level(m, n, k):
+    """The fp16 epilogue narrows a tile with two instructions per value when every value of it rounds to a normal fp16
+    number and with the general rule otherwise.  C[i, j] = hi_i + lo_i * s_j is exact in fp32 and sits on, just above
+    or just below a rounding tie of the reference's add-the-first-dropped-bit rule (core/half_precision.h:50-83);
+    rows in the upper half of the output also hold zeros, results below the normal range, sums that overflow, and
+    infinities, so their tiles take the general path.  Either way: the oracle's bits."""
+    rng = np.random.default_rng(37)
+    e = rng.integers(-3, 15, m)
+    hi = (1.0 + rng.integers(0, 1024, m) / 1024.0) * np.exp2(e) * rng.choice([-1.0, 1.0], m)
+    ulp = np.exp2(e - 10.0)
+    frac = rng.choice([0.5, 0.5 * (1 + 2.0 ** -10), 0.5 * (1 - 2.0 ** -10), 0.25, 0.0, 0.75], m)
+    lo = frac * ulp * np.sign(hi) * rng.choice([-1.0, 1.0], m)
+    special = np.arange(m) >= m // 2
+    pick = rng.integers(0, 6, m)
+    hi = np.where(special & (pick == 0), 0.0, hi); lo = np.where(special & (pick == 0), 0.0, lo)                    # exact zero
+    hi = np.where(special & (pick == 1), 2.0 ** -15 * 1.5, hi); lo = np.where(special & (pick == 1), 2.0 ** -24, lo)     # subnormal result
+    hi = np.where(special & (pick == 2), 65504.0, hi); lo = np.where(special & (pick == 2), 16.0, lo)               # 65520: the reference's infinity
+    hi = np.where(special & (pick == 3), np.inf, hi); lo = np.where(special & (pick == 3), 0.0, lo)
+    hi = np.where(special & (pick == 4), 2.0 ** -14, hi); lo = np.where(special & (pick == 4), -(2.0 ** -24), lo)   # just below the smallest normal
+    a64 = np.zeros((m, k)); a64[:, 0] = hi; a64[:, 1] = lo
+    b64 = np.zeros((k, n)); b64[0, :] = 1.0; b64[1, :] = rng.choice([1.0, -1.0, 0.5, 0.0], n)
+    a, b = oracle.to_storage(a64, F16), oracle.to_storage(b64, F16)
+    assert np.array_equal(oracle.to_f64(a, F16)[:, :2], a64[:, :2])                  # the construction is representable
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = oracle_gemm(a, b, F16)
+    got = device_gemm(a, b, F16)
+    assert capi.last_gemm_kernel().startswith("mfma16_")
+    assert np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
 def test_batched_strided_views(dt):
     rng = np.random.default_rng(34)
@@ -500,10 +531,17 @@ def test_fp32_pipelined_kernel(batch, m, k, n, layout):
     assert capi.gemm_kernel_name(batch, m, k, n, a_rc, b_rc, (n, 1), F32) == "pipe32_128x128"
     got = device_gemm(a, b, F32)
     _check(got, a, b, F32, k)
-    # a bias or an accumulated C is not this kernel's: the same call must still be right through the one that takes over
+    assert capi.last_gemm_kernel() == "pipe32_128x128"
+    # the bias per column is this kernel's too
     bias = rand_storage(rng, (n,), F32)
+    got = device_gemm(a, b, F32, bias=bias)
+    assert capi.last_gemm_kernel() == "pipe32_128x128"
+    _check(got, a, b, F32, k, bias=bias)
+    # an accumulated C is not (reading C back leaves the product bound by memory either way): the same call must still be
+    # right through the kernel that takes over
     c0 = rand_storage(rng, (batch, m, n), F32)
     got = device_gemm(a, b, F32, bias=bias, c_init=c0, accumulate=True)
+    assert capi.last_gemm_kernel() != "pipe32_128x128"
     _check(got, a, b, F32, k, bias=bias, c_init=c0, accumulate=True)
 
 
@@ -551,9 +589,15 @@ def test_16bit_pipelined_kernel(batch, m, k, n, dt, layout):
         assert capi.gemm_kernel_name(batch, m, k, n, a_rc, b_rc, (n, 1), dt) == "pipe16_128x128"
     got = device_gemm(a, b, dt)
     _check(got, a, b, dt, k)
+    resident = layout[0] == "n" or m % 8 == 0
     bias = rand_storage(rng, (n,), dt)
+    got = device_gemm(a, b, dt, bias=bias)                                     # the bias per column is this kernel's too
+    if resident:
+        assert capi.last_gemm_kernel() == "pipe16_128x128"
+    _check(got, a, b, dt, k, bias=bias)
     c0 = rand_storage(rng, (batch, m, n), dt)
-    got = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)          # not this kernel's: through the one that takes over
+    got = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)          # accumulation is not: through the one that takes over
+    assert capi.last_gemm_kernel() != "pipe16_128x128"
     _check(got, a, b, dt, k, bias=bias, c_init=c0, accumulate=True)
 
 
@@ -617,10 +661,13 @@ def test_16bit_narrow_output_kernel(batch, m, k, n, dt, layout):
     assert capi.gemm_kernel_name(batch, m, k, n, a_rc, b_rc, (n, 1), dt) == "pipe16k_128x64"
     got = device_gemm(a, b, dt)
     _check(got, a, b, dt, k)
+    # the bias per column and the accumulation into C (the gradient rule of ops/ops.c:6781-6788) are this kernel's too
     bias = rand_storage(rng, (n,), dt)
     c0 = rand_storage(rng, (batch, m, n), dt)
-    got = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)          # not this kernel's: through the one that takes over
-    _check(got, a, b, dt, k, bias=bias, c_init=c0, accumulate=True)
+    for kw in ({"bias": bias}, {"c_init": c0, "accumulate": True}, {"bias": bias, "c_init": c0, "accumulate": True}):
+        got = device_gemm(a, b, dt, **kw)
+        assert capi.last_gemm_kernel() == "pipe16k_128x64", kw.keys()
+        _check(got, a, b, dt, k, **kw)
 
 
 @pytest.mark.parametrize("layout", LAYOUTS)
@@ -649,6 +696,23 @@ def test_16bit_narrow_output_kernel_bit_exact(layout):
         d.free()
     assert np.array_equal(oracle.to_f64(out[:, :, :n], dt), want)
     assert np.array_equal(out[:, :, n:], c0[:, :, n:])
+    # with a bias and an accumulated C every rounding of the reference's three ops is visible (sums up to 1800 need more
+    # than bf16's 8 bits): the oracle's bits, from this kernel and from the tiled one that a misaligned bias falls back to
+    bias = oracle.to_storage(rng.integers(-40, 41, (n + 8,)).astype(np.float64), dt)
+    cacc = oracle.to_storage(rng.integers(-300, 301, (batch, m, n)).astype(np.float64), dt)
+    want_bits = oracle_gemm(a, b, dt, bias=bias[:n], c_init=cacc, accumulate=True)
+    got = device_gemm(a, b, dt, bias=bias[:n], c_init=cacc, accumulate=True)
+    assert capi.last_gemm_kernel() == "pipe16k_128x64"
+    assert np.array_equal(got, want_bits)
+    dbias_all = capi.DeviceBuffer.from_numpy(bias)
+    da, db, dc = capi.DeviceBuffer.from_numpy(a_st), capi.DeviceBuffer.from_numpy(b_st), capi.DeviceBuffer.from_numpy(cacc)
+    capi.gemm(dc.ptr, da.ptr, db.ptr, dbias_all.at(2), batch, m, k, n, a_str, b_str, (m * n, n, 1), True, dt)      # bias at a 2-byte offset
+    capi.synchronize()
+    assert capi.last_gemm_kernel() != "pipe16k_128x64"
+    tiled = dc.to_numpy(capi.NP_STORAGE[dt], (batch, m, n))
+    assert np.array_equal(tiled, oracle_gemm(a, b, dt, bias=bias[1:n + 1], c_init=cacc, accumulate=True))
+    for d in (da, db, dc, dbias_all):
+        d.free()
 
 
 # ---- and its fp32 twin (any n up to 64, any C strides)
@@ -667,10 +731,13 @@ def test_fp32_narrow_output_kernel(batch, m, k, n, layout):
     assert capi.gemm_kernel_name(batch, m, k, n, a_rc, b_rc, (n, 1), F32) == "pipe32k_128x64"
     got = device_gemm(a, b, F32)
     _check(got, a, b, F32, k)
+    # the bias per column and the accumulation into C are this kernel's too
     bias = rand_storage(rng, (n,), F32)
     c0 = rand_storage(rng, (batch, m, n), F32)
-    got = device_gemm(a, b, F32, bias=bias, c_init=c0, accumulate=True)          # not this kernel's: through the one that takes over
-    _check(got, a, b, F32, k, bias=bias, c_init=c0, accumulate=True)
+    for kw in ({"bias": bias}, {"c_init": c0, "accumulate": True}, {"bias": bias, "c_init": c0, "accumulate": True}):
+        got = device_gemm(a, b, F32, **kw)
+        assert capi.last_gemm_kernel() == "pipe32k_128x64", kw.keys()
+        _check(got, a, b, F32, k, **kw)
 
 
 @pytest.mark.parametrize("layout", LAYOUTS)
@@ -696,6 +763,12 @@ def test_fp32_narrow_output_kernel_bit_exact_strided_c(layout):
         d.free()
     assert np.array_equal(out[:, :n, :m], want.transpose(0, 2, 1))
     assert np.array_equal(out[:, n:, :], c0[:, n:, :]) and np.array_equal(out[:, :, m:], c0[:, :, m:])
+    # integers with a bias and an accumulated C: exact in fp32, so the oracle's bits
+    bias = rng.integers(-40, 41, (n,)).astype(np.float32)
+    cacc = rng.integers(-300, 301, (batch, m, n)).astype(np.float32)
+    got = device_gemm(a, b, F32, bias=bias, c_init=cacc, accumulate=True)
+    assert capi.last_gemm_kernel() == "pipe32k_128x64"
+    assert np.array_equal(got, oracle_gemm(a, b, F32, bias=bias, c_init=cacc, accumulate=True))
 
 
 def test_fp32_short_reduction_integers_bit_exact():
