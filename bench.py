@@ -477,12 +477,23 @@ def attention_times(capi, dt_name="bf16"):
             out[name]["TFLOP/s"] = round(flops / ms / 1e9, 1)
             out[name]["frac_mfma"] = round(flops / ms / 1e9 / PEAK_TFLOPS[dt_name], 3)       # these GEMMs sit near the ridge: both fractions are given
             out[name]["kernel"] = gemm_names[name]
-    out["fwd_bwd_ms"] = round(total + out["scale"]["us"] * 1e-3, 4)     # the scale runs twice (S/8 and dS/8)
+    # The scalar multiply and the softmax next to it as one pass each way (rp_hip_scaled_softmax and its gradient: the bits
+    # of the two ops, the scaled tensor neither written nor re-read), which is how the drop-in runs `s.op_mul_scalar(c).op_softmax()`
+    fused_ops = {
+        "scale+softmax": (lambda: capi.check(L.rp_hip_scaled_softmax(d_p.ptr, d_s.ptr, scale, Z * S, S, 1, dt), "scaled_softmax"), 2 * ss * Z * esz),
+        "softmax_bwd+scale": (lambda: capi.check(L.rp_hip_backwards_scaled_softmax(d_dp.ptr, d_p.ptr, d_dss.ptr, scale, Z * S, S, 1, dt), "backwards_scaled_softmax"), 3 * ss * Z * esz),
+    }
+    for name, (fn, nbytes) in fused_ops.items():
+        ms = _time_graph(capi, fn, 10, 2)
+        out[name] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1), "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 3)}
+    out["fwd_bwd_ms_separate_scale"] = round(total + out["scale"]["us"] * 1e-3, 4)     # every reference op its own launch; the scale runs twice (S/8 and dS/8)
+    gemms = sum(out[k]["us"] for k in ("S=Q.Kt", "O=P.V", "dP=dO.Vt", "dV=Pt.dO", "dQ=dS.K", "dK=dSt.Q"))
+    out["fwd_bwd_ms"] = round((gemms + out["scale+softmax"]["us"] + out["softmax_bwd+scale"]["us"]) * 1e-3, 4)
     # the same forward (S, scale, softmax, O) as one fused kernel that never writes S or P
     fused = lambda: capi.check(L.rp_hip_attention_forward(d_o.ptr, d_q.ptr, d_k.ptr, d_v.ptr, None, Z, S, S, D,
                                                           sd, D, sd, D, sd, D, sd, D, 0.125, dt), "rp_hip_attention_forward")
     ms = _time_graph(capi, fused, 10, 2)
-    chain = sum(out[k]["us"] for k in ("S=Q.Kt", "scale", "softmax", "O=P.V"))
+    chain = sum(out[k]["us"] for k in ("S=Q.Kt", "scale+softmax", "O=P.V"))
     nbytes = 4 * sd * Z * esz
     out["fused_forward"] = {"us": round(ms * 1e3, 1), "unfused_chain_us": round(chain, 1), "TFLOP/s": round(4.0 * Z * S * S * D / ms / 1e9, 1),
                             "GB/s": round(nbytes / ms / 1e6, 1)}

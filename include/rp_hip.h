@@ -172,6 +172,21 @@ int log_softmax_kernel_device(void* out, const void* x, size_t outer_size, size_
 /* ops/grad_device.cu:1236-1291 */
 int backwards_softmax_device(const void* grad_c, const void* softmax_out, void* grad_x,
                              size_t outer_size, size_t dim_size, size_t inner_size, int dtype);
+/* softmax(x * scalar) and its gradient in one pass each, with the roundings of the two reference ops they stand for
+ * (mul_scalar_kernel_device then softmax_kernel_device, functional/functional.h:380,404; their gradients in reverse
+ * order): bit for bit what the two launches leave, without writing or re-reading the scaled tensor.  scalar: float*
+ * for every dtype but float64 (double*), as for mul_scalar_kernel_device.  out may not alias x. */
+int rp_hip_scaled_softmax(void* out, const void* x, const void* scalar, size_t outer_size, size_t dim_size, size_t inner_size, int dtype);
+int rp_hip_backwards_scaled_softmax(const void* grad_c, const void* softmax_out, void* grad_x, const void* scalar,
+                                    size_t outer_size, size_t dim_size, size_t inner_size, int dtype);
+/* mul_scalar_kernel_device whose launch may be postponed until the calling thread's next call into this library (any
+ * call: launches, copies, synchronisation, freeing one of the two buffers), which then runs it first, so later work
+ * sees the product as if it had been launched at once.  A host layer that learns, at that next call, that the product
+ * will never be read (an eager API cannot know it earlier) takes the record back with rp_hip_take_deferred(out, &x,
+ * &scalar) (1 and the source and scalar when a multiply into `out` was still pending, 0 otherwise) and passes them
+ * to rp_hip_scaled_softmax instead.  One record per thread.  No counterpart in the reference, whose ops launch at once. */
+int rp_hip_mul_scalar_deferred(void* out, const void* x, const void* scalar, size_t size, int dtype);
+int rp_hip_take_deferred(const void* out, const void** x, double* scalar);
 /* ops/ops.h:260, ops/grad_device.cu:1256-1310 (values of ops/grad_host.c:1428-1500): grad_x = grad_c - exp(y) * sum over
  * the axis of grad_c, with y the output of log_softmax; the gradient of op_log_softmax (ops/ops.c:5693-5719). */
 int backwards_log_softmax_device(const void* grad_c, const void* log_softmax_out, void* grad_x,

@@ -62,6 +62,10 @@ SIGNATURES = {
     "softmax_kernel_device": (_i, [_vp, _vp, _sz, _sz, _sz, _i]),
     "log_softmax_kernel_device": (_i, [_vp, _vp, _sz, _sz, _sz, _i]),
     "backwards_softmax_device": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _i]),
+    "rp_hip_scaled_softmax": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _i]),
+    "rp_hip_backwards_scaled_softmax": (_i, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _i]),
+    "rp_hip_mul_scalar_deferred": (_i, [_vp, _vp, _vp, _sz, _i]),
+    "rp_hip_take_deferred": (_i, [_vp, ctypes.POINTER(_vp), ctypes.POINTER(_d)]),
     "backwards_log_softmax_device": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _i]),
     "contiguous_copy_kernel_device": (_i, [_vp, _vp, _i, _ip, _ip, _sz, _i]),
     "sum_all_kernel_device": (_i, [_vp, _vp, _sz, _i]),

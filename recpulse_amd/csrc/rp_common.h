@@ -20,6 +20,11 @@ int device_cu_count();                                   // compute units of the
 // observed to run on one XCD (one L2).  Measured once per device with a short kernel and a blocking read-back; a
 // first query made while the calling thread's stream records a graph answers false and measures later.
 bool workgroups_share_xcd_by_residue();
+// Launches the calling thread's postponed scalar multiply, if there is one (rp_hip_mul_scalar_deferred).  current_stream()
+// calls it, so every launch and stream-ordered copy is preceded by it; entry points that reach the device without asking
+// for the stream call it themselves.  deferred_touches: the postponed multiply reads or writes a buffer starting at ptr.
+void flush_deferred();
+bool deferred_touches(const void* ptr);
 
 inline size_t dtype_size(int dtype) {                    // reference core/half_precision.h:10-18
     switch (dtype) {

@@ -239,8 +239,10 @@ __global__ void softmax_rows_kernel(T* out, const T* x, size_t rows, size_t dim)
 // Rows that fit a wave's registers (dim <= 64 lanes * CH chunks * 16 bytes, dim a whole number of 16-byte
 // vectors, aligned rows): each lane loads CH 16-byte pieces of the row once, everything else happens in
 // registers, and the result leaves as 16-byte stores.  One wave per row, four rows per block.
+// With has_scale the input is first multiplied by the scalar and rounded to T, which is what a separate scalar multiply
+// in front of the softmax leaves in memory (reference ops/ops.c:6022-6086 then 5721-5788): one pass instead of two, same bits.
 template <typename T, bool LOG, int CH>
-__global__ void __launch_bounds__(kThreads) softmax_rows_reg_kernel(T* out, const T* x, size_t rows, int dim) {
+__global__ void __launch_bounds__(kThreads) softmax_rows_reg_kernel(T* out, const T* x, size_t rows, int dim, bool has_scale, typename traits<T>::acc scale) {
     using A = typename traits<T>::acc;
     constexpr int VEC = 16 / sizeof(T);
     const int lane = threadIdx.x & 63;
@@ -264,7 +266,9 @@ __global__ void __launch_bounds__(kThreads) softmax_rows_reg_kernel(T* out, cons
             memcpy(t, &raw[c], 16);
 #pragma unroll
             for (int e = 0; e < VEC; e++) {
-                v[c][e] = in ? widen(t[e]) : lowest<A>();
+                A xv = widen(t[e]);
+                if (has_scale) xv = widen(narrow<T>(xv * scale));
+                v[c][e] = in ? xv : lowest<A>();
                 mx = v[c][e] > mx ? v[c][e] : mx;
             }
         }
@@ -300,8 +304,10 @@ __global__ void __launch_bounds__(kThreads) softmax_rows_reg_kernel(T* out, cons
     }
 }
 
+// With has_scale the gradient is rounded to T and then multiplied by the scalar and rounded again: the softmax's own
+// gradient followed by that of a scalar multiply in front of it (reference ops/grad_host.c:1387-1398, ops/ops.c:6022-6086).
 template <typename T, int CH>
-__global__ void __launch_bounds__(kThreads) backwards_softmax_rows_reg_kernel(const T* gc, const T* y, T* gx, size_t rows, int dim) {
+__global__ void __launch_bounds__(kThreads) backwards_softmax_rows_reg_kernel(const T* gc, const T* y, T* gx, size_t rows, int dim, bool has_scale, typename traits<T>::acc scale) {
     using A = typename traits<T>::acc;
     constexpr int VEC = 16 / sizeof(T);
     const int lane = threadIdx.x & 63;
@@ -340,7 +346,10 @@ __global__ void __launch_bounds__(kThreads) backwards_softmax_rows_reg_kernel(co
             if (e0 >= dim) continue;
             T o[VEC];
 #pragma unroll
-            for (int e = 0; e < VEC; e++) o[e] = narrow<T>(s[c][e] * (g[c][e] - dot));
+            for (int e = 0; e < VEC; e++) {
+                o[e] = narrow<T>(s[c][e] * (g[c][e] - dot));
+                if (has_scale) o[e] = narrow<T>(widen(o[e]) * scale);
+            }
             u32x4_t w;
             memcpy(&w, o, 16);
             __builtin_nontemporal_store(w, (u32x4_t*)(gx + row0 + e0));
@@ -358,24 +367,24 @@ static int reg_row_chunks(size_t dim, const void* p0, const void* p1, const void
 }
 
 template <typename T, int CH>
-static void launch_softmax_reg_ch(T* out, const T* x, size_t rows, size_t dim, unsigned blocks, bool take_log) {
-    if (take_log) hipLaunchKernelGGL((softmax_rows_reg_kernel<T, true, CH>), dim3(blocks), dim3(kThreads), 0, current_stream(), out, x, rows, (int)dim);
-    else          hipLaunchKernelGGL((softmax_rows_reg_kernel<T, false, CH>), dim3(blocks), dim3(kThreads), 0, current_stream(), out, x, rows, (int)dim);
+static void launch_softmax_reg_ch(T* out, const T* x, size_t rows, size_t dim, unsigned blocks, bool take_log, bool has_scale, typename traits<T>::acc scale) {
+    if (take_log) hipLaunchKernelGGL((softmax_rows_reg_kernel<T, true, CH>), dim3(blocks), dim3(kThreads), 0, current_stream(), out, x, rows, (int)dim, has_scale, scale);
+    else          hipLaunchKernelGGL((softmax_rows_reg_kernel<T, false, CH>), dim3(blocks), dim3(kThreads), 0, current_stream(), out, x, rows, (int)dim, has_scale, scale);
 }
 // launch the register kernel when the rows qualify; false means the caller takes the general one
 template <typename T>
-static bool launch_softmax_reg(T* out, const T* x, size_t rows, size_t dim, unsigned blocks, bool take_log) {
+static bool launch_softmax_reg(T* out, const T* x, size_t rows, size_t dim, unsigned blocks, bool take_log, bool has_scale = false, typename traits<T>::acc scale = 1) {
     switch (reg_row_chunks<T>(dim, out, x, nullptr)) {
-        case 1: launch_softmax_reg_ch<T, 1>(out, x, rows, dim, blocks, take_log); return true;
-        case 2: launch_softmax_reg_ch<T, 2>(out, x, rows, dim, blocks, take_log); return true;
-        case 4: launch_softmax_reg_ch<T, 4>(out, x, rows, dim, blocks, take_log); return true;
-        case 8: launch_softmax_reg_ch<T, 8>(out, x, rows, dim, blocks, take_log); return true;
+        case 1: launch_softmax_reg_ch<T, 1>(out, x, rows, dim, blocks, take_log, has_scale, scale); return true;
+        case 2: launch_softmax_reg_ch<T, 2>(out, x, rows, dim, blocks, take_log, has_scale, scale); return true;
+        case 4: launch_softmax_reg_ch<T, 4>(out, x, rows, dim, blocks, take_log, has_scale, scale); return true;
+        case 8: launch_softmax_reg_ch<T, 8>(out, x, rows, dim, blocks, take_log, has_scale, scale); return true;
         default: return false;
     }
 }
 template <typename T>
-static bool launch_bsoftmax_reg(const T* gc, const T* y, T* gx, size_t rows, size_t dim, unsigned blocks) {
-#define RP_BSOFTMAX_REG(CH) hipLaunchKernelGGL((backwards_softmax_rows_reg_kernel<T, CH>), dim3(blocks), dim3(kThreads), 0, current_stream(), gc, y, gx, rows, (int)dim)
+static bool launch_bsoftmax_reg(const T* gc, const T* y, T* gx, size_t rows, size_t dim, unsigned blocks, bool has_scale = false, typename traits<T>::acc scale = 1) {
+#define RP_BSOFTMAX_REG(CH) hipLaunchKernelGGL((backwards_softmax_rows_reg_kernel<T, CH>), dim3(blocks), dim3(kThreads), 0, current_stream(), gc, y, gx, rows, (int)dim, has_scale, scale)
     switch (reg_row_chunks<T>(dim, gc, y, gx)) {
         case 1: RP_BSOFTMAX_REG(1); return true;
         case 2: RP_BSOFTMAX_REG(2); return true;
@@ -706,6 +715,30 @@ static int convert_from(void* dst, const void* src, int src_dtype, size_t size) 
     return check_launch("convert_kernel") ? 0 : -1;
 }
 
+// ---- a scalar multiply whose launch is postponed -----------------------------------
+// rp_hip_mul_scalar_deferred records the multiply instead of launching it.  Everything the calling thread does next in
+// this library passes flush_deferred() first (current_stream() calls it, so does every entry point that touches the
+// device without asking for the stream), which launches the recorded kernel: later work sees the product exactly as if
+// it had been launched at once.  The one exception is a caller that knows the product will never be read and takes the
+// record back with rp_hip_take_deferred, to hand source and scalar to rp_hip_scaled_softmax: the product is then
+// never written.  One record per thread; recording a second multiply launches the first.
+namespace rp {
+
+struct DeferredScale { bool active; void* out; const void* x; double sd; float sf; size_t size; int dtype; };
+static thread_local DeferredScale g_deferred = {false, nullptr, nullptr, 0.0, 0.f, 0, 0};
+
+void flush_deferred() {
+    if (!g_deferred.active) return;
+    const DeferredScale d = g_deferred;
+    g_deferred.active = false;                          // (the launch below asks for the stream again)
+    const void* scalar = d.dtype == RP_DTYPE_FLOAT64 ? (const void*)&d.sd : (const void*)&d.sf;
+    (void)mul_scalar_kernel_device(d.out, d.x, scalar, d.size, d.dtype);
+}
+
+bool deferred_touches(const void* ptr) { return g_deferred.active && (ptr == g_deferred.out || ptr == g_deferred.x); }
+
+}  // namespace rp
+
 extern "C" {
 
 int add_kernel_device(void* out, const void* x1, const void* x2, size_t size, int dtype) {
@@ -797,6 +830,57 @@ int backwards_softmax_device(const void* grad_c, const void* softmax_out, void* 
                                                    outer_size, dim_size, inner_size));
     }
     return check_launch("backwards_softmax kernel") ? 0 : -1;
+}
+
+int rp_hip_mul_scalar_deferred(void* out, const void* x, const void* scalar, size_t size, int dtype) {
+    RP_REQUIRE(out && x && scalar && size, "rp_hip_mul_scalar_deferred");
+    if (!dtype_size(dtype)) { set_error("rp_hip_mul_scalar_deferred: unsupported dtype %d", dtype); return -1; }
+    flush_deferred();
+    g_deferred.out = out; g_deferred.x = x; g_deferred.size = size; g_deferred.dtype = dtype;
+    if (dtype == RP_DTYPE_FLOAT64) { g_deferred.sd = *(const double*)scalar; g_deferred.sf = (float)g_deferred.sd; }
+    else { g_deferred.sf = *(const float*)scalar; g_deferred.sd = (double)g_deferred.sf; }
+    g_deferred.active = true;
+    return 0;
+}
+
+int rp_hip_take_deferred(const void* out, const void** x, double* scalar) {
+    if (!g_deferred.active || g_deferred.out != out) return 0;
+    if (x) *x = g_deferred.x;
+    if (scalar) *scalar = g_deferred.sd;
+    g_deferred.active = false;
+    return 1;
+}
+
+int rp_hip_scaled_softmax(void* out, const void* x, const void* scalar, size_t outer_size, size_t dim_size, size_t inner_size, int dtype) {
+    RP_REQUIRE(out && x && scalar && outer_size && dim_size && inner_size, "rp_hip_scaled_softmax");
+    if (inner_size == 1) {
+        bool done = false;
+        unsigned blocks = grid_for(outer_size * 64, kThreads, 1u << 16);
+        RP_DISPATCH_DTYPE(dtype, {
+            using A = typename traits<T>::acc;
+            done = launch_softmax_reg<T>((T*)out, (const T*)x, outer_size, dim_size, blocks, false, true, *(const A*)scalar);
+        });
+        if (done) return check_launch("softmax kernel") ? 0 : -1;
+    }
+    // rows the one-pass kernel does not take: the two passes, the product going through `out`
+    if (mul_scalar_kernel_device(out, x, scalar, outer_size * dim_size * inner_size, dtype) != 0) return -1;
+    return softmax_kernel_device(out, out, outer_size, dim_size, inner_size, dtype);
+}
+
+int rp_hip_backwards_scaled_softmax(const void* grad_c, const void* softmax_out, void* grad_x, const void* scalar,
+                                    size_t outer_size, size_t dim_size, size_t inner_size, int dtype) {
+    RP_REQUIRE(grad_c && softmax_out && grad_x && scalar && outer_size && dim_size && inner_size, "rp_hip_backwards_scaled_softmax");
+    if (inner_size == 1) {
+        bool done = false;
+        unsigned blocks = grid_for(outer_size * 64, kThreads, 1u << 16);
+        RP_DISPATCH_DTYPE(dtype, {
+            using A = typename traits<T>::acc;
+            done = launch_bsoftmax_reg<T>((const T*)grad_c, (const T*)softmax_out, (T*)grad_x, outer_size, dim_size, blocks, true, *(const A*)scalar);
+        });
+        if (done) return check_launch("backwards_softmax kernel") ? 0 : -1;
+    }
+    if (backwards_softmax_device(grad_c, softmax_out, grad_x, outer_size, dim_size, inner_size, dtype) != 0) return -1;
+    return mul_scalar_kernel_device(grad_x, grad_x, scalar, outer_size * dim_size * inner_size, dtype);
 }
 
 int backwards_log_softmax_device(const void* grad_c, const void* log_softmax_out, void* grad_x,

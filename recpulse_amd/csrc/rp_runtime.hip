@@ -25,7 +25,7 @@ void set_error(const char* fmt, ...) {
     if (getenv("RP_HIP_VERBOSE")) fprintf(stderr, "rp_hip: %s\n", g_error);
 }
 
-hipStream_t current_stream() { return g_stream; }
+hipStream_t current_stream() { flush_deferred(); return g_stream; }
 
 bool check_hip(hipError_t e, const char* what) {
     if (e == hipSuccess) return true;
@@ -190,6 +190,9 @@ int rp_hip_device_count(int* count) {
 }
 
 int rp_hip_set_device(int device_id) {
+    int cur = -1;
+    if (hipGetDevice(&cur) != hipSuccess) { (void)hipGetLastError(); cur = -1; }
+    if (cur != device_id) flush_deferred();             // a postponed multiply belongs to the device it was recorded on
     return check_hip(hipSetDevice(device_id), "hipSetDevice") ? 0 : -1;
 }
 
@@ -246,6 +249,7 @@ int rp_hip_malloc(void** ptr, size_t bytes) {
 
 int rp_hip_free(void* ptr) {
     if (!ptr) return 0;
+    if (deferred_touches(ptr)) flush_deferred();        // a postponed multiply still uses the block: it runs first, in stream order before any reuse
     Pool& p = pool();
     {
         std::lock_guard<std::mutex> lk(p.mu);
@@ -336,13 +340,14 @@ int rp_hip_memcpy_d2d(void* dst, const void* src, size_t bytes) {
 }
 
 int rp_hip_synchronize(void) {
+    flush_deferred();
     return check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize") ? 0 : -1;
 }
 
 const char* rp_hip_last_error(void) { return g_error; }
 
-int rp_hip_set_stream(void* stream) { g_stream = (hipStream_t)stream; return 0; }
-void* rp_hip_get_stream(void) { return (void*)g_stream; }
+int rp_hip_set_stream(void* stream) { flush_deferred(); g_stream = (hipStream_t)stream; return 0; }      // (a postponed multiply belongs to the stream it was recorded on)
+void* rp_hip_get_stream(void) { flush_deferred(); return (void*)g_stream; }                               // (the caller may launch work of its own on it)
 
 int rp_hip_stream_create(void** stream) {
     if (!stream) { set_error("rp_hip_stream_create: null argument"); return -1; }
@@ -367,6 +372,7 @@ int rp_hip_stream_synchronize(void) {
 int rp_hip_graph_capture_begin(void) {
     if (!g_stream) { set_error("rp_hip_graph_capture_begin: set a created stream first (the null stream cannot be captured)"); return -1; }
     if (g_capture.active) { set_error("rp_hip_graph_capture_begin: this thread is already recording"); return -1; }
+    flush_deferred();                                   // work asked for before the recording stays outside it
     if (!check_hip(hipStreamBeginCapture(g_stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture")) return -1;
     g_capture.active = true;
     g_capture.freed.clear();
@@ -376,6 +382,7 @@ int rp_hip_graph_capture_begin(void) {
 int rp_hip_graph_capture_end(void** graph_exec) {
     if (!graph_exec) { set_error("rp_hip_graph_capture_end: null argument"); return -1; }
     hipGraph_t graph = nullptr;
+    flush_deferred();                                   // and work asked for inside it is part of it
     std::vector<HeldBlock> held;
     held.swap(g_capture.freed);
     g_capture.active = false;

@@ -6,6 +6,7 @@
 // reference (python/tensor_python.c:2294-2297).
 #include <pybind11/numpy.h>
 #include <pybind11/pybind11.h>
+#include <pybind11/eval.h>
 #include <pybind11/stl.h>
 
 #include <cstring>
@@ -122,6 +123,10 @@ std::vector<int> targets_from(const py::object& o) {  // a sequence of ints or a
 
 }  // namespace
 
+// Reference count that `self` shows inside a method called on a temporary (a call result that no name holds), or 0 when
+// a temporary cannot be told from a named object on this interpreter: then nothing is ever treated as one.
+static int g_temporary_refs = 0;
+
 PYBIND11_MODULE(recpulse_cuda, m) {
     m.doc() = "RecPulse tensor module for the matmul path, MI355X device layer underneath";
 
@@ -196,7 +201,14 @@ PYBIND11_MODULE(recpulse_cuda, m) {
              py::arg("k"), py::arg("v"), py::arg("scale"))
         .def("op_add", [](PyTensor& a, PyTensor& b) { return wrap(op_add(a.t, b.t), "op_add"); })
         .def("op_relu", [](PyTensor& a) { return wrap(op_relu(a.t), "op_relu"); })
-        .def("op_softmax", [](PyTensor& a, int dim) { return wrap(op_softmax(a.t, dim), "op_softmax"); }, py::arg("dim") = -1)
+        // `x.op_mul_scalar(s).op_softmax()`: the scaled tensor is a temporary that nothing can read once this call has
+        // returned, which its reference count shows (g_temporary_refs, measured when the module is loaded)
+        .def("op_softmax", [](py::object self, int dim) {
+            PyTensor& a = self.cast<PyTensor&>();
+            const bool temporary = g_temporary_refs > 0 && (int)self.ref_count() <= g_temporary_refs;
+            return wrap(temporary ? op_softmax_consume(a.t, dim) : op_softmax(a.t, dim), "op_softmax");
+        }, py::arg("dim") = -1)
+        .def("_refs", [](py::object self, int) { return (int)self.ref_count(); }, py::arg("dim") = -1)      // the same argument shape as op_softmax: its count is the yardstick
         .def("op_log_softmax", [](PyTensor& a, int dim) { return wrap(op_log_softmax(a.t, dim), "op_log_softmax"); }, py::arg("dim") = -1)
         .def("op_mul_scalar", [](PyTensor& a, double s) { return wrap(op_mul_scalar(a.t, s), "op_mul_scalar"); })
         .def("op_sum_all", [](PyTensor& a) { return wrap(op_sum_all(a.t), "op_sum_all"); })
@@ -296,5 +308,13 @@ PYBIND11_MODULE(recpulse_cuda, m) {
     }, py::arg("shape"), py::arg("dtype") = "float32", py::arg("device") = "cpu");
     m.def("_fail_gemm_after", [](int n) { rp_debug_fail_gemm_after(n); }, py::arg("n"));      // fault injection for tests of the error paths
     m.def("manual_seed", [](unsigned long long seed) { rp_manual_seed(seed); });
+    // how a temporary looks to a method on this interpreter: call the yardstick on one, and on a named object
+    try {
+        py::dict scope;
+        scope["T"] = m.attr("zeros");
+        py::exec("named = T([1])\nn = named._refs()\nt = T([1]).copy()._refs()\nn2 = named.copy().copy()._refs()", py::globals(), scope);
+        const int n = scope["n"].cast<int>(), t = scope["t"].cast<int>(), t2 = scope["n2"].cast<int>();
+        if (t == t2 && t < n) g_temporary_refs = t;
+    } catch (py::error_already_set& e) { g_temporary_refs = 0; }
     m.def("device_count", []() { int n = 0; for (int i = 0; i < 64 && validate_device_id(i); i++) n = i + 1; return n; });
 }

@@ -791,6 +791,9 @@ void split_dims(const Tensor* x, int dim, size_t* outer, size_t* d, size_t* inne
     *d = x->shape[dim];
 }
 
+void backward_mul_scalar_fn(GradFn* self, Tensor* grad_output);
+double scalar_of(GradFn* mul_scalar_fn);
+
 void backward_softmax_fn(GradFn* self, Tensor* grad_output) {        // reference ops/ops.c:5665-5719; y is the op's own output
     Tensor* x = self->inputs[0];
     if (!needs_grad(x)) return;
@@ -799,6 +802,20 @@ void backward_softmax_fn(GradFn* self, Tensor* grad_output) {        // referenc
     size_t outer, d, inner;
     split_dims(y, dim, &outer, &d, &inner);
     Tensor* gd = dense(grad_output);
+    // x = source * scalar that nothing but this node refers to (no other consumer, no Python object): its gradient is of
+    // no use to anyone, so the source gets its own directly, rounded twice like the two reference ops, in one pass
+    GradFn* xf = x->metadata->grad_fn;
+    if (xf && xf->backward == backward_mul_scalar_fn && x->refcount == 1 && !x->metadata->grad && !x->metadata->is_leaf && needs_grad(xf->inputs[0])) {
+        Tensor* src = xf->inputs[0];
+        const double sd = scalar_of(xf);
+        const float sf = (float)sd;
+        Tensor* g = empty_tensor(src->dtype, src->device_id, src->ndim, src->shape);
+        if (g && gd && on_device(x->device_id) &&
+            rp_hip_backwards_scaled_softmax(gd->data, y->data, g->data, x->dtype == DTYPE_FLOAT64 ? (const void*)&sd : (const void*)&sf, outer, d, inner, x->dtype) == 0) accumulate_grad(src, g);
+        else { dev_fail("softmax backward"); free_tensor(g); }
+        free_tensor(gd);
+        return;
+    }
     Tensor* g = empty_tensor(x->dtype, x->device_id, x->ndim, x->shape);
     if (g && gd && on_device(x->device_id) && backwards_softmax_device(gd->data, y->data, g->data, outer, d, inner, x->dtype) == 0) accumulate_grad(x, g);
     else { dev_fail("softmax backward"); free_tensor(g); }
@@ -820,6 +837,7 @@ void backward_log_softmax_fn(GradFn* self, Tensor* grad_output) {    // referenc
 }
 
 struct ScalarSaved { double s; };
+double scalar_of(GradFn* mul_scalar_fn) { return ((ScalarSaved*)mul_scalar_fn->saved_data)->s; }
 
 void backward_mul_scalar_fn(GradFn* self, Tensor* grad_output) {     // reference ops/ops.c:5966-6020
     Tensor* x = self->inputs[0];
@@ -1389,7 +1407,7 @@ Tensor* op_relu(Tensor* x) {                           // reference ops/ops.c:23
     return out;
 }
 
-static Tensor* softmax_any(Tensor* x, int dim, bool take_log) {
+static Tensor* softmax_any(Tensor* x, int dim, bool take_log, bool input_dead = false) {
     if (!x) return nullptr;
     if (dim < 0) dim += x->ndim;
     if (dim < 0 || dim >= x->ndim) { fail("softmax: dimension out of range"); return nullptr; }
@@ -1398,8 +1416,17 @@ static Tensor* softmax_any(Tensor* x, int dim, bool take_log) {
     Tensor* out = xd ? empty_tensor(x->dtype, x->device_id, x->ndim, x->shape) : nullptr;
     size_t outer, d, inner;
     split_dims(x, dim, &outer, &d, &inner);
-    int rc = (out && on_device(x->device_id)) ? (take_log ? log_softmax_kernel_device(out->data, xd->data, outer, d, inner, x->dtype)
-                                                          : softmax_kernel_device(out->data, xd->data, outer, d, inner, x->dtype)) : -1;
+    int rc = -1;
+    const void* src = nullptr;
+    double sd = 1.0;
+    if (out && !take_log && input_dead && xd == x && rp_hip_take_deferred(x->data, &src, &sd) == 1) {
+        // x is a scalar multiple whose kernel has not been launched and whose values nobody will read: it never is
+        const float sf = (float)sd;
+        rc = on_device(x->device_id) ? rp_hip_scaled_softmax(out->data, src, x->dtype == DTYPE_FLOAT64 ? (const void*)&sd : (const void*)&sf, outer, d, inner, x->dtype) : -1;
+    } else if (out && on_device(x->device_id)) {
+        rc = take_log ? log_softmax_kernel_device(out->data, xd->data, outer, d, inner, x->dtype)
+                      : softmax_kernel_device(out->data, xd->data, outer, d, inner, x->dtype);
+    }
     free_tensor(xd);
     if (rc != 0) { dev_fail("softmax"); free_tensor(out); return nullptr; }
     if (needs_grad(x)) {
@@ -1412,6 +1439,7 @@ static Tensor* softmax_any(Tensor* x, int dim, bool take_log) {
 }
 
 Tensor* op_softmax(Tensor* x, int dim) { return softmax_any(x, dim, false); }            // reference ops/ops.c:5721-5788
+Tensor* op_softmax_consume(Tensor* x, int dim) { return softmax_any(x, dim, false, true); }
 Tensor* op_log_softmax(Tensor* x, int dim) { return softmax_any(x, dim, true); }
 
 Tensor* op_mul_scalar(Tensor* x, double scalar) {      // reference ops/ops.c:6022-6086
@@ -1419,7 +1447,12 @@ Tensor* op_mul_scalar(Tensor* x, double scalar) {      // reference ops/ops.c:60
     Tensor* xd = dense(x);
     Tensor* out = xd ? empty_tensor(x->dtype, x->device_id, x->ndim, x->shape) : nullptr;
     float sf = (float)scalar;                           // scalars are narrowed to float for every dtype but float64 (reference python/tensor_python.c:475-485)
-    int rc = out ? rp_mul_scalar(out->data, xd->data, x->dtype == DTYPE_FLOAT64 ? (const void*)&scalar : (const void*)&sf, x->size, x->dtype, x->device_id) : -1;
+    const void* sp = x->dtype == DTYPE_FLOAT64 ? (const void*)&scalar : (const void*)&sf;
+    int rc = -1;
+    // On the device the launch is left to the library's next call from this thread (which runs it first, whatever that
+    // call is): if that call turns out to be a softmax whose caller lets the product die, the product is never written.
+    if (out && x->device_id >= 0) rc = on_device(x->device_id) ? (rp_hip_mul_scalar_deferred(out->data, xd->data, sp, x->size, x->dtype) == 0 ? 0 : dev_fail("mul_scalar")) : dev_fail("set device");
+    else if (out) rc = rp_mul_scalar(out->data, xd->data, sp, x->size, x->dtype, x->device_id);
     free_tensor(xd);
     if (rc != 0) { free_tensor(out); return nullptr; }
     if (needs_grad(x)) {

@@ -108,6 +108,8 @@ Tensor* op_attention(Tensor* q, Tensor* k, Tensor* v, double scale);   /* softma
 Tensor* op_add(Tensor* x1, Tensor* x2);
 Tensor* op_relu(Tensor* x);
 Tensor* op_softmax(Tensor* x, int dim);
+Tensor* op_softmax_consume(Tensor* x, int dim);   /* op_softmax for a caller that states nothing will read x's values after this call (the binding: x is a temporary);
+                                                     an x that is a still-unlaunched op_mul_scalar result is then never written: softmax(scale * source) in one pass */
 Tensor* op_log_softmax(Tensor* x, int dim);
 Tensor* op_mul_scalar(Tensor* x, double scalar);
 Tensor* op_sum_all(Tensor* x);

@@ -468,3 +468,43 @@ def test_log_softmax_backward(dtype, tol):
         (torch.log_softmax(tx, dim) * torch.tensor(host(wt).reshape(x.shape))).sum().backward()
         np.testing.assert_allclose(host(y), torch.log_softmax(tx, dim).detach().numpy(), rtol=tol * 5, atol=tol * 5)
         assert oracle.rel_err(host(xt.grad), tx.grad.numpy()) <= tol * 10, dim
+
+
+# ---- `x.op_mul_scalar(s).op_softmax()`: the scaled tensor is a temporary; forward and backward each run one pass less
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_scaled_softmax_chain_with_and_without_a_held_intermediate(dtype):
+    """The chained form never writes the scaled scores (its scalar multiply is still unlaunched when the softmax consumes
+    it) and its backward hands the scores their gradient in one pass; with the intermediate held in a variable both stay
+    two ops (reference ops/ops.c:6022-6086, 5721-5788).  Same bits either way, forward and backward, and the held
+    intermediate reads back as the product."""
+    rng = np.random.default_rng(33)
+    s0 = rng.normal(0, 2, (6, 40, 64))
+    up = rng.normal(0, 1, (6, 40, 64))
+
+    def run(chained):
+        s = dev(s0, dtype, grad=True)
+        w = dev(up, dtype)
+        if chained:
+            p = s.op_mul_scalar(0.125).op_softmax()
+            held = None
+        else:
+            held = s.op_mul_scalar(0.125)
+            p = held.op_softmax()
+        loss = p.op_matmul(w.transpose(1, 2)).op_sum_all()
+        loss.backward()
+        return host(p), host(s.grad), (host(held) if held is not None else None)
+
+    p1, g1, _ = run(True)
+    p2, g2, held = run(False)
+    assert np.array_equal(p1, p2) and np.array_equal(g1, g2)
+    assert np.array_equal(held, host(dev(s0, dtype).op_mul_scalar(0.125)))
+    code = {"float32": oracle.F32, "bfloat16": oracle.BF16}[dtype]
+    scaled = oracle.mul_scalar(oracle.to_storage(s0, code), 0.125, code)
+    assert np.array_equal(held, oracle.to_f64(scaled, code))
+    want = oracle.to_f64(oracle.softmax(scaled, code), code)
+    assert oracle.rel_err(p1, want) <= (2e-6 if dtype == "float32" else 1.6e-2)
+    # a temporary that other work touches before the softmax is materialised like any other tensor
+    s = dev(s0, dtype)
+    t = s.op_mul_scalar(0.125)
+    u = t.op_relu()
+    assert np.array_equal(host(u), np.maximum(host(t), 0.0))

@@ -353,3 +353,75 @@ def test_narrowing_to_fp16_every_exponent_and_rounding_case():
     got, want, w = got[~nan], want[~nan], w[~nan]
     bad = np.nonzero(got != want)[0]
     assert bad.size == 0, [(hex(int(w[i])), hex(int(got[i])), hex(int(want[i]))) for i in bad[:8]]
+
+
+# ---- softmax(x * scalar) and its gradient in one pass; a scalar multiply whose launch is postponed
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_scaled_softmax_is_the_two_ops_bit_for_bit(dt):
+    """rp_hip_scaled_softmax / rp_hip_backwards_scaled_softmax against mul_scalar_kernel_device + softmax_kernel_device and
+    backwards_softmax_device + mul_scalar_kernel_device (reference ops/ops.c:6022-6086, 5721-5788, grad_host.c:1387-1398):
+    rows the one-pass kernels take (whole 16-byte vectors, up to 4096 elements) and rows they hand to the two launches."""
+    rng = np.random.default_rng(47)
+    for shape, dim in (((33, 512), -1), ((5, 1024), -1), ((7, 64), -1), ((3, 2040), -1), ((9, 10), -1), ((3, 17, 5), 1), ((2, 4104), -1)):
+        x = rand_storage(rng, shape, dt, dist="normal")
+        g = rand_storage(rng, shape, dt)
+        d = dim % len(shape)
+        outer = int(np.prod(shape[:d])); n = shape[d]; inner = int(np.prod(shape[d + 1:]))
+        for scalar in (0.125, 1.0 / 3.0):
+            dx, dg = Dev(x, dt), Dev(g, dt)
+            t, y, y1, gt, g2, g1 = (Dev.empty(shape, dt) for _ in range(6))
+            capi.check(L().mul_scalar_kernel_device(t.ptr, dx.ptr, scalar_arg(scalar, dt), x.size, dt), "mul_scalar")
+            capi.check(L().softmax_kernel_device(y.ptr, t.ptr, outer, n, inner, dt), "softmax")
+            capi.check(L().rp_hip_scaled_softmax(y1.ptr, dx.ptr, scalar_arg(scalar, dt), outer, n, inner, dt), "scaled_softmax")
+            assert np.array_equal(y.numpy(), y1.numpy()), (shape, scalar)
+            capi.check(L().backwards_softmax_device(dg.ptr, y.ptr, gt.ptr, outer, n, inner, dt), "backwards_softmax")
+            capi.check(L().mul_scalar_kernel_device(g2.ptr, gt.ptr, scalar_arg(scalar, dt), x.size, dt), "mul_scalar")
+            capi.check(L().rp_hip_backwards_scaled_softmax(dg.ptr, y.ptr, g1.ptr, scalar_arg(scalar, dt), outer, n, inner, dt), "backwards_scaled_softmax")
+            assert np.array_equal(g2.numpy(), g1.numpy()), (shape, scalar)
+
+
+@pytest.mark.parametrize("dt", [BF16, F32], ids=lambda d: NAMES[d])
+def test_postponed_scalar_multiply_runs_before_whatever_follows(dt):
+    """rp_hip_mul_scalar_deferred leaves its launch to the thread's next call into the library.  Whatever that call is
+    (a copy to the host, another kernel reading the product, freeing the source, a second postponed multiply, a
+    synchronisation) the product is there as if launched at once; only rp_hip_take_deferred keeps it from being written."""
+    rng = np.random.default_rng(48)
+    n = 4096
+    x = rand_storage(rng, (n,), dt)
+    want = oracle.mul_scalar(x, 0.125, dt)
+    sentinel = rand_storage(rng, (n,), dt)
+
+    def fresh():
+        return Dev(x, dt), Dev(sentinel, dt)
+
+    # a copy to the host
+    dx, do = fresh()
+    capi.check(L().rp_hip_mul_scalar_deferred(do.ptr, dx.ptr, scalar_arg(0.125, dt), n, dt), "deferred")
+    assert np.array_equal(do.buf.to_numpy(capi.NP_STORAGE[dt], (n,)), want)
+    # a kernel that reads the product
+    dx, do = fresh()
+    d2 = Dev.empty((n,), dt)
+    capi.check(L().rp_hip_mul_scalar_deferred(do.ptr, dx.ptr, scalar_arg(0.125, dt), n, dt), "deferred")
+    capi.check(L().relu_kernel_device(d2.ptr, do.ptr, n, dt), "relu")
+    assert np.array_equal(d2.numpy(), oracle.relu(want, dt))
+    # freeing the source
+    dx, do = fresh()
+    capi.check(L().rp_hip_mul_scalar_deferred(do.ptr, dx.ptr, scalar_arg(0.125, dt), n, dt), "deferred")
+    dx.buf.free()
+    assert np.array_equal(do.numpy(), want)
+    # a second postponed multiply, then a synchronisation
+    dx, do = fresh()
+    do2 = Dev(sentinel, dt)
+    capi.check(L().rp_hip_mul_scalar_deferred(do.ptr, dx.ptr, scalar_arg(0.125, dt), n, dt), "deferred")
+    capi.check(L().rp_hip_mul_scalar_deferred(do2.ptr, dx.ptr, scalar_arg(2.0, dt), n, dt), "deferred")
+    capi.synchronize()
+    assert np.array_equal(do.numpy(), want) and np.array_equal(do2.numpy(), oracle.mul_scalar(x, 2.0, dt))
+    # taken back: never written, and the source and scalar come back for the one-pass softmax
+    dx, do = fresh()
+    capi.check(L().rp_hip_mul_scalar_deferred(do.ptr, dx.ptr, scalar_arg(0.125, dt), n, dt), "deferred")
+    src, s = ctypes.c_void_p(), ctypes.c_double()
+    assert L().rp_hip_take_deferred(do.ptr, ctypes.byref(src), ctypes.byref(s)) == 1
+    assert src.value == dx.ptr and s.value == 0.125
+    assert L().rp_hip_take_deferred(do.ptr, ctypes.byref(src), ctypes.byref(s)) == 0
+    capi.synchronize()
+    assert np.array_equal(do.numpy(), sentinel)
