@@ -22,8 +22,15 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-u
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
+def _flags_stamp(extra):
+    """The compile line an object was built with, kept beside the objects: a change of flags rebuilds everything."""
+    import hashlib
+    return hashlib.sha256(" ".join([HIPCC] + FLAGS + list(extra)).encode()).hexdigest()
+
+
 def _fresh(obj, src):
-    """True when obj is newer than its source and every header under csrc/ and include/."""
+    """True when obj is newer than its source and every header under csrc/ and include/ (and the flags have not changed:
+    build() clears the objects when they have).  Sources that include other .hip files are not tracked: none does."""
     if not os.path.exists(obj):
         return False
     t = os.path.getmtime(obj)
@@ -34,7 +41,7 @@ def _fresh(obj, src):
 
 def _compile(src, extra, force=True):
     obj = os.path.join(BUILD_DIR, src.replace(".hip", ".o"))
-    if not force and not extra and _fresh(obj, src):
+    if not force and _fresh(obj, src):
         return obj
     cmd = [HIPCC] + FLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -52,6 +59,12 @@ def build(extra_flags=(), verbose=True, force=True):
     os.makedirs(LIB_DIR, exist_ok=True)
     os.makedirs(BUILD_DIR, exist_ok=True)
     extra = list(extra_flags)
+    stamp_path = os.path.join(BUILD_DIR, "flags.sha256")
+    stamp = _flags_stamp(extra)
+    if not force and (not os.path.exists(stamp_path) or open(stamp_path).read().strip() != stamp):
+        force = True                                  # objects of another compile line
+    with open(stamp_path, "w") as f:
+        f.write(stamp + "\n")
     with ThreadPoolExecutor(max_workers=8) as ex:
         objs = list(ex.map(lambda s: _compile(s, extra, force), SOURCES))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
@@ -67,16 +80,18 @@ HOST_DIR = os.path.join(HERE, "host")
 DROPIN_DIR = os.path.join(HERE, "dropin")
 
 
-def build_host(verbose=True):
+def build_host(verbose=True, test_hooks=True):
     """Build the CPython extension `recpulse_cuda` (host tensor / autograd layer + pybind11 binding) into
-    recpulse_amd/dropin/, linked against lib/librp_hip.so.  Plain g++: the host layer includes no HIP header."""
+    recpulse_amd/dropin/, linked against lib/librp_hip.so.  Plain g++: the host layer includes no HIP header.
+    test_hooks compiles the fault-injection entry the error-path tests use (`_fail_gemm_after`); a build for
+    deployment passes False and the symbol does not exist."""
     import sysconfig
     import pybind11
     os.makedirs(DROPIN_DIR, exist_ok=True)
     ext = sysconfig.get_config_var("EXT_SUFFIX")
     out = os.path.join(DROPIN_DIR, "recpulse_cuda" + ext)
-    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall",
-           "-I" + pybind11.get_include(), "-I" + sysconfig.get_paths()["include"],
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall"] + (["-DRP_TEST_HOOKS"] if test_hooks else []) + [
+           "-ffp-contract=off", "-I" + pybind11.get_include(), "-I" + sysconfig.get_paths()["include"],
            os.path.join(HOST_DIR, "rp_host.cpp"), os.path.join(HOST_DIR, "py_module.cpp"),
            "-o", out, "-L" + LIB_DIR, "-lrp_hip", "-Wl,-rpath,$ORIGIN/../lib"]
     res = subprocess.run(cmd, capture_output=True, text=True)

@@ -16,6 +16,9 @@ bool check_hip(hipError_t e, const char* what);          // false (and error tex
 bool check_launch(const char* what);                     // hipGetLastError after a launch
 bool stream_is_capturing();                              // the calling thread's stream is recording a graph
 int device_cu_count();                                   // compute units of the current device (0 when it cannot be read)
+// Kernel families can be switched off for cross-checks and same-machine comparisons: RP_HIP_DISABLE holds a comma-separated
+// list of names (read once per process).  The dispatcher then takes what it would take if that kernel did not exist.
+bool path_disabled(const char* name);
 // True when, on the current device, workgroups of a one-dimensional grid whose linear ids are equal modulo 8 were
 // observed to run on one XCD (one L2).  Measured once per device with a short kernel and a blocking read-back; a
 // first query made while the calling thread's stream records a graph answers false and measures later.

@@ -131,7 +131,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t splitk_rsrc(const float* parti
 
 // The device's block of SPLITK_MAX_TILES zeroed arrival counters (created on first use, kept for the life of the
 // process), or nullptr when the single-launch finish cannot be used: more tiles than counters, partials of 2 GiB
-// or more, RP_HIP_SPLITK_TWO_LAUNCH=1, or an allocation failure (then last_error is set and *failed is true).
+// or more, "one_launch_splitk" in RP_HIP_DISABLE, or an allocation failure (then last_error is set and *failed is true).
 // Like the workspace pool the block is not stream-aware: launches that may run at the same time on different
 // streams of one device must be serialised by the caller.
 int* splitk_arrival_counters(long long tiles, size_t partial_bytes, bool* failed);

@@ -29,28 +29,14 @@ namespace rp {
 // ============================================================================
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
-static bool force_generic() {
-    static int v = -1;
-    if (v < 0) { const char* e = getenv("RP_HIP_FORCE_GENERIC"); v = (e && e[0] == '1') ? 1 : 0; }
-    return v == 1;
-}
+// rows up to which a deep 16-bit GEMM with few output tiles splits k
+constexpr int SKINNY_MAX_ROWS = 128;
 
-static bool tiny_off() {                           // RP_HIP_NO_TINY=1: small fp32 GEMMs take the tiled kernels with a k split instead
-    static int v = -1;
-    if (v < 0) { const char* e = getenv("RP_HIP_NO_TINY"); v = (e && e[0] == '1') ? 1 : 0; }
-    return v == 1;
-}
-
-static bool wide64() {                             // RP_HIP_NO_64X256=1: outputs of at most 64 rows keep the square tiles
-    static int v = -1;
-    if (v < 0) { const char* e = getenv("RP_HIP_NO_64X256"); v = (e && e[0] == '1') ? 0 : 1; }
-    return v == 1;
-}
-
-static int skinny_max_rows() {                     // RP_HIP_SKINNY_MAX_M: rows up to which a deep 16-bit GEMM with few output tiles splits k
-    static int v = -1;
-    if (v < 0) { const char* e = getenv("RP_HIP_SKINNY_MAX_M"); v = e ? atoi(e) : 128; if (v < 32) v = 32; }
-    return v;
+// Tile counts that decide between kernels stand for "one tile per CU" and "half of the CUs": they follow the device
+// (whole rounds of the 8 XCDs, as the launchers size their grids); 256 where no device can be asked.
+static int cu_tiles() {
+    const int n = device_cu_count() / 8 * 8;
+    return n >= 8 ? n : 256;
 }
 
 // Tile of the 16-bit MFMA kernel for an output of batch x m x n with reduction length k.
@@ -60,55 +46,25 @@ static void choose_tile16(Plan& p, int batch, int m, int k, int n) {
     const long long tiles128 = (long long)((m + 127) / 128) * ((n + 127) / 128) * batch;
     // the 256 x 256 tile runs one block per CU, so it needs a k loop long enough to hide its prologue and
     // epilogue; with fewer than four slabs the smaller tile (two blocks per CU) overlaps them instead
-    if (m >= 256 && n >= 256 && tiles256 >= 128 && k >= 4 * M16_BK) { p.bm = 256; p.bn = 256; p.name = "mfma16_256x256"; }
+    if (m >= 256 && n >= 256 && tiles256 >= cu_tiles() / 2 && k >= 4 * M16_BK) { p.bm = 256; p.bn = 256; p.name = "mfma16_256x256"; }
     // fewer than 128 tiles of 128 x 128 would leave over half the CUs idle: the 64 x 64 tile quadruples the workgroups
     // (1024^3: 10.9 -> 7.3 us)
     // at most 64 rows: a 64 x 256 tile (the same 64 x 64 patch per wave as the 128 x 128 tile, none of it past the last row)
     // (64 x 128 while k is short: two blocks share a CU and one's loads and stores overlap the other's few slabs)
-    else if (m <= 64 && n >= 256 && wide64() && (long long)((n + 255) / 256) * batch >= 128) {
+    else if (m <= 64 && n >= 256 && !path_disabled("wide64") && (long long)((n + 255) / 256) * batch >= cu_tiles() / 2) {
         p.bm = 64; p.bn = k <= 1024 ? 128 : 256; p.name = k <= 1024 ? "mfma16_64x128" : "mfma16_64x256";
     }
-    else if ((m > 64 || n > 64) && tiles128 >= 128) { p.bm = 128; p.bn = 128; p.name = "mfma16_128x128"; }
+    else if ((m > 64 || n > 64) && tiles128 >= cu_tiles() / 2) { p.bm = 128; p.bn = 128; p.name = "mfma16_128x128"; }
     else { p.bm = 64; p.bn = 64; p.name = "mfma16_64x64"; }
     p.edge = (m % p.bm) || (n % p.bn) || (k % M16_BK);
 }
 
 // Decide the kernel family and tile from shapes and strides alone (pointer
 // alignment is checked by the caller, which may still fall back to generic).
-static bool direct32_off() {                       // RP_HIP_NO_DIRECT32=1: short-k fp32 GEMMs keep the LDS-tiled kernel
-    static int v = -1;
-    if (v < 0) { const char* e = getenv("RP_HIP_NO_DIRECT32"); v = (e && e[0] == '1') ? 1 : 0; }
-    return v == 1;
-}
-
-static bool pipe32_off() {                       // RP_HIP_NO_PIPE32=1: k-contiguous short-k fp32 GEMMs keep the kernel that stages through registers
-    static int v = -1;
-    if (v < 0) { const char* e = getenv("RP_HIP_NO_PIPE32"); v = (e && e[0] == '1') ? 1 : 0; }
-    return v == 1;
-}
-
-static bool pipe16_off() {                       // RP_HIP_NO_PIPE16=1: the same for the 16-bit kernel
-    static int v = -1;
-    if (v < 0) { const char* e = getenv("RP_HIP_NO_PIPE16"); v = (e && e[0] == '1') ? 1 : 0; }
-    return v == 1;
-}
-
-static bool pipe16k_off() {                        // RP_HIP_NO_PIPE16K=1: narrow 16-bit outputs keep the general tiled kernel
-    static int v = -1;
-    if (v < 0) { const char* e = getenv("RP_HIP_NO_PIPE16K"); v = (e && e[0] == '1') ? 1 : 0; }
-    return v == 1;
-}
-
-static bool pipe32k_off() {                        // RP_HIP_NO_PIPE32K=1: narrow fp32 outputs keep the general tiled kernel
-    static int v = -1;
-    if (v < 0) { const char* e = getenv("RP_HIP_NO_PIPE32K"); v = (e && e[0] == '1') ? 1 : 0; }
-    return v == 1;
-}
-
 static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long a_cs, long long b_rs, long long b_cs,
                       long long c_rs, long long c_cs, long long a_bs, long long b_bs, int dtype, bool allow_direct = true) {
     Plan p{FAM_GENERIC, 64, 64, false, false, true, "generic"};
-    if (force_generic()) return p;
+    if (path_disabled("mfma")) return p;
     const int vec = 16 / (int)dtype_size(dtype);                // elements per 16-byte vector
     // operand layouts: KC = unit stride along k, MC = unit stride along the free axis.
     // Extent-1 axes make the other stride irrelevant, but vector loads still need alignment of the non-unit stride.
@@ -125,11 +81,11 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     const bool is16 = dtype == RP_DTYPE_FLOAT16 || dtype == RP_DTYPE_BFLOAT16;
 
     // 16-bit, few rows, deep k: split k over many blocks so that B streams at HBM speed (output columns in whole 8s).
-    // Up to 32 rows always; up to skinny_max_rows() when the 128 x 128 tiles of the output would occupy under half the
+    // Up to 32 rows always; up to SKINNY_MAX_ROWS when the 128 x 128 tiles of the output would occupy under half the
     // CUs and k is deep enough to be worth a second launch for the partial sums (64 x 1024 x 4096: 6.6 us on 64 x 64 tiles
     // in one launch against 9.4 us split; 64 x 4096 x 1024: 16.4 against 9.1).
     const long long tiles128_16 = (long long)((m + 127) / 128) * ((n + 127) / 128);
-    if (is16 && mfma_ok && batch == 1 && (m <= 32 || (m <= skinny_max_rows() && tiles128_16 < 128 && k >= 2048)) && n % 8 == 0 && n >= 256 && k >= 1024 &&
+    if (is16 && mfma_ok && batch == 1 && (m <= 32 || (m <= SKINNY_MAX_ROWS && tiles128_16 < cu_tiles() / 2 && k >= 2048)) && n % 8 == 0 && n >= 256 && k >= 1024 &&
         (long long)k * n >= (1ll << 22)) {
         p.fam = FAM_MFMA16_SKINNY; p.bm = 32; p.bn = 128; p.edge = true; p.a_mc = !a_kc; p.b_mc = b_mc;
         p.name = (!p.a_mc && p.b_mc && m <= 16) ? "mfma16_stream_32x256" : "mfma16_skinny_32x128";
@@ -144,15 +100,15 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     }
     // fp32, an output of fewer than 64 tiles of 64 x 64 and a k that one workgroup walks in a few microseconds: one launch
     // of 16 x 16 tiles with k split over the four waves of a workgroup, any strides (no split over workgroups, no second launch)
-    if (dtype == RP_DTYPE_FLOAT32 && k <= 2048 && (long long)((m + 63) / 64) * ((n + 63) / 64) * batch < 64 && !tiny_off()) {
+    if (dtype == RP_DTYPE_FLOAT32 && k <= 2048 && (long long)((m + 63) / 64) * ((n + 63) / 64) * batch < 64 && !path_disabled("tiny")) {
         p.fam = FAM_TINY; p.bm = 16; p.bn = 16; p.name = "tiny32_16x16";
         return p;
     }
     // fp32 with k <= 64, any operand layout with a unit stride and at least one 128 x 128 tile per CU: one resident workgroup per
     // CU whose fetching waves fill LDS directly and whose multiplying waves store the previous tile between the MFMAs
-    if (dtype == RP_DTYPE_FLOAT32 && allow_direct && !pipe32_off() && k <= 64 && k % 4 == 0 && ((a_cs == 1 && a_rs % 4 == 0) || (a_rs == 1 && a_cs % 4 == 0)) &&
+    if (dtype == RP_DTYPE_FLOAT32 && allow_direct && !path_disabled("pipe32") && k <= 64 && k % 4 == 0 && ((a_cs == 1 && a_rs % 4 == 0) || (a_rs == 1 && a_cs % 4 == 0)) &&
         ((b_rs == 1 && b_cs % 4 == 0) || (b_cs == 1 && b_rs % 4 == 0)) &&
-        batch_ok && m > 64 && n > 64 && (long long)((m + 127) / 128) * ((n + 127) / 128) * batch >= 256) {
+        batch_ok && m > 64 && n > 64 && (long long)((m + 127) / 128) * ((n + 127) / 128) * batch >= cu_tiles()) {
         p.fam = FAM_PIPE32; p.bm = 128; p.bn = 128; p.a_mc = !(a_cs == 1 && a_rs % 4 == 0); p.b_mc = !(b_rs == 1 && b_cs % 4 == 0); p.edge = (m % 128) || (n % 128); p.name = "pipe32_128x128";
         return p;
     }
@@ -160,28 +116,28 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     // 128 x 128: no k loop to pipeline, so every wave multiplies a 64 x 64 patch straight out of registers (no LDS, no
     // barrier).  (With unit stride along k a lane's loads touch 64 cache lines per instruction and the vector cache's
     // tag lookups take longer than the MFMAs: those layouts keep LDS.)
-    if (dtype == RP_DTYPE_FLOAT32 && allow_direct && !direct32_off() && k > 32 && k <= 64 && a_rs == 1 && a_cs != 1 && b_cs == 1 && b_rs != 1 &&
+    if (dtype == RP_DTYPE_FLOAT32 && allow_direct && !path_disabled("direct32") && k > 32 && k <= 64 && a_rs == 1 && a_cs != 1 && b_cs == 1 && b_rs != 1 &&
         (a_cs != 1 || (k % 4 == 0 && a_rs % 4 == 0 && a_bs % 4 == 0)) && (b_rs != 1 || (k % 4 == 0 && b_cs % 4 == 0 && b_bs % 4 == 0)) &&
-        m >= 64 && n >= 64 && (long long)((m + 127) / 128) * ((n + 127) / 128) * batch >= 128) {
+        m >= 64 && n >= 64 && (long long)((m + 127) / 128) * ((n + 127) / 128) * batch >= cu_tiles() / 2) {
         p.fam = FAM_DIRECT32; p.bm = 128; p.bn = 128; p.a_mc = a_cs != 1; p.b_mc = b_rs != 1; p.name = "direct32_128x128";
         return p;
     }
     // the same for bf16 / fp16 (C row-major): there the stores and the narrowing are what takes time
-    if (is16 && allow_direct && !pipe16_off() && k <= 64 && k % 8 == 0 && (a_kc || a_mc) && (b_kc || b_mc) && batch_ok &&
-        c_cs == 1 && c_rs % 8 == 0 && n % 8 == 0 && m > 64 && n > 64 && (long long)((m + 127) / 128) * ((n + 127) / 128) * batch >= 256) {
+    if (is16 && allow_direct && !path_disabled("pipe16") && k <= 64 && k % 8 == 0 && (a_kc || a_mc) && (b_kc || b_mc) && batch_ok &&
+        c_cs == 1 && c_rs % 8 == 0 && n % 8 == 0 && m > 64 && n > 64 && (long long)((m + 127) / 128) * ((n + 127) / 128) * batch >= cu_tiles()) {
         p.fam = FAM_PIPE16; p.bm = 128; p.bn = 128; p.a_mc = !a_kc; p.b_mc = !b_kc; p.edge = (m % 128) || (n % 128); p.name = "pipe16_128x128";
         return p;
     }
     // bf16 / fp16, at most 64 output columns, at least one 128-row tile per CU (O = P.V per head, a tall matrix times a narrow
     // one): bound by reading A; the resident kernel whose fetching waves keep three k slabs in flight into LDS
-    if (is16 && allow_direct && !pipe16k_off() && n <= 64 && n % 8 == 0 && k % 8 == 0 && k >= 64 && (a_kc || a_mc) && (b_kc || b_mc) && batch_ok &&
-        c_cs == 1 && c_rs % 8 == 0 && m > 64 && (long long)((m + 127) / 128) * batch >= 256) {
+    if (is16 && allow_direct && !path_disabled("pipe16k") && n <= 64 && n % 8 == 0 && k % 8 == 0 && k >= 64 && (a_kc || a_mc) && (b_kc || b_mc) && batch_ok &&
+        c_cs == 1 && c_rs % 8 == 0 && m > 64 && (long long)((m + 127) / 128) * batch >= cu_tiles()) {
         p.fam = FAM_PIPE16K; p.bm = 128; p.bn = 64; p.a_mc = !a_kc; p.b_mc = !b_kc; p.edge = (m % 128) || n != 64; p.name = "pipe16k_128x64";
         return p;
     }
     // the same in fp32 (any C strides): bound by the MFMAs, which the resident kernel keeps fed without a wait per slab
-    if (dtype == RP_DTYPE_FLOAT32 && allow_direct && !pipe32k_off() && n <= 64 && k % 4 == 0 && k >= 32 && (a_kc || (a_rs == 1 && a_cs % 4 == 0)) &&
-        (b_kc || (b_cs == 1 && b_rs % 4 == 0)) && batch_ok && m > 64 && (long long)((m + 127) / 128) * batch >= 256) {
+    if (dtype == RP_DTYPE_FLOAT32 && allow_direct && !path_disabled("pipe32k") && n <= 64 && k % 4 == 0 && k >= 32 && (a_kc || (a_rs == 1 && a_cs % 4 == 0)) &&
+        (b_kc || (b_cs == 1 && b_rs % 4 == 0)) && batch_ok && m > 64 && (long long)((m + 127) / 128) * batch >= cu_tiles()) {
         p.fam = FAM_PIPE32K; p.bm = 128; p.bn = 64; p.a_mc = !a_kc; p.b_mc = !b_kc; p.edge = (m % 128) || n != 64; p.name = "pipe32k_128x64";
         return p;
     }
@@ -195,7 +151,7 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
         p.fam = FAM_MFMAW;
         long long tiles128 = (long long)((m + 127) / 128) * ((n + 127) / 128) * batch;
         // a 128 x 128 tile over a 64-wide output would compute and fetch half of it for nothing
-        if (m > 64 && n > 64 && tiles128 >= 128) { p.bm = 128; p.bn = 128; p.name = (dtype == RP_DTYPE_FLOAT32) ? "mfma32_128x128" : "mfma64_128x128"; }
+        if (m > 64 && n > 64 && tiles128 >= cu_tiles() / 2) { p.bm = 128; p.bn = 128; p.name = (dtype == RP_DTYPE_FLOAT32) ? "mfma32_128x128" : "mfma64_128x128"; }
         else { p.bm = 64; p.bn = 64; p.name = (dtype == RP_DTYPE_FLOAT32) ? "mfma32_64x64" : "mfma64_64x64"; }
         p.edge = (m % p.bm) || (n % p.bn) || (k % (dtype == RP_DTYPE_FLOAT32 ? 32 : 16));
     }
@@ -268,7 +224,7 @@ int launch_gemm_segmented_b(const GemmArgs& g, int dtype) {
     }
     Plan p{FAM_MFMAW, 64, 64, !a_kc, g.seg_k > 0, true, "mfmaw"};
     const long long tiles128 = (long long)((g.m + 127) / 128) * ((g.n + 127) / 128) * g.batch;
-    if (g.m > 64 && g.n > 64 && tiles128 >= 128) { p.bm = 128; p.bn = 128; }
+    if (g.m > 64 && g.n > 64 && tiles128 >= cu_tiles() / 2) { p.bm = 128; p.bn = 128; }
     p.edge = (g.m % p.bm) || (g.n % p.bn) || (g.k % bk);
     return launch_mfmaw(g, p, dtype);
 }

@@ -271,10 +271,8 @@ int* splitk_arrival_counters(long long tiles, size_t partial_bytes, bool* failed
     constexpr int MAX_DEVICES = 64;
     static std::mutex mu;
     static int* blocks[MAX_DEVICES] = {};
-    static int two_launch = -1;
     *failed = false;
-    if (two_launch < 0) { const char* e = getenv("RP_HIP_SPLITK_TWO_LAUNCH"); two_launch = (e && e[0] == '1') ? 1 : 0; }
-    if (two_launch == 1 || tiles > SPLITK_MAX_TILES || partial_bytes >= (1ull << 31)) return nullptr;
+    if (path_disabled("one_launch_splitk") || tiles > SPLITK_MAX_TILES || partial_bytes >= (1ull << 31)) return nullptr;
     if (noalloc_active()) {                              // inside the entry point that allocates nothing: its fixed counters
         int* fixed = noalloc_arrival_counters();
         if (!fixed) *failed = true;
@@ -371,23 +369,14 @@ static int launch_generic_t(const GemmArgs& g) {
     return check_launch("gemm_generic_kernel") ? 0 : -1;
 }
 
-static int skinny_k_per_block() {
-    static int v = -1;
-    if (v < 0) { const char* e = getenv("RP_HIP_SKINNY_KPB"); v = e ? atoi(e) : 0; if (v < 0) v = 0; }
-    return v;
-}
-
 template <typename T>
 static int launch_skinny_t(const GemmArgs& g) {
     constexpr int VEC = 16 / sizeof(T);
     int groups = (g.n + 64 * VEC - 1) / (64 * VEC);
     // enough blocks to put two on every CU, each wave keeping at least 32 k rows
-    int k_per_block = skinny_k_per_block();
-    if (k_per_block == 0) {
-        int want = (512 + groups - 1) / groups;
-        k_per_block = (g.k + want - 1) / want;
-        if (k_per_block < 256) k_per_block = 256;
-    }
+    const int want = (512 + groups - 1) / groups;
+    int k_per_block = (g.k + want - 1) / want;
+    if (k_per_block < 256) k_per_block = 256;
     if (k_per_block > 2048) k_per_block = 2048;            // bounds the LDS copy of A (2048 x 8 floats = 64 KB)
     k_per_block = (k_per_block + SK_WAVES - 1) / SK_WAVES * SK_WAVES;
     int nsplit = (g.k + k_per_block - 1) / k_per_block;

@@ -20,7 +20,8 @@ namespace rp {
 // the column, lane / 32 the k half).  The A operand is a 16-byte load of row
 // lane % 32 (zero beyond m).  MFMA c therefore accumulates the 32 x 32 tile of
 // output columns {8j + c}; 8 accumulators cover the wave's 256 columns.
-// Loads for four rounds are always in flight per wave and are issued
+// Loads for two rounds are always in flight per wave (deeper queues only add
+// waiting: four rounds in flight cost 0.6 us per launch, one round 3.5 us) and are issued
 // unconditionally (out-of-range rounds get an empty buffer descriptor and read
 // zeros), so the waits the compiler inserts count loads exactly.
 //
@@ -47,7 +48,7 @@ namespace rp {
 // ============================================================================
 constexpr int SS_WAVES = 4, SS_COLS = 256, SS_ROUND = 16, SS_RED_PITCH = SS_COLS + 8;
 constexpr int SS_MAX_M = 16;
-constexpr int SS_DEPTH = 4;            // rounds a wave keeps in flight (register slots)
+constexpr int SS_DEPTH = 2;            // rounds a wave keeps in flight (register slots): 16 KB per wave, 16 MB over the chip
 
 template <typename T, int MT>          // MT: rows the epilogue keeps (8 or 16; m <= MT)
 __global__ void __launch_bounds__(256) gemm_stream16_kernel(GemmArgs g, float* partials, int groups, int nsplit, int* arrivals, int local) {
@@ -286,12 +287,6 @@ static int launch_stream16(const GemmArgs& g, int dtype) {
     return rc;
 }
 
-static bool tiled_skinny_forced() {          // RP_HIP_SKINNY_TILED=1: measure the tiled kernel on shapes the streaming one takes
-    static int v = -1;
-    if (v < 0) { const char* e = getenv("RP_HIP_SKINNY_TILED"); v = (e && e[0] == '1') ? 1 : 0; }
-    return v == 1;
-}
-
 // ---- tiled kernel for the other operand layouts ----
 template <typename T>
 static int launch_skinny16_t(const GemmArgs& g, const Plan& p, float* partials, int nsplit, int k_per_split) {
@@ -304,7 +299,7 @@ static int launch_skinny16_t(const GemmArgs& g, const Plan& p, float* partials, 
 
 int launch_mfma16_skinny(const GemmArgs& g, const Plan& p, int dtype) {
     if (dtype != RP_DTYPE_BFLOAT16 && dtype != RP_DTYPE_FLOAT16) { set_error("mfma16 skinny GEMM: unsupported dtype %d", dtype); return -1; }
-    if (!p.a_mc && p.b_mc && g.m <= SS_MAX_M && !tiled_skinny_forced()) return launch_stream16(g, dtype);
+    if (!p.a_mc && p.b_mc && g.m <= SS_MAX_M && !path_disabled("stream16")) return launch_stream16(g, dtype);
     constexpr int BN = 128;
     const int tiles = ((g.n + BN - 1) / BN) * ((g.m + 31) / 32);
     // about three blocks per CU in flight, each split at least four slabs deep

@@ -439,13 +439,6 @@ static int mw_launch_shortk(const GemmArgs& g, bool edge) {
     return launch(gemm_mfmaw_shortk_kernel<T, BM, BN, A_MC, B_MC, false>);
 }
 
-// fp32, k of at most two slabs, at least 128 tiles of 128 x 128: the resident, cross-tile pipelined kernel
-static bool shortk_off() {                        // RP_HIP_NO_SHORTK=1 keeps the general kernel
-    static int v = -1;
-    if (v < 0) { const char* e = getenv("RP_HIP_NO_SHORTK"); v = (e && e[0] == '1') ? 1 : 0; }
-    return v == 1;
-}
-
 template <typename T, int BM, int BN, bool A_MC, bool B_MC, bool EDGE, bool SPLITK>
 static int mw_launch(const GemmArgs& g, dim3 grid, int tiles_m, int tiles_n, float* partials, int k_per_split) {
     constexpr size_t smem = mw_smem_bytes<T>(BM, BN);
@@ -505,7 +498,8 @@ static int launch_mfmaw_t(const GemmArgs& g, const Plan& p) {
 }
 
 int launch_mfmaw(const GemmArgs& g, const Plan& p, int dtype) {
-    if (dtype == RP_DTYPE_FLOAT32 && p.bm == 128 && g.k <= 2 * mfmaw_cfg<float>::BK && !shortk_off() && g.seg_k == 0 && g.seg_n == 0 && g.c_fold_from == 0 && !g.bias_by_row) {
+    // fp32, k of at most two slabs, at least 128 tiles of 128 x 128: the resident, cross-tile pipelined kernel
+    if (dtype == RP_DTYPE_FLOAT32 && p.bm == 128 && g.k <= 2 * mfmaw_cfg<float>::BK && !path_disabled("shortk") && g.seg_k == 0 && g.seg_n == 0 && g.c_fold_from == 0 && !g.bias_by_row) {
         const bool edge = p.edge || g.k != 2 * mfmaw_cfg<float>::BK;
         if (!p.a_mc && p.b_mc) return mw_launch_shortk<float, 128, 128, false, true>(g, edge);
         if (!p.a_mc && !p.b_mc) return mw_launch_shortk<float, 128, 128, false, false>(g, edge);

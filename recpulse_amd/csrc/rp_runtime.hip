@@ -9,6 +9,7 @@
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <string>
 #include <unordered_map>
 #include <vector>
 
@@ -43,11 +44,14 @@ int device_cu_count() {
     int n = cached[dev].load(std::memory_order_relaxed);
     if (n == 0) {
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) { (void)hipGetLastError(); n = 0; }
-        const char* e = getenv("RP_HIP_CU_COUNT");           // measurement aid: pretend the device has this many CUs
-        if (e && atoi(e) > 0) n = atoi(e);
         cached[dev].store(n, std::memory_order_relaxed);
     }
     return n;
+}
+
+bool path_disabled(const char* name) {
+    static const std::string list = [] { const char* e = getenv("RP_HIP_DISABLE"); return std::string(",") + (e ? e : "") + ","; }();
+    return list.find(std::string(",") + name + ",") != std::string::npos;
 }
 
 // ---- workgroup placement -----------------------------------------------------
@@ -79,8 +83,7 @@ bool workgroups_share_xcd_by_residue() {
     std::lock_guard<std::mutex> lock(mu);
     st = state[dev].load(std::memory_order_acquire);
     if (st != 0) return st == 1;
-    const char* off = getenv("RP_HIP_NO_L2_EXCHANGE");
-    bool holds = !(off && off[0] == '1');
+    bool holds = !path_disabled("l2_exchange");
     static int seen[PLACEMENT_BLOCKS];
     for (int rep = 0; rep < 3 && holds; rep++) {
         hipLaunchKernelGGL(record_xcc_kernel, dim3(PLACEMENT_BLOCKS), dim3(256), 0, current_stream());

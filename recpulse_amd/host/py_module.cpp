@@ -306,7 +306,9 @@ PYBIND11_MODULE(recpulse_cuda, m) {
         auto s = to_shape(shape);
         return wrap(rp_rand(parse_dtype(dtype), parse_device(device), (int)s.size(), s.data()), "rand");
     }, py::arg("shape"), py::arg("dtype") = "float32", py::arg("device") = "cpu");
+#ifdef RP_TEST_HOOKS
     m.def("_fail_gemm_after", [](int n) { rp_debug_fail_gemm_after(n); }, py::arg("n"));      // fault injection for tests of the error paths
+#endif
     m.def("manual_seed", [](unsigned long long seed) { rp_manual_seed(seed); });
     // how a temporary looks to a method on this interpreter: call the yardstick on one, and on a named object
     try {

@@ -240,8 +240,10 @@ const char* rp_last_error(void) { return g_err; }
 
 // Fault injection for tests of the error paths: the n-th GEMM issued by the host layer from now on (n = 1 is the next
 // one) fails before anything is launched; n <= 0 switches it off.  Nothing else reads this counter.
+#ifdef RP_TEST_HOOKS
 static thread_local int g_fail_gemm_in = 0;
 void rp_debug_fail_gemm_after(int n) { g_fail_gemm_in = n > 0 ? n : 0; }
+#endif
 
 // ======================================================================== core
 bool validate_device_id(int device_id) {              // reference core/tensor.c:10-16
@@ -627,7 +629,9 @@ int device_gemm(Tensor* c, Tensor* a, bool a_t, Tensor* b, bool b_t, Tensor* bia
     if (ba == 1) a_bs = 0;
     if (bb == 1) b_bs = 0;
     if (!on_device(c->device_id)) return dev_fail("set device");
+#ifdef RP_TEST_HOOKS
     if (g_fail_gemm_in > 0 && --g_fail_gemm_in == 0) { fail("matmul: failure injected by rp_debug_fail_gemm_after"); return -1; }
+#endif
     int rc = rp_hip_gemm_strided_batched(c->data, a->data, b->data, bias ? bias->data : nullptr, batch, m, k, n,
                                          a_bs, a_rs, a_cs, b_bs, b_rs, b_cs, c_bs, c->strides[cn - 2], c->strides[cn - 1], accumulate, c->dtype);
     return rc == 0 ? 0 : dev_fail("matmul");

@@ -66,7 +66,9 @@ struct GradFn {                                     /* reference ops/ops.h:14-20
 
 size_t dtype_size(DType dtype);
 const char* rp_last_error(void);
-void rp_debug_fail_gemm_after(int n);      /* tests of the error paths: the n-th GEMM from now on fails; n <= 0 switches it off */
+#ifdef RP_TEST_HOOKS
+void rp_debug_fail_gemm_after(int n);      /* tests of the error paths: the n-th GEMM from now on fails; n <= 0 switches it off.  Only in builds with -DRP_TEST_HOOKS */
+#endif
 
 /* ---- core ---- */
 bool validate_device_id(int device_id);

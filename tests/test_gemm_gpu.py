@@ -306,7 +306,7 @@ def test_streaming_rows_finish_repeats_bit_for_bit_over_hundreds_of_launches(m):
 
 def test_streaming_rows_both_exchanges_give_the_same_bits(tmp_path):
     """The k-split finish goes through the XCD's own L2 when workgroup placement was verified, and through memory at
-    device scope otherwise (RP_HIP_NO_L2_EXCHANGE=1 forces that, read once per process): a child process computes
+    device scope otherwise (RP_HIP_DISABLE=l2_exchange forces that, read once per process): a child process computes
     the same products the other way, and the bits must agree (same partial sums, same order)."""
     import subprocess
     import sys
@@ -322,9 +322,9 @@ def test_streaming_rows_both_exchanges_give_the_same_bits(tmp_path):
         "np.savez(sys.argv[1], **out)\n"
     ) % (os.path.dirname(os.path.abspath(__file__)), os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
     results = []
-    for flag in ("0", "1"):
-        path = str(tmp_path / f"exchange{flag}.npz")
-        env = dict(os.environ, RP_HIP_NO_L2_EXCHANGE=flag)
+    for flag in ("", "l2_exchange"):
+        path = str(tmp_path / f"exchange_{flag or 'on'}.npz")
+        env = dict(os.environ, RP_HIP_DISABLE=flag)
         subprocess.run([sys.executable, "-c", code, path], check=True, env=env, timeout=300)
         results.append(np.load(path))
     for key in results[0].files:
