@@ -208,6 +208,77 @@ Tensor* make_view(Tensor* x, int ndim, const int* shape, const int* strides, siz
 // dense tensor of the same values (new reference either way), like ensure_contiguous (reference ops/ops.c:21-25)
 Tensor* dense(Tensor* x) { return rp_is_contiguous(x) ? tensor_retain(x) : rp_contiguous(x); }
 
+// ---- host (CPU) arithmetic for tensors with device_id == -1 ----
+// The reference runs these on the host when a tensor lives there (functional/functional.c:978-1003, 58-74).  Results are
+// those of its loops: every output element accumulates its products in the order l = 0 .. k-1, multiply then add in the
+// accumulation type, no fused multiply-add (the host layer is compiled with -ffp-contract=off); 16-bit operands go
+// through float32 and are narrowed once (functional/functional.c:986-1000).  The loops here are blocked over the output
+// (4 rows x 64 columns of accumulators, the k loop innermost per block and vectorisable across columns), which changes
+// which element is worked on when, not the order of any element's sum.
+template <typename A>
+void host_matmul_acc(A* C, const A* Am, const A* Bm, int m, int k, int n) {
+    constexpr int RB = 4, CB = 64;
+    for (int i0 = 0; i0 < m; i0 += RB) {
+        const int ib = m - i0 < RB ? m - i0 : RB;
+        for (int j0 = 0; j0 < n; j0 += CB) {
+            const int jb = n - j0 < CB ? n - j0 : CB;
+            A acc[RB][CB];
+            for (int ii = 0; ii < ib; ii++) for (int jj = 0; jj < jb; jj++) acc[ii][jj] = (A)0;
+            for (int l = 0; l < k; l++) {
+                const A* brow = Bm + (size_t)l * n + j0;
+                for (int ii = 0; ii < ib; ii++) {
+                    const A a = Am[(size_t)(i0 + ii) * k + l];
+                    for (int jj = 0; jj < jb; jj++) acc[ii][jj] += a * brow[jj];
+                }
+            }
+            for (int ii = 0; ii < ib; ii++) for (int jj = 0; jj < jb; jj++) C[(size_t)(i0 + ii) * n + j0 + jj] = acc[ii][jj];
+        }
+    }
+}
+
+// element i of a host array as the accumulation type of its dtype (float, or double for float64), and back with one rounding
+template <typename A> A host_load(const void* p, size_t i, DType dt) { return (A)load_as_double(p, i, dt); }
+template <typename A> void host_store(void* p, size_t i, DType dt, A v) { store_from_double(p, i, dt, (double)v); }
+
+// C[z] = (accumulate ? C[z] : 0) + A[z] . B[z] (+ bias) on strided host operands: each operand is gathered into a dense
+// array of the accumulation type (the reference's contiguous copies and its float32 pivot in one step), multiplied, and
+// the result goes through the same chain of roundings as the device epilogue: product, + bias, + old value, each rounded
+// to the tensor type (ops/ops.c:6838, 162, 6785).
+template <typename A>
+int host_gemm_t(void* C, const void* Ap, const void* Bp, const void* bias, int batch, int m, int k, int n,
+                long long a_bs, long long a_rs, long long a_cs, long long b_bs, long long b_rs, long long b_cs,
+                long long c_bs, long long c_rs, long long c_cs, int accumulate, DType dt) {
+    std::vector<A> a((size_t)m * k), b((size_t)k * n), c((size_t)m * n);
+    for (int z = 0; z < batch; z++) {
+        for (int i = 0; i < m; i++) for (int l = 0; l < k; l++) a[(size_t)i * k + l] = host_load<A>(Ap, (size_t)(z * a_bs + i * a_rs + l * a_cs), dt);
+        for (int l = 0; l < k; l++) for (int j = 0; j < n; j++) b[(size_t)l * n + j] = host_load<A>(Bp, (size_t)(z * b_bs + l * b_rs + j * b_cs), dt);
+        host_matmul_acc<A>(c.data(), a.data(), b.data(), m, k, n);
+        for (int i = 0; i < m; i++)
+            for (int j = 0; j < n; j++) {
+                const size_t at = (size_t)(z * c_bs + i * c_rs + j * c_cs);
+                A old = accumulate ? host_load<A>(C, at, dt) : (A)0;
+                host_store<A>(C, at, dt, c[(size_t)i * n + j]);
+                if (bias) host_store<A>(C, at, dt, host_load<A>(C, at, dt) + host_load<A>(bias, (size_t)j, dt));
+                if (accumulate) host_store<A>(C, at, dt, old + host_load<A>(C, at, dt));
+            }
+    }
+    return 0;
+}
+
+int host_gemm(void* C, const void* A, const void* B, const void* bias, int batch, int m, int k, int n,
+              long long a_bs, long long a_rs, long long a_cs, long long b_bs, long long b_rs, long long b_cs,
+              long long c_bs, long long c_rs, long long c_cs, int accumulate, DType dt) {
+    if (dt == DTYPE_FLOAT64) return host_gemm_t<double>(C, A, B, bias, batch, m, k, n, a_bs, a_rs, a_cs, b_bs, b_rs, b_cs, c_bs, c_rs, c_cs, accumulate, dt);
+    return host_gemm_t<float>(C, A, B, bias, batch, m, k, n, a_bs, a_rs, a_cs, b_bs, b_rs, b_cs, c_bs, c_rs, c_cs, accumulate, dt);
+}
+
+// out = x1 + x2 element by element in the accumulation type, rounded once (functional/functional_host.c, 16-bit through float32)
+void host_add(void* out, const void* x1, const void* x2, size_t size, DType dt) {
+    if (dt == DTYPE_FLOAT64) { for (size_t i = 0; i < size; i++) ((double*)out)[i] = ((const double*)x1)[i] + ((const double*)x2)[i]; return; }
+    if (dt == DTYPE_FLOAT32) { for (size_t i = 0; i < size; i++) ((float*)out)[i] = ((const float*)x1)[i] + ((const float*)x2)[i]; return; }
+    for (size_t i = 0; i < size; i++) host_store<float>(out, i, dt, host_load<float>(x1, i, dt) + host_load<float>(x2, i, dt));
+}
+
 // Accumulate rule of every backward function (reference ops/ops.c:6781-6788): the first gradient is stored,
 // later ones are added in place.  `g` is consumed.
 void accumulate_grad(Tensor* x, Tensor* g) {
@@ -216,6 +287,10 @@ void accumulate_grad(Tensor* x, Tensor* g) {
     if (!m->grad) { m->grad = g; return; }
     if (m->grad->device_id >= 0) {
         if (on_device(x->device_id)) add_kernel_device(m->grad->data, m->grad->data, g->data, x->size, x->dtype);
+    } else {
+        Tensor* gd = dense(g);                          // (gradients are made dense before they are added, like on the device)
+        if (gd && rp_is_contiguous(m->grad)) host_add(m->grad->data, m->grad->data, gd->data, x->size, x->dtype);
+        free_tensor(gd);
     }
     free_tensor(g);
 }
@@ -458,14 +533,14 @@ int tensor_backward(Tensor* root) {
 // ================================================================== functional
 int rp_matmul(void* C, const void* A, const void* B, int m, int k, int n, DType dtype, int device_id) {    // reference functional/functional.c:978-1006
     if (!C || !A || !B || m <= 0 || k <= 0 || n <= 0) return -1;
-    if (device_id == -1) { fail("matmul on host tensors is not provided by this build; move the operands to a GPU"); return -1; }
+    if (device_id == -1) return host_gemm(C, A, B, nullptr, 1, m, k, n, 0, k, 1, 0, n, 1, 0, n, 1, 0, dtype);     // reference :986-1000
     if (!on_device(device_id)) return dev_fail("set device");
     return matmul_kernel_device(C, A, B, m, k, n, dtype) == 0 ? 0 : dev_fail("matmul");
 }
 
 int rp_add(void* out, const void* x1, const void* x2, size_t size, DType dtype, int device_id) {           // reference functional/functional.c:58-74
     if (!out || !x1 || !x2 || size == 0) return -1;
-    if (device_id == -1) { fail("add on host tensors is not provided by this build"); return -1; }
+    if (device_id == -1) { host_add(out, x1, x2, size, dtype); return 0; }
     if (!on_device(device_id)) return dev_fail("set device");
     return add_kernel_device(out, x1, x2, size, dtype) == 0 ? 0 : dev_fail("add");
 }
@@ -628,6 +703,9 @@ int device_gemm(Tensor* c, Tensor* a, bool a_t, Tensor* b, bool b_t, Tensor* bia
     if ((ba != batch && ba != 1) || (bb != batch && bb != 1)) { fail("matmul: batch sizes differ"); return -1; }
     if (ba == 1) a_bs = 0;
     if (bb == 1) b_bs = 0;
+    if (c->device_id == -1)
+        return host_gemm(c->data, a->data, b->data, bias ? bias->data : nullptr, batch, m, k, n, a_bs, a_rs, a_cs, b_bs, b_rs, b_cs,
+                         c_bs, c->strides[cn - 2], c->strides[cn - 1], accumulate, c->dtype);
     if (!on_device(c->device_id)) return dev_fail("set device");
 #ifdef RP_TEST_HOOKS
     if (g_fail_gemm_in > 0 && --g_fail_gemm_in == 0) { fail("matmul: failure injected by rp_debug_fail_gemm_after"); return -1; }
@@ -691,6 +769,33 @@ Tensor* reduce_grad_to_shape(Tensor* grad, int target_ndim, const int* target_sh
     Tensor* g = dense(grad);
     if (!g) return nullptr;
     size_t target_size = shape_size(target_ndim, target_shape);
+    if (g->device_id == -1) {
+        // host tensors: the reference's loop (ops/ops.c:7027-7086): every gradient element, in row-major order, is added to
+        // the target element its index folds onto, in float32 (float64 for float64), rounded once at the end
+        const int lead = g->ndim - target_ndim;
+        if (lead < 0) { fail("reduce_grad_to_shape: shapes do not broadcast"); free_tensor(g); return nullptr; }
+        std::vector<double> acc64(g->dtype == DTYPE_FLOAT64 ? target_size : 0, 0.0);
+        std::vector<float> acc32(g->dtype == DTYPE_FLOAT64 ? 0 : target_size, 0.f);
+        std::vector<long long> tstride(target_ndim);
+        long long st = 1;
+        for (int d = target_ndim - 1; d >= 0; d--) { tstride[d] = st; st *= target_shape[d]; }
+        for (size_t i = 0; i < g->size; i++) {
+            size_t rem = i; long long to = 0;
+            for (int d = g->ndim - 1; d >= 0; d--) {
+                const long long c = (long long)(rem % g->shape[d]); rem /= g->shape[d];
+                if (d >= lead && target_shape[d - lead] != 1) to += c * tstride[d - lead];
+            }
+            if (g->dtype == DTYPE_FLOAT64) acc64[to] += ((const double*)g->data)[i];
+            else acc32[to] += host_load<float>(g->data, i, g->dtype);
+        }
+        Tensor* out = empty_tensor(g->dtype, -1, target_ndim, target_shape);
+        for (size_t i = 0; out && i < target_size; i++) {
+            if (g->dtype == DTYPE_FLOAT64) ((double*)out->data)[i] = acc64[i];
+            else host_store<float>(out->data, i, g->dtype, acc32[i]);
+        }
+        free_tensor(g);
+        return out;
+    }
     // trailing-dims case (bias of Linear): grad viewed as [outer, inner], columns summed top to bottom
     bool trailing = target_ndim <= g->ndim;
     for (int d = 0; trailing && d < target_ndim; d++) trailing = target_shape[target_ndim - 1 - d] == g->shape[g->ndim - 1 - d];
@@ -753,7 +858,7 @@ GradSlot grad_slot(Tensor* target) {
 void backward_linear_fn(GradFn* self, Tensor* grad_output) {
     Tensor* x = self->inputs[0]; Tensor* w = self->inputs[1];
     Tensor* bias = self->num_inputs > 2 ? self->inputs[2] : nullptr;
-    if (x->ndim == 2 && w->ndim == 2 && on_device(x->device_id)) {
+    if (x->ndim == 2 && w->ndim == 2 && x->device_id >= 0 && on_device(x->device_id)) {
         // one call for the three gradients: a single launch for layers as small as an MLP's
         Tensor* g = dense(grad_output);
         GradSlot sx = grad_slot(x), sw = grad_slot(w), sb = grad_slot(bias);
@@ -1173,7 +1278,6 @@ Tensor* op_matmul(Tensor* a, Tensor* b) {              // reference ops/ops.c:68
     if (b->ndim > 2 && b->ndim != a->ndim) { fail("op_matmul: batched operands need equal rank"); return nullptr; }
     for (int d = 0; b->ndim > 2 && d < a->ndim - 2; d++)
         if (a->shape[d] != b->shape[d]) { fail("op_matmul: batch dimensions differ"); return nullptr; }
-    if (a->device_id == -1) { fail("op_matmul on host tensors is not provided by this build; move the operands to a GPU"); return nullptr; }
     std::vector<int> shape(a->shape, a->shape + a->ndim);
     shape[a->ndim - 1] = b->shape[b->ndim - 1];
     Tensor* out = empty_tensor(a->dtype, a->device_id, a->ndim, shape.data());
@@ -1193,7 +1297,6 @@ Tensor* op_linear(Tensor* x, Tensor* w, Tensor* bias) {
     if (!x || !w) return nullptr;
     if (x->ndim < 2 || w->ndim != 2 || !same_place(x, w) || x->shape[x->ndim - 1] != w->shape[0]) { fail("op_linear: shape, dtype or device mismatch"); return nullptr; }
     if (bias && (bias->ndim != 1 || bias->shape[0] != w->shape[1] || !same_place(x, bias) || !rp_is_contiguous(bias))) { fail("op_linear: bias must be a dense vector of out_features"); return nullptr; }
-    if (x->device_id == -1) { fail("op_linear on host tensors is not provided by this build; move the operands to a GPU"); return nullptr; }
     std::vector<int> shape(x->shape, x->shape + x->ndim);
     shape[x->ndim - 1] = w->shape[1];
     Tensor* out = empty_tensor(x->dtype, x->device_id, x->ndim, shape.data());
@@ -1377,7 +1480,6 @@ Tensor* op_gru_cell(Tensor* x, Tensor* h, Tensor* w_ih, Tensor* w_hh, Tensor* b_
 Tensor* op_add(Tensor* x1, Tensor* x2) {               // reference ops/ops.c:129-210
     if (!x1 || !x2) return nullptr;
     if (!same_place(x1, x2)) { fail("op_add: dtype or device mismatch"); return nullptr; }
-    if (x1->device_id == -1) { fail("op_add on host tensors is not provided by this build"); return nullptr; }
     int nd = x1->ndim > x2->ndim ? x1->ndim : x2->ndim;
     if (nd > 8) { fail("op_add: more than 8 dimensions"); return nullptr; }
     std::vector<int> shape(nd);
@@ -1392,7 +1494,21 @@ Tensor* op_add(Tensor* x1, Tensor* x2) {               // reference ops/ops.c:12
     Tensor* out = empty_tensor(x1->dtype, x1->device_id, nd, shape.data());
     if (!out) return nullptr;
     int rc;
-    if (!on_device(x1->device_id)) rc = -1;
+    if (x1->device_id == -1) {
+        // host tensors: both operands expanded to the output shape with stride-0 dimensions (functional/functional.c:1959-1966)
+        // and added element by element in row-major order
+        Tensor* e1 = rp_expand(x1, nd, shape.data());
+        Tensor* e2 = rp_expand(x2, nd, shape.data());
+        rc = (e1 && e2) ? 0 : -1;
+        for (size_t i = 0; rc == 0 && i < out->size; i++) {
+            size_t rem = i; long long o1 = 0, o2 = 0;
+            for (int d = nd - 1; d >= 0; d--) { const long long c = (long long)(rem % shape[d]); rem /= shape[d]; o1 += c * e1->strides[d]; o2 += c * e2->strides[d]; }
+            if (x1->dtype == DTYPE_FLOAT64) ((double*)out->data)[i] = ((const double*)e1->data)[o1] + ((const double*)e2->data)[o2];
+            else host_store<float>(out->data, i, x1->dtype, host_load<float>(e1->data, (size_t)o1, x1->dtype) + host_load<float>(e2->data, (size_t)o2, x1->dtype));
+        }
+        free_tensor(e1); free_tensor(e2);
+    }
+    else if (!on_device(x1->device_id)) rc = -1;
     else if (same_shape(x1, x2) && rp_is_contiguous(x1) && rp_is_contiguous(x2)) rc = add_kernel_device(out->data, x1->data, x2->data, x1->size, x1->dtype);
     else {
         Tensor* e1 = rp_expand(x1, nd, shape.data());

@@ -1,5 +1,9 @@
 """Host-side logic of the drop-in (no GPU): tensor construction, dtype rules, view algebra, Module bookkeeping,
-error conventions.  Compute ops are device-only in this build and must refuse host tensors loudly."""
+error conventions, and the matmul path on host tensors (op_matmul, op_linear, op_add and their gradients), which the
+host layer computes in the reference's summation order.  Every other op is device-only and must refuse host tensors loudly."""
+import json
+import os
+
 import numpy as np
 import pytest
 
@@ -84,17 +88,84 @@ def test_copy_and_grad_flags():
         rp.values([1.0]).backward()                                        # no requires_grad (reference core/tensor.c:221)
 
 
-def test_compute_on_host_tensors_is_refused_loudly():
+def test_host_tensors_compute_matmul_and_add_and_refuse_the_rest():
+    """The matmul path runs on host tensors too (reference functional/functional.c:978-1003): op_matmul, op_linear, op_add
+    and their gradients.  Every other op is provided on the device only and fails loudly on the host."""
     a = rp.values([1.0, 2.0, 3.0, 4.0]).reshape([2, 2])
-    with pytest.raises(RuntimeError, match="op_matmul operation failed"):
-        a.op_matmul(a)
-    for call in (lambda: a.op_add(a), lambda: a.op_relu(), lambda: a.op_softmax(), lambda: a.op_sum_all(),
-                 lambda: a.op_linear(a), lambda: a.op_cross_entropy_loss([0, 1])):
+    assert np.array_equal(a.op_matmul(a).to_numpy(), [[7.0, 10.0], [15.0, 22.0]])
+    assert np.array_equal(a.op_add(a).to_numpy(), [[2.0, 4.0], [6.0, 8.0]])
+    for call in (lambda: a.op_relu(), lambda: a.op_softmax(), lambda: a.op_sum_all(), lambda: a.op_cross_entropy_loss([0, 1])):
         with pytest.raises(RuntimeError, match="operation failed"):
             call()
     assert np.allclose(a.mul_scalar(0.5).to_numpy(), [[0.5, 1.0], [1.5, 2.0]])        # initialiser helper stays on the host
     with pytest.raises(RuntimeError, match="op_matmul operation failed"):               # shape errors come first, device or not
         a.op_matmul(rp.zeros([3, 2]))
+
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")))
+
+
+def _host(arr, dtype="float32", grad=False):
+    t = rp.from_numpy(np.ascontiguousarray(arr, dtype=np.float64 if dtype == "float64" else np.float32))
+    if dtype not in ("float32", "float64"):
+        t = t.to(dtype=dtype)
+    return t.requires_grad_(True) if grad else t
+
+
+def _np(t):
+    return t.to(dtype="float64").to_numpy()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float64", "float16", "bfloat16"])
+def test_host_matmul_known_answers_of_the_reference(dtype):
+    """The reference's own known answers for the path, on 'cpu' (tests/unit/test_functional.py:281-302,
+    tests/autograd/test_matmul_autograd.py:35-128, 215-287)."""
+    for key in ("matmul_2x3_3x2", "matmul_identity"):
+        c = _host(GOLD[key]["a"], dtype).op_matmul(_host(GOLD[key]["b"], dtype))
+        assert np.array_equal(_np(c), np.array(GOLD[key]["c"], dtype=np.float64)), key
+    for key in ("backward_a", "backward_both_2x2", "backward_nonsquare_2x4_4x3") + (("backward_f64_2x2",) if dtype == "float64" else ()):
+        a, b = _host(GOLD[key]["a"], dtype, grad=True), _host(GOLD[key]["b"], dtype, grad=True)
+        a.op_matmul(b).backward()                          # root seeded with ones of its own shape: the gradient of the sum
+        assert np.allclose(_np(a.grad), GOLD[key]["da"], rtol=1e-15, atol=0), key
+        assert np.allclose(_np(b.grad), GOLD[key]["db"], rtol=1e-15, atol=0), key
+
+
+@pytest.mark.parametrize("dtype,code", [("float32", oracle.F32), ("float64", oracle.F64), ("float16", oracle.F16), ("bfloat16", oracle.BF16)])
+def test_host_matmul_is_the_reference_loop_bit_for_bit(dtype, code):
+    """Blocked over the output, but every element still sums its products in the order l = 0 .. k-1 without fused
+    multiply-adds: the bits of the reference's i-j-l loop (the oracle, itself pinned to the reference's compiled kernel)
+    on ragged shapes, on a transposed view, with a broadcast bias, and for both gradients."""
+    rng = np.random.default_rng(7)
+    for m, k, n in [(3, 4, 5), (16, 32, 8), (1, 7, 1), (64, 64, 64), (5, 130, 67), (70, 9, 129)]:
+        a64, b64, bias64 = rng.uniform(-1, 1, (m, k)), rng.uniform(-1, 1, (k, n)), rng.uniform(-1, 1, (n,))
+        a_st, b_st, bias_st = (oracle.to_storage(x, code) for x in (a64, b64, bias64))
+        a, b, bias = (_host(oracle.to_f64(x, code), dtype, grad=True) for x in (a_st, b_st, bias_st))
+        y = a.op_matmul(b)
+        want = oracle.matmul(a_st, b_st, code)
+        assert np.array_equal(_np(y), oracle.to_f64(want, code)), (m, k, n)
+        z = y.op_add(bias)
+        assert np.array_equal(_np(z), oracle.to_f64(oracle.bias_add(want, bias_st, code), code))
+        z.backward()
+        ones = oracle.to_storage(np.ones((m, n)), code)
+        da, db, dbias = oracle.matmul_backward(a_st, b_st, ones, code) + (oracle.reduce_rows(ones, code),)
+        assert np.array_equal(_np(a.grad), oracle.to_f64(da, code)) and np.array_equal(_np(b.grad), oracle.to_f64(db, code))
+        assert np.array_equal(_np(bias.grad), oracle.to_f64(dbias, code))
+        # the same product from a transposed, non-contiguous view of A (reference tests/stress/stress_gradcheck.py:228-243)
+        at = _host(oracle.to_f64(np.ascontiguousarray(a_st.T), code), dtype)
+        assert np.array_equal(_np(at.transpose(0, 1).op_matmul(b)), oracle.to_f64(want, code))
+
+
+def test_config1_linear_forward_on_the_host_matches_the_oracle():
+    """BASELINE configuration 1 as the reference runs it on its CPU path: Y = X[128,784] @ W[784,256] + b[256], fp32."""
+    from recpulse.module import Linear
+    rng = np.random.default_rng(0)
+    x = rng.uniform(0, 1, (128, 784)).astype(np.float32)
+    w = rng.normal(0, np.sqrt(1.0 / 784), (784, 256)).astype(np.float32)
+    b = rng.normal(0, 0.1, (256,)).astype(np.float32)
+    fc = Linear(784, 256)
+    fc.weight.copy_(rp.from_numpy(w)); fc.bias.copy_(rp.from_numpy(b))
+    y = fc(rp.from_numpy(x))
+    assert np.array_equal(y.to_numpy(), oracle.linear_forward(x, w, b, oracle.F32))
 
 
 def test_linear_registers_parameters_like_the_reference():
