@@ -575,8 +575,10 @@ def conv2d_times(capi, dt_name="bf16"):
 
 
 def lstm_step_times(capi, dt_name="bf16"):
-    """One LSTM step (batch 64, input 1024, hidden 1024) forward + backward through the C ABI: 2 + 4 GEMMs, the two
-    fused element-wise kernels and the bias reduction, each launch on its own and the whole step from one HIP graph."""
+    """One LSTM step (batch 64, input 1024, hidden 1024) forward + backward through the C ABI: the two gate products,
+    the four gradient products (as two launches of two matrices each, the way the host layer issues them, and one by
+    one), the two fused element-wise kernels and the bias reduction; each launch on its own and the whole step from one
+    HIP graph."""
     rng = np.random.default_rng(5)
     B, I, H = 64, 1024, 1024
     G = 4 * H
@@ -605,20 +607,37 @@ def lstm_step_times(capi, dt_name="bf16"):
         "dWhh=ht.dg": (lambda: capi.gemm(d_dwh.ptr, d_h.ptr, d_dg.ptr, None, 1, H, B, G, (0, 1, H), (0, G, 1), (0, G, 1), False, dt), 2.0 * B * H * G, (B * H + B * G + H * G) * esz),
         "db": (lambda: capi.check(L.rp_hip_reduce_rows(d_db.ptr, d_dg.ptr, B, G, 0, dt), "reduce_rows"), 0.0, (B * G + G) * esz),
     }
-    for fn, _, _ in ops.values():
+    # With input size = hidden size the host layer issues the two input gradients, and the two weight gradients, as one
+    # launch each over a batch of two: the second matrix of every operand is addressed by its distance from the first.
+    def dist(p, q):
+        return (q.ptr - p.ptr) // esz
+    pairs = {
+        "dx,dh=dg.W^t (pair)": (lambda: capi.gemm(d_dx.ptr, d_dg.ptr, d_wi.ptr, None, 2, B, G, I, (0, G, 1), (dist(d_wi, d_wh), 1, G), (dist(d_dx, d_dh), I, 1), False, dt),
+                                4.0 * B * I * G, 2 * (B * G + I * G + B * I) * esz),
+        "dW=x^t.dg,h^t.dg (pair)": (lambda: capi.gemm(d_dwi.ptr, d_x.ptr, d_dg.ptr, None, 2, I, B, G, (dist(d_x, d_h), 1, I), (0, G, 1), (dist(d_dwi, d_dwh), G, 1), False, dt),
+                                    4.0 * B * I * G, 2 * (B * I + B * G + I * G) * esz),
+    }
+    paired = {k: v for k, v in ops.items() if k in ("gates=x.Wih", "gates+=h.Whh", "cell_fwd", "cell_bwd")}
+    paired.update(pairs)
+    paired["db"] = ops["db"]
+    for fn, _, _ in list(ops.values()) + list(pairs.values()):
         fn()
     out = {}
-    for name, (fn, flops, nbytes) in ops.items():
+    for name, (fn, flops, nbytes) in list(ops.items()) + list(pairs.items()):
         ms = _time_graph(capi, fn, 20, 2)
         out[name] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1)}
-    def step():
-        for fn, _, _ in ops.values():
-            fn()
-    ms = _time_graph(capi, step, 10, 2)
+    def step_of(group):
+        def step():
+            for fn, _, _ in group.values():
+                fn()
+        return step
+    ms = _time_graph(capi, step_of(paired), 10, 2)
     total_bytes = sum(nb for _, _, nb in ops.values())
     out["step_ms"] = round(ms, 4)
     out["step_GB/s"] = round(total_bytes / ms / 1e6, 1)
-    out["launches"] = len(ops)
+    out["launches"] = len(paired)
+    out["step_ms_separate_gradients"] = round(_time_graph(capi, step_of(ops), 10, 2), 4)
+    out["launches_separate_gradients"] = len(ops)
     return out
 
 
@@ -740,6 +759,8 @@ def main():
                     help="run only the conv2d layer's launches in bf16 (for profiling those kernels alone)")
     ap.add_argument("--mlp-only", action="store_true",
                     help="run only the configuration-2 MLP step (C ABI from a HIP graph, eager, and through the drop-in Python API)")
+    ap.add_argument("--lstm-only", action="store_true",
+                    help="time only the LSTM step (per-launch table and whole step), for profiling runs")
     ap.add_argument("--sustain", type=float, default=0.0,
                     help="run the forward 8192^3 bf16 GEMM back to back for this many seconds on --data operands while polling amd-smi "
                          "for shader clock and socket power, and print those figures (evidence for the power-limit reading of the headline)")
@@ -787,6 +808,9 @@ def main():
         return
     if args.attention_only:
         print(json.dumps({"attention_bf16": attention_times(capi, "bf16"), "attention_f32": attention_times(capi, "f32")}))
+        return
+    if args.lstm_only:
+        print(json.dumps({"lstm_step_bf16": lstm_step_times(capi, "bf16"), "lstm_step_f32": lstm_step_times(capi, "f32")}))
         return
     if args.mlp_only:
         out = mlp_step_time(capi)

@@ -103,7 +103,10 @@ int matmul_kernel_device(void* C, const void* A, const void* B, int m, int k, in
  *
  * X_z[i,j] lives at X + z*x_bs + i*x_rs + j*x_cs (strides in ELEMENTS, any
  * sign-free combination: transposed and permuted views are passed as they
- * are and are never copied).  bias is NULL or a dense vector of n elements.
+ * are and are never copied; the batch strides x_bs alone may also be
+ * negative, so that one call can cover separately allocated matrices of one
+ * shape: pass matrix 0 and the distances to matrix 1).  Output matrices must
+ * not overlap.  bias is NULL or a dense vector of n elements.
  * accumulate != 0 adds the product into the existing C (beta = 1).
  * fp16/bf16 accumulate in fp32 and narrow once per reference op in the chain
  * (matmul, then bias add, then accumulation), with the reference's rounding.

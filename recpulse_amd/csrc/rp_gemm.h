@@ -197,7 +197,7 @@ bool pipe32k_takes(const GemmArgs& g);         // and its fp32 twin
 int launch_pipe32k(const GemmArgs& g);
 int launch_gemm_segmented_b(const GemmArgs& g, int dtype);
 int launch_linear_backward_tiny(const GemmArgs& gx, const GemmArgs& gw, void* db, const void* dy, int rows, int cols, int accumulate_db);
-// adds k-split partials [nsplit][part_rows][n] (fp32, rows beyond g.m unused) in split order and runs the epilogue into C
+// adds k-split partials [g.batch][nsplit][part_rows][n] (fp32, rows beyond g.m unused) in split order and runs the epilogue into C
 int launch_splitk_combine(const GemmArgs& g, const float* partials, int nsplit, int part_rows, int dtype);
 
 }  // namespace rp

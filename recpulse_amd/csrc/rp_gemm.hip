@@ -83,12 +83,15 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     // 16-bit, few rows, deep k: split k over many blocks so that B streams at HBM speed (output columns in whole 8s).
     // Up to 32 rows always; up to SKINNY_MAX_ROWS when the 128 x 128 tiles of the output would occupy under half the
     // CUs and k is deep enough to be worth a second launch for the partial sums (64 x 1024 x 4096: 6.6 us on 64 x 64 tiles
-    // in one launch against 9.4 us split; 64 x 4096 x 1024: 16.4 against 9.1).
-    const long long tiles128_16 = (long long)((m + 127) / 128) * ((n + 127) / 128);
-    if (is16 && mfma_ok && batch == 1 && (m <= 32 || (m <= SKINNY_MAX_ROWS && tiles128_16 < cu_tiles() / 2 && k >= 2048)) && n % 8 == 0 && n >= 256 && k >= 1024 &&
+    // in one launch against 9.4 us split; 64 x 4096 x 1024: 16.4 against 9.1).  A short batch of such products is
+    // split the same way while its tiles together stay under half the CUs.
+    const long long tiles128_16 = (long long)((m + 127) / 128) * ((n + 127) / 128) * batch;
+    const bool few_rows = batch == 1 ? (m <= 32 || (m <= SKINNY_MAX_ROWS && tiles128_16 < cu_tiles() / 2 && k >= 2048))
+                                     : (m <= SKINNY_MAX_ROWS && tiles128_16 < cu_tiles() / 2 && k >= 2048);
+    if (is16 && mfma_ok && few_rows && n % 8 == 0 && n >= 256 && k >= 1024 &&
         (long long)k * n >= (1ll << 22)) {
         p.fam = FAM_MFMA16_SKINNY; p.bm = 32; p.bn = 128; p.edge = true; p.a_mc = !a_kc; p.b_mc = b_mc;
-        p.name = (!p.a_mc && p.b_mc && m <= 16) ? "mfma16_stream_32x256" : "mfma16_skinny_32x128";
+        p.name = (batch == 1 && !p.a_mc && p.b_mc && m <= 16) ? "mfma16_stream_32x256" : "mfma16_skinny_32x128";
         return p;
     }
     // VALU skinny: few rows, row-major B, enough columns and depth to be worth streaming
@@ -319,8 +322,10 @@ int rp_hip_gemm_strided_batched(void* C, const void* A, const void* B, const voi
         return -1;
     }
     if (!dtype_size(dtype)) { set_error("rp_hip_gemm_strided_batched: unsupported dtype %d", dtype); return -1; }
-    if (a_rs < 0 || a_cs < 0 || b_rs < 0 || b_cs < 0 || c_rs < 0 || c_cs < 0 || a_bs < 0 || b_bs < 0 || c_bs < 0) {
-        set_error("rp_hip_gemm_strided_batched: negative stride");
+    // (Batch strides may have any sign: matrix z of an operand starts z strides from matrix 0, which lets one launch
+    // cover separately allocated matrices of equal shape.  Row and column strides address inside a matrix.)
+    if (a_rs < 0 || a_cs < 0 || b_rs < 0 || b_cs < 0 || c_rs < 0 || c_cs < 0) {
+        set_error("rp_hip_gemm_strided_batched: negative row or column stride");
         return -1;
     }
     // the batch rides on a grid axis that holds at most 65535 blocks: longer batches go in chunks

@@ -245,8 +245,8 @@ __global__ void __launch_bounds__(256) gemm_splitk_combine_kernel(GemmArgs g, co
     if (item >= g.m * quads) return;
     const int r = item / quads, c0 = (item - r * quads) * 4;
     f32x4_t sum = {0.f, 0.f, 0.f, 0.f};
-    const float* q = partials + (long long)r * g.n + c0;
     const long long split_stride = (long long)part_rows * g.n;
+    const float* q = partials + (long long)blockIdx.y * nsplit * split_stride + (long long)r * g.n + c0;      // matrix blockIdx.y of the batch
     int s = 0;
     for (; s + 8 <= nsplit; s += 8) {
         f32x4_t v[8];
@@ -256,7 +256,7 @@ __global__ void __launch_bounds__(256) gemm_splitk_combine_kernel(GemmArgs g, co
         for (int u = 0; u < 8; u++) sum += v[u];
     }
     for (; s < nsplit; s++) sum += *(const f32x4_t*)(q + s * split_stride);
-    T* C = (T*)g.C;
+    T* C = (T*)g.C + (long long)blockIdx.y * g.c_bs;
     const T* bias = (const T*)g.bias;
     const bool has_bias = bias != nullptr, accum = g.accumulate != 0;
 #pragma unroll
@@ -301,8 +301,8 @@ __global__ void __launch_bounds__(256) gemm_splitk_combine_scalar_kernel(GemmArg
     const int item = blockIdx.x * 256 + threadIdx.x;
     if (item >= g.m * g.n) return;
     const int r = item / g.n, c = item - r * g.n;
-    const float* q = partials + (long long)r * g.n + c;
     const long long split_stride = (long long)part_rows * g.n;
+    const float* q = partials + (long long)blockIdx.y * nsplit * split_stride + (long long)r * g.n + c;
     float sum = 0.f;
     int s = 0;
     for (; s + 8 <= nsplit; s += 8) {
@@ -313,7 +313,7 @@ __global__ void __launch_bounds__(256) gemm_splitk_combine_scalar_kernel(GemmArg
         for (int u = 0; u < 8; u++) sum += v[u];
     }
     for (; s < nsplit; s++) sum += q[s * split_stride];
-    T* C = (T*)g.C;
+    T* C = (T*)g.C + (long long)blockIdx.y * g.c_bs;
     const T* bias = (const T*)g.bias;
     const bool has_bias = bias != nullptr, accum = g.accumulate != 0;
     T* p = C + (long long)r * g.c_rs + (long long)c * g.c_cs;
@@ -323,7 +323,7 @@ __global__ void __launch_bounds__(256) gemm_splitk_combine_scalar_kernel(GemmArg
 
 int launch_splitk_combine(const GemmArgs& g, const float* partials, int nsplit, int part_rows, int dtype) {
     if (g.n % 4) {
-        dim3 sgrid((g.m * g.n + 255) / 256);
+        dim3 sgrid((g.m * g.n + 255) / 256, g.batch);
         switch (dtype) {
             case RP_DTYPE_FLOAT32:  hipLaunchKernelGGL(gemm_splitk_combine_scalar_kernel<float>, sgrid, dim3(256), 0, current_stream(), g, partials, nsplit, part_rows); break;
             case RP_DTYPE_FLOAT16:  hipLaunchKernelGGL(gemm_splitk_combine_scalar_kernel<f16_t>, sgrid, dim3(256), 0, current_stream(), g, partials, nsplit, part_rows); break;
@@ -333,7 +333,7 @@ int launch_splitk_combine(const GemmArgs& g, const float* partials, int nsplit, 
         return check_launch("gemm_splitk_combine_scalar_kernel") ? 0 : -1;
     }
     int items = g.m * (g.n / 4);
-    dim3 grid((items + 255) / 256);
+    dim3 grid((items + 255) / 256, g.batch);
     switch (dtype) {
         case RP_DTYPE_FLOAT32:  hipLaunchKernelGGL(gemm_splitk_combine_kernel<float>, grid, dim3(256), 0, current_stream(), g, partials, nsplit, part_rows); break;
         case RP_DTYPE_FLOAT16:  hipLaunchKernelGGL(gemm_splitk_combine_kernel<f16_t>, grid, dim3(256), 0, current_stream(), g, partials, nsplit, part_rows); break;

@@ -13,7 +13,8 @@ namespace rp {
 // Block tile BM x BN, k slab 64, 256 threads = 4 waves (one per SIMD) in a
 // WGM x (4/WGM) grid, each wave owning a (BM/WGM) x (BN/(4/WGM)) patch of
 // 32x32x16 MFMA tiles.  With SPLITK the grid's z axis splits k: every block
-// writes its fp32 partial tile to a workspace and a combine kernel finishes.
+// writes its fp32 partial tile to a workspace [matrix][split][m][n] and a
+// combine kernel finishes.
 //
 // Software pipeline, per slab s (4 k-steps of 16):
 //   k-steps 0-2  MFMAs on fragments(ks) | read fragments(ks+1) | a third of: registers of slab s+1 -> other
@@ -587,7 +588,7 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
                 if (EDGE && gm >= g.m) break;
                 // n is a multiple of 8 on this path, so the 8 columns are all in or all out
                 if (!EDGE || gn + 8 <= g.n) {
-                    float* prow = partials + ((long long)blockIdx.z * g.m + gm) * g.n + gn;
+                    float* prow = partials + (((long long)z * gridDim.z + blockIdx.z) * g.m + gm) * g.n + gn;
                     *(f32x4_t*)prow = *(const f32x4_t*)(region + r * EP + ecol);
                     *(f32x4_t*)(prow + 4) = *(const f32x4_t*)(region + r * EP + ecol + 4);
                 }
@@ -597,7 +598,7 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     }   // tiles of this workgroup
 }
 
-// Launch one instantiation.  nsplit > 1 selects the split-k variant: partials must hold nsplit * m * n floats.
+// Launch one instantiation.  nsplit > 1 selects the split-k variant: partials must hold batch * nsplit * m * n floats.
 template <typename T, int BM, int BN, int WGM, bool A_MC, bool B_MC, bool EDGE, bool SPLITK>
 static int m16_launch(const GemmArgs& g, float* partials, int nsplit, int k_per_split) {
     int tiles_m = (g.m + BM - 1) / BM, tiles_n = (g.n + BN - 1) / BN;

@@ -42,7 +42,7 @@ namespace rp {
 // column group 8i + x are given slots of XCD x.  When the host has verified that
 // rule on the device (`local`), the partials and the arrival count never leave
 // that XCD's L2: plain stores (complete when the L2 has them), an atomic that the
-// L2 executes, and loads behind an invalidate of the finishing CU's vector cache.
+// L2 executes, and plain loads (the finishing CU's vector cache holds none of them yet).
 // Otherwise they are exchanged at device scope (written through to memory and
 // read back from there), which costs about 1.5 us more per launch.
 // ============================================================================
@@ -299,9 +299,9 @@ static int launch_skinny16_t(const GemmArgs& g, const Plan& p, float* partials, 
 
 int launch_mfma16_skinny(const GemmArgs& g, const Plan& p, int dtype) {
     if (dtype != RP_DTYPE_BFLOAT16 && dtype != RP_DTYPE_FLOAT16) { set_error("mfma16 skinny GEMM: unsupported dtype %d", dtype); return -1; }
-    if (!p.a_mc && p.b_mc && g.m <= SS_MAX_M && !path_disabled("stream16")) return launch_stream16(g, dtype);
+    if (g.batch == 1 && !p.a_mc && p.b_mc && g.m <= SS_MAX_M && !path_disabled("stream16")) return launch_stream16(g, dtype);
     constexpr int BN = 128;
-    const int tiles = ((g.n + BN - 1) / BN) * ((g.m + 31) / 32);
+    const int tiles = ((g.n + BN - 1) / BN) * ((g.m + 31) / 32) * g.batch;
     // about three blocks per CU in flight, each split at least four slabs deep
     int nsplit = (768 + tiles - 1) / tiles;
     int max_split = g.k / (4 * M16_BK) > 0 ? g.k / (4 * M16_BK) : 1;
@@ -309,7 +309,7 @@ int launch_mfma16_skinny(const GemmArgs& g, const Plan& p, int dtype) {
     int k_per_split = ((g.k + nsplit - 1) / nsplit + M16_BK - 1) / M16_BK * M16_BK;
     nsplit = (g.k + k_per_split - 1) / k_per_split;
     void* ws = nullptr;
-    if (gemm_workspace(&ws, (size_t)nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
+    if (gemm_workspace(&ws, (size_t)g.batch * nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
     int rc;
     if (dtype == RP_DTYPE_BFLOAT16) rc = launch_skinny16_t<bf16_t>(g, p, (float*)ws, nsplit, k_per_split);
     else rc = launch_skinny16_t<f16_t>(g, p, (float*)ws, nsplit, k_per_split);

@@ -272,7 +272,7 @@ __global__ void __launch_bounds__(256, 2) gemm_mfmaw_kernel(GemmArgs g, int tile
             memcpy(vals, &raw, 16);
             if constexpr (SPLITK) {
                 // fp32 partial tile [split][m][n]; n is a multiple of 4 on this path, so the vector is wholly in or out
-                if (!EDGE || gn + V <= g.n) *(uint4*)(partials + ((long long)blockIdx.z * g.m + gm) * g.n + gn) = raw;
+                if (!EDGE || gn + V <= g.n) *(uint4*)(partials + (((long long)z * gridDim.z + blockIdx.z) * g.m + gm) * g.n + gn) = raw;
                 continue;
             }
             T* crow = C + (long long)gm * g.c_rs;
@@ -475,11 +475,12 @@ static int launch_mfmaw_layout(const GemmArgs& g, const Plan& p, float* partials
 template <typename T>
 static int launch_mfmaw_t(const GemmArgs& g, const Plan& p) {
     // Small outputs with a deep k leave most CUs idle: split k so that about 256 blocks run (each split at
-    // least two slabs deep), and add the partials in split order afterwards.  fp32 only, one matrix at a time.
+    // least two slabs deep), and add the partials [matrix][split][m][n] in split order afterwards.  fp32 only; a batch
+    // is split the same way while all its tiles together leave CUs idle.
     int nsplit = 1, k_per_split = 0;
     constexpr int BK = mfmaw_cfg<T>::BK;
-    if (sizeof(T) == 4 && g.batch == 1 && p.bm == 64 && g.n % 4 == 0 && g.seg_k == 0 && g.seg_n == 0 && g.c_fold_from == 0 && !g.bias_by_row) {   // (segments and the folded store: never split)
-        int tiles = ((g.m + 63) / 64) * ((g.n + 63) / 64);
+    if (sizeof(T) == 4 && p.bm == 64 && g.n % 4 == 0 && g.seg_k == 0 && g.seg_n == 0 && g.c_fold_from == 0 && !g.bias_by_row) {   // (segments and the folded store: never split)
+        int tiles = ((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch;
         int want = (256 + tiles - 1) / tiles, deep = g.k / (2 * BK);
         nsplit = want < deep ? want : deep;
         if (nsplit > 1) {
@@ -489,7 +490,7 @@ static int launch_mfmaw_t(const GemmArgs& g, const Plan& p) {
         if (nsplit < 2) nsplit = 1;
     }
     void* ws = nullptr;
-    if (nsplit > 1 && gemm_workspace(&ws, (size_t)nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
+    if (nsplit > 1 && gemm_workspace(&ws, (size_t)g.batch * nsplit * g.m * g.n * sizeof(float)) != 0) return -1;
     int rc = (p.bm == 128) ? launch_mfmaw_layout<T, 128, 128>(g, p, (float*)ws, nsplit, k_per_split)
                            : launch_mfmaw_layout<T, 64, 64>(g, p, (float*)ws, nsplit, k_per_split);
     if (rc == 0 && nsplit > 1) rc = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, traits<T>::code);

@@ -740,6 +740,56 @@ void gemm_grad(Tensor* target, Tensor* a, bool a_t, Tensor* b, bool b_t) {
     free_tensor(aa); free_tensor(bb);
 }
 
+// Two operand gradients of equal shapes whose products agree in every stride (the input half and the recurrent half
+// of a cell step with input size = hidden size) as ONE launch over a batch of two: matrix 1 of each operand is
+// addressed by its distance from matrix 0, which the strided entry accepts with either sign.  Each matrix gets the
+// roundings of a gemm_grad call of its own (a k split may add its fp32 partial sums in different groups).  False when
+// the pair does not qualify (nothing was launched).
+bool same_matrix_layout(const Tensor* p, const Tensor* q) {
+    return p->ndim == 2 && q->ndim == 2 && p->dtype == q->dtype && p->device_id == q->device_id && p->shape[0] == q->shape[0] &&
+           p->shape[1] == q->shape[1] && p->strides[0] == q->strides[0] && p->strides[1] == q->strides[1];
+}
+
+bool element_distance(const Tensor* from, const Tensor* to, long long* out) {
+    const long long bytes = (const char*)to->data - (const char*)from->data, esz = (long long)dtype_size(from->dtype);
+    if (bytes % esz) return false;
+    *out = bytes / esz;
+    return true;
+}
+
+bool gemm_grad_pair(Tensor* t1, Tensor* a1, Tensor* b1, Tensor* t2, Tensor* a2, Tensor* b2, bool a_t, bool b_t) {
+    if (t1 == t2 || t1->device_id < 0 || !same_matrix_layout(a1, a2) || !same_matrix_layout(b1, b2) || a1->dtype != b1->dtype || a1->dtype != t1->dtype ||
+        t1->ndim != 2 || t2->ndim != 2 || t1->shape[0] != t2->shape[0] || t1->shape[1] != t2->shape[1] || t1->dtype != t2->dtype ||
+        a1->device_id != t1->device_id || b1->device_id != t1->device_id || t2->device_id != t1->device_id)
+        return false;
+    Meta* m1 = ensure_meta(t1); Meta* m2 = ensure_meta(t2);
+    const bool into1 = m1->grad && rp_is_contiguous(m1->grad), into2 = m2->grad && rp_is_contiguous(m2->grad);
+    if (into1 != into2 || (!into1 && (m1->grad || m2->grad))) return false;          // both accumulate in place, or both are new
+    Tensor* g1 = into1 ? m1->grad : empty_tensor(t1->dtype, t1->device_id, 2, t1->shape);
+    Tensor* g2 = into2 ? m2->grad : empty_tensor(t2->dtype, t2->device_id, 2, t2->shape);
+    long long a_bs = 0, b_bs = 0, c_bs = 0;
+    bool launched = false;
+    if (g1 && g2 && g1 != g2 && element_distance(a1, a2, &a_bs) && element_distance(b1, b2, &b_bs) && element_distance(g1, g2, &c_bs) && c_bs != 0 &&
+        on_device(t1->device_id)) {
+        long long a_rs = a1->strides[0], a_cs = a1->strides[1], b_rs = b1->strides[0], b_cs = b1->strides[1];
+        if (a_t) std::swap(a_rs, a_cs);
+        if (b_t) std::swap(b_rs, b_cs);
+        const int m = a_t ? a1->shape[1] : a1->shape[0], k = a_t ? a1->shape[0] : a1->shape[1], n = b_t ? b1->shape[0] : b1->shape[1];
+        launched = true;
+        if (rp_hip_gemm_strided_batched(g1->data, a1->data, b1->data, nullptr, 2, m, k, n, a_bs, a_rs, a_cs, b_bs, b_rs, b_cs,
+                                        c_bs, g1->strides[0], g1->strides[1], into1 ? 1 : 0, t1->dtype) != 0) {
+            dev_fail("matmul backward (pair)");
+            if (!into1) { free_tensor(g1); free_tensor(g2); }
+        } else if (!into1) {
+            accumulate_grad(t1, g1);
+            accumulate_grad(t2, g2);
+        }
+    } else if (!into1) {
+        free_tensor(g1); free_tensor(g2);
+    }
+    return launched;
+}
+
 // dA = dC · Bᵀ and dB = Aᵀ · dC (reference ops/ops.c:6759-6814), with the transposes passed as stride views
 // and accumulation done by the GEMM itself instead of rp_transpose + rp_contiguous + rp_matmul + rp_add.
 void backward_matmul_fn(GradFn* self, Tensor* grad_output) {
@@ -1138,6 +1188,24 @@ void bias_grad(Tensor* bias, Tensor* dgates) {
     if (bias && needs_grad(bias)) accumulate_grad(bias, reduce_grad_to_shape(dgates, bias->ndim, bias->shape));
 }
 
+// The four products of a cell's backward: dx = dgi · W_ihᵀ, dh = dgh · W_hhᵀ, dW_ih = xᵀ · dgi, dW_hh = hᵀ · dgh
+// (h_grad_to: the tensor that receives dh; null when the caller has already issued that product; h_operand: the
+// recurrent input when it differs from h_grad_to).  The two input gradients, and the two weight gradients, go out as
+// one launch each where their shapes agree.
+void cell_gemm_grads(Tensor* x, Tensor* h_grad_to, Tensor* w_ih, Tensor* w_hh, Tensor* dgi, Tensor* dgh, Tensor* h_operand = nullptr) {
+    Tensor* h = h_operand ? h_operand : h_grad_to;
+    const bool dx = needs_grad(x), dh = h_grad_to && needs_grad(h_grad_to);
+    if (!(dx && dh && gemm_grad_pair(x, dgi, w_ih, h_grad_to, dgh, w_hh, false, true))) {
+        if (dx) gemm_grad(x, dgi, false, w_ih, true);
+        if (dh) gemm_grad(h_grad_to, dgh, false, w_hh, true);
+    }
+    const bool dwi = needs_grad(w_ih), dwh = needs_grad(w_hh);
+    if (!(dwi && dwh && gemm_grad_pair(w_ih, x, dgi, w_hh, h, dgh, true, false))) {
+        if (dwi) gemm_grad(w_ih, x, true, dgi, false);
+        if (dwh) gemm_grad(w_hh, h, true, dgh, false);
+    }
+}
+
 void backward_lstm_cell_fn(GradFn* self, Tensor* grad_output) {
     Tensor* x = self->inputs[0]; Tensor* h = self->inputs[1]; Tensor* c = self->inputs[2];
     Tensor* w_ih = self->inputs[3]; Tensor* w_hh = self->inputs[4]; Tensor* b_ih = self->inputs[5]; Tensor* b_hh = self->inputs[6];
@@ -1153,10 +1221,7 @@ void backward_lstm_cell_fn(GradFn* self, Tensor* grad_output) {
               rp_hip_lstm_cell_backward(dgates->data, dc->data, dhc->data, sv->act->data, hcd->data, sv->state->data, sv->state->strides[0], batch, hidden, x->dtype) == 0;
     if (!ok) dev_fail("op_lstm_cell backward");
     if (ok && needs_grad(c)) { accumulate_grad(c, dc); dc = nullptr; }
-    if (ok && needs_grad(x)) gemm_grad(x, dgates, false, w_ih, true);
-    if (ok && needs_grad(h)) gemm_grad(h, dgates, false, w_hh, true);
-    if (ok && needs_grad(w_ih)) gemm_grad(w_ih, x, true, dgates, false);
-    if (ok && needs_grad(w_hh)) gemm_grad(w_hh, h, true, dgates, false);
+    if (ok) cell_gemm_grads(x, h, w_ih, w_hh, dgates, dgates);
     if (ok) { bias_grad(b_ih, dgates); bias_grad(b_hh, dgates); }
     free_tensor(dhc); free_tensor(hcd); free_tensor(dgates); free_tensor(dc);
 }
@@ -1179,9 +1244,7 @@ void backward_gru_cell_fn(GradFn* self, Tensor* grad_output) {
         accumulate_grad(h, dh_direct); dh_direct = nullptr;           // dh * z, then the part through gh on top of it
         gemm_grad(h, dgh, false, w_hh, true);
     }
-    if (ok && needs_grad(x)) gemm_grad(x, dgi, false, w_ih, true);
-    if (ok && needs_grad(w_ih)) gemm_grad(w_ih, x, true, dgi, false);
-    if (ok && needs_grad(w_hh)) gemm_grad(w_hh, h, true, dgh, false);
+    if (ok) cell_gemm_grads(x, nullptr, w_ih, w_hh, dgi, dgh, h);
     if (ok) { bias_grad(b_ih, dgi); bias_grad(b_hh, dgh); }
     free_tensor(dh); free_tensor(dgi); free_tensor(dgh); free_tensor(dh_direct);
 }

@@ -12,7 +12,7 @@ import pytest
 
 import oracle
 from recpulse_amd import capi
-from devhelp import Dev, ALL, BF16, F16, F32, F64, NAMES, device_gemm, f64_gemm, oracle_gemm, rand_storage, tol
+from devhelp import Dev, ALL, BF16, F16, F32, F64, NAMES, device_gemm, elem_strides, f64_gemm, oracle_gemm, rand_storage, tol
 
 pytestmark = pytest.mark.gpu
 GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")))
@@ -304,6 +304,50 @@ def test_streaming_rows_finish_repeats_bit_for_bit_over_hundreds_of_launches(m):
     assert oracle.rel_err(oracle.to_f64(first, dt), want) <= tol(dt, k)
 
 
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_tiled_rows_split_k_ragged(layout):
+    """More rows or another operand layout: the tiled kernel splits k across the grid and a second kernel adds the
+    partial tiles in split order.  Ragged k (a partial last slab, splits of unequal length) and n (a partial last
+    strip, a number of strips that is not a multiple of 8), several row tiles, bias and accumulation; repeated
+    launches reproduce the first bit for bit."""
+    rng = np.random.default_rng(43)
+    for dt, m, k, n in [(BF16, 32, 8192, 2048), (F16, 24, 4104, 1288), (BF16, 17, 1032, 4096), (F16, 104, 4160, 1160), (BF16, 8, 2048, 2048)]:
+        if (layout == "nn" and m <= 16) or (layout[0] == "t" and m % 8):
+            continue                                   # the streaming kernel's case; a transposed A needs whole 16-byte vectors along m
+        a, b = _operands(rng, m, k, n, dt, layout)
+        a_st = (a.strides[0] // 2, a.strides[1] // 2); b_st = (b.strides[0] // 2, b.strides[1] // 2)
+        assert capi.gemm_kernel_name(1, m, k, n, a_st, b_st, (n, 1), dt) == "mfma16_skinny_32x128"
+        bias = rand_storage(rng, (n,), dt); c0 = rand_storage(rng, (m, n), dt)
+        first = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)
+        _check(first, a, b, dt, k, bias=bias, c_init=c0, accumulate=True)
+        for _ in range(10):
+            assert np.array_equal(first, device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True))
+    # integer data is exact in fp32 whatever the split: bit-equal to the oracle
+    a, b = _operands(rng, 32, 4096, 1024, BF16, layout)
+    a[...] = oracle.to_storage(rng.integers(-2, 3, a.shape).astype(np.float64), BF16)
+    b[...] = oracle.to_storage(rng.integers(-2, 3, b.shape).astype(np.float64), BF16)
+    assert np.array_equal(device_gemm(a, b, BF16), oracle_gemm(a, b, BF16))
+
+
+def test_tiled_rows_repeat_bit_for_bit_over_hundreds_of_launches():
+    """The tiled k-split kernel and its combine kernel share one workspace from the pool across back-to-back launches:
+    300 launches without synchronisation in between leave the bits of the first."""
+    rng = np.random.default_rng(44)
+    m, k, n, dt = 32, 8192, 8192, BF16
+    a = rand_storage(rng, (m, k), dt); b = rand_storage(rng, (k, n), dt)
+    assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == "mfma16_skinny_32x128"
+    da, db = capi.DeviceBuffer.from_numpy(a), capi.DeviceBuffer.from_numpy(b)
+    outs = [capi.DeviceBuffer(m * n * 2) for _ in range(300)]
+    for dc in outs:
+        capi.gemm(dc.ptr, da.ptr, db.ptr, None, 1, m, k, n, (0, k, 1), (0, n, 1), (0, n, 1), False, dt)
+    capi.synchronize()
+    first = outs[0].to_numpy(np.uint16, (m, n))
+    for i, dc in enumerate(outs[1:], 1):
+        assert np.array_equal(first, dc.to_numpy(np.uint16, (m, n))), f"launch {i} differs from launch 0"
+    want = oracle.to_f64(a, dt) @ oracle.to_f64(b, dt)
+    assert oracle.rel_err(oracle.to_f64(first, dt), want) <= tol(dt, k)
+
+
 def test_streaming_rows_both_exchanges_give_the_same_bits(tmp_path):
     """The k-split finish goes through the XCD's own L2 when workgroup placement was verified, and through memory at
     device scope otherwise (RP_HIP_DISABLE=l2_exchange forces that, read once per process): a child process computes
@@ -316,7 +360,7 @@ def test_streaming_rows_both_exchanges_give_the_same_bits(tmp_path):
         "from devhelp import device_gemm, rand_storage, BF16, F16\n"
         "rng = np.random.default_rng(42)\n"
         "out = {}\n"
-        "for i, (dt, m, k, n) in enumerate([(BF16, 1, 8192, 8192), (BF16, 8, 8192, 8192), (F16, 16, 4104, 1288), (BF16, 11, 2048, 2048)]):\n"
+        "for i, (dt, m, k, n) in enumerate([(BF16, 1, 8192, 8192), (BF16, 8, 8192, 8192), (F16, 16, 4104, 1288), (BF16, 11, 2048, 2048), (BF16, 32, 8192, 8192), (F16, 27, 4104, 1288)]):\n"
         "    a = rand_storage(rng, (m, k), dt); b = rand_storage(rng, (k, n), dt)\n"
         "    out[str(i)] = device_gemm(a, b, dt)\n"
         "np.savez(sys.argv[1], **out)\n"
@@ -329,6 +373,51 @@ def test_streaming_rows_both_exchanges_give_the_same_bits(tmp_path):
         results.append(np.load(path))
     for key in results[0].files:
         assert np.array_equal(results[0][key], results[1][key]), f"case {key}: the two exchanges disagree"
+
+
+@pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
+def test_pair_of_separately_allocated_matrices_in_one_launch(dt):
+    """Batch strides of either sign: a batch of two whose second matrices are separate allocations, addressed by their
+    distances from the first (how a recurrent cell's backward issues its input-side and recurrent-side products
+    together).  Every matrix must equal the oracle's product of its own operands, whichever of the two allocations
+    lies higher in memory; the deep-k shape takes the k-split kernel with a batch, the short-k one the resident kernel."""
+    rng = np.random.default_rng(45)
+    es = np.dtype(capi.NP_STORAGE[dt]).itemsize
+    cases = [(64, 4096, 1024, "nt"), (1024, 64, 4096, "tn"), (33, 70, 65, "nn"), (64, 2048, 512, "nn")]
+    if dt == F64:
+        cases = cases[2:]
+    for m, k, n, layout in cases:
+        mats = []
+        for _ in range(2):
+            a, b = _operands(rng, m, k, n, dt, layout)
+            c0 = rand_storage(rng, (m, n), dt)
+            mats.append((a, b, c0))
+        for accumulate in (False, True):
+            for order in ((0, 1), (1, 0)):
+                # allocations in the given order, so that both signs of every distance occur
+                bufs = {}
+                for i in order:
+                    a, b, c0 = mats[i]
+                    # (an operand view starts at its buffer's first element: uploading a dense copy of the view's
+                    # transpose-free form and passing the view's strides addresses the same elements)
+                    bufs[i] = (capi.DeviceBuffer.from_numpy(np.ascontiguousarray(a if layout[0] == "n" else a.T)),
+                               capi.DeviceBuffer.from_numpy(np.ascontiguousarray(b if layout[1] == "n" else b.T)),
+                               capi.DeviceBuffer.from_numpy(c0))
+                a0, b0, _ = mats[0]
+                dist = [(bufs[1][j].ptr - bufs[0][j].ptr) for j in range(3)]
+                assert all(d % es == 0 for d in dist)
+                a_st = (dist[0] // es,) + tuple(elem_strides(a0)); b_st = (dist[1] // es,) + tuple(elem_strides(b0))
+                capi.gemm(bufs[0][2].ptr, bufs[0][0].ptr, bufs[0][1].ptr, None, 2, m, k, n, a_st, b_st, (dist[2] // es, n, 1), accumulate, dt)
+                capi.synchronize()
+                if dt in (BF16, F16) and k >= 2048 and k * n >= 1 << 22:
+                    assert capi.last_gemm_kernel() == "mfma16_skinny_32x128"
+                for i in (0, 1):
+                    a, b, c0 = mats[i]
+                    got = bufs[i][2].to_numpy(capi.NP_STORAGE[dt], (m, n))
+                    _check(got, a, b, dt, k, c_init=c0 if accumulate else None, accumulate=accumulate)
+                for i in (0, 1):
+                    for d in bufs[i]:
+                        d.free()
 
 
 @pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])

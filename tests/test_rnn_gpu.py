@@ -105,7 +105,7 @@ def _seed_loss(outs, ups, dt):
 
 
 @pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
-@pytest.mark.parametrize("dims", [(5, 7, 8), (32, 64, 128), (3, 40, 24)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("dims", [(5, 7, 8), (32, 64, 128), (3, 40, 24), (16, 64, 64), (64, 512, 512)], ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("bias", [True, False], ids=["bias", "nobias"])
 def test_lstm_cell_step(dt, dims, bias):
     B, I, H = dims
@@ -134,7 +134,7 @@ def test_lstm_cell_step(dt, dims, bias):
 
 
 @pytest.mark.parametrize("dt", ALL, ids=lambda d: NAMES[d])
-@pytest.mark.parametrize("dims", [(5, 7, 8), (32, 64, 128), (3, 40, 24)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("dims", [(5, 7, 8), (32, 64, 128), (3, 40, 24), (16, 64, 64), (64, 512, 512)], ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("bias", [True, False], ids=["bias", "nobias"])
 def test_gru_cell_step(dt, dims, bias):
     B, I, H = dims
