@@ -159,13 +159,16 @@ def test_gru_cell_step(dt, dims, bias):
 
 
 @pytest.mark.parametrize("kind", ["lstm", "gru"])
+@pytest.mark.parametrize("sizes", [(10, 16), (16, 16)], ids=["in10_hid16", "in16_hid16"])
 @pytest.mark.parametrize("dt,bound", [(F64, 1e-11), (F32, 1e-4), (BF16, 5e-2)], ids=["f64", "f32", "bf16"])
-def test_unrolled_sequence_vs_torch(kind, dt, bound):
+def test_unrolled_sequence_vs_torch(kind, dt, bound, sizes):
     """Six time steps through the module (state fed back as views of the packed output for the LSTM), loss on every
-    step's h: forward values and every parameter gradient against torch's cell in float64."""
+    step's h: forward values and every parameter gradient against torch's cell in float64.  With input size = hidden
+    size the backward issues its gradient products in pairs, from the second step on accumulating into the weights'
+    existing gradients."""
     import torch
     rng = np.random.default_rng(104)
-    B, I, H, steps = 4, 10, 16, 6
+    B, (I, H), steps = 4, sizes, 6
     rp.manual_seed(5)
     cell = (LSTMCell if kind == "lstm" else GRUCell)(I, H).to(device="cuda", dtype=DT_NAME[dt])
     for b in (cell.bias_ih, cell.bias_hh):
