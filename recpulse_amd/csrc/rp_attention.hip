@@ -72,7 +72,7 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_fwd16_kernel(A
     // Q^T as a B operand: lane (h, c) holds d = 16*ks + 8h .. +7 of query row q0 + c (zero beyond sq)
     const char* q_end = (const char*)(Q + ((long long)(g.sq - 1) * g.q_rs + D));
     const char* q_base = (const char*)(Q + (long long)q0 * g.q_rs);
-    const __amdgpu_buffer_rsrc_t q_rsrc = m16_rsrc(q_base, q0 < g.sq ? (long long)(q_end - q_base) : 0);
+    const __amdgpu_buffer_rsrc_t q_rsrc = buffer_rsrc(q_base, q0 < g.sq ? (long long)(q_end - q_base) : 0);
     s16x8_t qf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ks++)
@@ -85,12 +85,12 @@ __global__ void __launch_bounds__(256, D <= 64 ? 3 : 1) attention_fwd16_kernel(A
     const char* v_end = (const char*)(V + ((long long)(g.sk - 1) * g.v_rs + D));
     auto load_blk = [&](u32x4_t (&r)[VPIECES], const uint16_t* M, long long rs, const char* end, int kb) {
         const char* mp = (const char*)(M + (long long)kb * rs);
-        const __amdgpu_buffer_rsrc_t rsrc = m16_rsrc(mp, kb < g.sk ? (long long)(end - mp) : 0);
+        const __amdgpu_buffer_rsrc_t rsrc = buffer_rsrc(mp, kb < g.sk ? (long long)(end - mp) : 0);
 #pragma unroll
         for (int i = 0; i < VPIECES; i++) {
             const int id = threadIdx.x + 256 * i, key = id / (D / 8), d8 = (id % (D / 8)) * 8;
             const bool live = AT_KEYS * D / 8 >= 256 || id < AT_KEYS * D / 8;
-            r[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, live ? (int)(((long long)key * rs + d8) * 2) : (int)M16_OOB, 0, 0);
+            r[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, live ? (int)(((long long)key * rs + d8) * 2) : (int)BUFFER_OOB, 0, 0);
         }
     };
     auto load_v = [&](u32x4_t (&vr)[VPIECES], int kb) { load_blk(vr, V, g.v_rs, v_end, kb); };
@@ -256,12 +256,12 @@ struct AttnBlock {
     static constexpr int PIECES = AT_KEYS * D / 8 / 256 > 0 ? AT_KEYS * D / 8 / 256 : 1;
     static __device__ __forceinline__ void load(u32x4_t (&r)[PIECES], const uint16_t* M, long long rs, int row0, int rows, const char* end) {
         const char* p = (const char*)(M + (long long)row0 * rs);
-        const __amdgpu_buffer_rsrc_t rsrc = m16_rsrc(p, row0 < rows ? (long long)(end - p) : 0);
+        const __amdgpu_buffer_rsrc_t rsrc = buffer_rsrc(p, row0 < rows ? (long long)(end - p) : 0);
 #pragma unroll
         for (int i = 0; i < PIECES; i++) {
             const int id = threadIdx.x + 256 * i, row = id / (D / 8), d8 = (id % (D / 8)) * 8;
             const bool live = AT_KEYS * D / 8 >= 256 || id < AT_KEYS * D / 8;
-            r[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, live ? (int)(((long long)row * rs + d8) * 2) : (int)M16_OOB, 0, 0);
+            r[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, live ? (int)(((long long)row * rs + d8) * 2) : (int)BUFFER_OOB, 0, 0);
         }
     }
     static __device__ __forceinline__ void store(const u32x4_t (&r)[PIECES], uint16_t* stage) {
@@ -306,7 +306,7 @@ struct AttnBlock {
 template <int KS>
 __device__ __forceinline__ void attn_load_rows(s16x8_t (&f)[KS], const uint16_t* M, long long rs, int row0, int rows, const char* end, int c, int h) {
     const char* p = (const char*)(M + (long long)row0 * rs);
-    const __amdgpu_buffer_rsrc_t rsrc = m16_rsrc(p, row0 < rows ? (long long)(end - p) : 0);
+    const __amdgpu_buffer_rsrc_t rsrc = buffer_rsrc(p, row0 < rows ? (long long)(end - p) : 0);
     const int voff = (int)(((long long)c * rs + 8 * h) * 2);
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) f[ks] = __builtin_bit_cast(s16x8_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, 32 * ks, 0));
@@ -481,7 +481,7 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) attention_bwd_dkv16_kern
     // L and Dq of the block's 32 queries: every lane requests query qb + lane % 32 (buffer loads, zero past sq, so
     // that no branch surrounds them and the wait for them can be counted); wave 0 puts them in LDS: its lower half
     // the L (in log2 units, +inf past sq, which makes those rows' probabilities exactly 0), its upper half Dq * scale
-    const __amdgpu_buffer_rsrc_t l_rsrc = m16_rsrc(Lz, (long long)g.sq * 4), d_rsrc = m16_rsrc(Dz, (long long)g.sq * 4);
+    const __amdgpu_buffer_rsrc_t l_rsrc = buffer_rsrc(Lz, (long long)g.sq * 4), d_rsrc = buffer_rsrc(Dz, (long long)g.sq * 4);
     float row_l = 0.f, row_d = 0.f;
     auto load_rowv = [&](int qb) {
         row_l = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(l_rsrc, (qb + c) * 4, 0, 0));

@@ -31,7 +31,7 @@ struct Blk32 {
     static_assert(PIECES >= 1, "a block is at least one piece per thread");
     static __device__ __forceinline__ void load(u32x4_t (&r)[PIECES], const float* M, long long rs, int row0, int rows, const char* end) {
         const char* p = (const char*)(M + (long long)row0 * rs);
-        const __amdgpu_buffer_rsrc_t rsrc = m16_rsrc(p, row0 < rows ? (long long)(end - p) : 0);      // rows past the end read zeros
+        const __amdgpu_buffer_rsrc_t rsrc = buffer_rsrc(p, row0 < rows ? (long long)(end - p) : 0);      // rows past the end read zeros
 #pragma unroll
         for (int i = 0; i < PIECES; i++) {
             const int id = threadIdx.x + 256 * i, row = id / (D / 4), d4 = (id % (D / 4)) * 4;
@@ -51,7 +51,7 @@ struct Blk32 {
 template <int KJ>
 __device__ __forceinline__ void load_half_row(float (&f)[KJ], const float* M, long long rs, int row0, int rows, const char* end, int c, int h) {
     const char* p = (const char*)(M + (long long)row0 * rs);
-    const __amdgpu_buffer_rsrc_t rsrc = m16_rsrc(p, row0 < rows ? (long long)(end - p) : 0);
+    const __amdgpu_buffer_rsrc_t rsrc = buffer_rsrc(p, row0 < rows ? (long long)(end - p) : 0);
     const int voff = (int)(((long long)c * rs + KJ * h) * 4);
 #pragma unroll
     for (int i = 0; i < KJ / 4; i++) {
@@ -320,7 +320,7 @@ __global__ void __launch_bounds__(256, D <= 32 ? 2 : 1) attention_bwd_dkv32_kern
     u32x4_t qr[Blk::PIECES], dor[Blk::PIECES];
     // L and Dq of the block's queries: every lane requests query qb + lane % 32 with unconditional buffer loads (zero
     // past sq); wave 0 puts them in LDS, L in log2 units and +inf past sq (those rows' probabilities become exactly 0)
-    const __amdgpu_buffer_rsrc_t l_rsrc = m16_rsrc(Lz, (long long)g.sq * 4), d_rsrc = m16_rsrc(Dz, (long long)g.sq * 4);
+    const __amdgpu_buffer_rsrc_t l_rsrc = buffer_rsrc(Lz, (long long)g.sq * 4), d_rsrc = buffer_rsrc(Dz, (long long)g.sq * 4);
     float row_l = 0.f, row_d = 0.f;
     auto load_rowv = [&](int qb) {
         row_l = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(l_rsrc, (qb + c) * 4, 0, 0));

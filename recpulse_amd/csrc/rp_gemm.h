@@ -3,6 +3,8 @@
 #pragma once
 #include "rp_common.h"
 
+#include <type_traits>
+
 #include <cstdlib>
 #include <cstring>
 
@@ -57,6 +59,35 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(4))) double f64x4_t;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
 typedef __attribute__((ext_vector_type(2))) unsigned int u32x2_t;
+
+// ---- small helpers shared by the kernels ----
+// compile-time loop: f(integral_constant<int, I>) for I in [I0, N)
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// Raw buffer descriptor over [base, base + bytes): loads past the end return zero, stores past it are dropped.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_rsrc(const void* base, long long bytes) {
+    const int n = bytes <= 0 ? 0 : (bytes > 0x7fffffffll ? 0x7fffffff : (int)bytes);
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, n, 0x00020000);
+}
+constexpr uint32_t BUFFER_OOB = 0x80000000u;     // an offset no descriptor covers
+
+// Tile `id` of a batch walked matrix by matrix, row-major inside a matrix: matrix and origin of its BM x BN tile.
+struct TileOrigin { int z, m0, n0; };
+template <int BM, int BN>
+__device__ __forceinline__ TileOrigin tile_origin(unsigned id, unsigned per_matrix, unsigned tiles_n) {
+    TileOrigin t;
+    const unsigned z = id / per_matrix, tile = id - z * per_matrix, tm = tile / tiles_n;
+    t.z = (int)z;
+    t.m0 = (int)tm * BM;
+    t.n0 = (int)(tile - tm * tiles_n) * BN;
+    return t;
+}
 
 // Tile scheduling shared by the MFMA kernels.
 // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2), so a
@@ -122,7 +153,6 @@ static inline int scheduled_grid(int tiles_m, int tiles_n) {
 // ----------------------------------------------------------------------------
 constexpr int SPLITK_DEVICE_SCOPE = 16;      // buffer cache-policy bit sc1
 constexpr int SPLITK_MAX_TILES = 1024;       // arrival counters per device
-constexpr uint32_t SPLITK_OOB = 0x80000000u; // an offset no partial buffer covers (they are kept below 2 GiB)
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t splitk_rsrc(const float* partials, long long bytes) {
     int n = bytes <= 0 ? 0 : (bytes > 0x7fffffffll ? 0x7fffffff : (int)bytes);

@@ -21,14 +21,6 @@ namespace rp {
 constexpr int D32_BM = 128, D32_BN = 128, D32_MAXK = 64;
 constexpr uint32_t D32_OOB = 0x80000000u;
 
-template <int I, int N, typename F>
-__device__ __forceinline__ void d32_static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        d32_static_for<I + 1, N>(f);
-    }
-}
-
 // One operand's 2 tiles x 32 k values per lane.  KC: unit stride along k; MC: unit stride along the free index.
 // fs / ks: strides of the free index and of k in elements; first: first free index of the wave's patch; extent: free extent.
 template <bool MC>
@@ -92,7 +84,7 @@ __global__ void __launch_bounds__(256, 2) gemm_direct32_kernel(GemmArgs g, int t
     // every load above is in flight before the first MFMA waits for its operands (the steps are straight-line code:
     // behind a branch the compiler would issue each group of loads only where it is consumed)
     __builtin_amdgcn_sched_barrier(0);
-    d32_static_for<0, 32>([&](auto tc_) {
+    static_for<0, 32>([&](auto tc_) {
         constexpr int t = decltype(tc_)::value;
 #pragma unroll
         for (int i = 0; i < 2; i++)

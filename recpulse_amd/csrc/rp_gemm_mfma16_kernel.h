@@ -88,20 +88,6 @@ __host__ __device__ constexpr size_t m16_smem_bytes(int bm, int bn, int wgm, boo
 typedef uint16_t __attribute__((address_space(3))) lds_u16;
 
 
-template <int I, int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
-
-// Raw buffer descriptor over [base, base + bytes): loads past the end return zero.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t m16_rsrc(const void* base, long long bytes) {
-    int n = bytes <= 0 ? 0 : (bytes > 0x7fffffffll ? 0x7fffffff : (int)bytes);
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, n, 0x00020000);
-}
-constexpr uint32_t M16_OOB = 0x80000000u;        // an offset no descriptor covers
 
 // Per-thread constants of one operand's slab traffic: NL 16-byte pieces per slab; piece i sits a fixed
 // number of rows (KC) or k-rows (MC) after piece 0, so LDS offsets are piece 0's plus a compile-time step.
@@ -231,17 +217,17 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     for (int i = 0; i < NA; i++) {
         int r = a_r0 + (A_MC ? 0 : i * MapA::PIECE_ROWS), kk = a_kk0 + (A_MC ? i * MapA::PIECE_ROWS : 0);
         a_goff[i] = (uint32_t)(((long long)r * a_fs + (long long)kk * a_ks) * 2);
-        if (EDGE && A_MC && m0 + r >= g.m) a_goff[i] = M16_OOB;
+        if (EDGE && A_MC && m0 + r >= g.m) a_goff[i] = BUFFER_OOB;
     }
 #pragma unroll
     for (int i = 0; i < NB; i++) {
         int r = b_r0 + (B_MC ? 0 : i * MapB::PIECE_ROWS), kk = b_kk0 + (B_MC ? i * MapB::PIECE_ROWS : 0);
         b_goff[i] = (uint32_t)(((long long)r * b_fs + (long long)kk * b_ks) * 2);
-        if (EDGE && B_MC && n0 + r >= g.n) b_goff[i] = M16_OOB;
+        if (EDGE && B_MC && n0 + r >= g.n) b_goff[i] = BUFFER_OOB;
         if (n_segmented) {
             const int j = n0 + r, seg = j / g.seg_n, c = j - seg * g.seg_n;
             const long long at = (long long)(seg / g.seg_w) * g.seg_sh + (long long)(seg % g.seg_w) * g.seg_sw + (long long)c * b_fs + (long long)kk * b_ks;
-            b_goff[i] = (EDGE && j >= g.n) ? M16_OOB : (uint32_t)(at * 2);        // the descriptor's end no longer stands for "past the last column"
+            b_goff[i] = (EDGE && j >= g.n) ? BUFFER_OOB : (uint32_t)(at * 2);        // the descriptor's end no longer stands for "past the last column"
         }
     }
     const int a_wr0 = MapA::lds_off(a_r0, a_kk0), b_wr0 = A_ELEMS + MapB::lds_off(b_r0, b_kk0);     // LDS element offsets of piece 0
@@ -261,8 +247,8 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
     int kleft = 0;        // k still in range counted from the slab the descriptors point at (EDGE, KC operands)
 
     auto point_at_slab = [&](int k0) {
-        a_rsrc = m16_rsrc(a_slab, EDGE ? (long long)(a_end - a_slab) : 0x7fffffffll);
-        b_rsrc = m16_rsrc(b_slab, EDGE ? (long long)(b_end - b_slab) : 0x7fffffffll);
+        a_rsrc = buffer_rsrc(a_slab, EDGE ? (long long)(a_end - a_slab) : 0x7fffffffll);
+        b_rsrc = buffer_rsrc(b_slab, EDGE ? (long long)(b_end - b_slab) : 0x7fffffffll);
         kleft = kend - kbeg - k0;
     };
     // Without edges piece i sits a uniform number of bytes after piece 0: one lane offset per operand plus a scalar
@@ -275,7 +261,7 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
             ra[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)a_goff[0], i * a_piece_step, 0);
         } else {
             uint32_t off = a_goff[i];
-            if (!A_MC && a_kk0 >= kleft) off = M16_OOB;
+            if (!A_MC && a_kk0 >= kleft) off = BUFFER_OOB;
             ra[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)off, 0, 0);
         }
     };
@@ -285,7 +271,7 @@ __global__ void __launch_bounds__(256) gemm_mfma16_kernel(GemmArgs g, int tiles_
             rb[i] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, n_segmented ? (int)b_goff[i] : (int)b_goff[0], n_segmented ? 0 : i * b_piece_step, 0);
         } else {
             uint32_t off = b_goff[i];
-            if (!B_MC && b_kk0 >= kleft) off = M16_OOB;
+            if (!B_MC && b_kk0 >= kleft) off = BUFFER_OOB;
             rb[i] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, (int)off, 0, 0);
         }
     };

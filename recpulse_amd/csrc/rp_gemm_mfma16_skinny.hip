@@ -74,8 +74,8 @@ __global__ void __launch_bounds__(256) gemm_stream16_kernel(GemmArgs g, float* p
     uint32_t b_off[8];
 #pragma unroll
     for (int e = 0; e < 8; e++)
-        b_off[e] = (n0 + 8 * j < g.n) ? (uint32_t)(((long long)(8 * h + e) * b_rs + 8 * j) * 2) : M16_OOB;
-    const uint32_t a_off = (j < g.m) ? (uint32_t)(((long long)j * a_rs + 8 * h) * 2) : M16_OOB;
+        b_off[e] = (n0 + 8 * j < g.n) ? (uint32_t)(((long long)(8 * h + e) * b_rs + 8 * j) * 2) : BUFFER_OOB;
+    const uint32_t a_off = (j < g.m) ? (uint32_t)(((long long)j * a_rs + 8 * h) * 2) : BUFFER_OOB;
 
     u32x4_t raw[SS_DEPTH][8], araw[SS_DEPTH];
     // request round r of this wave into register slot SLOT (r beyond the wave's share reads zeros)
@@ -85,11 +85,11 @@ __global__ void __launch_bounds__(256) gemm_stream16_kernel(GemmArgs g, float* p
         const bool live = r < my_rounds;
         const char* bb = (const char*)(Bm + (long long)kr * b_rs + n0);
         const char* ab = (const char*)(Am + kr);
-        __amdgpu_buffer_rsrc_t b_rsrc = m16_rsrc(bb, live ? (long long)(b_end - bb) : 0);
-        __amdgpu_buffer_rsrc_t a_rsrc = m16_rsrc(ab, live ? (long long)(a_end - ab) : 0);
+        __amdgpu_buffer_rsrc_t b_rsrc = buffer_rsrc(bb, live ? (long long)(b_end - bb) : 0);
+        __amdgpu_buffer_rsrc_t a_rsrc = buffer_rsrc(ab, live ? (long long)(a_end - ab) : 0);
 #pragma unroll
         for (int e = 0; e < 8; e++) raw[SLOT][e] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, (int)b_off[e], 0, 2);
-        araw[SLOT] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)((kr + 8 * h < g.k) ? a_off : M16_OOB), 0, 0);
+        araw[SLOT] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)((kr + 8 * h < g.k) ? a_off : BUFFER_OOB), 0, 0);
     };
 
     f32x16_t acc[8];
@@ -135,7 +135,7 @@ __global__ void __launch_bounds__(256) gemm_stream16_kernel(GemmArgs g, float* p
     const T* bias = (const T*)g.bias;
     const bool has_bias = bias != nullptr, accum = g.accumulate != 0;
     const bool c_vec = g.c_cs == 1 && g.c_rs % 4 == 0 && ((uintptr_t)C & 7) == 0;       // a quad of outputs is one aligned 8-byte store
-    const __amdgpu_buffer_rsrc_t part_rsrc = m16_rsrc(partials, partials ? (long long)nsplit * g.m * g.n * 4 : 0);
+    const __amdgpu_buffer_rsrc_t part_rsrc = buffer_rsrc(partials, partials ? (long long)nsplit * g.m * g.n * 4 : 0);
     // four outputs of one row: the epilogue of each, stored as one vector where the layout allows
     auto store_quad = [&](int row, int col, f32x4_t sum) {
         T y[4];
@@ -213,7 +213,7 @@ __global__ void __launch_bounds__(256) gemm_stream16_kernel(GemmArgs g, float* p
             const int idx = threadIdx.x + 256 * q;
             row[q] = r0 + idx / QPR; col[q] = n0 + (idx % QPR) * 4;
             live[q] = row[q] < g.m && col[q] < g.n;
-            at[q] = live[q] ? ((long long)row[q] * g.n + col[q]) * 4 : (long long)M16_OOB;      // bytes; dead quads read zeros
+            at[q] = live[q] ? ((long long)row[q] * g.n + col[q]) * 4 : (long long)BUFFER_OOB;      // bytes; dead quads read zeros
         }
         f32x4_t sum[QN];
 #pragma unroll
@@ -225,7 +225,7 @@ __global__ void __launch_bounds__(256) gemm_stream16_kernel(GemmArgs g, float* p
 #pragma unroll
                 for (int q = 0; q < QN; q++) {
                     const bool in = live[q] && sp + u < nsplit;
-                    const int off = in ? (int)(at[q] + (sp + u) * split_stride * 4) : (int)M16_OOB;
+                    const int off = in ? (int)(at[q] + (sp + u) * split_stride * 4) : (int)BUFFER_OOB;
                     if (local) v[q][u] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, off, 0, 0);
                     else v[q][u] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, off, 0, SPLITK_DEVICE_SCOPE);
                 }

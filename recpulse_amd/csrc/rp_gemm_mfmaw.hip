@@ -28,14 +28,6 @@ template <> struct mfmaw_cfg<double> {
     static __device__ __forceinline__ int acc_row(int v, int lane) { return 4 * v + (lane >> 4); }
 };
 
-template <int I, int N, typename F>
-__device__ __forceinline__ void mw_static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        mw_static_for<I + 1, N>(f);
-    }
-}
-
 // One operand's slab traffic, a 16-byte piece per thread at a time: piece i of thread t covers V consecutive
 // elements along the operand's unit-stride axis.  LDS is k-major, [BK][ROWS + PAD]; a KC piece (V consecutive k
 // of one row) is transposed on the way in with V scalar writes.
@@ -187,9 +179,9 @@ __global__ void __launch_bounds__(256, 2) gemm_mfmaw_kernel(GemmArgs g, int tile
     };
 
     // prologue: slab 0 into stage 0, slab 1 into registers, fragments(0) of slab 0
-    mw_static_for<0, NP_ALL>([&](auto pc) { load_piece(pc, 0); });
-    mw_static_for<0, NP_ALL>([&](auto pc) { store_piece(pc, smem); });
-    if (nslabs > 1) mw_static_for<0, NP_ALL>([&](auto pc) { load_piece(pc, BK); });
+    static_for<0, NP_ALL>([&](auto pc) { load_piece(pc, 0); });
+    static_for<0, NP_ALL>([&](auto pc) { store_piece(pc, smem); });
+    if (nslabs > 1) static_for<0, NP_ALL>([&](auto pc) { load_piece(pc, BK); });
     __syncthreads();
     read_frags(smem, 0, 0);
 
@@ -200,14 +192,14 @@ __global__ void __launch_bounds__(256, 2) gemm_mfmaw_kernel(GemmArgs g, int tile
         constexpr bool NEXT = decltype(next_tag)::value, NEXT2 = decltype(next2_tag)::value;
         const T* stage = smem + (s & 1) * STAGE;
         T* other = smem + ((s & 1) ^ 1) * STAGE;
-        mw_static_for<0, NKS>([&](auto ksc) {
+        static_for<0, NKS>([&](auto ksc) {
             constexpr int ks = decltype(ksc)::value, slot = ks & 1;
             if constexpr (ks + 1 < NKS) {
                 read_frags(stage, ks + 1, slot ^ 1);
                 // this k-step's share of the slab traffic
                 constexpr int P0 = (NP_ALL * ks) / (NKS - 1), P1 = (NP_ALL * (ks + 1)) / (NKS - 1);
                 if constexpr (NEXT) {
-                    mw_static_for<P0, P1>([&](auto pc) {
+                    static_for<P0, P1>([&](auto pc) {
                         store_piece(pc, other);
                         if constexpr (NEXT2) load_piece(pc, (s + 2) * BK);
                     });
@@ -338,10 +330,10 @@ __global__ void __launch_bounds__(256, (BM <= 64 ? 4 : 2)) gemm_mfmaw_shortk_ker
         const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN;
         const T* A = (const T*)g.A + (long long)z * g.a_bs;
         const T* B = (const T*)g.B + (long long)z * g.b_bs;
-        mw_static_for<0, 2>([&](auto sc) {
+        static_for<0, 2>([&](auto sc) {
             constexpr int sl = decltype(sc)::value;
             if (sl < slabs) {
-                mw_static_for<0, NP_ALL>([&](auto pc) {
+                static_for<0, NP_ALL>([&](auto pc) {
                     constexpr int p = decltype(pc)::value;
                     if constexpr (p < NA) regs[sl][p] = SlabA::load(A, a_fs, a_ks, m0, sl * BK, g.m, g.k, t, p);
                     else regs[sl][p] = SlabB::load(B, b_fs, b_ks, n0, sl * BK, g.n, g.k, t, p - NA);
@@ -356,10 +348,10 @@ __global__ void __launch_bounds__(256, (BM <= 64 ? 4 : 2)) gemm_mfmaw_shortk_ker
         const int z = (int)(id / per_matrix), tile = (int)(id % per_matrix);
         const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN;
         // this tile's operands: registers -> LDS (every wave has finished reading the previous tile: barrier at the loop's end)
-        mw_static_for<0, 2>([&](auto sc) {
+        static_for<0, 2>([&](auto sc) {
             constexpr int sl = decltype(sc)::value;
             if (sl < slabs) {
-                mw_static_for<0, NP_ALL>([&](auto pc) {
+                static_for<0, NP_ALL>([&](auto pc) {
                     constexpr int p = decltype(pc)::value;
                     if constexpr (p < NA) SlabA::store(smem + sl * STAGE, regs[sl][p], t, p);
                     else SlabB::store(smem + sl * STAGE + A_ELEMS, regs[sl][p], t, p - NA);
@@ -387,7 +379,7 @@ __global__ void __launch_bounds__(256, (BM <= 64 ? 4 : 2)) gemm_mfmaw_shortk_ker
         read_frags(smem, 0, 0);
         for (int sl = 0; sl < slabs; sl++) {
             const T* stage = smem + sl * STAGE;
-            mw_static_for<0, NKS>([&](auto ksc) {
+            static_for<0, NKS>([&](auto ksc) {
                 constexpr int ks = decltype(ksc)::value, slot = ks & 1;
                 if constexpr (ks + 1 < NKS) read_frags(stage, ks + 1, slot ^ 1);
                 else if (sl + 1 < slabs) read_frags(stage + STAGE, 0, slot ^ 1);

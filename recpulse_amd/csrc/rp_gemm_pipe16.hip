@@ -30,35 +30,8 @@ constexpr int P16_BM = 128, P16_BN = 128, P16_MAXK = 64;
 constexpr int P16_ROW_BYTES = 128;                                   // one LDS row: 64 16-bit values
 constexpr int P16_TILE_BYTES = (P16_BM + P16_BN) * P16_ROW_BYTES;    // 32 KB: A rows, then B rows
 constexpr int P16_NBUF = 3;                                          // LDS tiles in rotation
-constexpr uint32_t P16_OOB = 0x80000000u;
 
 typedef __attribute__((address_space(3))) void* p16_lds_t;
-
-template <int I, int N, typename F>
-__device__ __forceinline__ void p16_static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        p16_static_for<I + 1, N>(f);
-    }
-}
-
-struct P16Tile {
-    int z, m0, n0;
-};
-
-__device__ __forceinline__ P16Tile p16_tile(unsigned id, unsigned per_matrix, unsigned tiles_n) {
-    P16Tile t;
-    const unsigned z = id / per_matrix, tile = id - z * per_matrix, tm = tile / tiles_n;
-    t.z = (int)z;
-    t.m0 = (int)tm * P16_BM;
-    t.n0 = (int)(tile - tm * tiles_n) * P16_BN;
-    return t;
-}
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t p16_rsrc(const void* base, long long span_bytes) {
-    const int n = span_bytes <= 0 ? 0 : (span_bytes > 0x7fffffffll ? 0x7fffffff : (int)span_bytes);
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, n, 0x00020000);
-}
 
 template <typename T> struct p16_ops;
 template <> struct p16_ops<bf16_t> {
@@ -119,15 +92,15 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
             const int krow = 4 * q + (lane >> 4);                       // k row within the wave's 16
             const int c32 = ((lane & 15) >> 1) ^ (krow & 7);            // which 32 bytes of the global k row (its half: lane & 1)
             const int free = (c32 * 2 + (lane & 1)) * 8;
-            a_off[q] = A_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * a_ks + free) * 2) : P16_OOB)
-                            : (piece * 8 < g.k ? (uint32_t)(((long long)row * a_fs + piece * 8) * 2) : P16_OOB);
-            b_off[q] = B_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * b_ks + free) * 2) : P16_OOB)
-                            : (piece * 8 < g.k ? (uint32_t)(((long long)row * b_fs + piece * 8) * 2) : P16_OOB);
+            a_off[q] = A_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * a_ks + free) * 2) : BUFFER_OOB)
+                            : (piece * 8 < g.k ? (uint32_t)(((long long)row * a_fs + piece * 8) * 2) : BUFFER_OOB);
+            b_off[q] = B_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * b_ks + free) * 2) : BUFFER_OOB)
+                            : (piece * 8 < g.k ? (uint32_t)(((long long)row * b_fs + piece * 8) * 2) : BUFFER_OOB);
         }
         auto fetch = [&](unsigned id, int buf) {
-            const P16Tile t = p16_tile(id, per_matrix, tiles_n);
-            const __amdgpu_buffer_rsrc_t ra = p16_rsrc((const uint16_t*)g.A + (long long)t.z * g.a_bs, a_span);
-            const __amdgpu_buffer_rsrc_t rb = p16_rsrc((const uint16_t*)g.B + (long long)t.z * g.b_bs, b_span);
+            const TileOrigin t = tile_origin<P16_BM, P16_BN>(id, per_matrix, tiles_n);
+            const __amdgpu_buffer_rsrc_t ra = buffer_rsrc((const uint16_t*)g.A + (long long)t.z * g.a_bs, a_span);
+            const __amdgpu_buffer_rsrc_t rb = buffer_rsrc((const uint16_t*)g.B + (long long)t.z * g.b_bs, b_span);
             const int sa = A_MC ? (int)(((long long)(16 * p) * a_ks + t.m0) * 2) : (int)((long long)(t.m0 + 32 * p) * a_fs * 2);
             const int sb = B_MC ? (int)(((long long)(16 * p) * b_ks + t.n0) * 2) : (int)((long long)(t.n0 + 32 * p) * b_fs * 2);
             // (both layouts put the wave's share at the same place: 32 rows of 128 bytes = 16 k rows of 256 bytes = 4 KB)
@@ -214,7 +187,7 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     u32x4_t rows[8];                    // the previous tile's row segments on their way from the staging patch to memory
     s16x8_t af[KST][2], bf[KST][2];     // [k step][tile]: eight k values of the lane's row
     u32x4_t bias_prev = {0u, 0u, 0u, 0u}, bias_cur = {0u, 0u, 0u, 0u};      // BIAS: of columns n0 + wn0 + 8 rp .. + 7 of the tile being stored / multiplied
-    auto load_bias = [&](const P16Tile& t) {
+    auto load_bias = [&](const TileOrigin& t) {
         const int gn = t.n0 + wn0 + 8 * rp;
         bias_cur = gn < g.n ? *(const u32x4_t*)((const uint16_t*)g.bias + gn) : u32x4_t{0u, 0u, 0u, 0u};       // (n is a multiple of 8)
     };
@@ -222,7 +195,7 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     auto widen_hi = [](uint32_t w) { T x; x.bits = (uint16_t)(w >> 16); return widen(x); };
 
     auto pack_all = [&]() {
-        p16_static_for<0, 16>([&](auto nc) {
+        static_for<0, 16>([&](auto nc) {
             constexpr int n = decltype(nc)::value, jm = n >> 3, in = (n >> 2) & 1, q = n & 3;
             const float v0 = acc[jm][in][4 * q], v1 = acc[jm][in][4 * q + 1], v2 = acc[jm][in][4 * q + 2], v3 = acc[jm][in][4 * q + 3];
             packed[n][0] = p16_ops<T>::pack(v0, v1);
@@ -246,12 +219,12 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
         }
     };
     // ... and to memory
-    auto row_store = [&](auto e_c, const P16Tile& t, const __amdgpu_buffer_rsrc_t& rc) {
+    auto row_store = [&](auto e_c, const TileOrigin& t, const __amdgpu_buffer_rsrc_t& rc) {
         constexpr int e = decltype(e_c)::value;
         const int gm = t.m0 + wm0 + 8 * e, gn = t.n0 + wn0;
         const int soff = (int)(((long long)gm * g.c_rs + gn) * 2);
         uint32_t voff = c_lane;
-        if constexpr (EDGE) voff = (gm + rr < g.m && gn + 8 * rp < g.n) ? c_lane : P16_OOB;      // (n is a multiple of 8: a piece is inside or outside as a whole)
+        if constexpr (EDGE) voff = (gm + rr < g.m && gn + 8 * rp < g.n) ? c_lane : BUFFER_OOB;      // (n is a multiple of 8: a piece is inside or outside as a whole)
         __builtin_amdgcn_raw_buffer_store_b128(rows[e], rc, (int)voff, soff, 2);          // (streaming store: the output is not read again by this kernel)
     };
 
@@ -273,16 +246,16 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     // are read (LDS tile `next`), so no MFMA ever waits for LDS.  If STORE, the previous tile (narrowed, in `packed`) goes
     // through the staging patch to memory meanwhile, in quarters of the MFMAs: staging writes 0..7 | writes 8..15 and row
     // reads 0..3 | row stores 0..3 and row reads 4..7 | row stores 4..7, so that no instruction waits for the one before it.
-    auto tile_pass = [&](auto store_c, int next, const P16Tile& prev) {
+    auto tile_pass = [&](auto store_c, int next, const TileOrigin& prev) {
         constexpr bool STORE = decltype(store_c)::value;
         constexpr int NM = 4 * KST, Q = NM / 4;                    // MFMAs per tile and per quarter
         constexpr int WR = 8 / Q, RD = 4 / Q;                       // staging writes and row reads / stores per MFMA in their quarters
         const unsigned char* next_base = p16_smem + next * P16_TILE_BYTES;
-        const __amdgpu_buffer_rsrc_t rc = p16_rsrc((uint16_t*)g.C + (long long)prev.z * g.c_bs, c_span);
+        const __amdgpu_buffer_rsrc_t rc = buffer_rsrc((uint16_t*)g.C + (long long)prev.z * g.c_bs, c_span);
         __syncthreads();                                   // the next tile is in LDS; this tile's pieces have all arrived in registers
-        p16_static_for<0, KST>([&](auto sc) {
+        static_for<0, KST>([&](auto sc) {
             constexpr int s = decltype(sc)::value;
-            p16_static_for<0, 4>([&](auto tc) {
+            static_for<0, 4>([&](auto tc) {
                 constexpr int t4 = decltype(tc)::value, jm = t4 >> 1, in = t4 & 1, mi = s * 4 + t4, phase = mi / Q, idx = mi % Q;
                 // operands swapped: the MFMA's rows are columns of C
                 if constexpr (s == 0) {
@@ -292,16 +265,16 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
                     acc[jm][in] = p16_ops<T>::mma(bf[s][in], af[s][jm], acc[jm][in]);
                 }
                 if constexpr (STORE) {
-                    if constexpr (phase == 0) p16_static_for<0, WR>([&](auto ec) { stage_write(std::integral_constant<int, idx * WR + decltype(ec)::value>{}); });
+                    if constexpr (phase == 0) static_for<0, WR>([&](auto ec) { stage_write(std::integral_constant<int, idx * WR + decltype(ec)::value>{}); });
                     if constexpr (phase == 1) {
-                        p16_static_for<0, WR>([&](auto ec) { stage_write(std::integral_constant<int, 8 + idx * WR + decltype(ec)::value>{}); });
-                        p16_static_for<0, RD>([&](auto ec) { row_read(std::integral_constant<int, idx * RD + decltype(ec)::value>{}); });
+                        static_for<0, WR>([&](auto ec) { stage_write(std::integral_constant<int, 8 + idx * WR + decltype(ec)::value>{}); });
+                        static_for<0, RD>([&](auto ec) { row_read(std::integral_constant<int, idx * RD + decltype(ec)::value>{}); });
                     }
                     if constexpr (phase == 2) {
-                        p16_static_for<0, RD>([&](auto ec) { row_store(std::integral_constant<int, idx * RD + decltype(ec)::value>{}, prev, rc); });
-                        p16_static_for<0, RD>([&](auto ec) { row_read(std::integral_constant<int, 4 + idx * RD + decltype(ec)::value>{}); });
+                        static_for<0, RD>([&](auto ec) { row_store(std::integral_constant<int, idx * RD + decltype(ec)::value>{}, prev, rc); });
+                        static_for<0, RD>([&](auto ec) { row_read(std::integral_constant<int, 4 + idx * RD + decltype(ec)::value>{}); });
                     }
-                    if constexpr (phase == 3) p16_static_for<0, RD>([&](auto ec) { row_store(std::integral_constant<int, 4 + idx * RD + decltype(ec)::value>{}, prev, rc); });
+                    if constexpr (phase == 3) static_for<0, RD>([&](auto ec) { row_store(std::integral_constant<int, 4 + idx * RD + decltype(ec)::value>{}, prev, rc); });
                     __builtin_amdgcn_sched_barrier(0);
                 }
             });
@@ -311,29 +284,29 @@ __global__ void __launch_bounds__(512) gemm_pipe16_kernel(GemmArgs g, int tiles_
     };
 
     __syncthreads();                                   // the first tile is in LDS
-    P16Tile prev = {0, 0, 0};
+    TileOrigin prev = {0, 0, 0};
     int next = 1;                                      // LDS tile of the tile after the current one
     unsigned id = first;
     if (id >= total) return;
-    p16_static_for<0, KST>([&](auto sc) { read_frags(p16_smem, sc); });
-    if constexpr (BIAS) load_bias(p16_tile(id, per_matrix, tiles_n));
+    static_for<0, KST>([&](auto sc) { read_frags(p16_smem, sc); });
+    if constexpr (BIAS) load_bias(tile_origin<P16_BM, P16_BN>(id, per_matrix, tiles_n));
     tile_pass(std::false_type{}, next, prev);
-    prev = p16_tile(id, per_matrix, tiles_n);
+    prev = tile_origin<P16_BM, P16_BN>(id, per_matrix, tiles_n);
     if constexpr (BIAS) bias_prev = bias_cur;
     next = next + 1 == P16_NBUF ? 0 : next + 1;
     id += stride;
     for (; id < total; id += stride) {
-        if constexpr (BIAS) load_bias(p16_tile(id, per_matrix, tiles_n));
+        if constexpr (BIAS) load_bias(tile_origin<P16_BM, P16_BN>(id, per_matrix, tiles_n));
         tile_pass(std::true_type{}, next, prev);
-        prev = p16_tile(id, per_matrix, tiles_n);
+        prev = tile_origin<P16_BM, P16_BN>(id, per_matrix, tiles_n);
         if constexpr (BIAS) bias_prev = bias_cur;
         next = next + 1 == P16_NBUF ? 0 : next + 1;
     }
     // the last tile
-    const __amdgpu_buffer_rsrc_t rc = p16_rsrc((uint16_t*)g.C + (long long)prev.z * g.c_bs, c_span);
-    p16_static_for<0, 16>([&](auto nc) { stage_write(nc); });
-    p16_static_for<0, 8>([&](auto ec) { row_read(ec); });
-    p16_static_for<0, 8>([&](auto ec) { row_store(ec, prev, rc); });
+    const __amdgpu_buffer_rsrc_t rc = buffer_rsrc((uint16_t*)g.C + (long long)prev.z * g.c_bs, c_span);
+    static_for<0, 16>([&](auto nc) { stage_write(nc); });
+    static_for<0, 8>([&](auto ec) { row_read(ec); });
+    static_for<0, 8>([&](auto ec) { row_store(ec, prev, rc); });
 }
 
 // ---- host side ----

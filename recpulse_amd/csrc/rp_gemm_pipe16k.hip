@@ -33,23 +33,9 @@ constexpr int K16_STAGE_BYTES = K16_A_BYTES + K16_B_BYTES;
 constexpr int K16_PATCH_BYTES = 32 * 128;                          // a wave's 32 x 64 outputs, 16 bit
 constexpr int K16_SMEM_BYTES = K16_NBUF * K16_STAGE_BYTES + 4 * K16_PATCH_BYTES;
 constexpr int K16_FETCH = 6;                                       // load instructions per fetching wave and slab
-constexpr uint32_t K16_OOB = 0x80000000u;
 
 typedef __attribute__((address_space(3))) void* k16_lds_t;
 typedef __attribute__((ext_vector_type(4))) short k16_s16x4_t;
-
-template <int I, int N, typename F>
-__device__ __forceinline__ void k16_static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        k16_static_for<I + 1, N>(f);
-    }
-}
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t k16_rsrc(const void* base, long long span_bytes) {
-    const int n = span_bytes <= 0 ? 0 : (span_bytes > 0x7fffffffll ? 0x7fffffff : (int)span_bytes);
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, n, 0x00020000);
-}
 
 template <typename T> struct k16_ops;
 template <> struct k16_ops<bf16_t> {
@@ -141,19 +127,19 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
             if (f_id >= total) return false;
             const unsigned z = f_id / (unsigned)tiles_m;
             const int m0 = (int)(f_id - z * (unsigned)tiles_m) * K16_BM, k0 = f_s * K16_BK, kleft = g.k - k0;
-            const __amdgpu_buffer_rsrc_t ra = k16_rsrc((const uint16_t*)g.A + (long long)z * g.a_bs, a_span);
-            const __amdgpu_buffer_rsrc_t rb = k16_rsrc((const uint16_t*)g.B + (long long)z * g.b_bs, b_span);
+            const __amdgpu_buffer_rsrc_t ra = buffer_rsrc((const uint16_t*)g.A + (long long)z * g.a_bs, a_span);
+            const __amdgpu_buffer_rsrc_t rb = buffer_rsrc((const uint16_t*)g.B + (long long)z * g.b_bs, b_span);
             const int sa = A_MC ? (int)((((long long)(k0 + 16 * p)) * a_ks + m0) * 2) : (int)(((long long)(m0 + 32 * p) * a_fs + k0) * 2);
             const int sb = B_MC ? (int)(((long long)(k0 + 16 * p)) * b_ks * 2) : (int)(((long long)(16 * p) * b_fs + k0) * 2);
             unsigned char* dst = k16_smem + f_stage * K16_STAGE_BYTES;
 #pragma unroll
             for (int q = 0; q < 4; q++)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (k16_lds_t)(dst + (A_MC ? 16 * p * 256 : 32 * p * 128) + q * 1024), 16,
-                                                         a_k[q] < kleft ? (int)a_off[q] : (int)K16_OOB, sa, 0, 0);
+                                                         a_k[q] < kleft ? (int)a_off[q] : (int)BUFFER_OOB, sa, 0, 0);
 #pragma unroll
             for (int q = 0; q < 2; q++)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (k16_lds_t)(dst + K16_A_BYTES + 16 * p * 128 + q * 1024), 16,
-                                                         b_k[q] < kleft ? (int)b_off[q] : (int)K16_OOB, sb, 0, 0);
+                                                         b_k[q] < kleft ? (int)b_off[q] : (int)BUFFER_OOB, sb, 0, 0);
             f_stage = f_stage + 1 == K16_NBUF ? 0 : f_stage + 1;
             if (++f_s == nslab) { f_s = 0; f_id += stride; }
             return true;
@@ -256,7 +242,7 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
         }
     };
     auto pack_all = [&]() {
-        k16_static_for<0, 8>([&](auto nc) {
+        static_for<0, 8>([&](auto nc) {
             constexpr int n = decltype(nc)::value, in = n >> 2, q = n & 3;
             float v0 = acc[in][4 * q], v1 = acc[in][4 * q + 1], v2 = acc[in][4 * q + 2], v3 = acc[in][4 * q + 3];
             if constexpr (EPI) {
@@ -284,7 +270,7 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
         const int gm = pm0 + 32 * wave + 8 * e;
         const int soff = (int)((long long)gm * g.c_rs * 2);
         uint32_t voff = c_lane;
-        if constexpr (EDGE) voff = (gm + rr < g.m && 8 * rp < g.n) ? c_lane : K16_OOB;      // (n is a multiple of 8: a piece is inside or outside as a whole)
+        if constexpr (EDGE) voff = (gm + rr < g.m && 8 * rp < g.n) ? c_lane : BUFFER_OOB;      // (n is a multiple of 8: a piece is inside or outside as a whole)
         __builtin_amdgcn_raw_buffer_store_b128(rows[e], rc, (int)voff, soff, 2);          // (streaming store: the output is not read again by this kernel)
     };
 
@@ -294,7 +280,7 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
         const int gm = pm0 + 32 * wave + 8 * e;
         const int soff = (int)((long long)gm * g.c_rs * 2);
         uint32_t voff = c_lane;
-        if constexpr (EDGE) voff = (gm + rr < g.m && 8 * rp < g.n) ? c_lane : K16_OOB;
+        if constexpr (EDGE) voff = (gm + rr < g.m && 8 * rp < g.n) ? c_lane : BUFFER_OOB;
         old[e] = __builtin_amdgcn_raw_buffer_load_b128(rc, (int)voff, soff, 0);
     };
     auto row_add_old = [&](auto e_c) {
@@ -311,14 +297,14 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
         constexpr bool STORE = decltype(store_c)::value;
         const unsigned char* next_base = k16_smem + next * K16_STAGE_BYTES;
         __syncthreads();                                   // the next slab is in LDS; this slab's fragments have all arrived in registers
-        k16_static_for<0, 4>([&](auto ksc) {
+        static_for<0, 4>([&](auto ksc) {
             constexpr int ks = decltype(ksc)::value;
-            k16_static_for<0, 2>([&](auto ic) {
+            static_for<0, 2>([&](auto ic) {
                 constexpr int in = decltype(ic)::value, mi = 2 * ks + in;
                 acc[in] = k16_ops<T>::mma(bf[ks][in], af[ks], acc[in]);          // operands swapped: the MFMA's rows are columns of C
                 if constexpr (STORE) {
-                    if constexpr (mi < 2) k16_static_for<0, 4>([&](auto ec) { stage_write(std::integral_constant<int, 4 * mi + decltype(ec)::value>{}); });
-                    else if constexpr (mi < 4) k16_static_for<0, 2>([&](auto ec) { row_read(std::integral_constant<int, 2 * (mi - 2) + decltype(ec)::value>{}); });
+                    if constexpr (mi < 2) static_for<0, 4>([&](auto ec) { stage_write(std::integral_constant<int, 4 * mi + decltype(ec)::value>{}); });
+                    else if constexpr (mi < 4) static_for<0, 2>([&](auto ec) { row_read(std::integral_constant<int, 2 * (mi - 2) + decltype(ec)::value>{}); });
                     else row_store(std::integral_constant<int, mi - 4>{}, pm0, rc);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -329,10 +315,10 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
 
     __syncthreads();                                   // slab 0 is in LDS
     if (first >= total) return;
-    k16_static_for<0, 4>([&](auto ksc) { read_frags(k16_smem, ksc); });
+    static_for<0, 4>([&](auto ksc) { read_frags(k16_smem, ksc); });
     int next = 1, pm0 = 0;
     bool pending = false;                              // a finished tile waits in `packed`
-    __amdgpu_buffer_rsrc_t rc = k16_rsrc(g.C, c_span);
+    __amdgpu_buffer_rsrc_t rc = buffer_rsrc(g.C, c_span);
     for (unsigned id = first; id < total; id += stride) {
 #pragma unroll
         for (int in = 0; in < 2; in++)
@@ -342,17 +328,17 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
             // this tile's place in C is known from the start: its old rows travel while the tile is multiplied
             const unsigned z = id / (unsigned)tiles_m;
             pm0 = (int)(id - z * (unsigned)tiles_m) * K16_BM;
-            rc = k16_rsrc((uint16_t*)g.C + (long long)z * g.c_bs, c_span);
-            if (accum) k16_static_for<0, 4>([&](auto ec) { old_load(ec, pm0, rc); });
+            rc = buffer_rsrc((uint16_t*)g.C + (long long)z * g.c_bs, c_span);
+            if (accum) static_for<0, 4>([&](auto ec) { old_load(ec, pm0, rc); });
             for (int s = 0; s < nslab; s++) {
                 slab_pass(std::false_type{}, next, pm0, rc);
                 next = next + 1 == K16_NBUF ? 0 : next + 1;
             }
             pack_all();
-            k16_static_for<0, 8>([&](auto nc) { stage_write(nc); });
-            k16_static_for<0, 4>([&](auto ec) { row_read(ec); });
-            if (accum) k16_static_for<0, 4>([&](auto ec) { row_add_old(ec); });
-            k16_static_for<0, 4>([&](auto ec) { row_store(ec, pm0, rc); });
+            static_for<0, 8>([&](auto nc) { stage_write(nc); });
+            static_for<0, 4>([&](auto ec) { row_read(ec); });
+            if (accum) static_for<0, 4>([&](auto ec) { row_add_old(ec); });
+            static_for<0, 4>([&](auto ec) { row_store(ec, pm0, rc); });
             continue;
         }
         for (int s = 0; s < nslab; s++) {
@@ -364,14 +350,14 @@ __global__ void __launch_bounds__(512) gemm_pipe16k_kernel(GemmArgs g, int tiles
         pack_all();
         const unsigned z = id / (unsigned)tiles_m;
         pm0 = (int)(id - z * (unsigned)tiles_m) * K16_BM;
-        rc = k16_rsrc((uint16_t*)g.C + (long long)z * g.c_bs, c_span);
+        rc = buffer_rsrc((uint16_t*)g.C + (long long)z * g.c_bs, c_span);
         pending = true;
     }
     if constexpr (EPI) return;
     // the last tile
-    k16_static_for<0, 8>([&](auto nc) { stage_write(nc); });
-    k16_static_for<0, 4>([&](auto ec) { row_read(ec); });
-    k16_static_for<0, 4>([&](auto ec) { row_store(ec, pm0, rc); });
+    static_for<0, 8>([&](auto nc) { stage_write(nc); });
+    static_for<0, 4>([&](auto ec) { row_read(ec); });
+    static_for<0, 4>([&](auto ec) { row_store(ec, pm0, rc); });
 }
 
 // ---- host side ----

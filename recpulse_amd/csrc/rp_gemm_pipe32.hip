@@ -30,38 +30,11 @@ namespace rp {
 constexpr int P32_BM = 128, P32_BN = 128, P32_MAXK = 64;
 constexpr int P32_ROW_BYTES = 256;                                   // one LDS row: 64 floats
 constexpr int P32_TILE_BYTES = (P32_BM + P32_BN) * P32_ROW_BYTES;    // 64 KB: A rows, then B rows
-constexpr uint32_t P32_OOB = 0x80000000u;
 
 typedef __attribute__((address_space(3))) void* p32_lds_t;
 
-template <int I, int N, typename F>
-__device__ __forceinline__ void p32_static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        p32_static_for<I + 1, N>(f);
-    }
-}
-
-struct P32Tile {
-    int z, m0, n0;
-};
-
-__device__ __forceinline__ P32Tile p32_tile(unsigned id, unsigned per_matrix, unsigned tiles_n) {
-    P32Tile t;
-    const unsigned z = id / per_matrix, tile = id - z * per_matrix, tm = tile / tiles_n;
-    t.z = (int)z;
-    t.m0 = (int)tm * P32_BM;
-    t.n0 = (int)(tile - tm * tiles_n) * P32_BN;
-    return t;
-}
-
 // (a bit cast applied directly to one element of a vector reads the wrong element with this compiler: pass the element by value)
 __device__ __forceinline__ uint32_t p32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t p32_rsrc(const void* base, long long span_bytes) {
-    const int n = span_bytes <= 0 ? 0 : (span_bytes > 0x7fffffffll ? 0x7fffffff : (int)span_bytes);
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, n, 0x00020000);
-}
 
 // KCH: 16-byte pieces of k per lane pair that are multiplied (8 for k <= 64, 4 for k <= 32); EDGE: m or n not whole tiles.
 // A_MC / B_MC: the operand has unit stride along its free index (m, n) instead of along k: it lies in LDS as 64 k rows of
@@ -93,15 +66,15 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
             const int krow = 2 * q + (lane >> 5);                       // k row within the wave's 16
             const int c128 = ((lane & 31) >> 3) ^ ((krow >> 2) & 3);    // which 128 bytes of the global k row (its 16-byte piece: lane & 7)
             const int free = c128 * 32 + (lane & 7) * 4;
-            a_off[q] = A_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * a_ks + free) * 4) : P32_OOB)
-                            : (piece * 4 < g.k ? (uint32_t)(((long long)row * a_fs + piece * 4) * 4) : P32_OOB);
-            b_off[q] = B_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * b_ks + free) * 4) : P32_OOB)
-                            : (piece * 4 < g.k ? (uint32_t)(((long long)row * b_fs + piece * 4) * 4) : P32_OOB);
+            a_off[q] = A_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * a_ks + free) * 4) : BUFFER_OOB)
+                            : (piece * 4 < g.k ? (uint32_t)(((long long)row * a_fs + piece * 4) * 4) : BUFFER_OOB);
+            b_off[q] = B_MC ? (16 * p + krow < g.k ? (uint32_t)(((long long)krow * b_ks + free) * 4) : BUFFER_OOB)
+                            : (piece * 4 < g.k ? (uint32_t)(((long long)row * b_fs + piece * 4) * 4) : BUFFER_OOB);
         }
         auto fetch = [&](unsigned id, int buf) {
-            const P32Tile t = p32_tile(id, per_matrix, tiles_n);
-            const __amdgpu_buffer_rsrc_t ra = p32_rsrc((const float*)g.A + (long long)t.z * g.a_bs, a_span);
-            const __amdgpu_buffer_rsrc_t rb = p32_rsrc((const float*)g.B + (long long)t.z * g.b_bs, b_span);
+            const TileOrigin t = tile_origin<P32_BM, P32_BN>(id, per_matrix, tiles_n);
+            const __amdgpu_buffer_rsrc_t ra = buffer_rsrc((const float*)g.A + (long long)t.z * g.a_bs, a_span);
+            const __amdgpu_buffer_rsrc_t rb = buffer_rsrc((const float*)g.B + (long long)t.z * g.b_bs, b_span);
             const int sa = A_MC ? (int)(((long long)(16 * p) * a_ks + t.m0) * 4) : (int)((long long)(t.m0 + 32 * p) * a_fs * 4);
             const int sb = B_MC ? (int)(((long long)(16 * p) * b_ks + t.n0) * 4) : (int)((long long)(t.n0 + 32 * p) * b_fs * 4);
             // (both layouts put the wave's share at the same place: 32 rows of 256 bytes = 16 k rows of 512 bytes = 8 KB)
@@ -140,7 +113,7 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
     f32x16_t acc[2][2][2];              // [set][i][j]
     f32x4_t af[2][2], bf[2][2];         // [slot][i or j]: four k values of the lane's row
     float bias_prev[2] = {0.f, 0.f}, bias_cur[2] = {0.f, 0.f};      // BIAS: of columns n0 + wn0 + 32 j + r of the tile being stored / multiplied
-    auto load_bias = [&](const P32Tile& t) {
+    auto load_bias = [&](const TileOrigin& t) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int gn = t.n0 + wn0 + 32 * j + r;
@@ -149,14 +122,14 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
     };
 
     // store number n (0..63) of accumulator set SET: register v of MFMA tile (i, j), i.e. columns 32j + r of rows 32i + 8(v / 4) + 4h + v % 4
-    auto store_one = [&](auto set_c, auto n_c, const P32Tile& t, const __amdgpu_buffer_rsrc_t& rc) {
+    auto store_one = [&](auto set_c, auto n_c, const TileOrigin& t, const __amdgpu_buffer_rsrc_t& rc) {
         constexpr int SET = decltype(set_c)::value, n = decltype(n_c)::value;
         constexpr int sj = n >> 5, si = (n >> 4) & 1, v = n & 15;
         constexpr int row = 32 * si + 8 * (v / 4) + (v % 4);
         const int gm = t.m0 + wm0 + row, gn = t.n0 + wn0 + 32 * sj;
         const int soff = (int)(((long long)gm * g.c_rs + (long long)gn * g.c_cs) * 4);
         uint32_t voff = c_lane;
-        if constexpr (EDGE) voff = (gm + 4 * h < g.m && gn + r < g.n) ? c_lane : P32_OOB;
+        if constexpr (EDGE) voff = (gm + 4 * h < g.m && gn + r < g.n) ? c_lane : BUFFER_OOB;
         float val = acc[SET][si][sj][v];
         if constexpr (BIAS) val = val + bias_prev[sj];
         __builtin_amdgcn_raw_buffer_store_b32(p32_bits(val), rc, (int)voff, soff, 2);          // (streaming store: the output is not read again by this kernel)
@@ -189,13 +162,13 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
     // write set CUR ^ 1 (the tile `prev`) meanwhile.  The block's barrier sits before the last piece's MFMAs, when every
     // LDS read of this tile has returned: behind it the other LDS tile holds the next tile, whose first pieces are read
     // under those MFMAs, and the fetching waves may overwrite this one.
-    auto tile_pass = [&](auto cur_c, auto store_c, int buf, const P32Tile& prev) {
+    auto tile_pass = [&](auto cur_c, auto store_c, int buf, const TileOrigin& prev) {
         constexpr int CUR = decltype(cur_c)::value;
         constexpr bool STORE = decltype(store_c)::value;
         const unsigned char* base = p32_smem + buf * P32_TILE_BYTES;
         const unsigned char* next_base = p32_smem + (buf ^ 1) * P32_TILE_BYTES;
-        const __amdgpu_buffer_rsrc_t rc = p32_rsrc((float*)g.C + (long long)prev.z * g.c_bs, c_span);
-        p32_static_for<0, KCH>([&](auto uc) {
+        const __amdgpu_buffer_rsrc_t rc = buffer_rsrc((float*)g.C + (long long)prev.z * g.c_bs, c_span);
+        static_for<0, KCH>([&](auto uc) {
             constexpr int u = decltype(uc)::value, slot = u & 1;
             if constexpr (u + 1 < KCH) {
                 read_frags(base, u + 1, slot ^ 1);
@@ -203,7 +176,7 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
                 __syncthreads();
                 read_frags(next_base, 0, slot ^ 1);
             }
-            p32_static_for<0, 16>([&](auto sc) {
+            static_for<0, 16>([&](auto sc) {
                 constexpr int s = decltype(sc)::value, e = s >> 2, i = (s >> 1) & 1, j = s & 1;
                 if constexpr (u == 0 && e == 0) {
                     const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -223,39 +196,39 @@ __global__ void __launch_bounds__(512) gemm_pipe32_kernel(GemmArgs g, int tiles_
     };
 
     __syncthreads();                                   // the first tile is in LDS
-    P32Tile prev = {0, 0, 0};
+    TileOrigin prev = {0, 0, 0};
     int buf = 0, last = 0;
     unsigned id = first;
     if (id >= total) return;
     read_frags(p32_smem, 0, 0);
-    if constexpr (BIAS) load_bias(p32_tile(id, per_matrix, tiles_n));
+    if constexpr (BIAS) load_bias(tile_origin<P32_BM, P32_BN>(id, per_matrix, tiles_n));
     tile_pass(std::integral_constant<int, 0>{}, std::false_type{}, buf, prev);
-    prev = p32_tile(id, per_matrix, tiles_n);
+    prev = tile_origin<P32_BM, P32_BN>(id, per_matrix, tiles_n);
     if constexpr (BIAS) { bias_prev[0] = bias_cur[0]; bias_prev[1] = bias_cur[1]; }
     buf ^= 1;
     id += stride;
     // two tiles per round, so that the accumulator sets are fixed registers
     while (id < total) {
-        if constexpr (BIAS) load_bias(p32_tile(id, per_matrix, tiles_n));
+        if constexpr (BIAS) load_bias(tile_origin<P32_BM, P32_BN>(id, per_matrix, tiles_n));
         tile_pass(std::integral_constant<int, 1>{}, std::true_type{}, buf, prev);
-        prev = p32_tile(id, per_matrix, tiles_n);
+        prev = tile_origin<P32_BM, P32_BN>(id, per_matrix, tiles_n);
         if constexpr (BIAS) { bias_prev[0] = bias_cur[0]; bias_prev[1] = bias_cur[1]; }
         buf ^= 1;
         id += stride;
         last = 1;
         if (id >= total) break;
-        if constexpr (BIAS) load_bias(p32_tile(id, per_matrix, tiles_n));
+        if constexpr (BIAS) load_bias(tile_origin<P32_BM, P32_BN>(id, per_matrix, tiles_n));
         tile_pass(std::integral_constant<int, 0>{}, std::true_type{}, buf, prev);
-        prev = p32_tile(id, per_matrix, tiles_n);
+        prev = tile_origin<P32_BM, P32_BN>(id, per_matrix, tiles_n);
         if constexpr (BIAS) { bias_prev[0] = bias_cur[0]; bias_prev[1] = bias_cur[1]; }
         buf ^= 1;
         id += stride;
         last = 0;
     }
     // the last tile's accumulators
-    const __amdgpu_buffer_rsrc_t rc = p32_rsrc((float*)g.C + (long long)prev.z * g.c_bs, c_span);
-    if (last == 0) p32_static_for<0, 64>([&](auto nc) { store_one(std::integral_constant<int, 0>{}, nc, prev, rc); });
-    else p32_static_for<0, 64>([&](auto nc) { store_one(std::integral_constant<int, 1>{}, nc, prev, rc); });
+    const __amdgpu_buffer_rsrc_t rc = buffer_rsrc((float*)g.C + (long long)prev.z * g.c_bs, c_span);
+    if (last == 0) static_for<0, 64>([&](auto nc) { store_one(std::integral_constant<int, 0>{}, nc, prev, rc); });
+    else static_for<0, 64>([&](auto nc) { store_one(std::integral_constant<int, 1>{}, nc, prev, rc); });
 }
 
 // ---- host side ----

@@ -29,22 +29,8 @@ constexpr int K32_B_BYTES = K32_BN * K32_BK * 4;                   //  8 KB
 constexpr int K32_STAGE_BYTES = K32_A_BYTES + K32_B_BYTES;
 constexpr int K32_SMEM_BYTES = K32_NBUF * K32_STAGE_BYTES;
 constexpr int K32_FETCH = 6;                                       // load instructions per fetching wave and slab
-constexpr uint32_t K32_OOB = 0x80000000u;
 
 typedef __attribute__((address_space(3))) void* k32_lds_t;
-
-template <int I, int N, typename F>
-__device__ __forceinline__ void k32_static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        k32_static_for<I + 1, N>(f);
-    }
-}
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t k32_rsrc(const void* base, long long span_bytes) {
-    const int n = span_bytes <= 0 ? 0 : (span_bytes > 0x7fffffffll ? 0x7fffffff : (int)span_bytes);
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, n, 0x00020000);
-}
 
 // (a bit cast applied directly to one element of a vector reads the wrong element with this compiler: pass the element by value)
 __device__ __forceinline__ uint32_t k32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
@@ -105,19 +91,19 @@ __global__ void __launch_bounds__(512) gemm_pipe32k_kernel(GemmArgs g, int tiles
             if (f_id >= total) return false;
             const unsigned z = f_id / (unsigned)tiles_m;
             const int m0 = (int)(f_id - z * (unsigned)tiles_m) * K32_BM, k0 = f_s * K32_BK, kleft = g.k - k0;
-            const __amdgpu_buffer_rsrc_t ra = k32_rsrc((const float*)g.A + (long long)z * g.a_bs, a_span);
-            const __amdgpu_buffer_rsrc_t rb = k32_rsrc((const float*)g.B + (long long)z * g.b_bs, b_span);
+            const __amdgpu_buffer_rsrc_t ra = buffer_rsrc((const float*)g.A + (long long)z * g.a_bs, a_span);
+            const __amdgpu_buffer_rsrc_t rb = buffer_rsrc((const float*)g.B + (long long)z * g.b_bs, b_span);
             const int sa = A_MC ? (int)((((long long)(k0 + 8 * p)) * a_ks + m0) * 4) : (int)(((long long)(m0 + 32 * p) * a_fs + k0) * 4);
             const int sb = B_MC ? (int)(((long long)(k0 + 8 * p)) * b_ks * 4) : (int)(((long long)(16 * p) * b_fs + k0) * 4);
             unsigned char* dst = k32_smem + f_stage * K32_STAGE_BYTES;
 #pragma unroll
             for (int q = 0; q < 4; q++)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (k32_lds_t)(dst + (A_MC ? 8 * p * 512 : 32 * p * 128) + q * 1024), 16,
-                                                         a_k[q] < kleft ? (int)a_off[q] : (int)K32_OOB, sa, 0, 0);
+                                                         a_k[q] < kleft ? (int)a_off[q] : (int)BUFFER_OOB, sa, 0, 0);
 #pragma unroll
             for (int q = 0; q < 2; q++)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (k32_lds_t)(dst + K32_A_BYTES + (B_MC ? 8 * p * 256 : 16 * p * 128) + q * 1024), 16,
-                                                         b_k[q] < kleft ? (int)b_off[q] : (int)K32_OOB, sb, 0, 0);
+                                                         b_k[q] < kleft ? (int)b_off[q] : (int)BUFFER_OOB, sb, 0, 0);
             f_stage = f_stage + 1 == K32_NBUF ? 0 : f_stage + 1;
             if (++f_s == nslab) { f_s = 0; f_id += stride; }
             return true;
@@ -195,7 +181,7 @@ __global__ void __launch_bounds__(512) gemm_pipe32k_kernel(GemmArgs g, int tiles
     auto slab_pass = [&](int next) {
         const unsigned char* next_base = k32_smem + next * K32_STAGE_BYTES;
         __syncthreads();                                   // the next slab is in LDS; this slab's values have all arrived in registers
-        k32_static_for<0, 4>([&](auto uc) {
+        static_for<0, 4>([&](auto uc) {
             constexpr int u = decltype(uc)::value;
 #pragma unroll
             for (int e = 0; e < 4; e++)
@@ -207,7 +193,7 @@ __global__ void __launch_bounds__(512) gemm_pipe32k_kernel(GemmArgs g, int tiles
 
     __syncthreads();                                   // slab 0 is in LDS
     if (first >= total) return;
-    k32_static_for<0, 4>([&](auto uc) { read_group(k32_smem, uc); });
+    static_for<0, 4>([&](auto uc) { read_group(k32_smem, uc); });
     int next = 1;
     for (unsigned id = first; id < total; id += stride) {
 #pragma unroll
@@ -217,16 +203,16 @@ __global__ void __launch_bounds__(512) gemm_pipe32k_kernel(GemmArgs g, int tiles
         // register v of tile j is row 8(v / 4) + 4h + v % 4, columns 32 j + r
         const unsigned z = id / (unsigned)tiles_m;
         const int gm0 = (int)(id - z * (unsigned)tiles_m) * K32_BM + 32 * wave;
-        const __amdgpu_buffer_rsrc_t rc = k32_rsrc((float*)g.C + (long long)z * g.c_bs, c_span);
+        const __amdgpu_buffer_rsrc_t rc = buffer_rsrc((float*)g.C + (long long)z * g.c_bs, c_span);
         auto place = [&](auto nc, int& soff, uint32_t& voff) {
             constexpr int n = decltype(nc)::value, j = n >> 4, v = n & 15, row = 8 * (v / 4) + (v % 4);
             const int gm = gm0 + row;
             soff = (int)(((long long)gm * g.c_rs + (long long)(32 * j) * g.c_cs) * 4);
             voff = c_lane;
-            if constexpr (EDGE) voff = (gm + 4 * h < g.m && 32 * j + r < g.n) ? c_lane : K32_OOB;
+            if constexpr (EDGE) voff = (gm + 4 * h < g.m && 32 * j + r < g.n) ? c_lane : BUFFER_OOB;
         };
         if constexpr (EPI) {
-            if (accum) k32_static_for<0, 32>([&](auto nc) {
+            if (accum) static_for<0, 32>([&](auto nc) {
                 int soff; uint32_t voff;
                 place(nc, soff, voff);
                 old[decltype(nc)::value] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rc, (int)voff, soff, 0));
@@ -237,7 +223,7 @@ __global__ void __launch_bounds__(512) gemm_pipe32k_kernel(GemmArgs g, int tiles
             next = next + 1 == K32_NBUF ? 0 : next + 1;
         }
         // the tile's stores
-        k32_static_for<0, 32>([&](auto nc) {
+        static_for<0, 32>([&](auto nc) {
             constexpr int n = decltype(nc)::value, j = n >> 4, v = n & 15;
             int soff; uint32_t voff;
             place(nc, soff, voff);
