@@ -316,7 +316,7 @@ def cpu_baseline_configs():
     return out
 
 
-def skinny_times(capi, quick_reps=20, rows=(1, 8, 32)):
+def skinny_times(capi, quick_reps=20, rows=(1, 8, 16, 32)):
     """Config 5a: bf16 A[m, 8192] x W[8192, 8192], replayed from a HIP graph; bytes are A, W and the output once."""
     out = {}
     rng = np.random.default_rng(4)

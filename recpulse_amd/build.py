@@ -14,7 +14,7 @@ LIB_DIR = os.path.join(HERE, "lib")
 BUILD_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(LIB_DIR, "librp_hip.so")
 SOURCES = ["rp_runtime.hip", "rp_elementwise.hip", "rp_gemm.hip", "rp_gemm_generic.hip", "rp_gemm_mfma16.hip", "rp_gemm_mfma16_256.hip",
-           "rp_gemm_mfma16_128.hip", "rp_gemm_mfma16_64.hip", "rp_gemm_mfma16_64x256.hip", "rp_gemm_mfma16_64x128.hip", "rp_gemm_mfma16_skinny.hip", "rp_gemm_mfmaw.hip", "rp_gemm_tiny.hip", "rp_gemm_direct32.hip", "rp_gemm_pipe32.hip", "rp_gemm_pipe16.hip", "rp_gemm_pipe16k.hip", "rp_gemm_pipe32k.hip",
+           "rp_gemm_mfma16_128.hip", "rp_gemm_mfma16_64.hip", "rp_gemm_mfma16_64x256.hip", "rp_gemm_mfma16_64x128.hip", "rp_gemm_mfma16_skinny.hip", "rp_gemm_mfma16_stream128.hip", "rp_gemm_mfmaw.hip", "rp_gemm_tiny.hip", "rp_gemm_direct32.hip", "rp_gemm_pipe32.hip", "rp_gemm_pipe16.hip", "rp_gemm_pipe16k.hip", "rp_gemm_pipe32k.hip",
            "rp_attention.hip", "rp_attention_f32.hip", "rp_conv.hip", "rp_rnn.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed-fp32 code generation is switched off for all device code

@@ -179,6 +179,8 @@ int* noalloc_arrival_counters();
 int launch_generic(const GemmArgs& g, int dtype);
 int launch_skinny(const GemmArgs& g, int dtype);
 int launch_mfma16(const GemmArgs& g, const Plan& p, int dtype);
+bool stream128_takes(const GemmArgs& g);          // few rows, row-major A and B: the streaming kernel on 128-column strips
+int launch_stream128(const GemmArgs& g, int dtype);
 int launch_mfmaw(const GemmArgs& g, const Plan& p, int dtype);
 int launch_tiny(const GemmArgs& g, int dtype);
 // The tiles of this workgroup in a grid of resident workgroups (one per CU): first, first + stride, ... below last.

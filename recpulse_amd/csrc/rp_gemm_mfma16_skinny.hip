@@ -1,9 +1,11 @@
-// bf16 / fp16 GEMMs with few rows (m <= 32) and deep k: the cost is streaming B once from HBM.
+// bf16 / fp16 GEMMs with few rows and deep k: the cost is streaming B once from HBM.
 //
-// Row-major A (m <= 16) times row-major B takes the streaming kernel below: B never touches LDS, and the k
-// splits are added inside the same launch by the last block to arrive.  Other operand layouts and 17..32 rows
-// take the tiled kernel with a 32 x 128 block tile, whose fp32 partials a second kernel combines.  Both split k
-// across the grid so that enough waves stream B to saturate HBM, and both add the splits in split order.
+// Row-major A times row-major B takes a streaming kernel, in which B never touches LDS and the k splits are added
+// inside the same launch by the last block to arrive: the one below on 256-column strips up to 4 rows, the one in
+// rp_gemm_mfma16_stream128.hip on 128-column strips up to 32 rows (this one again, up to 16 rows, when that one is
+// switched off).  Other operand layouts and more rows take the tiled kernel with a 32 x 128 block tile, whose fp32
+// partials a second kernel combines.  All split k across the grid so that enough waves stream B to saturate HBM,
+// and all add the splits in split order.
 #include "rp_gemm_mfma16_kernel.h"
 
 
@@ -299,7 +301,11 @@ static int launch_skinny16_t(const GemmArgs& g, const Plan& p, float* partials, 
 
 int launch_mfma16_skinny(const GemmArgs& g, const Plan& p, int dtype) {
     if (dtype != RP_DTYPE_BFLOAT16 && dtype != RP_DTYPE_FLOAT16) { set_error("mfma16 skinny GEMM: unsupported dtype %d", dtype); return -1; }
-    if (g.batch == 1 && !p.a_mc && p.b_mc && g.m <= SS_MAX_M && !path_disabled("stream16")) return launch_stream16(g, dtype);
+    // row-major A and B: 256-column strips up to 4 rows (0.2 us faster there), 128-column strips up to 32 rows
+    const bool wide = g.batch == 1 && !p.a_mc && p.b_mc && g.m <= SS_MAX_M && !path_disabled("stream16");
+    const bool narrow = !p.a_mc && p.b_mc && stream128_takes(g);
+    if (wide && (g.m <= 4 || !narrow)) return launch_stream16(g, dtype);
+    if (narrow) return launch_stream128(g, dtype);
     constexpr int BN = 128;
     const int tiles = ((g.n + BN - 1) / BN) * ((g.m + 31) / 32) * g.batch;
     // about three blocks per CU in flight, each split at least four slabs deep

@@ -1,0 +1,264 @@
+// bf16 / fp16 GEMMs with at most 32 rows, row-major A and B, deep k: the streaming kernel on 128-column strips.
+#include "rp_gemm_mfma16_kernel.h"
+#include "rp_gemm_splitk_finish.h"
+
+namespace rp {
+
+// ============================================================================
+// Like the 256-column streaming kernel (rp_gemm_mfma16_skinny.hip), B goes from
+// memory to registers to the MFMAs without touching LDS, k is split over the
+// four waves of a workgroup and over the workgroups of a column group, and the
+// last workgroup of a group to arrive adds the group's fp32 partials through
+// the XCD's L2.  What differs is the strip: a wave owns 128 adjacent columns
+// (256 bytes of a row of B), so a grid of one workgroup per CU needs half as
+// many splits of k, and the partial sums that the finishing workgroup reads are
+// a quarter of the wider kernel's for the same number of rows.
+//
+// A round is 16 RS rows of k (RS = 2: 32 rows), multiplied in RS steps of 16, one
+// v_mfma_f32_16x16x16 per 16 x 16 output tile and step.  In that instruction
+// lane (q, j) = (lane / 16, lane % 16) supplies four k values of row j (A) or
+// column j (B), and any assignment of a round's k values to (step, q) works as
+// long as A and B agree.  It is chosen for A's sake: lane (q, j) loads the 8 RS
+// bytes A[j][4 RS q .. 4 RS q + 4 RS - 1] of the round with one instruction (the
+// four q lanes of a row read one contiguous piece of the row's cache line), and
+// step t uses k = 4 RS q + 4t .. + 3.  With the natural assignment (k = 16t + 4q ..,
+// RS = 1) every step fetches 8 bytes out of each row's line again; these are L2
+// hits, but at 16 rows they cost 1.3 us per launch.  Longer rounds save more of
+// them and deal k to the waves in coarser pieces, which B's stream likes less:
+// at RS = 4 the launch takes 0.3 us longer than at RS = 2 for every m, and
+// RS = 1 is the faster one only below 8 rows (m = 32: 29.3 / 27.0 / 27.9 us for
+// RS = 1 / 2 / 4).
+// For B, step t reads rows 4 RS q + 4t + e (e = 0 .. 3): lane (q, j) loads 16
+// bytes (columns 8j .. 8j+7) of each, a load instruction covers four 256-byte
+// row segments 4 RS rows apart, and the 4 x 8 block of 16-bit values a lane
+// holds is transposed in registers (byte permutes) into 8 B-operands, one per
+// column residue c: operand c carries column 8j + c.  MFMA (f, c) accumulates the
+// 16 x 16 tile of rows 16f .. 16f+15 and columns {8j + c}.
+//
+// 256-byte strips stream at the full rate only with about 8 KB of loads in
+// flight per wave (a read-only probe: 19.5 - 20.2 us for 134 MB with two steps
+// in flight, 23.6 with one, 21.6 with three), so a wave keeps two steps of 4 KB
+// in flight, across round boundaries.  A's registers alternate between two sets
+// by round; a set is refilled for the round after next as soon as its last step
+// has copied its operands out.  The loop body is a pair of rounds, so that
+// register sets and slots are compile-time choices and nothing is copied at the
+// back edge.
+// ============================================================================
+constexpr int S8_WAVES = 4, S8_COLS = 128, S8_STEP = 16, S8_PITCH = S8_COLS + 8;
+constexpr int S8_MAX_M = 32;
+constexpr int S8_RS = 2;                // steps per round: 32 rows of k
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
+
+template <typename T> struct s8_ops;
+template <> struct s8_ops<bf16_t> {
+    static __device__ __forceinline__ f32x4_t mma(u32x2_t a, u32x2_t b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a), __builtin_bit_cast(s16x4_t, b), c, 0, 0, 0);
+    }
+};
+template <> struct s8_ops<f16_t> {
+    static __device__ __forceinline__ f32x4_t mma(u32x2_t a, u32x2_t b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a), __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
+    }
+};
+
+template <typename T, int MR, int RS>
+__global__ void __launch_bounds__(256) gemm_stream128_kernel(GemmArgs g, float* partials, int groups, int nsplit, int* arrivals, int local) {
+    constexpr int NF = MR / 16;                                           // A fragments (16 rows each)
+    constexpr int S8_ROUND = S8_STEP * RS;                                // k rows of a round (RS steps)
+    extern __shared__ __attribute__((aligned(16))) float red[];          // [S8_WAVES][MR][S8_PITCH]
+    __shared__ bool arrived_last;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);       // scalar, so that buffer descriptors built from it are too
+    const int q = lane >> 4, j = lane & 15;
+    // block b stands for (XCD b % 8, slot b / 8): all splits of column group 8i + x run on XCD x
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int group = (slot / nsplit) * 8 + xcd, split = slot % nsplit;
+    if (group >= groups) return;                                           // (whole blocks, before any barrier)
+    const int n0 = group * S8_COLS;
+    // rounds are dealt cyclically: round r of k belongs to split r % nsplit and, inside the block, to wave (r / nsplit) % 4
+    const int total_rounds = (g.k + S8_ROUND - 1) / S8_ROUND;
+    const int mine = total_rounds > split ? (total_rounds - split + nsplit - 1) / nsplit : 0;      // rounds of this block
+    const int my_rounds = mine > wave ? (mine - wave + S8_WAVES - 1) / S8_WAVES : 0;               // and of this wave
+
+    const uint16_t* Bm = (const uint16_t*)g.B;
+    const uint16_t* Am = (const uint16_t*)g.A;
+    const long long b_rs = g.b_rs, a_rs = g.a_rs;
+    const char* b_end = (const char*)(Bm + ((long long)(g.k - 1) * b_rs + g.n));
+    const char* a_end = (const char*)(Am + ((long long)(g.m - 1) * a_rs + g.k));
+    const int b_step = (int)(4 * b_rs * 2);                               // bytes from a step's rows to the next step's
+
+    uint32_t b_off[4], a_off[NF];
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+        b_off[e] = (n0 + 8 * j < g.n) ? (uint32_t)(((long long)(4 * RS * q + e) * b_rs + 8 * j) * 2) : BUFFER_OOB;      // (n is a multiple of 8)
+#pragma unroll
+    for (int f = 0; f < NF; f++)
+        a_off[f] = (16 * f + j < g.m) ? (uint32_t)(((long long)(16 * f + j) * a_rs + 4 * RS * q) * 2) : BUFFER_OOB;
+    auto round_k = [&](int r) { return ((r * S8_WAVES + wave) * nsplit + split) * S8_ROUND; };
+
+    u32x4_t raw[2][4];                 // two steps of B in flight
+    uint32_t a_buf[2][NF][2 * RS];     // a lane's 4 * RS k values of a round, per fragment; rounds alternate between the two sets
+    // request step t of round r of this wave into register slot SLOT (rounds beyond the wave's share read zeros)
+    auto request_b = [&](auto slotc, int r, int t) {
+        constexpr int SLOT = decltype(slotc)::value;
+        const int kr = round_k(r);
+        const char* bb = (const char*)(Bm + (long long)kr * b_rs + n0);
+        __amdgpu_buffer_rsrc_t b_rsrc = buffer_rsrc(bb, r < my_rounds ? (long long)(b_end - bb) : 0);
+#pragma unroll
+        for (int e = 0; e < 4; e++) raw[SLOT][e] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, (int)b_off[e], t * b_step, 2);       // (streamed: read once)
+    };
+    auto request_a = [&](auto parc, int r) {
+        uint32_t (&dst)[NF][2 * RS] = a_buf[decltype(parc)::value];
+        const int kr = round_k(r);
+        const char* ab = (const char*)(Am + kr);
+        __amdgpu_buffer_rsrc_t a_rsrc = buffer_rsrc(ab, r < my_rounds ? (long long)(a_end - ab) : 0);
+#pragma unroll
+        for (int f = 0; f < NF; f++) {
+            if constexpr (RS == 1) {                         // (k is a multiple of 8 and the quad starts at a multiple of 4: wholly in or out)
+                const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(a_rsrc, (int)((kr + 4 * q < g.k) ? a_off[f] : BUFFER_OOB), 0, 0);
+                dst[f][0] = v[0]; dst[f][1] = v[1];
+            } else {
+#pragma unroll
+                for (int hh = 0; hh < RS / 2; hh++) {        // eight k values at a time, wholly in or out
+                    const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)((kr + 4 * RS * q + 8 * hh < g.k) ? a_off[f] + 16 * hh : BUFFER_OOB), 0, 0);
+                    dst[f][4 * hh] = v[0]; dst[f][4 * hh + 1] = v[1]; dst[f][4 * hh + 2] = v[2]; dst[f][4 * hh + 3] = v[3];
+                }
+            }
+        }
+    };
+
+    f32x4_t acc[NF][8];
+#pragma unroll
+    for (int f = 0; f < NF; f++)
+#pragma unroll
+        for (int c = 0; c < 8; c++) acc[f][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    // Step S of a pair of rounds (S = 0 .. 2 RS - 1: round r0 + S / RS, its step S % RS): multiply it out of slot
+    // S % 2, refill the slot with the step two ahead and, after a round's last step, its A registers with the round
+    // two ahead.
+    auto consume = [&](auto sc, int r0) {
+        constexpr int S = decltype(sc)::value, SLOT = S & 1, PAR = S / RS, T_ = S % RS;
+        // in-register 4 x 8 transpose of 16-bit values: operand c, dword d = (k row 2d, k row 2d+1) of column c
+        u32x2_t opb[8];
+#pragma unroll
+        for (int c = 0; c < 8; c++)
+#pragma unroll
+            for (int d = 0; d < 2; d++)
+                opb[c][d] = __builtin_amdgcn_perm(raw[SLOT][2 * d + 1][c / 2], raw[SLOT][2 * d][c / 2], (c & 1) ? 0x07060302u : 0x05040100u);
+        // (A's quad is moved to registers of its own, so that the refill below can land in the registers it came from)
+        u32x2_t opa[NF];
+#pragma unroll
+        for (int f = 0; f < NF; f++)
+#pragma unroll
+            for (int d = 0; d < 2; d++) asm volatile("v_mov_b32 %0, %1" : "=v"(opa[f][d]) : "v"(a_buf[PAR][f][2 * T_ + d]));
+        // The operands must exist before the slot is refilled: then the refill can land in the very registers the
+        // slot occupies and nothing has to be copied (behind a full wait) at the loop's back edge.
+#pragma unroll
+        for (int c = 0; c < 8; c++) asm volatile("" : "+v"(opb[c]) : : "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        request_b(std::integral_constant<int, SLOT>{}, r0 + (S + 2) / RS, (S + 2) % RS);
+        if constexpr (T_ == RS - 1) request_a(std::integral_constant<int, PAR>{}, r0 + PAR + 2);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int f = 0; f < NF; f++)
+#pragma unroll
+            for (int c = 0; c < 8; c++) acc[f][c] = s8_ops<T>::mma(opa[f], opb[c], acc[f][c]);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // (requests stay in program order: the wait for a register counts the loads issued after its own)
+    request_a(std::integral_constant<int, 0>{}, 0);
+    request_a(std::integral_constant<int, 1>{}, 1);
+    request_b(std::integral_constant<int, 0>{}, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    request_b(std::integral_constant<int, 1>{}, 1 / RS, 1 % RS);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int r0 = 0; r0 < my_rounds; r0 += 2)
+        static_for<0, 2 * RS>([&](auto sc) { consume(sc, r0); });
+
+    // ---- the block's waves add their tiles through LDS ----
+    // accumulator register v of tile (f, c) holds row 16f + 4q + v at column 8j + c: a lane's 8 residues of one row are
+    // 8 adjacent columns, two 16-byte stores at consecutive addresses across the lanes of a row
+    const SplitkOutput<T> out(g);
+    const __amdgpu_buffer_rsrc_t part_rsrc = buffer_rsrc(partials, partials ? (long long)nsplit * g.m * g.n * 4 : 0);
+#pragma unroll
+    for (int f = 0; f < NF; f++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int r = 16 * f + 4 * q + v;
+            if (r >= g.m) continue;
+            float* dst = red + (wave * MR + r) * S8_PITCH + 8 * j;
+            *(f32x4_t*)dst = f32x4_t{acc[f][0][v], acc[f][1][v], acc[f][2][v], acc[f][3][v]};
+            *(f32x4_t*)(dst + 4) = f32x4_t{acc[f][4][v], acc[f][5][v], acc[f][6][v], acc[f][7][v]};
+        }
+    __syncthreads();
+    constexpr int QPR = S8_COLS / 4;                     // quads per row of the block's columns
+#pragma unroll
+    for (int i = 0; i < MR / 8; i++) {
+        const int idx = threadIdx.x + 256 * i, r = idx / QPR, gn = n0 + (idx % QPR) * 4;
+        if (r >= g.m || gn >= g.n) continue;                             // n is a multiple of 4, so a quad is wholly in or out
+        const int at_lds = r * S8_PITCH + (idx % QPR) * 4;
+        f32x4_t sum = *(const f32x4_t*)(red + at_lds);
+#pragma unroll
+        for (int w = 1; w < S8_WAVES; w++) sum += *(const f32x4_t*)(red + w * MR * S8_PITCH + at_lds);
+        if (nsplit > 1) {
+            const long long at = ((long long)split * g.m + r) * g.n + gn;
+            if (!arrivals) *(f32x4_t*)(partials + at) = sum;
+            else if (local) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sum), part_rsrc, (int)(at * 4), 0, 0);
+            else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sum), part_rsrc, (int)(at * 4), 0, SPLITK_DEVICE_SCOPE);
+        } else out.store_quad(r, gn, sum);
+    }
+    if (nsplit == 1 || !arrivals) return;
+
+    // ---- single-launch finish: the last block of this column group to arrive adds all splits ----
+    if (!splitk_arrive(arrivals + group, nsplit, local != 0, &arrived_last)) return;
+    splitk_finish_window<T, S8_COLS, MR / 8, 4>(g, out, part_rsrc, nsplit, 0, g.m, n0, local != 0, arrivals + group);
+}
+
+template <typename T, int MR, int RS>
+static int launch_stream128_mr(const GemmArgs& g, float* partials, int groups, int nsplit, int* arrivals, int local) {
+    constexpr size_t smem = (size_t)S8_WAVES * MR * S8_PITCH * sizeof(float);
+    auto kern = gemm_stream128_kernel<T, MR, RS>;
+    if (smem > 64 * 1024 && !check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem), "hipFuncSetAttribute")) return -1;
+    hipLaunchKernelGGL(kern, dim3(8 * ((groups + 7) / 8) * nsplit), dim3(256), smem, current_stream(), g, partials, groups, nsplit, arrivals, local);
+    return check_launch("gemm_stream128_kernel") ? 0 : -1;
+}
+
+template <typename T>
+static int launch_stream128_t(const GemmArgs& g, float* partials, int groups, int nsplit, int* arrivals, int local) {
+    if (g.m <= 16) return launch_stream128_mr<T, 16, S8_RS>(g, partials, groups, nsplit, arrivals, local);
+    return launch_stream128_mr<T, 32, S8_RS>(g, partials, groups, nsplit, arrivals, local);
+}
+
+bool stream128_takes(const GemmArgs& g) {
+    return g.batch == 1 && g.m <= S8_MAX_M && g.a_cs == 1 && g.b_cs == 1 && g.n % 8 == 0 && g.k % 8 == 0 && !path_disabled("stream128");
+}
+
+int launch_stream128(const GemmArgs& g, int dtype) {
+    const int groups = (g.n + S8_COLS - 1) / S8_COLS;
+    constexpr int QUANTUM = S8_WAVES * S8_STEP * S8_RS;             // k rows one pass of a block's waves covers
+    // one block per CU (a wave per SIMD), each at least two passes deep
+    const int cus = device_cu_count() >= 8 ? device_cu_count() / 8 * 8 : 256;
+    int nsplit = (cus + groups - 1) / groups;
+    int max_split = g.k / (2 * QUANTUM) > 0 ? g.k / (2 * QUANTUM) : 1;
+    if (nsplit > max_split) nsplit = max_split;
+    const size_t part_bytes = (size_t)nsplit * g.m * g.n * sizeof(float);
+    void* ws = nullptr;
+    if (nsplit > 1 && gemm_workspace(&ws, part_bytes) != 0) return -1;
+    int* arrivals = nullptr;
+    if (nsplit > 1) {
+        bool failed = false;
+        arrivals = splitk_arrival_counters(groups, part_bytes, &failed);
+        if (failed) { gemm_workspace_release(ws); return -1; }
+    }
+    const int local = arrivals && workgroups_share_xcd_by_residue() ? 1 : 0;
+    int rc;
+    if (dtype == RP_DTYPE_BFLOAT16) rc = launch_stream128_t<bf16_t>(g, (float*)ws, groups, nsplit, arrivals, local);
+    else rc = launch_stream128_t<f16_t>(g, (float*)ws, groups, nsplit, arrivals, local);
+    if (rc == 0 && nsplit > 1 && !arrivals) rc = launch_splitk_combine(g, (const float*)ws, nsplit, g.m, dtype);
+    if (ws) gemm_workspace_release(ws);          // back to the pool while the kernels are still queued: safe for later work on this stream; held with the graph while one is being recorded
+    return rc;
+}
+
+}  // namespace rp

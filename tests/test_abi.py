@@ -45,9 +45,10 @@ def test_kernel_selection_names():
     assert name(1, 8192, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "mfma16_256x256"
     assert name(1, 8192, 8192, 8192, (1, 8192), (8192, 1), (8192, 1), capi.F16) == "mfma16_256x256"       # A^T view
     assert name(1, 1, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "mfma16_stream_32x256"
-    assert name(1, 8, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "mfma16_stream_32x256"
-    assert name(1, 16, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F16) == "mfma16_stream_32x256"
-    assert name(1, 32, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F16) == "mfma16_skinny_32x128"
+    assert name(1, 8, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "mfma16_stream_32x128"      # above 4 rows: 128-column strips
+    assert name(1, 16, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F16) == "mfma16_stream_32x128"
+    assert name(1, 32, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F16) == "mfma16_stream_32x128"
+    assert name(1, 33, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F16) == "mfma16_skinny_32x128"
     assert name(1, 8, 8192, 8192, (8192, 1), (1, 8192), (8192, 1), capi.BF16) == "mfma16_skinny_32x128"
     assert name(1, 8, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F32) == "skinny"
     assert name(1, 128, 784, 256, (784, 1), (256, 1), (256, 1), capi.F32) == "tiny32_16x16"          # a small fp32 output: one launch of 16 x 16 tiles

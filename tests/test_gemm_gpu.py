@@ -249,7 +249,7 @@ def test_skinny_rows_mfma_split_k(dt, layout):
             continue                                   # a transposed A needs whole 16-byte vectors along m
         a, b = _operands(rng, m, k, n, dt, layout)
         a_st = (a.strides[0] // 2, a.strides[1] // 2); b_st = (b.strides[0] // 2, b.strides[1] // 2)
-        want_kernel = "mfma16_stream_32x256" if layout == "nn" and m <= 16 else "mfma16_skinny_32x128"
+        want_kernel = _stream_kernel(m) if layout == "nn" else "mfma16_skinny_32x128"
         assert capi.gemm_kernel_name(1, m, k, n, a_st, b_st, (n, 1), dt) == want_kernel
         bias = rand_storage(rng, (n,), dt); c0 = rand_storage(rng, (m, n), dt)
         got = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)
@@ -261,15 +261,21 @@ def test_skinny_rows_mfma_split_k(dt, layout):
     assert np.array_equal(device_gemm(a, b, dt), oracle_gemm(a, b, dt))
 
 
-@pytest.mark.parametrize("m", [1, 3, 8, 11, 16])
+def _stream_kernel(m):
+    """Row-major A and B with at most 32 rows: 256-column strips up to 4 rows, 128-column strips above."""
+    return "mfma16_stream_32x256" if m <= 4 else "mfma16_stream_32x128"
+
+
+@pytest.mark.parametrize("m", [1, 3, 5, 8, 11, 16, 17, 27, 32])
 def test_streaming_rows_single_launch_finish(m):
     """Row-major A times row-major B with few rows: one launch, the last block of a column group to arrive adds the
     k splits.  Repeated launches must reproduce the first result bit for bit (fixed summation order, counters left
-    clean), with ragged k and n, a bias and an accumulating epilogue."""
+    clean), with ragged k (a partial last round, waves with unequal numbers of rounds) and n (a partial last strip, a
+    number of strips that is not a multiple of 8), a bias and an accumulating epilogue."""
     rng = np.random.default_rng(39)
-    for dt, k, n in [(BF16, 8192, 2048), (F16, 4104, 1288), (BF16, 1024, 4096)]:
+    for dt, k, n in [(BF16, 8192, 2048), (F16, 4104, 1288), (BF16, 1024, 4096), (F16, 1064, 8200)]:
         a, b = _operands(rng, m, k, n, dt, "nn")
-        assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == "mfma16_stream_32x256"
+        assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == _stream_kernel(m)
         bias = rand_storage(rng, (n,), dt); c0 = rand_storage(rng, (m, n), dt)
         first = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)
         _check(first, a, b, dt, k, bias=bias, c_init=c0, accumulate=True)
@@ -281,7 +287,7 @@ def test_streaming_rows_single_launch_finish(m):
     assert np.array_equal(device_gemm(a, b, BF16), oracle_gemm(a, b, BF16))
 
 
-@pytest.mark.parametrize("m", [1, 8, 16])
+@pytest.mark.parametrize("m", [1, 8, 16, 32])
 def test_streaming_rows_finish_repeats_bit_for_bit_over_hundreds_of_launches(m):
     """The finish exchanges partial sums between the workgroups of a column group while other groups still stream:
     launched back to back a few hundred times on resident operands (no synchronisation in between), every launch
@@ -290,7 +296,7 @@ def test_streaming_rows_finish_repeats_bit_for_bit_over_hundreds_of_launches(m):
     k = n = 8192
     dt = BF16
     a = rand_storage(rng, (m, k), dt); b = rand_storage(rng, (k, n), dt)
-    assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == "mfma16_stream_32x256"
+    assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == _stream_kernel(m)
     da, db = capi.DeviceBuffer.from_numpy(a), capi.DeviceBuffer.from_numpy(b)
     launches = 300
     outs = [capi.DeviceBuffer(m * n * 2) for _ in range(launches)]
@@ -312,8 +318,8 @@ def test_tiled_rows_split_k_ragged(layout):
     launches reproduce the first bit for bit."""
     rng = np.random.default_rng(43)
     for dt, m, k, n in [(BF16, 32, 8192, 2048), (F16, 24, 4104, 1288), (BF16, 17, 1032, 4096), (F16, 104, 4160, 1160), (BF16, 8, 2048, 2048)]:
-        if (layout == "nn" and m <= 16) or (layout[0] == "t" and m % 8):
-            continue                                   # the streaming kernel's case; a transposed A needs whole 16-byte vectors along m
+        if (layout == "nn" and m <= 32) or (layout[0] == "t" and m % 8):
+            continue                                   # the streaming kernels' case; a transposed A needs whole 16-byte vectors along m
         a, b = _operands(rng, m, k, n, dt, layout)
         a_st = (a.strides[0] // 2, a.strides[1] // 2); b_st = (b.strides[0] // 2, b.strides[1] // 2)
         assert capi.gemm_kernel_name(1, m, k, n, a_st, b_st, (n, 1), dt) == "mfma16_skinny_32x128"
@@ -323,7 +329,7 @@ def test_tiled_rows_split_k_ragged(layout):
         for _ in range(10):
             assert np.array_equal(first, device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True))
     # integer data is exact in fp32 whatever the split: bit-equal to the oracle
-    a, b = _operands(rng, 32, 4096, 1024, BF16, layout)
+    a, b = _operands(rng, 40, 4096, 1024, BF16, layout)
     a[...] = oracle.to_storage(rng.integers(-2, 3, a.shape).astype(np.float64), BF16)
     b[...] = oracle.to_storage(rng.integers(-2, 3, b.shape).astype(np.float64), BF16)
     assert np.array_equal(device_gemm(a, b, BF16), oracle_gemm(a, b, BF16))
@@ -333,7 +339,7 @@ def test_tiled_rows_repeat_bit_for_bit_over_hundreds_of_launches():
     """The tiled k-split kernel and its combine kernel share one workspace from the pool across back-to-back launches:
     300 launches without synchronisation in between leave the bits of the first."""
     rng = np.random.default_rng(44)
-    m, k, n, dt = 32, 8192, 8192, BF16
+    m, k, n, dt = 40, 8192, 8192, BF16
     a = rand_storage(rng, (m, k), dt); b = rand_storage(rng, (k, n), dt)
     assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == "mfma16_skinny_32x128"
     da, db = capi.DeviceBuffer.from_numpy(a), capi.DeviceBuffer.from_numpy(b)

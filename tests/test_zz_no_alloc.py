@@ -49,9 +49,10 @@ def _both(rng, m, k, n, dtype, bias=False, accumulate=False, b_transposed=False)
 
 # (kernel the dispatcher picks, first shape, second smaller shape): every split-k launcher that takes a workspace
 CASES = [
-    ("mfma16_stream_32x256", BF16, (8, 4096, 4096), (4, 2048, 2048), {}),                 # partial sums + arrival counters, single launch
-    ("mfma16_stream_32x256", F16, (16, 8192, 2048), (1, 4096, 1024), {"bias": True}),
-    ("mfma16_skinny_32x128", BF16, (32, 4096, 4096), (20, 2048, 2048), {"accumulate": True}),      # tiled split-k + combine launch
+    ("mfma16_stream_32x256", BF16, (4, 4096, 4096), (2, 2048, 2048), {}),                 # partial sums + arrival counters, single launch
+    ("mfma16_stream_32x128", F16, (16, 8192, 2048), (8, 4096, 1024), {"bias": True}),     # the same on 128-column strips
+    ("mfma16_stream_32x128", BF16, (32, 4096, 4096), (20, 2048, 2048), {"accumulate": True}),
+    ("mfma16_skinny_32x128", BF16, (40, 4096, 4096), (33, 2048, 2048), {"accumulate": True}),      # tiled split-k + combine launch
     ("mfma16_skinny_32x128", BF16, (8, 4096, 2048), (8, 2048, 2048), {"b_transposed": True}),
     ("skinny", F32, (4, 4096, 4096), (2, 2048, 1024), {}),                                # VALU streaming kernel
     ("mfma32_64x64", F32, (128, 4096, 256), (64, 4096, 128), {"bias": True}),             # fp32 MFMA split-k
@@ -97,10 +98,10 @@ def test_noalloc_rejects_a_workspace_beyond_the_fixed_array():
     assert np.array_equal(want, got)
 
 
-@pytest.mark.parametrize("m,k,n", [(8, 4096, 4096), (32, 4096, 4096)])
+@pytest.mark.parametrize("m,k,n", [(4, 4096, 4096), (8, 4096, 4096), (40, 4096, 4096)])
 def test_noalloc_recorded_into_a_graph_replays_like_the_eager_call(m, k, n):
     """The callers the entry point is for include code under HIP graph capture.  After a warm eager call the entry is
-    recorded on a created stream (single-launch k-split finish at 8 rows, partial sums + combine launch at 32), the
+    recorded on a created stream (single-launch k-split finish at 4 and 8 rows, partial sums + combine launch at 40), the
     graph is replayed three times with other work and a synchronisation in between, and every replay must leave the
     eager result; neither the recording nor the replays may touch the allocator."""
     rng = np.random.default_rng(74)
