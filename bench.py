@@ -392,8 +392,31 @@ def square_sweep(capi, sizes=(1024, 4096)):
     return out
 
 
+def skinny_fresh_process(rows=(1, 8, 16, 32)):
+    """The same few-row launches, each row timed by a child process that runs nothing else.  A launch of these kernels
+    takes 1.0 - 1.4 us longer once the process has run certain other kernels after its first few-row launch (a 1024^3
+    GEMM does it, a second kernel type of the few-row family does it; the kernel trace shows the time inside the kernel;
+    the cause was not found), so the figure of a row depends on what ran before it.  `us` in the table is the row timed
+    in this process, in the order 1, 8, 16, 32 after the headline GEMMs; this is the row alone in a process of its own."""
+    import subprocess
+    out = {}
+    for m in rows:
+        try:
+            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--skinny-row", str(m)], capture_output=True, text=True, timeout=180)
+            out[m] = json.loads(r.stdout.strip().splitlines()[-1])["us"] if r.returncode == 0 else None
+        except Exception:
+            out[m] = None
+    return out
+
+
 def secondary(capi, quick_reps=20):
     out = skinny_times(capi, quick_reps)
+    k = n = 8192
+    for m, us in skinny_fresh_process().items():
+        row = out.get(f"skinny_bf16_m{m}")
+        if row is not None and us is not None:
+            row["us_fresh_process"] = us
+            row["frac_hbm_fresh_process"] = (m * k + k * n + m * n) * 2 / (us * 1e-6) / 1e9 / PEAK_HBM_GBS
     out["square_sweep"] = square_sweep(capi)
     out["gemm_f16_8192"] = f16_time(capi)
     out.update(wide_times(capi))
@@ -747,6 +770,7 @@ def main():
     ap.add_argument("--data", choices=["normal", "ints", "ones", "zeros"], default="normal",
                     help="operand values of the headline GEMMs: N(0,1) (the configuration) or low-toggle data, to show how far the "
                          "power-managed shader clock, and with it the throughput, depends on the values multiplied")
+    ap.add_argument("--skinny-row", type=int, default=0, help="time the few-row bf16 GEMM with this many rows and nothing else (what --skinny figures 'fresh process' come from)")
     ap.add_argument("--skinny-only", action="store_true",
                     help="run only the few-row bf16 GEMMs of configuration 5a and print their figures (for profiling that kernel alone)")
     ap.add_argument("--wide-only", action="store_true",
@@ -796,6 +820,9 @@ def main():
         return
     if args.skinny_only:
         print(json.dumps({"skinny": skinny_times(capi, rows=(1, 8, 32))}))
+        return
+    if args.skinny_row > 0:
+        print(json.dumps({"us": skinny_times(capi, rows=(args.skinny_row,))[f"skinny_bf16_m{args.skinny_row}"]["us"]}))
         return
     if args.sweep_only:
         print(json.dumps({"square_sweep": square_sweep(capi)}))
