@@ -179,7 +179,8 @@ int* noalloc_arrival_counters();
 int launch_generic(const GemmArgs& g, int dtype);
 int launch_skinny(const GemmArgs& g, int dtype);
 int launch_mfma16(const GemmArgs& g, const Plan& p, int dtype);
-bool stream128_takes(const GemmArgs& g);          // few rows, row-major A and B: the streaming kernel on 128-column strips
+bool stream128_shape(int batch, int m, int k, int n);      // shapes the streaming kernel on 128-column strips is chosen for (row-major A and B)
+bool stream128_takes(const GemmArgs& g);
 int launch_stream128(const GemmArgs& g, int dtype);
 int launch_mfmaw(const GemmArgs& g, const Plan& p, int dtype);
 int launch_tiny(const GemmArgs& g, int dtype);

@@ -91,10 +91,8 @@ static Plan make_plan(int batch, int m, int k, int n, long long a_rs, long long 
     if (is16 && mfma_ok && few_rows && n % 8 == 0 && n >= 256 && k >= 1024 &&
         (long long)k * n >= (1ll << 22)) {
         p.fam = FAM_MFMA16_SKINNY; p.bm = 32; p.bn = 128; p.edge = true; p.a_mc = !a_kc; p.b_mc = b_mc;
-        // row-major A and B: the streaming kernels (256-column strips up to 4 rows, 128-column strips up to 32)
-        const bool nn = batch == 1 && !p.a_mc && p.b_mc;
-        const bool narrow = nn && m <= 32 && k % 8 == 0 && !path_disabled("stream128"), wide = nn && m <= 16 && !path_disabled("stream16");
-        p.name = (wide && (m <= 4 || !narrow)) ? "mfma16_stream_32x256" : narrow ? "mfma16_stream_32x128" : "mfma16_skinny_32x128";
+        // row-major A and B with at most 32 rows: the streaming kernel, for the shapes it is the right one for
+        p.name = (batch == 1 && !p.a_mc && p.b_mc && stream128_shape(batch, m, k, n)) ? "mfma16_stream_32x128" : "mfma16_skinny_32x128";
         return p;
     }
     // VALU skinny: few rows, row-major B, enough columns and depth to be worth streaming

@@ -1,18 +1,40 @@
-// bf16 / fp16 GEMMs with at most 32 rows, row-major A and B, deep k: the streaming kernel on 128-column strips.
+// bf16 / fp16 GEMMs with at most 32 rows, row-major A and B, deep k: the streaming kernel (128-column strips).
 #include "rp_gemm_mfma16_kernel.h"
 #include "rp_gemm_splitk_finish.h"
 
 namespace rp {
 
 // ============================================================================
-// Like the 256-column streaming kernel (rp_gemm_mfma16_skinny.hip), B goes from
-// memory to registers to the MFMAs without touching LDS, k is split over the
-// four waves of a workgroup and over the workgroups of a column group, and the
-// last workgroup of a group to arrive adds the group's fp32 partials through
-// the XCD's L2.  What differs is the strip: a wave owns 128 adjacent columns
-// (256 bytes of a row of B), so a grid of one workgroup per CU needs half as
-// many splits of k, and the partial sums that the finishing workgroup reads are
-// a quarter of the wider kernel's for the same number of rows.
+// B goes from memory to registers to the MFMAs without touching LDS.  One wave
+// owns 128 adjacent columns of B (256 bytes of a row) and a set of "rounds" of
+// k; the four waves of a workgroup share the columns and split k, and so do the
+// workgroups of a column group, so that one workgroup per CU streams B.
+//
+// Rounds are dealt cyclically: round r of k belongs to split r % nsplit, and
+// inside a block to wave (r / nsplit) % 4.  At any moment the grid as a whole
+// therefore reads one contiguous window of B (nsplit * 4 rounds of whole rows),
+// which the memory system serves 5 - 8 % faster than the same blocks each
+// walking a range of k of its own (the ranges lie a power of two apart).  Loads
+// are issued unconditionally (out-of-range rounds get an empty buffer
+// descriptor and read zeros), so the waits the compiler inserts count loads
+// exactly.
+//
+// The block's 4 waves add their tiles through LDS in wave order and the block
+// writes one fp32 partial (or, without a k split, the finished output).  With
+// `arrivals` the block then counts itself in, and the last block of its column
+// group to do so adds the group's partials in split order and writes the output
+// (otherwise a second kernel does).  Strips of 128 columns rather than wider
+// ones keep that finish small: with one workgroup per CU an 8192-column output
+// takes 4 splits, and the finishing block reads 4 x m rows of 512 bytes.
+//
+// Placement.  The grid is one-dimensional and block b stands for (XCD x = b % 8,
+// slot b / 8): workgroups are dealt to the XCDs round robin, so all splits of
+// column group 8i + x are given slots of XCD x.  When the host has verified that
+// rule on the device (`local`), the partials and the arrival count never leave
+// that XCD's L2: plain stores (complete when the L2 has them), an atomic that the
+// L2 executes, and plain loads (the finishing CU's vector cache holds none of
+// them yet).  Otherwise they are exchanged at device scope (written through to
+// memory and read back from there), which costs about 1.5 us more per launch.
 //
 // A round is 16 RS rows of k (RS = 2: 32 rows), multiplied in RS steps of 16, one
 // v_mfma_f32_16x16x16 per 16 x 16 output tile and step.  In that instruction
@@ -231,18 +253,32 @@ static int launch_stream128_t(const GemmArgs& g, float* partials, int groups, in
     return launch_stream128_mr<T, 32, S8_RS>(g, partials, groups, nsplit, arrivals, local);
 }
 
-bool stream128_takes(const GemmArgs& g) {
-    return g.batch == 1 && g.m <= S8_MAX_M && g.a_cs == 1 && g.b_cs == 1 && g.n % 8 == 0 && g.k % 8 == 0 && !path_disabled("stream128");
+// k splits for an output of n columns: one block per CU (a wave per SIMD), each at least two passes of its waves deep
+static int stream128_nsplit(int k, int n) {
+    const int groups = (n + S8_COLS - 1) / S8_COLS;
+    constexpr int QUANTUM = S8_WAVES * S8_STEP * S8_RS;      // k rows one pass of a block's waves covers
+    const int cus = device_cu_count() >= 8 ? device_cu_count() / 8 * 8 : 256;
+    const int nsplit = (cus + groups - 1) / groups;
+    const int max_split = k / (2 * QUANTUM) > 0 ? k / (2 * QUANTUM) : 1;
+    return nsplit < max_split ? nsplit : max_split;
 }
+
+// Shapes the kernel is the right one for.  A narrow output with a deep k would need many splits, and the one block
+// that finishes a column group reads nsplit x m rows of 512 bytes: beyond 256 such rows the tiled kernel with its
+// separate combine launch is faster (32 x 8192 x 2048: 16.1 us here against 14.1).  So it is for a B under 32 MB that
+// needs more than 8 splits, where two short launches beat one launch with a finish chain (16 x 4096 x 2048: 10.4 us
+// here against 8.5; 2 x 8192 x 1024: 10.9 against 8.4).
+bool stream128_shape(int batch, int m, int k, int n) {
+    if (batch != 1 || m > S8_MAX_M || n % 8 || k % 8 || path_disabled("stream128")) return false;
+    const int nsplit = stream128_nsplit(k, n);
+    return (long long)nsplit * m <= 256 && (nsplit <= 8 || (long long)k * n >= (1ll << 24));
+}
+
+bool stream128_takes(const GemmArgs& g) { return g.a_cs == 1 && g.b_cs == 1 && stream128_shape(g.batch, g.m, g.k, g.n); }
 
 int launch_stream128(const GemmArgs& g, int dtype) {
     const int groups = (g.n + S8_COLS - 1) / S8_COLS;
-    constexpr int QUANTUM = S8_WAVES * S8_STEP * S8_RS;             // k rows one pass of a block's waves covers
-    // one block per CU (a wave per SIMD), each at least two passes deep
-    const int cus = device_cu_count() >= 8 ? device_cu_count() / 8 * 8 : 256;
-    int nsplit = (cus + groups - 1) / groups;
-    int max_split = g.k / (2 * QUANTUM) > 0 ? g.k / (2 * QUANTUM) : 1;
-    if (nsplit > max_split) nsplit = max_split;
+    const int nsplit = stream128_nsplit(g.k, g.n);
     const size_t part_bytes = (size_t)nsplit * g.m * g.n * sizeof(float);
     void* ws = nullptr;
     if (nsplit > 1 && gemm_workspace(&ws, part_bytes) != 0) return -1;

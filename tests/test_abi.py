@@ -44,11 +44,13 @@ def test_kernel_selection_names():
     name = capi.gemm_kernel_name
     assert name(1, 8192, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "mfma16_256x256"
     assert name(1, 8192, 8192, 8192, (1, 8192), (8192, 1), (8192, 1), capi.F16) == "mfma16_256x256"       # A^T view
-    assert name(1, 1, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "mfma16_stream_32x256"
-    assert name(1, 8, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "mfma16_stream_32x128"      # above 4 rows: 128-column strips
+    assert name(1, 1, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "mfma16_stream_32x128"
+    assert name(1, 8, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.BF16) == "mfma16_stream_32x128"
     assert name(1, 16, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F16) == "mfma16_stream_32x128"
     assert name(1, 32, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F16) == "mfma16_stream_32x128"
     assert name(1, 33, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F16) == "mfma16_skinny_32x128"
+    assert name(1, 32, 8192, 2048, (8192, 1), (2048, 1), (2048, 1), capi.F16) == "mfma16_skinny_32x128"      # 16 splits x 32 rows: its finish would be too long
+    assert name(1, 16, 4096, 2048, (4096, 1), (2048, 1), (2048, 1), capi.F16) == "mfma16_skinny_32x128"      # a small B that would need 16 splits
     assert name(1, 8, 8192, 8192, (8192, 1), (1, 8192), (8192, 1), capi.BF16) == "mfma16_skinny_32x128"
     assert name(1, 8, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), capi.F32) == "skinny"
     assert name(1, 128, 784, 256, (784, 1), (256, 1), (256, 1), capi.F32) == "tiny32_16x16"          # a small fp32 output: one launch of 16 x 16 tiles

@@ -249,7 +249,7 @@ def test_skinny_rows_mfma_split_k(dt, layout):
             continue                                   # a transposed A needs whole 16-byte vectors along m
         a, b = _operands(rng, m, k, n, dt, layout)
         a_st = (a.strides[0] // 2, a.strides[1] // 2); b_st = (b.strides[0] // 2, b.strides[1] // 2)
-        want_kernel = _stream_kernel(m) if layout == "nn" else "mfma16_skinny_32x128"
+        want_kernel = _stream_kernel(m, k, n) if layout == "nn" else "mfma16_skinny_32x128"
         assert capi.gemm_kernel_name(1, m, k, n, a_st, b_st, (n, 1), dt) == want_kernel
         bias = rand_storage(rng, (n,), dt); c0 = rand_storage(rng, (m, n), dt)
         got = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)
@@ -261,9 +261,13 @@ def test_skinny_rows_mfma_split_k(dt, layout):
     assert np.array_equal(device_gemm(a, b, dt), oracle_gemm(a, b, dt))
 
 
-def _stream_kernel(m):
-    """Row-major A and B with at most 32 rows: 256-column strips up to 4 rows, 128-column strips above."""
-    return "mfma16_stream_32x256" if m <= 4 else "mfma16_stream_32x128"
+def _stream_kernel(m, k, n):
+    """Row-major A and B with at most 32 rows take the streaming kernel unless the split of k it would need makes its
+    finish too long (the dispatcher's rule, restated for a device of 256 CUs): then the tiled kernel."""
+    groups = -(-n // 128)
+    nsplit = min(-(-256 // groups), max(1, k // 256))            # at least two passes of 128 rows per block
+    takes = m <= 32 and n % 8 == 0 and k % 8 == 0 and nsplit * m <= 256 and (nsplit <= 8 or k * n >= 1 << 24)
+    return "mfma16_stream_32x128" if takes else "mfma16_skinny_32x128"
 
 
 @pytest.mark.parametrize("m", [1, 3, 5, 8, 11, 16, 17, 27, 32])
@@ -273,9 +277,11 @@ def test_streaming_rows_single_launch_finish(m):
     clean), with ragged k (a partial last round, waves with unequal numbers of rounds) and n (a partial last strip, a
     number of strips that is not a multiple of 8), a bias and an accumulating epilogue."""
     rng = np.random.default_rng(39)
-    for dt, k, n in [(BF16, 8192, 2048), (F16, 4104, 1288), (BF16, 1024, 4096), (F16, 1064, 8200)]:
+    for dt, k, n in [(BF16, 8192, 4096), (F16, 4104, 4104), (BF16, 1024, 4096), (F16, 1064, 8200), (BF16, 8192, 2048)]:
         a, b = _operands(rng, m, k, n, dt, "nn")
-        assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == _stream_kernel(m)
+        assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == _stream_kernel(m, k, n)
+        if (k, n) != (8192, 2048):
+            assert _stream_kernel(m, k, n) == "mfma16_stream_32x128"          # (the shapes meant for the streaming kernel do take it)
         bias = rand_storage(rng, (n,), dt); c0 = rand_storage(rng, (m, n), dt)
         first = device_gemm(a, b, dt, bias=bias, c_init=c0, accumulate=True)
         _check(first, a, b, dt, k, bias=bias, c_init=c0, accumulate=True)
@@ -296,7 +302,7 @@ def test_streaming_rows_finish_repeats_bit_for_bit_over_hundreds_of_launches(m):
     k = n = 8192
     dt = BF16
     a = rand_storage(rng, (m, k), dt); b = rand_storage(rng, (k, n), dt)
-    assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == _stream_kernel(m)
+    assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == "mfma16_stream_32x128"
     da, db = capi.DeviceBuffer.from_numpy(a), capi.DeviceBuffer.from_numpy(b)
     launches = 300
     outs = [capi.DeviceBuffer(m * n * 2) for _ in range(launches)]
@@ -318,8 +324,8 @@ def test_tiled_rows_split_k_ragged(layout):
     launches reproduce the first bit for bit."""
     rng = np.random.default_rng(43)
     for dt, m, k, n in [(BF16, 32, 8192, 2048), (F16, 24, 4104, 1288), (BF16, 17, 1032, 4096), (F16, 104, 4160, 1160), (BF16, 8, 2048, 2048)]:
-        if (layout == "nn" and m <= 32) or (layout[0] == "t" and m % 8):
-            continue                                   # the streaming kernels' case; a transposed A needs whole 16-byte vectors along m
+        if (layout == "nn" and _stream_kernel(m, k, n) != "mfma16_skinny_32x128") or (layout[0] == "t" and m % 8):
+            continue                                   # the streaming kernel's case; a transposed A needs whole 16-byte vectors along m
         a, b = _operands(rng, m, k, n, dt, layout)
         a_st = (a.strides[0] // 2, a.strides[1] // 2); b_st = (b.strides[0] // 2, b.strides[1] // 2)
         assert capi.gemm_kernel_name(1, m, k, n, a_st, b_st, (n, 1), dt) == "mfma16_skinny_32x128"

@@ -49,9 +49,9 @@ def _both(rng, m, k, n, dtype, bias=False, accumulate=False, b_transposed=False)
 
 # (kernel the dispatcher picks, first shape, second smaller shape): every split-k launcher that takes a workspace
 CASES = [
-    ("mfma16_stream_32x256", BF16, (4, 4096, 4096), (2, 2048, 2048), {}),                 # partial sums + arrival counters, single launch
-    ("mfma16_stream_32x128", F16, (16, 8192, 2048), (8, 4096, 1024), {"bias": True}),     # the same on 128-column strips
-    ("mfma16_stream_32x128", BF16, (32, 4096, 4096), (20, 2048, 2048), {"accumulate": True}),
+    ("mfma16_stream_32x128", BF16, (4, 4096, 4096), (2, 2048, 4096), {}),                 # partial sums + arrival counters, single launch
+    ("mfma16_stream_32x128", F16, (16, 8192, 2048), (8, 4096, 4096), {"bias": True}),
+    ("mfma16_stream_32x128", BF16, (32, 4096, 4096), (20, 2048, 8192), {"accumulate": True}),
     ("mfma16_skinny_32x128", BF16, (40, 4096, 4096), (33, 2048, 2048), {"accumulate": True}),      # tiled split-k + combine launch
     ("mfma16_skinny_32x128", BF16, (8, 4096, 2048), (8, 2048, 2048), {"b_transposed": True}),
     ("skinny", F32, (4, 4096, 4096), (2, 2048, 1024), {}),                                # VALU streaming kernel
