@@ -393,11 +393,12 @@ def square_sweep(capi, sizes=(1024, 4096)):
 
 
 def skinny_fresh_process(rows=(1, 8, 16, 32)):
-    """The same few-row launches, each row timed by a child process that runs nothing else.  A launch of these kernels
-    takes 1.0 - 1.4 us longer once the process has run certain other kernels after its first few-row launch (a 1024^3
-    GEMM does it, a second kernel type of the few-row family does it; the kernel trace shows the time inside the kernel;
-    the cause was not found), so the figure of a row depends on what ran before it.  `us` in the table is the row timed
-    in this process, in the order 1, 8, 16, 32 after the headline GEMMs; this is the row alone in a process of its own."""
+    """The same few-row launches, each row timed by a child process that runs nothing else.  Streaming kernels can take
+    about 5 % longer once a process has run several kinds of kernel (the library's plain load-only kernel goes from 23.0
+    to 24.0 - 24.8 us per pass over the same 134 MB after a GEMM of another kind has run; the kernel trace shows the
+    time inside the kernels; the cause was not found), so a row's figure can depend on what ran before it.  `us` in the
+    table is the row timed in this process, in the order 1, 8, 16, 32 after the headline GEMMs; this is the row alone in
+    a process of its own."""
     import subprocess
     out = {}
     for m in rows:
