@@ -215,23 +215,39 @@ __global__ void __launch_bounds__(256) gemm_stream128_kernel(GemmArgs g, float* 
             *(f32x4_t*)(dst + 4) = f32x4_t{acc[f][4][v], acc[f][5][v], acc[f][6][v], acc[f][7][v]};
         }
     __syncthreads();
-    constexpr int QPR = S8_COLS / 4;                     // quads per row of the block's columns
+    // (all sums first, then the stores back to back with the kind of store chosen once: with the choice inside the loop
+    // the compiler waits for each store's acknowledgement before the next quad's LDS reads)
+    constexpr int QPR = S8_COLS / 4, NQ = MR / 8;        // quads per row of the block's columns, quads per thread
+    f32x4_t sum[NQ];
+    int qrow[NQ], qcol[NQ];
+    bool qlive[NQ];
 #pragma unroll
-    for (int i = 0; i < MR / 8; i++) {
-        const int idx = threadIdx.x + 256 * i, r = idx / QPR, gn = n0 + (idx % QPR) * 4;
-        if (r >= g.m || gn >= g.n) continue;                             // n is a multiple of 4, so a quad is wholly in or out
-        const int at_lds = r * S8_PITCH + (idx % QPR) * 4;
-        f32x4_t sum = *(const f32x4_t*)(red + at_lds);
+    for (int i = 0; i < NQ; i++) {
+        const int idx = threadIdx.x + 256 * i;
+        qrow[i] = idx / QPR; qcol[i] = n0 + (idx % QPR) * 4;
+        qlive[i] = qrow[i] < g.m && qcol[i] < g.n;                       // n is a multiple of 4, so a quad is wholly in or out
+        const int at_lds = qrow[i] * S8_PITCH + (idx % QPR) * 4;        // (rows from m to MR hold nothing and are not stored)
+        sum[i] = *(const f32x4_t*)(red + at_lds);
 #pragma unroll
-        for (int w = 1; w < S8_WAVES; w++) sum += *(const f32x4_t*)(red + w * MR * S8_PITCH + at_lds);
-        if (nsplit > 1) {
-            const long long at = ((long long)split * g.m + r) * g.n + gn;
-            if (!arrivals) *(f32x4_t*)(partials + at) = sum;
-            else if (local) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sum), part_rsrc, (int)(at * 4), 0, 0);
-            else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sum), part_rsrc, (int)(at * 4), 0, SPLITK_DEVICE_SCOPE);
-        } else out.store_quad(r, gn, sum);
+        for (int w = 1; w < S8_WAVES; w++) sum[i] += *(const f32x4_t*)(red + w * MR * S8_PITCH + at_lds);
     }
-    if (nsplit == 1 || !arrivals) return;
+    if (nsplit == 1) { out.store_quads(qrow, qcol, qlive, sum); return; }
+    if (!arrivals) {
+#pragma unroll
+        for (int i = 0; i < NQ; i++)
+            if (qlive[i]) *(f32x4_t*)(partials + ((long long)split * g.m + qrow[i]) * g.n + qcol[i]) = sum[i];
+        return;
+    }
+    int part_off[NQ];                                    // (dead quads: an offset beyond the buffer, the store is dropped)
+#pragma unroll
+    for (int i = 0; i < NQ; i++) part_off[i] = qlive[i] ? (int)((((long long)split * g.m + qrow[i]) * g.n + qcol[i]) * 4) : (int)BUFFER_OOB;
+    if (local) {
+#pragma unroll
+        for (int i = 0; i < NQ; i++) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sum[i]), part_rsrc, part_off[i], 0, 0);
+    } else {
+#pragma unroll
+        for (int i = 0; i < NQ; i++) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sum[i]), part_rsrc, part_off[i], 0, SPLITK_DEVICE_SCOPE);
+    }
 
     // ---- single-launch finish: the last block of this column group to arrive adds all splits ----
     if (!splitk_arrive(arrivals + group, nsplit, local != 0, &arrived_last)) return;
