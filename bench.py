@@ -316,21 +316,38 @@ def cpu_baseline_configs():
     return out
 
 
-def skinny_times(capi, quick_reps=20, rows=(1, 8, 16, 32)):
-    """Config 5a: bf16 A[m, 8192] x W[8192, 8192], replayed from a HIP graph; bytes are A, W and the output once."""
+def skinny_times(capi, quick_reps=20, rows=(1, 8, 16, 32), weights=8):
+    """Config 5a: bf16 A[m, 8192] x W[8192, 8192], replayed from a HIP graph; bytes are A, W and the output once.
+
+    `us` replays the product with the one W that was allocated first.  How fast a W streams depends on more than the
+    kernel: the same launch on the same buffers takes 21.4 - 22.0 us (m = 1, 8) on the W a process allocates first
+    while little else has moved through memory, and 23.1 - 23.2 us on W's allocated later or on the first one after
+    other large transfers (uploads, GEMMs on other buffers); re-reading the same 134 MB every launch also saves about
+    0.5 us against reading a different W each time.  `us_weights_in_turn` is the launch with `weights` different W's
+    in turn (1 GB in all, more than any cache holds): what a caller that walks through many weight matrices sees."""
     out = {}
     rng = np.random.default_rng(4)
     k = n = 8192
     w = _normal_bf16(rng, (k, n))
-    d_w = capi.DeviceBuffer.from_numpy(w)
+    d_ws = [capi.DeviceBuffer.from_numpy(w) for _ in range(max(1, weights))]
+    d_w = d_ws[0]
     for m in rows:
         a = _normal_bf16(rng, (m, k))
         d_a = capi.DeviceBuffer.from_numpy(a); d_y = capi.DeviceBuffer(m * n * 2)
-        fn = lambda: capi.gemm(d_y.ptr, d_a.ptr, d_w.ptr, None, 1, m, k, n, (0, k, 1), (0, n, 1), (0, n, 1), False, capi.BF16)
-        ms = _time_graph(capi, fn, quick_reps, 2)
+        product = lambda d_b: capi.gemm(d_y.ptr, d_a.ptr, d_b.ptr, None, 1, m, k, n, (0, k, 1), (0, n, 1), (0, n, 1), False, capi.BF16)
+        ms = _time_graph(capi, lambda: product(d_w), quick_reps, 2)
         nbytes = (m * k + k * n + m * n) * 2
-        out[f"skinny_bf16_m{m}"] = {"us": ms * 1e3, "GB/s": nbytes / (ms * 1e-3) / 1e9, "frac_hbm": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
-                                    "kernel": capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), capi.BF16)}
+        row = {"us": ms * 1e3, "GB/s": nbytes / (ms * 1e-3) / 1e9, "frac_hbm": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+               "kernel": capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), capi.BF16)}
+        if len(d_ws) > 1:
+            turn = [0]
+            def next_weight():
+                product(d_ws[turn[0] % len(d_ws)]); turn[0] += 1
+            reps = (quick_reps + len(d_ws) - 1) // len(d_ws) * len(d_ws)          # every W equally often
+            ms_turn = _time_graph(capi, next_weight, reps, 2)
+            row["us_weights_in_turn"] = ms_turn * 1e3
+            row["frac_hbm_weights_in_turn"] = nbytes / (ms_turn * 1e-3) / 1e9 / PEAK_HBM_GBS
+        out[f"skinny_bf16_m{m}"] = row
     return out
 
 
@@ -392,32 +409,8 @@ def square_sweep(capi, sizes=(1024, 4096)):
     return out
 
 
-def skinny_fresh_process(rows=(1, 8, 16, 32)):
-    """The same few-row launches, each row timed by a child process that runs nothing else.  Streaming kernels can take
-    about 5 % longer once a process has run several kinds of kernel (the library's plain load-only kernel goes from 23.0
-    to 24.0 - 24.8 us per pass over the same 134 MB after a GEMM of another kind has run; the kernel trace shows the
-    time inside the kernels; the cause was not found), so a row's figure can depend on what ran before it.  `us` in the
-    table is the row timed in this process, in the order 1, 8, 16, 32 after the headline GEMMs; this is the row alone in
-    a process of its own."""
-    import subprocess
-    out = {}
-    for m in rows:
-        try:
-            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--skinny-row", str(m)], capture_output=True, text=True, timeout=180)
-            out[m] = json.loads(r.stdout.strip().splitlines()[-1])["us"] if r.returncode == 0 else None
-        except Exception:
-            out[m] = None
-    return out
-
-
 def secondary(capi, quick_reps=20):
     out = skinny_times(capi, quick_reps)
-    k = n = 8192
-    for m, us in skinny_fresh_process().items():
-        row = out.get(f"skinny_bf16_m{m}")
-        if row is not None and us is not None:
-            row["us_fresh_process"] = us
-            row["frac_hbm_fresh_process"] = (m * k + k * n + m * n) * 2 / (us * 1e-6) / 1e9 / PEAK_HBM_GBS
     out["square_sweep"] = square_sweep(capi)
     out["gemm_f16_8192"] = f16_time(capi)
     out.update(wide_times(capi))
@@ -771,7 +764,6 @@ def main():
     ap.add_argument("--data", choices=["normal", "ints", "ones", "zeros"], default="normal",
                     help="operand values of the headline GEMMs: N(0,1) (the configuration) or low-toggle data, to show how far the "
                          "power-managed shader clock, and with it the throughput, depends on the values multiplied")
-    ap.add_argument("--skinny-row", type=int, default=0, help="time the few-row bf16 GEMM with this many rows and nothing else (what --skinny figures 'fresh process' come from)")
     ap.add_argument("--skinny-only", action="store_true",
                     help="run only the few-row bf16 GEMMs of configuration 5a and print their figures (for profiling that kernel alone)")
     ap.add_argument("--wide-only", action="store_true",
@@ -820,10 +812,7 @@ def main():
         print(json.dumps({"sustained_gemm_8192": sustained(capi, args.sustain, args.data, dtype=args.sustain_dtype)}))
         return
     if args.skinny_only:
-        print(json.dumps({"skinny": skinny_times(capi, rows=(1, 8, 32))}))
-        return
-    if args.skinny_row > 0:
-        print(json.dumps({"us": skinny_times(capi, rows=(args.skinny_row,))[f"skinny_bf16_m{args.skinny_row}"]["us"]}))
+        print(json.dumps({"skinny": skinny_times(capi)}))
         return
     if args.sweep_only:
         print(json.dumps({"square_sweep": square_sweep(capi)}))
