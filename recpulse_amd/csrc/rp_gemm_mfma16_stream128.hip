@@ -36,26 +36,23 @@ namespace rp {
 // them yet).  Otherwise they are exchanged at device scope (written through to
 // memory and read back from there), which costs about 1.5 us more per launch.
 //
-// A round is 16 RS rows of k (RS = 2: 32 rows), multiplied in RS steps of 16, one
-// v_mfma_f32_16x16x16 per 16 x 16 output tile and step.  In that instruction
-// lane (q, j) = (lane / 16, lane % 16) supplies four k values of row j (A) or
-// column j (B), and any assignment of a round's k values to (step, q) works as
-// long as A and B agree.  It is chosen for A's sake: lane (q, j) loads the 8 RS
-// bytes A[j][4 RS q .. 4 RS q + 4 RS - 1] of the round with one instruction (the
-// four q lanes of a row read one contiguous piece of the row's cache line), and
-// step t uses k = 4 RS q + 4t .. + 3.  With the natural assignment (k = 16t + 4q ..,
-// RS = 1) every step fetches 8 bytes out of each row's line again; these are L2
-// hits, but at 16 rows they cost 1.3 us per launch.  Longer rounds save more of
-// them and deal k to the waves in coarser pieces, which B's stream likes less:
-// at RS = 4 the launch takes 0.3 us longer than at RS = 2 for every m, and
-// RS = 1 is the faster one only below 8 rows (m = 32: 29.3 / 27.0 / 27.9 us for
-// RS = 1 / 2 / 4).
-// For B, step t reads rows 4 RS q + 4t + e (e = 0 .. 3): lane (q, j) loads 16
-// bytes (columns 8j .. 8j+7) of each, a load instruction covers four 256-byte
-// row segments 4 RS rows apart, and the 4 x 8 block of 16-bit values a lane
-// holds is transposed in registers (byte permutes) into 8 B-operands, one per
-// column residue c: operand c carries column 8j + c.  MFMA (f, c) accumulates the
-// 16 x 16 tile of rows 16f .. 16f+15 and columns {8j + c}.
+// A round is 32 rows of k, loaded in two steps of 16 and multiplied by one
+// v_mfma_f32_16x16x32 per 16 x 16 output tile.  In that instruction lane
+// (q, j) = (lane / 16, lane % 16) supplies the eight k values 8q .. 8q+7 of row j
+// (A) or column j (B).  For A that is one 16-byte load per lane and round: the
+// four q lanes of a row read 64 contiguous bytes of the row's cache line.  (With
+// 16-row rounds and v_mfma_f32_16x16x16, lane (q, j) fetches 8 bytes out of each
+// row's line per step; these are L2 hits, but at 16 rows they cost 1.3 us per
+// launch.  64-row rounds read A in whole lines but deal k to the waves in
+// coarser pieces, which B's stream likes less: 0.3 us longer at every m.  Two
+// 16x16x16 per tile and round instead of one 16x16x32 cost 0.1 - 0.2 us.)
+// For B, step t reads rows 8q + 4t + e (e = 0 .. 3): lane (q, j) loads 16 bytes
+// (columns 8j .. 8j+7) of each, a load instruction covers four 256-byte row
+// segments 8 rows apart, and the 4 x 8 block of 16-bit values a lane holds is
+// transposed in registers (byte permutes) into 8 half operands, one per column
+// residue c: residue c carries column 8j + c.  The first step's halves wait in
+// registers for the second's; MFMA (f, c) accumulates the 16 x 16 tile of rows
+// 16f .. 16f+15 and columns {8j + c}.
 //
 // 256-byte strips stream at the full rate only with about 8 KB of loads in
 // flight per wave (a read-only probe: 19.5 - 20.2 us for 134 MB with two steps
@@ -68,26 +65,24 @@ namespace rp {
 // ============================================================================
 constexpr int S8_WAVES = 4, S8_COLS = 128, S8_STEP = 16, S8_PITCH = S8_COLS + 8;
 constexpr int S8_MAX_M = 32;
-constexpr int S8_RS = 2;                // steps per round: 32 rows of k
-typedef short s16x4_t __attribute__((ext_vector_type(4)));
-typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
+constexpr int S8_RS = 2;                // steps per round: 32 rows of k, one v_mfma_f32_16x16x32 per tile
 
 template <typename T> struct s8_ops;
 template <> struct s8_ops<bf16_t> {
-    static __device__ __forceinline__ f32x4_t mma(u32x2_t a, u32x2_t b, f32x4_t c) {
-        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a), __builtin_bit_cast(s16x4_t, b), c, 0, 0, 0);
+    static __device__ __forceinline__ f32x4_t mma32(u32x4_t a, u32x4_t b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
     }
 };
 template <> struct s8_ops<f16_t> {
-    static __device__ __forceinline__ f32x4_t mma(u32x2_t a, u32x2_t b, f32x4_t c) {
-        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a), __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
+    static __device__ __forceinline__ f32x4_t mma32(u32x4_t a, u32x4_t b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
     }
 };
 
-template <typename T, int MR, int RS>
+template <typename T, int MR>
 __global__ void __launch_bounds__(256) gemm_stream128_kernel(GemmArgs g, float* partials, int groups, int nsplit, int* arrivals, int local) {
     constexpr int NF = MR / 16;                                           // A fragments (16 rows each)
-    constexpr int S8_ROUND = S8_STEP * RS;                                // k rows of a round (RS steps)
+    constexpr int RS = S8_RS, S8_ROUND = S8_STEP * RS;                    // steps and k rows of a round
     extern __shared__ __attribute__((aligned(16))) float red[];          // [S8_WAVES][MR][S8_PITCH]
     __shared__ bool arrived_last;
     const int lane = threadIdx.x & 63;
@@ -137,16 +132,9 @@ __global__ void __launch_bounds__(256) gemm_stream128_kernel(GemmArgs g, float* 
         __amdgpu_buffer_rsrc_t a_rsrc = buffer_rsrc(ab, r < my_rounds ? (long long)(a_end - ab) : 0);
 #pragma unroll
         for (int f = 0; f < NF; f++) {
-            if constexpr (RS == 1) {                         // (k is a multiple of 8 and the quad starts at a multiple of 4: wholly in or out)
-                const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(a_rsrc, (int)((kr + 4 * q < g.k) ? a_off[f] : BUFFER_OOB), 0, 0);
-                dst[f][0] = v[0]; dst[f][1] = v[1];
-            } else {
-#pragma unroll
-                for (int hh = 0; hh < RS / 2; hh++) {        // eight k values at a time, wholly in or out
-                    const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)((kr + 4 * RS * q + 8 * hh < g.k) ? a_off[f] + 16 * hh : BUFFER_OOB), 0, 0);
-                    dst[f][4 * hh] = v[0]; dst[f][4 * hh + 1] = v[1]; dst[f][4 * hh + 2] = v[2]; dst[f][4 * hh + 3] = v[3];
-                }
-            }
+            // (k is a multiple of 8 and the lane's piece starts at a multiple of 8: wholly in or out)
+            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)((kr + 8 * q < g.k) ? a_off[f] : BUFFER_OOB), 0, 0);
+            dst[f][0] = v[0]; dst[f][1] = v[1]; dst[f][2] = v[2]; dst[f][3] = v[3];
         }
     };
 
@@ -156,9 +144,10 @@ __global__ void __launch_bounds__(256) gemm_stream128_kernel(GemmArgs g, float* 
 #pragma unroll
         for (int c = 0; c < 8; c++) acc[f][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    // Step S of a pair of rounds (S = 0 .. 2 RS - 1: round r0 + S / RS, its step S % RS): multiply it out of slot
-    // S % 2, refill the slot with the step two ahead and, after a round's last step, its A registers with the round
-    // two ahead.
+    // Step S of a pair of rounds (S = 0 .. 3: round r0 + S / 2, its step S % 2): transpose it out of slot S % 2, refill
+    // the slot with the step two ahead and, at a round's second step, multiply the round and refill its A registers
+    // with the round two ahead.
+    u32x2_t held[8];                   // the first step's halves of the B operands of the round being multiplied
     auto consume = [&](auto sc, int r0) {
         constexpr int S = decltype(sc)::value, SLOT = S & 1, PAR = S / RS, T_ = S % RS;
         // in-register 4 x 8 transpose of 16-bit values: operand c, dword d = (k row 2d, k row 2d+1) of column c
@@ -168,25 +157,36 @@ __global__ void __launch_bounds__(256) gemm_stream128_kernel(GemmArgs g, float* 
 #pragma unroll
             for (int d = 0; d < 2; d++)
                 opb[c][d] = __builtin_amdgcn_perm(raw[SLOT][2 * d + 1][c / 2], raw[SLOT][2 * d][c / 2], (c & 1) ? 0x07060302u : 0x05040100u);
-        // (A's quad is moved to registers of its own, so that the refill below can land in the registers it came from)
-        u32x2_t opa[NF];
+        // A round of 32 k is one v_mfma_f32_16x16x32 per tile: lane (q, j) supplies k = 8q .. 8q+7, which is its A load as
+        // it stands and, for B, the first step's half followed by the second's.  The first step only transposes (its
+        // halves wait in `held`), the second multiplies.  Either way the operands must exist before the slot is
+        // refilled: then the refill can land in the very registers the slot occupies and nothing has to be copied
+        // (behind a full wait) at the loop's back edge.
+        if constexpr (T_ == 0) {
 #pragma unroll
-        for (int f = 0; f < NF; f++)
+            for (int c = 0; c < 8; c++) { held[c] = opb[c]; asm volatile("" : "+v"(held[c]) : : "memory"); }
+            __builtin_amdgcn_sched_barrier(0);
+            request_b(std::integral_constant<int, SLOT>{}, r0 + (S + 2) / RS, (S + 2) % RS);
+            __builtin_amdgcn_sched_barrier(0);
+        } else {
+            // (A's operand is moved to registers of its own, so that the refill below can land in the registers it came from)
+            u32x4_t opa[NF];
 #pragma unroll
-            for (int d = 0; d < 2; d++) asm volatile("v_mov_b32 %0, %1" : "=v"(opa[f][d]) : "v"(a_buf[PAR][f][2 * T_ + d]));
-        // The operands must exist before the slot is refilled: then the refill can land in the very registers the
-        // slot occupies and nothing has to be copied (behind a full wait) at the loop's back edge.
+            for (int f = 0; f < NF; f++)
 #pragma unroll
-        for (int c = 0; c < 8; c++) asm volatile("" : "+v"(opb[c]) : : "memory");
-        __builtin_amdgcn_sched_barrier(0);
-        request_b(std::integral_constant<int, SLOT>{}, r0 + (S + 2) / RS, (S + 2) % RS);
-        if constexpr (T_ == RS - 1) request_a(std::integral_constant<int, PAR>{}, r0 + PAR + 2);
-        __builtin_amdgcn_sched_barrier(0);
+                for (int d = 0; d < 4; d++) asm volatile("v_mov_b32 %0, %1" : "=v"(opa[f][d]) : "v"(a_buf[PAR][f][d]));
 #pragma unroll
-        for (int f = 0; f < NF; f++)
+            for (int c = 0; c < 8; c++) asm volatile("" : "+v"(opb[c]) : : "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            request_b(std::integral_constant<int, SLOT>{}, r0 + (S + 2) / RS, (S + 2) % RS);
+            request_a(std::integral_constant<int, PAR>{}, r0 + PAR + 2);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int c = 0; c < 8; c++) acc[f][c] = s8_ops<T>::mma(opa[f], opb[c], acc[f][c]);
-        __builtin_amdgcn_sched_barrier(0);
+            for (int f = 0; f < NF; f++)
+#pragma unroll
+                for (int c = 0; c < 8; c++) acc[f][c] = s8_ops<T>::mma32(opa[f], u32x4_t{held[c][0], held[c][1], opb[c][0], opb[c][1]}, acc[f][c]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     };
 
     // (requests stay in program order: the wait for a register counts the loads issued after its own)
@@ -254,10 +254,10 @@ __global__ void __launch_bounds__(256) gemm_stream128_kernel(GemmArgs g, float* 
     splitk_finish_window<T, S8_COLS, MR / 8, 4>(g, out, part_rsrc, nsplit, 0, g.m, n0, local != 0, arrivals + group);
 }
 
-template <typename T, int MR, int RS>
+template <typename T, int MR>
 static int launch_stream128_mr(const GemmArgs& g, float* partials, int groups, int nsplit, int* arrivals, int local) {
     constexpr size_t smem = (size_t)S8_WAVES * MR * S8_PITCH * sizeof(float);
-    auto kern = gemm_stream128_kernel<T, MR, RS>;
+    auto kern = gemm_stream128_kernel<T, MR>;
     if (smem > 64 * 1024 && !check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem), "hipFuncSetAttribute")) return -1;
     hipLaunchKernelGGL(kern, dim3(8 * ((groups + 7) / 8) * nsplit), dim3(256), smem, current_stream(), g, partials, groups, nsplit, arrivals, local);
     return check_launch("gemm_stream128_kernel") ? 0 : -1;
@@ -265,8 +265,8 @@ static int launch_stream128_mr(const GemmArgs& g, float* partials, int groups, i
 
 template <typename T>
 static int launch_stream128_t(const GemmArgs& g, float* partials, int groups, int nsplit, int* arrivals, int local) {
-    if (g.m <= 16) return launch_stream128_mr<T, 16, S8_RS>(g, partials, groups, nsplit, arrivals, local);
-    return launch_stream128_mr<T, 32, S8_RS>(g, partials, groups, nsplit, arrivals, local);
+    if (g.m <= 16) return launch_stream128_mr<T, 16>(g, partials, groups, nsplit, arrivals, local);
+    return launch_stream128_mr<T, 32>(g, partials, groups, nsplit, arrivals, local);
 }
 
 // k splits for an output of n columns: one block per CU (a wave per SIMD), each at least two passes of its waves deep
