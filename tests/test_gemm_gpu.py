@@ -293,6 +293,43 @@ def test_streaming_rows_single_launch_finish(m):
     assert np.array_equal(device_gemm(a, b, BF16), oracle_gemm(a, b, BF16))
 
 
+@pytest.mark.parametrize("dt", [BF16, F16], ids=lambda d: NAMES[d])
+def test_streaming_rows_output_layouts(dt):
+    """The streaming kernel writes its output in three ways (one 8-byte vector per four columns without and with
+    bias / accumulation, value by value when C's layout has no such vectors), from two places (the k-split finish,
+    and the block itself when k is too short to split).  Every layout of C must hold the bits of the dense result,
+    and the elements of C's buffer that are not part of C must keep theirs."""
+    rng = np.random.default_rng(41)
+    for m, k, n in [(8, 2048, 4096), (5, 1024, 32776), (27, 4096, 4104)]:           # 8 splits; no split (257 strips); ragged, 8 splits
+        assert capi.gemm_kernel_name(1, m, k, n, (k, 1), (n, 1), (n, 1), dt) == "mfma16_stream_32x128"
+        a, b = _operands(rng, m, k, n, dt, "nn")
+        bias = rand_storage(rng, (n,), dt); c0 = rand_storage(rng, (m, n), dt)
+        for with_epilogue in (False, True):
+            kw = dict(bias=bias, c_init=c0, accumulate=True) if with_epilogue else {}
+            dense = device_gemm(a, b, dt, **kw)
+            _check(dense, a, b, dt, k, **kw)
+            da, db, dbias = capi.DeviceBuffer.from_numpy(a), capi.DeviceBuffer.from_numpy(b), capi.DeviceBuffer.from_numpy(bias)
+            for what, shape, view_of in [("padded rows, vectors", (m, n + 24), lambda buf: buf[:, :n]),
+                                         ("odd row pitch", (m, n + 3), lambda buf: buf[:, :n]),
+                                         ("column-major", (n, m + 2), lambda buf: buf[:, :m].T)]:
+                host = np.full(shape, 0x7e31, dtype=capi.NP_STORAGE[dt])           # a pattern no result has everywhere
+                guard = host.copy()
+                if with_epilogue:
+                    view_of(host)[...] = c0
+                c_view = view_of(host)
+                dc = capi.DeviceBuffer.from_numpy(host)
+                capi.gemm(dc.ptr, da.ptr, db.ptr, dbias.ptr if with_epilogue else None, 1, m, k, n, (0, k, 1), (0, n, 1),
+                          (0,) + tuple(elem_strides(c_view)), with_epilogue, dt)
+                capi.synchronize()
+                out = dc.to_numpy(capi.NP_STORAGE[dt], shape)
+                dc.free()
+                assert np.array_equal(view_of(out), dense), (what, m, k, n, with_epilogue)
+                view_of(out)[...] = 0x7e31
+                assert np.array_equal(out, guard), ("wrote outside C", what, m, k, n)
+            for d in (da, db, dbias):
+                d.free()
+
+
 @pytest.mark.parametrize("m", [1, 8, 16, 32])
 def test_streaming_rows_finish_repeats_bit_for_bit_over_hundreds_of_launches(m):
     """The finish exchanges partial sums between the workgroups of a column group while other groups still stream:
