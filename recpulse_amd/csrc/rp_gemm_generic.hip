@@ -2,6 +2,7 @@
 // shape and stride, and the skinny split-k kernel for a few rows of A against a
 // row-major B (bound by streaming B from HBM).
 #include "rp_gemm.h"
+#include "rp_gemm_splitk_finish.h"
 
 #include <mutex>
 
@@ -256,14 +257,20 @@ __global__ void __launch_bounds__(256) gemm_splitk_combine_kernel(GemmArgs g, co
         for (int u = 0; u < 8; u++) sum += v[u];
     }
     for (; s < nsplit; s++) sum += *(const f32x4_t*)(q + s * split_stride);
-    T* C = (T*)g.C + (long long)blockIdx.y * g.c_bs;
-    const T* bias = (const T*)g.bias;
-    const bool has_bias = bias != nullptr, accum = g.accumulate != 0;
+    if constexpr (sizeof(T) == 2) {                    // 16-bit outputs: one 8-byte store where the layout allows, no branch per value without bias and accumulation
+        const SplitkOutput<T> out(g, (long long)blockIdx.y * g.c_bs);
+        if (out.plain()) out.store_quad_plain(r, c0, sum);
+        else out.store_quad(r, c0, sum);
+    } else {
+        T* C = (T*)g.C + (long long)blockIdx.y * g.c_bs;
+        const T* bias = (const T*)g.bias;
+        const bool has_bias = bias != nullptr, accum = g.accumulate != 0;
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
-        T* p = C + (long long)r * g.c_rs + (long long)(c0 + e) * g.c_cs;
-        T old = accum ? *p : T{};
-        *p = finish<T>(sum[e], has_bias, has_bias ? bias[c0 + e] : T{}, accum, old);
+        for (int e = 0; e < 4; e++) {
+            T* p = C + (long long)r * g.c_rs + (long long)(c0 + e) * g.c_cs;
+            T old = accum ? *p : T{};
+            *p = finish<T>(sum[e], has_bias, has_bias ? bias[c0 + e] : T{}, accum, old);
+        }
     }
 }
 

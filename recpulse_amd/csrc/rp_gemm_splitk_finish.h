@@ -12,9 +12,10 @@ struct SplitkOutput {
     const T* bias;
     long long c_rs, c_cs;
     bool has_bias, accum, c_vec;
-    __device__ __forceinline__ explicit SplitkOutput(const GemmArgs& g)
-        : C((T*)g.C), bias((const T*)g.bias), c_rs(g.c_rs), c_cs(g.c_cs), has_bias(g.bias != nullptr), accum(g.accumulate != 0),
-          c_vec(g.c_cs == 1 && g.c_rs % 4 == 0 && ((uintptr_t)g.C & 7) == 0) {}
+    // (c_offset: elements from g.C to the matrix of a batch that is written)
+    __device__ __forceinline__ explicit SplitkOutput(const GemmArgs& g, long long c_offset = 0)
+        : C((T*)g.C + c_offset), bias((const T*)g.bias), c_rs(g.c_rs), c_cs(g.c_cs), has_bias(g.bias != nullptr), accum(g.accumulate != 0),
+          c_vec(g.c_cs == 1 && g.c_rs % 4 == 0 && ((uintptr_t)((T*)g.C + c_offset) & 7) == 0) {}
     // True when an output needs nothing but the rounding and can be stored as one vector: callers then take
     // store_quad_plain, which has no branch per value (the general form below decides bias, accumulation and layout
     // for every value again, some sixty scalar branches for four quads).
