@@ -773,7 +773,8 @@ def main():
     ap.add_argument("--attention-only", action="store_true",
                     help="run only the configuration-4 attention launches in bf16, unfused and fused (for profiling those kernels alone)")
     ap.add_argument("--conv-only", action="store_true",
-                    help="run only the conv2d layer's launches in bf16 (for profiling those kernels alone)")
+                    help="run only the conv2d layer's launches (for profiling those kernels alone), in --conv-dtype")
+    ap.add_argument("--conv-dtype", choices=["bf16", "f32"], default="bf16")
     ap.add_argument("--mlp-only", action="store_true",
                     help="run only the configuration-2 MLP step (C ABI from a HIP graph, eager, and through the drop-in Python API)")
     ap.add_argument("--lstm-only", action="store_true",
@@ -836,7 +837,7 @@ def main():
         print(json.dumps({"mlp_f32_step": out}))
         return
     if args.conv_only:
-        print(json.dumps({"conv2d_bf16": conv2d_times(capi, "bf16")}))
+        print(json.dumps({"conv2d_" + args.conv_dtype: conv2d_times(capi, args.conv_dtype)}))
         return
     if args.wide_only:
         print(json.dumps({"wide": wide_times(capi, (("gemm_f32_4096", "f32", 4096), ("gemm_f64_2048", "f64", 2048), ("gemm_f64_4096", "f64", 4096)))}))
