@@ -319,12 +319,13 @@ def cpu_baseline_configs():
 def skinny_times(capi, quick_reps=20, rows=(1, 8, 16, 32), weights=8):
     """Config 5a: bf16 A[m, 8192] x W[8192, 8192], replayed from a HIP graph; bytes are A, W and the output once.
 
-    `us` replays the product with the one W that was allocated first.  How fast a W streams depends on more than the
-    kernel: the same launch on the same buffers takes 21.4 - 22.0 us (m = 1, 8) on the W a process allocates first
-    while little else has moved through memory, and 23.1 - 23.2 us on W's allocated later or on the first one after
-    other large transfers (uploads, GEMMs on other buffers); re-reading the same 134 MB every launch also saves about
-    0.5 us against reading a different W each time.  `us_weights_in_turn` is the launch with `weights` different W's
-    in turn (1 GB in all, more than any cache holds): what a caller that walks through many weight matrices sees."""
+    `us` replays the product with one W, the first one the process streams.  How fast a W streams depends on more than
+    the kernel: the same launch takes 21.4 - 22.0 us (m = 1, 8) on the first W a process streams and 23.1 - 23.2 us on
+    every W used after it, a fixed 1.2 us at the start of each launch whatever the size of W and whichever allocation
+    it is; the first W loses the advantage when other large transfers or GEMMs run in between.  Re-reading the same
+    134 MB every launch also saves about 0.5 us against reading a different W each time.  `us_weights_in_turn` is the
+    launch with `weights` different W's in turn (1 GB in all, more than any cache holds): what a caller that walks
+    through many weight matrices sees."""
     out = {}
     rng = np.random.default_rng(4)
     k = n = 8192
